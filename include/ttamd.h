@@ -1,0 +1,162 @@
+/*
+ * ttamd.h — C ABI of the MI355X (gfx950) GEMM backend for tinytensor.
+ *
+ * This is the drop-in boundary: everything a `BackendAMD : tinytensor::BackendBase`
+ * adapter needs for the GEMM hot path (matmul, batched matmul, nn::Linear, conv2d lowered
+ * to GEMM and their backward GEMMs).  Plain pointers and sizes only; every pointer named
+ * "device pointer" is memory obtained from ttamd_malloc (or any hipMalloc'ed memory of the
+ * same device).  Each entry cites the reference interface it stands in for
+ * (paths relative to the tinytensor source tree, v1.0.6).
+ *
+ * Conventions
+ *   - dtype codes follow tinytensor::ScalarType (include/tt/scalar.h:21-29).
+ *   - Strides and offsets are in ELEMENTS, as in tinytensor::Tensor::stride()/offset()
+ *     (include/tt/tensor.h:245-255).  Strides must be >= 0; 0 (expanded dims) is allowed.
+ *   - GEMM shapes use the reference's letters: lhs [B,N,K] . rhs [B,K,M] -> out [B,N,M]
+ *     (tinytensor/tensor/backend/cpu/matmul.cpp:25-33).
+ *   - Work is enqueued on `stream` (a hipStream_t passed as void*; NULL = the default
+ *     stream, which is what the reference's GPU backend uses,
+ *     tinytensor/tensor/backend/cuda/kernel_launch.cuh:19-29).  Calls do not synchronise;
+ *     ttamd_memcpy_d2h and ttamd_device_synchronize do.
+ *   - Every function returns a ttamd_status.  The adapter maps TTAMD_ERR_INVALID_ARGUMENT,
+ *     TTAMD_ERR_INVALID_DEVICE, TTAMD_ERR_UNSUPPORTED_DTYPE and TTAMD_ERR_OUT_OF_MEMORY to
+ *     `throw TTException` (include/tt/exception.h:15-25) and TTAMD_ERR_LAUNCH to TT_ERROR
+ *     (print + exit(1), include/tt/exception.h:28-36), mirroring
+ *     cuda/kernel_launch.cuh:25-28 and cuda/backend_cuda.cpp:53-63.
+ */
+#ifndef TTAMD_H_
+#define TTAMD_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum ttamd_status {
+    TTAMD_OK = 0,
+    TTAMD_ERR_INVALID_ARGUMENT = 1, /* shape/stride/pointer contract violated        -> TTException */
+    TTAMD_ERR_INVALID_DEVICE = 2,   /* device id out of range                        -> TTException */
+    TTAMD_ERR_UNSUPPORTED_DTYPE = 3,/* bool (matmul rejects it) or unknown code      -> TTException */
+    TTAMD_ERR_OUT_OF_MEMORY = 4,    /* hipMalloc failed                              -> TTException */
+    TTAMD_ERR_LAUNCH = 5            /* kernel launch / runtime failure               -> TT_ERROR    */
+} ttamd_status;
+
+typedef enum ttamd_dtype {
+    TTAMD_BOOL = 0,
+    TTAMD_U8 = 1,
+    TTAMD_I16 = 2,
+    TTAMD_I32 = 3,
+    TTAMD_I64 = 4,
+    TTAMD_F32 = 5,
+    TTAMD_F64 = 6
+} ttamd_dtype;
+
+/* A 3-D strided view of device memory: what a tinytensor::Tensor carries
+ * (storage pointer, offset(), stride(); include/tt/tensor.h:245-255). */
+typedef struct ttamd_view3 {
+    const void *data;  /* device pointer to element 0 of the storage */
+    int64_t offset;    /* element offset of the view's first element */
+    int64_t stride[3]; /* element strides: batch, row, column        */
+} ttamd_view3;
+
+/* A 4-D strided view (NCHW order of dims, arbitrary strides). */
+typedef struct ttamd_view4 {
+    const void *data;
+    int64_t offset;
+    int64_t stride[4];
+} ttamd_view4;
+
+/* Epilogue fused into the GEMM's store phase.  All fields 0/NULL = plain C = A.B, which is
+ * what BackendBase::batched_matmul computes.  The other modes serve the callers either side
+ * of the GEMM: nn::Linear's `+ bias->expand()` (tinytensor/nn/linear.cpp:45-48), the ReLU
+ * that follows it in an MLP, and conv2d's per-channel bias (cpu/conv.cpp:115-124). */
+typedef struct ttamd_epilogue {
+    const void *bias; /* device pointer, same dtype as the GEMM, or NULL                      */
+    int32_t bias_mode;/* 0 none, 1 = bias[column] (Linear), 2 = bias[row] (conv channel)      */
+    int32_t relu;     /* 1: out = max(out, 0) after the bias                                  */
+    int32_t accumulate;/* 1: out += result instead of out = result (grad accumulation)        */
+} ttamd_epilogue;
+
+/* ---- library / device ------------------------------------------------------------------ */
+
+/* BackendBase::get_device_count (tinytensor/tensor/backend_base.h:321). */
+ttamd_status ttamd_device_count(int *count);
+
+/* Human-readable text for the last non-OK status returned on this thread
+ * (the message the adapter puts into the TTException). */
+const char *ttamd_last_error_string(void);
+
+/* Name of the GPU architecture the loaded code object targets ("gfx950"). */
+const char *ttamd_target_arch(void);
+
+/* ---- storage: DeviceMemory<T> of the GPU peer (cuda/data_types.cuh:28-101) ------------- */
+
+/* Allocation with per-device byte counters (BackendBase::current_memory_allocated /
+ * total_memory_allocated, backend_base.h:317-318). */
+ttamd_status ttamd_malloc(int device, size_t bytes, void **out);
+ttamd_status ttamd_free(int device, void *ptr, size_t bytes);
+ttamd_status ttamd_memory_allocated(int device, uint64_t *current_bytes, uint64_t *total_bytes);
+
+/* Blocking copies: BackendBase::from_vec (backend_base.h:35-48) and to_vec (:55-60). */
+ttamd_status ttamd_memcpy_h2d(int device, void *dst_device, const void *src_host, size_t bytes);
+ttamd_status ttamd_memcpy_d2h(int device, void *dst_host, const void *src_device, size_t bytes);
+ttamd_status ttamd_memset_zero(int device, void *dst_device, size_t bytes, void *stream);
+ttamd_status ttamd_device_synchronize(int device);
+
+/* BackendBase::identity applied to a strided view = Tensor::contiguous()/clone()
+ * (tinytensor/tensor/tensor.cpp:583-596; CPU form cpu/unary.cpp:26-58, index map common/util.h:18-34).
+ * Copies the view (ndim <= 8, element strides >= 0) into dense row-major `out`.  The GEMM entry points
+ * do not need it; it serves the callers around them (reshape of a non-dense view). */
+ttamd_status ttamd_contiguous(int device, ttamd_dtype dtype, int ndim, const int64_t *shape, const int64_t *stride,
+                              const void *data, int64_t offset, void *out, void *stream);
+
+/* ---- the hot path ---------------------------------------------------------------------- */
+
+/* BackendBase::batched_matmul (backend_base.h:130; CPU: cpu/matmul.cpp:25-74,
+ * GPU peer: cuda/matmul.cu:26-78).  out[b] = lhs[b] . rhs[b] for b < B, out dense row-major
+ * [B,N,M].  lhs/rhs may be any non-negative-stride view (permuted, expanded, offset): the
+ * kernels read the view in place, no contiguous copy is made.  f32/f64 run on MFMA; u8/i16/
+ * i32/i64 wrap modulo 2^n like the reference's SIMD lanes.  `epilogue` may be NULL. */
+ttamd_status ttamd_batched_matmul(int device, ttamd_dtype dtype, int B, int N, int K, int M,
+                                  const ttamd_view3 *lhs, const ttamd_view3 *rhs, void *out,
+                                  const ttamd_epilogue *epilogue, void *stream);
+
+/* BackendBase::conv2d (backend_base.h:269-275; CPU: cpu/conv.cpp:36-134).  input [B,C,H,W],
+ * weight [O,C,k,k] (square kernel), bias [O] or NULL, zero padding; out dense [B,O,Ho,Wo] with
+ * Ho = (H + 2*padding - k)/stride + 1.  Implicit GEMM: no im2col buffer is materialised. */
+ttamd_status ttamd_conv2d_forward(int device, ttamd_dtype dtype, const ttamd_view4 *input, const ttamd_view4 *weight,
+                                  const void *bias, void *out, int B, int C, int H, int W, int O, int k, int stride,
+                                  int padding, void *stream);
+
+/* BackendBase::conv2d_backward (backend_base.h:277-284; CPU: cpu/conv.cpp:136-294).
+ * grad_out dense [B,O,Ho,Wo] (the reference reads it as dense storage, conv.cpp:199).
+ * Writes grad_input [B,C,H,W], grad_weight [O,C,k,k] and, when grad_bias != NULL,
+ * grad_bias [O] = sum of grad_out over batch and space (conv.cpp:289).  grad_input is a
+ * gather over output positions (no scatter-add, so no write race); grad_weight reduces over
+ * the batch inside one GEMM.  `workspace`/`workspace_bytes`: device scratch for the split
+ * reduction of grad_weight; query the size with ttamd_conv2d_backward_workspace. */
+ttamd_status ttamd_conv2d_backward_workspace(ttamd_dtype dtype, int B, int C, int H, int W, int O, int k, int stride,
+                                             int padding, size_t *bytes);
+ttamd_status ttamd_conv2d_backward(int device, ttamd_dtype dtype, const void *grad_out, const ttamd_view4 *input,
+                                   const ttamd_view4 *weight, void *grad_input, void *grad_weight, void *grad_bias,
+                                   int B, int C, int H, int W, int O, int k, int stride, int padding, void *workspace,
+                                   size_t workspace_bytes, void *stream);
+
+/* ---- timing (no reference counterpart: the reference has no timers; used by the benchmark
+ * to bracket kernels with HIP events on the stream they run on) ------------------------ */
+ttamd_status ttamd_event_create(int device, void **event);
+ttamd_status ttamd_event_destroy(void *event);
+ttamd_status ttamd_event_record(void *event, void *stream);
+ttamd_status ttamd_event_elapsed_ms(void *start, void *stop, float *ms); /* synchronises on `stop` */
+
+/* Name of the kernel variant the dispatcher would pick for a batched_matmul call with these
+ * arguments (for profiles and tests; does not launch).  Returned pointer is static. */
+const char *ttamd_batched_matmul_variant(ttamd_dtype dtype, int B, int N, int K, int M, const ttamd_view3 *lhs,
+                                         const ttamd_view3 *rhs);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* TTAMD_H_ */

@@ -1,0 +1,11 @@
+"""tinytensor_amd — MI355X (gfx950) GEMM backend for tinytensor: Python mirror of the host interface.
+
+The product is libttamd.so (HIP kernels behind the C ABI of include/ttamd.h).  This package is the
+thin host-side mirror of tinytensor's Tensor/backend interface for the GEMM path, used by the parity
+tests and the benchmark: same names, argument meaning and error behaviour as the reference's C++ API.
+"""
+from .tensor import (  # noqa: F401
+    BackendAMD, Device, Tensor, TTException, conv2d, conv2d_backward, get_backend, kAMD, linear, matmul,
+    matmul_backward,
+)
+from . import _capi  # noqa: F401

@@ -1,0 +1,78 @@
+"""ctypes binding of libttamd.so (the C ABI declared in include/ttamd.h).
+
+There is no CPU fallback: if the HIP library has not been built the import fails with
+instructions, and every call that needs a GPU reports the library's own error text.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "csrc", "libttamd.so")
+
+OK, ERR_INVALID_ARGUMENT, ERR_INVALID_DEVICE, ERR_UNSUPPORTED_DTYPE, ERR_OUT_OF_MEMORY, ERR_LAUNCH = range(6)
+BOOL, U8, I16, I32, I64, F32, F64 = range(7)
+
+
+class View3(C.Structure):
+    _fields_ = [("data", C.c_void_p), ("offset", C.c_int64), ("stride", C.c_int64 * 3)]
+
+
+class View4(C.Structure):
+    _fields_ = [("data", C.c_void_p), ("offset", C.c_int64), ("stride", C.c_int64 * 4)]
+
+
+class Epilogue(C.Structure):
+    _fields_ = [("bias", C.c_void_p), ("bias_mode", C.c_int32), ("relu", C.c_int32), ("accumulate", C.c_int32)]
+
+
+def _bind(lib: C.CDLL) -> None:
+    i, vp, sz = C.c_int, C.c_void_p, C.c_size_t
+    sig = {
+        "ttamd_device_count": (i, [C.POINTER(i)]),
+        "ttamd_last_error_string": (C.c_char_p, []),
+        "ttamd_target_arch": (C.c_char_p, []),
+        "ttamd_malloc": (i, [i, sz, C.POINTER(vp)]),
+        "ttamd_free": (i, [i, vp, sz]),
+        "ttamd_memory_allocated": (i, [i, C.POINTER(C.c_uint64), C.POINTER(C.c_uint64)]),
+        "ttamd_memcpy_h2d": (i, [i, vp, vp, sz]),
+        "ttamd_memcpy_d2h": (i, [i, vp, vp, sz]),
+        "ttamd_memset_zero": (i, [i, vp, sz, vp]),
+        "ttamd_device_synchronize": (i, [i]),
+        "ttamd_contiguous": (i, [i, i, i, C.POINTER(C.c_int64), C.POINTER(C.c_int64), vp, C.c_int64, vp, vp]),
+        "ttamd_batched_matmul": (i, [i, i, i, i, i, i, C.POINTER(View3), C.POINTER(View3), vp, C.POINTER(Epilogue), vp]),
+        "ttamd_batched_matmul_variant": (C.c_char_p, [i, i, i, i, i, C.POINTER(View3), C.POINTER(View3)]),
+        "ttamd_conv2d_forward": (i, [i, i, C.POINTER(View4), C.POINTER(View4), vp, vp] + [i] * 8 + [vp]),
+        "ttamd_conv2d_backward_workspace": (i, [i] + [i] * 8 + [C.POINTER(sz)]),
+        "ttamd_conv2d_backward": (i, [i, i, vp, C.POINTER(View4), C.POINTER(View4), vp, vp, vp] + [i] * 8 + [vp, sz, vp]),
+        "ttamd_event_create": (i, [i, C.POINTER(vp)]),
+        "ttamd_event_destroy": (i, [vp]),
+        "ttamd_event_record": (i, [vp, vp]),
+        "ttamd_event_elapsed_ms": (i, [vp, vp, C.POINTER(C.c_float)]),
+    }
+    missing = [name for name in sig if not hasattr(lib, name)]
+    if missing:
+        raise ImportError(f"{LIB_PATH} lacks {missing}: rebuild it (make -C tinytensor_amd/csrc)")
+    for name, (res, args) in sig.items():
+        fn = getattr(lib, name)
+        fn.restype = res
+        fn.argtypes = args
+
+
+def load() -> C.CDLL:
+    if not os.path.exists(LIB_PATH):
+        raise ImportError(
+            f"{LIB_PATH} is missing: build the HIP library first "
+            "(python -c 'import __graft_entry__ as g; g.build()' or make -C tinytensor_amd/csrc). "
+            "tinytensor_amd has no CPU fallback.")
+    lib = C.CDLL(LIB_PATH)
+    _bind(lib)
+    return lib
+
+
+lib = load()
+
+
+def last_error() -> str:
+    return lib.ttamd_last_error_string().decode()

@@ -1,0 +1,66 @@
+// common.h — internal declarations shared by the HIP sources of libttamd (gfx950 only).
+#ifndef TTAMD_CSRC_COMMON_H_
+#define TTAMD_CSRC_COMMON_H_
+
+#include <hip/hip_runtime.h>
+
+#include <cstdarg>
+#include <cstdint>
+#include <cstdio>
+
+#include "ttamd.h"
+
+namespace ttamd {
+
+// Thread-local text for ttamd_last_error_string().
+void set_error(const char *fmt, ...) __attribute__((format(printf, 1, 2)));
+
+// Makes `device` current; TTAMD_ERR_INVALID_DEVICE when the id is out of range.
+ttamd_status use_device(int device);
+
+inline size_t dtype_size(ttamd_dtype dt) {
+    switch (dt) {
+    case TTAMD_BOOL:
+    case TTAMD_U8: return 1;
+    case TTAMD_I16: return 2;
+    case TTAMD_I32:
+    case TTAMD_F32: return 4;
+    case TTAMD_I64:
+    case TTAMD_F64: return 8;
+    }
+    return 0;
+}
+
+#define TTAMD_HIP_CHECK(expr)                                                                  \
+    do {                                                                                       \
+        hipError_t e_ = (expr);                                                                \
+        if (e_ != hipSuccess) {                                                                \
+            ::ttamd::set_error("%s failed: %s (%s:%d)", #expr, hipGetErrorString(e_), __FILE__, __LINE__); \
+            return TTAMD_ERR_LAUNCH;                                                           \
+        }                                                                                      \
+    } while (0)
+
+// One GEMM problem as the kernels see it.  Conventional letters inside the kernels:
+// C[M,N] = A[M,K] . B[K,N]  (the C ABI's N,K,M map to M,K,N here).
+// Pointers already include the view's element offset.
+struct GemmArgs {
+    const void *A;
+    const void *B;
+    void *C;
+    int64_t a_sb, a_sm, a_sk;  // element strides of A: batch, row (m), column (k)
+    int64_t b_sb, b_sk, b_sn;  // element strides of B: batch, row (k), column (n)
+    int M, N, K, batch;
+    const void *bias;
+    int bias_mode, relu, accumulate;
+};
+
+// Launchers (defined in gemm_mfma.hip / gemm_simt.hip).  `variant_only`: fill *variant with the
+// kernel name that would run and return without launching.
+ttamd_status launch_gemm_mfma(ttamd_dtype dt, const GemmArgs &g, hipStream_t stream, const char **variant,
+                              bool variant_only, bool *handled);
+ttamd_status launch_gemm_simt(ttamd_dtype dt, const GemmArgs &g, hipStream_t stream, const char **variant,
+                              bool variant_only);
+
+}  // namespace ttamd
+
+#endif  // TTAMD_CSRC_COMMON_H_

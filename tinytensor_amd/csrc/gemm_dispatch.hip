@@ -1,0 +1,119 @@
+// gemm_dispatch.hip — ttamd_batched_matmul: argument contract and kernel selection.
+// Stands where BackendBase::batched_matmul does (tinytensor/tensor/backend_base.h:130); the
+// frontend has already promoted dtypes, rejected bool and lifted 1-D/2-D operands to 3-D
+// (tinytensor/tensor/tensor.cpp:2390-2484), so this layer only re-checks what would otherwise
+// become an out-of-bounds access on the device.
+#include "common.h"
+
+using namespace ttamd;
+
+namespace {
+
+ttamd_status build_args(ttamd_dtype dtype, int B, int N, int K, int M, const ttamd_view3 *lhs, const ttamd_view3 *rhs,
+                        void *out, const ttamd_epilogue *ep, GemmArgs *g, bool need_pointers) {
+    if (dtype == TTAMD_BOOL) {
+        set_error("matmul does not support boolean tensors");
+        return TTAMD_ERR_UNSUPPORTED_DTYPE;
+    }
+    const size_t esz = dtype_size(dtype);
+    if (esz == 0 || dtype < TTAMD_BOOL || dtype > TTAMD_F64) {
+        set_error("matmul: unknown dtype code %d", static_cast<int>(dtype));
+        return TTAMD_ERR_UNSUPPORTED_DTYPE;
+    }
+    if (B < 0 || N < 0 || K < 0 || M < 0) {
+        set_error("batched_matmul: negative extent (B=%d N=%d K=%d M=%d)", B, N, K, M);
+        return TTAMD_ERR_INVALID_ARGUMENT;
+    }
+    if (!lhs || !rhs) {
+        set_error("batched_matmul: NULL operand view");
+        return TTAMD_ERR_INVALID_ARGUMENT;
+    }
+    for (int i = 0; i < 3; ++i) {
+        if (lhs->stride[i] < 0 || rhs->stride[i] < 0) {
+            set_error("batched_matmul: negative strides are not supported");
+            return TTAMD_ERR_INVALID_ARGUMENT;
+        }
+    }
+    if (lhs->offset < 0 || rhs->offset < 0) {
+        set_error("batched_matmul: negative view offset");
+        return TTAMD_ERR_INVALID_ARGUMENT;
+    }
+    const bool empty_out = B == 0 || N == 0 || M == 0;
+    if (need_pointers && !empty_out) {
+        if (!out) {
+            set_error("batched_matmul: out is NULL");
+            return TTAMD_ERR_INVALID_ARGUMENT;
+        }
+        if (K > 0 && (!lhs->data || !rhs->data)) {
+            set_error("batched_matmul: operand data pointer is NULL");
+            return TTAMD_ERR_INVALID_ARGUMENT;
+        }
+        if (reinterpret_cast<uintptr_t>(out) % esz != 0 || reinterpret_cast<uintptr_t>(lhs->data) % esz != 0 ||
+            reinterpret_cast<uintptr_t>(rhs->data) % esz != 0) {
+            set_error("batched_matmul: pointers must be aligned to the element size");
+            return TTAMD_ERR_INVALID_ARGUMENT;
+        }
+    }
+    if (ep) {
+        if (ep->bias_mode < 0 || ep->bias_mode > 2 || (ep->bias_mode != 0 && !ep->bias)) {
+            set_error("batched_matmul: invalid epilogue (bias_mode=%d, bias=%p)", ep->bias_mode, ep->bias);
+            return TTAMD_ERR_INVALID_ARGUMENT;
+        }
+    }
+    g->A = static_cast<const char *>(lhs->data) + lhs->offset * static_cast<int64_t>(esz);
+    g->B = static_cast<const char *>(rhs->data) + rhs->offset * static_cast<int64_t>(esz);
+    g->C = out;
+    g->a_sb = lhs->stride[0];
+    g->a_sm = lhs->stride[1];
+    g->a_sk = lhs->stride[2];
+    g->b_sb = rhs->stride[0];
+    g->b_sk = rhs->stride[1];
+    g->b_sn = rhs->stride[2];
+    g->M = N;  // kernels use C[M,N] = A[M,K] . B[K,N]
+    g->K = K;
+    g->N = M;
+    g->batch = B;
+    g->bias = ep ? ep->bias : nullptr;
+    g->bias_mode = ep ? ep->bias_mode : 0;
+    g->relu = ep ? ep->relu : 0;
+    g->accumulate = ep ? ep->accumulate : 0;
+    return TTAMD_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+ttamd_status ttamd_batched_matmul(int device, ttamd_dtype dtype, int B, int N, int K, int M, const ttamd_view3 *lhs,
+                                  const ttamd_view3 *rhs, void *out, const ttamd_epilogue *epilogue, void *stream) {
+    GemmArgs g;
+    if (ttamd_status s = build_args(dtype, B, N, K, M, lhs, rhs, out, epilogue, &g, true)) return s;
+    if (ttamd_status s = use_device(device)) return s;
+    if (B == 0 || N == 0 || M == 0) return TTAMD_OK;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const char *variant = nullptr;
+    bool handled = false;
+    if (K > 0) {
+        if (ttamd_status s = launch_gemm_mfma(dtype, g, st, &variant, false, &handled)) return s;
+        if (handled) return TTAMD_OK;
+    }
+    // K == 0 also lands here: the vector-ALU kernel then stores the empty sum (0, + bias).
+    return launch_gemm_simt(dtype, g, st, &variant, false);
+}
+
+const char *ttamd_batched_matmul_variant(ttamd_dtype dtype, int B, int N, int K, int M, const ttamd_view3 *lhs,
+                                         const ttamd_view3 *rhs) {
+    GemmArgs g;
+    if (build_args(dtype, B, N, K, M, lhs, rhs, nullptr, nullptr, &g, false) != TTAMD_OK) return "invalid";
+    if (B == 0 || N == 0 || M == 0) return "empty";
+    const char *variant = "none";
+    bool handled = false;
+    if (K > 0) {
+        if (launch_gemm_mfma(dtype, g, nullptr, &variant, true, &handled) != TTAMD_OK) return "invalid";
+        if (handled) return variant;
+    }
+    if (launch_gemm_simt(dtype, g, nullptr, &variant, true) != TTAMD_OK) return "invalid";
+    return variant;
+}
+
+}  // extern "C"

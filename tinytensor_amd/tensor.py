@@ -1,0 +1,411 @@
+"""Host-side mirror of tinytensor's Tensor / BackendBase interface for the GEMM path.
+
+Only what the hot path needs: strided views over device storage (shape, stride, offset in
+elements, exactly what tinytensor::Tensor carries, include/tt/tensor.h:245-255), the `matmul`
+frontend (tinytensor/tensor/tensor.cpp:2390-2484), the autograd call pattern of the backward GEMMs
+(tinytensor/autograd/binary_ops.cpp:165-179), nn::Linear's forward (tinytensor/nn/linear.cpp:42-50),
+conv2d / conv2d_backward (tinytensor/tensor/backend_base.h:269-284) and the storage interop
+(from_vec / to_vec, backend_base.h:35-60).  All arithmetic happens in libttamd.so; nothing here
+computes on the host.
+"""
+from __future__ import annotations
+
+import ctypes as C
+from dataclasses import dataclass
+
+import numpy as np
+
+from . import _capi
+from ._capi import lib
+
+_NP_OF = {_capi.BOOL: np.bool_, _capi.U8: np.uint8, _capi.I16: np.int16, _capi.I32: np.int32, _capi.I64: np.int64,
+          _capi.F32: np.float32, _capi.F64: np.float64}
+_CODE_OF = {np.dtype(v): k for k, v in _NP_OF.items()}
+# promotion follows the ScalarType order bool < u8 < i16 < i32 < i64 < f32 < f64 (include/tt/scalar.h:21-29)
+
+
+class TTException(Exception):
+    """tinytensor::TTException (include/tt/exception.h:15-25)."""
+
+
+@dataclass(frozen=True)
+class Device:
+    backend: str
+    id: int = 0
+
+    def __str__(self) -> str:
+        return f"{self.backend}:{self.id}"
+
+
+kAMD = Device("amd", 0)
+
+
+def _check(status: int) -> None:
+    """Status -> exception mapping documented in include/ttamd.h."""
+    if status == _capi.OK:
+        return
+    msg = _capi.last_error()
+    if status == _capi.ERR_LAUNCH:
+        # The reference prints and exits (TT_ERROR, include/tt/exception.h:28-36); a Python host raises.
+        raise RuntimeError(f"unrecoverable device error: {msg}")
+    raise TTException(msg)
+
+
+class _Storage:
+    """Owning device allocation (peer of DeviceMemory<T>, cuda/data_types.cuh:28-101)."""
+
+    def __init__(self, nbytes: int, device: Device):
+        self.nbytes = int(nbytes)
+        self.device = device
+        p = C.c_void_p()
+        _check(lib.ttamd_malloc(device.id, self.nbytes, C.byref(p)))
+        self.ptr = p.value or 0
+
+    def __del__(self):
+        if getattr(self, "ptr", 0):
+            lib.ttamd_free(self.device.id, C.c_void_p(self.ptr), self.nbytes)
+            self.ptr = 0
+
+
+def _dense_strides(shape) -> tuple:
+    st, acc = [], 1
+    for s in reversed(shape):
+        st.append(acc)
+        acc *= s
+    return tuple(reversed(st))
+
+
+class Tensor:
+    """Strided view over device storage."""
+
+    def __init__(self, storage: _Storage, dtype: int, shape, stride=None, offset: int = 0):
+        self.storage = storage
+        self.dtype = dtype
+        self.shape = tuple(int(s) for s in shape)
+        self.stride = tuple(int(s) for s in (stride if stride is not None else _dense_strides(self.shape)))
+        self.offset = int(offset)
+
+    # ---- construction / readback -------------------------------------------------------------
+    @staticmethod
+    def from_numpy(a: np.ndarray, device: Device = kAMD) -> "Tensor":
+        """Tensor(std::vector<T>, shape, device) -> BackendBase::from_vec (backend_base.h:35-48)."""
+        a = np.ascontiguousarray(a)
+        if a.dtype not in _CODE_OF:
+            raise TTException(f"unsupported dtype {a.dtype}")
+        st = _Storage(max(a.nbytes, 1), device)
+        if a.nbytes:
+            _check(lib.ttamd_memcpy_h2d(device.id, C.c_void_p(st.ptr), C.c_void_p(a.ctypes.data), a.nbytes))
+        return Tensor(st, _CODE_OF[a.dtype], a.shape)
+
+    @staticmethod
+    def empty(shape, dtype: int, device: Device = kAMD) -> "Tensor":
+        n = int(np.prod(shape)) if len(shape) else 1
+        st = _Storage(max(n * np.dtype(_NP_OF[dtype]).itemsize, 1), device)
+        return Tensor(st, dtype, shape)
+
+    def storage_to_numpy(self) -> np.ndarray:
+        """BackendBase::to_vec: the WHOLE storage as a flat host array (backend_base.h:55-60)."""
+        npdt = np.dtype(_NP_OF[self.dtype])
+        out = np.empty(self.storage.nbytes // npdt.itemsize, dtype=npdt)
+        if out.nbytes:
+            _check(lib.ttamd_memcpy_d2h(self.device.id, C.c_void_p(out.ctypes.data), C.c_void_p(self.storage.ptr),
+                                        out.nbytes))
+        return out
+
+    def to_numpy(self) -> np.ndarray:
+        """Host copy of this view (Tensor::to_vec applies the view after the download)."""
+        flat = self.storage_to_numpy()
+        isz = flat.itemsize
+        v = np.lib.stride_tricks.as_strided(flat[self.offset:], shape=self.shape,
+                                            strides=tuple(s * isz for s in self.stride), writeable=False)
+        return np.array(v)
+
+    # ---- properties ----------------------------------------------------------------------------
+    @property
+    def device(self) -> Device:
+        return self.storage.device
+
+    def dim(self) -> int:
+        return len(self.shape)
+
+    def size(self, i: int) -> int:
+        return self.shape[i]
+
+    def numel(self) -> int:
+        return int(np.prod(self.shape)) if self.shape else 1
+
+    def is_contiguous(self) -> bool:
+        return self.stride == _dense_strides(self.shape)
+
+    @property
+    def itemsize(self) -> int:
+        return np.dtype(_NP_OF[self.dtype]).itemsize
+
+    # ---- views (tinytensor/autograd/shape_ops.cpp:24-146: only shape/stride/offset change) -------
+    def permute(self, *dims) -> "Tensor":
+        if len(dims) == 1 and isinstance(dims[0], (tuple, list)):
+            dims = tuple(dims[0])
+        if sorted(dims) != list(range(self.dim())):
+            raise TTException(f"Invalid permutation {dims} for {self.dim()} dimensions")
+        return Tensor(self.storage, self.dtype, [self.shape[d] for d in dims], [self.stride[d] for d in dims],
+                      self.offset)
+
+    def unsqueeze(self, dim: int) -> "Tensor":
+        if dim < 0:
+            dim += self.dim() + 1
+        shape = list(self.shape)
+        stride = list(self.stride)
+        shape.insert(dim, 1)
+        stride.insert(dim, 0)  # a size-1 dimension is never stepped over; no copy is needed
+        return Tensor(self.storage, self.dtype, shape, stride, self.offset)
+
+    def squeeze(self, dim: int) -> "Tensor":
+        if self.shape[dim] != 1:
+            return self
+        shape = list(self.shape)
+        stride = list(self.stride)
+        del shape[dim], stride[dim]
+        return Tensor(self.storage, self.dtype, shape, stride, self.offset)
+
+    def expand(self, shape) -> "Tensor":
+        shape = tuple(shape)
+        if len(shape) != self.dim():
+            raise TTException("expand: rank mismatch")
+        stride = []
+        for have, want, st in zip(self.shape, shape, self.stride):
+            if have == want:
+                stride.append(st)
+            elif have == 1:
+                stride.append(0)
+            else:
+                raise TTException(f"expand: cannot expand {self.shape} to {shape}")
+        return Tensor(self.storage, self.dtype, shape, stride, self.offset)
+
+    def contiguous(self) -> "Tensor":
+        """Tensor::contiguous (tensor.cpp:583-591): self if dense, else the identity op into new storage."""
+        return self if self.is_contiguous() else get_backend(self.device).identity(self)
+
+    def reshape(self, shape) -> "Tensor":
+        """Tensor::reshape (tensor.cpp:1371-1387): a view when dense, a clone otherwise."""
+        shape = list(shape)
+        if shape.count(-1) == 1:
+            known = int(np.prod([s for s in shape if s != -1]))
+            shape[shape.index(-1)] = self.numel() // max(known, 1)
+        if int(np.prod(shape)) != self.numel():
+            raise TTException(f"reshape: {self.shape} cannot be viewed as {tuple(shape)}")
+        base = self.contiguous()
+        return Tensor(base.storage, base.dtype, shape, None, base.offset)
+
+    def flatten(self, start: int = 0, end: int = -1) -> "Tensor":
+        n = self.dim()
+        if n == 0:
+            return self.reshape([1])
+        start %= n
+        end %= n
+        merged = int(np.prod(self.shape[start:end + 1]))
+        return self.reshape(list(self.shape[:start]) + [merged] + list(self.shape[end + 1:]))
+
+    def view3(self) -> _capi.View3:
+        v = _capi.View3()
+        v.data = self.storage.ptr
+        v.offset = self.offset
+        for i in range(3):
+            v.stride[i] = self.stride[i]
+        return v
+
+    def view4(self) -> _capi.View4:
+        v = _capi.View4()
+        v.data = self.storage.ptr
+        v.offset = self.offset
+        for i in range(4):
+            v.stride[i] = self.stride[i]
+        return v
+
+
+# -------------------------------------------------------------------------------------------------
+class BackendAMD:
+    """The methods of tinytensor::BackendBase (tensor/backend_base.h:23-322) that the GEMM path uses."""
+
+    def get_device_count(self) -> int:
+        n = C.c_int()
+        _check(lib.ttamd_device_count(C.byref(n)))
+        return n.value
+
+    def current_memory_allocated(self, device_id: int) -> int:
+        cur, tot = C.c_uint64(), C.c_uint64()
+        _check(lib.ttamd_memory_allocated(device_id, C.byref(cur), C.byref(tot)))
+        return cur.value
+
+    def total_memory_allocated(self, device_id: int) -> int:
+        cur, tot = C.c_uint64(), C.c_uint64()
+        _check(lib.ttamd_memory_allocated(device_id, C.byref(cur), C.byref(tot)))
+        return tot.value
+
+    def synchronize(self, device_id: int = 0) -> None:
+        _check(lib.ttamd_device_synchronize(device_id))
+
+    def identity(self, t: Tensor) -> Tensor:
+        """BackendBase::identity on a view = clone into dense storage (cpu/unary.cpp:26-58)."""
+        out = Tensor.empty(t.shape, t.dtype, t.device)
+        nd = t.dim()
+        shape = (C.c_int64 * max(nd, 1))(*t.shape)
+        stride = (C.c_int64 * max(nd, 1))(*t.stride)
+        _check(lib.ttamd_contiguous(t.device.id, t.dtype, nd, shape, stride, C.c_void_p(t.storage.ptr), t.offset,
+                                    C.c_void_p(out.storage.ptr), None))
+        return out
+
+    def batched_matmul(self, lhs: Tensor, rhs: Tensor, bias: Tensor | None = None, bias_mode: int = 0,
+                       relu: bool = False, out: Tensor | None = None, accumulate: bool = False) -> Tensor:
+        """BackendBase::batched_matmul (backend_base.h:130).  The keyword arguments select the fused
+        epilogue of ttamd_batched_matmul; with the defaults this is the reference call exactly."""
+        assert lhs.dim() == 3 and rhs.dim() == 3 and lhs.size(2) == rhs.size(1)
+        B, N, K = lhs.shape
+        M = rhs.size(2)
+        if out is None:
+            out = Tensor.empty((B, N, M), lhs.dtype, lhs.device)
+        ep = None
+        if bias is not None or relu or accumulate:
+            ep = _capi.Epilogue()
+            ep.bias = (bias.storage.ptr + bias.offset * bias.itemsize) if bias is not None else None
+            ep.bias_mode = bias_mode if bias is not None else 0
+            ep.relu = int(relu)
+            ep.accumulate = int(accumulate)
+        lv, rv = lhs.view3(), rhs.view3()
+        _check(lib.ttamd_batched_matmul(lhs.device.id, lhs.dtype, B, N, K, M, C.byref(lv), C.byref(rv),
+                                        C.c_void_p(out.storage.ptr), C.byref(ep) if ep is not None else None, None))
+        return out
+
+    def batched_matmul_variant(self, lhs: Tensor, rhs: Tensor) -> str:
+        B, N, K = lhs.shape
+        lv, rv = lhs.view3(), rhs.view3()
+        return lib.ttamd_batched_matmul_variant(lhs.dtype, B, N, K, rhs.size(2), C.byref(lv), C.byref(rv)).decode()
+
+    def conv2d(self, input: Tensor, weight: Tensor, bias: Tensor | None, stride: int, padding: int) -> Tensor:
+        """BackendBase::conv2d (backend_base.h:269-275)."""
+        B, Cc, H, W = input.shape
+        O, _, k, _ = weight.shape
+        Ho = (H + 2 * padding - k) // stride + 1
+        Wo = (W + 2 * padding - k) // stride + 1
+        out = Tensor.empty((B, O, Ho, Wo), input.dtype, input.device)
+        iv, wv = input.view4(), weight.view4()
+        bptr = None
+        if bias is not None:
+            bias = bias.contiguous()
+            bptr = C.c_void_p(bias.storage.ptr + bias.offset * bias.itemsize)
+        _check(lib.ttamd_conv2d_forward(input.device.id, input.dtype, C.byref(iv), C.byref(wv), bptr,
+                                        C.c_void_p(out.storage.ptr), B, Cc, H, W, O, k, stride, padding, None))
+        return out
+
+    def conv2d_backward(self, grad_output: Tensor, input: Tensor, weight: Tensor, bias: Tensor | None, stride: int,
+                        padding: int):
+        """BackendBase::conv2d_backward (backend_base.h:277-284) -> (grad_input, grad_weight, grad_bias|None)."""
+        B, Cc, H, W = input.shape
+        O, _, k, _ = weight.shape
+        go = grad_output.contiguous()
+        gx = Tensor.empty(input.shape, input.dtype, input.device)
+        gw = Tensor.empty(weight.shape, input.dtype, input.device)
+        gb = Tensor.empty((O,), input.dtype, input.device) if bias is not None else None
+        ws_bytes = C.c_size_t()
+        _check(lib.ttamd_conv2d_backward_workspace(input.dtype, B, Cc, H, W, O, k, stride, padding, C.byref(ws_bytes)))
+        ws = _Storage(max(ws_bytes.value, 1), input.device)
+        iv, wv = input.view4(), weight.view4()
+        _check(lib.ttamd_conv2d_backward(
+            input.device.id, input.dtype, C.c_void_p(go.storage.ptr + go.offset * go.itemsize), C.byref(iv),
+            C.byref(wv), C.c_void_p(gx.storage.ptr), C.c_void_p(gw.storage.ptr),
+            C.c_void_p(gb.storage.ptr) if gb is not None else None, B, Cc, H, W, O, k, stride, padding,
+            C.c_void_p(ws.ptr), ws.nbytes, None))
+        self.synchronize(input.device.id)  # the workspace is released when this frame returns
+        return gx, gw, gb
+
+
+_BACKEND = BackendAMD()
+
+
+def get_backend(device: Device) -> BackendAMD:
+    """get_backend(Device) (tinytensor/tensor/backend_register.cpp:19-38)."""
+    if device.backend != "amd":
+        raise TTException(f"Unknown device type {device.backend}")
+    return _BACKEND
+
+
+# -------------------------------------------------------------------------------------------------
+def _promote(lhs: Tensor, rhs: Tensor):
+    if lhs.device != rhs.device:
+        raise TTException(f"Expected tensors on the same device, given {lhs.device} and {rhs.device}")
+    dt = max(lhs.dtype, rhs.dtype)
+    if dt == _capi.BOOL:
+        raise TTException("matmul does not support boolean tensors")
+    if lhs.dtype != dt or rhs.dtype != dt:
+        # Tensor::to(dtype) is an elementwise cast outside the GEMM path; the callers of this mirror
+        # hand over operands of one dtype.
+        raise TTException("mixed-dtype matmul needs a cast op, which this backend slice does not provide")
+    return lhs, rhs
+
+
+def matmul(lhs: Tensor, rhs: Tensor) -> Tensor:
+    """tinytensor::matmul (tensor/tensor.cpp:2390-2484): rank dispatch onto batched_matmul."""
+    lhs, rhs = _promote(lhs, rhs)
+    be = get_backend(lhs.device)
+    ls, rs = lhs.shape, rhs.shape
+    if lhs.dim() == 1 and rhs.dim() == 1:
+        if ls[0] != rs[0]:
+            raise TTException(f"Invalid shapes for dot product. LHS={ls} and RHS={rs}")
+        return be.batched_matmul(lhs.reshape([1, 1, ls[0]]), rhs.reshape([1, rs[0], 1])).flatten()
+    if lhs.dim() == 1 and rhs.dim() == 2:
+        if ls[0] != rs[0]:
+            raise TTException(f"Invalid shape for matrix multiplication. LHS={ls} and RHS={rs}")
+        return be.batched_matmul(lhs.reshape([1, 1, ls[0]]), rhs.unsqueeze(0)).flatten()
+    if lhs.dim() == 2 and rhs.dim() == 1:
+        if ls[1] != rs[0]:
+            raise TTException(f"Invalid shape for matrix multiplication. LHS={ls} and RHS={rs}")
+        return be.batched_matmul(lhs.unsqueeze(0), rhs.reshape([1, rs[0], 1])).flatten()
+    if lhs.dim() == 2 and rhs.dim() == 2:
+        if ls[1] != rs[0]:
+            raise TTException(f"Invalid shape for matrix multiplication. LHS={ls} and RHS={rs}")
+        return be.batched_matmul(lhs.unsqueeze(0), rhs.unsqueeze(0)).squeeze(0)
+    if lhs.dim() == 3 and rhs.dim() == 3:
+        if ls[2] != rs[1] or ls[0] != rs[0]:
+            raise TTException(f"Invalid shape for batched matrix multiplication. LHS={ls} and RHS={rs}")
+        return be.batched_matmul(lhs, rhs)
+    raise TTException("Unsupported sizes. Try reshaping or broadcasting.")
+
+
+def matmul_backward(lhs: Tensor, rhs: Tensor, grad_output: Tensor):
+    """TensorBatchedMatmul::backward (autograd/binary_ops.cpp:173-179): dA = dC.B^T, dB = A^T.dC, both
+    on permute({0,2,1}) VIEWS.  Both gradients are always computed, as in the reference."""
+    return matmul(grad_output, rhs.permute(0, 2, 1)), matmul(lhs.permute(0, 2, 1), grad_output)
+
+
+def linear(input: Tensor, weight: Tensor, bias: Tensor | None = None, relu: bool = False) -> Tensor:
+    """nn::Linear::forward (nn/linear.cpp:42-50): matmul(input.flatten(0,-2), weight) + bias, weight
+    [in,out].  The bias add (and an optional ReLU that follows it) is fused into the GEMM epilogue."""
+    x2 = input.flatten(0, -2) if input.dim() != 2 else input
+    if x2.size(1) != weight.size(0):
+        raise TTException(f"Invalid shape for matrix multiplication. LHS={x2.shape} and RHS={weight.shape}")
+    _promote(x2, weight)
+    out = get_backend(input.device).batched_matmul(x2.unsqueeze(0), weight.unsqueeze(0), bias=bias, bias_mode=1,
+                                                   relu=relu)
+    return out.reshape(list(input.shape[:-1]) + [weight.size(1)])
+
+
+def conv2d(input: Tensor, weight: Tensor, bias: Tensor | None = None, stride: int = 1, padding: int = 0) -> Tensor:
+    """tinytensor::conv2d argument checks (tensor/tensor.cpp:3089-3167) then BackendBase::conv2d."""
+    if input.dim() != 4 or weight.dim() != 4:
+        raise TTException("conv2d expects 4-D input [B,C,H,W] and weight [O,C,k,k]")
+    if input.size(1) != weight.size(1):
+        raise TTException("conv2d: input channels do not match weight channels")
+    if weight.size(2) != weight.size(3):
+        raise TTException("conv2d: only square kernels are supported")
+    if stride <= 0 or padding < 0:
+        raise TTException("conv2d: stride must be > 0 and padding >= 0")
+    if bias is not None and (bias.dim() != 1 or bias.size(0) != weight.size(0)):
+        raise TTException("conv2d: bias must have one entry per output channel")
+    if input.dtype != weight.dtype or input.dtype == _capi.BOOL:
+        raise TTException("conv2d: operands must share one non-bool dtype")
+    return get_backend(input.device).conv2d(input, weight, bias, stride, padding)
+
+
+def conv2d_backward(grad_output: Tensor, input: Tensor, weight: Tensor, bias: Tensor | None = None, stride: int = 1,
+                    padding: int = 0):
+    """TensorConv2d::backward (autograd/conv_ops.cpp:55-80) -> BackendBase::conv2d_backward."""
+    return get_backend(input.device).conv2d_backward(grad_output, input, weight, bias, stride, padding)
