@@ -64,6 +64,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--n", type=int, default=4096, help="square size (the metric is quoted at 4096)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="first run one dense 256 MiB copy kernel (known HBM traffic) to scale profiler byte counters")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
@@ -72,6 +74,12 @@ def main():
     import numpy as np
 
     import tinytensor_amd as tt
+
+    if args.copy_calibration:
+        # 64 Mi f32 elements: reads 256 MiB and writes 256 MiB, both exactly known.
+        src = tt.Tensor.empty((64 * 1024 * 1024,), tt._capi.F32)
+        tt.get_backend(tt.kAMD).identity(tt.Tensor(src.storage, src.dtype, (8192, 8192), (8192, 1), 0))
+        tt.get_backend(tt.kAMD).synchronize(0)
 
     n = args.n
     flop = 2.0 * n * n * n

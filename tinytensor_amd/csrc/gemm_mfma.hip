@@ -158,7 +158,9 @@ struct Stager {
         }
     }
 
-    // Loads tile kt.  k_left = K - kt*BK; `edge` = tile overlaps the row bound (MC masks needed).
+    // Loads the next tile.  k_left = K - kt*BK; `edge` = tile overlaps the row bound (MC masks needed).
+    // MASK = false is the steady state (full k tile, interior rows): loads only, no selects.
+    template <bool MASK>
     __device__ __forceinline__ void load(__amdgpu_buffer_rsrc_t rsrc, int tid, int k_left, bool edge,
                                          uint32_t k_step_b) {
         const bool k_tail = k_left < BK;
@@ -166,6 +168,10 @@ struct Stager {
         for (int p = 0; p < P; ++p) {
             V v = Vec<T, VEC>::load(rsrc, voff[p]);
             voff[p] += k_step_b;
+            if constexpr (!MASK) {
+                reg[p] = v;
+                continue;
+            }
             if constexpr (KC) {
                 if (k_tail) {
                     const int col = col_of(p, tid);
@@ -268,12 +274,11 @@ __global__ void __launch_bounds__(kThreads) gemm_mfma_kernel(GemmArgs g, int til
     using FrA = Fragment<T, StA::LD, A_KC, NBM>;
     using FrB = Fragment<T, StB::LD, B_KC, NBN>;
 
+    // LDS: [A buf 0][A buf 1][B buf 0][B buf 1]; addressed as offsets from the one shared base so that
+    // every access stays a DS instruction (no generic-pointer loads, which would also wait on vmcnt).
     extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
-    T *lds_a[2], *lds_b[2];
-    lds_a[0] = reinterpret_cast<T *>(smem_raw);
-    lds_a[1] = lds_a[0] + StA::LDS_ELEMS;
-    lds_b[0] = lds_a[1] + StA::LDS_ELEMS;
-    lds_b[1] = lds_b[0] + StB::LDS_ELEMS;
+    T *const smem = reinterpret_cast<T *>(smem_raw);
+    constexpr int kBOff = 2 * StA::LDS_ELEMS;
 
     const int tid = threadIdx.x;
     const int lane = tid % 64;
@@ -327,10 +332,11 @@ __global__ void __launch_bounds__(kThreads) gemm_mfma_kernel(GemmArgs g, int til
             for (int e = 0; e < M::NACC; ++e) acc[i][j][e] = T(0);
 
     const int KT = (g.K + BK - 1) / BK;
-    sa.load(a_rsrc, tid, g.K, a_edge, a_sk_b * BK);
-    sb.load(b_rsrc, tid, g.K, b_edge, b_sk_b * BK);
-    sa.store(lds_a[0], tid);
-    sb.store(lds_b[0], tid);
+    const bool interior = !a_edge && !b_edge;  // workgroup-uniform
+    sa.template load<true>(a_rsrc, tid, g.K, a_edge, a_sk_b * BK);
+    sb.template load<true>(b_rsrc, tid, g.K, b_edge, b_sk_b * BK);
+    sa.store(smem, tid);
+    sb.store(smem + kBOff, tid);
     __syncthreads();
 
     for (int kt = 0; kt < KT; ++kt) {
@@ -338,11 +344,16 @@ __global__ void __launch_bounds__(kThreads) gemm_mfma_kernel(GemmArgs g, int til
         const bool more = kt + 1 < KT;
         if (more) {
             const int k_left = g.K - (kt + 1) * BK;
-            sa.load(a_rsrc, tid, k_left, a_edge, a_sk_b * BK);
-            sb.load(b_rsrc, tid, k_left, b_edge, b_sk_b * BK);
+            if (interior && k_left >= BK) {
+                sa.template load<false>(a_rsrc, tid, k_left, false, a_sk_b * BK);
+                sb.template load<false>(b_rsrc, tid, k_left, false, b_sk_b * BK);
+            } else {
+                sa.template load<true>(a_rsrc, tid, k_left, a_edge, a_sk_b * BK);
+                sb.template load<true>(b_rsrc, tid, k_left, b_edge, b_sk_b * BK);
+            }
         }
-        const T *la = lds_a[cur];
-        const T *lb = lds_b[cur];
+        const T *la = smem + cur * StA::LDS_ELEMS;
+        const T *lb = smem + kBOff + cur * StB::LDS_ELEMS;
 #pragma unroll
         for (int c = 0; c < BK / kChunk; ++c) {
             FrA fa;
@@ -357,8 +368,8 @@ __global__ void __launch_bounds__(kThreads) gemm_mfma_kernel(GemmArgs g, int til
                     for (int bn = 0; bn < NBN; ++bn) acc[bm][bn] = M::mma(fa.v[bm][j], fb.v[bn][j], acc[bm][bn]);
         }
         if (more) {
-            sa.store(lds_a[cur ^ 1], tid);
-            sb.store(lds_b[cur ^ 1], tid);
+            sa.store(smem + (cur ^ 1) * StA::LDS_ELEMS, tid);
+            sb.store(smem + kBOff + (cur ^ 1) * StB::LDS_ELEMS, tid);
         }
         __syncthreads();
     }
