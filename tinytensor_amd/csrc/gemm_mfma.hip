@@ -263,7 +263,7 @@ __device__ __forceinline__ int remap_xcd(int pid, int total) {
 
 // ---------------------------------------------------------------------------------------------
 template <typename T, int BM, int BN, int BK, int WGM, int WGN, bool A_KC, int A_VEC, bool B_KC, int B_VEC>
-__global__ void __launch_bounds__(kThreads) gemm_mfma_kernel(GemmArgs g, int tiles_m, int tiles_n) {
+__global__ void __launch_bounds__(kThreads, 2) gemm_mfma_kernel(GemmArgs g, int tiles_m, int tiles_n) {
     using M = Mfma<T>;
     static_assert(WGM * WGN == kWaves, "4 waves per workgroup");
     constexpr int WM = BM / WGM, WN = BN / WGN;
@@ -332,28 +332,15 @@ __global__ void __launch_bounds__(kThreads) gemm_mfma_kernel(GemmArgs g, int til
             for (int e = 0; e < M::NACC; ++e) acc[i][j][e] = T(0);
 
     const int KT = (g.K + BK - 1) / BK;
-    const bool interior = !a_edge && !b_edge;  // workgroup-uniform
     sa.template load<true>(a_rsrc, tid, g.K, a_edge, a_sk_b * BK);
     sb.template load<true>(b_rsrc, tid, g.K, b_edge, b_sk_b * BK);
     sa.store(smem, tid);
     sb.store(smem + kBOff, tid);
     __syncthreads();
 
-    for (int kt = 0; kt < KT; ++kt) {
-        const int cur = kt & 1;
-        const bool more = kt + 1 < KT;
-        if (more) {
-            const int k_left = g.K - (kt + 1) * BK;
-            if (interior && k_left >= BK) {
-                sa.template load<false>(a_rsrc, tid, k_left, false, a_sk_b * BK);
-                sb.template load<false>(b_rsrc, tid, k_left, false, b_sk_b * BK);
-            } else {
-                sa.template load<true>(a_rsrc, tid, k_left, a_edge, a_sk_b * BK);
-                sb.template load<true>(b_rsrc, tid, k_left, b_edge, b_sk_b * BK);
-            }
-        }
-        const T *la = smem + cur * StA::LDS_ELEMS;
-        const T *lb = smem + kBOff + cur * StB::LDS_ELEMS;
+    auto compute = [&](int buf) {
+        const T *la = smem + buf * StA::LDS_ELEMS;
+        const T *lb = smem + kBOff + buf * StB::LDS_ELEMS;
 #pragma unroll
         for (int c = 0; c < BK / kChunk; ++c) {
             FrA fa;
@@ -367,34 +354,81 @@ __global__ void __launch_bounds__(kThreads) gemm_mfma_kernel(GemmArgs g, int til
 #pragma unroll
                     for (int bn = 0; bn < NBN; ++bn) acc[bm][bn] = M::mma(fa.v[bm][j], fb.v[bn][j], acc[bm][bn]);
         }
-        if (more) {
+    };
+
+    // Tiles 0 .. KT-2: prefetch tile kt+1 into registers, multiply tile kt out of LDS, then park the
+    // prefetched tile in the other LDS buffer.  The last tile is multiplied after the loop, so the loop
+    // body has no conditionals.  MASK = false is the steady state (interior workgroup, K a multiple of BK).
+    auto pipeline = [&]<bool MASK>() {
+        for (int kt = 0; kt + 1 < KT; ++kt) {
+            const int cur = kt & 1;
+            const int k_left = g.K - (kt + 1) * BK;
+            sa.template load<MASK>(a_rsrc, tid, k_left, a_edge, a_sk_b * BK);
+            sb.template load<MASK>(b_rsrc, tid, k_left, b_edge, b_sk_b * BK);
+            compute(cur);
             sa.store(smem + (cur ^ 1) * StA::LDS_ELEMS, tid);
             sb.store(smem + kBOff + (cur ^ 1) * StB::LDS_ELEMS, tid);
+            __syncthreads();
         }
-        __syncthreads();
+    };
+    if (!a_edge && !b_edge && g.K % BK == 0) {
+        pipeline.template operator()<false>();
+    } else {
+        pipeline.template operator()<true>();
     }
+    if (KT > 0) compute((KT - 1) & 1);
 
     // Epilogue: registers -> C (dense row-major), optional bias / ReLU / accumulate.
     T *__restrict__ C = static_cast<T *>(g.C) + static_cast<int64_t>(batch) * g.M * g.N;
     const T *__restrict__ bias = static_cast<const T *>(g.bias);
     const int jcol = lane % M::MB;
+    auto finish = [&](T v, int m, int n, int64_t idx) {
+        if (g.bias_mode == 1) v += bias[n];
+        if (g.bias_mode == 2) v += bias[m];
+        if (g.relu) v = v > T(0) ? v : T(0);
+        if (g.accumulate) v += C[idx];
+        return v;
+    };
+    if constexpr (FrB::PAIRED) {
+        // Blocks 2p and 2p+1 of an MC-layout B operand hold columns n and n+1 of the same lane: store them
+        // together so that a wave writes whole contiguous row segments.
+        const bool can_pair = (g.N % 2 == 0) && (reinterpret_cast<uintptr_t>(C) % (2 * sizeof(T)) == 0);
 #pragma unroll
-    for (int bn = 0; bn < NBN; ++bn) {
-        const int n = n0 + FrB::index_of(wn0, bn, jcol);
-        if (n >= g.N) continue;
-        const T bcol = g.bias_mode == 1 ? bias[n] : T(0);
+        for (int pr = 0; pr < NBN / 2; ++pr) {
+            const int n = n0 + FrB::index_of(wn0, 2 * pr, jcol);  // even column; n + 1 belongs to block 2p+1
 #pragma unroll
-        for (int bm = 0; bm < NBM; ++bm) {
+            for (int bm = 0; bm < NBM; ++bm) {
 #pragma unroll
-            for (int e = 0; e < M::NACC; ++e) {
-                const int m = m0 + FrA::index_of(wm0, bm, M::acc_row(e, lane));
-                if (m >= g.M) continue;
-                T v = acc[bm][bn][e] + bcol;
-                if (g.bias_mode == 2) v += bias[m];
-                if (g.relu) v = v > T(0) ? v : T(0);
-                const int64_t idx = static_cast<int64_t>(m) * g.N + n;
-                if (g.accumulate) v += C[idx];
-                C[idx] = v;
+                for (int e = 0; e < M::NACC; ++e) {
+                    const int m = m0 + FrA::index_of(wm0, bm, M::acc_row(e, lane));
+                    if (m >= g.M) continue;
+                    const int64_t idx = static_cast<int64_t>(m) * g.N + n;
+                    if (can_pair && n + 1 < g.N) {
+                        typename M::pair_t out;
+                        out[0] = finish(acc[bm][2 * pr][e], m, n, idx);
+                        out[1] = finish(acc[bm][2 * pr + 1][e], m, n + 1, idx + 1);
+                        *reinterpret_cast<typename M::pair_t *>(&C[idx]) = out;
+                    } else {
+                        if (n < g.N) C[idx] = finish(acc[bm][2 * pr][e], m, n, idx);
+                        if (n + 1 < g.N) C[idx + 1] = finish(acc[bm][2 * pr + 1][e], m, n + 1, idx + 1);
+                    }
+                }
+            }
+        }
+    } else {
+#pragma unroll
+        for (int bn = 0; bn < NBN; ++bn) {
+            const int n = n0 + FrB::index_of(wn0, bn, jcol);
+            if (n >= g.N) continue;
+#pragma unroll
+            for (int bm = 0; bm < NBM; ++bm) {
+#pragma unroll
+                for (int e = 0; e < M::NACC; ++e) {
+                    const int m = m0 + FrA::index_of(wm0, bm, M::acc_row(e, lane));
+                    if (m >= g.M) continue;
+                    const int64_t idx = static_cast<int64_t>(m) * g.N + n;
+                    C[idx] = finish(acc[bm][bn][e], m, n, idx);
+                }
             }
         }
     }
