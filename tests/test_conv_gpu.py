@@ -1,0 +1,121 @@
+"""GPU parity tests for ttamd_conv2d_forward / ttamd_conv2d_backward through the C ABI, against the CPU
+oracle (im2col + the reference GEMM order) and the reference tests' own naive loop and data patterns
+(tests/test_conv.cpp:29-143).  Float tolerance: max relative error <= 1e-4 (f32) / 1e-12 (f64); exact for the
+integer dtypes and for integer-valued float data.
+"""
+import numpy as np
+import pytest
+
+from helpers import ALL_NON_BOOL, max_rel_error, tol_of
+
+pytestmark = pytest.mark.gpu
+
+
+def dev(tt, a):
+    return tt.Tensor.from_numpy(a)
+
+
+@pytest.mark.parametrize("dtype", ALL_NON_BOOL)
+@pytest.mark.parametrize("S,P", [(1, 0), (2, 1)])
+def test_forward_reference_pattern_exact(tt, oracle, dtype, S, P):
+    # tests/test_conv.cpp:99-143: B4, C3 -> 128, 64x64, k3, data i % 10 (exact in every dtype; u8/i16 wrap)
+    Bn, Cc, O, H, W, k = 4, 3, 128, 64, 64, 3
+    x = (np.arange(Bn * Cc * H * W) % 10).astype(dtype).reshape(Bn, Cc, H, W)
+    w = (np.arange(O * Cc * k * k) % 10).astype(dtype).reshape(O, Cc, k, k)
+    got = tt.conv2d(dev(tt, x), dev(tt, w), None, S, P).to_numpy()
+    want = oracle.conv2d_forward(x, w, None, S, P)
+    assert got.shape == want.shape
+    assert np.array_equal(got, want)
+    if dtype in (np.float32, np.uint8):
+        assert np.array_equal(want[:1], oracle.conv2d_naive(x[:1], w, S, P))  # the reference test's own oracle
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+@pytest.mark.parametrize("geom", [
+    # B, C, O, H, W, k, S, P
+    (2, 5, 7, 9, 11, 3, 1, 1),
+    (3, 4, 70, 13, 10, 5, 2, 2),
+    (2, 3, 6, 8, 8, 1, 1, 0),
+    (1, 8, 16, 17, 19, 3, 3, 1),
+    (2, 2, 3, 6, 7, 2, 2, 0),
+    (2, 16, 64, 12, 12, 3, 1, 1),
+])
+def test_forward_backward_random(tt, oracle, dtype, geom):
+    Bn, Cc, O, H, W, k, S, P = geom
+    rng = np.random.default_rng(sum(geom))
+    x = rng.normal(0, 0.5, (Bn, Cc, H, W)).astype(dtype)
+    w = rng.normal(0, 0.5, (O, Cc, k, k)).astype(dtype)
+    b = rng.normal(0, 0.5, (O,)).astype(dtype)
+    tol = tol_of(dtype)
+    out = tt.conv2d(dev(tt, x), dev(tt, w), dev(tt, b), S, P).to_numpy()
+    want = oracle.conv2d_forward(x, w, b, S, P)
+    assert max_rel_error(out, want) <= tol
+    g = rng.normal(0, 1, want.shape).astype(dtype)
+    gx, gw, gb = tt.conv2d_backward(dev(tt, g), dev(tt, x), dev(tt, w), dev(tt, b), S, P)
+    wx, ww, wb = oracle.conv2d_backward(g, x, w, True, S, P)
+    assert max_rel_error(gx.to_numpy(), wx) <= tol
+    assert max_rel_error(gw.to_numpy(), ww) <= tol
+    assert max_rel_error(gb.to_numpy(), wb) <= tol
+    # without a bias the third gradient is absent, as in the reference's optional
+    gx2, gw2, gb2 = tt.conv2d_backward(dev(tt, g), dev(tt, x), dev(tt, w), None, S, P)
+    assert gb2 is None and np.array_equal(gx2.to_numpy(), gx.to_numpy()) and np.array_equal(gw2.to_numpy(), gw.to_numpy())
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+def test_backward_exact_on_integer_data_and_adjoints(tt, oracle, dtype):
+    rng = np.random.default_rng(8)
+    Bn, Cc, O, H, W, k, S, P = 3, 4, 5, 9, 8, 3, 2, 1
+    x = rng.integers(-3, 4, (Bn, Cc, H, W)).astype(dtype)
+    w = rng.integers(-3, 4, (O, Cc, k, k)).astype(dtype)
+    out = tt.conv2d(dev(tt, x), dev(tt, w), None, S, P).to_numpy()
+    assert np.array_equal(out, oracle.conv2d_forward(x, w, None, S, P))
+    g = rng.integers(-3, 4, out.shape).astype(dtype)
+    gx, gw, gb = tt.conv2d_backward(dev(tt, g), dev(tt, x), dev(tt, w), dev(tt, np.zeros(O, dtype)), S, P)
+    wx, ww, wb = oracle.conv2d_backward(g, x, w, True, S, P)
+    assert np.array_equal(gx.to_numpy(), wx) and np.array_equal(gw.to_numpy(), ww) and np.array_equal(gb.to_numpy(), wb)
+    # adjoint identities <g, conv(x,w)> = <gx, x> = <gw, w>
+    lhs = np.sum(g.astype(np.float64) * out)
+    assert lhs == np.sum(gx.to_numpy().astype(np.float64) * x) == np.sum(gw.to_numpy().astype(np.float64) * w)
+
+
+def test_config4_conv_forward_backward(tt, oracle):
+    # BASELINE config 4: input [64,32,28,28], weight [64,32,3,3], stride 1, padding 1, normal(0, 0.1) from a seed.
+    x = oracle.Generator(0).normal(0.0, 0.1, (64, 32, 28, 28))
+    w = oracle.Generator(1).normal(0.0, 0.1, (64, 32, 3, 3))
+    tx, tw = dev(tt, x), dev(tt, w)
+    out = tt.conv2d(tx, tw, None, 1, 1).to_numpy()
+    want = oracle.conv2d_forward(x, w, None, 1, 1)
+    assert out.shape == (64, 64, 28, 28)
+    assert max_rel_error(out, want) <= 1e-4
+    # backward with g = ones (what backward() seeds) and with a random g
+    for g in (np.ones_like(want), oracle.Generator(2).uniform_real(-1, 1, want.shape)):
+        gx, gw, _ = tt.conv2d_backward(dev(tt, g), tx, tw, None, 1, 1)
+        wx, ww, _ = oracle.conv2d_backward(g, x, w, False, 1, 1)
+        assert max_rel_error(gx.to_numpy(), wx) <= 1e-4
+        assert max_rel_error(gw.to_numpy(), ww) <= 1e-4
+        # adjoint identity at full size, in f64
+        lhs = np.sum(g.astype(np.float64) * out)
+        assert abs(lhs - np.sum(gx.to_numpy().astype(np.float64) * x)) <= 1e-4 * abs(lhs)
+        assert abs(lhs - np.sum(gw.to_numpy().astype(np.float64) * w)) <= 1e-4 * abs(lhs)
+
+
+def test_strided_input_view_and_errors(tt, oracle):
+    rng = np.random.default_rng(3)
+    xs = rng.integers(-3, 4, (2, 9, 8, 4)).astype(np.float32)  # stored NHWC
+    x = np.ascontiguousarray(xs.transpose(0, 3, 1, 2))         # logical NCHW
+    w = rng.integers(-3, 4, (6, 4, 3, 3)).astype(np.float32)
+    tx = dev(tt, xs).permute(0, 3, 1, 2)
+    assert not tx.is_contiguous()
+    got = tt.conv2d(tx, dev(tt, w), None, 1, 1).to_numpy()
+    assert np.array_equal(got, oracle.conv2d_forward(x, w, None, 1, 1))
+    # a permuted weight is made dense by the adapter, as the reference's reshape does
+    wt = dev(tt, np.ascontiguousarray(w.transpose(1, 0, 2, 3))).permute(1, 0, 2, 3)
+    assert np.array_equal(tt.conv2d(tx, wt, None, 1, 1).to_numpy(), got)
+    with pytest.raises(tt.TTException):
+        tt.conv2d(dev(tt, x), dev(tt, rng.random((6, 5, 3, 3)).astype(np.float32)))  # channel mismatch
+    with pytest.raises(tt.TTException):
+        tt.conv2d(dev(tt, x), dev(tt, rng.random((6, 4, 3, 2)).astype(np.float32)))  # non-square kernel
+    with pytest.raises(tt.TTException):
+        tt.conv2d(dev(tt, x), dev(tt, w), None, 0, 0)                                  # stride 0
+    with pytest.raises(tt.TTException):
+        tt.conv2d(dev(tt, x[:, :, :2, :2]), dev(tt, w), None, 1, 0)                    # kernel larger than input

@@ -1,19 +1,724 @@
-// conv.hip — conv2d forward/backward as implicit GEMM (placeholder entry points while the kernels land).
-#include "common.h"
-using namespace ttamd;
-extern "C" {
-ttamd_status ttamd_conv2d_forward(int, ttamd_dtype, const ttamd_view4 *, const ttamd_view4 *, const void *, void *, int,
-                                  int, int, int, int, int, int, int, void *) {
-    set_error("conv2d_forward: not implemented yet");
-    return TTAMD_ERR_INVALID_ARGUMENT;
+// conv.hip — conv2d forward / backward as implicit GEMM on the matrix cores (gfx950).
+//
+// Stands where BackendBase::conv2d / conv2d_backward do (tinytensor/tensor/backend_base.h:269-284).  The
+// reference lowers each image to an explicit im2col matrix and runs one small GEMM per image
+// (tinytensor/tensor/backend/cpu/conv.cpp:108-128, 208-272; index maps cpu/kernel/conv.hpp:12-118).
+// Here the same three products run as batched GEMMs whose "column matrix" operand is never
+// materialised: a gather stager computes the im2col address of every element it fetches and lets the
+// buffer load return zero for padding.  With kk = (c, p, q) and n = (h, w):
+//
+//   forward      out[b][o][n]  = sum_kk  W[o][kk]      * x[b][c][S h + p - P][S w + q - P]     (+ bias[o])
+//   grad_weight  gW[o][kk]     = sum_b sum_n g[b][o][n] * x[b][c][S h + p - P][S w + q - P]
+//   grad_input   gX[b][c][y][x] = sum_(o,p,q) W[o][c][p][q] * g[b][o][(y+P-p)/S][(x+P-q)/S]   (when divisible, in range)
+//
+// grad_input is the gather form of the reference's col2im scatter-add (conv.hpp:83-118): every output
+// element is owned by one lane, so there is no write race and the result is deterministic.
+// grad_weight reduces over the batch: one workgroup column per group of images accumulates in registers,
+// partial tiles go to the caller's workspace and are summed in image order (the reference's order,
+// conv.cpp:239-244).  Integer dtypes (forward only; autograd never differentiates them) use a direct
+// vector-ALU kernel with wrap-around arithmetic.
+#include "mfma_core.h"
+
+namespace ttamd {
+namespace {
+
+using namespace mfma;
+
+// Exact unsigned division by a runtime-invariant divisor (Granlund & Montgomery): q = x / d for all 32-bit x.
+struct FastDiv {
+    uint32_t mul, sh1, sh2, d;
+    __device__ __forceinline__ uint32_t div(uint32_t x) const {
+        const uint32_t t = __umulhi(mul, x);
+        return (t + ((x - t) >> sh1)) >> sh2;
+    }
+    __device__ __forceinline__ void divmod(uint32_t x, uint32_t &q, uint32_t &r) const {
+        q = div(x);
+        r = x - q * d;
+    }
+};
+
+FastDiv make_fastdiv(uint32_t d) {
+    FastDiv f{};
+    f.d = d;
+    uint32_t L = 0;
+    while ((1ull << L) < d) ++L;
+    f.mul = static_cast<uint32_t>(((1ull << 32) * ((1ull << L) - d)) / d + 1);
+    f.sh1 = L < 1 ? L : 1;
+    f.sh2 = L > 0 ? L - 1 : 0;
+    return f;
 }
-ttamd_status ttamd_conv2d_backward_workspace(ttamd_dtype, int, int, int, int, int, int, int, int, size_t *bytes) {
-    if (bytes) *bytes = 0;
+
+struct ConvGeom {
+    int B, C, H, W, O, k, S, P, Ho, Wo;
+    int64_t xs_b;              // input batch stride (elements)
+    int32_t xs_c, xs_h, xs_w;  // input channel / row / column strides (elements)
+    int64_t w_so;              // weight stride of the output channel; (c,p,q) are dense behind it
+    FastDiv d_kk, d_k, d_Wo, d_W, d_S;
+};
+
+// ---------------------------------------------------------------------------------------------
+// B operand of the forward product: Xu[kk][n] gathered from image b.  MC layout (n contiguous), one
+// element per load.  A lane keeps one output position n for the whole kernel; the kk of a pass is
+// wave-uniform, so its (c, p, q) decode runs on the scalar unit.
+template <typename T, int ROWS, int BK>
+struct Im2colStager : TileLayout<T, ROWS, BK, false> {
+    using L = TileLayout<T, ROWS, BK, false>;
+    static constexpr int LPP = kThreads / ROWS;  // k lines per pass
+    static constexpr int P = BK / LPP;
+    static_assert(ROWS % 64 == 0 && BK % LPP == 0, "a wave must share its k line");
+    T reg[P];
+    __amdgpu_buffer_rsrc_t rsrc;
+    const ConvGeom *g;
+    int n_local, line0, k_next, K;
+    int ih0, iw0;       // input coordinates of tap (0,0) for this lane's output position
+    int32_t base_b;     // byte offset of (ih0, iw0) inside the image (may be negative under padding)
+    bool n_ok;
+
+    __device__ __forceinline__ void init(const ConvGeom &geo, const T *image, int64_t image_bytes, int tid, int n0) {
+        g = &geo;
+        rsrc = make_rsrc(image, image_bytes);
+        n_local = tid % ROWS;
+        line0 = __builtin_amdgcn_readfirstlane(tid / ROWS);
+        k_next = 0;
+        K = geo.C * geo.k * geo.k;
+        const int n = n0 + n_local;
+        n_ok = n < geo.Ho * geo.Wo;
+        uint32_t h, w;
+        geo.d_Wo.divmod(static_cast<uint32_t>(n_ok ? n : 0), h, w);
+        ih0 = geo.S * static_cast<int>(h) - geo.P;
+        iw0 = geo.S * static_cast<int>(w) - geo.P;
+        base_b = (ih0 * geo.xs_h + iw0 * geo.xs_w) * static_cast<int32_t>(sizeof(T));
+    }
+
+    template <bool MASK>
+    __device__ __forceinline__ void load(int /*k_left*/) {
+#pragma unroll
+        for (int p = 0; p < P; ++p) {
+            const int kk = k_next + p * LPP + line0;  // wave-uniform
+            uint32_t c, r, pp, q;
+            g->d_kk.divmod(static_cast<uint32_t>(kk), c, r);
+            g->d_k.divmod(r, pp, q);
+            const int32_t koff = (static_cast<int32_t>(c) * g->xs_c + static_cast<int32_t>(pp) * g->xs_h +
+                                  static_cast<int32_t>(q) * g->xs_w) * static_cast<int32_t>(sizeof(T));
+            const int ih = ih0 + static_cast<int>(pp), iw = iw0 + static_cast<int>(q);
+            const bool ok = n_ok && kk < K && static_cast<unsigned>(ih) < static_cast<unsigned>(g->H) &&
+                            static_cast<unsigned>(iw) < static_cast<unsigned>(g->W);
+            reg[p] = Vec<T, 1>::load(rsrc, ok ? static_cast<uint32_t>(base_b + koff) : kOob);
+        }
+        k_next += BK;
+    }
+
+    __device__ __forceinline__ void store(T *lds) const {
+#pragma unroll
+        for (int p = 0; p < P; ++p) lds[(p * LPP + line0) * L::LD + n_local] = reg[p];
+    }
+};
+
+// ---------------------------------------------------------------------------------------------
+// B operand of grad_weight: XuT[n][j] with n = output position (the reduction index) and j = (c,p,q)
+// (the column index).  KC layout (n contiguous), one element per load.  The j of each pass is fixed for
+// the whole kernel and decoded once; the n of a lane advances by BK per tile.
+template <typename T, int ROWS, int BK>
+struct Im2colTStager : TileLayout<T, ROWS, BK, true> {
+    using L = TileLayout<T, ROWS, BK, true>;
+    static constexpr int RPP = kThreads / BK;  // j rows per pass
+    static constexpr int P = ROWS / RPP;
+    static_assert(ROWS % RPP == 0, "tile must split evenly");
+    T reg[P];
+    __amdgpu_buffer_rsrc_t rsrc;
+    const ConvGeom *g;
+    int32_t joff[P];  // byte offset of tap (c, p - P, q - P)
+    int16_t dp[P], dq[P];
+    bool j_ok[P];
+    int k_local, row0, k_next, HoWo;
+
+    __device__ __forceinline__ void init(const ConvGeom &geo, int tid, int j0) {
+        g = &geo;
+        k_local = tid % BK;
+        row0 = tid / BK;
+        HoWo = geo.Ho * geo.Wo;
+        const int J = geo.C * geo.k * geo.k;
+#pragma unroll
+        for (int p = 0; p < P; ++p) {
+            const int j = j0 + p * RPP + row0;
+            j_ok[p] = j < J;
+            uint32_t c, r, pp, q;
+            geo.d_kk.divmod(static_cast<uint32_t>(j_ok[p] ? j : 0), c, r);
+            geo.d_k.divmod(r, pp, q);
+            dp[p] = static_cast<int16_t>(static_cast<int>(pp) - geo.P);
+            dq[p] = static_cast<int16_t>(static_cast<int>(q) - geo.P);
+            joff[p] = (static_cast<int32_t>(c) * geo.xs_c + dp[p] * geo.xs_h + dq[p] * geo.xs_w) *
+                      static_cast<int32_t>(sizeof(T));
+        }
+    }
+
+    // Points the stager at image `image` and restarts the reduction index.
+    __device__ __forceinline__ void set_image(const T *image, int64_t image_bytes) {
+        rsrc = make_rsrc(image, image_bytes);
+        k_next = 0;
+    }
+
+    template <bool MASK>
+    __device__ __forceinline__ void load(int /*k_left*/) {
+        const int n = k_next + k_local;
+        const bool n_ok = n < HoWo;
+        uint32_t h, w;
+        g->d_Wo.divmod(static_cast<uint32_t>(n_ok ? n : 0), h, w);
+        const int ih0 = g->S * static_cast<int>(h), iw0 = g->S * static_cast<int>(w);
+        const int32_t base_b = (ih0 * g->xs_h + iw0 * g->xs_w) * static_cast<int32_t>(sizeof(T));
+#pragma unroll
+        for (int p = 0; p < P; ++p) {
+            const int ih = ih0 + dp[p], iw = iw0 + dq[p];
+            const bool ok = n_ok && j_ok[p] && static_cast<unsigned>(ih) < static_cast<unsigned>(g->H) &&
+                            static_cast<unsigned>(iw) < static_cast<unsigned>(g->W);
+            reg[p] = Vec<T, 1>::load(rsrc, ok ? static_cast<uint32_t>(base_b + joff[p]) : kOob);
+        }
+        k_next += BK;
+    }
+
+    __device__ __forceinline__ void store(T *lds) const {
+#pragma unroll
+        for (int p = 0; p < P; ++p) lds[(p * RPP + row0) * L::LD + k_local] = reg[p];
+    }
+};
+
+// ---------------------------------------------------------------------------------------------
+// A operand of grad_input: Wt[c][kk] = W[o][c][p][q] with kk = (o,p,q).  KC layout, one element per load;
+// a lane keeps one kk per tile (decoded per tile), the channel row varies per pass.
+template <typename T, int ROWS, int BK>
+struct WeightTStager : TileLayout<T, ROWS, BK, true> {
+    using L = TileLayout<T, ROWS, BK, true>;
+    static constexpr int RPP = kThreads / BK;
+    static constexpr int P = ROWS / RPP;
+    T reg[P];
+    __amdgpu_buffer_rsrc_t rsrc;
+    const ConvGeom *g;
+    int k_local, row0, k_next, K, c0, kk2;
+
+    __device__ __forceinline__ void init(const ConvGeom &geo, const T *weight, int64_t weight_bytes, int tid, int c0_) {
+        g = &geo;
+        rsrc = make_rsrc(weight, weight_bytes);
+        k_local = tid % BK;
+        row0 = tid / BK;
+        k_next = 0;
+        kk2 = geo.k * geo.k;
+        K = geo.O * kk2;
+        c0 = c0_;
+    }
+
+    template <bool MASK>
+    __device__ __forceinline__ void load(int /*k_left*/) {
+        const int kk = k_next + k_local;
+        const bool k_ok = kk < K;
+        uint32_t o, r;
+        g->d_kk.divmod(static_cast<uint32_t>(k_ok ? kk : 0), o, r);
+        const int64_t koff = static_cast<int64_t>(o) * g->w_so + r;  // elements
+#pragma unroll
+        for (int p = 0; p < P; ++p) {
+            const int c = c0 + p * RPP + row0;
+            const bool ok = k_ok && c < g->C;
+            const int64_t off = (koff + static_cast<int64_t>(c) * kk2) * static_cast<int64_t>(sizeof(T));
+            reg[p] = Vec<T, 1>::load(rsrc, ok ? static_cast<uint32_t>(off) : kOob);
+        }
+        k_next += BK;
+    }
+
+    __device__ __forceinline__ void store(T *lds) const {
+#pragma unroll
+        for (int p = 0; p < P; ++p) lds[(p * RPP + row0) * L::LD + k_local] = reg[p];
+    }
+};
+
+// B operand of grad_input: G[kk][n] = g[b][o][(y+P-p)/S][(x+P-q)/S], kk = (o,p,q), n = (y,x).  MC layout;
+// the lane's input position is fixed, kk is wave-uniform per pass.
+template <typename T, int ROWS, int BK>
+struct DgradStager : TileLayout<T, ROWS, BK, false> {
+    using L = TileLayout<T, ROWS, BK, false>;
+    static constexpr int LPP = kThreads / ROWS;
+    static constexpr int P = BK / LPP;
+    static_assert(ROWS % 64 == 0 && BK % LPP == 0, "a wave must share its k line");
+    T reg[P];
+    __amdgpu_buffer_rsrc_t rsrc;
+    const ConvGeom *g;
+    int n_local, line0, k_next, K, HoWo;
+    int yP, xP;  // y + P, x + P for this lane's input position
+    bool n_ok;
+
+    __device__ __forceinline__ void init(const ConvGeom &geo, const T *gout_image, int64_t bytes, int tid, int n0) {
+        g = &geo;
+        rsrc = make_rsrc(gout_image, bytes);
+        n_local = tid % ROWS;
+        line0 = __builtin_amdgcn_readfirstlane(tid / ROWS);
+        k_next = 0;
+        HoWo = geo.Ho * geo.Wo;
+        K = geo.O * geo.k * geo.k;
+        const int n = n0 + n_local;
+        n_ok = n < geo.H * geo.W;
+        uint32_t y, x;
+        geo.d_W.divmod(static_cast<uint32_t>(n_ok ? n : 0), y, x);
+        yP = static_cast<int>(y) + geo.P;
+        xP = static_cast<int>(x) + geo.P;
+    }
+
+    template <bool MASK>
+    __device__ __forceinline__ void load(int /*k_left*/) {
+#pragma unroll
+        for (int p = 0; p < P; ++p) {
+            const int kk = k_next + p * LPP + line0;  // wave-uniform
+            uint32_t o, r, pp, q;
+            g->d_kk.divmod(static_cast<uint32_t>(kk), o, r);
+            g->d_k.divmod(r, pp, q);
+            const int ty = yP - static_cast<int>(pp), tx = xP - static_cast<int>(q);
+            bool ok = n_ok && kk < K && ty >= 0 && tx >= 0;
+            uint32_t oh, rh, ow, rw;
+            g->d_S.divmod(static_cast<uint32_t>(ok ? ty : 0), oh, rh);
+            g->d_S.divmod(static_cast<uint32_t>(ok ? tx : 0), ow, rw);
+            ok = ok && rh == 0 && rw == 0 && static_cast<int>(oh) < g->Ho && static_cast<int>(ow) < g->Wo;
+            const uint32_t off = (o * static_cast<uint32_t>(HoWo) + oh * static_cast<uint32_t>(g->Wo) + ow) *
+                                 static_cast<uint32_t>(sizeof(T));
+            reg[p] = Vec<T, 1>::load(rsrc, ok ? off : kOob);
+        }
+        k_next += BK;
+    }
+
+    __device__ __forceinline__ void store(T *lds) const {
+#pragma unroll
+        for (int p = 0; p < P; ++p) lds[(p * LPP + line0) * L::LD + n_local] = reg[p];
+    }
+};
+
+// ---------------------------------------------------------------------------------------------
+// forward: M = O, N = Ho*Wo, K = C*k*k, one GEMM per image.
+template <typename T, int BM, int BN, int BK, int A_VEC>
+__global__ void __launch_bounds__(kThreads, 2)
+conv_fwd_kernel(ConvGeom geo, const T *x, const T *w, const T *bias, T *out, int64_t image_bytes, int tiles_m, int tiles_n) {
+    using StA = Stager<T, BM, BK, true, A_VEC>;
+    using StB = Im2colStager<T, BN, BK>;
+    using Engine = TileEngine<T, BM, BN, BK, 2, 2, StA, StB>;
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
+    T *const smem = reinterpret_cast<T *>(smem_raw);
+    const int tid = threadIdx.x;
+    int b, tm, tn;
+    decode_tile(remap_xcd(blockIdx.x, gridDim.x), tiles_m, tiles_n, b, tm, tn);
+    const int m0 = tm * BM, n0 = tn * BN;
+    const int M_ = geo.O, N_ = geo.Ho * geo.Wo, K = geo.C * geo.k * geo.k;
+    StA sa;
+    StB sb;
+    sa.init(w + static_cast<int64_t>(m0) * geo.w_so, tid, M_ - m0, geo.w_so, 1, K);
+    sb.init(geo, x + static_cast<int64_t>(b) * geo.xs_b, image_bytes, tid, n0);
+    Engine eng;
+    eng.init(tid);
+    eng.run(sa, sb, smem, K, false);
+    store_tile_dense<T>(eng, out + static_cast<int64_t>(b) * M_ * N_, M_, N_, m0, n0, bias, bias ? 2 : 0, 0, 0);
+}
+
+// grad_input: M = C, N = H*W, K = O*k*k, one GEMM per image.
+template <typename T, int BM, int BN, int BK>
+__global__ void __launch_bounds__(kThreads, 2)
+conv_dgrad_kernel(ConvGeom geo, const T *gout, const T *w, T *gin, int64_t weight_bytes, int tiles_m, int tiles_n) {
+    using StA = WeightTStager<T, BM, BK>;
+    using StB = DgradStager<T, BN, BK>;
+    using Engine = TileEngine<T, BM, BN, BK, 2, 2, StA, StB>;
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
+    T *const smem = reinterpret_cast<T *>(smem_raw);
+    const int tid = threadIdx.x;
+    int b, tm, tn;
+    decode_tile(remap_xcd(blockIdx.x, gridDim.x), tiles_m, tiles_n, b, tm, tn);
+    const int m0 = tm * BM, n0 = tn * BN;
+    const int M_ = geo.C, N_ = geo.H * geo.W, K = geo.O * geo.k * geo.k;
+    const int64_t g_image = static_cast<int64_t>(geo.O) * geo.Ho * geo.Wo;
+    StA sa;
+    StB sb;
+    sa.init(geo, w, weight_bytes, tid, m0);
+    sb.init(geo, gout + static_cast<int64_t>(b) * g_image, g_image * static_cast<int64_t>(sizeof(T)), tid, n0);
+    Engine eng;
+    eng.init(tid);
+    eng.run(sa, sb, smem, K, false);
+    store_tile_dense<T>(eng, gin + static_cast<int64_t>(b) * M_ * N_, M_, N_, m0, n0, static_cast<const T *>(nullptr), 0, 0, 0);
+}
+
+// grad_weight: M = O, N = C*k*k, K = Ho*Wo per image; workgroup column `split` accumulates images
+// [split*group, min(B, (split+1)*group)) in registers and writes one partial tile.
+template <typename T, int BM, int BN, int BK, int A_VEC>
+__global__ void __launch_bounds__(kThreads, 2)
+conv_wgrad_kernel(ConvGeom geo, const T *gout, const T *x, T *partial, int64_t image_bytes, int group, int tiles_m, int tiles_n) {
+    using StA = Stager<T, BM, BK, true, A_VEC>;
+    using StB = Im2colTStager<T, BN, BK>;
+    using Engine = TileEngine<T, BM, BN, BK, 2, 2, StA, StB>;
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
+    T *const smem = reinterpret_cast<T *>(smem_raw);
+    const int tid = threadIdx.x;
+    int split, tm, tn;
+    decode_tile(remap_xcd(blockIdx.x, gridDim.x), tiles_m, tiles_n, split, tm, tn);
+    const int m0 = tm * BM, n0 = tn * BN;
+    const int M_ = geo.O, N_ = geo.C * geo.k * geo.k, K = geo.Ho * geo.Wo;
+    const int64_t g_image = static_cast<int64_t>(geo.O) * K;
+    StA sa;
+    StB sb;
+    sb.init(geo, tid, n0);
+    Engine eng;
+    eng.init(tid);
+    const int b_end = (split + 1) * group < geo.B ? (split + 1) * group : geo.B;
+    for (int b = split * group; b < b_end; ++b) {
+        sa.init(gout + b * g_image + static_cast<int64_t>(m0) * K, tid, M_ - m0, K, 1, K);
+        sb.set_image(x + static_cast<int64_t>(b) * geo.xs_b, image_bytes);
+        eng.run(sa, sb, smem, K, false);
+        __syncthreads();  // the next image's prologue overwrites LDS buffer 0
+    }
+    store_tile_dense<T>(eng, partial + static_cast<int64_t>(split) * M_ * N_, M_, N_, m0, n0, static_cast<const T *>(nullptr), 0, 0, 0);
+}
+
+// out[i] = sum over splits of partial[s][i], in increasing s (image order).
+template <typename T>
+__global__ void __launch_bounds__(256) reduce_splits_kernel(const T *__restrict__ partial, T *__restrict__ out, int64_t n, int splits) {
+    const int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    T acc = partial[i];
+    for (int s = 1; s < splits; ++s) acc += partial[static_cast<int64_t>(s) * n + i];
+    out[i] = acc;
+}
+
+// grad_bias[o] = sum over batch and space of grad_out[b][o][.] (cpu/conv.cpp:289).  One workgroup per channel.
+template <typename T>
+__global__ void __launch_bounds__(256) bias_grad_kernel(const T *__restrict__ gout, T *__restrict__ gb, int B, int O, int HoWo) {
+    __shared__ T red[256];
+    const int o = blockIdx.x;
+    T acc = T(0);
+    for (int b = 0; b < B; ++b) {
+        const T *p = gout + (static_cast<int64_t>(b) * O + o) * HoWo;
+        for (int i = threadIdx.x; i < HoWo; i += 256) acc += p[i];
+    }
+    red[threadIdx.x] = acc;
+    __syncthreads();
+    for (int s = 128; s > 0; s >>= 1) {
+        if (static_cast<int>(threadIdx.x) < s) red[threadIdx.x] += red[threadIdx.x + s];
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) gb[o] = red[0];
+}
+
+// Direct forward for the integer dtypes: one lane per output element, wrap-around arithmetic in unsigned
+// registers (same value modulo 2^n as the reference's SIMD lanes, cpu/kernel/simd.h:120-127).
+template <typename T, typename Acc>
+__global__ void __launch_bounds__(256)
+conv_fwd_direct_kernel(ConvGeom geo, const T *__restrict__ x, const T *__restrict__ w, const T *__restrict__ bias, T *__restrict__ out, int64_t total) {
+    const int64_t idx = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (idx >= total) return;
+    const int HoWo = geo.Ho * geo.Wo;
+    const int n = static_cast<int>(idx % HoWo);
+    const int o = static_cast<int>((idx / HoWo) % geo.O);
+    const int b = static_cast<int>(idx / (static_cast<int64_t>(HoWo) * geo.O));
+    const int h = n / geo.Wo, ww = n % geo.Wo;
+    Acc acc = Acc(0);
+    for (int c = 0; c < geo.C; ++c)
+        for (int p = 0; p < geo.k; ++p)
+            for (int q = 0; q < geo.k; ++q) {
+                const int ih = geo.S * h + p - geo.P, iw = geo.S * ww + q - geo.P;
+                if (ih < 0 || iw < 0 || ih >= geo.H || iw >= geo.W) continue;
+                const Acc xv = static_cast<Acc>(x[b * geo.xs_b + static_cast<int64_t>(c) * geo.xs_c + static_cast<int64_t>(ih) * geo.xs_h + static_cast<int64_t>(iw) * geo.xs_w]);
+                const Acc wv = static_cast<Acc>(w[o * geo.w_so + (c * geo.k + p) * geo.k + q]);
+                acc += xv * wv;
+            }
+    T v = static_cast<T>(acc);
+    if (bias) v = static_cast<T>(v + bias[o]);
+    out[idx] = v;
+}
+
+// ---------------------------------------------------------------------------------------------
+// host side
+
+struct ConvPlan {
+    ConvGeom geo;
+    const void *x;
+    const void *w;
+    int64_t image_bytes;   // bytes reachable from an image's first element
+    int64_t weight_bytes;  // bytes reachable from the weight's first element
+};
+
+ttamd_status make_plan(const char *who, ttamd_dtype dtype, const ttamd_view4 *input, const ttamd_view4 *weight, int B, int C,
+                       int H, int W, int O, int k, int stride, int padding, ConvPlan *plan) {
+    if (dtype == TTAMD_BOOL || dtype_size(dtype) == 0 || dtype < TTAMD_BOOL || dtype > TTAMD_F64) {
+        set_error("%s does not support dtype code %d", who, static_cast<int>(dtype));
+        return TTAMD_ERR_UNSUPPORTED_DTYPE;
+    }
+    if (!input || !weight) {
+        set_error("%s: NULL operand view", who);
+        return TTAMD_ERR_INVALID_ARGUMENT;
+    }
+    if (B < 0 || C <= 0 || H <= 0 || W <= 0 || O <= 0 || k <= 0 || stride <= 0 || padding < 0) {
+        set_error("%s: invalid geometry (B=%d C=%d H=%d W=%d O=%d k=%d stride=%d padding=%d)", who, B, C, H, W, O, k,
+                  stride, padding);
+        return TTAMD_ERR_INVALID_ARGUMENT;
+    }
+    const int Ho = (H + 2 * padding - k) / stride + 1, Wo = (W + 2 * padding - k) / stride + 1;
+    if (H + 2 * padding < k || W + 2 * padding < k || Ho <= 0 || Wo <= 0) {
+        set_error("%s: kernel %d does not fit the padded input %dx%d", who, k, H + 2 * padding, W + 2 * padding);
+        return TTAMD_ERR_INVALID_ARGUMENT;
+    }
+    for (int i = 0; i < 4; ++i) {
+        if (input->stride[i] < 0 || weight->stride[i] < 0) {
+            set_error("%s: negative strides are not supported", who);
+            return TTAMD_ERR_INVALID_ARGUMENT;
+        }
+    }
+    if (input->offset < 0 || weight->offset < 0) {
+        set_error("%s: negative view offset", who);
+        return TTAMD_ERR_INVALID_ARGUMENT;
+    }
+    // The weight is used as the matrix [O, C*k*k] (cpu/conv.cpp:69 reshapes it, cloning a non-dense view):
+    // its (c,p,q) dimensions must already be dense; the adapter calls contiguous() otherwise.
+    if ((C > 1 && weight->stride[1] != static_cast<int64_t>(k) * k) || (k > 1 && (weight->stride[2] != k || weight->stride[3] != 1))) {
+        set_error("%s: weight dimensions (C,k,k) must be dense; make the weight contiguous first", who);
+        return TTAMD_ERR_INVALID_ARGUMENT;
+    }
+    const size_t esz = dtype_size(dtype);
+    const int64_t x_reach = (static_cast<int64_t>(C - 1) * input->stride[1] + static_cast<int64_t>(H - 1) * input->stride[2] +
+                             static_cast<int64_t>(W - 1) * input->stride[3] + 1) * static_cast<int64_t>(esz);
+    const int64_t w_reach = (static_cast<int64_t>(O - 1) * weight->stride[0] + static_cast<int64_t>(C) * k * k) * static_cast<int64_t>(esz);
+    const int64_t limit = 0x7fffffffLL;
+    if (x_reach >= limit || w_reach >= limit || static_cast<int64_t>(O) * Ho * Wo * static_cast<int64_t>(esz) >= limit ||
+        static_cast<int64_t>(C) * k * k >= (1 << 24) || static_cast<int64_t>(O) * k * k >= (1 << 24) ||
+        static_cast<int64_t>(H) * W >= limit / 8 || input->stride[1] >= limit / 8 || input->stride[2] >= limit / 8 ||
+        input->stride[3] >= limit / 8) {
+        set_error("%s: one image or the weight exceeds the 2 GiB addressing range of the kernels", who);
+        return TTAMD_ERR_INVALID_ARGUMENT;
+    }
+    ConvGeom &g = plan->geo;
+    g = ConvGeom{};
+    g.B = B; g.C = C; g.H = H; g.W = W; g.O = O; g.k = k; g.S = stride; g.P = padding; g.Ho = Ho; g.Wo = Wo;
+    g.xs_b = input->stride[0];
+    g.xs_c = static_cast<int32_t>(input->stride[1]);
+    g.xs_h = static_cast<int32_t>(input->stride[2]);
+    g.xs_w = static_cast<int32_t>(input->stride[3]);
+    g.w_so = weight->stride[0];
+    g.d_kk = make_fastdiv(static_cast<uint32_t>(k) * k);
+    g.d_k = make_fastdiv(static_cast<uint32_t>(k));
+    g.d_Wo = make_fastdiv(static_cast<uint32_t>(Wo));
+    g.d_W = make_fastdiv(static_cast<uint32_t>(W));
+    g.d_S = make_fastdiv(static_cast<uint32_t>(stride));
+    plan->x = static_cast<const char *>(input->data) + input->offset * static_cast<int64_t>(esz);
+    plan->w = static_cast<const char *>(weight->data) + weight->offset * static_cast<int64_t>(esz);
+    plan->image_bytes = x_reach;
+    plan->weight_bytes = w_reach;
     return TTAMD_OK;
 }
-ttamd_status ttamd_conv2d_backward(int, ttamd_dtype, const void *, const ttamd_view4 *, const ttamd_view4 *, void *,
-                                   void *, void *, int, int, int, int, int, int, int, int, void *, size_t, void *) {
-    set_error("conv2d_backward: not implemented yet");
-    return TTAMD_ERR_INVALID_ARGUMENT;
+
+template <class Kernel>
+ttamd_status set_lds(Kernel kernel, size_t lds_bytes) {
+    if (lds_bytes > 48 * 1024)
+        TTAMD_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                            static_cast<int>(lds_bytes)));
+    return TTAMD_OK;
 }
+
+template <typename T>
+struct ConvTiles {
+    static constexpr int BK = sizeof(T) == 4 ? 32 : 16;
+};
+
+// 16-byte loads of the weight / grad_out matrix need aligned rows.
+template <typename T>
+bool rows_vectorizable(const void *ptr, int64_t row_stride, int64_t image_stride) {
+    constexpr int VK = Mfma<T>::VK;
+    return reinterpret_cast<uintptr_t>(ptr) % 16 == 0 && row_stride % VK == 0 && image_stride % VK == 0;
 }
+
+template <typename T>
+ttamd_status forward_mfma(const ConvPlan &pl, const void *bias, void *out, hipStream_t st) {
+    constexpr int BK = ConvTiles<T>::BK, VK = Mfma<T>::VK;
+    const ConvGeom &g = pl.geo;
+    const int M_ = g.O, N_ = g.Ho * g.Wo;
+    const int tiles_m = (M_ + 63) / 64, tiles_n = (N_ + 63) / 64;
+    const int64_t blocks = static_cast<int64_t>(tiles_m) * tiles_n * g.B;
+    if (blocks > 0x7fffffff) {
+        set_error("conv2d: too many workgroups");
+        return TTAMD_ERR_INVALID_ARGUMENT;
+    }
+    const bool vec = rows_vectorizable<T>(pl.w, g.w_so, 0);
+    auto launch = [&](auto kernel, size_t lds) -> ttamd_status {
+        if (ttamd_status s = set_lds(kernel, lds)) return s;
+        kernel<<<dim3(static_cast<unsigned>(blocks)), dim3(kThreads), lds, st>>>(
+            g, static_cast<const T *>(pl.x), static_cast<const T *>(pl.w), static_cast<const T *>(bias), static_cast<T *>(out),
+            pl.image_bytes, tiles_m, tiles_n);
+        TTAMD_HIP_CHECK(hipGetLastError());
+        return TTAMD_OK;
+    };
+    if (vec) {
+        using E = TileEngine<T, 64, 64, BK, 2, 2, Stager<T, 64, BK, true, VK>, Im2colStager<T, 64, BK>>;
+        return launch(conv_fwd_kernel<T, 64, 64, BK, VK>, E::kLdsBytes);
+    }
+    using E = TileEngine<T, 64, 64, BK, 2, 2, Stager<T, 64, BK, true, 1>, Im2colStager<T, 64, BK>>;
+    return launch(conv_fwd_kernel<T, 64, 64, BK, 1>, E::kLdsBytes);
+}
+
+template <typename T, typename Acc>
+ttamd_status forward_direct(const ConvPlan &pl, const void *bias, void *out, hipStream_t st) {
+    const ConvGeom &g = pl.geo;
+    const int64_t total = static_cast<int64_t>(g.B) * g.O * g.Ho * g.Wo;
+    const int64_t blocks = (total + 255) / 256;
+    if (blocks > 0x7fffffff) {
+        set_error("conv2d: too many workgroups");
+        return TTAMD_ERR_INVALID_ARGUMENT;
+    }
+    conv_fwd_direct_kernel<T, Acc><<<dim3(static_cast<unsigned>(blocks)), dim3(256), 0, st>>>(
+        g, static_cast<const T *>(pl.x), static_cast<const T *>(pl.w), static_cast<const T *>(bias), static_cast<T *>(out), total);
+    TTAMD_HIP_CHECK(hipGetLastError());
+    return TTAMD_OK;
+}
+
+// Images per grad_weight split: one per image unless that would need more than 64 MiB of partial tiles.
+int wgrad_group(size_t esz, int B, int C, int O, int k) {
+    const int64_t tile_bytes = static_cast<int64_t>(O) * C * k * k * static_cast<int64_t>(esz);
+    const int64_t cap = 64LL << 20;
+    int64_t max_splits = cap / (tile_bytes > 0 ? tile_bytes : 1);
+    if (max_splits < 1) max_splits = 1;
+    if (max_splits >= B) return 1;
+    return static_cast<int>((B + max_splits - 1) / max_splits);
+}
+
+template <typename T>
+ttamd_status backward_mfma(const ConvPlan &pl, const void *gout, void *gin, void *gw, void *gb, void *ws, size_t ws_bytes,
+                           hipStream_t st) {
+    constexpr int BK = ConvTiles<T>::BK, VK = Mfma<T>::VK;
+    const ConvGeom &g = pl.geo;
+    const int HoWo = g.Ho * g.Wo;
+    // grad_input
+    {
+        const int M_ = g.C, N_ = g.H * g.W;
+        const int tiles_m = (M_ + 63) / 64, tiles_n = (N_ + 63) / 64;
+        const int64_t blocks = static_cast<int64_t>(tiles_m) * tiles_n * g.B;
+        if (blocks > 0x7fffffff) {
+            set_error("conv2d_backward: too many workgroups");
+            return TTAMD_ERR_INVALID_ARGUMENT;
+        }
+        using E = TileEngine<T, 64, 64, BK, 2, 2, WeightTStager<T, 64, BK>, DgradStager<T, 64, BK>>;
+        auto kernel = conv_dgrad_kernel<T, 64, 64, BK>;
+        if (ttamd_status s = set_lds(kernel, E::kLdsBytes)) return s;
+        kernel<<<dim3(static_cast<unsigned>(blocks)), dim3(kThreads), E::kLdsBytes, st>>>(
+            g, static_cast<const T *>(gout), static_cast<const T *>(pl.w), static_cast<T *>(gin), pl.weight_bytes, tiles_m, tiles_n);
+        TTAMD_HIP_CHECK(hipGetLastError());
+    }
+    // grad_weight
+    {
+        const int M_ = g.O, N_ = g.C * g.k * g.k;
+        const int group = wgrad_group(sizeof(T), g.B, g.C, g.O, g.k);
+        const int splits = (g.B + group - 1) / group;
+        const int64_t tile_elems = static_cast<int64_t>(M_) * N_;
+        T *partial = static_cast<T *>(gw);
+        if (splits > 1) {
+            if (!ws || ws_bytes < static_cast<size_t>(splits) * tile_elems * sizeof(T)) {
+                set_error("conv2d_backward: workspace of %zu bytes is smaller than the %zu bytes required", ws_bytes,
+                          static_cast<size_t>(splits) * tile_elems * sizeof(T));
+                return TTAMD_ERR_INVALID_ARGUMENT;
+            }
+            partial = static_cast<T *>(ws);
+        }
+        const int tiles_m = (M_ + 63) / 64, tiles_n = (N_ + 63) / 64;
+        const int64_t blocks = static_cast<int64_t>(tiles_m) * tiles_n * splits;
+        const bool vec = rows_vectorizable<T>(gout, HoWo, static_cast<int64_t>(g.O) * HoWo);
+        auto launch = [&](auto kernel, size_t lds) -> ttamd_status {
+            if (ttamd_status s = set_lds(kernel, lds)) return s;
+            kernel<<<dim3(static_cast<unsigned>(blocks)), dim3(kThreads), lds, st>>>(
+                g, static_cast<const T *>(gout), static_cast<const T *>(pl.x), partial, pl.image_bytes, group, tiles_m, tiles_n);
+            TTAMD_HIP_CHECK(hipGetLastError());
+            return TTAMD_OK;
+        };
+        if (vec) {
+            using E = TileEngine<T, 64, 64, BK, 2, 2, Stager<T, 64, BK, true, VK>, Im2colTStager<T, 64, BK>>;
+            if (ttamd_status s = launch(conv_wgrad_kernel<T, 64, 64, BK, VK>, E::kLdsBytes)) return s;
+        } else {
+            using E = TileEngine<T, 64, 64, BK, 2, 2, Stager<T, 64, BK, true, 1>, Im2colTStager<T, 64, BK>>;
+            if (ttamd_status s = launch(conv_wgrad_kernel<T, 64, 64, BK, 1>, E::kLdsBytes)) return s;
+        }
+        if (splits > 1) {
+            const int64_t rb = (tile_elems + 255) / 256;
+            reduce_splits_kernel<T><<<dim3(static_cast<unsigned>(rb)), dim3(256), 0, st>>>(partial, static_cast<T *>(gw), tile_elems, splits);
+            TTAMD_HIP_CHECK(hipGetLastError());
+        }
+    }
+    if (gb) {
+        bias_grad_kernel<T><<<dim3(g.O), dim3(256), 0, st>>>(static_cast<const T *>(gout), static_cast<T *>(gb), g.B, g.O, HoWo);
+        TTAMD_HIP_CHECK(hipGetLastError());
+    }
+    return TTAMD_OK;
+}
+
+}  // namespace
+}  // namespace ttamd
+
+using namespace ttamd;
+
+extern "C" {
+
+ttamd_status ttamd_conv2d_forward(int device, ttamd_dtype dtype, const ttamd_view4 *input, const ttamd_view4 *weight,
+                                  const void *bias, void *out, int B, int C, int H, int W, int O, int k, int stride,
+                                  int padding, void *stream) {
+    ConvPlan pl;
+    if (ttamd_status s = make_plan("conv2d", dtype, input, weight, B, C, H, W, O, k, stride, padding, &pl)) return s;
+    if (ttamd_status s = use_device(device)) return s;
+    if (B == 0) return TTAMD_OK;
+    if (!input->data || !weight->data || !out) {
+        set_error("conv2d: NULL data pointer");
+        return TTAMD_ERR_INVALID_ARGUMENT;
+    }
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    switch (dtype) {
+    case TTAMD_F32: return forward_mfma<float>(pl, bias, out, st);
+    case TTAMD_F64: return forward_mfma<double>(pl, bias, out, st);
+    case TTAMD_U8: return forward_direct<uint8_t, uint32_t>(pl, bias, out, st);
+    case TTAMD_I16: return forward_direct<int16_t, uint32_t>(pl, bias, out, st);
+    case TTAMD_I32: return forward_direct<int32_t, uint32_t>(pl, bias, out, st);
+    case TTAMD_I64: return forward_direct<int64_t, uint64_t>(pl, bias, out, st);
+    default: break;
+    }
+    set_error("conv2d does not support dtype code %d", static_cast<int>(dtype));
+    return TTAMD_ERR_UNSUPPORTED_DTYPE;
+}
+
+ttamd_status ttamd_conv2d_backward_workspace(ttamd_dtype dtype, int B, int C, int H, int W, int O, int k, int stride,
+                                             int padding, size_t *bytes) {
+    (void)H; (void)W; (void)stride; (void)padding;
+    if (!bytes) {
+        set_error("conv2d_backward_workspace: bytes is NULL");
+        return TTAMD_ERR_INVALID_ARGUMENT;
+    }
+    *bytes = 0;
+    if (dtype != TTAMD_F32 && dtype != TTAMD_F64) {
+        set_error("conv2d_backward supports f32 and f64 only (autograd never differentiates integer tensors)");
+        return TTAMD_ERR_UNSUPPORTED_DTYPE;
+    }
+    if (B <= 0 || C <= 0 || O <= 0 || k <= 0) return TTAMD_OK;
+    const size_t esz = dtype_size(dtype);
+    const int group = wgrad_group(esz, B, C, O, k);
+    const int splits = (B + group - 1) / group;
+    if (splits > 1) *bytes = static_cast<size_t>(splits) * O * C * k * k * esz;
+    return TTAMD_OK;
+}
+
+ttamd_status ttamd_conv2d_backward(int device, ttamd_dtype dtype, const void *grad_out, const ttamd_view4 *input,
+                                   const ttamd_view4 *weight, void *grad_input, void *grad_weight, void *grad_bias,
+                                   int B, int C, int H, int W, int O, int k, int stride, int padding, void *workspace,
+                                   size_t workspace_bytes, void *stream) {
+    if (dtype != TTAMD_F32 && dtype != TTAMD_F64) {
+        set_error("conv2d_backward supports f32 and f64 only (autograd never differentiates integer tensors)");
+        return TTAMD_ERR_UNSUPPORTED_DTYPE;
+    }
+    ConvPlan pl;
+    if (ttamd_status s = make_plan("conv2d_backward", dtype, input, weight, B, C, H, W, O, k, stride, padding, &pl)) return s;
+    if (ttamd_status s = use_device(device)) return s;
+    if (!grad_weight || !input->data || !weight->data || (B > 0 && (!grad_out || !grad_input))) {
+        set_error("conv2d_backward: NULL data pointer");
+        return TTAMD_ERR_INVALID_ARGUMENT;
+    }
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    if (B == 0) {
+        // no images: the weight (and bias) gradients are empty sums
+        if (ttamd_status s = ttamd_memset_zero(device, grad_weight, static_cast<size_t>(O) * C * k * k * dtype_size(dtype), stream)) return s;
+        if (grad_bias) return ttamd_memset_zero(device, grad_bias, static_cast<size_t>(O) * dtype_size(dtype), stream);
+        return TTAMD_OK;
+    }
+    if (dtype == TTAMD_F32) return backward_mfma<float>(pl, grad_out, grad_input, grad_weight, grad_bias, workspace, workspace_bytes, st);
+    return backward_mfma<double>(pl, grad_out, grad_input, grad_weight, grad_bias, workspace, workspace_bytes, st);
+}
+
+}  // extern "C"

@@ -1,0 +1,456 @@
+// mfma_core.h — device-side building blocks of the matrix-core kernels (gfx950 only).
+//
+// One workgroup = 4 wavefronts of 64 lanes computing a BM x BN tile of C = A . B:
+//   * operand tiles (BM x BK, BN x BK) are staged global -> registers -> LDS by a "stager" per operand;
+//     two LDS buffers per operand, the loads of tile t+1 are issued before the MFMA work of tile t and
+//     parked in the other buffer afterwards, one barrier per tile;
+//   * fp32: v_mfma_f32_32x32x2_f32, fp64: v_mfma_f64_16x16x4_f64; accumulators stay in registers;
+//   * LDS layout follows the operand's memory layout, so nothing is transposed on the way in:
+//       KC  element (r, k) at r * LD + k   (k contiguous; rows padded by one 16-byte vector so that 16-byte
+//                                           fragment reads of consecutive rows land in distinct banks)
+//       MC  element (r, k) at k * LD + r   (row/column index contiguous)
+//     fragment reads pair k indices so that both operands agree whatever their layouts;
+//   * all global reads are buffer loads that carry the operand's byte extent: a lane that is out of the tile
+//     uses an offset with bit 31 set and receives zero instead of touching memory.
+//
+// A stager is any type with
+//     static constexpr bool kKC; static constexpr int LD, LDS_ELEMS;
+//     template <bool MASK> void load(int k_left);   // fetch the next BK-deep tile into registers
+//     void store(T *lds) const;                       // write those registers to an LDS buffer
+// Stager<> below reads a strided matrix view; conv.hip adds gather stagers (implicit im2col).
+#ifndef TTAMD_CSRC_MFMA_CORE_H_
+#define TTAMD_CSRC_MFMA_CORE_H_
+
+#include "common.h"
+
+namespace ttamd {
+namespace mfma {
+
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef double f64x4 __attribute__((ext_vector_type(4)));
+typedef double f64x2 __attribute__((ext_vector_type(2)));
+
+constexpr int kThreads = 256;
+constexpr int kWaves = 4;
+constexpr int kChunk = 8;               // k extent of one fragment read (both dtypes)
+constexpr uint32_t kOob = 0x80000000u;  // byte offset that is out of range for every buffer used here
+
+// ---------------------------------------------------------------------------------------------
+// MFMA instruction traits.  A lane l holds A[i = l % MB][k = l / MB] and B[k = l / MB][j = l % MB].
+template <typename T>
+struct Mfma;
+
+template <>
+struct Mfma<float> {
+    static constexpr int MB = 32;  // block is MB x MB
+    static constexpr int VK = 4;   // elements in 16 bytes = k steps per chunk
+    static constexpr int NACC = 16;
+    using acc_t = f32x16;
+    using vec_t = f32x4;
+    using pair_t = f32x2;
+    static __device__ __forceinline__ acc_t mma(float a, float b, acc_t c) {
+        return __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, c, 0, 0, 0);
+    }
+    // accumulator element e of lane l is C[acc_row(e,l)][l % MB]
+    static __device__ __forceinline__ int acc_row(int e, int lane) { return (e / 4) * 8 + (lane / 32) * 4 + (e % 4); }
+};
+
+template <>
+struct Mfma<double> {
+    static constexpr int MB = 16;
+    static constexpr int VK = 2;
+    static constexpr int NACC = 4;
+    using acc_t = f64x4;
+    using vec_t = f64x2;
+    using pair_t = f64x2;
+    static __device__ __forceinline__ acc_t mma(double a, double b, acc_t c) {
+        return __builtin_amdgcn_mfma_f64_16x16x4f64(a, b, c, 0, 0, 0);
+    }
+    static __device__ __forceinline__ int acc_row(int e, int lane) { return 4 * e + lane / 16; }
+};
+
+// ---------------------------------------------------------------------------------------------
+// Typed buffer loads of 1 element or of one 16-byte vector.
+template <typename T, int VEC>
+struct Vec;
+template <>
+struct Vec<float, 1> {
+    using type = float;
+    static __device__ __forceinline__ type load(__amdgpu_buffer_rsrc_t r, uint32_t off) {
+        return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(r, off, 0, 0));
+    }
+};
+template <>
+struct Vec<float, 4> {
+    using type = f32x4;
+    static __device__ __forceinline__ type load(__amdgpu_buffer_rsrc_t r, uint32_t off) {
+        return __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(r, off, 0, 0));
+    }
+};
+template <>
+struct Vec<double, 1> {
+    using type = double;
+    static __device__ __forceinline__ type load(__amdgpu_buffer_rsrc_t r, uint32_t off) {
+        return __builtin_bit_cast(double, __builtin_amdgcn_raw_buffer_load_b64(r, off, 0, 0));
+    }
+};
+template <>
+struct Vec<double, 2> {
+    using type = f64x2;
+    static __device__ __forceinline__ type load(__amdgpu_buffer_rsrc_t r, uint32_t off) {
+        return __builtin_bit_cast(f64x2, __builtin_amdgcn_raw_buffer_load_b128(r, off, 0, 0));
+    }
+};
+
+template <typename T, int VEC>
+__device__ __forceinline__ void zero_component(typename Vec<T, VEC>::type &v, int j) {
+    if constexpr (VEC == 1) {
+        v = T(0);
+    } else {
+        v[j] = T(0);
+    }
+}
+
+// Raw buffer descriptor over [base, base + bytes), bytes clamped to 2^31 - 1 (offsets >= 2^31 are the
+// out-of-range marker).
+template <typename T>
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const T *base, int64_t bytes) {
+    const int rec = bytes > 0x7fffffff ? 0x7fffffff : (bytes < 0 ? 0 : static_cast<int>(bytes));
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<T *>(base), 0, rec, 0x00020000);
+}
+
+// LDS geometry shared by every stager of a given layout.
+template <typename T, int ROWS, int BK, bool KC>
+struct TileLayout {
+    static constexpr bool kKC = KC;
+    static constexpr int PAD = Mfma<T>::VK;  // one 16-byte vector
+    static constexpr int LD = KC ? (BK + PAD) : (ROWS + PAD);
+    static constexpr int LDS_ELEMS = KC ? ROWS * LD : BK * LD;
+};
+
+// ---------------------------------------------------------------------------------------------
+// Stager for a strided matrix view (ROWS along m or n, BK along k).  Vectors of VEC elements run along k
+// for KC (operand's k stride is 1 when VEC > 1) and along the row index for MC (row stride 1 when VEC > 1).
+template <typename T, int ROWS, int BK, bool KC, int VEC>
+struct Stager : TileLayout<T, ROWS, BK, KC> {
+    using L = TileLayout<T, ROWS, BK, KC>;
+    using V = typename Vec<T, VEC>::type;
+    static constexpr int VPL = (KC ? BK : ROWS) / VEC;  // vectors per LDS line
+    static constexpr int NV = ROWS * BK / VEC;
+    static constexpr int P = NV / kThreads;
+    static_assert(NV % kThreads == 0, "tile must split evenly over the workgroup");
+
+    V reg[P];
+    uint32_t voff[P];
+    int nval[P];  // MC only: valid components of the vector along the row dimension
+    __amdgpu_buffer_rsrc_t rsrc;
+    uint32_t k_step_b;
+    int tid;
+    bool edge;
+
+    // line/column coordinates of pass p for this lane
+    static __device__ __forceinline__ int line_of(int p, int tid) { return (p * kThreads + tid) / VPL; }
+    static __device__ __forceinline__ int col_of(int p, int tid) { return ((p * kThreads + tid) % VPL) * VEC; }
+
+    // base: element (row 0 of this tile, k = 0); rows_left: valid rows from there; strides in elements;
+    // K: full reduction length (sizes the buffer extent).
+    __device__ __forceinline__ void init(const T *base, int tid_, int rows_left, int64_t s_row, int64_t s_k, int K) {
+        tid = tid_;
+        edge = rows_left < ROWS;
+        int64_t ext = (static_cast<int64_t>(rows_left - 1) * s_row + static_cast<int64_t>(K - 1) * s_k + 1) * sizeof(T);
+        // With 16-byte loads the extent is rounded up to the vector size: the base is 16-byte aligned, so the
+        // last vector stays inside the allocation's final 16-byte block and its tail is masked anyway.
+        if (VEC > 1) ext = (ext + 15) & ~static_cast<int64_t>(15);
+        rsrc = make_rsrc(base, ext);
+        const uint32_t s_row_b = static_cast<uint32_t>(s_row * sizeof(T)), s_k_b = static_cast<uint32_t>(s_k * sizeof(T));
+        k_step_b = s_k_b * BK;
+#pragma unroll
+        for (int p = 0; p < P; ++p) {
+            const int line = line_of(p, tid), col = col_of(p, tid);
+            if constexpr (KC) {
+                voff[p] = line < rows_left ? (line * s_row_b + col * s_k_b) : kOob;
+                nval[p] = VEC;
+            } else {
+                int nv = rows_left - col;
+                nv = nv < 0 ? 0 : (nv > VEC ? VEC : nv);
+                nval[p] = nv;
+                voff[p] = nv > 0 ? (col * s_row_b + line * s_k_b) : kOob;
+            }
+        }
+    }
+
+    // Fetches the next tile; k_left = K - (first k of that tile).  MASK = false is the steady state
+    // (full k tile, interior rows): loads only, no selects.
+    template <bool MASK>
+    __device__ __forceinline__ void load(int k_left) {
+        const bool k_tail = k_left < BK;
+#pragma unroll
+        for (int p = 0; p < P; ++p) {
+            V v = Vec<T, VEC>::load(rsrc, voff[p]);
+            voff[p] += k_step_b;
+            if constexpr (!MASK) {
+                reg[p] = v;
+                continue;
+            }
+            if constexpr (KC) {
+                if (k_tail) {
+                    const int col = col_of(p, tid);
+#pragma unroll
+                    for (int j = 0; j < VEC; ++j)
+                        if (col + j >= k_left) zero_component<T, VEC>(v, j);
+                }
+            } else {
+                if (k_tail) {
+                    if (line_of(p, tid) >= k_left) {
+#pragma unroll
+                        for (int j = 0; j < VEC; ++j) zero_component<T, VEC>(v, j);
+                    }
+                }
+                if (VEC > 1 && edge) {
+#pragma unroll
+                    for (int j = 0; j < VEC; ++j)
+                        if (j >= nval[p]) zero_component<T, VEC>(v, j);
+                }
+            }
+            reg[p] = v;
+        }
+    }
+
+    __device__ __forceinline__ void store(T *lds) const {
+#pragma unroll
+        for (int p = 0; p < P; ++p) {
+            const int line = line_of(p, tid), col = col_of(p, tid);
+            *reinterpret_cast<V *>(&lds[line * L::LD + col]) = reg[p];
+        }
+    }
+};
+
+// ---------------------------------------------------------------------------------------------
+// LDS -> MFMA operand fragments for NB blocks of one wave, one chunk of 8 k.
+// Step j of a chunk multiplies k = chunk*8 + VK*kg + j, kg = lane / MB, for both operands.
+template <typename T, int LD, bool KC, int NB>
+struct Fragment {
+    using M = Mfma<T>;
+    static constexpr bool PAIRED = (!KC) && (NB % 2 == 0);
+    T v[NB][M::VK];
+
+    // w0 = first tile-local row of this wave.
+    __device__ __forceinline__ void read(const T *lds, int w0, int chunk, int lane) {
+        const int i = lane % M::MB, kg = lane / M::MB;
+        const int kb = chunk * kChunk + M::VK * kg;
+        if constexpr (KC) {
+#pragma unroll
+            for (int b = 0; b < NB; ++b) {
+                const typename M::vec_t t = *reinterpret_cast<const typename M::vec_t *>(&lds[(w0 + b * M::MB + i) * LD + kb]);
+#pragma unroll
+                for (int j = 0; j < M::VK; ++j) v[b][j] = t[j];
+            }
+        } else if constexpr (PAIRED) {
+#pragma unroll
+            for (int j = 0; j < M::VK; ++j)
+#pragma unroll
+                for (int pr = 0; pr < NB / 2; ++pr) {
+                    const typename M::pair_t t =
+                        *reinterpret_cast<const typename M::pair_t *>(&lds[(kb + j) * LD + w0 + pr * 2 * M::MB + 2 * i]);
+                    v[2 * pr][j] = t[0];
+                    v[2 * pr + 1][j] = t[1];
+                }
+        } else {
+#pragma unroll
+            for (int j = 0; j < M::VK; ++j)
+#pragma unroll
+                for (int b = 0; b < NB; ++b) v[b][j] = lds[(kb + j) * LD + w0 + b * M::MB + i];
+        }
+    }
+
+    // tile-local row (or column) that block b, in-block index i stands for
+    static __device__ __forceinline__ int index_of(int w0, int b, int i) {
+        if constexpr (PAIRED) {
+            return w0 + (b / 2) * 2 * M::MB + 2 * i + (b % 2);
+        } else {
+            return w0 + b * M::MB + i;
+        }
+    }
+};
+
+// Each XCD receives every 8th workgroup id; give it a contiguous range of logical ids instead.
+__device__ __forceinline__ int remap_xcd(int pid, int total) {
+    constexpr int XCDS = 8;
+    const int q = total / XCDS, r = total % XCDS;
+    const int xcd = pid % XCDS, idx = pid / XCDS;
+    return xcd * q + (xcd < r ? xcd : r) + idx;
+}
+
+// Logical workgroup id -> (batch, tile row, tile column); tiles are walked in groups of 8 tile rows so that
+// the workgroups resident on one XCD share operand panels through its L2.
+__device__ __forceinline__ void decode_tile(int pid, int tiles_m, int tiles_n, int &batch, int &tm, int &tn) {
+    const int tiles = tiles_m * tiles_n;
+    batch = pid / tiles;
+    pid -= batch * tiles;
+    constexpr int GROUP = 8;
+    const int group_sz = GROUP * tiles_n;
+    const int first_m = (pid / group_sz) * GROUP;
+    const int gm = (tiles_m - first_m) < GROUP ? (tiles_m - first_m) : GROUP;
+    tm = first_m + (pid % group_sz) % gm;
+    tn = (pid % group_sz) / gm;
+}
+
+// ---------------------------------------------------------------------------------------------
+// The tile engine: software pipeline + MFMA loop + register -> memory walk of the finished tile.
+template <typename T, int BM, int BN, int BK, int WGM, int WGN, class StA, class StB>
+struct TileEngine {
+    using M = Mfma<T>;
+    static_assert(WGM * WGN == kWaves, "4 waves per workgroup");
+    static constexpr int WM = BM / WGM, WN = BN / WGN;
+    static constexpr int NBM = WM / M::MB, NBN = WN / M::MB;
+    static_assert(WM % M::MB == 0 && WN % M::MB == 0 && BK % kChunk == 0, "tile shape");
+    using FrA = Fragment<T, StA::LD, StA::kKC, NBM>;
+    using FrB = Fragment<T, StB::LD, StB::kKC, NBN>;
+    // LDS: [A buf 0][A buf 1][B buf 0][B buf 1]; addressed as offsets from the one shared base so that every
+    // access stays a DS instruction (generic-pointer loads would also wait on the global-load counter).
+    static constexpr int kBOff = 2 * StA::LDS_ELEMS;
+    static constexpr size_t kLdsBytes = 2 * (StA::LDS_ELEMS + StB::LDS_ELEMS) * sizeof(T);
+
+    typename M::acc_t acc[NBM][NBN];
+    int lane, wm0, wn0;
+
+    __device__ __forceinline__ void init(int tid) {
+        lane = tid % 64;
+        const int wave = tid / 64;
+        wm0 = (wave / WGN) * WM;
+        wn0 = (wave % WGN) * WN;
+#pragma unroll
+        for (int i = 0; i < NBM; ++i)
+#pragma unroll
+            for (int j = 0; j < NBN; ++j)
+#pragma unroll
+                for (int e = 0; e < M::NACC; ++e) acc[i][j][e] = T(0);
+    }
+
+    __device__ __forceinline__ void compute(const T *smem, int buf) {
+        const T *la = smem + buf * StA::LDS_ELEMS;
+        const T *lb = smem + kBOff + buf * StB::LDS_ELEMS;
+#pragma unroll
+        for (int c = 0; c < BK / kChunk; ++c) {
+            FrA fa;
+            FrB fb;
+            fa.read(la, wm0, c, lane);
+            fb.read(lb, wn0, c, lane);
+#pragma unroll
+            for (int j = 0; j < M::VK; ++j)
+#pragma unroll
+                for (int bm = 0; bm < NBM; ++bm)
+#pragma unroll
+                    for (int bn = 0; bn < NBN; ++bn) acc[bm][bn] = M::mma(fa.v[bm][j], fb.v[bn][j], acc[bm][bn]);
+        }
+    }
+
+    // K: reduction length.  `unmasked`: workgroup-uniform promise that every tile is full and interior.
+    __device__ __forceinline__ void run(StA &sa, StB &sb, T *smem, int K, bool unmasked) {
+        const int KT = (K + BK - 1) / BK;
+        sa.template load<true>(K);
+        sb.template load<true>(K);
+        sa.store(smem);
+        sb.store(smem + kBOff);
+        __syncthreads();
+        // Tiles 0 .. KT-2: prefetch tile kt+1 into registers, multiply tile kt out of LDS, then park the
+        // prefetched tile in the other LDS buffer.  The last tile is multiplied after the loop, so the loop
+        // body has no conditionals.
+        auto pipeline = [&]<bool MASK>() {
+            for (int kt = 0; kt + 1 < KT; ++kt) {
+                const int cur = kt & 1;
+                const int k_left = K - (kt + 1) * BK;
+                sa.template load<MASK>(k_left);
+                sb.template load<MASK>(k_left);
+                compute(smem, cur);
+                sa.store(smem + (cur ^ 1) * StA::LDS_ELEMS);
+                sb.store(smem + kBOff + (cur ^ 1) * StB::LDS_ELEMS);
+                __syncthreads();
+            }
+        };
+        if (unmasked) {
+            pipeline.template operator()<false>();
+        } else {
+            pipeline.template operator()<true>();
+        }
+        if (KT > 0) compute(smem, (KT - 1) & 1);
+    }
+
+    // Walks the finished tile.  `one(m, n, v)` receives a single element at tile-local (m, n);
+    // `two(m, n, v0, v1)` receives columns n and n + 1 of the same row (only called when B is MC/paired and
+    // `pairs_ok`); both are expected to do their own bounds checks against the matrix size.
+    template <class One, class Two>
+    __device__ __forceinline__ void for_each(bool pairs_ok, One one, Two two) {
+        const int jcol = lane % M::MB;
+        if constexpr (FrB::PAIRED) {
+#pragma unroll
+            for (int pr = 0; pr < NBN / 2; ++pr) {
+                const int n = FrB::index_of(wn0, 2 * pr, jcol);  // even column; n + 1 belongs to block 2p+1
+#pragma unroll
+                for (int bm = 0; bm < NBM; ++bm)
+#pragma unroll
+                    for (int e = 0; e < M::NACC; ++e) {
+                        const int m = FrA::index_of(wm0, bm, M::acc_row(e, lane));
+                        if (pairs_ok) {
+                            two(m, n, acc[bm][2 * pr][e], acc[bm][2 * pr + 1][e]);
+                        } else {
+                            one(m, n, acc[bm][2 * pr][e]);
+                            one(m, n + 1, acc[bm][2 * pr + 1][e]);
+                        }
+                    }
+            }
+        } else {
+#pragma unroll
+            for (int bn = 0; bn < NBN; ++bn) {
+                const int n = FrB::index_of(wn0, bn, jcol);
+#pragma unroll
+                for (int bm = 0; bm < NBM; ++bm)
+#pragma unroll
+                    for (int e = 0; e < M::NACC; ++e) one(FrA::index_of(wm0, bm, M::acc_row(e, lane)), n, acc[bm][bn][e]);
+            }
+        }
+    }
+};
+
+// Dense row-major store of a finished tile with the optional bias / ReLU / accumulate epilogue.
+// C points at the matrix (already offset to the batch), M x N its size, (m0, n0) the tile origin.
+template <typename T, class Engine>
+__device__ __forceinline__ void store_tile_dense(Engine &eng, T *__restrict__ C, int M_, int N_, int m0, int n0,
+                                                 const T *__restrict__ bias, int bias_mode, int relu, int accumulate) {
+    using pair_t = typename Mfma<T>::pair_t;
+    auto finish = [&](T v, int m, int n, int64_t idx) {
+        if (bias_mode == 1) v += bias[n];
+        if (bias_mode == 2) v += bias[m];
+        if (relu) v = v > T(0) ? v : T(0);
+        if (accumulate) v += C[idx];
+        return v;
+    };
+    const bool pairs_ok = (N_ % 2 == 0) && (reinterpret_cast<uintptr_t>(C) % (2 * sizeof(T)) == 0);
+    eng.for_each(
+        pairs_ok,
+        [&](int ml, int nl, T v) {
+            const int m = m0 + ml, n = n0 + nl;
+            if (m < M_ && n < N_) {
+                const int64_t idx = static_cast<int64_t>(m) * N_ + n;
+                C[idx] = finish(v, m, n, idx);
+            }
+        },
+        [&](int ml, int nl, T v0, T v1) {
+            // n is even and N_ is even, so n + 1 < N_ whenever n < N_: a wave writes whole row segments
+            const int m = m0 + ml, n = n0 + nl;
+            if (m < M_ && n < N_) {
+                const int64_t idx = static_cast<int64_t>(m) * N_ + n;
+                pair_t out;
+                out[0] = finish(v0, m, n, idx);
+                out[1] = finish(v1, m, n + 1, idx + 1);
+                *reinterpret_cast<pair_t *>(&C[idx]) = out;
+            }
+        });
+}
+
+}  // namespace mfma
+}  // namespace ttamd
+
+#endif  // TTAMD_CSRC_MFMA_CORE_H_

@@ -287,6 +287,7 @@ class BackendAMD:
         Ho = (H + 2 * padding - k) // stride + 1
         Wo = (W + 2 * padding - k) // stride + 1
         out = Tensor.empty((B, O, Ho, Wo), input.dtype, input.device)
+        weight = weight.contiguous()  # used as the matrix [O, C*k*k], as cpu/conv.cpp:69 reshapes it
         iv, wv = input.view4(), weight.view4()
         bptr = None
         if bias is not None:
@@ -302,6 +303,7 @@ class BackendAMD:
         B, Cc, H, W = input.shape
         O, _, k, _ = weight.shape
         go = grad_output.contiguous()
+        weight = weight.contiguous()
         gx = Tensor.empty(input.shape, input.dtype, input.device)
         gw = Tensor.empty(weight.shape, input.dtype, input.device)
         gb = Tensor.empty((O,), input.dtype, input.device) if bias is not None else None
