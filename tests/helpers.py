@@ -64,3 +64,39 @@ def naive_exact(A, B):
     if bits < 64:
         full = full & np.uint64((1 << bits) - 1)
     return full.astype(np.dtype(f"uint{bits}")).view(dt) if dt != np.uint8 else full.astype(np.uint8)
+
+
+# ---- MLP training step of BASELINE config 5, written once over an abstract GEMM --------------------------
+def mlp_train_step(X, T, params, mm, mm_bwd, masks=None):
+    """One forward + backward of Linear-ReLU-Linear-ReLU-Linear + mse_loss(mean), following the reference's
+    op sequence: nn::Linear::forward = matmul + bias.expand (nn/linear.cpp:42-50), relu backward mask
+    `input < 0 -> 0 else 1` (autograd/unary_ops.cpp:568-573), mse = pow(y - t, 2).mean() (nn/loss.cpp:69-72)
+    whose backward is ((1/N) * 2) * (y - t), and matmul backward dA = dC.B^T, dB = A^T.dC on transposed VIEWS
+    (autograd/binary_ops.cpp:173-179).  `mm(a, b)` multiplies 2-D host arrays; `mm_bwd(a, b, g)` returns (dA, dB).
+    Elementwise work is numpy on the host for both sides of a comparison, so only the GEMMs differ.
+    `masks` = (mask1, mask2) overrides the ReLU-backward masks: the mask is a step function of z, so two runs
+    whose z differ in the last bit can disagree on an element with z ~ 0 and then differ by a whole rank-one
+    term downstream; a comparison of the GEMMs shares the masks of one run."""
+    (W1, b1), (W2, b2), (W3, b3) = params
+    f = X.dtype.type
+    z1 = mm(X, W1) + b1
+    a1 = np.maximum(z1, f(0))
+    z2 = mm(a1, W2) + b2
+    a2 = np.maximum(z2, f(0))
+    y = mm(a2, W3) + b3
+    diff = y - T
+    loss = np.mean(diff * diff, dtype=X.dtype)
+    gy = (f(1) / f(y.size) * f(2)) * diff
+    out = {"y": y, "loss": loss}
+    out["db3"] = gy.sum(axis=0, dtype=X.dtype)
+    da2, out["dW3"] = mm_bwd(a2, W3, gy)
+    m1 = np.where(z1 < 0, f(0), f(1)) if masks is None else masks[0]
+    m2 = np.where(z2 < 0, f(0), f(1)) if masks is None else masks[1]
+    out["masks"] = (m1, m2)
+    dz2 = da2 * m2
+    out["db2"] = dz2.sum(axis=0, dtype=X.dtype)
+    da1, out["dW2"] = mm_bwd(a1, W2, dz2)
+    dz1 = da1 * m1
+    out["db1"] = dz1.sum(axis=0, dtype=X.dtype)
+    out["dX"], out["dW1"] = mm_bwd(X, W1, dz1)  # dX is computed (and discarded) by the reference too
+    return out
