@@ -17,6 +17,12 @@ if ROOT not in sys.path:
 
 PEAK_TFLOPS = {"f32": 157.3, "f64": 78.6}  # MI355X dense matrix peaks
 
+# Bytes moved between the L2s and the memory fabric per launch of the default workload, from the rocprofv3
+# FETCH_SIZE / WRITE_SIZE passes summarised in profiles/gemm_4096_f32_f64_mfma.txt (scaled by the same counters'
+# reading for a copy kernel of known size: x2.000 for reads, x1.000 for writes).  Only valid for that exact
+# kernel and size; reported as null otherwise.  Algorithmic bytes are 3 * 4096^2 * 4 = 201.3e6.
+MEASURED_TRAFFIC = {("mfma_f32_128x128_akc4_bmc4", 4096): (365531.4 * 2.0 + 65536.0) * 1024.0}
+
 
 def gpu_gemm_timing(tt, np, dtype, n, steps, warmup):
     """Returns (wall ms/step, event-timed average kernel ms, variant name, C as numpy)."""
@@ -60,8 +66,8 @@ def gpu_gemm_timing(tt, np, dtype, n, steps, warmup):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=50)
-    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--steps", type=int, default=100)
+    ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--n", type=int, default=4096, help="square size (the metric is quoted at 4096)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--copy-calibration", action="store_true",
@@ -126,7 +132,8 @@ def main():
         "config": {"workload": f"configs[2]: fp32 {n}x{n} @ {n}x{n}, dense row-major", "kernel": variant,
                    "parity_k_scaled_err_rows0_63": parity},
         "roofline": {"bound": "mfma", "achieved": round(achieved_tflops, 2), "peak": PEAK_TFLOPS["f32"],
-                     "unit": "TFLOP/s", "frac": round(achieved_tflops / PEAK_TFLOPS["f32"], 4), "traffic": None,
+                     "unit": "TFLOP/s", "frac": round(achieved_tflops / PEAK_TFLOPS["f32"], 4),
+                     "traffic": MEASURED_TRAFFIC.get((variant, n)), "algorithmic_bytes": 3.0 * n * n * 4,
                      "kernel_ms": round(kern_ms, 4)},
         "cpu_baseline": cpu,
         "fp64": {"kernel": variant64, "kernel_ms": round(kern64, 4), "achieved": round(f64_tflops, 2),
