@@ -63,6 +63,85 @@ def gpu_gemm_timing(tt, np, dtype, n, steps, warmup):
     return wall_ms, ms.value / steps, variant, (A, B, out)
 
 
+def time_launches(tt, fn, iters, warmup):
+    """Average milliseconds per call of fn() (which enqueues GPU work on the default stream), by HIP events."""
+    lib = tt._capi.lib
+    for _ in range(warmup):
+        fn()
+    tt.get_backend(tt.kAMD).synchronize(0)
+    e0, e1 = C.c_void_p(), C.c_void_p()
+    lib.ttamd_event_create(0, C.byref(e0))
+    lib.ttamd_event_create(0, C.byref(e1))
+    lib.ttamd_event_record(e0, None)
+    for _ in range(iters):
+        fn()
+    lib.ttamd_event_record(e1, None)
+    ms = C.c_float()
+    lib.ttamd_event_elapsed_ms(e0, e1, C.byref(ms))
+    lib.ttamd_event_destroy(e0)
+    lib.ttamd_event_destroy(e1)
+    return ms.value / iters
+
+
+def detail_report(tt, np, path):
+    """Times every BASELINE configuration (GPU only, inputs resident) and writes a JSON report to `path`.
+    Not part of the one-line contract; used to track the small-shape, strided and conv paths."""
+    from oracle import tt_oracle as oracle  # seeded input generation only
+
+    be = tt.get_backend(tt.kAMD)
+    rows = []
+
+    def gemm_case(name, tA, tB, iters=200):
+        Bn, N, K = tA.shape
+        M = tB.shape[2]
+        out = tt.Tensor.empty((Bn, N, M), tA.dtype)
+        ms = time_launches(tt, lambda: be.batched_matmul(tA, tB, out=out), iters, 20)
+        flop = 2.0 * Bn * N * K * M
+        nbytes = (Bn * N * K + Bn * K * M + Bn * N * M) * tA.itemsize
+        rows.append({"case": name, "kernel": be.batched_matmul_variant(tA, tB), "ms": round(ms, 5),
+                     "GFLOP/s": round(flop / ms / 1e6, 1), "GB/s": round(nbytes / ms / 1e6, 1)})
+
+    f32 = np.float32
+    g = oracle.Generator(0)
+    A = tt.Tensor.from_numpy(g.uniform_real(-1, 1, (1, 256, 512)))
+    B = tt.Tensor.from_numpy(g.uniform_real(-1, 1, (1, 512, 256)))
+    gemm_case("cfg1 f32 256x512x256", A, B)
+    A = tt.Tensor.from_numpy(g.uniform_real(-1, 1, (32, 128, 64)))
+    Bs = tt.Tensor.from_numpy(g.uniform_real(-1, 1, (32, 128, 64)))
+    gemm_case("cfg2 f32 32x(128x64x128) B=transposed view", A, Bs.permute(0, 2, 1))
+    for dt, nm in ((f32, "f32"), (np.float64, "f64")):
+        S = tt.Tensor.from_numpy(np.zeros((1, 4096, 4096), dt))
+        gemm_case(f"cfg3 {nm} 4096^3 A.B", S, S, 30)
+        gemm_case(f"cfg3 {nm} 4096^3 A.B^T (view)", S, S.permute(0, 2, 1), 30)
+        gemm_case(f"cfg3 {nm} 4096^3 A^T.B (view)", S.permute(0, 2, 1), S, 30)
+    # config 5: the nine GEMMs of one MLP training step (batch 1024, 784-1024-1024-10)
+    X = tt.Tensor.from_numpy(np.zeros((1, 1024, 784), f32))
+    W1 = tt.Tensor.from_numpy(np.zeros((1, 784, 1024), f32))
+    H = tt.Tensor.from_numpy(np.zeros((1, 1024, 1024), f32))
+    W3 = tt.Tensor.from_numpy(np.zeros((1, 1024, 10), f32))
+    Y = tt.Tensor.from_numpy(np.zeros((1, 1024, 10), f32))
+    t = lambda x: x.permute(0, 2, 1)
+    for name, a, b in (("fwd1 X.W1", X, W1), ("fwd2 H.W2", H, H), ("fwd3 H.W3 (N=10)", H, W3),
+                       ("bwd3 dH=dY.W3^T (K=10)", Y, t(W3)), ("bwd3 dW3=H^T.dY (N=10)", t(H), Y),
+                       ("bwd2 dH=dZ.W2^T", H, t(H)), ("bwd2 dW2=H^T.dZ", t(H), H),
+                       ("bwd1 dX=dZ.W1^T", H, t(W1)), ("bwd1 dW1=X^T.dZ", t(X), H)):
+        gemm_case("cfg5 " + name, a, b)
+    # config 4: conv2d forward / backward, input [64,32,28,28], weight [64,32,3,3], s1 p1
+    x = tt.Tensor.from_numpy(oracle.Generator(0).normal(0, 0.1, (64, 32, 28, 28)))
+    w = tt.Tensor.from_numpy(oracle.Generator(1).normal(0, 0.1, (64, 32, 3, 3)))
+    go = tt.Tensor.from_numpy(np.ones((64, 64, 28, 28), f32))
+    ms = time_launches(tt, lambda: be.conv2d(x, w, None, 1, 1), 100, 10)
+    rows.append({"case": "cfg4 conv2d forward (incl. output allocation)", "ms": round(ms, 5),
+                 "GFLOP/s": round(1.850e9 / ms / 1e6, 1)})
+    ms = time_launches(tt, lambda: be.conv2d_backward(go, x, w, None, 1, 1), 50, 5)
+    rows.append({"case": "cfg4 conv2d backward (data + weight, incl. allocations and sync)", "ms": round(ms, 5),
+                 "GFLOP/s": round(3.700e9 / ms / 1e6, 1)})
+    with open(path, "w") as f:
+        json.dump(rows, f, indent=1)
+    for r in rows:
+        print(json.dumps(r), file=sys.stderr)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -72,6 +151,7 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="first run one dense 256 MiB copy kernel (known HBM traffic) to scale profiler byte counters")
+    ap.add_argument("--detail", metavar="FILE", help="also time every BASELINE configuration and write a JSON report")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
@@ -86,6 +166,9 @@ def main():
         src = tt.Tensor.empty((64 * 1024 * 1024,), tt._capi.F32)
         tt.get_backend(tt.kAMD).identity(tt.Tensor(src.storage, src.dtype, (8192, 8192), (8192, 1), 0))
         tt.get_backend(tt.kAMD).synchronize(0)
+
+    if args.detail:
+        detail_report(tt, np, args.detail)
 
     n = args.n
     flop = 2.0 * n * n * n
