@@ -208,7 +208,7 @@ def test_unaligned_views_fall_back_to_elementwise_loads(tt, oracle, dtype):
     tA = tt.Tensor(tt.Tensor.from_numpy(baseA).storage, code, (1, N, K), (N * K, K, 1), 1)
     tB = tt.Tensor(tt.Tensor.from_numpy(baseB).storage, code, (1, K, M), (K * M, M, 1), 1)
     be = tt.get_backend(tt.kAMD)
-    assert be.batched_matmul_variant(tA, tB).endswith("akc1_bmc1")
+    assert "akc1_bmc1" in be.batched_matmul_variant(tA, tB)
     got = be.batched_matmul(tA, tB).to_numpy()[0]
     A, B = baseA[1:].reshape(N, K), baseB[1:].reshape(K, M)
     check_close(got, oracle.matmul(A, B), A, B, dtype)
@@ -226,7 +226,10 @@ def test_variant_selection(tt):
     small = tt.Tensor.from_numpy(np.zeros((1, 256, 512), f32))
     assert be.batched_matmul_variant(small, small.permute(0, 2, 1)).startswith("mfma_f32_64x64")
     thin = tt.Tensor.from_numpy(np.zeros((1, 512, 10), f32))
-    assert be.batched_matmul_variant(small, thin).startswith("simt_f32_128x16")
+    assert be.batched_matmul_variant(small, thin).startswith("mfma_f32_64x64_akc4_bmc1_splitk")  # few tiles, long K
+    thin_i = tt.Tensor.from_numpy(np.zeros((1, 512, 10), np.int32))
+    small_i = tt.Tensor.from_numpy(np.zeros((1, 256, 512), np.int32))
+    assert be.batched_matmul_variant(small_i, thin_i) == "simt_i32_128x16"
     i32 = tt.Tensor.from_numpy(np.zeros((1, 64, 64), np.int32))
     assert be.batched_matmul_variant(i32, i32) == "simt_i32_64x64"
 
@@ -266,7 +269,7 @@ def test_epilogue_bias_relu_accumulate(tt, oracle, dtype):
     rb = rng.integers(-4, 5, (200,)).astype(dtype)
     got = be.batched_matmul(dev(tt, X[None]), dev(tt, W[None]), bias=dev(tt, rb), bias_mode=2).to_numpy()[0]
     assert np.array_equal(got, X @ W + rb[:, None])
-    # thin output (vector-ALU kernel) takes the same epilogue
+    # thin output (split-K path: the epilogue runs in the reduction kernel) takes the same epilogue
     W10 = rng.integers(-4, 5, (96, 10)).astype(dtype)
     b10 = rng.integers(-4, 5, (10,)).astype(dtype)
     got = tt.linear(dev(tt, X), dev(tt, W10), dev(tt, b10), relu=True).to_numpy()

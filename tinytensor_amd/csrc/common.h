@@ -40,6 +40,11 @@ inline size_t dtype_size(ttamd_dtype dt) {
         }                                                                                      \
     } while (0)
 
+// Device scratch owned by the library, one growing buffer per (device, stream): kernels enqueued on one stream
+// run in order, so consecutive calls on that stream may share it; calls on different streams get different
+// buffers.  Growing allocates (hipMalloc) and frees the old buffer (hipFree, which waits for the device).
+ttamd_status stream_scratch(int device, hipStream_t stream, size_t bytes, void **out);
+
 // One GEMM problem as the kernels see it.  Conventional letters inside the kernels:
 // C[M,N] = A[M,K] . B[K,N]  (the C ABI's N,K,M map to M,K,N here).
 // Pointers already include the view's element offset.
@@ -56,7 +61,7 @@ struct GemmArgs {
 
 // Launchers (defined in gemm_mfma.hip / gemm_simt.hip).  `variant_only`: fill *variant with the
 // kernel name that would run and return without launching.
-ttamd_status launch_gemm_mfma(ttamd_dtype dt, const GemmArgs &g, hipStream_t stream, const char **variant,
+ttamd_status launch_gemm_mfma(ttamd_dtype dt, const GemmArgs &g, int device, hipStream_t stream, const char **variant,
                               bool variant_only, bool *handled);
 ttamd_status launch_gemm_simt(ttamd_dtype dt, const GemmArgs &g, hipStream_t stream, const char **variant,
                               bool variant_only);

@@ -94,7 +94,7 @@ ttamd_status ttamd_batched_matmul(int device, ttamd_dtype dtype, int B, int N, i
     const char *variant = nullptr;
     bool handled = false;
     if (K > 0) {
-        if (ttamd_status s = launch_gemm_mfma(dtype, g, st, &variant, false, &handled)) return s;
+        if (ttamd_status s = launch_gemm_mfma(dtype, g, device, st, &variant, false, &handled)) return s;
         if (handled) return TTAMD_OK;
     }
     // K == 0 also lands here: the vector-ALU kernel then stores the empty sum (0, + bias).
@@ -109,7 +109,7 @@ const char *ttamd_batched_matmul_variant(ttamd_dtype dtype, int B, int N, int K,
     const char *variant = "none";
     bool handled = false;
     if (K > 0) {
-        if (launch_gemm_mfma(dtype, g, nullptr, &variant, true, &handled) != TTAMD_OK) return "invalid";
+        if (launch_gemm_mfma(dtype, g, 0, nullptr, &variant, true, &handled) != TTAMD_OK) return "invalid";
         if (handled) return variant;
     }
     if (launch_gemm_simt(dtype, g, nullptr, &variant, true) != TTAMD_OK) return "invalid";

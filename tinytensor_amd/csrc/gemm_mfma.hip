@@ -14,8 +14,11 @@ namespace {
 
 using namespace mfma;
 
+// ksplit > 1: the reduction is cut into `ksplit` ranges of `k_chunk` (a multiple of BK); workgroup column z =
+// batch * ksplit + split writes the raw partial tile to `partial[z]` and splitk_reduce_kernel finishes the job.
 template <typename T, int BM, int BN, int BK, int WGM, int WGN, bool A_KC, int A_VEC, bool B_KC, int B_VEC>
-__global__ void __launch_bounds__(kThreads, 2) gemm_mfma_kernel(GemmArgs g, int tiles_m, int tiles_n) {
+__global__ void __launch_bounds__(kThreads, 2)
+gemm_mfma_kernel(GemmArgs g, int tiles_m, int tiles_n, int ksplit, int k_chunk, T *partial) {
     using StA = Stager<T, BM, BK, A_KC, A_VEC>;
     using StB = Stager<T, BN, BK, B_KC, B_VEC>;
     using Engine = TileEngine<T, BM, BN, BK, WGM, WGN, StA, StB>;
@@ -23,24 +26,53 @@ __global__ void __launch_bounds__(kThreads, 2) gemm_mfma_kernel(GemmArgs g, int 
     T *const smem = reinterpret_cast<T *>(smem_raw);
 
     const int tid = threadIdx.x;
-    int batch, tm, tn;
-    decode_tile(remap_xcd(blockIdx.x, gridDim.x), tiles_m, tiles_n, batch, tm, tn);
+    int z, tm, tn;
+    decode_tile(remap_xcd(blockIdx.x, gridDim.x), tiles_m, tiles_n, z, tm, tn);
+    const int batch = z / ksplit, split = z - batch * ksplit;
+    const int k0 = split * k_chunk;
+    const int Kc = (g.K - k0) < k_chunk ? (g.K - k0) : k_chunk;
     const int m0 = tm * BM, n0 = tn * BN;
 
-    // Operand bases at the tile's first row / column; the stagers size their buffer extents from there.
-    const T *a_base = static_cast<const T *>(g.A) + static_cast<int64_t>(batch) * g.a_sb + static_cast<int64_t>(m0) * g.a_sm;
-    const T *b_base = static_cast<const T *>(g.B) + static_cast<int64_t>(batch) * g.b_sb + static_cast<int64_t>(n0) * g.b_sn;
+    // Operand bases at the tile's first row / column and first k; the stagers size their buffer extents from there.
+    const T *a_base = static_cast<const T *>(g.A) + static_cast<int64_t>(batch) * g.a_sb + static_cast<int64_t>(m0) * g.a_sm +
+                      static_cast<int64_t>(k0) * g.a_sk;
+    const T *b_base = static_cast<const T *>(g.B) + static_cast<int64_t>(batch) * g.b_sb + static_cast<int64_t>(n0) * g.b_sn +
+                      static_cast<int64_t>(k0) * g.b_sk;
     StA sa;
     StB sb;
-    sa.init(a_base, tid, g.M - m0, g.a_sm, g.a_sk, g.K);
-    sb.init(b_base, tid, g.N - n0, g.b_sn, g.b_sk, g.K);
+    sa.init(a_base, tid, g.M - m0, g.a_sm, g.a_sk, Kc);
+    sb.init(b_base, tid, g.N - n0, g.b_sn, g.b_sk, Kc);
 
     Engine eng;
     eng.init(tid);
-    eng.run(sa, sb, smem, g.K, !sa.edge && !sb.edge && g.K % BK == 0);
+    eng.run(sa, sb, smem, Kc, !sa.edge && !sb.edge && Kc % BK == 0);
 
-    T *C = static_cast<T *>(g.C) + static_cast<int64_t>(batch) * g.M * g.N;
-    store_tile_dense<T>(eng, C, g.M, g.N, m0, n0, static_cast<const T *>(g.bias), g.bias_mode, g.relu, g.accumulate);
+    if (ksplit == 1) {
+        T *C = static_cast<T *>(g.C) + static_cast<int64_t>(batch) * g.M * g.N;
+        store_tile_dense<T>(eng, C, g.M, g.N, m0, n0, static_cast<const T *>(g.bias), g.bias_mode, g.relu, g.accumulate);
+    } else {
+        store_tile_dense<T>(eng, partial + static_cast<int64_t>(z) * g.M * g.N, g.M, g.N, m0, n0,
+                            static_cast<const T *>(nullptr), 0, 0, 0);
+    }
+}
+
+// C[b][i] = epilogue(sum over s of partial[b * ksplit + s][i]), s ascending (deterministic).
+template <typename T>
+__global__ void __launch_bounds__(256) splitk_reduce_kernel(GemmArgs g, const T *__restrict__ partial, int ksplit) {
+    const int64_t mn = static_cast<int64_t>(g.M) * g.N;
+    const int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (i >= mn) return;
+    const int batch = blockIdx.y;
+    const T *p = partial + static_cast<int64_t>(batch) * ksplit * mn + i;
+    T v = p[0];
+    for (int s = 1; s < ksplit; ++s) v += p[static_cast<int64_t>(s) * mn];
+    const T *bias = static_cast<const T *>(g.bias);
+    if (g.bias_mode == 1) v += bias[i % g.N];
+    if (g.bias_mode == 2) v += bias[i / g.N];
+    if (g.relu) v = v > T(0) ? v : T(0);
+    T *C = static_cast<T *>(g.C) + static_cast<int64_t>(batch) * mn;
+    if (g.accumulate) v += C[i];
+    C[i] = v;
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -62,8 +94,13 @@ OperandClass classify(const void *ptr, int64_t s_row, int64_t s_k, int64_t s_b, 
     return {s_k <= s_row, 1};
 }
 
+struct SplitPlan {
+    int ksplit = 1;
+    int k_chunk = 0;
+};
+
 template <typename T, int BM, int BN, int BK, int WGM, int WGN, bool A_KC, int A_VEC, bool B_KC, int B_VEC>
-ttamd_status launch_variant(const GemmArgs &g, hipStream_t stream) {
+ttamd_status launch_variant(const GemmArgs &g, const SplitPlan &sp, int device, hipStream_t stream) {
     using StA = Stager<T, BM, BK, A_KC, A_VEC>;
     using StB = Stager<T, BN, BK, B_KC, B_VEC>;
     constexpr size_t lds_bytes = TileEngine<T, BM, BN, BK, WGM, WGN, StA, StB>::kLdsBytes;
@@ -75,22 +112,35 @@ ttamd_status launch_variant(const GemmArgs &g, hipStream_t stream) {
         configured = true;
     }
     const int tiles_m = (g.M + BM - 1) / BM, tiles_n = (g.N + BN - 1) / BN;
-    const int64_t blocks = static_cast<int64_t>(tiles_m) * tiles_n * g.batch;
+    const int64_t blocks = static_cast<int64_t>(tiles_m) * tiles_n * g.batch * sp.ksplit;
     if (blocks > 0x7fffffff) {
         set_error("batched_matmul: %lld workgroups exceed the grid limit", static_cast<long long>(blocks));
         return TTAMD_ERR_INVALID_ARGUMENT;
     }
-    kernel<<<dim3(static_cast<unsigned>(blocks)), dim3(kThreads), lds_bytes, stream>>>(g, tiles_m, tiles_n);
+    T *partial = nullptr;
+    if (sp.ksplit > 1) {
+        void *ws = nullptr;
+        const size_t bytes = static_cast<size_t>(sp.ksplit) * g.batch * g.M * g.N * sizeof(T);
+        if (ttamd_status st = stream_scratch(device, stream, bytes, &ws)) return st;
+        partial = static_cast<T *>(ws);
+    }
+    kernel<<<dim3(static_cast<unsigned>(blocks)), dim3(kThreads), lds_bytes, stream>>>(g, tiles_m, tiles_n, sp.ksplit,
+                                                                                      sp.ksplit > 1 ? sp.k_chunk : g.K, partial);
     TTAMD_HIP_CHECK(hipGetLastError());
+    if (sp.ksplit > 1) {
+        const int64_t mn = static_cast<int64_t>(g.M) * g.N;
+        splitk_reduce_kernel<T><<<dim3(static_cast<unsigned>((mn + 255) / 256), g.batch), dim3(256), 0, stream>>>(g, partial, sp.ksplit);
+        TTAMD_HIP_CHECK(hipGetLastError());
+    }
     return TTAMD_OK;
 }
 
-template <typename T, int BM, int BN, int BK, int WGM, int WGN, int VEC>
-ttamd_status launch_layouts(const GemmArgs &g, bool a_kc, bool b_kc, hipStream_t stream) {
-    if (a_kc && b_kc) return launch_variant<T, BM, BN, BK, WGM, WGN, true, VEC, true, VEC>(g, stream);
-    if (a_kc && !b_kc) return launch_variant<T, BM, BN, BK, WGM, WGN, true, VEC, false, VEC>(g, stream);
-    if (!a_kc && b_kc) return launch_variant<T, BM, BN, BK, WGM, WGN, false, VEC, true, VEC>(g, stream);
-    return launch_variant<T, BM, BN, BK, WGM, WGN, false, VEC, false, VEC>(g, stream);
+template <typename T, int BM, int BN, int BK, int WGM, int WGN, int A_VEC, int B_VEC>
+ttamd_status launch_layouts(const GemmArgs &g, bool a_kc, bool b_kc, const SplitPlan &sp, int device, hipStream_t stream) {
+    if (a_kc && b_kc) return launch_variant<T, BM, BN, BK, WGM, WGN, true, A_VEC, true, B_VEC>(g, sp, device, stream);
+    if (a_kc && !b_kc) return launch_variant<T, BM, BN, BK, WGM, WGN, true, A_VEC, false, B_VEC>(g, sp, device, stream);
+    if (!a_kc && b_kc) return launch_variant<T, BM, BN, BK, WGM, WGN, false, A_VEC, true, B_VEC>(g, sp, device, stream);
+    return launch_variant<T, BM, BN, BK, WGM, WGN, false, A_VEC, false, B_VEC>(g, sp, device, stream);
 }
 
 template <typename T>
@@ -108,14 +158,39 @@ struct TileShapes<double> {
     static constexpr const char *prefix = "mfma_f64";
 };
 
+// Split the reduction when the output has too few tiles to fill 256 CUs and K is long enough to share out.
+// Every split gets a whole number of BK tiles; at most 64 splits and 32 MiB of partial tiles.
 template <typename T>
-ttamd_status launch_mfma_typed(const GemmArgs &g, hipStream_t stream, const char **variant, bool variant_only,
+SplitPlan plan_split(const GemmArgs &g, int bm, int bn, int bk) {
+    SplitPlan sp;
+    sp.k_chunk = g.K;
+    const int64_t tiles = static_cast<int64_t>((g.M + bm - 1) / bm) * ((g.N + bn - 1) / bn) * g.batch;
+    const int k_tiles = (g.K + bk - 1) / bk;
+    if (tiles >= 128 || k_tiles < 4 || g.batch > 65535) return sp;
+    int want = static_cast<int>((256 + tiles - 1) / tiles);
+    const int max_by_k = k_tiles / 2;  // at least two k tiles per split
+    if (want > max_by_k) want = max_by_k;
+    if (want > 64) want = 64;
+    const int64_t bytes_per_split = static_cast<int64_t>(g.batch) * g.M * g.N * static_cast<int64_t>(sizeof(T));
+    const int64_t cap = (32LL << 20) / (bytes_per_split > 0 ? bytes_per_split : 1);
+    if (want > cap) want = static_cast<int>(cap);
+    if (want < 2) return sp;
+    const int chunk_tiles = (k_tiles + want - 1) / want;
+    sp.k_chunk = chunk_tiles * bk;
+    sp.ksplit = (g.K + sp.k_chunk - 1) / sp.k_chunk;
+    if (sp.ksplit < 2) {
+        sp.ksplit = 1;
+        sp.k_chunk = g.K;
+    }
+    return sp;
+}
+
+template <typename T>
+ttamd_status launch_mfma_typed(const GemmArgs &g, int device, hipStream_t stream, const char **variant, bool variant_only,
                                bool *handled) {
     using TS = TileShapes<T>;
     constexpr int VK = Mfma<T>::VK;
     *handled = false;
-    // Very thin outputs leave a 64-wide MFMA tile almost empty: those go to the vector-ALU kernel.
-    if (g.M <= 16 || g.N <= 16) return TTAMD_OK;
 
     OperandClass ca = classify<T>(g.A, g.a_sm, g.a_sk, g.a_sb, g.batch);
     OperandClass cb = classify<T>(g.B, g.b_sn, g.b_sk, g.b_sb, g.batch);
@@ -130,25 +205,32 @@ ttamd_status launch_mfma_typed(const GemmArgs &g, hipStream_t stream, const char
     const int64_t b_reach = (static_cast<int64_t>(bm - 1) * g.b_sn + static_cast<int64_t>(g.K - 1) * g.b_sk + VK) * sizeof(T);
     if (a_reach >= 0x7fffffffLL || b_reach >= 0x7fffffffLL) return TTAMD_OK;
 
-    static thread_local char name[96];
-    snprintf(name, sizeof(name), "%s_%s_a%s%d_b%s%d", TS::prefix, large ? "128x128" : "64x64", ca.kc ? "kc" : "mc",
-             vec ? VK : 1, cb.kc ? "kc" : "mc", vec ? VK : 1);
+    const SplitPlan sp = large ? SplitPlan{1, g.K} : plan_split<T>(g, TS::SBM, TS::SBN, TS::SBK);
+
+    static thread_local char name[112];
+    char split_tag[24] = "";
+    if (sp.ksplit > 1) snprintf(split_tag, sizeof(split_tag), "_splitk%d", sp.ksplit);
+    snprintf(name, sizeof(name), "%s_%s_a%s%d_b%s%d%s", TS::prefix, large ? "128x128" : "64x64", ca.kc ? "kc" : "mc",
+             ca.vec, cb.kc ? "kc" : "mc", cb.vec, split_tag);
     *variant = name;
     *handled = true;
     if (variant_only) return TTAMD_OK;
 
-    if (large) return launch_layouts<T, TS::LBM, TS::LBN, TS::LBK, 2, 2, VK>(g, ca.kc, cb.kc, stream);
-    if (vec) return launch_layouts<T, TS::SBM, TS::SBN, TS::SBK, 2, 2, VK>(g, ca.kc, cb.kc, stream);
-    return launch_layouts<T, TS::SBM, TS::SBN, TS::SBK, 2, 2, 1>(g, ca.kc, cb.kc, stream);
+    // The large tile exists for 16-byte operands only; the small tile for every mix of 16-byte and element-wise.
+    if (large) return launch_layouts<T, TS::LBM, TS::LBN, TS::LBK, 2, 2, VK, VK>(g, ca.kc, cb.kc, sp, device, stream);
+    if (ca.vec > 1 && cb.vec > 1) return launch_layouts<T, TS::SBM, TS::SBN, TS::SBK, 2, 2, VK, VK>(g, ca.kc, cb.kc, sp, device, stream);
+    if (ca.vec > 1) return launch_layouts<T, TS::SBM, TS::SBN, TS::SBK, 2, 2, VK, 1>(g, ca.kc, cb.kc, sp, device, stream);
+    if (cb.vec > 1) return launch_layouts<T, TS::SBM, TS::SBN, TS::SBK, 2, 2, 1, VK>(g, ca.kc, cb.kc, sp, device, stream);
+    return launch_layouts<T, TS::SBM, TS::SBN, TS::SBK, 2, 2, 1, 1>(g, ca.kc, cb.kc, sp, device, stream);
 }
 
 }  // namespace
 
-ttamd_status launch_gemm_mfma(ttamd_dtype dt, const GemmArgs &g, hipStream_t stream, const char **variant,
+ttamd_status launch_gemm_mfma(ttamd_dtype dt, const GemmArgs &g, int device, hipStream_t stream, const char **variant,
                               bool variant_only, bool *handled) {
     *handled = false;
-    if (dt == TTAMD_F32) return launch_mfma_typed<float>(g, stream, variant, variant_only, handled);
-    if (dt == TTAMD_F64) return launch_mfma_typed<double>(g, stream, variant, variant_only, handled);
+    if (dt == TTAMD_F32) return launch_mfma_typed<float>(g, device, stream, variant, variant_only, handled);
+    if (dt == TTAMD_F64) return launch_mfma_typed<double>(g, device, stream, variant, variant_only, handled);
     return TTAMD_OK;
 }
 

@@ -114,11 +114,18 @@ __device__ __forceinline__ void zero_component(typename Vec<T, VEC>::type &v, in
 }
 
 // Raw buffer descriptor over [base, base + bytes), bytes clamped to 2^31 - 1 (offsets >= 2^31 are the
-// out-of-range marker).
+// out-of-range marker).  Base and size are the same for every lane of a workgroup; they are passed through
+// readfirstlane so that the descriptor provably lives in scalar registers (otherwise each buffer load is
+// wrapped in a waterfall loop, which also fences the instruction scheduler).
 template <typename T>
 __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const T *base, int64_t bytes) {
-    const int rec = bytes > 0x7fffffff ? 0x7fffffff : (bytes < 0 ? 0 : static_cast<int>(bytes));
-    return __builtin_amdgcn_make_buffer_rsrc(const_cast<T *>(base), 0, rec, 0x00020000);
+    int rec = bytes > 0x7fffffff ? 0x7fffffff : (bytes < 0 ? 0 : static_cast<int>(bytes));
+    const uint64_t addr = reinterpret_cast<uint64_t>(base);
+    const uint32_t lo = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(addr));
+    const uint32_t hi = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(addr >> 32));
+    rec = __builtin_amdgcn_readfirstlane(rec);
+    T *uniform_base = reinterpret_cast<T *>((static_cast<uint64_t>(hi) << 32) | lo);
+    return __builtin_amdgcn_make_buffer_rsrc(uniform_base, 0, rec, 0x00020000);
 }
 
 // LDS geometry shared by every stager of a given layout.
@@ -364,7 +371,11 @@ struct TileEngine {
                 const int k_left = K - (kt + 1) * BK;
                 sa.template load<MASK>(k_left);
                 sb.template load<MASK>(k_left);
+                // Keep the global loads ahead of the MFMA work: left alone, the scheduler sinks them to just
+                // before the LDS stores and their latency is exposed on every tile.
+                __builtin_amdgcn_sched_barrier(0);
                 compute(smem, cur);
+                __builtin_amdgcn_sched_barrier(0);
                 sa.store(smem + (cur ^ 1) * StA::LDS_ELEMS);
                 sb.store(smem + kBOff + (cur ^ 1) * StB::LDS_ELEMS);
                 __syncthreads();

@@ -5,6 +5,9 @@
 
 #include <atomic>
 #include <cstring>
+#include <map>
+#include <mutex>
+#include <utility>
 
 namespace ttamd {
 
@@ -33,6 +36,33 @@ ttamd_status use_device(int device) {
         return TTAMD_ERR_INVALID_DEVICE;
     }
     TTAMD_HIP_CHECK(hipSetDevice(device));
+    return TTAMD_OK;
+}
+
+ttamd_status stream_scratch(int device, hipStream_t stream, size_t bytes, void **out) {
+    struct Buf {
+        void *ptr = nullptr;
+        size_t bytes = 0;
+    };
+    static std::mutex mu;
+    static std::map<std::pair<int, hipStream_t>, Buf> bufs;  // lives until the process ends
+    std::lock_guard<std::mutex> lock(mu);
+    Buf &b = bufs[{device, stream}];
+    if (b.bytes < bytes) {
+        size_t want = bytes < (size_t(4) << 20) ? (size_t(4) << 20) : bytes;
+        want = (want + 255) & ~size_t(255);
+        void *p = nullptr;
+        hipError_t e = hipMalloc(&p, want);
+        if (e != hipSuccess) {
+            (void)hipGetLastError();
+            set_error("Unable to allocate %zu bytes of scratch on AMD device %d: %s", want, device, hipGetErrorString(e));
+            return TTAMD_ERR_OUT_OF_MEMORY;
+        }
+        if (b.ptr) TTAMD_HIP_CHECK(hipFree(b.ptr));  // waits for kernels that may still read the old buffer
+        b.ptr = p;
+        b.bytes = want;
+    }
+    *out = b.ptr;
     return TTAMD_OK;
 }
 
