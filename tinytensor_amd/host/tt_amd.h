@@ -1,0 +1,425 @@
+// tt_amd.h — C++20 host side of the AMD GEMM backend: the slice of tinytensor's Tensor / backend interface that
+// the GEMM path needs, written over the C ABI of include/ttamd.h.  Header-only; link with libttamd.so.
+//
+// It mirrors the reference's names, argument meaning and error behaviour so that code (and tests) written
+// against tinytensor read the same here:
+//   Tensor(std::vector<T>, Shape, Device) / to_vec<T>()      include/tt/tensor.h:134-189, 370
+//   shape/stride/offset/permute/reshape/expand/...           include/tt/tensor.h:245-283, 600-650 (views only
+//                                                            rewrite shape/stride/offset, autograd/shape_ops.cpp:24-146)
+//   matmul(lhs, rhs)                                         tinytensor/tensor/tensor.cpp:2390-2484
+//   matmul backward (dA = dC.B^T, dB = A^T.dC on views)       tinytensor/autograd/binary_ops.cpp:165-179
+//   conv2d / conv2d_backward                                 tinytensor/tensor/tensor.cpp:3089-3167, backend_base.h:269-284
+//   nn::Linear                                               tinytensor/nn/linear.cpp:20-50
+//   BackendAMD (the BackendBase methods on the path)         tinytensor/tensor/backend_base.h:23-322
+//   TTException                                              include/tt/exception.h:15-25
+// All arithmetic runs in libttamd.so; there is no CPU fallback.
+#ifndef TT_AMD_HOST_H_
+#define TT_AMD_HOST_H_
+
+#include <algorithm>
+#include <cstdint>
+#include <cstdlib>
+#include <exception>
+#include <iostream>
+#include <memory>
+#include <numeric>
+#include <optional>
+#include <string>
+#include <tuple>
+#include <type_traits>
+#include <utility>
+#include <vector>
+
+#include "ttamd.h"
+
+namespace tt_amd {
+
+class TTException : public std::exception {
+public:
+    explicit TTException(std::string message) : message_(std::move(message)) {}
+    [[nodiscard]] auto what() const noexcept -> const char * override { return message_.c_str(); }
+
+private:
+    std::string message_;
+};
+
+// Status -> the reference's error model: TTException for user-visible problems, print + exit(1) for
+// unrecoverable device failures (TT_ERROR, include/tt/exception.h:28-36).
+inline void check(ttamd_status s) {
+    if (s == TTAMD_OK) return;
+    if (s == TTAMD_ERR_LAUNCH) {
+        std::cout << ttamd_last_error_string() << std::endl;
+        std::exit(1);
+    }
+    throw TTException(ttamd_last_error_string());
+}
+
+enum class ScalarType { bool8 = 0, u8, i16, i32, i64, f32, f64 };  // include/tt/scalar.h:21-29
+constexpr ScalarType kBool = ScalarType::bool8, kU8 = ScalarType::u8, kI16 = ScalarType::i16, kI32 = ScalarType::i32,
+                     kI64 = ScalarType::i64, kF32 = ScalarType::f32, kF64 = ScalarType::f64;
+
+template <typename T>
+struct to_scalar;
+template <> struct to_scalar<bool> { static constexpr ScalarType type = kBool; };
+template <> struct to_scalar<uint8_t> { static constexpr ScalarType type = kU8; };
+template <> struct to_scalar<int16_t> { static constexpr ScalarType type = kI16; };
+template <> struct to_scalar<int32_t> { static constexpr ScalarType type = kI32; };
+template <> struct to_scalar<int64_t> { static constexpr ScalarType type = kI64; };
+template <> struct to_scalar<float> { static constexpr ScalarType type = kF32; };
+template <> struct to_scalar<double> { static constexpr ScalarType type = kF64; };
+
+inline auto dtype_size(ScalarType t) -> std::size_t {
+    switch (t) {
+    case kBool: case kU8: return 1;
+    case kI16: return 2;
+    case kI32: case kF32: return 4;
+    default: return 8;
+    }
+}
+inline auto promote_types(ScalarType a, ScalarType b) -> ScalarType { return static_cast<int>(a) > static_cast<int>(b) ? a : b; }
+
+enum class Backend { amd };
+struct Device {
+    Backend backend;
+    int id;
+    constexpr auto operator==(const Device &other) const -> bool { return backend == other.backend && id == other.id; }
+};
+constexpr Device kAMD = Device{Backend::amd, 0};
+
+class Shape {  // include/tt/shape.h:20-123
+public:
+    Shape() = default;
+    explicit Shape(std::vector<int> dims) : dims_(std::move(dims)) {}
+    Shape(std::initializer_list<int> dims) : dims_(dims) {}
+    [[nodiscard]] auto numel() const noexcept -> int {
+        return std::accumulate(dims_.begin(), dims_.end(), 1, [](int a, int b) { return a * b; });
+    }
+    [[nodiscard]] auto ndim() const noexcept -> int { return static_cast<int>(dims_.size()); }
+    [[nodiscard]] auto size() const noexcept -> int { return ndim(); }
+    auto operator[](int i) -> int & { return dims_.at(static_cast<std::size_t>(i < 0 ? i + ndim() : i)); }
+    auto operator[](int i) const -> int { return dims_.at(static_cast<std::size_t>(i < 0 ? i + ndim() : i)); }
+    [[nodiscard]] auto to_vec() const -> const std::vector<int> & { return dims_; }
+    auto operator==(const Shape &o) const -> bool { return dims_ == o.dims_; }
+
+private:
+    std::vector<int> dims_;
+};
+
+// Owning device allocation (peer of the reference's DeviceMemory<T>, cuda/data_types.cuh:28-101).
+class StorageAMD {
+public:
+    StorageAMD(std::size_t bytes, int device_id) : bytes_(bytes ? bytes : 1), device_(device_id) {
+        check(ttamd_malloc(device_, bytes_, &ptr_));
+    }
+    ~StorageAMD() { ttamd_free(device_, ptr_, bytes_); }
+    StorageAMD(const StorageAMD &) = delete;
+    StorageAMD &operator=(const StorageAMD &) = delete;
+    void *ptr_ = nullptr;
+    std::size_t bytes_;
+    int device_;
+};
+
+class Tensor;
+class BackendAMD;
+inline auto get_backend(Device device) -> const BackendAMD *;
+
+class Tensor {
+public:
+    Tensor() = default;
+    // Tensor(std::vector<T>, Shape, Device): uploads through BackendBase::from_vec.
+    template <typename T>
+    Tensor(const std::vector<T> &data, Shape shape, Device device);
+    template <typename T>
+    Tensor(const std::vector<T> &data, Device device) : Tensor(data, Shape({static_cast<int>(data.size())}), device) {}
+    // Internal constructor of backend results (tensor.cpp:351-358) and of views.
+    Tensor(std::shared_ptr<StorageAMD> storage, ScalarType dtype, Shape shape, Device device)
+        : storage_(std::move(storage)), dtype_(dtype), shape_(std::move(shape)), stride_(dense_stride(shape_)), device_(device) {}
+    Tensor(std::shared_ptr<StorageAMD> storage, ScalarType dtype, Shape shape, Shape stride, int offset, Device device)
+        : storage_(std::move(storage)), dtype_(dtype), shape_(std::move(shape)), stride_(std::move(stride)), offset_(offset),
+          device_(device) {}
+
+    [[nodiscard]] auto dtype() const -> ScalarType { return dtype_; }
+    [[nodiscard]] auto device() const -> Device { return device_; }
+    [[nodiscard]] auto offset() const -> int { return offset_; }
+    [[nodiscard]] auto shape() const -> const Shape & { return shape_; }
+    [[nodiscard]] auto stride() const -> const Shape & { return stride_; }
+    [[nodiscard]] auto numel() const -> int { return shape_.numel(); }
+    [[nodiscard]] auto dim() const -> int { return shape_.ndim(); }
+    [[nodiscard]] auto size(int d) const -> int { return shape_[d]; }
+    [[nodiscard]] auto is_contiguous() const -> bool { return stride_ == dense_stride(shape_); }
+    [[nodiscard]] auto storage() const -> const std::shared_ptr<StorageAMD> & { return storage_; }
+    [[nodiscard]] auto data_ptr() const -> void * {
+        return static_cast<char *>(storage_->ptr_) + static_cast<std::size_t>(offset_) * dtype_size(dtype_);
+    }
+
+    [[nodiscard]] auto contiguous() const -> Tensor;  // tensor.cpp:583-591
+    [[nodiscard]] auto permute(const std::vector<int> &dims) const -> Tensor {
+        if (static_cast<int>(dims.size()) != dim()) throw TTException("permute: wrong number of dimensions");
+        std::vector<int> sh, st, seen(dims.size(), 0);
+        for (int d : dims) {
+            if (d < 0 || d >= dim() || seen[static_cast<std::size_t>(d)]++) throw TTException("permute: invalid permutation");
+            sh.push_back(shape_[d]);
+            st.push_back(stride_[d]);
+        }
+        return {storage_, dtype_, Shape(sh), Shape(st), offset_, device_};
+    }
+    [[nodiscard]] auto unsqueeze(int d) const -> Tensor {
+        if (d < 0) d += dim() + 1;
+        auto sh = shape_.to_vec(), st = stride_.to_vec();
+        sh.insert(sh.begin() + d, 1);
+        st.insert(st.begin() + d, 0);  // a size-1 dimension is never stepped over: a pure view, no clone
+        return {storage_, dtype_, Shape(sh), Shape(st), offset_, device_};
+    }
+    [[nodiscard]] auto squeeze(int d) const -> Tensor {
+        if (shape_[d] != 1) return *this;
+        auto sh = shape_.to_vec(), st = stride_.to_vec();
+        if (d < 0) d += dim();
+        sh.erase(sh.begin() + d);
+        st.erase(st.begin() + d);
+        return {storage_, dtype_, Shape(sh), Shape(st), offset_, device_};
+    }
+    [[nodiscard]] auto expand(const Shape &shape) const -> Tensor {
+        if (shape.ndim() != dim()) throw TTException("expand: rank mismatch");
+        std::vector<int> st;
+        for (int i = 0; i < dim(); ++i) {
+            if (shape_[i] == shape[i]) st.push_back(stride_[i]);
+            else if (shape_[i] == 1) st.push_back(0);
+            else throw TTException("expand: incompatible shape");
+        }
+        return {storage_, dtype_, shape, Shape(st), offset_, device_};
+    }
+    [[nodiscard]] auto reshape(const Shape &shape) const -> Tensor {  // a view when dense, a clone otherwise (tensor.cpp:1371-1387)
+        if (shape.numel() != numel()) throw TTException("reshape: element counts differ");
+        const Tensor base = contiguous();
+        return {base.storage_, dtype_, shape, dense_stride(shape), base.offset_, device_};
+    }
+    [[nodiscard]] auto flatten(int start_dim = 0, int end_dim = -1) const -> Tensor {
+        if (dim() == 0) return reshape(Shape({1}));
+        if (start_dim < 0) start_dim += dim();
+        if (end_dim < 0) end_dim += dim();
+        std::vector<int> sh;
+        int merged = 1;
+        for (int i = 0; i < dim(); ++i) {
+            if (i < start_dim || i > end_dim) sh.push_back(shape_[i]);
+            else {
+                merged *= shape_[i];
+                if (i == end_dim) sh.push_back(merged);
+            }
+        }
+        return reshape(Shape(sh));
+    }
+    template <typename T>
+    [[nodiscard]] auto to_vec() const -> std::vector<T>;  // dense host copy of this view (tensor.cpp:555)
+
+    static auto dense_stride(const Shape &shape) -> Shape {
+        std::vector<int> st(static_cast<std::size_t>(shape.ndim()), 1);
+        for (int i = shape.ndim() - 2; i >= 0; --i) st[static_cast<std::size_t>(i)] = st[static_cast<std::size_t>(i) + 1] * shape[i + 1];
+        return Shape(st);
+    }
+
+private:
+    std::shared_ptr<StorageAMD> storage_;
+    ScalarType dtype_ = kF32;
+    Shape shape_, stride_;
+    int offset_ = 0;
+    Device device_ = kAMD;
+};
+
+// The BackendBase methods that the GEMM path uses (tinytensor/tensor/backend_base.h:23-322).
+class BackendAMD {
+public:
+    template <typename T>
+    [[nodiscard]] auto from_vec(const std::vector<T> &data, int device_id) const -> std::shared_ptr<StorageAMD> {
+        static_assert(!std::is_same_v<T, bool>, "upload bool data as uint8_t");
+        auto st = std::make_shared<StorageAMD>(data.size() * sizeof(T), device_id);
+        check(ttamd_memcpy_h2d(device_id, st->ptr_, data.data(), data.size() * sizeof(T)));
+        return st;
+    }
+    // to_vec fills the host vector with the WHOLE storage (backend_base.h:55-60).
+    template <typename T>
+    void to_vec(const Tensor &tensor, std::vector<T> &data_out) const {
+        const auto &st = tensor.storage();
+        data_out.resize(st->bytes_ / sizeof(T));
+        check(ttamd_memcpy_d2h(st->device_, data_out.data(), st->ptr_, data_out.size() * sizeof(T)));
+    }
+    [[nodiscard]] auto identity(const Tensor &t) const -> Tensor {  // clone of a view into dense storage
+        auto out = std::make_shared<StorageAMD>(static_cast<std::size_t>(t.numel()) * dtype_size(t.dtype()), t.device().id);
+        std::vector<int64_t> sh(t.shape().to_vec().begin(), t.shape().to_vec().end()), st(t.stride().to_vec().begin(), t.stride().to_vec().end());
+        check(ttamd_contiguous(t.device().id, static_cast<ttamd_dtype>(t.dtype()), t.dim(), sh.data(), st.data(), t.storage()->ptr_,
+                               t.offset(), out->ptr_, nullptr));
+        return {out, t.dtype(), t.shape(), t.device()};
+    }
+    // BackendBase::batched_matmul (backend_base.h:130): operands are read in place, whatever their strides.
+    [[nodiscard]] auto batched_matmul(const Tensor &lhs, const Tensor &rhs, const ttamd_epilogue *epilogue = nullptr) const -> Tensor {
+        const int B = lhs.size(0), N = lhs.size(1), K = lhs.size(2), M = rhs.size(2);
+        const ttamd_view3 l = view3(lhs), r = view3(rhs);
+        auto out = std::make_shared<StorageAMD>(static_cast<std::size_t>(B) * N * M * dtype_size(lhs.dtype()), lhs.device().id);
+        check(ttamd_batched_matmul(lhs.device().id, static_cast<ttamd_dtype>(lhs.dtype()), B, N, K, M, &l, &r, out->ptr_, epilogue, nullptr));
+        return {out, lhs.dtype(), Shape({B, N, M}), lhs.device()};
+    }
+    [[nodiscard]] auto conv2d(const Tensor &input, const Tensor &weight, const std::optional<Tensor> &bias, int stride, int padding) const
+        -> Tensor {
+        const int B = input.size(0), C = input.size(1), H = input.size(2), W = input.size(3), O = weight.size(0), k = weight.size(2);
+        const int Ho = (H + 2 * padding - k) / stride + 1, Wo = (W + 2 * padding - k) / stride + 1;
+        const Tensor w = weight.contiguous();  // used as the matrix [O, C*k*k], as cpu/conv.cpp:69 reshapes it
+        const std::optional<Tensor> b = bias ? std::optional<Tensor>(bias->contiguous()) : std::nullopt;
+        const ttamd_view4 iv = view4(input), wv = view4(w);
+        auto out = std::make_shared<StorageAMD>(static_cast<std::size_t>(std::max(B * O * Ho * Wo, 0)) * dtype_size(input.dtype()), input.device().id);
+        check(ttamd_conv2d_forward(input.device().id, static_cast<ttamd_dtype>(input.dtype()), &iv, &wv, b ? b->data_ptr() : nullptr, out->ptr_,
+                                   B, C, H, W, O, k, stride, padding, nullptr));
+        return {out, input.dtype(), Shape({B, O, Ho, Wo}), input.device()};
+    }
+    [[nodiscard]] auto conv2d_backward(const Tensor &grad_output, const Tensor &input, const Tensor &weight, const std::optional<Tensor> &bias,
+                                       int stride, int padding) const -> std::tuple<Tensor, Tensor, std::optional<Tensor>> {
+        const int B = input.size(0), C = input.size(1), H = input.size(2), W = input.size(3), O = weight.size(0), k = weight.size(2);
+        const int dev = input.device().id;
+        const auto dt = static_cast<ttamd_dtype>(input.dtype());
+        const std::size_t esz = dtype_size(input.dtype());
+        const Tensor go = grad_output.contiguous(), w = weight.contiguous();
+        auto gx = std::make_shared<StorageAMD>(static_cast<std::size_t>(input.numel()) * esz, dev);
+        auto gw = std::make_shared<StorageAMD>(static_cast<std::size_t>(weight.numel()) * esz, dev);
+        std::shared_ptr<StorageAMD> gb = bias ? std::make_shared<StorageAMD>(static_cast<std::size_t>(O) * esz, dev) : nullptr;
+        std::size_t ws_bytes = 0;
+        check(ttamd_conv2d_backward_workspace(dt, B, C, H, W, O, k, stride, padding, &ws_bytes));
+        StorageAMD ws(ws_bytes, dev);
+        const ttamd_view4 iv = view4(input), wv = view4(w);
+        check(ttamd_conv2d_backward(dev, dt, go.data_ptr(), &iv, &wv, gx->ptr_, gw->ptr_, gb ? gb->ptr_ : nullptr, B, C, H, W, O, k, stride,
+                                    padding, ws.ptr_, ws_bytes, nullptr));
+        check(ttamd_device_synchronize(dev));  // the workspace is released when this scope ends
+        std::optional<Tensor> grad_bias;
+        if (gb) grad_bias = Tensor(gb, input.dtype(), Shape({O}), input.device());
+        return {Tensor(gx, input.dtype(), input.shape(), input.device()), Tensor(gw, input.dtype(), weight.shape(), input.device()), grad_bias};
+    }
+    [[nodiscard]] auto current_memory_allocated(int device_id) const -> uint64_t {
+        uint64_t cur = 0, tot = 0;
+        check(ttamd_memory_allocated(device_id, &cur, &tot));
+        return cur;
+    }
+    [[nodiscard]] auto total_memory_allocated(int device_id) const -> uint64_t {
+        uint64_t cur = 0, tot = 0;
+        check(ttamd_memory_allocated(device_id, &cur, &tot));
+        return tot;
+    }
+    [[nodiscard]] auto get_device_count() const -> int {
+        int n = 0;
+        check(ttamd_device_count(&n));
+        return n;
+    }
+
+    static auto view3(const Tensor &t) -> ttamd_view3 {
+        return {t.storage()->ptr_, t.offset(), {t.stride()[0], t.stride()[1], t.stride()[2]}};
+    }
+    static auto view4(const Tensor &t) -> ttamd_view4 {
+        return {t.storage()->ptr_, t.offset(), {t.stride()[0], t.stride()[1], t.stride()[2], t.stride()[3]}};
+    }
+};
+
+inline auto get_backend(Device) -> const BackendAMD * {  // backend_register.cpp:19-38
+    static const std::unique_ptr<BackendAMD> backend = std::make_unique<BackendAMD>();
+    return backend.get();
+}
+
+template <typename T>
+Tensor::Tensor(const std::vector<T> &data, Shape shape, Device device) : dtype_(to_scalar<T>::type), shape_(std::move(shape)), device_(device) {
+    if (shape_.numel() != static_cast<int>(data.size())) throw TTException("Tensor: data size does not match the shape");
+    stride_ = dense_stride(shape_);
+    if constexpr (std::is_same_v<T, bool>) {
+        std::vector<uint8_t> bytes(data.begin(), data.end());  // bool is stored as uint8_t (backend_base.h:36-37)
+        storage_ = get_backend(device)->from_vec(bytes, device.id);
+    } else {
+        storage_ = get_backend(device)->from_vec(data, device.id);
+    }
+}
+
+inline auto Tensor::contiguous() const -> Tensor { return is_contiguous() ? *this : get_backend(device_)->identity(*this); }
+
+template <typename T>
+auto Tensor::to_vec() const -> std::vector<T> {
+    if (to_scalar<T>::type != dtype_) throw TTException("to_vec: element type does not match the tensor dtype");
+    const Tensor dense = contiguous();  // callers clone first (tensor.cpp:555), then the whole storage comes back
+    std::vector<T> whole;
+    get_backend(device_)->to_vec(dense, whole);
+    return {whole.begin() + dense.offset(), whole.begin() + dense.offset() + dense.numel()};
+}
+
+// tinytensor::matmul (tensor.cpp:2390-2484): rank dispatch onto batched_matmul; bool is rejected.
+inline auto matmul(const Tensor &lhs, const Tensor &rhs) -> Tensor {
+    if (!(lhs.device() == rhs.device())) throw TTException("Expected tensors on the same device");
+    const auto promoted = promote_types(lhs.dtype(), rhs.dtype());
+    if (promoted == kBool) throw TTException("matmul does not support boolean tensors");
+    if (lhs.dtype() != rhs.dtype()) throw TTException("mixed-dtype matmul needs a cast op, which this backend slice does not provide");
+    const auto *be = get_backend(lhs.device());
+    const auto &ls = lhs.shape(), &rs = rhs.shape();
+    if (ls.ndim() == 1 && rs.ndim() == 1) {
+        if (ls[0] != rs[0]) throw TTException("Invalid shapes for dot product. Both LHS and RHS must have same dimensions");
+        return be->batched_matmul(lhs.reshape({1, 1, ls[0]}), rhs.reshape({1, rs[0], 1})).flatten();
+    }
+    if (ls.ndim() == 1 && rs.ndim() == 2) {
+        if (ls[0] != rs[0]) throw TTException("Invalid shape for matrix multiplication. Length of LHS should equal size of RHS dimension 0");
+        return be->batched_matmul(lhs.reshape({1, 1, ls[0]}), rhs.unsqueeze(0)).flatten();
+    }
+    if (ls.ndim() == 2 && rs.ndim() == 1) {
+        if (ls[1] != rs[0]) throw TTException("Invalid shape for matrix multiplication. Length of RHS should equal size of LHS dimension 1");
+        return be->batched_matmul(lhs.unsqueeze(0), rhs.reshape({1, rs[0], 1})).flatten();
+    }
+    if (ls.ndim() == 2 && rs.ndim() == 2) {
+        if (ls[1] != rs[0]) throw TTException("Invalid shape for matrix multiplication. Size of LHS dimension 1 should equal size of RHS dimension 0");
+        return be->batched_matmul(lhs.unsqueeze(0), rhs.unsqueeze(0)).squeeze(0);
+    }
+    if (ls.ndim() == 3 && rs.ndim() == 3) {
+        if (ls[2] != rs[1] || ls[0] != rs[0]) throw TTException("Invalid shape for batched matrix multiplication");
+        return be->batched_matmul(lhs, rhs);
+    }
+    throw TTException("Unsupported sizes. Try reshaping or broadcasting.");
+}
+
+// TensorBatchedMatmul::backward (autograd/binary_ops.cpp:173-179): both gradients, on permuted VIEWS.
+inline auto matmul_backward(const Tensor &lhs, const Tensor &rhs, const Tensor &grad_output) -> std::pair<Tensor, Tensor> {
+    return {matmul(grad_output, rhs.permute({0, 2, 1})), matmul(lhs.permute({0, 2, 1}), grad_output)};
+}
+
+// tinytensor::conv2d argument checks (tensor.cpp:3089-3167).
+inline auto conv2d(const Tensor &input, const Tensor &weight, const std::optional<Tensor> &bias = {}, int stride = 1, int padding = 0) -> Tensor {
+    if (input.dim() != 4 || weight.dim() != 4) throw TTException("conv2d expects 4-D input [B,C,H,W] and weight [O,C,k,k]");
+    if (input.size(1) != weight.size(1)) throw TTException("conv2d: input channels do not match weight channels");
+    if (weight.size(2) != weight.size(3)) throw TTException("conv2d: only square kernels are supported");
+    if (stride <= 0 || padding < 0) throw TTException("conv2d: stride must be > 0 and padding >= 0");
+    if (bias && (bias->dim() != 1 || bias->size(0) != weight.size(0))) throw TTException("conv2d: bias must have one entry per output channel");
+    if (input.dtype() != weight.dtype() || input.dtype() == kBool) throw TTException("conv2d: operands must share one non-bool dtype");
+    return get_backend(input.device())->conv2d(input, weight, bias, stride, padding);
+}
+inline auto conv2d_backward(const Tensor &grad_output, const Tensor &input, const Tensor &weight, const std::optional<Tensor> &bias = {},
+                            int stride = 1, int padding = 0) {
+    return get_backend(input.device())->conv2d_backward(grad_output, input, weight, bias, stride, padding);
+}
+
+namespace nn {
+// nn::Linear (nn/linear.cpp:20-50): weight is [in_features, out_features]; forward = matmul + bias.  The bias add
+// (and an optional ReLU that follows it) is fused into the GEMM's store phase.
+class Linear {
+public:
+    Linear(Tensor weight_, std::optional<Tensor> bias_) : weight(std::move(weight_)), bias(std::move(bias_)) {
+        if (weight.dim() != 2) throw TTException("Linear: weight must be [in_features, out_features]");
+    }
+    [[nodiscard]] auto forward(const Tensor &input, bool fuse_relu = false) const -> Tensor {
+        const Tensor x2 = input.dim() == 2 ? input : input.flatten(0, -2);
+        if (x2.size(1) != weight.size(0)) throw TTException("Invalid shape for matrix multiplication");
+        if (x2.dtype() != weight.dtype() || x2.dtype() == kBool) throw TTException("Linear: operands must share one non-bool dtype");
+        ttamd_epilogue ep{};
+        std::optional<Tensor> b = bias ? std::optional<Tensor>(bias->contiguous()) : std::nullopt;
+        ep.bias = b ? b->data_ptr() : nullptr;
+        ep.bias_mode = b ? 1 : 0;
+        ep.relu = fuse_relu ? 1 : 0;
+        Tensor out = get_backend(input.device())->batched_matmul(x2.unsqueeze(0), weight.unsqueeze(0), &ep);
+        auto sh = input.shape().to_vec();
+        sh.back() = weight.size(1);
+        return out.reshape(Shape(sh));
+    }
+    Tensor weight;
+    std::optional<Tensor> bias;
+};
+}  // namespace nn
+
+}  // namespace tt_amd
+
+#endif  // TT_AMD_HOST_H_
