@@ -110,16 +110,13 @@ def detail_report(tt, np, path):
     Bs = tt.Tensor.from_numpy(g.uniform_real(-1, 1, (32, 128, 64)))
     gemm_case("cfg2 f32 32x(128x64x128) B=transposed view", A, Bs.permute(0, 2, 1))
     for dt, nm in ((f32, "f32"), (np.float64, "f64")):
-        S = tt.Tensor.from_numpy(np.zeros((1, 4096, 4096), dt))
+        S = tt.Tensor.from_numpy(oracle.Generator(3).uniform_real(-1, 1, (1, 4096, 4096), dt))
         gemm_case(f"cfg3 {nm} 4096^3 A.B", S, S, 30)
         gemm_case(f"cfg3 {nm} 4096^3 A.B^T (view)", S, S.permute(0, 2, 1), 30)
         gemm_case(f"cfg3 {nm} 4096^3 A^T.B (view)", S.permute(0, 2, 1), S, 30)
     # config 5: the nine GEMMs of one MLP training step (batch 1024, 784-1024-1024-10)
-    X = tt.Tensor.from_numpy(np.zeros((1, 1024, 784), f32))
-    W1 = tt.Tensor.from_numpy(np.zeros((1, 784, 1024), f32))
-    H = tt.Tensor.from_numpy(np.zeros((1, 1024, 1024), f32))
-    W3 = tt.Tensor.from_numpy(np.zeros((1, 1024, 10), f32))
-    Y = tt.Tensor.from_numpy(np.zeros((1, 1024, 10), f32))
+    rnd = lambda *shape: tt.Tensor.from_numpy(g.uniform_real(-1, 1, shape))
+    X, W1, H, W3, Y = rnd(1, 1024, 784), rnd(1, 784, 1024), rnd(1, 1024, 1024), rnd(1, 1024, 10), rnd(1, 1024, 10)
     t = lambda x: x.permute(0, 2, 1)
     for name, a, b in (("fwd1 X.W1", X, W1), ("fwd2 H.W2", H, H), ("fwd3 H.W3 (N=10)", H, W3),
                        ("bwd3 dH=dY.W3^T (K=10)", Y, t(W3)), ("bwd3 dW3=H^T.dY (N=10)", t(H), Y),

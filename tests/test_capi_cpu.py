@@ -76,9 +76,9 @@ def test_variant_names_without_gpu(tt):
         return lib.ttamd_batched_matmul_variant(dtype, B, N, K, M, C.byref(a), C.byref(b)).decode()
 
     n = 4096
-    assert variant(capi.F32, 1, n, n, n, (0, n, 1), (0, n, 1)) == "mfma_f32_128x128_akc4_bmc4"
-    assert variant(capi.F32, 1, n, n, n, (0, n, 1), (0, 1, n)) == "mfma_f32_128x128_akc4_bkc4"      # A . B^T
-    assert variant(capi.F32, 1, n, n, n, (0, 1, n), (0, n, 1)) == "mfma_f32_128x128_amc4_bmc4"      # A^T . B
+    assert variant(capi.F32, 1, n, n, n, (0, n, 1), (0, n, 1)) == "mfma_f32_256x128_akc4_bmc4"
+    assert variant(capi.F32, 1, n, n, n, (0, n, 1), (0, 1, n)) == "mfma_f32_256x128_akc4_bkc4"      # A . B^T
+    assert variant(capi.F32, 1, n, n, n, (0, 1, n), (0, n, 1)) == "mfma_f32_256x128_amc4_bmc4"      # A^T . B
     assert variant(capi.F64, 1, n, n, n, (0, n, 1), (0, n, 1)) == "mfma_f64_128x128_akc2_bmc2"
     assert variant(capi.F32, 32, 128, 64, 128, (8192, 64, 1), (8192, 1, 64)) == "mfma_f32_64x64_akc4_bkc4"  # config 2
     assert variant(capi.F32, 1, 256, 512, 256, (0, 512, 1), (0, 256, 1)) == "mfma_f32_64x64_akc4_bmc4_splitk8"  # config 1

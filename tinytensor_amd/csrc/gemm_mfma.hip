@@ -147,12 +147,16 @@ template <typename T>
 struct TileShapes;
 template <>
 struct TileShapes<float> {
+    static constexpr bool kHasXL = true;
+    static constexpr int XBM = 256, XBN = 128, XBK = 16;  // extra large: 4 waves of 128 x 64 (4 x 2 MFMA blocks)
     static constexpr int LBM = 128, LBN = 128, LBK = 32;  // large: 4 waves of 64 x 64
     static constexpr int SBM = 64, SBN = 64, SBK = 32;    // small: 4 waves of 32 x 32
     static constexpr const char *prefix = "mfma_f32";
 };
 template <>
 struct TileShapes<double> {
+    static constexpr bool kHasXL = false;                  // a 128 x 64 wave tile would need 256 accumulator registers
+    static constexpr int XBM = 128, XBN = 128, XBK = 16;
     static constexpr int LBM = 128, LBN = 128, LBK = 16;  // 4 waves of 64 x 64 (4 x 4 blocks of 16 x 16)
     static constexpr int SBM = 64, SBN = 64, SBK = 16;    // 4 waves of 32 x 32
     static constexpr const char *prefix = "mfma_f64";
@@ -196,27 +200,33 @@ ttamd_status launch_mfma_typed(const GemmArgs &g, int device, hipStream_t stream
     OperandClass cb = classify<T>(g.B, g.b_sn, g.b_sk, g.b_sb, g.batch);
     const bool vec = ca.vec > 1 && cb.vec > 1;
 
+    // Tile choice: the biggest tile that still gives the 256 CUs (2 workgroups each) enough workgroups.
+    const int64_t tiles_xl = static_cast<int64_t>((g.M + TS::XBM - 1) / TS::XBM) * ((g.N + TS::XBN - 1) / TS::XBN) * g.batch;
     const int64_t tiles_large = static_cast<int64_t>((g.M + TS::LBM - 1) / TS::LBM) * ((g.N + TS::LBN - 1) / TS::LBN) * g.batch;
-    const bool large = vec && tiles_large >= 192;
-    const int bm = large ? TS::LBM : TS::SBM;
+    const bool xl = TS::kHasXL && vec && tiles_xl >= 384;
+    const bool large = !xl && vec && tiles_large >= 192;
+    const int bm = xl ? TS::XBM : (large ? TS::LBM : TS::SBM);
 
     // 32-bit buffer addressing: the bytes reachable from a tile's first row must stay below 2^31.
     const int64_t a_reach = (static_cast<int64_t>(bm - 1) * g.a_sm + static_cast<int64_t>(g.K - 1) * g.a_sk + VK) * sizeof(T);
     const int64_t b_reach = (static_cast<int64_t>(bm - 1) * g.b_sn + static_cast<int64_t>(g.K - 1) * g.b_sk + VK) * sizeof(T);
     if (a_reach >= 0x7fffffffLL || b_reach >= 0x7fffffffLL) return TTAMD_OK;
 
-    const SplitPlan sp = large ? SplitPlan{1, g.K} : plan_split<T>(g, TS::SBM, TS::SBN, TS::SBK);
+    const SplitPlan sp = (xl || large) ? SplitPlan{1, g.K} : plan_split<T>(g, TS::SBM, TS::SBN, TS::SBK);
 
     static thread_local char name[112];
     char split_tag[24] = "";
     if (sp.ksplit > 1) snprintf(split_tag, sizeof(split_tag), "_splitk%d", sp.ksplit);
-    snprintf(name, sizeof(name), "%s_%s_a%s%d_b%s%d%s", TS::prefix, large ? "128x128" : "64x64", ca.kc ? "kc" : "mc",
+    snprintf(name, sizeof(name), "%s_%s_a%s%d_b%s%d%s", TS::prefix, xl ? "256x128" : (large ? "128x128" : "64x64"), ca.kc ? "kc" : "mc",
              ca.vec, cb.kc ? "kc" : "mc", cb.vec, split_tag);
     *variant = name;
     *handled = true;
     if (variant_only) return TTAMD_OK;
 
     // The large tile exists for 16-byte operands only; the small tile for every mix of 16-byte and element-wise.
+    if constexpr (TS::kHasXL) {
+        if (xl) return launch_layouts<T, TS::XBM, TS::XBN, TS::XBK, 2, 2, VK, VK>(g, ca.kc, cb.kc, sp, device, stream);
+    }
     if (large) return launch_layouts<T, TS::LBM, TS::LBN, TS::LBK, 2, 2, VK, VK>(g, ca.kc, cb.kc, sp, device, stream);
     if (ca.vec > 1 && cb.vec > 1) return launch_layouts<T, TS::SBM, TS::SBN, TS::SBK, 2, 2, VK, VK>(g, ca.kc, cb.kc, sp, device, stream);
     if (ca.vec > 1) return launch_layouts<T, TS::SBM, TS::SBN, TS::SBK, 2, 2, VK, 1>(g, ca.kc, cb.kc, sp, device, stream);
