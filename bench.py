@@ -83,7 +83,7 @@ def time_launches(tt, fn, iters, warmup):
     return ms.value / iters
 
 
-def detail_report(tt, np, path):
+def detail_report(tt, np, path, cpu=True):
     """Times every BASELINE configuration (GPU only, inputs resident) and writes a JSON report to `path`.
     Not part of the one-line contract; used to track the small-shape, strided and conv paths."""
     from oracle import tt_oracle as oracle  # seeded input generation only
@@ -127,12 +127,36 @@ def detail_report(tt, np, path):
     x = tt.Tensor.from_numpy(oracle.Generator(0).normal(0, 0.1, (64, 32, 28, 28)))
     w = tt.Tensor.from_numpy(oracle.Generator(1).normal(0, 0.1, (64, 32, 3, 3)))
     go = tt.Tensor.from_numpy(np.ones((64, 64, 28, 28), f32))
-    ms = time_launches(tt, lambda: be.conv2d(x, w, None, 1, 1), 100, 10)
-    rows.append({"case": "cfg4 conv2d forward (incl. output allocation)", "ms": round(ms, 5),
+    out = be.conv2d(x, w, None, 1, 1)
+    ms = time_launches(tt, lambda: be.conv2d(x, w, None, 1, 1, out=out), 100, 10)
+    rows.append({"case": "cfg4 conv2d forward", "kernel": "conv_fwd_kernel (implicit GEMM)", "ms": round(ms, 5),
                  "GFLOP/s": round(1.850e9 / ms / 1e6, 1)})
-    ms = time_launches(tt, lambda: be.conv2d_backward(go, x, w, None, 1, 1), 50, 5)
-    rows.append({"case": "cfg4 conv2d backward (data + weight, incl. allocations and sync)", "ms": round(ms, 5),
-                 "GFLOP/s": round(3.700e9 / ms / 1e6, 1)})
+    be.conv2d_backward(go, x, w, None, 1, 1)
+    bufs = be.last_conv_buffers
+    ms = time_launches(tt, lambda: be.conv2d_backward(go, x, w, None, 1, 1, buffers=bufs), 50, 5)
+    rows.append({"case": "cfg4 conv2d backward (grad_input + grad_weight)", "kernel": "conv_dgrad_kernel + conv_wgrad_kernel + reduce",
+                 "ms": round(ms, 5), "GFLOP/s": round(3.700e9 / ms / 1e6, 1)})
+    if cpu:
+        # The same configurations on the CPU oracle (one core), timed once each.
+        xh, wh = oracle.Generator(0).normal(0, 0.1, (64, 32, 28, 28)), oracle.Generator(1).normal(0, 0.1, (64, 32, 3, 3))
+        for name, fn in (
+            ("cfg1 f32 256x512x256", lambda: oracle.matmul(np.ones((256, 512), f32), np.ones((512, 256), f32), "fast")),
+            ("cfg2 f32 32x(128x64x128) B=transposed view",
+             lambda: oracle.matmul(np.ones((32, 128, 64), f32), np.ones((32, 128, 64), f32).transpose(0, 2, 1), "fast")),
+            ("cfg4 conv2d forward", lambda: oracle.conv2d_forward(xh, wh, None, 1, 1, "fast")),
+            ("cfg4 conv2d backward (grad_input + grad_weight)",
+             lambda: oracle.conv2d_backward(np.ones((64, 64, 28, 28), f32), xh, wh, False, 1, 1, "fast")),
+            ("cfg5 fwd2 H.W2", lambda: oracle.matmul(np.ones((1024, 1024), f32), np.ones((1024, 1024), f32), "fast")),
+            ("cfg5 fwd3 H.W3 (N=10)", lambda: oracle.matmul(np.ones((1024, 1024), f32), np.ones((1024, 10), f32), "fast")),
+        ):
+            fn()
+            t0 = time.perf_counter()
+            fn()
+            dt = (time.perf_counter() - t0) * 1e3
+            for r in rows:
+                if r["case"] == name:
+                    r["cpu_oracle_ms_1core"] = round(dt, 3)
+                    r["speedup_vs_cpu"] = round(dt / r["ms"], 1)
     with open(path, "w") as f:
         json.dump(rows, f, indent=1)
     for r in rows:
@@ -165,7 +189,7 @@ def main():
         tt.get_backend(tt.kAMD).synchronize(0)
 
     if args.detail:
-        detail_report(tt, np, args.detail)
+        detail_report(tt, np, args.detail, cpu=not args.no_cpu)
 
     n = args.n
     flop = 2.0 * n * n * n

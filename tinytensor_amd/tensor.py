@@ -280,13 +280,15 @@ class BackendAMD:
         lv, rv = lhs.view3(), rhs.view3()
         return lib.ttamd_batched_matmul_variant(lhs.dtype, B, N, K, rhs.size(2), C.byref(lv), C.byref(rv)).decode()
 
-    def conv2d(self, input: Tensor, weight: Tensor, bias: Tensor | None, stride: int, padding: int) -> Tensor:
-        """BackendBase::conv2d (backend_base.h:269-275)."""
+    def conv2d(self, input: Tensor, weight: Tensor, bias: Tensor | None, stride: int, padding: int,
+               out: Tensor | None = None) -> Tensor:
+        """BackendBase::conv2d (backend_base.h:269-275).  `out`: reuse a result tensor (benchmarks)."""
         B, Cc, H, W = input.shape
         O, _, k, _ = weight.shape
         Ho = (H + 2 * padding - k) // stride + 1
         Wo = (W + 2 * padding - k) // stride + 1
-        out = Tensor.empty((B, O, Ho, Wo), input.dtype, input.device)
+        if out is None:
+            out = Tensor.empty((B, O, Ho, Wo), input.dtype, input.device)
         weight = weight.contiguous()  # used as the matrix [O, C*k*k], as cpu/conv.cpp:69 reshapes it
         iv, wv = input.view4(), weight.view4()
         bptr = None
@@ -298,25 +300,34 @@ class BackendAMD:
         return out
 
     def conv2d_backward(self, grad_output: Tensor, input: Tensor, weight: Tensor, bias: Tensor | None, stride: int,
-                        padding: int):
-        """BackendBase::conv2d_backward (backend_base.h:277-284) -> (grad_input, grad_weight, grad_bias|None)."""
+                        padding: int, buffers=None):
+        """BackendBase::conv2d_backward (backend_base.h:277-284) -> (grad_input, grad_weight, grad_bias|None).
+        `buffers` = (gx, gw, gb, workspace_storage) from an earlier call reuses the results (benchmarks); the call
+        then does not synchronise."""
         B, Cc, H, W = input.shape
         O, _, k, _ = weight.shape
         go = grad_output.contiguous()
         weight = weight.contiguous()
-        gx = Tensor.empty(input.shape, input.dtype, input.device)
-        gw = Tensor.empty(weight.shape, input.dtype, input.device)
-        gb = Tensor.empty((O,), input.dtype, input.device) if bias is not None else None
-        ws_bytes = C.c_size_t()
-        _check(lib.ttamd_conv2d_backward_workspace(input.dtype, B, Cc, H, W, O, k, stride, padding, C.byref(ws_bytes)))
-        ws = _Storage(max(ws_bytes.value, 1), input.device)
+        if buffers is not None:
+            gx, gw, gb, ws = buffers
+        else:
+            gx = Tensor.empty(input.shape, input.dtype, input.device)
+            gw = Tensor.empty(weight.shape, input.dtype, input.device)
+            gb = Tensor.empty((O,), input.dtype, input.device) if bias is not None else None
+            ws_bytes = C.c_size_t()
+            _check(lib.ttamd_conv2d_backward_workspace(input.dtype, B, Cc, H, W, O, k, stride, padding,
+                                                       C.byref(ws_bytes)))
+            ws = _Storage(max(ws_bytes.value, 1), input.device)
         iv, wv = input.view4(), weight.view4()
         _check(lib.ttamd_conv2d_backward(
             input.device.id, input.dtype, C.c_void_p(go.storage.ptr + go.offset * go.itemsize), C.byref(iv),
             C.byref(wv), C.c_void_p(gx.storage.ptr), C.c_void_p(gw.storage.ptr),
             C.c_void_p(gb.storage.ptr) if gb is not None else None, B, Cc, H, W, O, k, stride, padding,
             C.c_void_p(ws.ptr), ws.nbytes, None))
+        if buffers is not None:
+            return gx, gw, gb
         self.synchronize(input.device.id)  # the workspace is released when this frame returns
+        self.last_conv_buffers = (gx, gw, gb, ws)
         return gx, gw, gb
 
 
