@@ -144,6 +144,36 @@ ttamd_status ttamd_conv2d_backward(int device, ttamd_dtype dtype, const void *gr
                                    int B, int C, int H, int W, int O, int k, int stride, int padding, void *workspace,
                                    size_t workspace_bytes, void *stream);
 
+/* ---- elementwise / reduction ops that an MLP training step needs around its GEMMs ------------
+ * (BackendBase::add, sub, mul, div, pow, maximum, minimum, lt, le, gt, ge, eq, ne: backend_base.h:109-131;
+ * relu & friends: :136-260; where: :263; sum: :148-149; full: :51.  CPU forms: cpu/binary.cpp:26-84,
+ * cpu/unary.cpp:26-82, cpu/kernel/reduce.hpp:15-48, functors in common/kernel/binary.hpp, unary.hpp.)
+ * Operands are strided views (ndim <= 8, element strides >= 0) of ONE shape: the frontend broadcasts with
+ * expand() before it calls the backend.  Results are dense row-major.  dtype = operand dtype; comparison
+ * results are bool (one byte, 0/1).  Integer arithmetic wraps; integer division by zero yields 0. */
+typedef enum ttamd_binary_op {
+    TTAMD_BIN_ADD = 0, TTAMD_BIN_SUB, TTAMD_BIN_MUL, TTAMD_BIN_DIV, TTAMD_BIN_POW, TTAMD_BIN_MAXIMUM, TTAMD_BIN_MINIMUM,
+    TTAMD_BIN_LT, TTAMD_BIN_LE, TTAMD_BIN_GT, TTAMD_BIN_GE, TTAMD_BIN_EQ, TTAMD_BIN_NE
+} ttamd_binary_op;
+typedef enum ttamd_unary_op {
+    TTAMD_UN_RELU = 0, TTAMD_UN_NEGATE, TTAMD_UN_ABS, TTAMD_UN_SQRT, TTAMD_UN_EXP, TTAMD_UN_LOG, TTAMD_UN_SIGMOID, TTAMD_UN_TANH
+} ttamd_unary_op;
+ttamd_status ttamd_binary(int device, ttamd_dtype dtype, int op, int ndim, const int64_t *shape, const void *lhs,
+                          int64_t lhs_offset, const int64_t *lhs_stride, const void *rhs, int64_t rhs_offset,
+                          const int64_t *rhs_stride, void *out, void *stream);
+ttamd_status ttamd_unary(int device, ttamd_dtype dtype, int op, int ndim, const int64_t *shape, const void *src,
+                         int64_t offset, const int64_t *stride, void *out, void *stream);
+/* BackendBase::where (backend_base.h:263): out = cond ? lhs : rhs; cond is a bool (one byte) view. */
+ttamd_status ttamd_where(int device, ttamd_dtype dtype, int ndim, const int64_t *shape, const void *cond,
+                         int64_t cond_offset, const int64_t *cond_stride, const void *lhs, int64_t lhs_offset,
+                         const int64_t *lhs_stride, const void *rhs, int64_t rhs_offset, const int64_t *rhs_stride,
+                         void *out, void *stream);
+/* BackendBase::sum(tensor) (dim = -1, one element out) and sum(tensor, dim) (that dimension removed). */
+ttamd_status ttamd_sum(int device, ttamd_dtype dtype, int ndim, const int64_t *shape, const void *src, int64_t offset,
+                       const int64_t *stride, int dim, void *out, void *stream);
+/* BackendBase::full (backend_base.h:51): `value` points at one host scalar of `dtype`. */
+ttamd_status ttamd_full(int device, ttamd_dtype dtype, const void *value, int64_t numel, void *out, void *stream);
+
 /* ---- timing (no reference counterpart: the reference has no timers; used by the benchmark
  * to bracket kernels with HIP events on the stream they run on) ------------------------ */
 ttamd_status ttamd_event_create(int device, void **event);

@@ -13,6 +13,9 @@ LIB_PATH = os.path.join(_HERE, "csrc", "libttamd.so")
 
 OK, ERR_INVALID_ARGUMENT, ERR_INVALID_DEVICE, ERR_UNSUPPORTED_DTYPE, ERR_OUT_OF_MEMORY, ERR_LAUNCH = range(6)
 BOOL, U8, I16, I32, I64, F32, F64 = range(7)
+BIN = {"add": 0, "sub": 1, "mul": 2, "div": 3, "pow": 4, "maximum": 5, "minimum": 6, "lt": 7, "le": 8, "gt": 9, "ge": 10,
+       "eq": 11, "ne": 12}
+UN = {"relu": 0, "negate": 1, "abs": 2, "sqrt": 3, "exp": 4, "log": 5, "sigmoid": 6, "tanh": 7}
 
 
 class View3(C.Structure):
@@ -41,6 +44,13 @@ def _bind(lib: C.CDLL) -> None:
         "ttamd_memset_zero": (i, [i, vp, sz, vp]),
         "ttamd_device_synchronize": (i, [i]),
         "ttamd_contiguous": (i, [i, i, i, C.POINTER(C.c_int64), C.POINTER(C.c_int64), vp, C.c_int64, vp, vp]),
+        "ttamd_binary": (i, [i, i, i, i, C.POINTER(C.c_int64), vp, C.c_int64, C.POINTER(C.c_int64), vp, C.c_int64,
+                             C.POINTER(C.c_int64), vp, vp]),
+        "ttamd_unary": (i, [i, i, i, i, C.POINTER(C.c_int64), vp, C.c_int64, C.POINTER(C.c_int64), vp, vp]),
+        "ttamd_where": (i, [i, i, i, C.POINTER(C.c_int64), vp, C.c_int64, C.POINTER(C.c_int64), vp, C.c_int64,
+                            C.POINTER(C.c_int64), vp, C.c_int64, C.POINTER(C.c_int64), vp, vp]),
+        "ttamd_sum": (i, [i, i, i, C.POINTER(C.c_int64), vp, C.c_int64, C.POINTER(C.c_int64), i, vp, vp]),
+        "ttamd_full": (i, [i, i, vp, C.c_int64, vp, vp]),
         "ttamd_batched_matmul": (i, [i, i, i, i, i, i, C.POINTER(View3), C.POINTER(View3), vp, C.POINTER(Epilogue), vp]),
         "ttamd_batched_matmul_variant": (C.c_char_p, [i, i, i, i, i, C.POINTER(View3), C.POINTER(View3)]),
         "ttamd_conv2d_forward": (i, [i, i, C.POINTER(View4), C.POINTER(View4), vp, vp] + [i] * 8 + [vp]),

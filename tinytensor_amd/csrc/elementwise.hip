@@ -5,6 +5,9 @@
 // grad_output) and moves raw bytes, so one kernel per element size serves every dtype.
 #include "common.h"
 
+#include <cstring>
+#include <type_traits>
+
 namespace ttamd {
 namespace {
 
@@ -38,6 +41,265 @@ ttamd_status launch_contiguous(const void *src, void *dst, const ViewDesc &v, in
     TTAMD_HIP_CHECK(hipGetLastError());
     return TTAMD_OK;
 }
+
+
+// ---------------------------------------------------------------------------------------------
+// Elementwise set that an MLP training step needs around its GEMMs (tinytensor/tensor/backend_base.h:
+// add/sub/mul/div/pow/maximum/minimum, lt/le/gt/ge/eq/ne, relu & friends, where, sum, full).  Operands are
+// strided views of ONE shape (the frontend has already broadcast with expand(), include/tt/tensor.h:600);
+// results are dense.  Functors follow tinytensor/tensor/backend/common/kernel/binary.hpp:20-140.
+
+__device__ __forceinline__ int64_t flat_of(int64_t rank, const ViewDesc &v) {
+    int64_t flat = 0;
+    for (int d = v.ndim - 1; d >= 0; --d) {
+        flat += (rank % v.shape[d]) * v.stride[d];
+        rank /= v.shape[d];
+    }
+    return flat;
+}
+
+enum { BIN_ADD = 0, BIN_SUB, BIN_MUL, BIN_DIV, BIN_POW, BIN_MAXIMUM, BIN_MINIMUM, BIN_LT, BIN_LE, BIN_GT, BIN_GE, BIN_EQ, BIN_NE, BIN_COUNT };
+enum { UN_RELU = 0, UN_NEGATE, UN_ABS, UN_SQRT, UN_EXP, UN_LOG, UN_SIGMOID, UN_TANH, UN_COUNT };
+
+template <typename T>
+__device__ __forceinline__ T pow_of(T a, T b) {
+    if constexpr (std::is_floating_point_v<T>) {
+        if (b == T(2)) return a * a;  // exact square, as a correctly rounded pow would give
+        return pow(a, b);
+    } else {
+        // integer power by squaring with wrap-around; negative exponents follow std::pow's real result truncated
+        using U = std::make_unsigned_t<T>;
+        if (b < T(0)) return a == T(1) ? T(1) : (a == T(-1) ? ((b & 1) ? T(-1) : T(1)) : T(0));
+        U base = static_cast<U>(a), r = 1;
+        U e = static_cast<U>(b);
+        while (e) {
+            if (e & 1) r *= base;
+            base *= base;
+            e >>= 1;
+        }
+        return static_cast<T>(r);
+    }
+}
+
+template <typename T, int OP>
+__device__ __forceinline__ auto binary_apply(T a, T b) {
+    if constexpr (OP == BIN_ADD) return static_cast<T>(a + b);
+    else if constexpr (OP == BIN_SUB) return static_cast<T>(a - b);
+    else if constexpr (OP == BIN_MUL) return static_cast<T>(a * b);
+    else if constexpr (OP == BIN_DIV) {
+        if constexpr (std::is_integral_v<T>) return static_cast<T>(b == T(0) ? T(0) : a / b);  // no trap on the device
+        else return static_cast<T>(a / b);
+    }
+    else if constexpr (OP == BIN_POW) return pow_of<T>(a, b);
+    else if constexpr (OP == BIN_MAXIMUM) return (a > b) ? a : b;
+    else if constexpr (OP == BIN_MINIMUM) return (a < b) ? a : b;
+    else if constexpr (OP == BIN_LT) return static_cast<uint8_t>(a < b);
+    else if constexpr (OP == BIN_LE) return static_cast<uint8_t>(a <= b);
+    else if constexpr (OP == BIN_GT) return static_cast<uint8_t>(a > b);
+    else if constexpr (OP == BIN_GE) return static_cast<uint8_t>(a >= b);
+    else if constexpr (OP == BIN_EQ) return static_cast<uint8_t>(a == b);
+    else return static_cast<uint8_t>(a != b);
+}
+
+template <typename T, int OP, bool DENSE>
+__global__ void __launch_bounds__(256) binary_kernel(const T *__restrict__ a, ViewDesc va, const T *__restrict__ b, ViewDesc vb,
+                                                    void *__restrict__ out, int64_t numel) {
+    using R = decltype(binary_apply<T, OP>(T(0), T(0)));
+    const int64_t step = static_cast<int64_t>(gridDim.x) * blockDim.x;
+    for (int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < numel; i += step) {
+        const T x = DENSE ? a[i] : a[flat_of(i, va)];
+        const T y = DENSE ? b[i] : b[flat_of(i, vb)];
+        static_cast<R *>(out)[i] = binary_apply<T, OP>(x, y);
+    }
+}
+
+template <typename T, int OP>
+__device__ __forceinline__ T unary_apply(T x) {
+    if constexpr (OP == UN_RELU) return x > T(0) ? x : T(0);
+    else if constexpr (OP == UN_NEGATE) return static_cast<T>(T(0) - x);
+    else if constexpr (OP == UN_ABS) {
+        if constexpr (std::is_unsigned_v<T>) return x;
+        else return x < T(0) ? static_cast<T>(T(0) - x) : x;
+    } else if constexpr (std::is_floating_point_v<T>) {
+        if constexpr (OP == UN_SQRT) return sqrt(x);
+        else if constexpr (OP == UN_EXP) return exp(x);
+        else if constexpr (OP == UN_LOG) return log(x);
+        else if constexpr (OP == UN_SIGMOID) return T(1) / (T(1) + exp(-x));
+        else return tanh(x);
+    } else {
+        return x;
+    }
+}
+
+template <typename T, int OP, bool DENSE>
+__global__ void __launch_bounds__(256) unary_kernel(const T *__restrict__ a, ViewDesc va, T *__restrict__ out, int64_t numel) {
+    const int64_t step = static_cast<int64_t>(gridDim.x) * blockDim.x;
+    for (int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < numel; i += step)
+        out[i] = unary_apply<T, OP>(DENSE ? a[i] : a[flat_of(i, va)]);
+}
+
+template <typename T>
+__global__ void __launch_bounds__(256) where_kernel(const uint8_t *__restrict__ c, ViewDesc vc, const T *__restrict__ a, ViewDesc va,
+                                                   const T *__restrict__ b, ViewDesc vb, T *__restrict__ out, int64_t numel) {
+    const int64_t step = static_cast<int64_t>(gridDim.x) * blockDim.x;
+    for (int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < numel; i += step)
+        out[i] = c[flat_of(i, vc)] ? a[flat_of(i, va)] : b[flat_of(i, vb)];
+}
+
+template <typename T>
+__global__ void __launch_bounds__(256) full_kernel(T *__restrict__ out, T value, int64_t numel) {
+    const int64_t step = static_cast<int64_t>(gridDim.x) * blockDim.x;
+    for (int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < numel; i += step) out[i] = value;
+}
+
+// sum over one dimension: one lane per output element walks the reduced dimension in index order, which is
+// the order of the reference's reduce_dim_kernel (cpu/kernel/reduce.hpp:15-32).  `outer` = view without `dim`.
+template <typename T>
+__global__ void __launch_bounds__(256) sum_dim_kernel(const T *__restrict__ a, ViewDesc outer, int64_t dim_len, int64_t dim_stride,
+                                                     T *__restrict__ out, int64_t n_out) {
+    const int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (i >= n_out) return;
+    const T *p = a + flat_of(i, outer);
+    T acc = T(0);
+    for (int64_t j = 0; j < dim_len; ++j) acc = static_cast<T>(acc + p[j * dim_stride]);
+    out[i] = acc;
+}
+
+// sum of everything: per-workgroup partial sums (stage 1) then one workgroup adds the partials (stage 2).
+template <typename T>
+__global__ void __launch_bounds__(256) sum_all_kernel(const T *__restrict__ a, ViewDesc v, bool dense, int64_t numel, T *__restrict__ out) {
+    __shared__ T red[256];
+    T acc = T(0);
+    const int64_t step = static_cast<int64_t>(gridDim.x) * blockDim.x;
+    for (int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < numel; i += step)
+        acc = static_cast<T>(acc + (dense ? a[i] : a[flat_of(i, v)]));
+    red[threadIdx.x] = acc;
+    __syncthreads();
+    for (int s = 128; s > 0; s >>= 1) {
+        if (static_cast<int>(threadIdx.x) < s) red[threadIdx.x] = static_cast<T>(red[threadIdx.x] + red[threadIdx.x + s]);
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) out[blockIdx.x] = red[0];
+}
+
+inline unsigned grid_for(int64_t numel) {
+    int64_t blocks = (numel + 255) / 256;
+    if (blocks > 8192) blocks = 8192;
+    return static_cast<unsigned>(blocks < 1 ? 1 : blocks);
+}
+
+inline bool is_dense(const ViewDesc &v) {
+    int64_t expect = 1;
+    for (int d = v.ndim - 1; d >= 0; --d) {
+        if (v.shape[d] != 1 && v.stride[d] != expect) return false;
+        expect *= v.shape[d];
+    }
+    return true;
+}
+
+ttamd_status make_view(const char *who, int ndim, const int64_t *shape, const int64_t *stride, ViewDesc *v, int64_t *numel) {
+    if (ndim < 0 || ndim > kMaxDims || (ndim > 0 && (!shape || !stride))) {
+        set_error("%s: ndim must be in [0,%d] with non-NULL shape/stride", who, kMaxDims);
+        return TTAMD_ERR_INVALID_ARGUMENT;
+    }
+    *v = ViewDesc{};
+    v->ndim = ndim;
+    int64_t n = 1;
+    for (int d = 0; d < ndim; ++d) {
+        if (shape[d] < 0 || stride[d] < 0) {
+            set_error("%s: negative extent or stride in dimension %d", who, d);
+            return TTAMD_ERR_INVALID_ARGUMENT;
+        }
+        v->shape[d] = shape[d];
+        v->stride[d] = stride[d];
+        n *= shape[d];
+    }
+    if (numel) *numel = n;
+    return TTAMD_OK;
+}
+
+template <typename T, int OP>
+ttamd_status launch_binary_op(const void *a, const ViewDesc &va, const void *b, const ViewDesc &vb, void *out, int64_t numel, hipStream_t st) {
+    if (is_dense(va) && is_dense(vb))
+        binary_kernel<T, OP, true><<<dim3(grid_for(numel)), dim3(256), 0, st>>>(static_cast<const T *>(a), va, static_cast<const T *>(b), vb, out, numel);
+    else
+        binary_kernel<T, OP, false><<<dim3(grid_for(numel)), dim3(256), 0, st>>>(static_cast<const T *>(a), va, static_cast<const T *>(b), vb, out, numel);
+    TTAMD_HIP_CHECK(hipGetLastError());
+    return TTAMD_OK;
+}
+
+template <typename T, int OP = 0>
+ttamd_status dispatch_binary(int op, const void *a, const ViewDesc &va, const void *b, const ViewDesc &vb, void *out, int64_t numel, hipStream_t st) {
+    if constexpr (OP < BIN_COUNT) {
+        if (op == OP) return launch_binary_op<T, OP>(a, va, b, vb, out, numel, st);
+        return dispatch_binary<T, OP + 1>(op, a, va, b, vb, out, numel, st);
+    } else {
+        set_error("binary: unknown op code %d", op);
+        return TTAMD_ERR_INVALID_ARGUMENT;
+    }
+}
+
+template <typename T, int OP = 0>
+ttamd_status dispatch_unary(int op, const void *a, const ViewDesc &va, void *out, int64_t numel, hipStream_t st) {
+    if constexpr (OP < UN_COUNT) {
+        if (op == OP) {
+            if (is_dense(va)) unary_kernel<T, OP, true><<<dim3(grid_for(numel)), dim3(256), 0, st>>>(static_cast<const T *>(a), va, static_cast<T *>(out), numel);
+            else unary_kernel<T, OP, false><<<dim3(grid_for(numel)), dim3(256), 0, st>>>(static_cast<const T *>(a), va, static_cast<T *>(out), numel);
+            TTAMD_HIP_CHECK(hipGetLastError());
+            return TTAMD_OK;
+        }
+        return dispatch_unary<T, OP + 1>(op, a, va, out, numel, st);
+    } else {
+        set_error("unary: unknown op code %d", op);
+        return TTAMD_ERR_INVALID_ARGUMENT;
+    }
+}
+
+template <typename T>
+ttamd_status sum_typed(int device, const void *a, const ViewDesc &v, int64_t numel, int dim, void *out, hipStream_t st) {
+    const T *src = static_cast<const T *>(a);
+    if (dim < 0) {
+        const unsigned blocks = numel > 256 * 64 ? 256 : 1;
+        if (blocks == 1) {
+            sum_all_kernel<T><<<dim3(1), dim3(256), 0, st>>>(src, v, is_dense(v), numel, static_cast<T *>(out));
+        } else {
+            void *ws = nullptr;
+            if (ttamd_status s = stream_scratch(device, st, blocks * sizeof(T), &ws)) return s;
+            sum_all_kernel<T><<<dim3(blocks), dim3(256), 0, st>>>(src, v, is_dense(v), numel, static_cast<T *>(ws));
+            ViewDesc pv{};
+            pv.ndim = 1;
+            pv.shape[0] = blocks;
+            pv.stride[0] = 1;
+            sum_all_kernel<T><<<dim3(1), dim3(256), 0, st>>>(static_cast<const T *>(ws), pv, true, blocks, static_cast<T *>(out));
+        }
+        TTAMD_HIP_CHECK(hipGetLastError());
+        return TTAMD_OK;
+    }
+    ViewDesc outer{};
+    for (int d = 0; d < v.ndim; ++d) {
+        if (d == dim) continue;
+        outer.shape[outer.ndim] = v.shape[d];
+        outer.stride[outer.ndim] = v.stride[d];
+        ++outer.ndim;
+    }
+    const int64_t n_out = v.shape[dim] ? numel / v.shape[dim] : 0;
+    if (n_out == 0) return TTAMD_OK;
+    sum_dim_kernel<T><<<dim3(static_cast<unsigned>((n_out + 255) / 256)), dim3(256), 0, st>>>(src, outer, v.shape[dim], v.stride[dim],
+                                                                                              static_cast<T *>(out), n_out);
+    TTAMD_HIP_CHECK(hipGetLastError());
+    return TTAMD_OK;
+}
+
+#define TTAMD_DISPATCH_DTYPE(dtype, CALL)                      \
+    switch (dtype) {                                           \
+    case TTAMD_U8: { using T_ = uint8_t; return CALL; }        \
+    case TTAMD_I16: { using T_ = int16_t; return CALL; }       \
+    case TTAMD_I32: { using T_ = int32_t; return CALL; }       \
+    case TTAMD_I64: { using T_ = int64_t; return CALL; }       \
+    case TTAMD_F32: { using T_ = float; return CALL; }         \
+    case TTAMD_F64: { using T_ = double; return CALL; }        \
+    default: break;                                            \
+    }
 
 }  // namespace
 }  // namespace ttamd
@@ -83,3 +345,162 @@ extern "C" ttamd_status ttamd_contiguous(int device, ttamd_dtype dtype, int ndim
     default: return launch_contiguous<uint64_t>(src, out, v, numel, st);
     }
 }
+
+extern "C" {
+
+ttamd_status ttamd_binary(int device, ttamd_dtype dtype, int op, int ndim, const int64_t *shape, const void *lhs, int64_t lhs_offset,
+                          const int64_t *lhs_stride, const void *rhs, int64_t rhs_offset, const int64_t *rhs_stride, void *out,
+                          void *stream) {
+    ViewDesc va, vb;
+    int64_t numel = 0;
+    if (ttamd_status s = make_view("binary", ndim, shape, lhs_stride, &va, &numel)) return s;
+    if (ttamd_status s = make_view("binary", ndim, shape, rhs_stride, &vb, nullptr)) return s;
+    const size_t esz = dtype_size(dtype);
+    if (dtype <= TTAMD_BOOL || dtype > TTAMD_F64 || esz == 0) {
+        set_error("binary: unsupported dtype code %d", static_cast<int>(dtype));
+        return TTAMD_ERR_UNSUPPORTED_DTYPE;
+    }
+    if (lhs_offset < 0 || rhs_offset < 0) {
+        set_error("binary: negative view offset");
+        return TTAMD_ERR_INVALID_ARGUMENT;
+    }
+    if (ttamd_status s = use_device(device)) return s;
+    if (numel == 0) return TTAMD_OK;
+    if (!lhs || !rhs || !out) {
+        set_error("binary: NULL data pointer");
+        return TTAMD_ERR_INVALID_ARGUMENT;
+    }
+    const void *a = static_cast<const char *>(lhs) + lhs_offset * static_cast<int64_t>(esz);
+    const void *b = static_cast<const char *>(rhs) + rhs_offset * static_cast<int64_t>(esz);
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    TTAMD_DISPATCH_DTYPE(dtype, (dispatch_binary<T_>(op, a, va, b, vb, out, numel, st)))
+    return TTAMD_ERR_UNSUPPORTED_DTYPE;
+}
+
+ttamd_status ttamd_unary(int device, ttamd_dtype dtype, int op, int ndim, const int64_t *shape, const void *src, int64_t offset,
+                         const int64_t *stride, void *out, void *stream) {
+    ViewDesc va;
+    int64_t numel = 0;
+    if (ttamd_status s = make_view("unary", ndim, shape, stride, &va, &numel)) return s;
+    const size_t esz = dtype_size(dtype);
+    if (dtype <= TTAMD_BOOL || dtype > TTAMD_F64 || esz == 0) {
+        set_error("unary: unsupported dtype code %d", static_cast<int>(dtype));
+        return TTAMD_ERR_UNSUPPORTED_DTYPE;
+    }
+    if (op >= UN_SQRT && op < UN_COUNT && dtype != TTAMD_F32 && dtype != TTAMD_F64) {
+        set_error("unary: op %d needs a floating point dtype", op);
+        return TTAMD_ERR_UNSUPPORTED_DTYPE;
+    }
+    if (offset < 0) {
+        set_error("unary: negative view offset");
+        return TTAMD_ERR_INVALID_ARGUMENT;
+    }
+    if (ttamd_status s = use_device(device)) return s;
+    if (numel == 0) return TTAMD_OK;
+    if (!src || !out) {
+        set_error("unary: NULL data pointer");
+        return TTAMD_ERR_INVALID_ARGUMENT;
+    }
+    const void *a = static_cast<const char *>(src) + offset * static_cast<int64_t>(esz);
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    TTAMD_DISPATCH_DTYPE(dtype, (dispatch_unary<T_>(op, a, va, out, numel, st)))
+    return TTAMD_ERR_UNSUPPORTED_DTYPE;
+}
+
+ttamd_status ttamd_where(int device, ttamd_dtype dtype, int ndim, const int64_t *shape, const void *cond, int64_t cond_offset,
+                         const int64_t *cond_stride, const void *lhs, int64_t lhs_offset, const int64_t *lhs_stride, const void *rhs,
+                         int64_t rhs_offset, const int64_t *rhs_stride, void *out, void *stream) {
+    ViewDesc vc, va, vb;
+    int64_t numel = 0;
+    if (ttamd_status s = make_view("where", ndim, shape, cond_stride, &vc, &numel)) return s;
+    if (ttamd_status s = make_view("where", ndim, shape, lhs_stride, &va, nullptr)) return s;
+    if (ttamd_status s = make_view("where", ndim, shape, rhs_stride, &vb, nullptr)) return s;
+    const size_t esz = dtype_size(dtype);
+    if (dtype <= TTAMD_BOOL || dtype > TTAMD_F64 || esz == 0) {
+        set_error("where: unsupported dtype code %d", static_cast<int>(dtype));
+        return TTAMD_ERR_UNSUPPORTED_DTYPE;
+    }
+    if (cond_offset < 0 || lhs_offset < 0 || rhs_offset < 0) {
+        set_error("where: negative view offset");
+        return TTAMD_ERR_INVALID_ARGUMENT;
+    }
+    if (ttamd_status s = use_device(device)) return s;
+    if (numel == 0) return TTAMD_OK;
+    if (!cond || !lhs || !rhs || !out) {
+        set_error("where: NULL data pointer");
+        return TTAMD_ERR_INVALID_ARGUMENT;
+    }
+    const uint8_t *c = static_cast<const uint8_t *>(cond) + cond_offset;
+    const void *a = static_cast<const char *>(lhs) + lhs_offset * static_cast<int64_t>(esz);
+    const void *b = static_cast<const char *>(rhs) + rhs_offset * static_cast<int64_t>(esz);
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    auto run = [&](auto tag) -> ttamd_status {
+        using T = decltype(tag);
+        where_kernel<T><<<dim3(grid_for(numel)), dim3(256), 0, st>>>(c, vc, static_cast<const T *>(a), va, static_cast<const T *>(b), vb,
+                                                                   static_cast<T *>(out), numel);
+        TTAMD_HIP_CHECK(hipGetLastError());
+        return TTAMD_OK;
+    };
+    TTAMD_DISPATCH_DTYPE(dtype, run(T_{}))
+    return TTAMD_ERR_UNSUPPORTED_DTYPE;
+}
+
+ttamd_status ttamd_sum(int device, ttamd_dtype dtype, int ndim, const int64_t *shape, const void *src, int64_t offset,
+                       const int64_t *stride, int dim, void *out, void *stream) {
+    ViewDesc va;
+    int64_t numel = 0;
+    if (ttamd_status s = make_view("sum", ndim, shape, stride, &va, &numel)) return s;
+    const size_t esz = dtype_size(dtype);
+    if (dtype <= TTAMD_BOOL || dtype > TTAMD_F64 || esz == 0) {
+        set_error("sum: unsupported dtype code %d", static_cast<int>(dtype));
+        return TTAMD_ERR_UNSUPPORTED_DTYPE;
+    }
+    if (dim >= ndim || offset < 0) {
+        set_error("sum: dim %d out of range for %d dimensions, or negative offset", dim, ndim);
+        return TTAMD_ERR_INVALID_ARGUMENT;
+    }
+    if (ttamd_status s = use_device(device)) return s;
+    if (!out || (numel > 0 && !src)) {
+        set_error("sum: NULL data pointer");
+        return TTAMD_ERR_INVALID_ARGUMENT;
+    }
+    const void *a = static_cast<const char *>(src) + offset * static_cast<int64_t>(esz);
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    TTAMD_DISPATCH_DTYPE(dtype, (sum_typed<T_>(device, a, va, numel, dim, out, st)))
+    return TTAMD_ERR_UNSUPPORTED_DTYPE;
+}
+
+ttamd_status ttamd_full(int device, ttamd_dtype dtype, const void *value, int64_t numel, void *out, void *stream) {
+    const size_t esz = dtype_size(dtype);
+    if (dtype < TTAMD_BOOL || dtype > TTAMD_F64 || esz == 0) {
+        set_error("full: unsupported dtype code %d", static_cast<int>(dtype));
+        return TTAMD_ERR_UNSUPPORTED_DTYPE;
+    }
+    if (!value || numel < 0) {
+        set_error("full: NULL value or negative count");
+        return TTAMD_ERR_INVALID_ARGUMENT;
+    }
+    if (ttamd_status s = use_device(device)) return s;
+    if (numel == 0) return TTAMD_OK;
+    if (!out) {
+        set_error("full: out is NULL");
+        return TTAMD_ERR_INVALID_ARGUMENT;
+    }
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    auto run = [&](auto tag) -> ttamd_status {
+        using W = decltype(tag);
+        W v;
+        memcpy(&v, value, sizeof(W));
+        full_kernel<W><<<dim3(grid_for(numel)), dim3(256), 0, st>>>(static_cast<W *>(out), v, numel);
+        TTAMD_HIP_CHECK(hipGetLastError());
+        return TTAMD_OK;
+    };
+    switch (esz) {
+    case 1: return run(uint8_t{});
+    case 2: return run(uint16_t{});
+    case 4: return run(uint32_t{});
+    default: return run(uint64_t{});
+    }
+}
+
+}  // extern "C"

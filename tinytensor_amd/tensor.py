@@ -205,6 +205,31 @@ class Tensor:
         merged = int(np.prod(self.shape[start:end + 1]))
         return self.reshape(list(self.shape[:start]) + [merged] + list(self.shape[end + 1:]))
 
+    # ---- elementwise ops around the GEMMs (frontend broadcasting, then one backend call) ----------
+    def _binary(self, other, op: str) -> "Tensor":
+        if not isinstance(other, Tensor):
+            other = full(self.shape, other, self.dtype, self.device)
+        a, b = broadcast_tensors(self, other)
+        return get_backend(self.device).binary(a, b, op)
+
+    def __add__(self, o): return self._binary(o, "add")
+    def __sub__(self, o): return self._binary(o, "sub")
+    def __mul__(self, o): return self._binary(o, "mul")
+    def __truediv__(self, o): return self._binary(o, "div")
+    def __lt__(self, o): return self._binary(o, "lt")
+    def __gt__(self, o): return self._binary(o, "gt")
+    def __rmul__(self, o): return self._binary(o, "mul")
+    def pow(self, o): return self._binary(o, "pow")
+    def relu(self): return get_backend(self.device).unary(self, "relu")
+    def sum(self, dim: int | None = None): return get_backend(self.device).sum(self, dim)
+
+    def mean(self):
+        """Tensor::mean(): sum() / numel (tinytensor/tensor/tensor.cpp mean -> sum, then div by N)."""
+        return self.sum() / float(self.numel())
+
+    def item(self):
+        return self.to_numpy().reshape(-1)[0]
+
     def view3(self) -> _capi.View3:
         v = _capi.View3()
         v.data = self.storage.ptr
@@ -252,6 +277,58 @@ class BackendAMD:
         stride = (C.c_int64 * max(nd, 1))(*t.stride)
         _check(lib.ttamd_contiguous(t.device.id, t.dtype, nd, shape, stride, C.c_void_p(t.storage.ptr), t.offset,
                                     C.c_void_p(out.storage.ptr), None))
+        return out
+
+    @staticmethod
+    def _i64(vals):
+        return (C.c_int64 * max(len(vals), 1))(*vals)
+
+    def binary(self, lhs: Tensor, rhs: Tensor, op: str) -> Tensor:
+        """BackendBase::add/sub/mul/div/pow/maximum/minimum and the comparisons (backend_base.h:109-131)."""
+        if lhs.shape != rhs.shape or lhs.dtype != rhs.dtype:
+            raise TTException(f"binary op {op}: operands must share shape and dtype")
+        code = _capi.BIN[op]
+        out = Tensor.empty(lhs.shape, _capi.BOOL if code >= _capi.BIN["lt"] else lhs.dtype, lhs.device)
+        _check(lib.ttamd_binary(lhs.device.id, lhs.dtype, code, lhs.dim(), self._i64(lhs.shape), C.c_void_p(lhs.storage.ptr),
+                                lhs.offset, self._i64(lhs.stride), C.c_void_p(rhs.storage.ptr), rhs.offset,
+                                self._i64(rhs.stride), C.c_void_p(out.storage.ptr), None))
+        return out
+
+    def unary(self, t: Tensor, op: str) -> Tensor:
+        """BackendBase::relu / negate / abs / sqrt / exp / log / sigmoid / tanh (backend_base.h:136-260)."""
+        out = Tensor.empty(t.shape, t.dtype, t.device)
+        _check(lib.ttamd_unary(t.device.id, t.dtype, _capi.UN[op], t.dim(), self._i64(t.shape), C.c_void_p(t.storage.ptr),
+                               t.offset, self._i64(t.stride), C.c_void_p(out.storage.ptr), None))
+        return out
+
+    def where(self, cond: Tensor, lhs: Tensor, rhs: Tensor) -> Tensor:
+        """BackendBase::where (backend_base.h:263)."""
+        if cond.dtype != _capi.BOOL or cond.shape != lhs.shape or lhs.shape != rhs.shape or lhs.dtype != rhs.dtype:
+            raise TTException("where: cond must be bool and all operands must share one shape")
+        out = Tensor.empty(lhs.shape, lhs.dtype, lhs.device)
+        _check(lib.ttamd_where(lhs.device.id, lhs.dtype, lhs.dim(), self._i64(lhs.shape), C.c_void_p(cond.storage.ptr),
+                               cond.offset, self._i64(cond.stride), C.c_void_p(lhs.storage.ptr), lhs.offset,
+                               self._i64(lhs.stride), C.c_void_p(rhs.storage.ptr), rhs.offset, self._i64(rhs.stride),
+                               C.c_void_p(out.storage.ptr), None))
+        return out
+
+    def sum(self, t: Tensor, dim: int | None = None) -> Tensor:
+        """BackendBase::sum(tensor) / sum(tensor, dim) (backend_base.h:148-149)."""
+        if dim is None:
+            out = Tensor.empty((1,), t.dtype, t.device)
+            d = -1
+        else:
+            d = dim % t.dim()
+            out = Tensor.empty(t.shape[:d] + t.shape[d + 1:], t.dtype, t.device)
+        _check(lib.ttamd_sum(t.device.id, t.dtype, t.dim(), self._i64(t.shape), C.c_void_p(t.storage.ptr), t.offset,
+                             self._i64(t.stride), d, C.c_void_p(out.storage.ptr), None))
+        return out
+
+    def full(self, value, numel: int, dtype: int, device: Device) -> Tensor:
+        """BackendBase::full (backend_base.h:51)."""
+        out = Tensor.empty((numel,), dtype, device)
+        host = np.array([value], dtype=_NP_OF[dtype])
+        _check(lib.ttamd_full(device.id, dtype, C.c_void_p(host.ctypes.data), numel, C.c_void_p(out.storage.ptr), None))
         return out
 
     def batched_matmul(self, lhs: Tensor, rhs: Tensor, bias: Tensor | None = None, bias_mode: int = 0,
@@ -339,6 +416,39 @@ def get_backend(device: Device) -> BackendAMD:
     if device.backend != "amd":
         raise TTException(f"Unknown device type {device.backend}")
     return _BACKEND
+
+
+def full(shape, value, dtype: int = _capi.F32, device: Device = kAMD) -> Tensor:
+    """tinytensor::full: a one-element storage expanded to `shape` (stride 0), like Tensor(Scalar).expand()."""
+    shape = tuple(shape)
+    one = get_backend(device).full(value, 1, dtype, device)
+    return Tensor(one.storage, dtype, shape, (0,) * len(shape), 0)
+
+
+def broadcast_tensors(a: Tensor, b: Tensor):
+    """Right-aligned broadcasting through unsqueeze + expand views (no data movement)."""
+    while a.dim() < b.dim():
+        a = a.unsqueeze(0)
+    while b.dim() < a.dim():
+        b = b.unsqueeze(0)
+    shape = []
+    for x, y in zip(a.shape, b.shape):
+        if x != y and x != 1 and y != 1:
+            raise TTException(f"Shapes {a.shape} and {b.shape} cannot be broadcast")
+        shape.append(max(x, y) if 0 not in (x, y) else 0)
+    return a.expand(shape), b.expand(shape)
+
+
+def where(cond: Tensor, lhs, rhs) -> Tensor:
+    """tinytensor::where with scalar or tensor branches."""
+    if not isinstance(lhs, Tensor):
+        lhs = full(cond.shape, lhs, rhs.dtype if isinstance(rhs, Tensor) else _capi.F32, cond.device)
+    if not isinstance(rhs, Tensor):
+        rhs = full(cond.shape, rhs, lhs.dtype, cond.device)
+    lhs, rhs = broadcast_tensors(lhs, rhs)
+    cond, lhs = broadcast_tensors(cond, lhs)
+    cond, rhs = broadcast_tensors(cond, rhs)
+    return get_backend(cond.device).where(cond, lhs, rhs)
 
 
 # -------------------------------------------------------------------------------------------------
