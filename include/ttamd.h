@@ -174,6 +174,14 @@ ttamd_status ttamd_sum(int device, ttamd_dtype dtype, int ndim, const int64_t *s
 /* BackendBase::full (backend_base.h:51): `value` points at one host scalar of `dtype`. */
 ttamd_status ttamd_full(int device, ttamd_dtype dtype, const void *value, int64_t numel, void *out, void *stream);
 
+/* BackendBase::uniform_real_ / normal_ (backend_base.h:96-103) for a dense float tensor with scalar parameters, as
+ * nn::Linear's default initialisation calls them (nn/init.cpp:30-52,106-112).  dist 0 = uniform_real(low = p0,
+ * high = p1), 1 = normal(mu = p0, std = p1).  *master_state is the caller's Generator state (tensor/random.cpp:46-63);
+ * it advances by numel outputs.  Per-element states are produced on the host and uploaded, as the reference's GPU
+ * backend does (cuda/distribution.cu:32-99), so uniform values are bit-identical to the CPU backend's. */
+ttamd_status ttamd_random_fill(int device, ttamd_dtype dtype, int dist, double p0, double p1, uint64_t *master_state,
+                               int64_t numel, void *out, void *stream);
+
 /* ---- timing (no reference counterpart: the reference has no timers; used by the benchmark
  * to bracket kernels with HIP events on the stream they run on) ------------------------ */
 ttamd_status ttamd_event_create(int device, void **event);

@@ -152,3 +152,28 @@ def test_mlp_training_step_entirely_on_device(tt, oracle):
         assert got[key].shape == want[key].shape
         assert max_rel_error(got[key], want[key]) <= 1e-4, key
     assert abs(float(got["loss"]) - float(want["loss"])) <= 1e-4 * abs(float(want["loss"]))
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+def test_seeded_draws_match_the_cpu_generator(tt, oracle, dtype):
+    code = tt._capi.F32 if dtype == np.float32 else tt._capi.F64
+    g_dev, g_cpu = tt.Generator(0), oracle.Generator(0)
+    assert g_dev.state.value == g_cpu.state
+    a = tt.uniform_real(-1.0, 1.0, (300, 17), g_dev, code).to_numpy()
+    assert np.array_equal(a, g_cpu.uniform_real(-1.0, 1.0, (300, 17), dtype))       # integer bit construction + one fma: exact
+    assert g_dev.state.value == g_cpu.state                                         # master generator advanced identically
+    b = tt.normal(0.0, 0.1, (5000,), g_dev, code).to_numpy()
+    want = g_cpu.normal(0.0, 0.1, (5000,), dtype)
+    assert g_dev.state.value == g_cpu.state
+    # Box-Muller goes through log1p / sqrt / sin of two different math libraries: tolerance, not bits
+    assert np.max(np.abs(b - want)) <= (2e-6 if dtype == np.float32 else 1e-13)
+    with pytest.raises(tt.TTException):
+        tt.uniform_real(1.0, 1.0, (4,), g_dev, code)
+
+
+def test_linear_default_init_on_device_equals_cpu_init(tt, oracle):
+    g_dev, g_cpu = tt.Generator(0), oracle.Generator(0)
+    for fan_in, fan_out in ((784, 1024), (1024, 10)):
+        W, b = tt.linear_init(fan_in, fan_out, g_dev)
+        Wc, bc = oracle.linear_init(g_cpu, fan_in, fan_out)
+        assert np.array_equal(W.to_numpy(), Wc) and np.array_equal(b.to_numpy(), bc)

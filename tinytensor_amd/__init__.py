@@ -5,7 +5,7 @@ thin host-side mirror of tinytensor's Tensor/backend interface for the GEMM path
 tests and the benchmark: same names, argument meaning and error behaviour as the reference's C++ API.
 """
 from .tensor import (  # noqa: F401
-    BackendAMD, Device, Tensor, TTException, broadcast_tensors, conv2d, conv2d_backward, full, get_backend, kAMD, linear,
+    BackendAMD, Device, Generator, Tensor, TTException, broadcast_tensors, linear_init, normal, uniform_real, conv2d, conv2d_backward, full, get_backend, kAMD, linear,
     matmul, matmul_backward, where,
 )
 from . import _capi  # noqa: F401

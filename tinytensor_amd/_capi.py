@@ -51,6 +51,7 @@ def _bind(lib: C.CDLL) -> None:
                             C.POINTER(C.c_int64), vp, C.c_int64, C.POINTER(C.c_int64), vp, vp]),
         "ttamd_sum": (i, [i, i, i, C.POINTER(C.c_int64), vp, C.c_int64, C.POINTER(C.c_int64), i, vp, vp]),
         "ttamd_full": (i, [i, i, vp, C.c_int64, vp, vp]),
+        "ttamd_random_fill": (i, [i, i, i, C.c_double, C.c_double, C.POINTER(C.c_uint64), C.c_int64, vp, vp]),
         "ttamd_batched_matmul": (i, [i, i, i, i, i, i, C.POINTER(View3), C.POINTER(View3), vp, C.POINTER(Epilogue), vp]),
         "ttamd_batched_matmul_variant": (C.c_char_p, [i, i, i, i, i, C.POINTER(View3), C.POINTER(View3)]),
         "ttamd_conv2d_forward": (i, [i, i, C.POINTER(View4), C.POINTER(View4), vp, vp] + [i] * 8 + [vp]),

@@ -182,6 +182,41 @@ __global__ void __launch_bounds__(256) sum_all_kernel(const T *__restrict__ a, V
     if (threadIdx.x == 0) out[blockIdx.x] = red[0];
 }
 
+// Seeded draws (tinytensor/tensor/random.cpp:36-43, backend/common/kernel/distribution.hpp:92-99, 232-246):
+// element i owns a generator whose state is the i-th output of the master generator; the states are produced on
+// the host and uploaded, exactly as the reference's GPU backend does (cuda/distribution.cu:32-99).
+__device__ __forceinline__ uint64_t xorshift64(uint64_t &x) {
+    x ^= x << 13;
+    x ^= x >> 7;
+    x ^= x << 17;
+    return x;
+}
+__device__ __forceinline__ float unit_sample(uint64_t &st, float) {
+    return __builtin_bit_cast(float, (static_cast<uint32_t>(xorshift64(st)) >> 9) | 0x3F800000u) - 1.0f;
+}
+__device__ __forceinline__ double unit_sample(uint64_t &st, double) {
+    return __builtin_bit_cast(double, (xorshift64(st) >> 12) | 0x3FF0000000000000ull) - 1.0;
+}
+template <typename T>
+__global__ void __launch_bounds__(256) uniform_real_kernel(const uint64_t *__restrict__ states, T low, T high, T *__restrict__ out, int64_t n) {
+    const int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    uint64_t st = states[i];
+    const T r = unit_sample(st, T(0));
+    out[i] = fma(r, high - low, low);  // r * (high - low) + low, contracted as the fma flavour of the host build does
+}
+template <typename T>
+__global__ void __launch_bounds__(256) normal_kernel(const uint64_t *__restrict__ states, T mu, T stddev, T *__restrict__ out, int64_t n) {
+    const int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    uint64_t st = states[i];
+    const T u1 = unit_sample(st, T(0));
+    const T u2 = unit_sample(st, T(0));
+    const T r = sqrt(T(-2) * log1p(-u1));
+    const T theta = T(2) * T(3.14159265358979323846) * u2;
+    out[i] = stddev * (r * sin(theta)) + mu;
+}
+
 inline unsigned grid_for(int64_t numel) {
     int64_t blocks = (numel + 255) / 256;
     if (blocks > 8192) blocks = 8192;
@@ -501,6 +536,71 @@ ttamd_status ttamd_full(int device, ttamd_dtype dtype, const void *value, int64_
     case 4: return run(uint32_t{});
     default: return run(uint64_t{});
     }
+}
+
+
+// dist: 0 = uniform_real(low = p0, high = p1), 1 = normal(mu = p0, std = p1).  *master_state is the host-side master
+// generator state (Generator::state); it advances by n outputs.
+ttamd_status ttamd_random_fill(int device, ttamd_dtype dtype, int dist, double p0, double p1, uint64_t *master_state, int64_t numel,
+                               void *out, void *stream) {
+    if (dtype != TTAMD_F32 && dtype != TTAMD_F64) {
+        set_error("random_fill: floating point dtypes only");
+        return TTAMD_ERR_UNSUPPORTED_DTYPE;
+    }
+    if (!master_state || numel < 0 || (dist != 0 && dist != 1) || (dist == 0 && !(p0 < p1))) {
+        set_error("random_fill: invalid arguments (Expected low < high for uniform_real)");
+        return TTAMD_ERR_INVALID_ARGUMENT;
+    }
+    if (ttamd_status s = use_device(device)) return s;
+    if (numel == 0) return TTAMD_OK;
+    if (!out) {
+        set_error("random_fill: out is NULL");
+        return TTAMD_ERR_INVALID_ARGUMENT;
+    }
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    // per-element generator states, produced on the host in order (cpu/distribution.cpp:31-38)
+    uint64_t *host_states = nullptr;
+    TTAMD_HIP_CHECK(hipHostMalloc(reinterpret_cast<void **>(&host_states), static_cast<size_t>(numel) * sizeof(uint64_t), hipHostMallocDefault));
+    uint64_t x = *master_state;
+    for (int64_t i = 0; i < numel; ++i) {
+        x ^= x << 13;
+        x ^= x >> 7;
+        x ^= x << 17;
+        host_states[i] = x;
+    }
+    *master_state = x;
+    void *dev_states = nullptr;
+    hipError_t e = hipMalloc(&dev_states, static_cast<size_t>(numel) * sizeof(uint64_t));
+    if (e != hipSuccess) {
+        (void)hipGetLastError();
+        (void)hipHostFree(host_states);
+        set_error("random_fill: unable to allocate %lld generator states", static_cast<long long>(numel));
+        return TTAMD_ERR_OUT_OF_MEMORY;
+    }
+    ttamd_status rc = TTAMD_OK;
+    auto fail = [&](hipError_t err, const char *what) {
+        set_error("%s failed: %s", what, hipGetErrorString(err));
+        rc = TTAMD_ERR_LAUNCH;
+    };
+    if ((e = hipMemcpyAsync(dev_states, host_states, static_cast<size_t>(numel) * sizeof(uint64_t), hipMemcpyHostToDevice, st)) != hipSuccess)
+        fail(e, "hipMemcpyAsync");
+    if (rc == TTAMD_OK) {
+        const unsigned blocks = static_cast<unsigned>((numel + 255) / 256);
+        const uint64_t *sp = static_cast<const uint64_t *>(dev_states);
+        if (dtype == TTAMD_F32) {
+            if (dist == 0) uniform_real_kernel<float><<<dim3(blocks), dim3(256), 0, st>>>(sp, static_cast<float>(p0), static_cast<float>(p1), static_cast<float *>(out), numel);
+            else normal_kernel<float><<<dim3(blocks), dim3(256), 0, st>>>(sp, static_cast<float>(p0), static_cast<float>(p1), static_cast<float *>(out), numel);
+        } else {
+            if (dist == 0) uniform_real_kernel<double><<<dim3(blocks), dim3(256), 0, st>>>(sp, p0, p1, static_cast<double *>(out), numel);
+            else normal_kernel<double><<<dim3(blocks), dim3(256), 0, st>>>(sp, p0, p1, static_cast<double *>(out), numel);
+        }
+        if ((e = hipGetLastError()) != hipSuccess) fail(e, "kernel launch");
+    }
+    // the staging buffers are released after the stream has consumed them
+    if ((e = hipStreamSynchronize(st)) != hipSuccess && rc == TTAMD_OK) fail(e, "hipStreamSynchronize");
+    (void)hipFree(dev_states);
+    (void)hipHostFree(host_states);
+    return rc;
 }
 
 }  // extern "C"

@@ -418,6 +418,46 @@ def get_backend(device: Device) -> BackendAMD:
     return _BACKEND
 
 
+class Generator:
+    """tinytensor::Generator (tensor/random.cpp:46-63): state = splitmix64(seed); xorshift64 steps."""
+
+    def __init__(self, seed: int = 0):
+        m = (1 << 64) - 1
+        r = (seed + 0x9E3779B97F4A7C15) & m
+        r = ((r ^ (r >> 30)) * 0xBF58476D1CE4E5B9) & m
+        r = ((r ^ (r >> 27)) * 0x94D049BB133111EB) & m
+        self.state = C.c_uint64(r ^ (r >> 31))
+
+
+def _random_fill(shape, dtype, dist, p0, p1, gen: Generator, device: Device) -> Tensor:
+    out = Tensor.empty(shape, dtype, device)
+    _check(lib.ttamd_random_fill(device.id, dtype, dist, p0, p1, C.byref(gen.state), out.numel(),
+                                 C.c_void_p(out.storage.ptr), None))
+    return out
+
+
+def uniform_real(low: float, high: float, shape, gen: Generator, dtype: int = _capi.F32, device: Device = kAMD) -> Tensor:
+    """tinytensor::uniform_real(low, high, shape, options, gen) (tensor/tensor.cpp:1773-1781)."""
+    if not low < high:
+        raise TTException("Expected low < high. At least one element violates this.")
+    return _random_fill(shape, dtype, 0, low, high, gen, device)
+
+
+def normal(mu: float, std: float, shape, gen: Generator, dtype: int = _capi.F32, device: Device = kAMD) -> Tensor:
+    return _random_fill(shape, dtype, 1, mu, std, gen, device)
+
+
+def linear_init(in_features: int, out_features: int, gen: Generator, dtype: int = _capi.F32, device: Device = kAMD):
+    """nn::Linear's constructor (nn/linear.cpp:20-40): weight [in,out] by kaiming_uniform_ (gain 1, fan = size(0)),
+    then bias ~ U(+-1/sqrt(fan)); both drawn from `gen` in that order."""
+    fan = float(in_features)
+    bound_w = (3.0 ** 0.5) * (1.0 / fan ** 0.5)
+    W = uniform_real(-bound_w, bound_w, (in_features, out_features), gen, dtype, device)
+    bound_b = 1.0 / fan ** 0.5
+    b = uniform_real(-bound_b, bound_b, (out_features,), gen, dtype, device)
+    return W, b
+
+
 def full(shape, value, dtype: int = _capi.F32, device: Device = kAMD) -> Tensor:
     """tinytensor::full: a one-element storage expanded to `shape` (stride 0), like Tensor(Scalar).expand()."""
     shape = tuple(shape)
