@@ -60,13 +60,14 @@ struct ConvGeom {
 // B operand of the forward product: Xu[kk][n] gathered from image b.  MC layout (n contiguous), one
 // element per load.  A lane keeps one output position n for the whole kernel; the kk of a pass is
 // wave-uniform, so its (c, p, q) decode runs on the scalar unit.
-template <typename T, int ROWS, int BK>
+template <typename T, int ROWS, int BK, int PF = 1>
 struct Im2colStager : TileLayout<T, ROWS, BK, false> {
     using L = TileLayout<T, ROWS, BK, false>;
     static constexpr int LPP = kThreads / ROWS;  // k lines per pass
     static constexpr int P = BK / LPP;
     static_assert(ROWS % 64 == 0 && BK % LPP == 0, "a wave must share its k line");
-    T reg[P];
+    static constexpr int kPF = PF;
+    T reg[PF][P];
     __amdgpu_buffer_rsrc_t rsrc;
     const ConvGeom *g;
     int n_local, line0, k_next, K;
@@ -90,7 +91,7 @@ struct Im2colStager : TileLayout<T, ROWS, BK, false> {
         base_b = (ih0 * geo.xs_h + iw0 * geo.xs_w) * static_cast<int32_t>(sizeof(T));
     }
 
-    template <bool MASK>
+    template <bool MASK, int SLOT = 0>
     __device__ __forceinline__ void load(int /*k_left*/) {
 #pragma unroll
         for (int p = 0; p < P; ++p) {
@@ -103,14 +104,15 @@ struct Im2colStager : TileLayout<T, ROWS, BK, false> {
             const int ih = ih0 + static_cast<int>(pp), iw = iw0 + static_cast<int>(q);
             const bool ok = n_ok && kk < K && static_cast<unsigned>(ih) < static_cast<unsigned>(g->H) &&
                             static_cast<unsigned>(iw) < static_cast<unsigned>(g->W);
-            reg[p] = Vec<T, 1>::load(rsrc, ok ? static_cast<uint32_t>(base_b + koff) : kOob);
+            reg[SLOT][p] = Vec<T, 1>::load(rsrc, ok ? static_cast<uint32_t>(base_b + koff) : kOob);
         }
         k_next += BK;
     }
 
+    template <int SLOT = 0>
     __device__ __forceinline__ void store(T *lds) const {
 #pragma unroll
-        for (int p = 0; p < P; ++p) lds[(p * LPP + line0) * L::LD + n_local] = reg[p];
+        for (int p = 0; p < P; ++p) lds[(p * LPP + line0) * L::LD + n_local] = reg[SLOT][p];
     }
 };
 
@@ -118,13 +120,14 @@ struct Im2colStager : TileLayout<T, ROWS, BK, false> {
 // B operand of grad_weight: XuT[n][j] with n = output position (the reduction index) and j = (c,p,q)
 // (the column index).  KC layout (n contiguous), one element per load.  The j of each pass is fixed for
 // the whole kernel and decoded once; the n of a lane advances by BK per tile.
-template <typename T, int ROWS, int BK>
+template <typename T, int ROWS, int BK, int PF = 1>
 struct Im2colTStager : TileLayout<T, ROWS, BK, true> {
     using L = TileLayout<T, ROWS, BK, true>;
     static constexpr int RPP = kThreads / BK;  // j rows per pass
     static constexpr int P = ROWS / RPP;
     static_assert(ROWS % RPP == 0, "tile must split evenly");
-    T reg[P];
+    static constexpr int kPF = PF;
+    T reg[PF][P];
     __amdgpu_buffer_rsrc_t rsrc;
     const ConvGeom *g;
     int32_t joff[P];  // byte offset of tap (c, p - P, q - P)
@@ -158,7 +161,7 @@ struct Im2colTStager : TileLayout<T, ROWS, BK, true> {
         k_next = 0;
     }
 
-    template <bool MASK>
+    template <bool MASK, int SLOT = 0>
     __device__ __forceinline__ void load(int /*k_left*/) {
         const int n = k_next + k_local;
         const bool n_ok = n < HoWo;
@@ -171,26 +174,28 @@ struct Im2colTStager : TileLayout<T, ROWS, BK, true> {
             const int ih = ih0 + dp[p], iw = iw0 + dq[p];
             const bool ok = n_ok && j_ok[p] && static_cast<unsigned>(ih) < static_cast<unsigned>(g->H) &&
                             static_cast<unsigned>(iw) < static_cast<unsigned>(g->W);
-            reg[p] = Vec<T, 1>::load(rsrc, ok ? static_cast<uint32_t>(base_b + joff[p]) : kOob);
+            reg[SLOT][p] = Vec<T, 1>::load(rsrc, ok ? static_cast<uint32_t>(base_b + joff[p]) : kOob);
         }
         k_next += BK;
     }
 
+    template <int SLOT = 0>
     __device__ __forceinline__ void store(T *lds) const {
 #pragma unroll
-        for (int p = 0; p < P; ++p) lds[(p * RPP + row0) * L::LD + k_local] = reg[p];
+        for (int p = 0; p < P; ++p) lds[(p * RPP + row0) * L::LD + k_local] = reg[SLOT][p];
     }
 };
 
 // ---------------------------------------------------------------------------------------------
 // A operand of grad_input: Wt[c][kk] = W[o][c][p][q] with kk = (o,p,q).  KC layout, one element per load;
 // a lane keeps one kk per tile (decoded per tile), the channel row varies per pass.
-template <typename T, int ROWS, int BK>
+template <typename T, int ROWS, int BK, int PF = 1>
 struct WeightTStager : TileLayout<T, ROWS, BK, true> {
     using L = TileLayout<T, ROWS, BK, true>;
     static constexpr int RPP = kThreads / BK;
     static constexpr int P = ROWS / RPP;
-    T reg[P];
+    static constexpr int kPF = PF;
+    T reg[PF][P];
     __amdgpu_buffer_rsrc_t rsrc;
     const ConvGeom *g;
     int k_local, row0, k_next, K, c0, kk2;
@@ -206,7 +211,7 @@ struct WeightTStager : TileLayout<T, ROWS, BK, true> {
         c0 = c0_;
     }
 
-    template <bool MASK>
+    template <bool MASK, int SLOT = 0>
     __device__ __forceinline__ void load(int /*k_left*/) {
         const int kk = k_next + k_local;
         const bool k_ok = kk < K;
@@ -218,26 +223,28 @@ struct WeightTStager : TileLayout<T, ROWS, BK, true> {
             const int c = c0 + p * RPP + row0;
             const bool ok = k_ok && c < g->C;
             const int64_t off = (koff + static_cast<int64_t>(c) * kk2) * static_cast<int64_t>(sizeof(T));
-            reg[p] = Vec<T, 1>::load(rsrc, ok ? static_cast<uint32_t>(off) : kOob);
+            reg[SLOT][p] = Vec<T, 1>::load(rsrc, ok ? static_cast<uint32_t>(off) : kOob);
         }
         k_next += BK;
     }
 
+    template <int SLOT = 0>
     __device__ __forceinline__ void store(T *lds) const {
 #pragma unroll
-        for (int p = 0; p < P; ++p) lds[(p * RPP + row0) * L::LD + k_local] = reg[p];
+        for (int p = 0; p < P; ++p) lds[(p * RPP + row0) * L::LD + k_local] = reg[SLOT][p];
     }
 };
 
 // B operand of grad_input: G[kk][n] = g[b][o][(y+P-p)/S][(x+P-q)/S], kk = (o,p,q), n = (y,x).  MC layout;
 // the lane's input position is fixed, kk is wave-uniform per pass.
-template <typename T, int ROWS, int BK>
+template <typename T, int ROWS, int BK, int PF = 1>
 struct DgradStager : TileLayout<T, ROWS, BK, false> {
     using L = TileLayout<T, ROWS, BK, false>;
     static constexpr int LPP = kThreads / ROWS;
     static constexpr int P = BK / LPP;
     static_assert(ROWS % 64 == 0 && BK % LPP == 0, "a wave must share its k line");
-    T reg[P];
+    static constexpr int kPF = PF;
+    T reg[PF][P];
     __amdgpu_buffer_rsrc_t rsrc;
     const ConvGeom *g;
     int n_local, line0, k_next, K, HoWo;
@@ -260,7 +267,7 @@ struct DgradStager : TileLayout<T, ROWS, BK, false> {
         xP = static_cast<int>(x) + geo.P;
     }
 
-    template <bool MASK>
+    template <bool MASK, int SLOT = 0>
     __device__ __forceinline__ void load(int /*k_left*/) {
 #pragma unroll
         for (int p = 0; p < P; ++p) {
@@ -276,14 +283,15 @@ struct DgradStager : TileLayout<T, ROWS, BK, false> {
             ok = ok && rh == 0 && rw == 0 && static_cast<int>(oh) < g->Ho && static_cast<int>(ow) < g->Wo;
             const uint32_t off = (o * static_cast<uint32_t>(HoWo) + oh * static_cast<uint32_t>(g->Wo) + ow) *
                                  static_cast<uint32_t>(sizeof(T));
-            reg[p] = Vec<T, 1>::load(rsrc, ok ? off : kOob);
+            reg[SLOT][p] = Vec<T, 1>::load(rsrc, ok ? off : kOob);
         }
         k_next += BK;
     }
 
+    template <int SLOT = 0>
     __device__ __forceinline__ void store(T *lds) const {
 #pragma unroll
-        for (int p = 0; p < P; ++p) lds[(p * LPP + line0) * L::LD + n_local] = reg[p];
+        for (int p = 0; p < P; ++p) lds[(p * LPP + line0) * L::LD + n_local] = reg[SLOT][p];
     }
 };
 

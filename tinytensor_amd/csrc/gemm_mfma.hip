@@ -16,11 +16,14 @@ using namespace mfma;
 
 // ksplit > 1: the reduction is cut into `ksplit` ranges of `k_chunk` (a multiple of BK); workgroup column z =
 // batch * ksplit + split writes the raw partial tile to `partial[z]` and splitk_reduce_kernel finishes the job.
-template <typename T, int BM, int BN, int BK, int WGM, int WGN, bool A_KC, int A_VEC, bool B_KC, int B_VEC>
+// PF = tiles kept in flight in registers: 1 for the big tiles (two workgroups per CU hide each other's load
+// latency, and registers are scarce), more for the 64 x 64 tile whose 16 MFMAs per k tile (~0.45 us) are far
+// shorter than a global load.
+template <typename T, int BM, int BN, int BK, int WGM, int WGN, bool A_KC, int A_VEC, bool B_KC, int B_VEC, int PF>
 __global__ void __launch_bounds__(kThreads, 2)
 gemm_mfma_kernel(GemmArgs g, int tiles_m, int tiles_n, int ksplit, int k_chunk, T *partial) {
-    using StA = Stager<T, BM, BK, A_KC, A_VEC>;
-    using StB = Stager<T, BN, BK, B_KC, B_VEC>;
+    using StA = Stager<T, BM, BK, A_KC, A_VEC, PF>;
+    using StB = Stager<T, BN, BK, B_KC, B_VEC, PF>;
     using Engine = TileEngine<T, BM, BN, BK, WGM, WGN, StA, StB>;
     extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
     T *const smem = reinterpret_cast<T *>(smem_raw);
@@ -94,6 +97,27 @@ OperandClass classify(const void *ptr, int64_t s_row, int64_t s_k, int64_t s_b, 
     return {s_k <= s_row, 1};
 }
 
+template <typename T>
+struct TileShapes;
+template <>
+struct TileShapes<float> {
+    static constexpr bool kHasXL = true;
+    static constexpr int XBM = 256, XBN = 128, XBK = 16;  // extra large: 4 waves of 128 x 64 (4 x 2 MFMA blocks)
+    static constexpr int LBM = 128, LBN = 128, LBK = 32;  // large: 4 waves of 64 x 64
+    static constexpr int SBM = 64, SBN = 64, SBK = 32;    // small: 4 waves of 32 x 32
+    static constexpr int SPF = 1;                          // deeper register prefetch measured slower (more registers, same stalls)
+    static constexpr const char *prefix = "mfma_f32";
+};
+template <>
+struct TileShapes<double> {
+    static constexpr bool kHasXL = false;                  // a 128 x 64 wave tile would need 256 accumulator registers
+    static constexpr int XBM = 128, XBN = 128, XBK = 16;
+    static constexpr int LBM = 128, LBN = 128, LBK = 16;  // 4 waves of 64 x 64 (4 x 4 blocks of 16 x 16)
+    static constexpr int SBM = 64, SBN = 64, SBK = 16;    // 4 waves of 32 x 32
+    static constexpr int SPF = 1;
+    static constexpr const char *prefix = "mfma_f64";
+};
+
 struct SplitPlan {
     int ksplit = 1;
     int k_chunk = 0;
@@ -101,10 +125,11 @@ struct SplitPlan {
 
 template <typename T, int BM, int BN, int BK, int WGM, int WGN, bool A_KC, int A_VEC, bool B_KC, int B_VEC>
 ttamd_status launch_variant(const GemmArgs &g, const SplitPlan &sp, int device, hipStream_t stream) {
-    using StA = Stager<T, BM, BK, A_KC, A_VEC>;
-    using StB = Stager<T, BN, BK, B_KC, B_VEC>;
+    constexpr int PF = (BM <= 64 && BN <= 64) ? TileShapes<T>::SPF : 1;
+    using StA = Stager<T, BM, BK, A_KC, A_VEC, PF>;
+    using StB = Stager<T, BN, BK, B_KC, B_VEC, PF>;
     constexpr size_t lds_bytes = TileEngine<T, BM, BN, BK, WGM, WGN, StA, StB>::kLdsBytes;
-    auto kernel = gemm_mfma_kernel<T, BM, BN, BK, WGM, WGN, A_KC, A_VEC, B_KC, B_VEC>;
+    auto kernel = gemm_mfma_kernel<T, BM, BN, BK, WGM, WGN, A_KC, A_VEC, B_KC, B_VEC, PF>;
     static bool configured = false;  // raising the dynamic LDS limit is per kernel, once
     if (!configured && lds_bytes > 48 * 1024) {
         TTAMD_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
@@ -142,25 +167,6 @@ ttamd_status launch_layouts(const GemmArgs &g, bool a_kc, bool b_kc, const Split
     if (!a_kc && b_kc) return launch_variant<T, BM, BN, BK, WGM, WGN, false, A_VEC, true, B_VEC>(g, sp, device, stream);
     return launch_variant<T, BM, BN, BK, WGM, WGN, false, A_VEC, false, B_VEC>(g, sp, device, stream);
 }
-
-template <typename T>
-struct TileShapes;
-template <>
-struct TileShapes<float> {
-    static constexpr bool kHasXL = true;
-    static constexpr int XBM = 256, XBN = 128, XBK = 16;  // extra large: 4 waves of 128 x 64 (4 x 2 MFMA blocks)
-    static constexpr int LBM = 128, LBN = 128, LBK = 32;  // large: 4 waves of 64 x 64
-    static constexpr int SBM = 64, SBN = 64, SBK = 32;    // small: 4 waves of 32 x 32
-    static constexpr const char *prefix = "mfma_f32";
-};
-template <>
-struct TileShapes<double> {
-    static constexpr bool kHasXL = false;                  // a 128 x 64 wave tile would need 256 accumulator registers
-    static constexpr int XBM = 128, XBN = 128, XBK = 16;
-    static constexpr int LBM = 128, LBN = 128, LBK = 16;  // 4 waves of 64 x 64 (4 x 4 blocks of 16 x 16)
-    static constexpr int SBM = 64, SBN = 64, SBK = 16;    // 4 waves of 32 x 32
-    static constexpr const char *prefix = "mfma_f64";
-};
 
 // Split the reduction when the output has too few tiles to fill 256 CUs and K is long enough to share out.
 // Every split gets a whole number of BK tiles; at most 64 splits and 32 MiB of partial tiles.

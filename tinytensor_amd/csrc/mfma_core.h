@@ -15,8 +15,9 @@
 //
 // A stager is any type with
 //     static constexpr bool kKC; static constexpr int LD, LDS_ELEMS;
-//     template <bool MASK> void load(int k_left);   // fetch the next BK-deep tile into registers
-//     void store(T *lds) const;                       // write those registers to an LDS buffer
+//     static constexpr int kPF;                                  // register slots = tiles kept in flight
+//     template <bool MASK, int SLOT> void load(int k_left);      // fetch the next BK-deep tile into slot SLOT
+//     template <int SLOT> void store(T *lds) const;              // write that slot to an LDS buffer
 // Stager<> below reads a strided matrix view; conv.hip adds gather stagers (implicit im2col).
 #ifndef TTAMD_CSRC_MFMA_CORE_H_
 #define TTAMD_CSRC_MFMA_CORE_H_
@@ -140,16 +141,18 @@ struct TileLayout {
 // ---------------------------------------------------------------------------------------------
 // Stager for a strided matrix view (ROWS along m or n, BK along k).  Vectors of VEC elements run along k
 // for KC (operand's k stride is 1 when VEC > 1) and along the row index for MC (row stride 1 when VEC > 1).
-template <typename T, int ROWS, int BK, bool KC, int VEC>
+// PF register slots hold PF tiles in flight (prefetch distance PF).
+template <typename T, int ROWS, int BK, bool KC, int VEC, int PF = 1>
 struct Stager : TileLayout<T, ROWS, BK, KC> {
     using L = TileLayout<T, ROWS, BK, KC>;
     using V = typename Vec<T, VEC>::type;
+    static constexpr int kPF = PF;
     static constexpr int VPL = (KC ? BK : ROWS) / VEC;  // vectors per LDS line
     static constexpr int NV = ROWS * BK / VEC;
     static constexpr int P = NV / kThreads;
     static_assert(NV % kThreads == 0, "tile must split evenly over the workgroup");
 
-    V reg[P];
+    V reg[PF][P];
     uint32_t voff[P];
     int nval[P];  // MC only: valid components of the vector along the row dimension
     __amdgpu_buffer_rsrc_t rsrc;
@@ -188,9 +191,9 @@ struct Stager : TileLayout<T, ROWS, BK, KC> {
         }
     }
 
-    // Fetches the next tile; k_left = K - (first k of that tile).  MASK = false is the steady state
-    // (full k tile, interior rows): loads only, no selects.
-    template <bool MASK>
+    // Fetches the next tile into register slot SLOT; k_left = K - (first k of that tile).  MASK = false is
+    // the steady state (full k tile, interior rows): loads only, no selects.
+    template <bool MASK, int SLOT = 0>
     __device__ __forceinline__ void load(int k_left) {
         const bool k_tail = k_left < BK;
 #pragma unroll
@@ -198,7 +201,7 @@ struct Stager : TileLayout<T, ROWS, BK, KC> {
             V v = Vec<T, VEC>::load(rsrc, voff[p]);
             voff[p] += k_step_b;
             if constexpr (!MASK) {
-                reg[p] = v;
+                reg[SLOT][p] = v;
                 continue;
             }
             if constexpr (KC) {
@@ -221,15 +224,16 @@ struct Stager : TileLayout<T, ROWS, BK, KC> {
                         if (j >= nval[p]) zero_component<T, VEC>(v, j);
                 }
             }
-            reg[p] = v;
+            reg[SLOT][p] = v;
         }
     }
 
+    template <int SLOT = 0>
     __device__ __forceinline__ void store(T *lds) const {
 #pragma unroll
         for (int p = 0; p < P; ++p) {
             const int line = line_of(p, tid), col = col_of(p, tid);
-            *reinterpret_cast<V *>(&lds[line * L::LD + col]) = reg[p];
+            *reinterpret_cast<V *>(&lds[line * L::LD + col]) = reg[SLOT][p];
         }
     }
 };
@@ -356,47 +360,81 @@ struct TileEngine {
     }
     __device__ __forceinline__ void compute(const T *smem, int buf) { compute_chunks(smem, buf, 0, BK / kChunk); }
 
+    // One pipeline step for tile kt, whose register slot arithmetic is static: tile t lives in slot t % PF.
+    //   LOAD: issue the global loads of tile kt + PF into slot kt % PF (free: tile kt is already in LDS);
+    //   multiply tile kt out of LDS buffer kt & 1; park tile kt + 1 (slot (kt + 1) % PF, loaded PF - 1 steps
+    //   ago) in the other LDS buffer, its stores slotted between the MFMAs of the last chunk.
+    template <int S, bool LOAD, bool MASK>
+    __device__ __forceinline__ void step(StA &sa, StB &sb, T *smem, int K, int kt) {
+        constexpr int PF = StA::kPF;
+        constexpr int NC = BK / kChunk;
+        constexpr int kLastMfmas = M::VK * NBM * NBN;  // MFMAs of one chunk
+        constexpr int kStores = StA::P + StB::P;       // LDS store instructions of one tile (per lane)
+        const int cur = kt & 1;
+        if constexpr (LOAD) {
+            const int k_left = K - (kt + PF) * BK;
+            sa.template load<MASK, S>(k_left);
+            sb.template load<MASK, S>(k_left);
+        }
+        // Keep the global loads ahead of the MFMA work: left alone, the scheduler sinks them to just before
+        // the LDS stores and their latency is exposed on every tile.
+        __builtin_amdgcn_sched_barrier(0);
+        compute_chunks(smem, cur, 0, NC - 1);
+        __builtin_amdgcn_sched_barrier(0);
+        // Last chunk: its MFMAs run with the LDS stores of the next tile slotted between them.  The other
+        // buffer was last read before the previous barrier, so it may be written as soon as the global data
+        // has arrived; by the time the last MFMA issues the stores have drained and the barrier costs no
+        // pipe time (stores placed after the MFMAs cost ~9 % at 4096^3).
+        compute_chunks(smem, cur, NC - 1, NC);
+        sa.template store<(S + 1) % PF>(smem + (cur ^ 1) * StA::LDS_ELEMS);
+        sb.template store<(S + 1) % PF>(smem + kBOff + (cur ^ 1) * StB::LDS_ELEMS);
+        if constexpr (kLastMfmas >= 2 * kStores) {
+#pragma unroll
+            for (int i = 0; i < kStores; ++i) {
+                __builtin_amdgcn_sched_group_barrier(0x008, kLastMfmas / kStores > 2 ? 2 : 1, 0);  // MFMA
+                __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);                                 // DS write
+            }
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        __syncthreads();
+    }
+
+    template <bool LOAD, bool MASK, int S = 0>
+    __device__ __forceinline__ void step_any(StA &sa, StB &sb, T *smem, int K, int kt, int slot) {
+        if constexpr (S < StA::kPF) {
+            if (slot == S) step<S, LOAD, MASK>(sa, sb, smem, K, kt);
+            else step_any<LOAD, MASK, S + 1>(sa, sb, smem, K, kt, slot);
+        }
+    }
+
     // K: reduction length.  `unmasked`: workgroup-uniform promise that every tile is full and interior.
     __device__ __forceinline__ void run(StA &sa, StB &sb, T *smem, int K, bool unmasked) {
+        constexpr int PF = StA::kPF;
+        static_assert(StA::kPF == StB::kPF, "both operands use the same prefetch distance");
         const int KT = (K + BK - 1) / BK;
-        sa.template load<true>(K);
-        sb.template load<true>(K);
-        sa.store(smem);
-        sb.store(smem + kBOff);
+        // Prologue: tile 0 goes straight to LDS, tiles 1 .. PF-1 are put in flight.
+        sa.template load<true, 0>(K);
+        sb.template load<true, 0>(K);
+        sa.template store<0>(smem);
+        sb.template store<0>(smem + kBOff);
+        prefetch_rest<1>(sa, sb, K, KT);
         __syncthreads();
-        // Tiles 0 .. KT-2: prefetch tile kt+1 into registers, multiply tile kt out of LDS, then park the
-        // prefetched tile in the other LDS buffer.  The last tile is multiplied after the loop, so the loop
-        // body has no conditionals.
-        constexpr int NC = BK / kChunk;
-        constexpr int kLastMfmas = M::VK * NBM * NBN;     // MFMAs of one chunk
-        constexpr int kStores = StA::P + StB::P;          // LDS store instructions of one tile (per lane)
+        // Tiles 0 .. KT-2 (the last tile is multiplied after the loop).  While kt + PF < KT every step also
+        // issues loads; the remaining steps only drain the slots.
         auto pipeline = [&]<bool MASK>() {
-            for (int kt = 0; kt + 1 < KT; ++kt) {
-                const int cur = kt & 1;
-                const int k_left = K - (kt + 1) * BK;
-                sa.template load<MASK>(k_left);
-                sb.template load<MASK>(k_left);
-                // Keep the global loads ahead of the MFMA work: left alone, the scheduler sinks them to just
-                // before the LDS stores and their latency is exposed on every tile.
-                __builtin_amdgcn_sched_barrier(0);
-                compute_chunks(smem, cur, 0, NC - 1);
-                __builtin_amdgcn_sched_barrier(0);
-                // Last chunk: its MFMAs run with the LDS stores of the prefetched tile slotted between them.
-                // The other buffer was last read before the previous barrier, so it may be written as soon as
-                // the global data has arrived; by the time the last MFMA issues the stores have drained and
-                // the barrier costs no pipe time (stores placed after the MFMAs cost ~9 % at 4096^3).
-                compute_chunks(smem, cur, NC - 1, NC);
-                sa.store(smem + (cur ^ 1) * StA::LDS_ELEMS);
-                sb.store(smem + kBOff + (cur ^ 1) * StB::LDS_ELEMS);
-                if constexpr (kLastMfmas >= 2 * kStores) {
-#pragma unroll
-                    for (int i = 0; i < kStores; ++i) {
-                        __builtin_amdgcn_sched_group_barrier(0x008, kLastMfmas / kStores > 2 ? 2 : 1, 0);  // MFMA
-                        __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);                                 // DS write
-                    }
+            int kt = 0;
+            if constexpr (PF == 1) {
+                for (; kt + 1 < KT; ++kt) step<0, true, MASK>(sa, sb, smem, K, kt);
+            } else {
+                int slot = 0;
+                for (; kt + PF < KT; ++kt) {
+                    step_any<true, MASK>(sa, sb, smem, K, kt, slot);
+                    slot = slot + 1 == PF ? 0 : slot + 1;
                 }
-                __builtin_amdgcn_sched_barrier(0);
-                __syncthreads();
+                for (; kt + 1 < KT; ++kt) {
+                    step_any<false, MASK>(sa, sb, smem, K, kt, slot);
+                    slot = slot + 1 == PF ? 0 : slot + 1;
+                }
             }
         };
         if (unmasked) {
@@ -405,6 +443,17 @@ struct TileEngine {
             pipeline.template operator()<true>();
         }
         if (KT > 0) compute(smem, (KT - 1) & 1);
+    }
+
+    template <int S>
+    __device__ __forceinline__ void prefetch_rest(StA &sa, StB &sb, int K, int KT) {
+        if constexpr (S < StA::kPF) {
+            if (S < KT) {
+                sa.template load<true, S>(K - S * BK);
+                sb.template load<true, S>(K - S * BK);
+            }
+            prefetch_rest<S + 1>(sa, sb, K, KT);
+        }
     }
 
     // Walks the finished tile.  `one(m, n, v)` receives a single element at tile-local (m, n);
