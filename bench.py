@@ -66,8 +66,15 @@ def gpu_gemm_timing(tt, np, dtype, n, steps, warmup):
 def time_launches(tt, fn, iters, warmup):
     """Average milliseconds per call of fn() (which enqueues GPU work on the default stream), by HIP events."""
     lib = tt._capi.lib
-    for _ in range(warmup):
+    # Warm up for at least `warmup` calls AND ~50 ms of GPU work: the clocks take tens of milliseconds to ramp,
+    # which would otherwise be charged to short kernels.
+    t_end = time.perf_counter() + 0.05
+    n = 0
+    while n < warmup or time.perf_counter() < t_end:
         fn()
+        n += 1
+        if n % 64 == 0:
+            tt.get_backend(tt.kAMD).synchronize(0)
     tt.get_backend(tt.kAMD).synchronize(0)
     e0, e1 = C.c_void_p(), C.c_void_p()
     lib.ttamd_event_create(0, C.byref(e0))

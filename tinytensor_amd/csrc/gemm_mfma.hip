@@ -9,6 +9,8 @@
 // kernel entry, the workgroup -> tile mapping and the host-side operand classification.
 #include "mfma_core.h"
 
+#include <cmath>
+
 namespace ttamd {
 namespace {
 
@@ -206,13 +208,29 @@ ttamd_status launch_mfma_typed(const GemmArgs &g, int device, hipStream_t stream
     OperandClass cb = classify<T>(g.B, g.b_sn, g.b_sk, g.b_sb, g.batch);
     const bool vec = ca.vec > 1 && cb.vec > 1;
 
-    // Tile choice: the biggest tile that still gives the 256 CUs (2 workgroups each) enough workgroups.
-    const int64_t tiles_xl = static_cast<int64_t>((g.M + TS::XBM - 1) / TS::XBM) * ((g.N + TS::XBN - 1) / TS::XBN) * g.batch;
-    const int64_t tiles_large = static_cast<int64_t>((g.M + TS::LBM - 1) / TS::LBM) * ((g.N + TS::LBN - 1) / TS::LBN) * g.batch;
-    const bool xl = TS::kHasXL && vec && tiles_xl >= 384;
-    const bool large = !xl && vec && tiles_large >= 192;
+    // Tile choice by a small cost model fitted to measurements on MI355X (256 CUs): a configuration keeps `per_cu`
+    // workgroups resident per CU and sustains `rate` flop/s when every slot is busy; workgroups are dealt to the
+    // CUs round-robin, so a partial last round costs a whole round as soon as any CU holds a full complement,
+    // and a fraction of it when the CUs are thinly populated (a workgroup alone on a CU runs faster).
+    const double scale = sizeof(T) == 4 ? 1.0 : 0.5;
+    auto estimate = [&](int bm_, int bn_, int per_cu, double rate) {
+        const double tiles = static_cast<double>((g.M + bm_ - 1) / bm_) * ((g.N + bn_ - 1) / bn_) * g.batch;
+        const double slots = 256.0 * per_cu;
+        const double rounds = std::floor(tiles / slots), frac = tiles / slots - rounds;
+        double last = 0.0;
+        if (frac > 0.0) {
+            const double fill = std::ceil(frac * per_cu - 1e-9) / per_cu;  // busiest CU's share of its slots
+            last = fill >= 1.0 ? 1.0 : 0.12 + 0.88 * fill;
+        }
+        const double round_time = 2.0 * bm_ * bn_ * static_cast<double>(g.K) * slots / (rate * scale);
+        return (rounds + last) * round_time;
+    };
+    const double t_small = estimate(TS::SBM, TS::SBN, 4, 119e12);
+    const double t_large = vec ? estimate(TS::LBM, TS::LBN, 2, 133e12) : 1e300;
+    const double t_xl = (TS::kHasXL && vec) ? estimate(TS::XBM, TS::XBN, 2, 141e12) : 1e300;
+    const bool xl = t_xl <= t_large && t_xl <= t_small;
+    const bool large = !xl && t_large <= t_small;
     const int bm = xl ? TS::XBM : (large ? TS::LBM : TS::SBM);
-
     // 32-bit buffer addressing: the bytes reachable from a tile's first row must stay below 2^31.
     const int64_t a_reach = (static_cast<int64_t>(bm - 1) * g.a_sm + static_cast<int64_t>(g.K - 1) * g.a_sk + VK) * sizeof(T);
     const int64_t b_reach = (static_cast<int64_t>(bm - 1) * g.b_sn + static_cast<int64_t>(g.K - 1) * g.b_sk + VK) * sizeof(T);
