@@ -78,6 +78,53 @@ def test_backward_exact_on_integer_data_and_adjoints(tt, oracle, dtype):
     assert lhs == np.sum(gx.to_numpy().astype(np.float64) * x) == np.sum(gw.to_numpy().astype(np.float64) * w)
 
 
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+@pytest.mark.parametrize("geom", [
+    # unit stride with rows that are a whole number of 16-byte vectors: the vector-gather kernels.
+    # B, C, O, H, W, k, P
+    (2, 3, 5, 8, 8, 3, 1),
+    (2, 4, 6, 12, 16, 5, 2),
+    (1, 2, 3, 10, 12, 7, 3),
+    (2, 3, 4, 9, 11, 4, 0),    # Wo = 8 but W = 11: grad_input takes the element-wise gather
+    (1, 2, 3, 8, 8, 9, 4),     # a whole vector left of the row
+    (1, 2, 3, 6, 8, 1, 2),     # padding wider than the kernel
+    (3, 70, 66, 6, 4, 3, 1),   # several channel tiles, one vector per row
+])
+def test_unit_stride_vector_gathers_exact(tt, oracle, dtype, geom):
+    Bn, Cc, O, H, W, k, P = geom
+    rng = np.random.default_rng(sum(geom))
+    x = rng.integers(-3, 4, (Bn, Cc, H, W)).astype(dtype)
+    w = rng.integers(-3, 4, (O, Cc, k, k)).astype(dtype)
+    b = rng.integers(-3, 4, (O,)).astype(dtype)
+    out = tt.conv2d(dev(tt, x), dev(tt, w), dev(tt, b), 1, P).to_numpy()
+    want = oracle.conv2d_forward(x, w, b, 1, P)
+    assert np.array_equal(out, want)
+    assert np.array_equal(want - b[None, :, None, None], oracle.conv2d_naive(x, w, 1, P))
+    g = rng.integers(-3, 4, want.shape).astype(dtype)
+    gx, gw, gb = tt.conv2d_backward(dev(tt, g), dev(tt, x), dev(tt, w), dev(tt, b), 1, P)
+    wx, ww, wb = oracle.conv2d_backward(g, x, w, True, 1, P)
+    assert np.array_equal(gx.to_numpy(), wx) and np.array_equal(gw.to_numpy(), ww) and np.array_equal(gb.to_numpy(), wb)
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+def test_unaligned_window_of_a_larger_image(tt, oracle, dtype):
+    # the input is a window [1:9, 3:15] of a stored [2,3,10,20] tensor: rows start at odd element offsets,
+    # so every 16-byte gather is unaligned, and the elements around the window are non-zero
+    rng = np.random.default_rng(12)
+    store = rng.integers(1, 5, (2, 3, 10, 20)).astype(dtype)
+    x = np.ascontiguousarray(store[:, :, 1:9, 3:15])
+    w = rng.integers(-3, 4, (5, 3, 3, 3)).astype(dtype)
+    ts = dev(tt, store)
+    tx = tt.Tensor(ts.storage, ts.dtype, (2, 3, 8, 12), (600, 200, 20, 1), 23)
+    out = tt.conv2d(tx, dev(tt, w), None, 1, 1).to_numpy()
+    want = oracle.conv2d_forward(x, w, None, 1, 1)
+    assert np.array_equal(out, want)
+    g = rng.integers(-3, 4, want.shape).astype(dtype)
+    gx, gw, _ = tt.conv2d_backward(dev(tt, g), tx, dev(tt, w), None, 1, 1)
+    wx, ww, _ = oracle.conv2d_backward(g, x, w, False, 1, 1)
+    assert np.array_equal(gx.to_numpy(), wx) and np.array_equal(gw.to_numpy(), ww)
+
+
 def test_config4_conv_forward_backward(tt, oracle):
     # BASELINE config 4: input [64,32,28,28], weight [64,32,3,3], stride 1, padding 1, normal(0, 0.1) from a seed.
     x = oracle.Generator(0).normal(0.0, 0.1, (64, 32, 28, 28))

@@ -75,8 +75,10 @@ struct Im2colStager : TileLayout<T, ROWS, BK, false> {
     int32_t base_b;     // byte offset of (ih0, iw0) inside the image (may be negative under padding)
     bool n_ok;
 
-    __device__ __forceinline__ void init(const ConvGeom &geo, const T *image, int64_t image_bytes, int tid, int n0) {
-        g = &geo;
+    __device__ __forceinline__ explicit Im2colStager(const ConvGeom &geo_) : g(&geo_) {}
+
+    __device__ __forceinline__ void init(const T *image, int64_t image_bytes, int tid, int n0) {
+        const ConvGeom &geo = *g;
         rsrc = make_rsrc(image, image_bytes);
         n_local = tid % ROWS;
         line0 = __builtin_amdgcn_readfirstlane(tid / ROWS);
@@ -135,8 +137,10 @@ struct Im2colTStager : TileLayout<T, ROWS, BK, true> {
     bool j_ok[P];
     int k_local, row0, k_next, HoWo;
 
-    __device__ __forceinline__ void init(const ConvGeom &geo, int tid, int j0) {
-        g = &geo;
+    __device__ __forceinline__ explicit Im2colTStager(const ConvGeom &geo_) : g(&geo_) {}
+
+    __device__ __forceinline__ void init(int tid, int j0) {
+        const ConvGeom &geo = *g;
         k_local = tid % BK;
         row0 = tid / BK;
         HoWo = geo.Ho * geo.Wo;
@@ -187,54 +191,6 @@ struct Im2colTStager : TileLayout<T, ROWS, BK, true> {
 };
 
 // ---------------------------------------------------------------------------------------------
-// A operand of grad_input: Wt[c][kk] = W[o][c][p][q] with kk = (o,p,q).  KC layout, one element per load;
-// a lane keeps one kk per tile (decoded per tile), the channel row varies per pass.
-template <typename T, int ROWS, int BK, int PF = 1>
-struct WeightTStager : TileLayout<T, ROWS, BK, true> {
-    using L = TileLayout<T, ROWS, BK, true>;
-    static constexpr int RPP = kThreads / BK;
-    static constexpr int P = ROWS / RPP;
-    static constexpr int kPF = PF;
-    T reg[PF][P];
-    __amdgpu_buffer_rsrc_t rsrc;
-    const ConvGeom *g;
-    int k_local, row0, k_next, K, c0, kk2;
-
-    __device__ __forceinline__ void init(const ConvGeom &geo, const T *weight, int64_t weight_bytes, int tid, int c0_) {
-        g = &geo;
-        rsrc = make_rsrc(weight, weight_bytes);
-        k_local = tid % BK;
-        row0 = tid / BK;
-        k_next = 0;
-        kk2 = geo.k * geo.k;
-        K = geo.O * kk2;
-        c0 = c0_;
-    }
-
-    template <bool MASK, int SLOT = 0>
-    __device__ __forceinline__ void load(int /*k_left*/) {
-        const int kk = k_next + k_local;
-        const bool k_ok = kk < K;
-        uint32_t o, r;
-        g->d_kk.divmod(static_cast<uint32_t>(k_ok ? kk : 0), o, r);
-        const int64_t koff = static_cast<int64_t>(o) * g->w_so + r;  // elements
-#pragma unroll
-        for (int p = 0; p < P; ++p) {
-            const int c = c0 + p * RPP + row0;
-            const bool ok = k_ok && c < g->C;
-            const int64_t off = (koff + static_cast<int64_t>(c) * kk2) * static_cast<int64_t>(sizeof(T));
-            reg[SLOT][p] = Vec<T, 1>::load(rsrc, ok ? static_cast<uint32_t>(off) : kOob);
-        }
-        k_next += BK;
-    }
-
-    template <int SLOT = 0>
-    __device__ __forceinline__ void store(T *lds) const {
-#pragma unroll
-        for (int p = 0; p < P; ++p) lds[(p * RPP + row0) * L::LD + k_local] = reg[SLOT][p];
-    }
-};
-
 // B operand of grad_input: G[kk][n] = g[b][o][(y+P-p)/S][(x+P-q)/S], kk = (o,p,q), n = (y,x).  MC layout;
 // the lane's input position is fixed, kk is wave-uniform per pass.
 template <typename T, int ROWS, int BK, int PF = 1>
@@ -251,8 +207,10 @@ struct DgradStager : TileLayout<T, ROWS, BK, false> {
     int yP, xP;  // y + P, x + P for this lane's input position
     bool n_ok;
 
-    __device__ __forceinline__ void init(const ConvGeom &geo, const T *gout_image, int64_t bytes, int tid, int n0) {
-        g = &geo;
+    __device__ __forceinline__ explicit DgradStager(const ConvGeom &geo_) : g(&geo_) {}
+
+    __device__ __forceinline__ void init(const T *gout_image, int64_t bytes, int tid, int n0) {
+        const ConvGeom &geo = *g;
         rsrc = make_rsrc(gout_image, bytes);
         n_local = tid % ROWS;
         line0 = __builtin_amdgcn_readfirstlane(tid / ROWS);
@@ -296,12 +254,199 @@ struct DgradStager : TileLayout<T, ROWS, BK, false> {
 };
 
 // ---------------------------------------------------------------------------------------------
-// forward: M = O, N = Ho*Wo, K = C*k*k, one GEMM per image.
-template <typename T, int BM, int BN, int BK, int A_VEC>
+// Vector gathers for unit stride.  With S = 1 and a unit column stride, VEC consecutive positions of one
+// plane row read VEC consecutive source elements src[ch][py + dy][px0 + dx .. + VEC - 1], so one 16-byte
+// buffer load (any 4-byte alignment) fetches them; components that fall left or right of the row are
+// cleared afterwards (the load itself stays inside the image: the descriptor checks its range per dword,
+// and a vector that would begin before the image's first element is fetched element by element instead).
+//
+//   FLIP = false: taps (c, a, b) of the input image, positions = output pixels, dy = a - P  (forward, grad_weight)
+//   FLIP = true:  taps (o, a, b) of grad_out,        positions = input pixels,  dy = P - a  (grad_input)
+template <bool FLIP>
+struct TapView {
+    int taps, positions, src_h, src_w, k, pad;
+    int32_t s_ch, s_h;
+    FastDiv d_kk, d_k, d_pw;
+    __device__ __forceinline__ explicit TapView(const ConvGeom &g) {
+        k = g.k;
+        pad = g.P;
+        d_kk = g.d_kk;
+        d_k = g.d_k;
+        if constexpr (FLIP) {
+            taps = g.O * g.k * g.k;
+            positions = g.H * g.W;
+            src_h = g.Ho;
+            src_w = g.Wo;
+            s_ch = g.Ho * g.Wo;
+            s_h = g.Wo;
+            d_pw = g.d_W;
+        } else {
+            taps = g.C * g.k * g.k;
+            positions = g.Ho * g.Wo;
+            src_h = g.H;
+            src_w = g.W;
+            s_ch = g.xs_c;
+            s_h = g.xs_h;
+            d_pw = g.d_Wo;
+        }
+    }
+    // (channel offset, dy, dx) of tap index t
+    __device__ __forceinline__ void tap(uint32_t t, int32_t &ch_off, int &dy, int &dx) const {
+        uint32_t ch, r, a, b;
+        d_kk.divmod(t, ch, r);
+        d_k.divmod(r, a, b);
+        ch_off = static_cast<int32_t>(ch) * s_ch;
+        dy = FLIP ? pad - static_cast<int>(a) : static_cast<int>(a) - pad;
+        dx = FLIP ? pad - static_cast<int>(b) : static_cast<int>(b) - pad;
+    }
+};
+
+// One gathered vector: elements e0 .. e0 + VEC - 1 of the image, columns x0 .. x0 + VEC - 1 of a row of width src_w.
+template <typename T, int VEC>
+__device__ __forceinline__ typename Vec<T, VEC>::type gather_row_vector(__amdgpu_buffer_rsrc_t rsrc, bool row_ok, int32_t e0,
+                                                                        int x0, int src_w) {
+    using V = typename Vec<T, VEC>::type;
+    constexpr int32_t SZ = static_cast<int32_t>(sizeof(T));
+    V v = Vec<T, VEC>::load(rsrc, (row_ok && e0 >= 0) ? static_cast<uint32_t>(e0 * SZ) : kOob);
+    if (row_ok && e0 < 0) {  // top-left corner of the first plane under padding
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) v[j] = Vec<T, 1>::load(rsrc, e0 + j >= 0 ? static_cast<uint32_t>((e0 + j) * SZ) : kOob);
+    }
+#pragma unroll
+    for (int j = 0; j < VEC; ++j)
+        if (static_cast<unsigned>(x0 + j) >= static_cast<unsigned>(src_w)) v[j] = T(0);
+    return v;
+}
+
+// MC layout (positions contiguous in LDS), vectors along the positions: B operand of forward and of
+// grad_input.  Requires positions-per-row % VEC == 0 so that a vector never crosses a plane row.
+template <typename T, int ROWS, int BK, int VEC, bool FLIP, int PF = 1>
+struct TapStagerMC : TileLayout<T, ROWS, BK, false> {
+    using L = TileLayout<T, ROWS, BK, false>;
+    using V = typename Vec<T, VEC>::type;
+    static constexpr int VPL = ROWS / VEC;       // vectors per k line
+    static constexpr int LPP = kThreads / VPL;   // k lines per pass
+    static constexpr int P = BK / LPP;
+    static_assert(VEC > 1 && ROWS % VEC == 0 && kThreads % VPL == 0 && BK % LPP == 0, "tile must split evenly");
+    static constexpr int kPF = PF;
+    V reg[PF][P];
+    __amdgpu_buffer_rsrc_t rsrc;
+    TapView<FLIP> tv;
+    int n_local, line0, k_next;
+    int py, px0;
+    bool n_ok;
+
+    __device__ __forceinline__ explicit TapStagerMC(const ConvGeom &geo) : tv(geo) {}
+
+    __device__ __forceinline__ void init(const T *image, int64_t image_bytes, int tid, int n0) {
+        rsrc = make_rsrc(image, image_bytes);
+        n_local = (tid % VPL) * VEC;
+        line0 = tid / VPL;
+        k_next = 0;
+        const int n = n0 + n_local;
+        n_ok = n < tv.positions;
+        uint32_t y, x;
+        tv.d_pw.divmod(static_cast<uint32_t>(n_ok ? n : 0), y, x);
+        py = static_cast<int>(y);
+        px0 = static_cast<int>(x);
+    }
+
+    template <bool MASK, int SLOT = 0>
+    __device__ __forceinline__ void load(int /*k_left*/) {
+#pragma unroll
+        for (int p = 0; p < P; ++p) {
+            const int kk = k_next + p * LPP + line0;
+            const bool k_ok = kk < tv.taps;
+            int32_t ch_off;
+            int dy, dx;
+            tv.tap(static_cast<uint32_t>(k_ok ? kk : 0), ch_off, dy, dx);
+            const int y = py + dy, x0 = px0 + dx;
+            const bool row_ok = n_ok && k_ok && static_cast<unsigned>(y) < static_cast<unsigned>(tv.src_h);
+            reg[SLOT][p] = gather_row_vector<T, VEC>(rsrc, row_ok, ch_off + y * tv.s_h + x0, x0, tv.src_w);
+        }
+        k_next += BK;
+    }
+
+    template <int SLOT = 0>
+    __device__ __forceinline__ void store(T *lds) const {
+#pragma unroll
+        for (int p = 0; p < P; ++p) *reinterpret_cast<V *>(&lds[(p * LPP + line0) * L::LD + n_local]) = reg[SLOT][p];
+    }
+};
+
+// KC layout (reduction index contiguous in LDS), vectors along the positions, which are the reduction
+// index here: B operand of grad_weight.  The tap of each pass is fixed for the whole kernel.
+template <typename T, int ROWS, int BK, int VEC, int PF = 1>
+struct TapStagerKC : TileLayout<T, ROWS, BK, true> {
+    using L = TileLayout<T, ROWS, BK, true>;
+    using V = typename Vec<T, VEC>::type;
+    static constexpr int VPL = BK / VEC;
+    static constexpr int RPP = kThreads / VPL;  // tap rows per pass
+    static constexpr int P = ROWS / RPP;
+    static_assert(VEC > 1 && BK % VEC == 0 && kThreads % VPL == 0 && ROWS % RPP == 0, "tile must split evenly");
+    static constexpr int kPF = PF;
+    V reg[PF][P];
+    __amdgpu_buffer_rsrc_t rsrc;
+    TapView<false> tv;
+    int32_t joff[P];
+    int16_t dy[P], dx[P];
+    bool j_ok[P];
+    int k_local, row0, k_next;
+
+    __device__ __forceinline__ explicit TapStagerKC(const ConvGeom &geo) : tv(geo) {}
+
+    __device__ __forceinline__ void init(int tid, int j0) {
+        k_local = (tid % VPL) * VEC;
+        row0 = tid / VPL;
+#pragma unroll
+        for (int p = 0; p < P; ++p) {
+            const int j = j0 + p * RPP + row0;
+            j_ok[p] = j < tv.taps;
+            int32_t ch_off;
+            int ddy, ddx;
+            tv.tap(static_cast<uint32_t>(j_ok[p] ? j : 0), ch_off, ddy, ddx);
+            dy[p] = static_cast<int16_t>(ddy);
+            dx[p] = static_cast<int16_t>(ddx);
+            joff[p] = ch_off + ddy * tv.s_h + ddx;
+        }
+    }
+
+    __device__ __forceinline__ void set_image(const T *image, int64_t image_bytes) {
+        rsrc = make_rsrc(image, image_bytes);
+        k_next = 0;
+    }
+
+    template <bool MASK, int SLOT = 0>
+    __device__ __forceinline__ void load(int /*k_left*/) {
+        const int n = k_next + k_local;
+        const bool n_ok = n < tv.positions;
+        uint32_t y, x;
+        tv.d_pw.divmod(static_cast<uint32_t>(n_ok ? n : 0), y, x);
+        const int py = static_cast<int>(y), px0 = static_cast<int>(x);
+        const int32_t base = py * tv.s_h + px0;
+#pragma unroll
+        for (int p = 0; p < P; ++p) {
+            const int yy = py + dy[p], x0 = px0 + dx[p];
+            const bool row_ok = n_ok && j_ok[p] && static_cast<unsigned>(yy) < static_cast<unsigned>(tv.src_h);
+            reg[SLOT][p] = gather_row_vector<T, VEC>(rsrc, row_ok, base + joff[p], x0, tv.src_w);
+        }
+        k_next += BK;
+    }
+
+    template <int SLOT = 0>
+    __device__ __forceinline__ void store(T *lds) const {
+#pragma unroll
+        for (int p = 0; p < P; ++p) *reinterpret_cast<V *>(&lds[(p * RPP + row0) * L::LD + k_local]) = reg[SLOT][p];
+    }
+};
+
+// ---------------------------------------------------------------------------------------------
+// forward: M = O, N = Ho*Wo, K = C*k*k, one GEMM per image.  StB gathers the image.
+template <typename T, int BK, int A_VEC, class StB>
 __global__ void __launch_bounds__(kThreads, 2)
 conv_fwd_kernel(ConvGeom geo, const T *x, const T *w, const T *bias, T *out, int64_t image_bytes, int tiles_m, int tiles_n) {
+    constexpr int BM = 64, BN = 64;
     using StA = Stager<T, BM, BK, true, A_VEC>;
-    using StB = Im2colStager<T, BN, BK>;
     using Engine = TileEngine<T, BM, BN, BK, 2, 2, StA, StB>;
     extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
     T *const smem = reinterpret_cast<T *>(smem_raw);
@@ -311,21 +456,35 @@ conv_fwd_kernel(ConvGeom geo, const T *x, const T *w, const T *bias, T *out, int
     const int m0 = tm * BM, n0 = tn * BN;
     const int M_ = geo.O, N_ = geo.Ho * geo.Wo, K = geo.C * geo.k * geo.k;
     StA sa;
-    StB sb;
+    StB sb(geo);
     sa.init(w + static_cast<int64_t>(m0) * geo.w_so, tid, M_ - m0, geo.w_so, 1, K);
-    sb.init(geo, x + static_cast<int64_t>(b) * geo.xs_b, image_bytes, tid, n0);
+    sb.init(x + static_cast<int64_t>(b) * geo.xs_b, image_bytes, tid, n0);
     Engine eng;
     eng.init(tid);
     eng.run(sa, sb, smem, K, false);
     store_tile_dense<T>(eng, out + static_cast<int64_t>(b) * M_ * N_, M_, N_, m0, n0, bias, bias ? 2 : 0, 0, 0);
 }
 
-// grad_input: M = C, N = H*W, K = O*k*k, one GEMM per image.
-template <typename T, int BM, int BN, int BK>
+// wt[c][(o, a, b)] = w[o][c][a][b]: the A operand of grad_input with its reduction index contiguous.
+template <typename T>
+__global__ void __launch_bounds__(256) weight_transpose_kernel(ConvGeom geo, const T *__restrict__ w, T *__restrict__ wt, int total) {
+    const int idx = blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= total) return;
+    const uint32_t k2 = static_cast<uint32_t>(geo.k * geo.k);
+    const uint32_t row = k2 * static_cast<uint32_t>(geo.O);
+    const uint32_t c = static_cast<uint32_t>(idx) / row, rem = static_cast<uint32_t>(idx) - c * row;
+    uint32_t o, r;
+    geo.d_kk.divmod(rem, o, r);
+    wt[idx] = w[static_cast<int64_t>(o) * geo.w_so + c * k2 + r];
+}
+
+// grad_input: M = C, N = H*W, K = O*k*k, one GEMM per image.  wt is the transposed weight [C, O*k*k];
+// StB gathers grad_out.
+template <typename T, int BK, int A_VEC, class StB>
 __global__ void __launch_bounds__(kThreads, 2)
-conv_dgrad_kernel(ConvGeom geo, const T *gout, const T *w, T *gin, int64_t weight_bytes, int tiles_m, int tiles_n) {
-    using StA = WeightTStager<T, BM, BK>;
-    using StB = DgradStager<T, BN, BK>;
+conv_dgrad_kernel(ConvGeom geo, const T *gout, const T *wt, T *gin, int tiles_m, int tiles_n) {
+    constexpr int BM = 64, BN = 64;
+    using StA = Stager<T, BM, BK, true, A_VEC>;
     using Engine = TileEngine<T, BM, BN, BK, 2, 2, StA, StB>;
     extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
     T *const smem = reinterpret_cast<T *>(smem_raw);
@@ -336,9 +495,9 @@ conv_dgrad_kernel(ConvGeom geo, const T *gout, const T *w, T *gin, int64_t weigh
     const int M_ = geo.C, N_ = geo.H * geo.W, K = geo.O * geo.k * geo.k;
     const int64_t g_image = static_cast<int64_t>(geo.O) * geo.Ho * geo.Wo;
     StA sa;
-    StB sb;
-    sa.init(geo, w, weight_bytes, tid, m0);
-    sb.init(geo, gout + static_cast<int64_t>(b) * g_image, g_image * static_cast<int64_t>(sizeof(T)), tid, n0);
+    StB sb(geo);
+    sa.init(wt + static_cast<int64_t>(m0) * K, tid, M_ - m0, K, 1, K);
+    sb.init(gout + static_cast<int64_t>(b) * g_image, g_image * static_cast<int64_t>(sizeof(T)), tid, n0);
     Engine eng;
     eng.init(tid);
     eng.run(sa, sb, smem, K, false);
@@ -347,11 +506,11 @@ conv_dgrad_kernel(ConvGeom geo, const T *gout, const T *w, T *gin, int64_t weigh
 
 // grad_weight: M = O, N = C*k*k, K = Ho*Wo per image; workgroup column `split` accumulates images
 // [split*group, min(B, (split+1)*group)) in registers and writes one partial tile.
-template <typename T, int BM, int BN, int BK, int A_VEC>
+template <typename T, int BK, int A_VEC, class StB>
 __global__ void __launch_bounds__(kThreads, 2)
 conv_wgrad_kernel(ConvGeom geo, const T *gout, const T *x, T *partial, int64_t image_bytes, int group, int tiles_m, int tiles_n) {
+    constexpr int BM = 64, BN = 64;
     using StA = Stager<T, BM, BK, true, A_VEC>;
-    using StB = Im2colTStager<T, BN, BK>;
     using Engine = TileEngine<T, BM, BN, BK, 2, 2, StA, StB>;
     extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
     T *const smem = reinterpret_cast<T *>(smem_raw);
@@ -362,8 +521,8 @@ conv_wgrad_kernel(ConvGeom geo, const T *gout, const T *x, T *partial, int64_t i
     const int M_ = geo.O, N_ = geo.C * geo.k * geo.k, K = geo.Ho * geo.Wo;
     const int64_t g_image = static_cast<int64_t>(geo.O) * K;
     StA sa;
-    StB sb;
-    sb.init(geo, tid, n0);
+    StB sb(geo);
+    sb.init(tid, n0);
     Engine eng;
     eng.init(tid);
     const int b_end = (split + 1) * group < geo.B ? (split + 1) * group : geo.B;
@@ -531,6 +690,25 @@ bool rows_vectorizable(const void *ptr, int64_t row_stride, int64_t image_stride
     return reinterpret_cast<uintptr_t>(ptr) % 16 == 0 && row_stride % VK == 0 && image_stride % VK == 0;
 }
 
+template <class Kernel>
+ttamd_status launch_conv(Kernel kernel, size_t lds, int64_t blocks, hipStream_t st, auto... args) {
+    if (blocks > 0x7fffffff) {
+        set_error("conv2d: too many workgroups");
+        return TTAMD_ERR_INVALID_ARGUMENT;
+    }
+    if (ttamd_status s = set_lds(kernel, lds)) return s;
+    kernel<<<dim3(static_cast<unsigned>(blocks)), dim3(kThreads), lds, st>>>(args...);
+    TTAMD_HIP_CHECK(hipGetLastError());
+    return TTAMD_OK;
+}
+
+// LDS bytes of the 64x64 engine built from the weight/grad_out stager and gather stager StB.
+template <typename T, int A_VEC, class StB>
+constexpr size_t conv_lds_bytes() {
+    constexpr int BK = ConvTiles<T>::BK;
+    return TileEngine<T, 64, 64, BK, 2, 2, Stager<T, 64, BK, true, A_VEC>, StB>::kLdsBytes;
+}
+
 template <typename T>
 ttamd_status forward_mfma(const ConvPlan &pl, const void *bias, void *out, hipStream_t st) {
     constexpr int BK = ConvTiles<T>::BK, VK = Mfma<T>::VK;
@@ -538,25 +716,18 @@ ttamd_status forward_mfma(const ConvPlan &pl, const void *bias, void *out, hipSt
     const int M_ = g.O, N_ = g.Ho * g.Wo;
     const int tiles_m = (M_ + 63) / 64, tiles_n = (N_ + 63) / 64;
     const int64_t blocks = static_cast<int64_t>(tiles_m) * tiles_n * g.B;
-    if (blocks > 0x7fffffff) {
-        set_error("conv2d: too many workgroups");
-        return TTAMD_ERR_INVALID_ARGUMENT;
-    }
-    const bool vec = rows_vectorizable<T>(pl.w, g.w_so, 0);
-    auto launch = [&](auto kernel, size_t lds) -> ttamd_status {
-        if (ttamd_status s = set_lds(kernel, lds)) return s;
-        kernel<<<dim3(static_cast<unsigned>(blocks)), dim3(kThreads), lds, st>>>(
-            g, static_cast<const T *>(pl.x), static_cast<const T *>(pl.w), static_cast<const T *>(bias), static_cast<T *>(out),
-            pl.image_bytes, tiles_m, tiles_n);
-        TTAMD_HIP_CHECK(hipGetLastError());
-        return TTAMD_OK;
+    const bool a_vec = rows_vectorizable<T>(pl.w, g.w_so, 0);
+    const bool b_vec = g.S == 1 && g.xs_w == 1 && g.Wo % VK == 0;
+    auto go = [&](auto kernel, size_t lds) {
+        return launch_conv(kernel, lds, blocks, st, g, static_cast<const T *>(pl.x), static_cast<const T *>(pl.w),
+                           static_cast<const T *>(bias), static_cast<T *>(out), pl.image_bytes, tiles_m, tiles_n);
     };
-    if (vec) {
-        using E = TileEngine<T, 64, 64, BK, 2, 2, Stager<T, 64, BK, true, VK>, Im2colStager<T, 64, BK>>;
-        return launch(conv_fwd_kernel<T, 64, 64, BK, VK>, E::kLdsBytes);
-    }
-    using E = TileEngine<T, 64, 64, BK, 2, 2, Stager<T, 64, BK, true, 1>, Im2colStager<T, 64, BK>>;
-    return launch(conv_fwd_kernel<T, 64, 64, BK, 1>, E::kLdsBytes);
+    using VecB = TapStagerMC<T, 64, BK, VK, false>;
+    using OneB = Im2colStager<T, 64, BK>;
+    if (a_vec && b_vec) return go(conv_fwd_kernel<T, BK, VK, VecB>, conv_lds_bytes<T, VK, VecB>());
+    if (a_vec) return go(conv_fwd_kernel<T, BK, VK, OneB>, conv_lds_bytes<T, VK, OneB>());
+    if (b_vec) return go(conv_fwd_kernel<T, BK, 1, VecB>, conv_lds_bytes<T, 1, VecB>());
+    return go(conv_fwd_kernel<T, BK, 1, OneB>, conv_lds_bytes<T, 1, OneB>());
 }
 
 template <typename T, typename Acc>
@@ -584,63 +755,85 @@ int wgrad_group(size_t esz, int B, int C, int O, int k) {
     return static_cast<int>((B + max_splits - 1) / max_splits);
 }
 
+// Workspace layout of conv2d_backward: the transposed weight [C, O*k*k] (rounded up to 256 bytes), then, when
+// grad_weight is split over the batch, `splits` partial [O, C*k*k] tiles.
+struct BackwardWorkspace {
+    size_t wt_bytes, partial_bytes;
+    int group, splits;
+    size_t total() const { return wt_bytes + partial_bytes; }
+};
+
+BackwardWorkspace backward_workspace(size_t esz, int B, int C, int O, int k) {
+    BackwardWorkspace w{};
+    const size_t tile = static_cast<size_t>(O) * C * k * k * esz;
+    w.wt_bytes = (tile + 255) & ~static_cast<size_t>(255);
+    w.group = wgrad_group(esz, B, C, O, k);
+    w.splits = (B + w.group - 1) / w.group;
+    w.partial_bytes = w.splits > 1 ? static_cast<size_t>(w.splits) * tile : 0;
+    return w;
+}
+
 template <typename T>
 ttamd_status backward_mfma(const ConvPlan &pl, const void *gout, void *gin, void *gw, void *gb, void *ws, size_t ws_bytes,
                            hipStream_t st) {
     constexpr int BK = ConvTiles<T>::BK, VK = Mfma<T>::VK;
     const ConvGeom &g = pl.geo;
     const int HoWo = g.Ho * g.Wo;
+    const BackwardWorkspace plan = backward_workspace(sizeof(T), g.B, g.C, g.O, g.k);
+    if (!ws || ws_bytes < plan.total()) {
+        set_error("conv2d_backward: workspace of %zu bytes is smaller than the %zu bytes required", ws_bytes, plan.total());
+        return TTAMD_ERR_INVALID_ARGUMENT;
+    }
+    T *const wt = static_cast<T *>(ws);
+    T *const partials = reinterpret_cast<T *>(static_cast<char *>(ws) + plan.wt_bytes);
     // grad_input
     {
+        const int Kd = g.O * g.k * g.k;
+        const int total = g.C * Kd;
+        weight_transpose_kernel<T><<<dim3((total + 255) / 256), dim3(256), 0, st>>>(g, static_cast<const T *>(pl.w), wt, total);
+        TTAMD_HIP_CHECK(hipGetLastError());
         const int M_ = g.C, N_ = g.H * g.W;
         const int tiles_m = (M_ + 63) / 64, tiles_n = (N_ + 63) / 64;
         const int64_t blocks = static_cast<int64_t>(tiles_m) * tiles_n * g.B;
-        if (blocks > 0x7fffffff) {
-            set_error("conv2d_backward: too many workgroups");
-            return TTAMD_ERR_INVALID_ARGUMENT;
-        }
-        using E = TileEngine<T, 64, 64, BK, 2, 2, WeightTStager<T, 64, BK>, DgradStager<T, 64, BK>>;
-        auto kernel = conv_dgrad_kernel<T, 64, 64, BK>;
-        if (ttamd_status s = set_lds(kernel, E::kLdsBytes)) return s;
-        kernel<<<dim3(static_cast<unsigned>(blocks)), dim3(kThreads), E::kLdsBytes, st>>>(
-            g, static_cast<const T *>(gout), static_cast<const T *>(pl.w), static_cast<T *>(gin), pl.weight_bytes, tiles_m, tiles_n);
-        TTAMD_HIP_CHECK(hipGetLastError());
+        const bool a_vec = rows_vectorizable<T>(wt, Kd, 0);
+        const bool b_vec = g.S == 1 && g.W % VK == 0;
+        auto go = [&](auto kernel, size_t lds) {
+            return launch_conv(kernel, lds, blocks, st, g, static_cast<const T *>(gout), static_cast<const T *>(wt),
+                               static_cast<T *>(gin), tiles_m, tiles_n);
+        };
+        using VecB = TapStagerMC<T, 64, BK, VK, true>;
+        using OneB = DgradStager<T, 64, BK>;
+        ttamd_status s;
+        if (a_vec && b_vec) s = go(conv_dgrad_kernel<T, BK, VK, VecB>, conv_lds_bytes<T, VK, VecB>());
+        else if (a_vec) s = go(conv_dgrad_kernel<T, BK, VK, OneB>, conv_lds_bytes<T, VK, OneB>());
+        else if (b_vec) s = go(conv_dgrad_kernel<T, BK, 1, VecB>, conv_lds_bytes<T, 1, VecB>());
+        else s = go(conv_dgrad_kernel<T, BK, 1, OneB>, conv_lds_bytes<T, 1, OneB>());
+        if (s) return s;
     }
     // grad_weight
     {
         const int M_ = g.O, N_ = g.C * g.k * g.k;
-        const int group = wgrad_group(sizeof(T), g.B, g.C, g.O, g.k);
-        const int splits = (g.B + group - 1) / group;
         const int64_t tile_elems = static_cast<int64_t>(M_) * N_;
-        T *partial = static_cast<T *>(gw);
-        if (splits > 1) {
-            if (!ws || ws_bytes < static_cast<size_t>(splits) * tile_elems * sizeof(T)) {
-                set_error("conv2d_backward: workspace of %zu bytes is smaller than the %zu bytes required", ws_bytes,
-                          static_cast<size_t>(splits) * tile_elems * sizeof(T));
-                return TTAMD_ERR_INVALID_ARGUMENT;
-            }
-            partial = static_cast<T *>(ws);
-        }
+        T *const partial = plan.splits > 1 ? partials : static_cast<T *>(gw);
         const int tiles_m = (M_ + 63) / 64, tiles_n = (N_ + 63) / 64;
-        const int64_t blocks = static_cast<int64_t>(tiles_m) * tiles_n * splits;
-        const bool vec = rows_vectorizable<T>(gout, HoWo, static_cast<int64_t>(g.O) * HoWo);
-        auto launch = [&](auto kernel, size_t lds) -> ttamd_status {
-            if (ttamd_status s = set_lds(kernel, lds)) return s;
-            kernel<<<dim3(static_cast<unsigned>(blocks)), dim3(kThreads), lds, st>>>(
-                g, static_cast<const T *>(gout), static_cast<const T *>(pl.x), partial, pl.image_bytes, group, tiles_m, tiles_n);
-            TTAMD_HIP_CHECK(hipGetLastError());
-            return TTAMD_OK;
+        const int64_t blocks = static_cast<int64_t>(tiles_m) * tiles_n * plan.splits;
+        const bool a_vec = rows_vectorizable<T>(gout, HoWo, static_cast<int64_t>(g.O) * HoWo);
+        const bool b_vec = g.S == 1 && g.xs_w == 1 && g.Wo % VK == 0;
+        auto go = [&](auto kernel, size_t lds) {
+            return launch_conv(kernel, lds, blocks, st, g, static_cast<const T *>(gout), static_cast<const T *>(pl.x),
+                               partial, pl.image_bytes, plan.group, tiles_m, tiles_n);
         };
-        if (vec) {
-            using E = TileEngine<T, 64, 64, BK, 2, 2, Stager<T, 64, BK, true, VK>, Im2colTStager<T, 64, BK>>;
-            if (ttamd_status s = launch(conv_wgrad_kernel<T, 64, 64, BK, VK>, E::kLdsBytes)) return s;
-        } else {
-            using E = TileEngine<T, 64, 64, BK, 2, 2, Stager<T, 64, BK, true, 1>, Im2colTStager<T, 64, BK>>;
-            if (ttamd_status s = launch(conv_wgrad_kernel<T, 64, 64, BK, 1>, E::kLdsBytes)) return s;
-        }
-        if (splits > 1) {
+        using VecB = TapStagerKC<T, 64, BK, VK>;
+        using OneB = Im2colTStager<T, 64, BK>;
+        ttamd_status s;
+        if (a_vec && b_vec) s = go(conv_wgrad_kernel<T, BK, VK, VecB>, conv_lds_bytes<T, VK, VecB>());
+        else if (a_vec) s = go(conv_wgrad_kernel<T, BK, VK, OneB>, conv_lds_bytes<T, VK, OneB>());
+        else if (b_vec) s = go(conv_wgrad_kernel<T, BK, 1, VecB>, conv_lds_bytes<T, 1, VecB>());
+        else s = go(conv_wgrad_kernel<T, BK, 1, OneB>, conv_lds_bytes<T, 1, OneB>());
+        if (s) return s;
+        if (plan.splits > 1) {
             const int64_t rb = (tile_elems + 255) / 256;
-            reduce_splits_kernel<T><<<dim3(static_cast<unsigned>(rb)), dim3(256), 0, st>>>(partial, static_cast<T *>(gw), tile_elems, splits);
+            reduce_splits_kernel<T><<<dim3(static_cast<unsigned>(rb)), dim3(256), 0, st>>>(partial, static_cast<T *>(gw), tile_elems, plan.splits);
             TTAMD_HIP_CHECK(hipGetLastError());
         }
     }
@@ -696,10 +889,7 @@ ttamd_status ttamd_conv2d_backward_workspace(ttamd_dtype dtype, int B, int C, in
         return TTAMD_ERR_UNSUPPORTED_DTYPE;
     }
     if (B <= 0 || C <= 0 || O <= 0 || k <= 0) return TTAMD_OK;
-    const size_t esz = dtype_size(dtype);
-    const int group = wgrad_group(esz, B, C, O, k);
-    const int splits = (B + group - 1) / group;
-    if (splits > 1) *bytes = static_cast<size_t>(splits) * O * C * k * k * esz;
+    *bytes = backward_workspace(dtype_size(dtype), B, C, O, k).total();
     return TTAMD_OK;
 }
 
