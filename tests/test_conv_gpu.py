@@ -39,6 +39,9 @@ def test_forward_reference_pattern_exact(tt, oracle, dtype, S, P):
     (1, 8, 16, 17, 19, 3, 3, 1),
     (2, 2, 3, 6, 7, 2, 2, 0),
     (2, 16, 64, 12, 12, 3, 1, 1),
+    (1, 3, 5, 40, 36, 3, 1, 1),    # long reduction per image: grad_weight in several position slices
+    (2, 3, 5, 41, 37, 3, 2, 1),    # the same with element-wise gathers
+    (2, 40, 48, 10, 12, 3, 1, 1),  # 64x64 tiles with ragged rows in every product
 ])
 def test_forward_backward_random(tt, oracle, dtype, geom):
     Bn, Cc, O, H, W, k, S, P = geom

@@ -13,9 +13,9 @@
 //
 // grad_input is the gather form of the reference's col2im scatter-add (conv.hpp:83-118): every output
 // element is owned by one lane, so there is no write race and the result is deterministic.
-// grad_weight reduces over the batch: one workgroup column per group of images accumulates in registers,
-// partial tiles go to the caller's workspace and are summed in image order (the reference's order,
-// conv.cpp:239-244).  Integer dtypes (forward only; autograd never differentiates them) use a direct
+// grad_weight reduces over the batch (conv.cpp:239-244): one workgroup column per (group of images, slice of
+// output positions) accumulates in registers, partial tiles go to the caller's workspace and are summed in a
+// fixed order.  Integer dtypes (forward only; autograd never differentiates them) use a direct
 // vector-ALU kernel with wrap-around arithmetic.
 #include "mfma_core.h"
 
@@ -159,10 +159,10 @@ struct Im2colTStager : TileLayout<T, ROWS, BK, true> {
         }
     }
 
-    // Points the stager at image `image` and restarts the reduction index.
-    __device__ __forceinline__ void set_image(const T *image, int64_t image_bytes) {
+    // Points the stager at image `image` and restarts the reduction index at k0.
+    __device__ __forceinline__ void set_image(const T *image, int64_t image_bytes, int k0) {
         rsrc = make_rsrc(image, image_bytes);
-        k_next = 0;
+        k_next = k0;
     }
 
     template <bool MASK, int SLOT = 0>
@@ -411,9 +411,9 @@ struct TapStagerKC : TileLayout<T, ROWS, BK, true> {
         }
     }
 
-    __device__ __forceinline__ void set_image(const T *image, int64_t image_bytes) {
+    __device__ __forceinline__ void set_image(const T *image, int64_t image_bytes, int k0) {
         rsrc = make_rsrc(image, image_bytes);
-        k_next = 0;
+        k_next = k0;
     }
 
     template <bool MASK, int SLOT = 0>
@@ -441,13 +441,17 @@ struct TapStagerKC : TileLayout<T, ROWS, BK, true> {
 };
 
 // ---------------------------------------------------------------------------------------------
+// Tile shapes: 64x64 (2x2 waves) or, for products with at most 32 rows, 32x128 (1x4 waves): every wave owns a
+// 32x32 block either way.
+template <typename T, int BM, int BN, int BK, class StA, class StB>
+using ConvEngine = TileEngine<T, BM, BN, BK, BM == 32 ? 1 : 2, BM == 32 ? 4 : 2, StA, StB>;
+
 // forward: M = O, N = Ho*Wo, K = C*k*k, one GEMM per image.  StB gathers the image.
-template <typename T, int BK, int A_VEC, class StB>
+template <typename T, int BM, int BN, int BK, int A_VEC, class StB>
 __global__ void __launch_bounds__(kThreads, 2)
 conv_fwd_kernel(ConvGeom geo, const T *x, const T *w, const T *bias, T *out, int64_t image_bytes, int tiles_m, int tiles_n) {
-    constexpr int BM = 64, BN = 64;
     using StA = Stager<T, BM, BK, true, A_VEC>;
-    using Engine = TileEngine<T, BM, BN, BK, 2, 2, StA, StB>;
+    using Engine = ConvEngine<T, BM, BN, BK, StA, StB>;
     extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
     T *const smem = reinterpret_cast<T *>(smem_raw);
     const int tid = threadIdx.x;
@@ -480,12 +484,11 @@ __global__ void __launch_bounds__(256) weight_transpose_kernel(ConvGeom geo, con
 
 // grad_input: M = C, N = H*W, K = O*k*k, one GEMM per image.  wt is the transposed weight [C, O*k*k];
 // StB gathers grad_out.
-template <typename T, int BK, int A_VEC, class StB>
+template <typename T, int BM, int BN, int BK, int A_VEC, class StB>
 __global__ void __launch_bounds__(kThreads, 2)
 conv_dgrad_kernel(ConvGeom geo, const T *gout, const T *wt, T *gin, int tiles_m, int tiles_n) {
-    constexpr int BM = 64, BN = 64;
     using StA = Stager<T, BM, BK, true, A_VEC>;
-    using Engine = TileEngine<T, BM, BN, BK, 2, 2, StA, StB>;
+    using Engine = ConvEngine<T, BM, BN, BK, StA, StB>;
     extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
     T *const smem = reinterpret_cast<T *>(smem_raw);
     const int tid = threadIdx.x;
@@ -504,45 +507,58 @@ conv_dgrad_kernel(ConvGeom geo, const T *gout, const T *wt, T *gin, int tiles_m,
     store_tile_dense<T>(eng, gin + static_cast<int64_t>(b) * M_ * N_, M_, N_, m0, n0, static_cast<const T *>(nullptr), 0, 0, 0);
 }
 
-// grad_weight: M = O, N = C*k*k, K = Ho*Wo per image; workgroup column `split` accumulates images
-// [split*group, min(B, (split+1)*group)) in registers and writes one partial tile.
+// grad_weight: M = O, N = C*k*k, K = Ho*Wo per image.  Workgroup column `part` = (image group, k slice)
+// accumulates slice [k0, k0 + k_chunk) of images [grp*group, min(B, (grp+1)*group)) in registers and writes one
+// partial tile; k_chunk is a multiple of BK.
 template <typename T, int BK, int A_VEC, class StB>
 __global__ void __launch_bounds__(kThreads, 2)
-conv_wgrad_kernel(ConvGeom geo, const T *gout, const T *x, T *partial, int64_t image_bytes, int group, int tiles_m, int tiles_n) {
+conv_wgrad_kernel(ConvGeom geo, const T *gout, const T *x, T *partial, int64_t image_bytes, int group, int kslices, int k_chunk,
+                  int tiles_m, int tiles_n) {
     constexpr int BM = 64, BN = 64;
     using StA = Stager<T, BM, BK, true, A_VEC>;
-    using Engine = TileEngine<T, BM, BN, BK, 2, 2, StA, StB>;
+    using Engine = ConvEngine<T, BM, BN, BK, StA, StB>;
     extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
     T *const smem = reinterpret_cast<T *>(smem_raw);
     const int tid = threadIdx.x;
-    int split, tm, tn;
-    decode_tile(remap_xcd(blockIdx.x, gridDim.x), tiles_m, tiles_n, split, tm, tn);
+    int part, tm, tn;
+    decode_tile(remap_xcd(blockIdx.x, gridDim.x), tiles_m, tiles_n, part, tm, tn);
     const int m0 = tm * BM, n0 = tn * BN;
     const int M_ = geo.O, N_ = geo.C * geo.k * geo.k, K = geo.Ho * geo.Wo;
+    const int grp = part / kslices, k0 = (part - grp * kslices) * k_chunk;
+    const int k_len = K - k0 < k_chunk ? K - k0 : k_chunk;
     const int64_t g_image = static_cast<int64_t>(geo.O) * K;
     StA sa;
     StB sb(geo);
     sb.init(tid, n0);
     Engine eng;
     eng.init(tid);
-    const int b_end = (split + 1) * group < geo.B ? (split + 1) * group : geo.B;
-    for (int b = split * group; b < b_end; ++b) {
-        sa.init(gout + b * g_image + static_cast<int64_t>(m0) * K, tid, M_ - m0, K, 1, K);
-        sb.set_image(x + static_cast<int64_t>(b) * geo.xs_b, image_bytes);
-        eng.run(sa, sb, smem, K, false);
+    const int b_end = (grp + 1) * group < geo.B ? (grp + 1) * group : geo.B;
+    for (int b = grp * group; b < b_end; ++b) {
+        sa.init(gout + b * g_image + static_cast<int64_t>(m0) * K + k0, tid, M_ - m0, K, 1, k_len);
+        sb.set_image(x + static_cast<int64_t>(b) * geo.xs_b, image_bytes, k0);
+        eng.run(sa, sb, smem, k_len, false);
         __syncthreads();  // the next image's prologue overwrites LDS buffer 0
     }
-    store_tile_dense<T>(eng, partial + static_cast<int64_t>(split) * M_ * N_, M_, N_, m0, n0, static_cast<const T *>(nullptr), 0, 0, 0);
+    store_tile_dense<T>(eng, partial + static_cast<int64_t>(part) * M_ * N_, M_, N_, m0, n0, static_cast<const T *>(nullptr), 0, 0, 0);
 }
 
-// out[i] = sum over splits of partial[s][i], in increasing s (image order).
+// out[i] = sum over parts of partial[s][i].  A workgroup owns 16 consecutive elements; its 16 lanes per element
+// each add every 16th part in increasing order, and a fixed tree adds the 16 sums (deterministic).
 template <typename T>
 __global__ void __launch_bounds__(256) reduce_splits_kernel(const T *__restrict__ partial, T *__restrict__ out, int64_t n, int splits) {
-    const int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
-    if (i >= n) return;
-    T acc = partial[i];
-    for (int s = 1; s < splits; ++s) acc += partial[static_cast<int64_t>(s) * n + i];
-    out[i] = acc;
+    __shared__ T red[16][17];
+    const int e = threadIdx.x % 16, lane_s = threadIdx.x / 16;
+    const int64_t i = static_cast<int64_t>(blockIdx.x) * 16 + e;
+    T acc = T(0);
+    if (i < n)
+        for (int s = lane_s; s < splits; s += 16) acc += partial[static_cast<int64_t>(s) * n + i];
+    red[lane_s][e] = acc;
+    __syncthreads();
+    for (int h = 8; h > 0; h >>= 1) {
+        if (lane_s < h) red[lane_s][e] += red[lane_s + h][e];
+        __syncthreads();
+    }
+    if (lane_s == 0 && i < n) out[i] = red[0][e];
 }
 
 // grad_bias[o] = sum over batch and space of grad_out[b][o][.] (cpu/conv.cpp:289).  One workgroup per channel.
@@ -702,19 +718,19 @@ ttamd_status launch_conv(Kernel kernel, size_t lds, int64_t blocks, hipStream_t 
     return TTAMD_OK;
 }
 
-// LDS bytes of the 64x64 engine built from the weight/grad_out stager and gather stager StB.
-template <typename T, int A_VEC, class StB>
+// LDS bytes of the engine built from the weight/grad_out stager and gather stager StB.
+template <typename T, int BM, int BN, int A_VEC, class StB>
 constexpr size_t conv_lds_bytes() {
     constexpr int BK = ConvTiles<T>::BK;
-    return TileEngine<T, 64, 64, BK, 2, 2, Stager<T, 64, BK, true, A_VEC>, StB>::kLdsBytes;
+    return ConvEngine<T, BM, BN, BK, Stager<T, BM, BK, true, A_VEC>, StB>::kLdsBytes;
 }
 
-template <typename T>
-ttamd_status forward_mfma(const ConvPlan &pl, const void *bias, void *out, hipStream_t st) {
+template <typename T, int BM, int BN>
+ttamd_status forward_mfma_tile(const ConvPlan &pl, const void *bias, void *out, hipStream_t st) {
     constexpr int BK = ConvTiles<T>::BK, VK = Mfma<T>::VK;
     const ConvGeom &g = pl.geo;
     const int M_ = g.O, N_ = g.Ho * g.Wo;
-    const int tiles_m = (M_ + 63) / 64, tiles_n = (N_ + 63) / 64;
+    const int tiles_m = (M_ + BM - 1) / BM, tiles_n = (N_ + BN - 1) / BN;
     const int64_t blocks = static_cast<int64_t>(tiles_m) * tiles_n * g.B;
     const bool a_vec = rows_vectorizable<T>(pl.w, g.w_so, 0);
     const bool b_vec = g.S == 1 && g.xs_w == 1 && g.Wo % VK == 0;
@@ -722,12 +738,18 @@ ttamd_status forward_mfma(const ConvPlan &pl, const void *bias, void *out, hipSt
         return launch_conv(kernel, lds, blocks, st, g, static_cast<const T *>(pl.x), static_cast<const T *>(pl.w),
                            static_cast<const T *>(bias), static_cast<T *>(out), pl.image_bytes, tiles_m, tiles_n);
     };
-    using VecB = TapStagerMC<T, 64, BK, VK, false>;
-    using OneB = Im2colStager<T, 64, BK>;
-    if (a_vec && b_vec) return go(conv_fwd_kernel<T, BK, VK, VecB>, conv_lds_bytes<T, VK, VecB>());
-    if (a_vec) return go(conv_fwd_kernel<T, BK, VK, OneB>, conv_lds_bytes<T, VK, OneB>());
-    if (b_vec) return go(conv_fwd_kernel<T, BK, 1, VecB>, conv_lds_bytes<T, 1, VecB>());
-    return go(conv_fwd_kernel<T, BK, 1, OneB>, conv_lds_bytes<T, 1, OneB>());
+    using VecB = TapStagerMC<T, BN, BK, VK, false>;
+    using OneB = Im2colStager<T, BN, BK>;
+    if (a_vec && b_vec) return go(conv_fwd_kernel<T, BM, BN, BK, VK, VecB>, conv_lds_bytes<T, BM, BN, VK, VecB>());
+    if (a_vec) return go(conv_fwd_kernel<T, BM, BN, BK, VK, OneB>, conv_lds_bytes<T, BM, BN, VK, OneB>());
+    if (b_vec) return go(conv_fwd_kernel<T, BM, BN, BK, 1, VecB>, conv_lds_bytes<T, BM, BN, 1, VecB>());
+    return go(conv_fwd_kernel<T, BM, BN, BK, 1, OneB>, conv_lds_bytes<T, BM, BN, 1, OneB>());
+}
+
+template <typename T>
+ttamd_status forward_mfma(const ConvPlan &pl, const void *bias, void *out, hipStream_t st) {
+    if (pl.geo.O <= 32) return forward_mfma_tile<T, 32, 128>(pl, bias, out, st);
+    return forward_mfma_tile<T, 64, 64>(pl, bias, out, st);
 }
 
 template <typename T, typename Acc>
@@ -756,20 +778,37 @@ int wgrad_group(size_t esz, int B, int C, int O, int k) {
 }
 
 // Workspace layout of conv2d_backward: the transposed weight [C, O*k*k] (rounded up to 256 bytes), then, when
-// grad_weight is split over the batch, `splits` partial [O, C*k*k] tiles.
+// grad_weight is computed in several parts, `parts` partial [O, C*k*k] tiles.  A part is (group of images,
+// slice of the output positions): enough of them to give every compute unit a few workgroups.
 struct BackwardWorkspace {
     size_t wt_bytes, partial_bytes;
-    int group, splits;
+    int group, splits;     // images per group, number of groups
+    int kslices, k_chunk;  // slices of the Ho*Wo reduction, positions per slice (a multiple of the k tile)
+    int parts() const { return splits * kslices; }
     size_t total() const { return wt_bytes + partial_bytes; }
 };
 
-BackwardWorkspace backward_workspace(size_t esz, int B, int C, int O, int k) {
+BackwardWorkspace backward_workspace(size_t esz, int B, int C, int H, int W, int O, int k, int stride, int padding) {
     BackwardWorkspace w{};
     const size_t tile = static_cast<size_t>(O) * C * k * k * esz;
     w.wt_bytes = (tile + 255) & ~static_cast<size_t>(255);
     w.group = wgrad_group(esz, B, C, O, k);
     w.splits = (B + w.group - 1) / w.group;
-    w.partial_bytes = w.splits > 1 ? static_cast<size_t>(w.splits) * tile : 0;
+    const int bk = esz == 4 ? 32 : 16;
+    const int Ho = (H + 2 * padding - k) / stride + 1, Wo = (W + 2 * padding - k) / stride + 1;
+    const int64_t K = static_cast<int64_t>(Ho) * Wo;
+    const int64_t k_tiles = (K + bk - 1) / bk;
+    const int64_t tiles = static_cast<int64_t>((O + 63) / 64) * ((static_cast<int64_t>(C) * k * k + 63) / 64);
+    int64_t want = 768 / (tiles * w.splits);                      // slices that bring the launch to ~3 workgroups per CU
+    if (want > k_tiles / 4) want = k_tiles / 4;                    // at least 4 k tiles per slice
+    const int64_t room = (64LL << 20) / static_cast<int64_t>(tile ? tile : 1) / w.splits;  // partial tiles <= 64 MiB
+    if (want > room) want = room;
+    if (want < 1) want = 1;
+    const int64_t chunk_tiles = (k_tiles + want - 1) / want;
+    w.k_chunk = static_cast<int>(chunk_tiles * bk);
+    w.kslices = static_cast<int>((k_tiles + chunk_tiles - 1) / chunk_tiles);
+    if (w.kslices < 1) w.kslices = 1;
+    w.partial_bytes = w.parts() > 1 ? static_cast<size_t>(w.parts()) * tile : 0;
     return w;
 }
 
@@ -779,7 +818,7 @@ ttamd_status backward_mfma(const ConvPlan &pl, const void *gout, void *gin, void
     constexpr int BK = ConvTiles<T>::BK, VK = Mfma<T>::VK;
     const ConvGeom &g = pl.geo;
     const int HoWo = g.Ho * g.Wo;
-    const BackwardWorkspace plan = backward_workspace(sizeof(T), g.B, g.C, g.O, g.k);
+    const BackwardWorkspace plan = backward_workspace(sizeof(T), g.B, g.C, g.H, g.W, g.O, g.k, g.S, g.P);
     if (!ws || ws_bytes < plan.total()) {
         set_error("conv2d_backward: workspace of %zu bytes is smaller than the %zu bytes required", ws_bytes, plan.total());
         return TTAMD_ERR_INVALID_ARGUMENT;
@@ -792,48 +831,51 @@ ttamd_status backward_mfma(const ConvPlan &pl, const void *gout, void *gin, void
         const int total = g.C * Kd;
         weight_transpose_kernel<T><<<dim3((total + 255) / 256), dim3(256), 0, st>>>(g, static_cast<const T *>(pl.w), wt, total);
         TTAMD_HIP_CHECK(hipGetLastError());
-        const int M_ = g.C, N_ = g.H * g.W;
-        const int tiles_m = (M_ + 63) / 64, tiles_n = (N_ + 63) / 64;
-        const int64_t blocks = static_cast<int64_t>(tiles_m) * tiles_n * g.B;
-        const bool a_vec = rows_vectorizable<T>(wt, Kd, 0);
-        const bool b_vec = g.S == 1 && g.W % VK == 0;
-        auto go = [&](auto kernel, size_t lds) {
-            return launch_conv(kernel, lds, blocks, st, g, static_cast<const T *>(gout), static_cast<const T *>(wt),
-                               static_cast<T *>(gin), tiles_m, tiles_n);
+        auto run = [&]<int BM, int BN>() -> ttamd_status {
+            const int M_ = g.C, N_ = g.H * g.W;
+            const int tiles_m = (M_ + BM - 1) / BM, tiles_n = (N_ + BN - 1) / BN;
+            const int64_t blocks = static_cast<int64_t>(tiles_m) * tiles_n * g.B;
+            const bool a_vec = rows_vectorizable<T>(wt, Kd, 0);
+            const bool b_vec = g.S == 1 && g.W % VK == 0;
+            auto go = [&](auto kernel, size_t lds) {
+                return launch_conv(kernel, lds, blocks, st, g, static_cast<const T *>(gout), static_cast<const T *>(wt),
+                                   static_cast<T *>(gin), tiles_m, tiles_n);
+            };
+            using VecB = TapStagerMC<T, BN, BK, VK, true>;
+            using OneB = DgradStager<T, BN, BK>;
+            if (a_vec && b_vec) return go(conv_dgrad_kernel<T, BM, BN, BK, VK, VecB>, conv_lds_bytes<T, BM, BN, VK, VecB>());
+            if (a_vec) return go(conv_dgrad_kernel<T, BM, BN, BK, VK, OneB>, conv_lds_bytes<T, BM, BN, VK, OneB>());
+            if (b_vec) return go(conv_dgrad_kernel<T, BM, BN, BK, 1, VecB>, conv_lds_bytes<T, BM, BN, 1, VecB>());
+            return go(conv_dgrad_kernel<T, BM, BN, BK, 1, OneB>, conv_lds_bytes<T, BM, BN, 1, OneB>());
         };
-        using VecB = TapStagerMC<T, 64, BK, VK, true>;
-        using OneB = DgradStager<T, 64, BK>;
-        ttamd_status s;
-        if (a_vec && b_vec) s = go(conv_dgrad_kernel<T, BK, VK, VecB>, conv_lds_bytes<T, VK, VecB>());
-        else if (a_vec) s = go(conv_dgrad_kernel<T, BK, VK, OneB>, conv_lds_bytes<T, VK, OneB>());
-        else if (b_vec) s = go(conv_dgrad_kernel<T, BK, 1, VecB>, conv_lds_bytes<T, 1, VecB>());
-        else s = go(conv_dgrad_kernel<T, BK, 1, OneB>, conv_lds_bytes<T, 1, OneB>());
+        const ttamd_status s = g.C <= 32 ? run.template operator()<32, 128>() : run.template operator()<64, 64>();
         if (s) return s;
     }
     // grad_weight
     {
         const int M_ = g.O, N_ = g.C * g.k * g.k;
         const int64_t tile_elems = static_cast<int64_t>(M_) * N_;
-        T *const partial = plan.splits > 1 ? partials : static_cast<T *>(gw);
+        const int parts = plan.parts();
+        T *const partial = parts > 1 ? partials : static_cast<T *>(gw);
         const int tiles_m = (M_ + 63) / 64, tiles_n = (N_ + 63) / 64;
-        const int64_t blocks = static_cast<int64_t>(tiles_m) * tiles_n * plan.splits;
+        const int64_t blocks = static_cast<int64_t>(tiles_m) * tiles_n * parts;
         const bool a_vec = rows_vectorizable<T>(gout, HoWo, static_cast<int64_t>(g.O) * HoWo);
         const bool b_vec = g.S == 1 && g.xs_w == 1 && g.Wo % VK == 0;
         auto go = [&](auto kernel, size_t lds) {
-            return launch_conv(kernel, lds, blocks, st, g, static_cast<const T *>(gout), static_cast<const T *>(pl.x),
-                               partial, pl.image_bytes, plan.group, tiles_m, tiles_n);
+            return launch_conv(kernel, lds, blocks, st, g, static_cast<const T *>(gout), static_cast<const T *>(pl.x), partial,
+                               pl.image_bytes, plan.group, plan.kslices, plan.k_chunk, tiles_m, tiles_n);
         };
         using VecB = TapStagerKC<T, 64, BK, VK>;
         using OneB = Im2colTStager<T, 64, BK>;
         ttamd_status s;
-        if (a_vec && b_vec) s = go(conv_wgrad_kernel<T, BK, VK, VecB>, conv_lds_bytes<T, VK, VecB>());
-        else if (a_vec) s = go(conv_wgrad_kernel<T, BK, VK, OneB>, conv_lds_bytes<T, VK, OneB>());
-        else if (b_vec) s = go(conv_wgrad_kernel<T, BK, 1, VecB>, conv_lds_bytes<T, 1, VecB>());
-        else s = go(conv_wgrad_kernel<T, BK, 1, OneB>, conv_lds_bytes<T, 1, OneB>());
+        if (a_vec && b_vec) s = go(conv_wgrad_kernel<T, BK, VK, VecB>, conv_lds_bytes<T, 64, 64, VK, VecB>());
+        else if (a_vec) s = go(conv_wgrad_kernel<T, BK, VK, OneB>, conv_lds_bytes<T, 64, 64, VK, OneB>());
+        else if (b_vec) s = go(conv_wgrad_kernel<T, BK, 1, VecB>, conv_lds_bytes<T, 64, 64, 1, VecB>());
+        else s = go(conv_wgrad_kernel<T, BK, 1, OneB>, conv_lds_bytes<T, 64, 64, 1, OneB>());
         if (s) return s;
-        if (plan.splits > 1) {
-            const int64_t rb = (tile_elems + 255) / 256;
-            reduce_splits_kernel<T><<<dim3(static_cast<unsigned>(rb)), dim3(256), 0, st>>>(partial, static_cast<T *>(gw), tile_elems, plan.splits);
+        if (parts > 1) {
+            const int64_t rb = (tile_elems + 15) / 16;
+            reduce_splits_kernel<T><<<dim3(static_cast<unsigned>(rb)), dim3(256), 0, st>>>(partial, static_cast<T *>(gw), tile_elems, parts);
             TTAMD_HIP_CHECK(hipGetLastError());
         }
     }
@@ -878,7 +920,6 @@ ttamd_status ttamd_conv2d_forward(int device, ttamd_dtype dtype, const ttamd_vie
 
 ttamd_status ttamd_conv2d_backward_workspace(ttamd_dtype dtype, int B, int C, int H, int W, int O, int k, int stride,
                                              int padding, size_t *bytes) {
-    (void)H; (void)W; (void)stride; (void)padding;
     if (!bytes) {
         set_error("conv2d_backward_workspace: bytes is NULL");
         return TTAMD_ERR_INVALID_ARGUMENT;
@@ -888,8 +929,10 @@ ttamd_status ttamd_conv2d_backward_workspace(ttamd_dtype dtype, int B, int C, in
         set_error("conv2d_backward supports f32 and f64 only (autograd never differentiates integer tensors)");
         return TTAMD_ERR_UNSUPPORTED_DTYPE;
     }
-    if (B <= 0 || C <= 0 || O <= 0 || k <= 0) return TTAMD_OK;
-    *bytes = backward_workspace(dtype_size(dtype), B, C, O, k).total();
+    if (B <= 0 || C <= 0 || O <= 0 || k <= 0 || H <= 0 || W <= 0 || stride <= 0 || padding < 0 || H + 2 * padding < k ||
+        W + 2 * padding < k)
+        return TTAMD_OK;  // ttamd_conv2d_backward rejects the geometry itself
+    *bytes = backward_workspace(dtype_size(dtype), B, C, H, W, O, k, stride, padding).total();
     return TTAMD_OK;
 }
 
