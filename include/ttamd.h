@@ -145,6 +145,21 @@ ttamd_status ttamd_conv2d_backward(int device, ttamd_dtype dtype, const void *gr
                                    int B, int C, int H, int W, int O, int k, int stride, int padding, void *workspace,
                                    size_t workspace_bytes, void *stream);
 
+/* BackendBase::max_pool2d / min_pool2d / avg_pool2d (backend_base.h:286-311; CPU: cpu/conv.cpp:296-349 over
+ * cpu/kernel/conv.hpp:121-161).  input [B,C,H,W] (any strides), square window k, zero-contribution padding;
+ * out dense [B,C,Ho,Wo] of the input's dtype, except avg of an integer input, which is f32
+ * (common/reduce.h:63-69).  The window is folded in the reference's order with its arithmetic
+ * (avg: out = x / (k*k) + out), so results are bit-identical to the CPU device's. */
+typedef enum { TTAMD_POOL_MAX = 0, TTAMD_POOL_MIN = 1, TTAMD_POOL_AVG = 2 } ttamd_pool_op;
+ttamd_status ttamd_pool2d_forward(int device, ttamd_dtype dtype, int op, const ttamd_view4 *input, void *out, int B,
+                                  int C, int H, int W, int k, int stride, int padding, void *stream);
+/* BackendBase::*_pool2d_backward (backend_base.h:288-311; CPU: cpu/conv.cpp:351-426 over conv.hpp:171-275); f32/f64.
+ * grad_out and result dense [B,C,Ho,Wo]; writes every element of grad_input [B,C,H,W] (dense).  max/min: an
+ * output's gradient is split evenly over the in-bounds window elements equal to the result. */
+ttamd_status ttamd_pool2d_backward(int device, ttamd_dtype dtype, int op, const void *grad_out, const ttamd_view4 *input,
+                                   const void *result, void *grad_input, int B, int C, int H, int W, int k, int stride,
+                                   int padding, void *stream);
+
 /* ---- elementwise / reduction ops that an MLP training step needs around its GEMMs ------------
  * (BackendBase::add, sub, mul, div, pow, maximum, minimum, lt, le, gt, ge, eq, ne: backend_base.h:109-131;
  * relu & friends: :136-260; where: :263; sum: :148-149; full: :51.  CPU forms: cpu/binary.cpp:26-84,
@@ -164,6 +179,16 @@ ttamd_status ttamd_binary(int device, ttamd_dtype dtype, int op, int ndim, const
                           const int64_t *rhs_stride, void *out, void *stream);
 ttamd_status ttamd_unary(int device, ttamd_dtype dtype, int op, int ndim, const int64_t *shape, const void *src,
                          int64_t offset, const int64_t *stride, void *out, void *stream);
+/* BackendBase::to (backend_base.h:74; CPU: cpu/cast.cpp:27-110): out[i] = static_cast<to>(view[i]), dense result of
+ * dtype `to`; a bool result is 1 for every non-zero element.  Float values outside the target integer's range
+ * are undefined in the reference and saturate here. */
+ttamd_status ttamd_cast(int device, ttamd_dtype from, ttamd_dtype to, int ndim, const int64_t *shape, const void *src,
+                        int64_t offset, const int64_t *stride, void *out, void *stream);
+/* BackendBase::assign (backend_base.h:78; CPU: cpu/kernel/assign.hpp:15-21): dst_view[i] = src_view[i] over one
+ * shape; both operands are strided views of the same dtype (any dtype, bool included). */
+ttamd_status ttamd_assign(int device, ttamd_dtype dtype, int ndim, const int64_t *shape, void *dst, int64_t dst_offset,
+                          const int64_t *dst_stride, const void *src, int64_t src_offset, const int64_t *src_stride,
+                          void *stream);
 /* BackendBase::where (backend_base.h:263): out = cond ? lhs : rhs; cond is a bool (one byte) view. */
 ttamd_status ttamd_where(int device, ttamd_dtype dtype, int ndim, const int64_t *shape, const void *cond,
                          int64_t cond_offset, const int64_t *cond_stride, const void *lhs, int64_t lhs_offset,

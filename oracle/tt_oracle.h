@@ -23,6 +23,10 @@
  *   tto_contiguous        brute force against explicit nested-loop indexing.
  *   tto_conv2d_*          naive 7-deep loop (reference test oracle), adjoint
  *                         identities for the backward pass.
+ *   tto_pool2d_*          torch.nn.functional max_pool2d / avg_pool2d and their autograd on
+ *                         the reference tests' shapes (what tests/test_conv.cpp:186-278 and
+ *                         tests/test_conv_autograd.cpp:109-230 compare with), plus a
+ *                         brute-force numpy window statement incl. ties and padding.
  *   tto_splitmix64 / xorshift64  published test vectors (Vigna's splitmix64.c
  *                         seed 1234567 stream; xorshift64 13/7/17 closed form).
  *   tto_uniform_real_*    closed form from the bit construction.
@@ -105,6 +109,14 @@ int tto_conv2d_backward(int dtype, const void *grad_out, const void *input, cons
 /* Naive 7-deep loop (tests/test_conv.cpp:29-73). */
 int tto_conv2d_naive(int dtype, const void *input, const void *weight, void *out, int B, int C, int H, int W, int O,
                      int k, int stride, int padding);
+
+/* ---- 2-D pooling (cpu/conv.cpp:296-426, cpu/kernel/conv.hpp:121-275; tt_oracle_pool.c) ----
+ * op: 0 max, 1 min, 2 avg.  Dense NCHW input; the result has the input's dtype except avg of an integer
+ * input, which is f32.  backward: f32 / f64 only; grad_out, result and grad_input share the input's dtype. */
+int tto_pool2d_forward(int dtype, int op, const void *input, void *out, int B, int C, int H, int W, int k, int stride,
+                       int padding);
+int tto_pool2d_backward(int dtype, int op, const void *grad_out, const void *input, const void *result, void *grad_input,
+                        int B, int C, int H, int W, int k, int stride, int padding);
 
 /* im2col / col2im index maps exposed for brute-force tests (conv.hpp:12-118), f64 only. */
 void tto_unroll_f64(const double *X, double *Xu, int b, int C, int H, int W, int k, int S, int P);

@@ -68,6 +68,10 @@ def _load(flavour: str) -> C.CDLL:
     lib.tto_conv2d_forward.argtypes = [i32, vp, vp, vp, vp] + [i32] * 8
     lib.tto_conv2d_backward.restype = i32
     lib.tto_conv2d_backward.argtypes = [i32, vp, vp, vp, vp, vp, vp] + [i32] * 8
+    lib.tto_pool2d_forward.restype = i32
+    lib.tto_pool2d_forward.argtypes = [i32, i32, vp, vp] + [i32] * 7
+    lib.tto_pool2d_backward.restype = i32
+    lib.tto_pool2d_backward.argtypes = [i32, i32, vp, vp, vp, vp] + [i32] * 7
     lib.tto_conv2d_naive.restype = i32
     lib.tto_conv2d_naive.argtypes = [i32, vp, vp, vp] + [i32] * 8
     for f in ("tto_unroll_f64", "tto_unroll_transpose_f64", "tto_col2im_f64"):
@@ -252,6 +256,38 @@ def conv2d_naive(x, w, stride=1, padding=0, flavour="fma"):
                                        padding)
     assert rc == 0
     return out
+
+
+# ----------------------------------------------------------------------------- pooling
+POOL_OPS = {"max": 0, "min": 1, "avg": 2}
+
+
+def pool2d_forward(x, op: str, kernel_size: int, stride: int, padding: int):
+    """max_pool2d / min_pool2d / avg_pool2d on the CPU device (cpu/conv.cpp:296-349, kernel conv.hpp:121-161).
+    avg of an integer input yields float32 (common/reduce.h:63-69)."""
+    x = np.ascontiguousarray(x)
+    Bn, Cc, H, W = x.shape
+    Ho = (H + 2 * padding - kernel_size) // stride + 1
+    Wo = (W + 2 * padding - kernel_size) // stride + 1
+    rdtype = np.float32 if (op == "avg" and x.dtype.kind != "f") else x.dtype
+    out = np.zeros((Bn, Cc, Ho, Wo), dtype=rdtype)
+    rc = lib().tto_pool2d_forward(CODE_OF[x.dtype], POOL_OPS[op], _ptr(x), _ptr(out), Bn, Cc, H, W, kernel_size, stride,
+                                  padding)
+    assert rc == 0
+    return out
+
+
+def pool2d_backward(gout, x, result, op: str, kernel_size: int, stride: int, padding: int):
+    """*_pool2d_backward (cpu/conv.cpp:351-426, kernels conv.hpp:171-275); float dtypes."""
+    x = np.ascontiguousarray(x)
+    gout = np.ascontiguousarray(gout, dtype=x.dtype)
+    result = np.ascontiguousarray(result, dtype=x.dtype)
+    Bn, Cc, H, W = x.shape
+    gx = np.zeros_like(x)
+    rc = lib().tto_pool2d_backward(CODE_OF[x.dtype], POOL_OPS[op], _ptr(gout), _ptr(x), _ptr(result), _ptr(gx), Bn, Cc, H,
+                                   W, kernel_size, stride, padding)
+    assert rc == 0
+    return gx
 
 
 # ----------------------------------------------------------------------------- nn::Linear / MLP step

@@ -6,6 +6,6 @@ tests and the benchmark: same names, argument meaning and error behaviour as the
 """
 from .tensor import (  # noqa: F401
     BackendAMD, Device, Generator, Tensor, TTException, broadcast_tensors, linear_init, normal, uniform_real, conv2d, conv2d_backward, full, get_backend, kAMD, linear,
-    matmul, matmul_backward, where,
+    matmul, matmul_backward, where, max_pool2d, min_pool2d, avg_pool2d, pool2d_backward,
 )
 from . import _capi  # noqa: F401

@@ -15,6 +15,7 @@ OK, ERR_INVALID_ARGUMENT, ERR_INVALID_DEVICE, ERR_UNSUPPORTED_DTYPE, ERR_OUT_OF_
 BOOL, U8, I16, I32, I64, F32, F64 = range(7)
 BIN = {"add": 0, "sub": 1, "mul": 2, "div": 3, "pow": 4, "maximum": 5, "minimum": 6, "lt": 7, "le": 8, "gt": 9, "ge": 10,
        "eq": 11, "ne": 12}
+POOL = {"max": 0, "min": 1, "avg": 2}
 UN = {"relu": 0, "negate": 1, "abs": 2, "sqrt": 3, "exp": 4, "log": 5, "sigmoid": 6, "tanh": 7}
 
 
@@ -47,6 +48,9 @@ def _bind(lib: C.CDLL) -> None:
         "ttamd_binary": (i, [i, i, i, i, C.POINTER(C.c_int64), vp, C.c_int64, C.POINTER(C.c_int64), vp, C.c_int64,
                              C.POINTER(C.c_int64), vp, vp]),
         "ttamd_unary": (i, [i, i, i, i, C.POINTER(C.c_int64), vp, C.c_int64, C.POINTER(C.c_int64), vp, vp]),
+        "ttamd_cast": (i, [i, i, i, i, C.POINTER(C.c_int64), vp, C.c_int64, C.POINTER(C.c_int64), vp, vp]),
+        "ttamd_assign": (i, [i, i, i, C.POINTER(C.c_int64), vp, C.c_int64, C.POINTER(C.c_int64), vp, C.c_int64,
+                             C.POINTER(C.c_int64), vp]),
         "ttamd_where": (i, [i, i, i, C.POINTER(C.c_int64), vp, C.c_int64, C.POINTER(C.c_int64), vp, C.c_int64,
                             C.POINTER(C.c_int64), vp, C.c_int64, C.POINTER(C.c_int64), vp, vp]),
         "ttamd_sum": (i, [i, i, i, C.POINTER(C.c_int64), vp, C.c_int64, C.POINTER(C.c_int64), i, vp, vp]),
@@ -57,6 +61,8 @@ def _bind(lib: C.CDLL) -> None:
         "ttamd_conv2d_forward": (i, [i, i, C.POINTER(View4), C.POINTER(View4), vp, vp] + [i] * 8 + [vp]),
         "ttamd_conv2d_backward_workspace": (i, [i] + [i] * 8 + [C.POINTER(sz)]),
         "ttamd_conv2d_backward": (i, [i, i, vp, C.POINTER(View4), C.POINTER(View4), vp, vp, vp] + [i] * 8 + [vp, sz, vp]),
+        "ttamd_pool2d_forward": (i, [i, i, i, C.POINTER(View4), vp] + [i] * 7 + [vp]),
+        "ttamd_pool2d_backward": (i, [i, i, i, vp, C.POINTER(View4), vp, vp] + [i] * 7 + [vp]),
         "ttamd_event_create": (i, [i, C.POINTER(vp)]),
         "ttamd_event_destroy": (i, [vp]),
         "ttamd_event_record": (i, [vp, vp]),

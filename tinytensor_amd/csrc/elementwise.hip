@@ -217,6 +217,26 @@ __global__ void __launch_bounds__(256) normal_kernel(const uint64_t *__restrict_
     out[i] = stddev * (r * sin(theta)) + mu;
 }
 
+// to(dtype): out[i] = static_cast<R>(view[i]) (tinytensor/tensor/backend/cpu/cast.cpp:27-34; bool keeps C++'s
+// "non-zero is true").
+template <typename T, typename R>
+__global__ void __launch_bounds__(256) cast_kernel(const T *__restrict__ a, ViewDesc va, bool dense, R *__restrict__ out, int64_t numel) {
+    const int64_t step = static_cast<int64_t>(gridDim.x) * blockDim.x;
+    for (int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < numel; i += step) {
+        const T x = dense ? a[i] : a[flat_of(i, va)];
+        out[i] = static_cast<R>(x);
+    }
+}
+
+// assign: lhs_view[i] = rhs_view[i] over one shape (tinytensor/tensor/backend/cpu/kernel/assign.hpp:15-21).
+// Moves raw bytes, so one kernel per element size serves every dtype.
+template <typename W>
+__global__ void __launch_bounds__(256) assign_kernel(W *__restrict__ dst, ViewDesc vd, const W *__restrict__ src, ViewDesc vs, int64_t numel) {
+    const int64_t step = static_cast<int64_t>(gridDim.x) * blockDim.x;
+    for (int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < numel; i += step)
+        dst[flat_of(i, vd)] = src[flat_of(i, vs)];
+}
+
 inline unsigned grid_for(int64_t numel) {
     int64_t blocks = (numel + 255) / 256;
     if (blocks > 8192) blocks = 8192;
@@ -323,6 +343,37 @@ ttamd_status sum_typed(int device, const void *a, const ViewDesc &v, int64_t num
                                                                                               static_cast<T *>(out), n_out);
     TTAMD_HIP_CHECK(hipGetLastError());
     return TTAMD_OK;
+}
+
+// bool is stored as one byte holding 0 or 1
+struct BoolByte {
+    uint8_t v;
+    __host__ __device__ BoolByte() : v(0) {}
+    template <typename X>
+    __host__ __device__ explicit BoolByte(X x) : v(x != X(0) ? 1 : 0) {}
+};
+
+template <typename T, typename R>
+ttamd_status launch_cast(const void *a, const ViewDesc &va, void *out, int64_t numel, hipStream_t st) {
+    cast_kernel<T, R><<<dim3(grid_for(numel)), dim3(256), 0, st>>>(static_cast<const T *>(a), va, is_dense(va), static_cast<R *>(out), numel);
+    TTAMD_HIP_CHECK(hipGetLastError());
+    return TTAMD_OK;
+}
+
+template <typename T>
+ttamd_status cast_from(ttamd_dtype to, const void *a, const ViewDesc &va, void *out, int64_t numel, hipStream_t st) {
+    switch (to) {
+    case TTAMD_BOOL: return launch_cast<T, BoolByte>(a, va, out, numel, st);
+    case TTAMD_U8: return launch_cast<T, uint8_t>(a, va, out, numel, st);
+    case TTAMD_I16: return launch_cast<T, int16_t>(a, va, out, numel, st);
+    case TTAMD_I32: return launch_cast<T, int32_t>(a, va, out, numel, st);
+    case TTAMD_I64: return launch_cast<T, int64_t>(a, va, out, numel, st);
+    case TTAMD_F32: return launch_cast<T, float>(a, va, out, numel, st);
+    case TTAMD_F64: return launch_cast<T, double>(a, va, out, numel, st);
+    default: break;
+    }
+    set_error("cast: unknown target dtype code %d", static_cast<int>(to));
+    return TTAMD_ERR_UNSUPPORTED_DTYPE;
 }
 
 #define TTAMD_DISPATCH_DTYPE(dtype, CALL)                      \
@@ -440,6 +491,70 @@ ttamd_status ttamd_unary(int device, ttamd_dtype dtype, int op, int ndim, const 
     hipStream_t st = static_cast<hipStream_t>(stream);
     TTAMD_DISPATCH_DTYPE(dtype, (dispatch_unary<T_>(op, a, va, out, numel, st)))
     return TTAMD_ERR_UNSUPPORTED_DTYPE;
+}
+
+ttamd_status ttamd_cast(int device, ttamd_dtype from, ttamd_dtype to, int ndim, const int64_t *shape, const void *src,
+                        int64_t offset, const int64_t *stride, void *out, void *stream) {
+    ViewDesc va;
+    int64_t numel = 0;
+    if (ttamd_status s = make_view("cast", ndim, shape, stride, &va, &numel)) return s;
+    if (from < TTAMD_BOOL || from > TTAMD_F64 || to < TTAMD_BOOL || to > TTAMD_F64) {
+        set_error("cast: unknown dtype code %d -> %d", static_cast<int>(from), static_cast<int>(to));
+        return TTAMD_ERR_UNSUPPORTED_DTYPE;
+    }
+    if (offset < 0) {
+        set_error("cast: negative view offset");
+        return TTAMD_ERR_INVALID_ARGUMENT;
+    }
+    if (ttamd_status s = use_device(device)) return s;
+    if (numel == 0) return TTAMD_OK;
+    if (!src || !out) {
+        set_error("cast: NULL data pointer");
+        return TTAMD_ERR_INVALID_ARGUMENT;
+    }
+    const void *a = static_cast<const char *>(src) + offset * static_cast<int64_t>(dtype_size(from));
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    if (from == TTAMD_BOOL) return cast_from<uint8_t>(to, a, va, out, numel, st);  // stored as 0 / 1
+    TTAMD_DISPATCH_DTYPE(from, (cast_from<T_>(to, a, va, out, numel, st)))
+    return TTAMD_ERR_UNSUPPORTED_DTYPE;
+}
+
+ttamd_status ttamd_assign(int device, ttamd_dtype dtype, int ndim, const int64_t *shape, void *dst, int64_t dst_offset,
+                          const int64_t *dst_stride, const void *src, int64_t src_offset, const int64_t *src_stride, void *stream) {
+    ViewDesc vd, vs;
+    int64_t numel = 0;
+    if (ttamd_status s = make_view("assign", ndim, shape, dst_stride, &vd, &numel)) return s;
+    if (ttamd_status s = make_view("assign", ndim, shape, src_stride, &vs, nullptr)) return s;
+    const size_t esz = dtype_size(dtype);
+    if (dtype < TTAMD_BOOL || dtype > TTAMD_F64 || esz == 0) {
+        set_error("assign: unknown dtype code %d", static_cast<int>(dtype));
+        return TTAMD_ERR_UNSUPPORTED_DTYPE;
+    }
+    if (dst_offset < 0 || src_offset < 0) {
+        set_error("assign: negative view offset");
+        return TTAMD_ERR_INVALID_ARGUMENT;
+    }
+    if (ttamd_status s = use_device(device)) return s;
+    if (numel == 0) return TTAMD_OK;
+    if (!dst || !src) {
+        set_error("assign: NULL data pointer");
+        return TTAMD_ERR_INVALID_ARGUMENT;
+    }
+    char *d = static_cast<char *>(dst) + dst_offset * static_cast<int64_t>(esz);
+    const char *a = static_cast<const char *>(src) + src_offset * static_cast<int64_t>(esz);
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    auto go = [&](auto tag) -> ttamd_status {
+        using W = decltype(tag);
+        assign_kernel<W><<<dim3(grid_for(numel)), dim3(256), 0, st>>>(reinterpret_cast<W *>(d), vd, reinterpret_cast<const W *>(a), vs, numel);
+        TTAMD_HIP_CHECK(hipGetLastError());
+        return TTAMD_OK;
+    };
+    switch (esz) {
+    case 1: return go(uint8_t{});
+    case 2: return go(uint16_t{});
+    case 4: return go(uint32_t{});
+    default: return go(uint64_t{});
+    }
 }
 
 ttamd_status ttamd_where(int device, ttamd_dtype dtype, int ndim, const int64_t *shape, const void *cond, int64_t cond_offset,

@@ -221,6 +221,14 @@ class Tensor:
     def __rmul__(self, o): return self._binary(o, "mul")
     def pow(self, o): return self._binary(o, "pow")
     def relu(self): return get_backend(self.device).unary(self, "relu")
+
+    def to(self, dtype: int) -> "Tensor":
+        """Tensor::to(ScalarType) (tensor/tensor.cpp:534-540): the tensor itself when the dtype already matches."""
+        return self if dtype == self.dtype else get_backend(self.device).to(self, dtype)
+
+    def assign(self, rhs: "Tensor") -> "Tensor":
+        get_backend(self.device).assign(self, rhs)
+        return self
     def sum(self, dim: int | None = None): return get_backend(self.device).sum(self, dim)
 
     def mean(self):
@@ -330,6 +338,46 @@ class BackendAMD:
         host = np.array([value], dtype=_NP_OF[dtype])
         _check(lib.ttamd_full(device.id, dtype, C.c_void_p(host.ctypes.data), numel, C.c_void_p(out.storage.ptr), None))
         return out
+
+    def to(self, t: Tensor, dtype: int) -> Tensor:
+        """BackendBase::to(tensor, dtype) (backend_base.h:74): element-wise static_cast into dense storage."""
+        out = Tensor.empty(t.shape, dtype, t.device)
+        _check(lib.ttamd_cast(t.device.id, t.dtype, dtype, t.dim(), self._i64(t.shape), C.c_void_p(t.storage.ptr), t.offset,
+                              self._i64(t.stride), C.c_void_p(out.storage.ptr), None))
+        return out
+
+    def assign(self, lhs: Tensor, rhs: Tensor) -> None:
+        """BackendBase::assign(lhs, rhs) (backend_base.h:78): writes rhs's elements through lhs's view."""
+        if lhs.shape != rhs.shape or lhs.dtype != rhs.dtype:
+            raise TTException("assign: operands must share shape and dtype")
+        _check(lib.ttamd_assign(lhs.device.id, lhs.dtype, lhs.dim(), self._i64(lhs.shape), C.c_void_p(lhs.storage.ptr),
+                                lhs.offset, self._i64(lhs.stride), C.c_void_p(rhs.storage.ptr), rhs.offset,
+                                self._i64(rhs.stride), None))
+
+    def pool2d(self, input: Tensor, op: str, kernel_size: int, stride: int, padding: int) -> Tensor:
+        """BackendBase::max_pool2d / min_pool2d / avg_pool2d (backend_base.h:286-311)."""
+        B, Cc, H, W = input.shape
+        Ho = (H + 2 * padding - kernel_size) // stride + 1
+        Wo = (W + 2 * padding - kernel_size) // stride + 1
+        rdtype = _capi.F32 if (op == "avg" and input.dtype not in (_capi.F32, _capi.F64)) else input.dtype
+        out = Tensor.empty((B, Cc, Ho, Wo), rdtype, input.device)
+        iv = input.view4()
+        _check(lib.ttamd_pool2d_forward(input.device.id, input.dtype, _capi.POOL[op], C.byref(iv), C.c_void_p(out.storage.ptr),
+                                        B, Cc, H, W, kernel_size, stride, padding, None))
+        return out
+
+    def pool2d_backward(self, grad_output: Tensor, input: Tensor, result: Tensor, op: str, kernel_size: int, stride: int,
+                        padding: int) -> Tensor:
+        """BackendBase::{max,min,avg}_pool2d_backward (backend_base.h:288-311)."""
+        B, Cc, H, W = input.shape
+        go, res = grad_output.contiguous(), result.contiguous()
+        gx = Tensor.empty(input.shape, input.dtype, input.device)
+        iv = input.view4()
+        _check(lib.ttamd_pool2d_backward(
+            input.device.id, input.dtype, _capi.POOL[op], C.c_void_p(go.storage.ptr + go.offset * go.itemsize), C.byref(iv),
+            C.c_void_p(res.storage.ptr + res.offset * res.itemsize), C.c_void_p(gx.storage.ptr), B, Cc, H, W, kernel_size,
+            stride, padding, None))
+        return gx
 
     def batched_matmul(self, lhs: Tensor, rhs: Tensor, bias: Tensor | None = None, bias_mode: int = 0,
                        relu: bool = False, out: Tensor | None = None, accumulate: bool = False) -> Tensor:
@@ -572,3 +620,37 @@ def conv2d_backward(grad_output: Tensor, input: Tensor, weight: Tensor, bias: Te
                     padding: int = 0):
     """TensorConv2d::backward (autograd/conv_ops.cpp:55-80) -> BackendBase::conv2d_backward."""
     return get_backend(input.device).conv2d_backward(grad_output, input, weight, bias, stride, padding)
+
+
+def _pool2d(input: Tensor, op: str, kernel_size: int, stride: int, padding: int) -> Tensor:
+    # argument checks of tinytensor::{max,min,avg}_pool2d (tensor/tensor.cpp:3169-3198)
+    if input.dtype == _capi.BOOL:
+        raise TTException(f"{op}_pool2d: bool tensors are not supported")
+    if input.dim() != 4:
+        raise TTException(f"Input shape {input.shape} expected to have 4 dimensions.")
+    if stride <= 0:
+        raise TTException(f"Stide of {stride} is expected to be positive.")
+    if padding < 0:
+        raise TTException(f"Padding of {padding} is expected to be non-negative.")
+    if input.size(2) + padding < kernel_size or input.size(3) + padding < kernel_size:
+        raise TTException(f"Kernel size {kernel_size} cannot be greater than input size ({input.size(2)}, {input.size(3)}) "
+                          f"+ padding {padding}")
+    return get_backend(input.device).pool2d(input, op, kernel_size, stride, padding)
+
+
+def max_pool2d(input: Tensor, kernel_size: int, stride: int, padding: int) -> Tensor:
+    return _pool2d(input, "max", kernel_size, stride, padding)
+
+
+def min_pool2d(input: Tensor, kernel_size: int, stride: int, padding: int) -> Tensor:
+    return _pool2d(input, "min", kernel_size, stride, padding)
+
+
+def avg_pool2d(input: Tensor, kernel_size: int, stride: int, padding: int) -> Tensor:
+    return _pool2d(input, "avg", kernel_size, stride, padding)
+
+
+def pool2d_backward(grad_output: Tensor, input: Tensor, result: Tensor, op: str, kernel_size: int, stride: int,
+                    padding: int) -> Tensor:
+    """Tensor{Max,Min,Avg}Pool2d::backward (autograd/conv_ops.cpp:100-190) -> BackendBase::*_pool2d_backward."""
+    return get_backend(input.device).pool2d_backward(grad_output, input, result, op, kernel_size, stride, padding)
