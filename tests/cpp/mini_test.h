@@ -56,10 +56,10 @@ inline int run_all(int argc, char **argv) {
     static void MINI_CAT(test_fn_, __LINE__)();                                \
     static mini::Registrar MINI_CAT(test_reg_, __LINE__)(name, MINI_CAT(test_fn_, __LINE__)); \
     static void MINI_CAT(test_fn_, __LINE__)()
-#define CHECK(cond)                                                             \
+#define CHECK(...)                                                              \
     do {                                                                        \
-        if (!(cond)) {                                                          \
-            std::printf("  %s:%d: CHECK(%s) failed\n", __FILE__, __LINE__, #cond); \
+        if (!(__VA_ARGS__)) {                                                   \
+            std::printf("  %s:%d: CHECK(%s) failed\n", __FILE__, __LINE__, #__VA_ARGS__); \
             ++mini::failures();                                                 \
         }                                                                       \
     } while (0)

@@ -1,0 +1,242 @@
+// test_ops_amd.cpp — the operations around the GEMMs on the AMD device, checked against plain host loops in the
+// style of the reference's tests/test_binary.cpp, test_reduce.cpp, test_to.cpp and the pooling cases of
+// tests/test_conv.cpp:186-278 (whose expected values come from a naive window loop here instead of libtorch):
+// elementwise binary / unary with broadcasting, where, sum, full, to(dtype), assign through views, max / min / avg
+// pooling forward and backward, seeded uniform draws and nn::Linear's default initialisation.
+#include "mini_test.h"
+
+#include <limits>
+
+using namespace tt_amd;
+
+namespace {
+template <typename T>
+std::vector<T> pattern(int n, int mod, int shift) {
+    std::vector<T> v;
+    for (int i = 0; i < n; ++i) v.push_back(static_cast<T>((i * 7 + 3) % mod + shift));
+    return v;
+}
+template <typename T, typename R, typename F>
+std::vector<R> pool_naive(const std::vector<T> &X, int B, int C, int H, int W, int K, int S, int P, R init, F fold) {
+    const int Ho = (H + 2 * P - K) / S + 1, Wo = (W + 2 * P - K) / S + 1;
+    std::vector<R> out(static_cast<std::size_t>(B) * C * Ho * Wo);
+    for (int bc = 0; bc < B * C; ++bc)
+        for (int h = 0; h < Ho; ++h)
+            for (int w = 0; w < Wo; ++w) {
+                R acc = init;
+                for (int p = 0; p < K; ++p)
+                    for (int q = 0; q < K; ++q) {
+                        const int hi = S * h + p - P, wi = S * w + q - P;
+                        const R x = (hi < 0 || wi < 0 || hi >= H || wi >= W) ? init : static_cast<R>(X[(static_cast<std::size_t>(bc) * H + hi) * W + wi]);
+                        acc = fold(x, acc);
+                    }
+                out[(static_cast<std::size_t>(bc) * Ho + h) * Wo + w] = acc;
+            }
+    return out;
+}
+}  // namespace
+
+TEST_CASE("Binary ops with broadcasting") {
+    auto test = []<typename T>(Device device) {
+        const int R = 37, Cn = 19;
+        const auto a = pattern<T>(R * Cn, 11, 1), b = pattern<T>(Cn, 5, 1);
+        const Tensor A(a, {R, Cn}, device), Bv(b, {Cn}, device);
+        std::vector<T> sum_, dif, prod, quot, mx;
+        std::vector<bool> less;
+        for (int i = 0; i < R * Cn; ++i) {
+            const T x = a[static_cast<std::size_t>(i)], y = b[static_cast<std::size_t>(i % Cn)];
+            sum_.push_back(static_cast<T>(x + y));
+            dif.push_back(static_cast<T>(x - y));
+            prod.push_back(static_cast<T>(x * y));
+            quot.push_back(static_cast<T>(x / y));
+            mx.push_back(x > y ? x : y);
+            less.push_back(x < y);
+        }
+        CHECK((A + Bv).template to_vec<T>() == sum_);
+        CHECK((A - Bv).template to_vec<T>() == dif);
+        CHECK((A * Bv).template to_vec<T>() == prod);
+        CHECK((A / Bv).template to_vec<T>() == quot);
+        CHECK(maximum(A, Bv).template to_vec<T>() == mx);
+        const Tensor L = A < Bv;
+        CHECK(L.dtype() == kBool);
+        CHECK(L.template to_vec<bool>() == less);
+        // a transposed view as the left operand
+        const Tensor At = A.permute({1, 0});
+        const auto t = (At + At).template to_vec<T>();
+        bool ok = true;
+        for (int c = 0; c < Cn; ++c)
+            for (int r = 0; r < R; ++r) ok = ok && t[static_cast<std::size_t>(c * R + r)] == static_cast<T>(2 * a[static_cast<std::size_t>(r * Cn + c)]);
+        CHECK(ok);
+        CHECK_THROWS_AS(std::ignore = A + Tensor(pattern<T>(R, 5, 1), {R}, device), TTException);  // not broadcastable
+    };
+    runner_all_except_bool(test);
+}
+
+TEST_CASE("Unary ops, where, sum, full") {
+    auto test = []<typename T>(Device device) {
+        const int N = 1000;
+        std::vector<T> a;
+        for (int i = 0; i < N; ++i) a.push_back(static_cast<T>((i % 13) - 6) / T(4));
+        const Tensor A(a, {10, 100}, device);
+        std::vector<T> r, e;
+        for (T x : a) {
+            r.push_back(x > T(0) ? x : T(0));
+            e.push_back(std::exp(x));
+        }
+        CHECK(relu(A).template to_vec<T>() == r);
+        CHECK(allclose(get_backend(device)->exp(A).template to_vec<T>(), e, 1e-6, 1e-7));
+        // relu backward as the reference writes it: where(input > 0, grad, 0) (autograd/unary_ops.cpp:568-573)
+        const Tensor zero = full(T(0), A.shape(), device), grad = full(T(2.5), A.shape(), device);
+        const auto g = where(A > zero, grad, zero).template to_vec<T>();
+        bool ok = true;
+        for (int i = 0; i < N; ++i) ok = ok && g[static_cast<std::size_t>(i)] == (a[static_cast<std::size_t>(i)] > T(0) ? T(2.5) : T(0));
+        CHECK(ok);
+        // sums of multiples of 1/4 are exact in any order
+        double total = 0;
+        for (T x : a) total += static_cast<double>(x);
+        CHECK(A.sum().template to_vec<T>() == std::vector<T>{static_cast<T>(total)});
+        std::vector<T> cols(100, T(0)), rows(10, T(0));
+        for (int i = 0; i < 10; ++i)
+            for (int j = 0; j < 100; ++j) {
+                cols[static_cast<std::size_t>(j)] += a[static_cast<std::size_t>(i * 100 + j)];
+                rows[static_cast<std::size_t>(i)] += a[static_cast<std::size_t>(i * 100 + j)];
+            }
+        CHECK(A.sum(0).template to_vec<T>() == cols);
+        CHECK(A.sum(-1).template to_vec<T>() == rows);
+    };
+    runner_floating_point(test);
+}
+
+TEST_CASE("To") {
+    auto test = []<typename T>(Device device) {
+        const auto a = pattern<T>(300, 100, 0);
+        const Tensor A(a, {3, 100}, device);
+        auto expect = [&]<typename R>(R) {
+            std::vector<R> e;
+            for (T x : a) e.push_back(static_cast<R>(x));
+            return e;
+        };
+        CHECK(A.to(kU8).template to_vec<uint8_t>() == expect(uint8_t{}));
+        CHECK(A.to(kI16).template to_vec<int16_t>() == expect(int16_t{}));
+        CHECK(A.to(kI32).template to_vec<int32_t>() == expect(int32_t{}));
+        CHECK(A.to(kI64).template to_vec<int64_t>() == expect(int64_t{}));
+        CHECK(A.to(kF32).template to_vec<float>() == expect(float{}));
+        CHECK(A.to(kF64).template to_vec<double>() == expect(double{}));
+        std::vector<bool> eb;
+        for (T x : a) eb.push_back(x != T(0));
+        CHECK(A.to(kBool).template to_vec<bool>() == eb);
+        CHECK(A.to(A.dtype()).storage() == A.storage());  // same dtype: the tensor itself (tensor.cpp:536-538)
+    };
+    runner_all_except_bool(test);
+}
+
+TEST_CASE("Assign through views") {
+    auto test = []<typename T>(Device device) {
+        auto base = pattern<T>(60, 50, 0);
+        const auto rhs = pattern<T>(12, 9, 60);
+        Tensor Bt(base, {6, 10}, device);
+        Tensor window(Bt.storage(), Bt.dtype(), Shape({4, 3}), Shape({10, 2}), 12, device);  // rows 1..4, columns 2,4,6
+        window.assign(Tensor(rhs, {3, 4}, device).permute({1, 0}));
+        for (int i = 0; i < 4; ++i)
+            for (int j = 0; j < 3; ++j) base[static_cast<std::size_t>((1 + i) * 10 + 2 + 2 * j)] = rhs[static_cast<std::size_t>(j * 4 + i)];
+        CHECK(Bt.template to_vec<T>() == base);
+        CHECK_THROWS_AS(window.assign(Tensor(rhs, {12}, device)), TTException);
+    };
+    runner_all_except_bool(test);
+}
+
+TEST_CASE("Pool2D Forward") {
+    auto test = []<typename T>(Device device) {
+        // tests/test_conv.cpp:186-278: B4 C128 68x28, k3 s2 p1
+        const int B = 4, C = 128, H = 68, W = 28, K = 3, S = 2, P = 1;
+        std::vector<T> x;
+        for (int i = 0; i < B * C * H * W; ++i) x.push_back(static_cast<T>((i * 2654435761u >> 7) % 97) - T(40 * (std::is_signed_v<T> ? 1 : 0)));
+        const Tensor X(x, {B, C, H, W}, device);
+        using L = std::numeric_limits<T>;
+        CHECK(max_pool2d(X, K, S, P).template to_vec<T>() ==
+              pool_naive<T, T>(x, B, C, H, W, K, S, P, L::lowest(), [](T v, T acc) { return v > acc ? v : acc; }));
+        CHECK(min_pool2d(X, K, S, P).template to_vec<T>() ==
+              pool_naive<T, T>(x, B, C, H, W, K, S, P, L::max(), [](T v, T acc) { return v < acc ? v : acc; }));
+        using R = std::conditional_t<std::is_floating_point_v<T>, T, float>;
+        const R n = static_cast<R>(K * K);
+        const Tensor avg = avg_pool2d(X, K, S, P);
+        CHECK(avg.dtype() == to_scalar<R>::type);
+        CHECK(avg.shape() == Shape({B, C, 34, 14}));
+        CHECK(avg.template to_vec<R>() == pool_naive<T, R>(x, B, C, H, W, K, S, P, R(0), [n](R v, R acc) { return (v / n) + acc; }));
+    };
+    runner_all_except_bool(test);
+    CHECK_THROWS_AS(std::ignore = max_pool2d(Tensor(std::vector<bool>(16, true), {1, 1, 4, 4}, kAMD), 2, 2, 0), TTException);
+    CHECK_THROWS_AS(std::ignore = avg_pool2d(Tensor(std::vector<float>(16, 1.f), {1, 4, 4}, kAMD), 2, 2, 0), TTException);
+    CHECK_THROWS_AS(std::ignore = min_pool2d(Tensor(std::vector<float>(16, 1.f), {1, 1, 4, 4}, kAMD), 6, 1, 1), TTException);
+}
+
+TEST_CASE("Pool2D Backward") {
+    auto test = []<typename T>(Device device) {
+        const int B = 2, C = 3, H = 9, W = 8, K = 3, S = 2, P = 1;
+        const int Ho = (H + 2 * P - K) / S + 1, Wo = (W + 2 * P - K) / S + 1;
+        std::vector<T> x, g;
+        for (int i = 0; i < B * C * H * W; ++i) x.push_back(static_cast<T>((i * 5) % 4));  // ties
+        for (int i = 0; i < B * C * Ho * Wo; ++i) g.push_back(static_cast<T>(i % 9 - 4));
+        const Tensor X(x, {B, C, H, W}, device), G(g, {B, C, Ho, Wo}, device);
+        for (int op = 0; op < 3; ++op) {
+            const Tensor res = op == 0 ? max_pool2d(X, K, S, P) : op == 1 ? min_pool2d(X, K, S, P) : avg_pool2d(X, K, S, P);
+            const Tensor gx = op == 0 ? max_pool2d_backward(G, X, res, K, S, P)
+                              : op == 1 ? min_pool2d_backward(G, X, res, K, S, P)
+                                        : avg_pool2d_backward(G, X, res, K, S, P);
+            const auto r = res.template to_vec<T>();
+            std::vector<T> want(x.size(), T(0));  // the reference's scatter loop (cpu/kernel/conv.hpp:171-275)
+            for (int bc = 0; bc < B * C; ++bc)
+                for (int h = 0; h < Ho; ++h)
+                    for (int w = 0; w < Wo; ++w) {
+                        const std::size_t ir = (static_cast<std::size_t>(bc) * Ho + h) * Wo + w;
+                        T count = op == 2 ? static_cast<T>(K * K) : T(0);
+                        auto each = [&](auto &&f) {
+                            for (int p = 0; p < K; ++p)
+                                for (int q = 0; q < K; ++q) {
+                                    const int hi = S * h + p - P, wi = S * w + q - P;
+                                    if (hi < 0 || wi < 0 || hi >= H || wi >= W) continue;
+                                    const std::size_t ii = (static_cast<std::size_t>(bc) * H + hi) * W + wi;
+                                    if (op == 2 || x[ii] == r[ir]) f(ii);
+                                }
+                        };
+                        if (op != 2) each([&](std::size_t) { count += T(1); });
+                        const T share = g[ir] / count;
+                        each([&](std::size_t ii) { want[ii] += share; });
+                    }
+            CHECK(gx.template to_vec<T>() == want);
+        }
+    };
+    runner_floating_point(test);
+}
+
+TEST_CASE("Seeded draws and Linear default init") {
+    Generator g1(42), g2(42), g3(43);
+    const Tensor a = uniform_real(-2.0, 3.0, {1000, 7}, g1), b = uniform_real(-2.0, 3.0, {1000, 7}, g2), c = uniform_real(-2.0, 3.0, {1000, 7}, g3);
+    const auto va = a.to_vec<float>(), vb = b.to_vec<float>(), vc = c.to_vec<float>();
+    CHECK(va == vb);
+    CHECK(va != vc);
+    CHECK(g1.state == g2.state);
+    double mean = 0;
+    bool in_range = true;
+    for (float v : va) {
+        mean += v;
+        in_range = in_range && v >= -2.0f && v < 3.0f;
+    }
+    CHECK(in_range);
+    CHECK(std::abs(mean / static_cast<double>(va.size()) - 0.5) < 0.06);
+    CHECK_THROWS_AS(std::ignore = uniform_real(1.0, 1.0, {4}, g1), TTException);
+    // nn::Linear(in, out): weight [in,out] ~ U(+-sqrt(3/in)), bias ~ U(+-1/sqrt(in)), drawn in that order
+    Generator gl(7), gr(7);
+    const nn::Linear layer(256, 64, true, gl);
+    CHECK(layer.weight.shape() == Shape({256, 64}));
+    CHECK(layer.bias->shape() == Shape({64}));
+    const double bw = std::sqrt(3.0 / 256.0), bb = 1.0 / 16.0;
+    CHECK(layer.weight.to_vec<float>() == uniform_real(-bw, bw, {256, 64}, gr).to_vec<float>());
+    CHECK(layer.bias->to_vec<float>() == uniform_real(-bb, bb, {64}, gr).to_vec<float>());
+    const Tensor X = uniform_real(-1.0, 1.0, {8, 256}, gr);
+    const Tensor Y = layer.forward(X);
+    CHECK(Y.shape() == Shape({8, 64}));
+    CHECK(allclose(Y.to_vec<float>(), (matmul(X, layer.weight) + *layer.bias).to_vec<float>(), 1e-5, 1e-6));
+}
+
+int main(int argc, char **argv) { return mini::run_all(argc, argv); }

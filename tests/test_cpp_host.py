@@ -8,7 +8,7 @@ import pytest
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 CPP = os.path.join(ROOT, "tests", "cpp")
-BINARIES = ["test_matmul_amd", "test_conv_amd"]
+BINARIES = ["test_matmul_amd", "test_conv_amd", "test_ops_amd"]
 
 
 def ensure_built():

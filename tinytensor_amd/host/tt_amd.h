@@ -9,7 +9,11 @@
 //   matmul(lhs, rhs)                                         tinytensor/tensor/tensor.cpp:2390-2484
 //   matmul backward (dA = dC.B^T, dB = A^T.dC on views)       tinytensor/autograd/binary_ops.cpp:165-179
 //   conv2d / conv2d_backward                                 tinytensor/tensor/tensor.cpp:3089-3167, backend_base.h:269-284
-//   nn::Linear                                               tinytensor/nn/linear.cpp:20-50
+//   nn::Linear (+ default initialisation)                    tinytensor/nn/linear.cpp:20-50, nn/init.cpp:30-52,106-112
+//   add/sub/mul/div/pow/..., relu/exp/..., where, sum, full,   tinytensor/tensor/backend_base.h:51-263 (operands are
+//   to(dtype), assign                                         broadcast with expand() views first, include/tt/tensor.h:600)
+//   max/min/avg_pool2d (+ backward)                          tinytensor/tensor/tensor.cpp:3169-3198, backend_base.h:286-311
+//   Generator, uniform_real, normal                          tinytensor/tensor/random.cpp:26-63, tensor.cpp:1773-1781
 //   BackendAMD (the BackendBase methods on the path)         tinytensor/tensor/backend_base.h:23-322
 //   TTException                                              include/tt/exception.h:15-25
 // All arithmetic runs in libttamd.so; there is no CPU fallback.
@@ -17,6 +21,7 @@
 #define TT_AMD_HOST_H_
 
 #include <algorithm>
+#include <cmath>
 #include <cstdint>
 #include <cstdlib>
 #include <exception>
@@ -210,6 +215,11 @@ public:
     }
     template <typename T>
     [[nodiscard]] auto to_vec() const -> std::vector<T>;  // dense host copy of this view (tensor.cpp:555)
+    [[nodiscard]] auto to(ScalarType dtype) const -> Tensor;  // tensor.cpp:534-540
+    [[nodiscard]] auto relu() const -> Tensor;
+    [[nodiscard]] auto sum() const -> Tensor;
+    [[nodiscard]] auto sum(int dim) const -> Tensor;
+    auto assign(const Tensor &rhs) -> Tensor &;  // writes rhs's elements through this view
 
     static auto dense_stride(const Shape &shape) -> Shape {
         std::vector<int> st(static_cast<std::size_t>(shape.ndim()), 1);
@@ -290,6 +300,135 @@ public:
         if (gb) grad_bias = Tensor(gb, input.dtype(), Shape({O}), input.device());
         return {Tensor(gx, input.dtype(), input.shape(), input.device()), Tensor(gw, input.dtype(), weight.shape(), input.device()), grad_bias};
     }
+    // ---- elementwise set (backend_base.h:51-263): operands share one shape; results are dense ----
+    [[nodiscard]] auto binary(const Tensor &lhs, const Tensor &rhs, ttamd_binary_op op) const -> Tensor {
+        if (!(lhs.shape() == rhs.shape()) || lhs.dtype() != rhs.dtype()) throw TTException("binary op: operands must share shape and dtype");
+        const ScalarType rt = op >= TTAMD_BIN_LT ? kBool : lhs.dtype();
+        auto out = std::make_shared<StorageAMD>(static_cast<std::size_t>(lhs.numel()) * dtype_size(rt), lhs.device().id);
+        const auto sh = i64(lhs.shape()), ls = i64(lhs.stride()), rs = i64(rhs.stride());
+        check(ttamd_binary(lhs.device().id, static_cast<ttamd_dtype>(lhs.dtype()), op, lhs.dim(), sh.data(), lhs.storage()->ptr_, lhs.offset(),
+                           ls.data(), rhs.storage()->ptr_, rhs.offset(), rs.data(), out->ptr_, nullptr));
+        return {out, rt, lhs.shape(), lhs.device()};
+    }
+#define TT_AMD_BINARY(NAME, CODE) \
+    [[nodiscard]] auto NAME(const Tensor &lhs, const Tensor &rhs) const -> Tensor { return binary(lhs, rhs, CODE); }
+    TT_AMD_BINARY(add, TTAMD_BIN_ADD)
+    TT_AMD_BINARY(sub, TTAMD_BIN_SUB)
+    TT_AMD_BINARY(mul, TTAMD_BIN_MUL)
+    TT_AMD_BINARY(div, TTAMD_BIN_DIV)
+    TT_AMD_BINARY(pow, TTAMD_BIN_POW)
+    TT_AMD_BINARY(maximum, TTAMD_BIN_MAXIMUM)
+    TT_AMD_BINARY(minimum, TTAMD_BIN_MINIMUM)
+    TT_AMD_BINARY(lt, TTAMD_BIN_LT)
+    TT_AMD_BINARY(le, TTAMD_BIN_LE)
+    TT_AMD_BINARY(gt, TTAMD_BIN_GT)
+    TT_AMD_BINARY(ge, TTAMD_BIN_GE)
+    TT_AMD_BINARY(eq, TTAMD_BIN_EQ)
+    TT_AMD_BINARY(ne, TTAMD_BIN_NE)
+#undef TT_AMD_BINARY
+    [[nodiscard]] auto unary(const Tensor &t, ttamd_unary_op op) const -> Tensor {
+        auto out = std::make_shared<StorageAMD>(static_cast<std::size_t>(t.numel()) * dtype_size(t.dtype()), t.device().id);
+        const auto sh = i64(t.shape()), st = i64(t.stride());
+        check(ttamd_unary(t.device().id, static_cast<ttamd_dtype>(t.dtype()), op, t.dim(), sh.data(), t.storage()->ptr_, t.offset(), st.data(),
+                          out->ptr_, nullptr));
+        return {out, t.dtype(), t.shape(), t.device()};
+    }
+#define TT_AMD_UNARY(NAME, CODE) \
+    [[nodiscard]] auto NAME(const Tensor &t) const -> Tensor { return unary(t, CODE); }
+    TT_AMD_UNARY(relu, TTAMD_UN_RELU)
+    TT_AMD_UNARY(negate, TTAMD_UN_NEGATE)
+    TT_AMD_UNARY(abs, TTAMD_UN_ABS)
+    TT_AMD_UNARY(sqrt, TTAMD_UN_SQRT)
+    TT_AMD_UNARY(exp, TTAMD_UN_EXP)
+    TT_AMD_UNARY(log, TTAMD_UN_LOG)
+    TT_AMD_UNARY(sigmoid, TTAMD_UN_SIGMOID)
+    TT_AMD_UNARY(tanh, TTAMD_UN_TANH)
+#undef TT_AMD_UNARY
+    [[nodiscard]] auto where(const Tensor &cond, const Tensor &lhs, const Tensor &rhs) const -> Tensor {
+        if (cond.dtype() != kBool || !(cond.shape() == lhs.shape()) || !(lhs.shape() == rhs.shape()) || lhs.dtype() != rhs.dtype())
+            throw TTException("where: cond must be bool and all operands must share one shape");
+        auto out = std::make_shared<StorageAMD>(static_cast<std::size_t>(lhs.numel()) * dtype_size(lhs.dtype()), lhs.device().id);
+        const auto sh = i64(lhs.shape()), cs = i64(cond.stride()), ls = i64(lhs.stride()), rs = i64(rhs.stride());
+        check(ttamd_where(lhs.device().id, static_cast<ttamd_dtype>(lhs.dtype()), lhs.dim(), sh.data(), cond.storage()->ptr_, cond.offset(),
+                          cs.data(), lhs.storage()->ptr_, lhs.offset(), ls.data(), rhs.storage()->ptr_, rhs.offset(), rs.data(), out->ptr_,
+                          nullptr));
+        return {out, lhs.dtype(), lhs.shape(), lhs.device()};
+    }
+    // sum(tensor) -> one element; sum(tensor, dim) -> that dimension removed (backend_base.h:148-149)
+    [[nodiscard]] auto sum(const Tensor &t, int dim = -1) const -> Tensor {
+        std::vector<int> osh;
+        if (dim < 0) osh = {1};
+        else
+            for (int d = 0; d < t.dim(); ++d)
+                if (d != dim) osh.push_back(t.size(d));
+        const Shape out_shape{osh};
+        auto out = std::make_shared<StorageAMD>(static_cast<std::size_t>(out_shape.numel()) * dtype_size(t.dtype()), t.device().id);
+        const auto sh = i64(t.shape()), st = i64(t.stride());
+        check(ttamd_sum(t.device().id, static_cast<ttamd_dtype>(t.dtype()), t.dim(), sh.data(), t.storage()->ptr_, t.offset(), st.data(), dim,
+                        out->ptr_, nullptr));
+        return {out, t.dtype(), out_shape, t.device()};
+    }
+    template <typename T>
+    [[nodiscard]] auto full(T value, int numel, Device device) const -> Tensor {  // backend_base.h:51
+        using S = std::conditional_t<std::is_same_v<T, bool>, uint8_t, T>;
+        const S v = static_cast<S>(value);
+        auto out = std::make_shared<StorageAMD>(static_cast<std::size_t>(numel) * sizeof(S), device.id);
+        check(ttamd_full(device.id, static_cast<ttamd_dtype>(to_scalar<T>::type), &v, numel, out->ptr_, nullptr));
+        return {out, to_scalar<T>::type, Shape({numel}), device};
+    }
+    [[nodiscard]] auto to(const Tensor &t, ScalarType dtype) const -> Tensor {  // backend_base.h:74
+        auto out = std::make_shared<StorageAMD>(static_cast<std::size_t>(t.numel()) * dtype_size(dtype), t.device().id);
+        const auto sh = i64(t.shape()), st = i64(t.stride());
+        check(ttamd_cast(t.device().id, static_cast<ttamd_dtype>(t.dtype()), static_cast<ttamd_dtype>(dtype), t.dim(), sh.data(),
+                         t.storage()->ptr_, t.offset(), st.data(), out->ptr_, nullptr));
+        return {out, dtype, t.shape(), t.device()};
+    }
+    void assign(Tensor &lhs, const Tensor &rhs) const {  // backend_base.h:78
+        if (!(lhs.shape() == rhs.shape()) || lhs.dtype() != rhs.dtype()) throw TTException("assign: operands must share shape and dtype");
+        const auto sh = i64(lhs.shape()), ls = i64(lhs.stride()), rs = i64(rhs.stride());
+        check(ttamd_assign(lhs.device().id, static_cast<ttamd_dtype>(lhs.dtype()), lhs.dim(), sh.data(), lhs.storage()->ptr_, lhs.offset(),
+                           ls.data(), rhs.storage()->ptr_, rhs.offset(), rs.data(), nullptr));
+    }
+    // ---- pooling (backend_base.h:286-311) ----
+    [[nodiscard]] auto pool2d(const Tensor &input, ttamd_pool_op op, int kernel_size, int stride, int padding) const -> Tensor {
+        const int B = input.size(0), C = input.size(1), H = input.size(2), W = input.size(3);
+        const int Ho = (H + 2 * padding - kernel_size) / stride + 1, Wo = (W + 2 * padding - kernel_size) / stride + 1;
+        const bool is_float = input.dtype() == kF32 || input.dtype() == kF64;
+        const ScalarType rt = (op == TTAMD_POOL_AVG && !is_float) ? kF32 : input.dtype();  // common/reduce.h:63-69
+        auto out = std::make_shared<StorageAMD>(static_cast<std::size_t>(std::max(B * C * Ho * Wo, 0)) * dtype_size(rt), input.device().id);
+        const ttamd_view4 iv = view4(input);
+        check(ttamd_pool2d_forward(input.device().id, static_cast<ttamd_dtype>(input.dtype()), op, &iv, out->ptr_, B, C, H, W, kernel_size,
+                                   stride, padding, nullptr));
+        return {out, rt, Shape({B, C, Ho, Wo}), input.device()};
+    }
+    [[nodiscard]] auto pool2d_backward(const Tensor &grad_output, const Tensor &input, const Tensor &result, ttamd_pool_op op, int kernel_size,
+                                       int stride, int padding) const -> Tensor {
+        const Tensor go = grad_output.contiguous(), res = result.contiguous();
+        auto gx = std::make_shared<StorageAMD>(static_cast<std::size_t>(input.numel()) * dtype_size(input.dtype()), input.device().id);
+        const ttamd_view4 iv = view4(input);
+        check(ttamd_pool2d_backward(input.device().id, static_cast<ttamd_dtype>(input.dtype()), op, go.data_ptr(), &iv, res.data_ptr(), gx->ptr_,
+                                    input.size(0), input.size(1), input.size(2), input.size(3), kernel_size, stride, padding, nullptr));
+        return {gx, input.dtype(), input.shape(), input.device()};
+    }
+#define TT_AMD_POOL(NAME, CODE)                                                                                                    \
+    [[nodiscard]] auto NAME(const Tensor &input, int kernel_size, int stride, int padding) const -> Tensor {                      \
+        return pool2d(input, CODE, kernel_size, stride, padding);                                                                  \
+    }                                                                                                                              \
+    [[nodiscard]] auto NAME##_backward(const Tensor &grad_output, const Tensor &input, const Tensor &result, int kernel_size,     \
+                                       int stride, int padding) const -> Tensor {                                                 \
+        return pool2d_backward(grad_output, input, result, CODE, kernel_size, stride, padding);                                    \
+    }
+    TT_AMD_POOL(max_pool2d, TTAMD_POOL_MAX)
+    TT_AMD_POOL(min_pool2d, TTAMD_POOL_MIN)
+    TT_AMD_POOL(avg_pool2d, TTAMD_POOL_AVG)
+#undef TT_AMD_POOL
+    // ---- seeded draws (backend_base.h:96-103 with scalar parameters): dist 0 uniform_real(low, high), 1 normal(mu, std) ----
+    [[nodiscard]] auto random_fill(int dist, double p0, double p1, const Shape &shape, uint64_t &generator_state, ScalarType dtype,
+                                   Device device) const -> Tensor {
+        auto out = std::make_shared<StorageAMD>(static_cast<std::size_t>(shape.numel()) * dtype_size(dtype), device.id);
+        check(ttamd_random_fill(device.id, static_cast<ttamd_dtype>(dtype), dist, p0, p1, &generator_state, shape.numel(), out->ptr_, nullptr));
+        return {out, dtype, shape, device};
+    }
     [[nodiscard]] auto current_memory_allocated(int device_id) const -> uint64_t {
         uint64_t cur = 0, tot = 0;
         check(ttamd_memory_allocated(device_id, &cur, &tot));
@@ -306,6 +445,11 @@ public:
         return n;
     }
 
+    static auto i64(const Shape &s) -> std::vector<int64_t> {
+        std::vector<int64_t> v(s.to_vec().begin(), s.to_vec().end());
+        if (v.empty()) v.push_back(1);  // rank 0: the C ABI wants non-NULL arrays
+        return v;
+    }
     static auto view3(const Tensor &t) -> ttamd_view3 {
         return {t.storage()->ptr_, t.offset(), {t.stride()[0], t.stride()[1], t.stride()[2]}};
     }
@@ -337,7 +481,7 @@ template <typename T>
 auto Tensor::to_vec() const -> std::vector<T> {
     if (to_scalar<T>::type != dtype_) throw TTException("to_vec: element type does not match the tensor dtype");
     const Tensor dense = contiguous();  // callers clone first (tensor.cpp:555), then the whole storage comes back
-    std::vector<T> whole;
+    std::vector<std::conditional_t<std::is_same_v<T, bool>, uint8_t, T>> whole;  // bool travels as bytes (tensor.cpp:558-564)
     get_backend(device_)->to_vec(dense, whole);
     return {whole.begin() + dense.offset(), whole.begin() + dense.offset() + dense.numel()};
 }
@@ -393,6 +537,106 @@ inline auto conv2d_backward(const Tensor &grad_output, const Tensor &input, cons
     return get_backend(input.device())->conv2d_backward(grad_output, input, weight, bias, stride, padding);
 }
 
+inline auto Tensor::to(ScalarType dtype) const -> Tensor { return dtype == dtype_ ? *this : get_backend(device_)->to(*this, dtype); }
+inline auto Tensor::relu() const -> Tensor { return get_backend(device_)->relu(*this); }
+inline auto Tensor::sum() const -> Tensor { return get_backend(device_)->sum(*this); }
+inline auto Tensor::sum(int dim) const -> Tensor { return get_backend(device_)->sum(*this, dim < 0 ? dim + this->dim() : dim); }
+inline auto Tensor::assign(const Tensor &rhs) -> Tensor & {
+    get_backend(device_)->assign(*this, rhs);
+    return *this;
+}
+
+// Right-aligned broadcasting through unsqueeze + expand views (no data movement), then one shape for the backend.
+inline auto broadcast_tensors(Tensor a, Tensor b) -> std::pair<Tensor, Tensor> {
+    while (a.dim() < b.dim()) a = a.unsqueeze(0);
+    while (b.dim() < a.dim()) b = b.unsqueeze(0);
+    std::vector<int> sh;
+    for (int d = 0; d < a.dim(); ++d) {
+        if (a.size(d) != b.size(d) && a.size(d) != 1 && b.size(d) != 1) throw TTException("Tensors are not broadcastable");
+        sh.push_back(std::max(a.size(d), b.size(d)));
+    }
+    return {a.expand(Shape(sh)), b.expand(Shape(sh))};
+}
+#define TT_AMD_FREE_BINARY(NAME)                                                                 \
+    inline auto NAME(const Tensor &lhs, const Tensor &rhs) -> Tensor {                           \
+        if (lhs.dtype() != rhs.dtype()) throw TTException(#NAME ": operands must share a dtype"); \
+        const auto [l, r] = broadcast_tensors(lhs, rhs);                                         \
+        return get_backend(lhs.device())->NAME(l, r);                                            \
+    }
+TT_AMD_FREE_BINARY(add)
+TT_AMD_FREE_BINARY(sub)
+TT_AMD_FREE_BINARY(mul)
+TT_AMD_FREE_BINARY(div)
+TT_AMD_FREE_BINARY(pow)
+TT_AMD_FREE_BINARY(maximum)
+TT_AMD_FREE_BINARY(minimum)
+TT_AMD_FREE_BINARY(lt)
+TT_AMD_FREE_BINARY(le)
+TT_AMD_FREE_BINARY(gt)
+TT_AMD_FREE_BINARY(ge)
+TT_AMD_FREE_BINARY(eq)
+TT_AMD_FREE_BINARY(ne)
+#undef TT_AMD_FREE_BINARY
+inline auto operator+(const Tensor &a, const Tensor &b) -> Tensor { return add(a, b); }
+inline auto operator-(const Tensor &a, const Tensor &b) -> Tensor { return sub(a, b); }
+inline auto operator*(const Tensor &a, const Tensor &b) -> Tensor { return mul(a, b); }
+inline auto operator/(const Tensor &a, const Tensor &b) -> Tensor { return div(a, b); }
+inline auto operator<(const Tensor &a, const Tensor &b) -> Tensor { return lt(a, b); }
+inline auto operator>(const Tensor &a, const Tensor &b) -> Tensor { return gt(a, b); }
+inline auto relu(const Tensor &t) -> Tensor { return t.relu(); }
+inline auto where(const Tensor &cond, const Tensor &lhs, const Tensor &rhs) -> Tensor {
+    const auto [l, r] = broadcast_tensors(lhs, rhs);
+    const auto [c, l2] = broadcast_tensors(cond, l);
+    const auto [c2, r2] = broadcast_tensors(c, r);
+    return get_backend(lhs.device())->where(c2, l2, r2);
+}
+// tinytensor::full: a one-element storage expanded to `shape` (stride 0), like Tensor(Scalar).expand().
+template <typename T>
+inline auto full(T value, const Shape &shape, Device device = kAMD) -> Tensor {
+    const Tensor one = get_backend(device)->full(value, 1, device);
+    return {one.storage(), one.dtype(), shape, Shape(std::vector<int>(static_cast<std::size_t>(shape.ndim()), 0)), 0, device};
+}
+
+// tinytensor::{max,min,avg}_pool2d argument checks (tensor.cpp:3169-3198).
+#define TT_AMD_FREE_POOL(NAME)                                                                                                        \
+    inline auto NAME(const Tensor &input, int kernel_size, int stride, int padding) -> Tensor {                                      \
+        if (input.dtype() == kBool) throw TTException(#NAME " does not support boolean tensors");                                     \
+        if (input.dim() != 4) throw TTException("Input shape expected to have 4 dimensions.");                                        \
+        if (stride <= 0) throw TTException("Stide is expected to be positive.");                                                      \
+        if (padding < 0) throw TTException("Padding is expected to be non-negative.");                                                \
+        if (input.size(2) + padding < kernel_size || input.size(3) + padding < kernel_size)                                           \
+            throw TTException("Kernel size cannot be greater than input size + padding");                                            \
+        return get_backend(input.device())->NAME(input, kernel_size, stride, padding);                                                \
+    }                                                                                                                                 \
+    inline auto NAME##_backward(const Tensor &grad_output, const Tensor &input, const Tensor &result, int kernel_size, int stride,    \
+                                int padding) -> Tensor {                                                                              \
+        return get_backend(input.device())->NAME##_backward(grad_output, input, result, kernel_size, stride, padding);                \
+    }
+TT_AMD_FREE_POOL(max_pool2d)
+TT_AMD_FREE_POOL(min_pool2d)
+TT_AMD_FREE_POOL(avg_pool2d)
+#undef TT_AMD_FREE_POOL
+
+// tinytensor::Generator (tensor/random.cpp:46-63): state = splitmix64(seed); the device draws advance it.
+class Generator {
+public:
+    explicit Generator(uint64_t seed = 0) {
+        uint64_t r = seed + 0x9E3779B97F4A7C15ull;
+        r = (r ^ (r >> 30)) * 0xBF58476D1CE4E5B9ull;
+        r = (r ^ (r >> 27)) * 0x94D049BB133111EBull;
+        state = r ^ (r >> 31);
+    }
+    uint64_t state;
+};
+// tinytensor::uniform_real(low, high, shape, options, gen) (tensor.cpp:1773-1781) and normal.
+inline auto uniform_real(double low, double high, const Shape &shape, Generator &gen, ScalarType dtype = kF32, Device device = kAMD) -> Tensor {
+    if (!(low < high)) throw TTException("Expected low < high. At least one element violates this.");
+    return get_backend(device)->random_fill(0, low, high, shape, gen.state, dtype, device);
+}
+inline auto normal(double mu, double std, const Shape &shape, Generator &gen, ScalarType dtype = kF32, Device device = kAMD) -> Tensor {
+    return get_backend(device)->random_fill(1, mu, std, shape, gen.state, dtype, device);
+}
+
 namespace nn {
 // nn::Linear (nn/linear.cpp:20-50): weight is [in_features, out_features]; forward = matmul + bias.  The bias add
 // (and an optional ReLU that follows it) is fused into the GEMM's store phase.
@@ -400,6 +644,17 @@ class Linear {
 public:
     Linear(Tensor weight_, std::optional<Tensor> bias_) : weight(std::move(weight_)), bias(std::move(bias_)) {
         if (weight.dim() != 2) throw TTException("Linear: weight must be [in_features, out_features]");
+    }
+    // Default initialisation (nn/linear.cpp:20-40): weight by kaiming_uniform_ with gain 1 and fan = weight.size(0)
+    // (nn/init.cpp:30-52,106-112), then bias ~ U(+-1/sqrt(fan)), both drawn from `gen` in that order.
+    Linear(int in_features, int out_features, bool with_bias, Generator &gen, ScalarType dtype = kF32, Device device = kAMD) {
+        const double fan = static_cast<double>(in_features);
+        const double bound_w = std::sqrt(3.0) * (1.0 / std::sqrt(fan));
+        weight = uniform_real(-bound_w, bound_w, Shape({in_features, out_features}), gen, dtype, device);
+        if (with_bias) {
+            const double bound_b = 1.0 / std::sqrt(fan);
+            bias = uniform_real(-bound_b, bound_b, Shape({out_features}), gen, dtype, device);
+        }
     }
     [[nodiscard]] auto forward(const Tensor &input, bool fuse_relu = false) const -> Tensor {
         const Tensor x2 = input.dim() == 2 ? input : input.flatten(0, -2);
