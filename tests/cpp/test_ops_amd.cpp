@@ -126,6 +126,18 @@ TEST_CASE("To") {
         for (T x : a) eb.push_back(x != T(0));
         CHECK(A.to(kBool).template to_vec<bool>() == eb);
         CHECK(A.to(A.dtype()).storage() == A.storage());  // same dtype: the tensor itself (tensor.cpp:536-538)
+        // matmul promotes mixed operands (tensor.cpp:2394-2399): T x f64 -> f64
+        const std::vector<double> w(100 * 2, 0.5);
+        const Tensor Y = matmul(A, Tensor(w, {100, 2}, device));
+        CHECK(Y.dtype() == kF64);
+        std::vector<double> ey;
+        for (int r = 0; r < 3; ++r) {
+            double acc = 0;
+            for (int k = 0; k < 100; ++k) acc += 0.5 * static_cast<double>(a[static_cast<std::size_t>(r * 100 + k)]);
+            ey.push_back(acc);
+            ey.push_back(acc);
+        }
+        CHECK(Y.template to_vec<double>() == ey);
     };
     runner_all_except_bool(test);
 }

@@ -48,6 +48,20 @@ def test_bool_is_rejected(tt):
         tt.matmul(b, c)
 
 
+def test_mixed_dtypes_are_promoted(tt):
+    # check_promote (tensor/tensor.cpp:2398-2399): both operands are cast to promote_types(lhs, rhs)
+    rng = np.random.default_rng(4)
+    a = rng.integers(-5, 6, (7, 9)).astype(np.int16)
+    for other, want_dtype in ((np.int64, np.int64), (np.float32, np.float32), (np.float64, np.float64), (np.bool_, np.int16)):
+        b = rng.integers(0, 2 if other == np.bool_ else 6, (9, 5)).astype(other)
+        got = tt.matmul(dev(tt, a), dev(tt, b)).to_numpy()
+        assert got.dtype == np.dtype(want_dtype)
+        assert np.array_equal(got, a.astype(want_dtype) @ b.astype(want_dtype))
+    out = tt.linear(dev(tt, a), dev(tt, np.ones((9, 5), np.float32)), dev(tt, np.arange(5, dtype=np.int32)))
+    assert out.to_numpy().dtype == np.float32
+    assert np.array_equal(out.to_numpy(), a.astype(np.float32) @ np.ones((9, 5), np.float32) + np.arange(5, dtype=np.float32))
+
+
 def test_shape_errors(tt):
     a = dev(tt, np.ones((3, 4), dtype=np.float32))
     with pytest.raises(tt.TTException):

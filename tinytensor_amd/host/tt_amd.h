@@ -487,11 +487,11 @@ auto Tensor::to_vec() const -> std::vector<T> {
 }
 
 // tinytensor::matmul (tensor.cpp:2390-2484): rank dispatch onto batched_matmul; bool is rejected.
-inline auto matmul(const Tensor &lhs, const Tensor &rhs) -> Tensor {
-    if (!(lhs.device() == rhs.device())) throw TTException("Expected tensors on the same device");
-    const auto promoted = promote_types(lhs.dtype(), rhs.dtype());
+inline auto matmul(const Tensor &lhs_, const Tensor &rhs_) -> Tensor {
+    if (!(lhs_.device() == rhs_.device())) throw TTException("Expected tensors on the same device");
+    const auto promoted = promote_types(lhs_.dtype(), rhs_.dtype());
     if (promoted == kBool) throw TTException("matmul does not support boolean tensors");
-    if (lhs.dtype() != rhs.dtype()) throw TTException("mixed-dtype matmul needs a cast op, which this backend slice does not provide");
+    const Tensor lhs = lhs_.to(promoted), rhs = rhs_.to(promoted);  // check_promote (tensor.cpp:2398-2399)
     const auto *be = get_backend(lhs.device());
     const auto &ls = lhs.shape(), &rs = rhs.shape();
     if (ls.ndim() == 1 && rs.ndim() == 1) {

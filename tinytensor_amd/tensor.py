@@ -546,11 +546,9 @@ def _promote(lhs: Tensor, rhs: Tensor):
     dt = max(lhs.dtype, rhs.dtype)
     if dt == _capi.BOOL:
         raise TTException("matmul does not support boolean tensors")
-    if lhs.dtype != dt or rhs.dtype != dt:
-        # Tensor::to(dtype) is an elementwise cast outside the GEMM path; the callers of this mirror
-        # hand over operands of one dtype.
-        raise TTException("mixed-dtype matmul needs a cast op, which this backend slice does not provide")
-    return lhs, rhs
+    # check_promote (tensor/tensor.cpp:2398-2399): operands are cast to promote_types(lhs, rhs), which orders the
+    # dtypes bool < u8 < i16 < i32 < i64 < f32 < f64 (common/scalar.cpp:17-26)
+    return lhs.to(dt), rhs.to(dt)
 
 
 def matmul(lhs: Tensor, rhs: Tensor) -> Tensor:
@@ -593,7 +591,9 @@ def linear(input: Tensor, weight: Tensor, bias: Tensor | None = None, relu: bool
     x2 = input.flatten(0, -2) if input.dim() != 2 else input
     if x2.size(1) != weight.size(0):
         raise TTException(f"Invalid shape for matrix multiplication. LHS={x2.shape} and RHS={weight.shape}")
-    _promote(x2, weight)
+    x2, weight = _promote(x2, weight)
+    if bias is not None:
+        bias = bias.to(x2.dtype)
     out = get_backend(input.device).batched_matmul(x2.unsqueeze(0), weight.unsqueeze(0), bias=bias, bias_mode=1,
                                                    relu=relu)
     return out.reshape(list(input.shape[:-1]) + [weight.size(1)])
