@@ -143,6 +143,70 @@ def detail_report(tt, np, path, cpu=True):
     ms = time_launches(tt, lambda: be.conv2d_backward(go, x, w, None, 1, 1, buffers=bufs), 50, 5)
     rows.append({"case": "cfg4 conv2d backward (grad_input + grad_weight)", "kernel": "conv_dgrad_kernel + conv_wgrad_kernel + reduce",
                  "ms": round(ms, 5), "GFLOP/s": round(3.700e9 / ms / 1e6, 1)})
+    # Streaming kernels around the GEMMs (HBM-bound; GB/s counts each operand and the result once), called through
+    # the C ABI with preallocated results so that no allocation is timed.
+    lib, cap = tt._capi.lib, tt._capi
+    i64 = lambda v: (C.c_int64 * len(v))(*v)
+    ptr = lambda t: C.c_void_p(t.storage.ptr)
+
+    def stream_case(name, kernel, nbytes, fn, iters=50):
+        ms = time_launches(tt, fn, iters, 5)
+        rows.append({"case": name, "kernel": kernel, "ms": round(ms, 5), "GB/s": round(nbytes / ms / 1e6, 1),
+                     "of_hbm_peak": round(nbytes / ms / 1e6 / 8000.0, 3)})
+
+    n = 8192
+    Ea = tt.Tensor.from_numpy(np.random.default_rng(0).random((n, n), dtype=f32))
+    Eo = tt.Tensor.empty((n, n), cap.F32)
+    Eo64 = tt.Tensor.empty((n, n), cap.F64)
+    sh, st, stT = i64((n, n)), i64((n, 1)), i64((1, n))
+    stream_case("add 8192x8192 f32", "binary_kernel", 3 * n * n * 4,
+                lambda: lib.ttamd_binary(0, cap.F32, cap.BIN["add"], 2, sh, ptr(Ea), 0, st, ptr(Ea), 0, st, ptr(Eo), None))
+    stream_case("relu 8192x8192 f32", "unary_kernel", 2 * n * n * 4,
+                lambda: lib.ttamd_unary(0, cap.F32, cap.UN["relu"], 2, sh, ptr(Ea), 0, st, ptr(Eo), None))
+    stream_case("contiguous of a transposed 8192x8192 f32 view", "contiguous_kernel", 2 * n * n * 4,
+                lambda: lib.ttamd_contiguous(0, cap.F32, 2, sh, stT, ptr(Ea), 0, ptr(Eo), None))
+    stream_case("cast 8192x8192 f32 -> f64", "cast_kernel", n * n * 12,
+                lambda: lib.ttamd_cast(0, cap.F32, cap.F64, 2, sh, ptr(Ea), 0, st, ptr(Eo64), None))
+    stream_case("sum 8192x8192 f32 (all)", "sum_all_kernel", n * n * 4,
+                lambda: lib.ttamd_sum(0, cap.F32, 2, sh, ptr(Ea), 0, st, -1, ptr(Eo), None))
+    m = 1024
+    shm, stm = i64((m, m)), i64((m, 1))
+    stream_case("cfg5 bias-free add 1024x1024 f32", "binary_kernel", 3 * m * m * 4,
+                lambda: lib.ttamd_binary(0, cap.F32, cap.BIN["add"], 2, shm, ptr(Ea), 0, stm, ptr(Ea), 0, stm, ptr(Eo), None), 200)
+    # pooling on [64,64,112,112] f32 (205 MB): k2 s2 p0 and k3 s2 p1
+    Pb, Pc, Ph, Pw = 64, 64, 112, 112
+    Px = tt.Tensor.from_numpy(np.random.default_rng(1).random((Pb, Pc, Ph, Pw), dtype=f32))
+    for k, S_, P_ in ((2, 2, 0), (3, 2, 1)):
+        Ho, Wo = (Ph + 2 * P_ - k) // S_ + 1, (Pw + 2 * P_ - k) // S_ + 1
+        Pout = tt.Tensor.empty((Pb, Pc, Ho, Wo), cap.F32)
+        Pg = tt.Tensor.from_numpy(np.ones((Pb, Pc, Ho, Wo), f32))
+        Pgx = tt.Tensor.empty((Pb, Pc, Ph, Pw), cap.F32)
+        iv = Px.view4()
+        in_b, out_b = Pb * Pc * Ph * Pw * 4, Pb * Pc * Ho * Wo * 4
+        for op in ("max", "avg"):
+            code = cap.POOL[op]
+            stream_case(f"{op}_pool2d forward k{k} s{S_} p{P_} [64,64,112,112] f32", "pool_forward_kernel", in_b + out_b,
+                        lambda: lib.ttamd_pool2d_forward(0, cap.F32, code, C.byref(iv), ptr(Pout), Pb, Pc, Ph, Pw, k, S_, P_, None), 30)
+            stream_case(f"{op}_pool2d backward k{k} s{S_} p{P_} [64,64,112,112] f32", "pool_backward_kernel", 2 * in_b + 2 * out_b,
+                        lambda: lib.ttamd_pool2d_backward(0, cap.F32, code, ptr(Pg), C.byref(iv), ptr(Pout), ptr(Pgx), Pb, Pc, Ph, Pw,
+                                                          k, S_, P_, None), 30)
+    if cpu:
+        ph = np.random.default_rng(1).random((8, 64, 112, 112), dtype=f32)  # an eighth of the batch
+        for k, S_, P_ in ((2, 2, 0), (3, 2, 1)):
+            for op in ("max", "avg"):
+                t0 = time.perf_counter()
+                res = oracle.pool2d_forward(ph, op, k, S_, P_)
+                t1 = time.perf_counter()
+                oracle.pool2d_backward(np.ones_like(res), ph, res, op, k, S_, P_)
+                t2 = time.perf_counter()
+                for r in rows:
+                    if r["case"] == f"{op}_pool2d forward k{k} s{S_} p{P_} [64,64,112,112] f32":
+                        r["cpu_oracle_ms_1core"] = round((t1 - t0) * 8e3, 1)
+                    if r["case"] == f"{op}_pool2d backward k{k} s{S_} p{P_} [64,64,112,112] f32":
+                        r["cpu_oracle_ms_1core"] = round((t2 - t1) * 8e3, 1)
+        for r in rows:
+            if "pool2d" in r["case"] and "cpu_oracle_ms_1core" in r:
+                r["speedup_vs_cpu"] = round(r["cpu_oracle_ms_1core"] / r["ms"], 1)
     if cpu:
         # The same configurations on the CPU oracle (one core), timed once each.
         xh, wh = oracle.Generator(0).normal(0, 0.1, (64, 32, 28, 28)), oracle.Generator(1).normal(0, 0.1, (64, 32, 3, 3))

@@ -301,10 +301,11 @@ struct TapView {
     }
 };
 
-// One gathered vector: elements e0 .. e0 + VEC - 1 of the image, columns x0 .. x0 + VEC - 1 of a row of width src_w.
+// One gathered vector: elements e0 .. e0 + VEC - 1 of the image.  The components outside the row are NOT cleared
+// here: touching the loaded registers would make the wave wait for the data before its MFMA work; the stagers
+// keep the first column x0 and clear them in store(), just before the LDS write (clear_outside_row).
 template <typename T, int VEC>
-__device__ __forceinline__ typename Vec<T, VEC>::type gather_row_vector(__amdgpu_buffer_rsrc_t rsrc, bool row_ok, int32_t e0,
-                                                                        int x0, int src_w) {
+__device__ __forceinline__ typename Vec<T, VEC>::type gather_row_vector(__amdgpu_buffer_rsrc_t rsrc, bool row_ok, int32_t e0) {
     using V = typename Vec<T, VEC>::type;
     constexpr int32_t SZ = static_cast<int32_t>(sizeof(T));
     V v = Vec<T, VEC>::load(rsrc, (row_ok && e0 >= 0) ? static_cast<uint32_t>(e0 * SZ) : kOob);
@@ -312,6 +313,12 @@ __device__ __forceinline__ typename Vec<T, VEC>::type gather_row_vector(__amdgpu
 #pragma unroll
         for (int j = 0; j < VEC; ++j) v[j] = Vec<T, 1>::load(rsrc, e0 + j >= 0 ? static_cast<uint32_t>((e0 + j) * SZ) : kOob);
     }
+    return v;
+}
+
+// Columns x0 .. x0 + VEC - 1 of a row of width src_w: components outside the row become 0.
+template <typename T, int VEC>
+__device__ __forceinline__ typename Vec<T, VEC>::type clear_outside_row(typename Vec<T, VEC>::type v, int x0, int src_w) {
 #pragma unroll
     for (int j = 0; j < VEC; ++j)
         if (static_cast<unsigned>(x0 + j) >= static_cast<unsigned>(src_w)) v[j] = T(0);
@@ -330,6 +337,7 @@ struct TapStagerMC : TileLayout<T, ROWS, BK, false> {
     static_assert(VEC > 1 && ROWS % VEC == 0 && kThreads % VPL == 0 && BK % LPP == 0, "tile must split evenly");
     static constexpr int kPF = PF;
     V reg[PF][P];
+    int col0[PF][P];  // first source column of each gathered vector
     __amdgpu_buffer_rsrc_t rsrc;
     TapView<FLIP> tv;
     int n_local, line0, k_next;
@@ -362,7 +370,8 @@ struct TapStagerMC : TileLayout<T, ROWS, BK, false> {
             tv.tap(static_cast<uint32_t>(k_ok ? kk : 0), ch_off, dy, dx);
             const int y = py + dy, x0 = px0 + dx;
             const bool row_ok = n_ok && k_ok && static_cast<unsigned>(y) < static_cast<unsigned>(tv.src_h);
-            reg[SLOT][p] = gather_row_vector<T, VEC>(rsrc, row_ok, ch_off + y * tv.s_h + x0, x0, tv.src_w);
+            reg[SLOT][p] = gather_row_vector<T, VEC>(rsrc, row_ok, ch_off + y * tv.s_h + x0);
+            col0[SLOT][p] = x0;
         }
         k_next += BK;
     }
@@ -370,7 +379,8 @@ struct TapStagerMC : TileLayout<T, ROWS, BK, false> {
     template <int SLOT = 0>
     __device__ __forceinline__ void store(T *lds) const {
 #pragma unroll
-        for (int p = 0; p < P; ++p) *reinterpret_cast<V *>(&lds[(p * LPP + line0) * L::LD + n_local]) = reg[SLOT][p];
+        for (int p = 0; p < P; ++p)
+            *reinterpret_cast<V *>(&lds[(p * LPP + line0) * L::LD + n_local]) = clear_outside_row<T, VEC>(reg[SLOT][p], col0[SLOT][p], tv.src_w);
     }
 };
 
@@ -386,6 +396,7 @@ struct TapStagerKC : TileLayout<T, ROWS, BK, true> {
     static_assert(VEC > 1 && BK % VEC == 0 && kThreads % VPL == 0 && ROWS % RPP == 0, "tile must split evenly");
     static constexpr int kPF = PF;
     V reg[PF][P];
+    int col0[PF];  // source column of the lane's first position, before the tap's dx
     __amdgpu_buffer_rsrc_t rsrc;
     TapView<false> tv;
     int32_t joff[P];
@@ -426,23 +437,31 @@ struct TapStagerKC : TileLayout<T, ROWS, BK, true> {
         const int32_t base = py * tv.s_h + px0;
 #pragma unroll
         for (int p = 0; p < P; ++p) {
-            const int yy = py + dy[p], x0 = px0 + dx[p];
+            const int yy = py + dy[p];
             const bool row_ok = n_ok && j_ok[p] && static_cast<unsigned>(yy) < static_cast<unsigned>(tv.src_h);
-            reg[SLOT][p] = gather_row_vector<T, VEC>(rsrc, row_ok, base + joff[p], x0, tv.src_w);
+            reg[SLOT][p] = gather_row_vector<T, VEC>(rsrc, row_ok, base + joff[p]);
         }
+        col0[SLOT] = px0;
         k_next += BK;
     }
 
     template <int SLOT = 0>
     __device__ __forceinline__ void store(T *lds) const {
 #pragma unroll
-        for (int p = 0; p < P; ++p) *reinterpret_cast<V *>(&lds[(p * RPP + row0) * L::LD + k_local]) = reg[SLOT][p];
+        for (int p = 0; p < P; ++p)
+            *reinterpret_cast<V *>(&lds[(p * RPP + row0) * L::LD + k_local]) =
+                clear_outside_row<T, VEC>(reg[SLOT][p], col0[SLOT] + dx[p], tv.src_w);
     }
 };
 
 // ---------------------------------------------------------------------------------------------
 // Tile shapes: 64x64 (2x2 waves) or, for products with at most 32 rows, 32x128 (1x4 waves): every wave owns a
 // 32x32 block either way.
+// Register prefetch distance of the conv kernels: tile t + kConvPF is requested while tile t is multiplied.  The
+// gathers spend several hundred cycles on address arithmetic before their loads issue and a k tile holds little
+// MFMA work (32x32 per wave), so one tile of lookahead leaves the load latency exposed.
+constexpr int kConvPF = 1;
+
 template <typename T, int BM, int BN, int BK, class StA, class StB>
 using ConvEngine = TileEngine<T, BM, BN, BK, BM == 32 ? 1 : 2, BM == 32 ? 4 : 2, StA, StB>;
 
@@ -450,7 +469,7 @@ using ConvEngine = TileEngine<T, BM, BN, BK, BM == 32 ? 1 : 2, BM == 32 ? 4 : 2,
 template <typename T, int BM, int BN, int BK, int A_VEC, class StB>
 __global__ void __launch_bounds__(kThreads, 2)
 conv_fwd_kernel(ConvGeom geo, const T *x, const T *w, const T *bias, T *out, int64_t image_bytes, int tiles_m, int tiles_n) {
-    using StA = Stager<T, BM, BK, true, A_VEC>;
+    using StA = Stager<T, BM, BK, true, A_VEC, kConvPF>;
     using Engine = ConvEngine<T, BM, BN, BK, StA, StB>;
     extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
     T *const smem = reinterpret_cast<T *>(smem_raw);
@@ -487,7 +506,7 @@ __global__ void __launch_bounds__(256) weight_transpose_kernel(ConvGeom geo, con
 template <typename T, int BM, int BN, int BK, int A_VEC, class StB>
 __global__ void __launch_bounds__(kThreads, 2)
 conv_dgrad_kernel(ConvGeom geo, const T *gout, const T *wt, T *gin, int tiles_m, int tiles_n) {
-    using StA = Stager<T, BM, BK, true, A_VEC>;
+    using StA = Stager<T, BM, BK, true, A_VEC, kConvPF>;
     using Engine = ConvEngine<T, BM, BN, BK, StA, StB>;
     extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
     T *const smem = reinterpret_cast<T *>(smem_raw);
@@ -515,7 +534,7 @@ __global__ void __launch_bounds__(kThreads, 2)
 conv_wgrad_kernel(ConvGeom geo, const T *gout, const T *x, T *partial, int64_t image_bytes, int group, int kslices, int k_chunk,
                   int tiles_m, int tiles_n) {
     constexpr int BM = 64, BN = 64;
-    using StA = Stager<T, BM, BK, true, A_VEC>;
+    using StA = Stager<T, BM, BK, true, A_VEC, kConvPF>;
     using Engine = ConvEngine<T, BM, BN, BK, StA, StB>;
     extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
     T *const smem = reinterpret_cast<T *>(smem_raw);
@@ -633,6 +652,10 @@ ttamd_status make_plan(const char *who, ttamd_dtype dtype, const ttamd_view4 *in
                   stride, padding);
         return TTAMD_ERR_INVALID_ARGUMENT;
     }
+    if (k >= (1 << 14) || padding >= (1 << 14)) {
+        set_error("%s: kernel size and padding must be below 16384", who);
+        return TTAMD_ERR_INVALID_ARGUMENT;
+    }
     const int Ho = (H + 2 * padding - k) / stride + 1, Wo = (W + 2 * padding - k) / stride + 1;
     if (H + 2 * padding < k || W + 2 * padding < k || Ho <= 0 || Wo <= 0) {
         set_error("%s: kernel %d does not fit the padded input %dx%d", who, k, H + 2 * padding, W + 2 * padding);
@@ -722,7 +745,7 @@ ttamd_status launch_conv(Kernel kernel, size_t lds, int64_t blocks, hipStream_t 
 template <typename T, int BM, int BN, int A_VEC, class StB>
 constexpr size_t conv_lds_bytes() {
     constexpr int BK = ConvTiles<T>::BK;
-    return ConvEngine<T, BM, BN, BK, Stager<T, BM, BK, true, A_VEC>, StB>::kLdsBytes;
+    return ConvEngine<T, BM, BN, BK, Stager<T, BM, BK, true, A_VEC, kConvPF>, StB>::kLdsBytes;
 }
 
 template <typename T, int BM, int BN>
@@ -738,8 +761,8 @@ ttamd_status forward_mfma_tile(const ConvPlan &pl, const void *bias, void *out, 
         return launch_conv(kernel, lds, blocks, st, g, static_cast<const T *>(pl.x), static_cast<const T *>(pl.w),
                            static_cast<const T *>(bias), static_cast<T *>(out), pl.image_bytes, tiles_m, tiles_n);
     };
-    using VecB = TapStagerMC<T, BN, BK, VK, false>;
-    using OneB = Im2colStager<T, BN, BK>;
+    using VecB = TapStagerMC<T, BN, BK, VK, false, kConvPF>;
+    using OneB = Im2colStager<T, BN, BK, kConvPF>;
     if (a_vec && b_vec) return go(conv_fwd_kernel<T, BM, BN, BK, VK, VecB>, conv_lds_bytes<T, BM, BN, VK, VecB>());
     if (a_vec) return go(conv_fwd_kernel<T, BM, BN, BK, VK, OneB>, conv_lds_bytes<T, BM, BN, VK, OneB>());
     if (b_vec) return go(conv_fwd_kernel<T, BM, BN, BK, 1, VecB>, conv_lds_bytes<T, BM, BN, 1, VecB>());
@@ -841,8 +864,8 @@ ttamd_status backward_mfma(const ConvPlan &pl, const void *gout, void *gin, void
                 return launch_conv(kernel, lds, blocks, st, g, static_cast<const T *>(gout), static_cast<const T *>(wt),
                                    static_cast<T *>(gin), tiles_m, tiles_n);
             };
-            using VecB = TapStagerMC<T, BN, BK, VK, true>;
-            using OneB = DgradStager<T, BN, BK>;
+            using VecB = TapStagerMC<T, BN, BK, VK, true, kConvPF>;
+            using OneB = DgradStager<T, BN, BK, kConvPF>;
             if (a_vec && b_vec) return go(conv_dgrad_kernel<T, BM, BN, BK, VK, VecB>, conv_lds_bytes<T, BM, BN, VK, VecB>());
             if (a_vec) return go(conv_dgrad_kernel<T, BM, BN, BK, VK, OneB>, conv_lds_bytes<T, BM, BN, VK, OneB>());
             if (b_vec) return go(conv_dgrad_kernel<T, BM, BN, BK, 1, VecB>, conv_lds_bytes<T, BM, BN, 1, VecB>());
@@ -865,8 +888,8 @@ ttamd_status backward_mfma(const ConvPlan &pl, const void *gout, void *gin, void
             return launch_conv(kernel, lds, blocks, st, g, static_cast<const T *>(gout), static_cast<const T *>(pl.x), partial,
                                pl.image_bytes, plan.group, plan.kslices, plan.k_chunk, tiles_m, tiles_n);
         };
-        using VecB = TapStagerKC<T, 64, BK, VK>;
-        using OneB = Im2colTStager<T, 64, BK>;
+        using VecB = TapStagerKC<T, 64, BK, VK, kConvPF>;
+        using OneB = Im2colTStager<T, 64, BK, kConvPF>;
         ttamd_status s;
         if (a_vec && b_vec) s = go(conv_wgrad_kernel<T, BK, VK, VecB>, conv_lds_bytes<T, 64, 64, VK, VecB>());
         else if (a_vec) s = go(conv_wgrad_kernel<T, BK, VK, OneB>, conv_lds_bytes<T, 64, 64, VK, OneB>());
