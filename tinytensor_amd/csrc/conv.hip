@@ -24,30 +24,6 @@ namespace {
 
 using namespace mfma;
 
-// Exact unsigned division by a runtime-invariant divisor (Granlund & Montgomery): q = x / d for all 32-bit x.
-struct FastDiv {
-    uint32_t mul, sh1, sh2, d;
-    __device__ __forceinline__ uint32_t div(uint32_t x) const {
-        const uint32_t t = __umulhi(mul, x);
-        return (t + ((x - t) >> sh1)) >> sh2;
-    }
-    __device__ __forceinline__ void divmod(uint32_t x, uint32_t &q, uint32_t &r) const {
-        q = div(x);
-        r = x - q * d;
-    }
-};
-
-FastDiv make_fastdiv(uint32_t d) {
-    FastDiv f{};
-    f.d = d;
-    uint32_t L = 0;
-    while ((1ull << L) < d) ++L;
-    f.mul = static_cast<uint32_t>(((1ull << 32) * ((1ull << L) - d)) / d + 1);
-    f.sh1 = L < 1 ? L : 1;
-    f.sh2 = L > 0 ? L - 1 : 0;
-    return f;
-}
-
 struct ConvGeom {
     int B, C, H, W, O, k, S, P, Ho, Wo;
     int64_t xs_b;              // input batch stride (elements)

@@ -32,8 +32,117 @@ __global__ void __launch_bounds__(256) contiguous_kernel(const W *__restrict__ s
     }
 }
 
+// Dense view: a plain copy, 16 bytes per lane.
+__global__ void __launch_bounds__(256) copy16_kernel(const uint4 *__restrict__ src, uint4 *__restrict__ dst, int64_t nvec) {
+    const int64_t step = static_cast<int64_t>(gridDim.x) * blockDim.x;
+    for (int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < nvec; i += step) dst[i] = src[i];
+}
+
+// Transposing copy for a view whose unit-stride dimension `fast` is not the last one (a permuted tensor): 64 x 64
+// tiles over (fast, last) go through LDS so that both the reads (along `fast`) and the writes (along the last
+// dimension) are coalesced.  The remaining dimensions are folded into the tile index.
+struct TransposeDesc {
+    ViewDesc outer;              // the dimensions other than `fast` and the last, with the source strides
+    int64_t outer_dst[kMaxDims];  // their strides in the dense result
+    int64_t rows, cols;          // extent of `fast` and of the last dimension
+    int64_t src_col_stride;      // source stride of the last dimension (the `fast` stride is 1)
+    int64_t dst_row_stride;      // dense stride of `fast` in the result (the last dimension's is 1)
+    int tiles_r, tiles_c;
+};
+
+template <typename W>
+__global__ void __launch_bounds__(256) transpose_copy_kernel(const W *__restrict__ src, W *__restrict__ dst, TransposeDesc t) {
+    __shared__ W tile[64][65];
+    int64_t id = blockIdx.x;
+    const int tc = static_cast<int>(id % t.tiles_c);
+    id /= t.tiles_c;
+    const int tr = static_cast<int>(id % t.tiles_r);
+    int64_t rank = id / t.tiles_r, s_off = 0, d_off = 0;
+    for (int d = t.outer.ndim - 1; d >= 0; --d) {
+        const int64_t i = rank % t.outer.shape[d];
+        rank /= t.outer.shape[d];
+        s_off += i * t.outer.stride[d];
+        d_off += i * t.outer_dst[d];
+    }
+    const int64_t r0 = static_cast<int64_t>(tr) * 64, c0 = static_cast<int64_t>(tc) * 64;
+    const int lane = threadIdx.x % 64, group = threadIdx.x / 64;
+    // read: lanes run along `fast` (unit source stride)
+    for (int c = group; c < 64; c += 4)
+        if (r0 + lane < t.rows && c0 + c < t.cols) tile[c][lane] = src[s_off + (r0 + lane) + (c0 + c) * t.src_col_stride];
+    __syncthreads();
+    // write: lanes run along the last dimension (unit result stride)
+    for (int r = group; r < 64; r += 4)
+        if (r0 + r < t.rows && c0 + lane < t.cols) dst[d_off + (r0 + r) * t.dst_row_stride + (c0 + lane)] = tile[lane][r];
+}
+
 template <typename W>
 ttamd_status launch_contiguous(const void *src, void *dst, const ViewDesc &v, int64_t numel, hipStream_t stream) {
+    // dense: plain copy
+    bool dense = true;
+    {
+        int64_t expect = 1;
+        for (int d = v.ndim - 1; d >= 0; --d) {
+            if (v.shape[d] != 1 && v.stride[d] != expect) dense = false;
+            expect *= v.shape[d];
+        }
+    }
+    if (dense) {
+        const int64_t bytes = numel * static_cast<int64_t>(sizeof(W));
+        int64_t done = 0;
+        if (reinterpret_cast<uintptr_t>(src) % 16 == 0 && reinterpret_cast<uintptr_t>(dst) % 16 == 0 && bytes >= 16) {
+            const int64_t nvec = bytes / 16;
+            int64_t blocks = (nvec + 255) / 256;
+            if (blocks > 8192) blocks = 8192;
+            copy16_kernel<<<dim3(static_cast<unsigned>(blocks)), dim3(256), 0, stream>>>(static_cast<const uint4 *>(src), static_cast<uint4 *>(dst), nvec);
+            done = nvec * 16 / static_cast<int64_t>(sizeof(W));
+        }
+        if (done < numel) {
+            ViewDesc flat{};
+            flat.ndim = 1;
+            flat.shape[0] = numel - done;
+            flat.stride[0] = 1;
+            contiguous_kernel<W><<<dim3(1), dim3(256), 0, stream>>>(static_cast<const W *>(src) + done, static_cast<W *>(dst) + done, flat, numel - done);
+        }
+        TTAMD_HIP_CHECK(hipGetLastError());
+        return TTAMD_OK;
+    }
+    // permuted: the last dimension is strided and another one has unit stride
+    const int last = v.ndim - 1;
+    int fast = -1;
+    if (v.ndim >= 2 && v.stride[last] != 1 && v.shape[last] >= 16)
+        for (int d = 0; d < last; ++d)
+            if (v.stride[d] == 1 && v.shape[d] >= 16) fast = d;
+    if (fast >= 0) {
+        TransposeDesc t{};
+        int64_t dense_stride[kMaxDims];
+        int64_t expect = 1;
+        for (int d = last; d >= 0; --d) {
+            dense_stride[d] = expect;
+            expect *= v.shape[d];
+        }
+        int64_t outer_count = 1;
+        for (int d = 0; d < last; ++d) {
+            if (d == fast) continue;
+            t.outer.shape[t.outer.ndim] = v.shape[d];
+            t.outer.stride[t.outer.ndim] = v.stride[d];
+            t.outer_dst[t.outer.ndim] = dense_stride[d];
+            ++t.outer.ndim;
+            outer_count *= v.shape[d];
+        }
+        t.rows = v.shape[fast];
+        t.cols = v.shape[last];
+        t.src_col_stride = v.stride[last];
+        t.dst_row_stride = dense_stride[fast];
+        const int64_t tiles_r = (t.rows + 63) / 64, tiles_c = (t.cols + 63) / 64;
+        const int64_t blocks = tiles_r * tiles_c * outer_count;
+        if (tiles_r <= 0x7fffffff && tiles_c <= 0x7fffffff && blocks <= 0x7fffffff) {
+            t.tiles_r = static_cast<int>(tiles_r);
+            t.tiles_c = static_cast<int>(tiles_c);
+            transpose_copy_kernel<W><<<dim3(static_cast<unsigned>(blocks)), dim3(256), 0, stream>>>(static_cast<const W *>(src), static_cast<W *>(dst), t);
+            TTAMD_HIP_CHECK(hipGetLastError());
+            return TTAMD_OK;
+        }
+    }
     int64_t blocks = (numel + 255) / 256;
     if (blocks > 65536) blocks = 65536;
     contiguous_kernel<W><<<dim3(static_cast<unsigned>(blocks)), dim3(256), 0, stream>>>(static_cast<const W *>(src),
@@ -138,6 +247,55 @@ __global__ void __launch_bounds__(256) unary_kernel(const T *__restrict__ a, Vie
         out[i] = unary_apply<T, OP>(DENSE ? a[i] : a[flat_of(i, va)]);
 }
 
+// Dense streaming forms: every lane moves one 16-byte vector of each T-typed operand per step (N = 16 / sizeof(T)
+// elements; a result of another width is written as one N-element vector too), so a wavefront requests 1 KiB per
+// load instruction.  Used when all operands are dense and 16-byte aligned; the last numel % N elements go through
+// the element-wise kernels.
+template <typename T, int N>
+using vec_t = T __attribute__((ext_vector_type(N)));
+
+template <typename T, int OP>
+__global__ void __launch_bounds__(256) binary_vec_kernel(const T *__restrict__ a, const T *__restrict__ b, void *__restrict__ out, int64_t nvec) {
+    constexpr int N = 16 / sizeof(T);
+    using R = decltype(binary_apply<T, OP>(T(0), T(0)));
+    const int64_t step = static_cast<int64_t>(gridDim.x) * blockDim.x;
+    for (int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < nvec; i += step) {
+        const vec_t<T, N> x = reinterpret_cast<const vec_t<T, N> *>(a)[i], y = reinterpret_cast<const vec_t<T, N> *>(b)[i];
+        vec_t<R, N> r;
+#pragma unroll
+        for (int j = 0; j < N; ++j) r[j] = binary_apply<T, OP>(x[j], y[j]);
+        static_cast<vec_t<R, N> *>(out)[i] = r;
+    }
+}
+
+template <typename T, int OP>
+__global__ void __launch_bounds__(256) unary_vec_kernel(const T *__restrict__ a, T *__restrict__ out, int64_t nvec) {
+    constexpr int N = 16 / sizeof(T);
+    const int64_t step = static_cast<int64_t>(gridDim.x) * blockDim.x;
+    for (int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < nvec; i += step) {
+        const vec_t<T, N> x = reinterpret_cast<const vec_t<T, N> *>(a)[i];
+        vec_t<T, N> r;
+#pragma unroll
+        for (int j = 0; j < N; ++j) r[j] = unary_apply<T, OP>(x[j]);
+        reinterpret_cast<vec_t<T, N> *>(out)[i] = r;
+    }
+}
+
+template <typename T>
+__global__ void __launch_bounds__(256) where_vec_kernel(const uint8_t *__restrict__ c, const T *__restrict__ a, const T *__restrict__ b,
+                                                       T *__restrict__ out, int64_t nvec) {
+    constexpr int N = 16 / sizeof(T);
+    const int64_t step = static_cast<int64_t>(gridDim.x) * blockDim.x;
+    for (int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < nvec; i += step) {
+        const vec_t<uint8_t, N> m = reinterpret_cast<const vec_t<uint8_t, N> *>(c)[i];
+        const vec_t<T, N> x = reinterpret_cast<const vec_t<T, N> *>(a)[i], y = reinterpret_cast<const vec_t<T, N> *>(b)[i];
+        vec_t<T, N> r;
+#pragma unroll
+        for (int j = 0; j < N; ++j) r[j] = m[j] ? x[j] : y[j];
+        reinterpret_cast<vec_t<T, N> *>(out)[i] = r;
+    }
+}
+
 template <typename T>
 __global__ void __launch_bounds__(256) where_kernel(const uint8_t *__restrict__ c, ViewDesc vc, const T *__restrict__ a, ViewDesc va,
                                                    const T *__restrict__ b, ViewDesc vb, T *__restrict__ out, int64_t numel) {
@@ -171,7 +329,18 @@ __global__ void __launch_bounds__(256) sum_all_kernel(const T *__restrict__ a, V
     __shared__ T red[256];
     T acc = T(0);
     const int64_t step = static_cast<int64_t>(gridDim.x) * blockDim.x;
-    for (int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < numel; i += step)
+    int64_t first = 0;  // elements [0, first) are covered by 16-byte loads
+    if (dense && reinterpret_cast<uintptr_t>(a) % 16 == 0) {
+        constexpr int N = 16 / sizeof(T);
+        const int64_t nvec = numel / N;
+        for (int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < nvec; i += step) {
+            const vec_t<T, N> x = reinterpret_cast<const vec_t<T, N> *>(a)[i];
+#pragma unroll
+            for (int j = 0; j < N; ++j) acc = static_cast<T>(acc + x[j]);
+        }
+        first = nvec * N;
+    }
+    for (int64_t i = first + static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < numel; i += step)
         acc = static_cast<T>(acc + (dense ? a[i] : a[flat_of(i, v)]));
     red[threadIdx.x] = acc;
     __syncthreads();
@@ -228,6 +397,20 @@ __global__ void __launch_bounds__(256) cast_kernel(const T *__restrict__ a, View
     }
 }
 
+template <typename T, typename R>
+__global__ void __launch_bounds__(256) cast_vec_kernel(const T *__restrict__ a, R *__restrict__ out, int64_t nvec) {
+    constexpr int N = 16 / sizeof(T);
+    const int64_t step = static_cast<int64_t>(gridDim.x) * blockDim.x;
+    for (int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < nvec; i += step) {
+        const vec_t<T, N> x = reinterpret_cast<const vec_t<T, N> *>(a)[i];
+        R r[N];
+#pragma unroll
+        for (int j = 0; j < N; ++j) r[j] = static_cast<R>(x[j]);
+#pragma unroll
+        for (int j = 0; j < N; ++j) out[i * N + j] = r[j];  // consecutive stores of one lane merge into vector stores
+    }
+}
+
 // assign: lhs_view[i] = rhs_view[i] over one shape (tinytensor/tensor/backend/cpu/kernel/assign.hpp:15-21).
 // Moves raw bytes, so one kernel per element size serves every dtype.
 template <typename W>
@@ -273,11 +456,23 @@ ttamd_status make_view(const char *who, int ndim, const int64_t *shape, const in
     return TTAMD_OK;
 }
 
+inline bool aligned16(const void *p) { return reinterpret_cast<uintptr_t>(p) % 16 == 0; }
+
 template <typename T, int OP>
 ttamd_status launch_binary_op(const void *a, const ViewDesc &va, const void *b, const ViewDesc &vb, void *out, int64_t numel, hipStream_t st) {
-    if (is_dense(va) && is_dense(vb))
-        binary_kernel<T, OP, true><<<dim3(grid_for(numel)), dim3(256), 0, st>>>(static_cast<const T *>(a), va, static_cast<const T *>(b), vb, out, numel);
-    else
+    if (is_dense(va) && is_dense(vb)) {
+        using R = std::conditional_t<(OP >= BIN_LT), uint8_t, T>;  // comparisons yield bool bytes
+        constexpr int N = 16 / sizeof(T);
+        int64_t done = 0;
+        if (aligned16(a) && aligned16(b) && aligned16(out) && numel >= N) {
+            const int64_t nvec = numel / N;
+            binary_vec_kernel<T, OP><<<dim3(grid_for(nvec)), dim3(256), 0, st>>>(static_cast<const T *>(a), static_cast<const T *>(b), out, nvec);
+            done = nvec * N;
+        }
+        if (done < numel)
+            binary_kernel<T, OP, true><<<dim3(1), dim3(256), 0, st>>>(static_cast<const T *>(a) + done, va, static_cast<const T *>(b) + done, vb,
+                                                                     static_cast<R *>(out) + done, numel - done);
+    } else
         binary_kernel<T, OP, false><<<dim3(grid_for(numel)), dim3(256), 0, st>>>(static_cast<const T *>(a), va, static_cast<const T *>(b), vb, out, numel);
     TTAMD_HIP_CHECK(hipGetLastError());
     return TTAMD_OK;
@@ -298,8 +493,17 @@ template <typename T, int OP = 0>
 ttamd_status dispatch_unary(int op, const void *a, const ViewDesc &va, void *out, int64_t numel, hipStream_t st) {
     if constexpr (OP < UN_COUNT) {
         if (op == OP) {
-            if (is_dense(va)) unary_kernel<T, OP, true><<<dim3(grid_for(numel)), dim3(256), 0, st>>>(static_cast<const T *>(a), va, static_cast<T *>(out), numel);
-            else unary_kernel<T, OP, false><<<dim3(grid_for(numel)), dim3(256), 0, st>>>(static_cast<const T *>(a), va, static_cast<T *>(out), numel);
+            if (is_dense(va)) {
+                constexpr int N = 16 / sizeof(T);
+                int64_t done = 0;
+                if (aligned16(a) && aligned16(out) && numel >= N) {
+                    const int64_t nvec = numel / N;
+                    unary_vec_kernel<T, OP><<<dim3(grid_for(nvec)), dim3(256), 0, st>>>(static_cast<const T *>(a), static_cast<T *>(out), nvec);
+                    done = nvec * N;
+                }
+                if (done < numel)
+                    unary_kernel<T, OP, true><<<dim3(1), dim3(256), 0, st>>>(static_cast<const T *>(a) + done, va, static_cast<T *>(out) + done, numel - done);
+            } else unary_kernel<T, OP, false><<<dim3(grid_for(numel)), dim3(256), 0, st>>>(static_cast<const T *>(a), va, static_cast<T *>(out), numel);
             TTAMD_HIP_CHECK(hipGetLastError());
             return TTAMD_OK;
         }
@@ -314,7 +518,7 @@ template <typename T>
 ttamd_status sum_typed(int device, const void *a, const ViewDesc &v, int64_t numel, int dim, void *out, hipStream_t st) {
     const T *src = static_cast<const T *>(a);
     if (dim < 0) {
-        const unsigned blocks = numel > 256 * 64 ? 256 : 1;
+        const unsigned blocks = numel > (1 << 22) ? 2048 : (numel > 256 * 64 ? 256 : 1);
         if (blocks == 1) {
             sum_all_kernel<T><<<dim3(1), dim3(256), 0, st>>>(src, v, is_dense(v), numel, static_cast<T *>(out));
         } else {
@@ -355,7 +559,17 @@ struct BoolByte {
 
 template <typename T, typename R>
 ttamd_status launch_cast(const void *a, const ViewDesc &va, void *out, int64_t numel, hipStream_t st) {
-    cast_kernel<T, R><<<dim3(grid_for(numel)), dim3(256), 0, st>>>(static_cast<const T *>(a), va, is_dense(va), static_cast<R *>(out), numel);
+    constexpr int N = 16 / sizeof(T);
+    const bool dense = is_dense(va);
+    int64_t done = 0;
+    if (dense && aligned16(a) && aligned16(out) && numel >= N) {
+        const int64_t nvec = numel / N;
+        cast_vec_kernel<T, R><<<dim3(grid_for(nvec)), dim3(256), 0, st>>>(static_cast<const T *>(a), static_cast<R *>(out), nvec);
+        done = nvec * N;
+    }
+    if (done < numel)
+        cast_kernel<T, R><<<dim3(grid_for(numel - done)), dim3(256), 0, st>>>(static_cast<const T *>(a) + (dense ? done : 0), va, dense,
+                                                                             static_cast<R *>(out) + done, numel - done);
     TTAMD_HIP_CHECK(hipGetLastError());
     return TTAMD_OK;
 }
@@ -586,8 +800,21 @@ ttamd_status ttamd_where(int device, ttamd_dtype dtype, int ndim, const int64_t 
     hipStream_t st = static_cast<hipStream_t>(stream);
     auto run = [&](auto tag) -> ttamd_status {
         using T = decltype(tag);
-        where_kernel<T><<<dim3(grid_for(numel)), dim3(256), 0, st>>>(c, vc, static_cast<const T *>(a), va, static_cast<const T *>(b), vb,
-                                                                   static_cast<T *>(out), numel);
+        constexpr int N = 16 / sizeof(T);
+        int64_t done = 0;
+        const bool dense = is_dense(vc) && is_dense(va) && is_dense(vb);
+        if (dense && aligned16(c) && aligned16(a) && aligned16(b) && aligned16(out) && numel >= N) {
+            const int64_t nvec = numel / N;
+            where_vec_kernel<T><<<dim3(grid_for(nvec)), dim3(256), 0, st>>>(c, static_cast<const T *>(a), static_cast<const T *>(b),
+                                                                          static_cast<T *>(out), nvec);
+            done = nvec * N;
+        }
+        if (done < numel) {
+            const int64_t skip = dense ? done : 0;  // a dense tail continues behind the vectors
+            where_kernel<T><<<dim3(grid_for(numel - done)), dim3(256), 0, st>>>(c + skip, vc, static_cast<const T *>(a) + skip, va,
+                                                                              static_cast<const T *>(b) + skip, vb,
+                                                                              static_cast<T *>(out) + done, numel - done);
+        }
         TTAMD_HIP_CHECK(hipGetLastError());
         return TTAMD_OK;
     };

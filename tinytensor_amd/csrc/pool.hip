@@ -14,6 +14,9 @@
 // Backward is the gather form of the reference's scatter-add: the lane that owns input (y, x) walks the outputs
 // whose window contains it in increasing (h, w) — the order in which the reference's loop adds to that
 // element — so the sums are bit-identical too, and nothing is written twice (no atomics, no zero-fill pass).
+// For max / min a first pass over the outputs computes each output's share (gradient / number of window elements
+// equal to the result) into the library's per-stream scratch, so the gather reads two values per covering output
+// instead of recounting its window.
 #include "common.h"
 
 #include <cfloat>
@@ -28,6 +31,10 @@ enum { POOL_MAX = 0, POOL_MIN = 1, POOL_AVG = 2 };
 struct PoolGeom {
     int B, C, H, W, K, S, P, Ho, Wo;
     int64_t xs_b, xs_c, xs_h, xs_w;  // input strides (elements)
+    // Work is laid out as (plane = b*C + c, block of 256 positions inside the plane) so that every index fits 32
+    // bits and is split with exact multiply-shift division instead of 64-bit division.
+    int out_blocks, in_blocks;        // blocks of 256 positions per output / input plane
+    FastDiv d_out_blocks, d_in_blocks, d_C, d_Wo, d_W, d_S;
 };
 
 template <typename R, int OP>
@@ -44,77 +51,102 @@ __device__ __forceinline__ R pool_init() {
     }
 }
 
+// Input plane of (b, c) through the view's strides.
+template <typename T>
+__device__ __forceinline__ const T *plane_of(const PoolGeom &g, const T *x, uint32_t plane) {
+    uint32_t b, c;
+    g.d_C.divmod(plane, b, c);
+    return x + static_cast<int64_t>(b) * g.xs_b + static_cast<int64_t>(c) * g.xs_c;
+}
+
 template <typename T, typename R, int OP>
-__global__ void __launch_bounds__(256) pool_forward_kernel(PoolGeom g, const T *__restrict__ x, R *__restrict__ out, int64_t total) {
-    const int64_t idx = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
-    if (idx >= total) return;
-    const int w = static_cast<int>(idx % g.Wo);
-    const int h = static_cast<int>((idx / g.Wo) % g.Ho);
-    const int64_t bc = idx / (static_cast<int64_t>(g.Wo) * g.Ho);
-    const int c = static_cast<int>(bc % g.C);
-    const int64_t b = bc / g.C;
-    const T *plane = x + b * g.xs_b + c * g.xs_c;
+__global__ void __launch_bounds__(256) pool_forward_kernel(PoolGeom g, const T *__restrict__ x, R *__restrict__ out) {
+    uint32_t plane, blk;
+    g.d_out_blocks.divmod(blockIdx.x, plane, blk);
+    const uint32_t pos = blk * 256 + threadIdx.x;
+    if (pos >= static_cast<uint32_t>(g.Ho * g.Wo)) return;
+    uint32_t h, w;
+    g.d_Wo.divmod(pos, h, w);
+    const T *src = plane_of(g, x, plane);
     const R n = static_cast<R>(g.K * g.K);
     R acc = pool_init<R, OP>();
     for (int p = 0; p < g.K; ++p) {
-        const int hi = g.S * h + p - g.P;
+        const int hi = g.S * static_cast<int>(h) + p - g.P;
         for (int q = 0; q < g.K; ++q) {
-            const int wi = g.S * w + q - g.P;
+            const int wi = g.S * static_cast<int>(w) + q - g.P;
             const bool in = !(hi < 0 || wi < 0 || hi >= g.H || wi >= g.W);
-            const R v = in ? static_cast<R>(plane[hi * g.xs_h + wi * g.xs_w]) : pool_init<R, OP>();
+            const R v = in ? static_cast<R>(src[hi * g.xs_h + wi * g.xs_w]) : pool_init<R, OP>();
             if constexpr (OP == POOL_MAX) acc = (v > acc) ? v : acc;
             else if constexpr (OP == POOL_MIN) acc = (v < acc) ? v : acc;
             else acc = (v / n) + acc;
         }
     }
-    out[idx] = acc;
+    out[static_cast<int64_t>(plane) * (g.Ho * g.Wo) + pos] = acc;
 }
 
-// floor(a / b) for b > 0 and any a
-__device__ __forceinline__ int floor_div(int a, int b) { return a >= 0 ? a / b : -((-a + b - 1) / b); }
+// max / min backward, first pass (one lane per output): share = grad_out / (number of in-bounds window elements
+// equal to the result), the amount each of those elements receives from this output (cpu/kernel/conv.hpp:188-203).
+template <typename R>
+__global__ void __launch_bounds__(256)
+pool_share_kernel(PoolGeom g, const R *__restrict__ gout, const R *__restrict__ x, const R *__restrict__ res, R *__restrict__ share) {
+    uint32_t plane, blk;
+    g.d_out_blocks.divmod(blockIdx.x, plane, blk);
+    const uint32_t pos = blk * 256 + threadIdx.x;
+    if (pos >= static_cast<uint32_t>(g.Ho * g.Wo)) return;
+    uint32_t h, w;
+    g.d_Wo.divmod(pos, h, w);
+    const R *src = plane_of(g, x, plane);
+    const int64_t o = static_cast<int64_t>(plane) * (g.Ho * g.Wo) + pos;
+    const R target = res[o];
+    R count = R(0);
+    for (int p = 0; p < g.K; ++p)
+        for (int q = 0; q < g.K; ++q) {
+            const int hi = g.S * static_cast<int>(h) + p - g.P, wi = g.S * static_cast<int>(w) + q - g.P;
+            const bool in = !(hi < 0 || wi < 0 || hi >= g.H || wi >= g.W);
+            count += (in && src[hi * g.xs_h + wi * g.xs_w] == target) ? R(1) : R(0);
+        }
+    share[o] = gout[o] / count;
+}
 
+// Backward gather (one lane per input element): adds, in increasing (h, w), what each output whose window
+// contains the element hands to it.  SELECT: `share` holds the per-output amounts of pool_share_kernel and only
+// outputs whose result equals the element contribute; otherwise `share` is grad_out and every output
+// contributes grad_out / (k*k).
 template <typename R, bool SELECT>
 __global__ void __launch_bounds__(256)
-pool_backward_kernel(PoolGeom g, const R *__restrict__ gout, const R *__restrict__ x, const R *__restrict__ res, R *__restrict__ gin,
-                     int64_t total) {
-    const int64_t idx = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
-    if (idx >= total) return;
-    const int xw = static_cast<int>(idx % g.W);
-    const int yh = static_cast<int>((idx / g.W) % g.H);
-    const int64_t bc = idx / (static_cast<int64_t>(g.W) * g.H);
-    const int c = static_cast<int>(bc % g.C);
-    const int64_t b = bc / g.C;
-    const R *plane = x + b * g.xs_b + c * g.xs_c;
-    const R *gplane = gout + bc * g.Ho * g.Wo;
-    const R *rplane = res + bc * g.Ho * g.Wo;
-    const R mine = plane[yh * g.xs_h + xw * g.xs_w];
-    // outputs h with 0 <= yh + P - S*h < K
-    int h_lo = floor_div(yh + g.P - g.K, g.S) + 1, h_hi = floor_div(yh + g.P, g.S);
-    int w_lo = floor_div(xw + g.P - g.K, g.S) + 1, w_hi = floor_div(xw + g.P, g.S);
-    h_lo = h_lo < 0 ? 0 : h_lo;
-    w_lo = w_lo < 0 ? 0 : w_lo;
+pool_backward_kernel(PoolGeom g, const R *__restrict__ share, const R *__restrict__ x, const R *__restrict__ res, R *__restrict__ gin) {
+    uint32_t plane, blk;
+    g.d_in_blocks.divmod(blockIdx.x, plane, blk);
+    const uint32_t pos = blk * 256 + threadIdx.x;
+    if (pos >= static_cast<uint32_t>(g.H * g.W)) return;
+    uint32_t yh, xw;
+    g.d_W.divmod(pos, yh, xw);
+    const int64_t obase = static_cast<int64_t>(plane) * (g.Ho * g.Wo);
+    const R *splane = share + obase;
+    // outputs h with 0 <= yh + P - S*h < K, clipped to [0, Ho)
+    const int ay = static_cast<int>(yh) + g.P, ax = static_cast<int>(xw) + g.P;
+    int h_lo = ay - g.K >= 0 ? static_cast<int>(g.d_S.div(static_cast<uint32_t>(ay - g.K))) + 1 : 0;
+    int w_lo = ax - g.K >= 0 ? static_cast<int>(g.d_S.div(static_cast<uint32_t>(ax - g.K))) + 1 : 0;
+    int h_hi = static_cast<int>(g.d_S.div(static_cast<uint32_t>(ay))), w_hi = static_cast<int>(g.d_S.div(static_cast<uint32_t>(ax)));
     h_hi = h_hi >= g.Ho ? g.Ho - 1 : h_hi;
     w_hi = w_hi >= g.Wo ? g.Wo - 1 : w_hi;
     R acc = R(0);
-    for (int h = h_lo; h <= h_hi; ++h)
-        for (int w = w_lo; w <= w_hi; ++w) {
-            const R go = gplane[h * g.Wo + w];
-            if constexpr (SELECT) {
-                const R target = rplane[h * g.Wo + w];
-                if (!(mine == target)) continue;
-                R count = R(0);
-                for (int p = 0; p < g.K; ++p)
-                    for (int q = 0; q < g.K; ++q) {
-                        const int hi = g.S * h + p - g.P, wi = g.S * w + q - g.P;
-                        const bool in = !(hi < 0 || wi < 0 || hi >= g.H || wi >= g.W);
-                        count += (in && plane[hi * g.xs_h + wi * g.xs_w] == target) ? R(1) : R(0);
-                    }
-                acc += go / count;
-            } else {
-                acc += go / static_cast<R>(g.K * g.K);
+    if constexpr (SELECT) {
+        const R mine = plane_of(g, x, plane)[static_cast<int64_t>(yh) * g.xs_h + static_cast<int64_t>(xw) * g.xs_w];
+        const R *rplane = res + obase;
+        for (int h = h_lo; h <= h_hi; ++h)
+            for (int w = w_lo; w <= w_hi; ++w) {
+                // both loads are issued before the comparison (no dependent second access); an output that does not
+                // select this element adds +0, which leaves the running sum's bits unchanged
+                const R target = rplane[h * g.Wo + w], amount = splane[h * g.Wo + w];
+                acc += (mine == target) ? amount : R(0);
             }
-        }
-    gin[idx] = acc;
+    } else {
+        const R n = static_cast<R>(g.K * g.K);
+        for (int h = h_lo; h <= h_hi; ++h)
+            for (int w = w_lo; w <= w_hi; ++w) acc += splane[h * g.Wo + w] / n;
+    }
+    gin[static_cast<int64_t>(plane) * (g.H * g.W) + pos] = acc;
 }
 
 ttamd_status make_pool_geom(const char *who, int op, const ttamd_view4 *input, int B, int C, int H, int W, int k, int stride,
@@ -144,18 +176,30 @@ ttamd_status make_pool_geom(const char *who, int op, const ttamd_view4 *input, i
     g->Ho = (H + 2 * padding - k) / stride + 1;
     g->Wo = (W + 2 * padding - k) / stride + 1;
     g->xs_b = input->stride[0]; g->xs_c = input->stride[1]; g->xs_h = input->stride[2]; g->xs_w = input->stride[3];
+    const int64_t in_plane = static_cast<int64_t>(H) * W, out_plane = static_cast<int64_t>(g->Ho) * g->Wo;
+    const int64_t planes = static_cast<int64_t>(B) * C;
+    const int64_t in_blocks = (in_plane + 255) / 256, out_blocks = (out_plane + 255) / 256;
+    if (in_plane >= 0x7fffffff || static_cast<int64_t>(H - 1) * g->xs_h + static_cast<int64_t>(W - 1) * g->xs_w >= 0x7fffffff ||
+        planes * in_blocks >= 0x7fffffff || planes * (out_blocks > 0 ? out_blocks : 1) >= 0x7fffffff || k >= (1 << 14) ||
+        padding >= (1 << 14)) {
+        set_error("%s: the tensor exceeds the 32-bit plane / launch range of the pooling kernels", who);
+        return TTAMD_ERR_INVALID_ARGUMENT;
+    }
+    g->in_blocks = static_cast<int>(in_blocks);
+    g->out_blocks = static_cast<int>(out_blocks > 0 ? out_blocks : 1);
+    g->d_in_blocks = make_fastdiv(static_cast<uint32_t>(g->in_blocks));
+    g->d_out_blocks = make_fastdiv(static_cast<uint32_t>(g->out_blocks));
+    g->d_C = make_fastdiv(static_cast<uint32_t>(C));
+    g->d_Wo = make_fastdiv(static_cast<uint32_t>(g->Wo > 0 ? g->Wo : 1));
+    g->d_W = make_fastdiv(static_cast<uint32_t>(W));
+    g->d_S = make_fastdiv(static_cast<uint32_t>(stride));
     return TTAMD_OK;
 }
 
 template <typename T, typename R, int OP>
 ttamd_status launch_forward(const PoolGeom &g, const void *x, void *out, hipStream_t st) {
-    const int64_t total = static_cast<int64_t>(g.B) * g.C * g.Ho * g.Wo;
-    const int64_t blocks = (total + 255) / 256;
-    if (blocks > 0x7fffffff) {
-        set_error("pool2d: too many workgroups");
-        return TTAMD_ERR_INVALID_ARGUMENT;
-    }
-    pool_forward_kernel<T, R, OP><<<dim3(static_cast<unsigned>(blocks)), dim3(256), 0, st>>>(g, static_cast<const T *>(x), static_cast<R *>(out), total);
+    const unsigned blocks = static_cast<unsigned>(static_cast<int64_t>(g.B) * g.C * g.out_blocks);
+    pool_forward_kernel<T, R, OP><<<dim3(blocks), dim3(256), 0, st>>>(g, static_cast<const T *>(x), static_cast<R *>(out));
     TTAMD_HIP_CHECK(hipGetLastError());
     return TTAMD_OK;
 }
@@ -169,20 +213,22 @@ ttamd_status forward_typed(int op, const PoolGeom &g, const void *x, void *out, 
 }
 
 template <typename R>
-ttamd_status backward_typed(int op, const PoolGeom &g, const void *gout, const void *x, const void *res, void *gin, hipStream_t st) {
-    const int64_t total = static_cast<int64_t>(g.B) * g.C * g.H * g.W;
-    const int64_t blocks = (total + 255) / 256;
-    if (blocks > 0x7fffffff) {
-        set_error("pool2d_backward: too many workgroups");
-        return TTAMD_ERR_INVALID_ARGUMENT;
+ttamd_status backward_typed(int device, int op, const PoolGeom &g, const void *gout, const void *x, const void *res, void *gin,
+                            hipStream_t st) {
+    const int64_t planes = static_cast<int64_t>(g.B) * g.C;
+    const dim3 in_grid(static_cast<unsigned>(planes * g.in_blocks)), out_grid(static_cast<unsigned>(planes * g.out_blocks)), block(256);
+    if (op == POOL_AVG) {
+        pool_backward_kernel<R, false><<<in_grid, block, 0, st>>>(g, static_cast<const R *>(gout), static_cast<const R *>(x),
+                                                                  static_cast<const R *>(res), static_cast<R *>(gin));
+    } else {
+        void *share = nullptr;
+        const size_t bytes = static_cast<size_t>(planes) * g.Ho * g.Wo * sizeof(R);
+        if (ttamd_status s = stream_scratch(device, st, bytes ? bytes : sizeof(R), &share)) return s;
+        pool_share_kernel<R><<<out_grid, block, 0, st>>>(g, static_cast<const R *>(gout), static_cast<const R *>(x),
+                                                         static_cast<const R *>(res), static_cast<R *>(share));
+        pool_backward_kernel<R, true><<<in_grid, block, 0, st>>>(g, static_cast<const R *>(share), static_cast<const R *>(x),
+                                                                 static_cast<const R *>(res), static_cast<R *>(gin));
     }
-    const dim3 grid(static_cast<unsigned>(blocks)), block(256);
-    if (op == POOL_AVG)
-        pool_backward_kernel<R, false><<<grid, block, 0, st>>>(g, static_cast<const R *>(gout), static_cast<const R *>(x),
-                                                               static_cast<const R *>(res), static_cast<R *>(gin), total);
-    else
-        pool_backward_kernel<R, true><<<grid, block, 0, st>>>(g, static_cast<const R *>(gout), static_cast<const R *>(x),
-                                                              static_cast<const R *>(res), static_cast<R *>(gin), total);
     TTAMD_HIP_CHECK(hipGetLastError());
     return TTAMD_OK;
 }
@@ -237,8 +283,8 @@ ttamd_status ttamd_pool2d_backward(int device, ttamd_dtype dtype, int op, const 
     }
     const void *x = static_cast<const char *>(input->data) + input->offset * static_cast<int64_t>(dtype_size(dtype));
     hipStream_t st = static_cast<hipStream_t>(stream);
-    if (dtype == TTAMD_F32) return backward_typed<float>(op, g, grad_out, x, result, grad_input, st);
-    return backward_typed<double>(op, g, grad_out, x, result, grad_input, st);
+    if (dtype == TTAMD_F32) return backward_typed<float>(device, op, g, grad_out, x, result, grad_input, st);
+    return backward_typed<double>(device, op, g, grad_out, x, result, grad_input, st);
 }
 
 }  // extern "C"
