@@ -156,11 +156,12 @@ def detail_report(tt, np, path, cpu=True):
 
     n = 8192
     Ea = tt.Tensor.from_numpy(np.random.default_rng(0).random((n, n), dtype=f32))
+    Eb = tt.Tensor.from_numpy(np.random.default_rng(2).random((n, n), dtype=f32))
     Eo = tt.Tensor.empty((n, n), cap.F32)
     Eo64 = tt.Tensor.empty((n, n), cap.F64)
     sh, st, stT = i64((n, n)), i64((n, 1)), i64((1, n))
     stream_case("add 8192x8192 f32", "binary_kernel", 3 * n * n * 4,
-                lambda: lib.ttamd_binary(0, cap.F32, cap.BIN["add"], 2, sh, ptr(Ea), 0, st, ptr(Ea), 0, st, ptr(Eo), None))
+                lambda: lib.ttamd_binary(0, cap.F32, cap.BIN["add"], 2, sh, ptr(Ea), 0, st, ptr(Eb), 0, st, ptr(Eo), None))
     stream_case("relu 8192x8192 f32", "unary_kernel", 2 * n * n * 4,
                 lambda: lib.ttamd_unary(0, cap.F32, cap.UN["relu"], 2, sh, ptr(Ea), 0, st, ptr(Eo), None))
     stream_case("contiguous of a transposed 8192x8192 f32 view", "contiguous_kernel", 2 * n * n * 4,
@@ -171,8 +172,8 @@ def detail_report(tt, np, path, cpu=True):
                 lambda: lib.ttamd_sum(0, cap.F32, 2, sh, ptr(Ea), 0, st, -1, ptr(Eo), None))
     m = 1024
     shm, stm = i64((m, m)), i64((m, 1))
-    stream_case("cfg5 bias-free add 1024x1024 f32", "binary_kernel", 3 * m * m * 4,
-                lambda: lib.ttamd_binary(0, cap.F32, cap.BIN["add"], 2, shm, ptr(Ea), 0, stm, ptr(Ea), 0, stm, ptr(Eo), None), 200)
+    stream_case("cfg5 add 1024x1024 f32", "binary_kernel", 3 * m * m * 4,
+                lambda: lib.ttamd_binary(0, cap.F32, cap.BIN["add"], 2, shm, ptr(Ea), 0, stm, ptr(Eb), 0, stm, ptr(Eo), None), 200)
     # pooling on [64,64,112,112] f32 (205 MB): k2 s2 p0 and k3 s2 p1
     Pb, Pc, Ph, Pw = 64, 64, 112, 112
     Px = tt.Tensor.from_numpy(np.random.default_rng(1).random((Pb, Pc, Ph, Pw), dtype=f32))
