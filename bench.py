@@ -245,6 +245,8 @@ def main():
     ap.add_argument("--copy-calibration", action="store_true",
                     help="first run one dense 256 MiB copy kernel (known HBM traffic) to scale profiler byte counters")
     ap.add_argument("--detail", metavar="FILE", help="also time every BASELINE configuration and write a JSON report")
+    ap.add_argument("--conv-loop", type=int, metavar="N", default=0,
+                    help="only run N conv2d forward + backward passes of BASELINE config 4 (a short target for profilers) and exit")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
@@ -259,6 +261,22 @@ def main():
         src = tt.Tensor.empty((64 * 1024 * 1024,), tt._capi.F32)
         tt.get_backend(tt.kAMD).identity(tt.Tensor(src.storage, src.dtype, (8192, 8192), (8192, 1), 0))
         tt.get_backend(tt.kAMD).synchronize(0)
+
+    if args.conv_loop:
+        be = tt.get_backend(tt.kAMD)
+        rng = np.random.default_rng(0)
+        x = tt.Tensor.from_numpy(rng.normal(0, 0.1, (64, 32, 28, 28)).astype(np.float32))
+        w = tt.Tensor.from_numpy(rng.normal(0, 0.1, (64, 32, 3, 3)).astype(np.float32))
+        out = be.conv2d(x, w, None, 1, 1)
+        go = tt.Tensor.from_numpy(np.ones(out.shape, np.float32))
+        be.conv2d_backward(go, x, w, None, 1, 1)
+        bufs = be.last_conv_buffers
+        for _ in range(args.conv_loop):
+            be.conv2d(x, w, None, 1, 1, out=out)
+            be.conv2d_backward(go, x, w, None, 1, 1, buffers=bufs)
+        be.synchronize(0)
+        print(json.dumps({"conv_loop": args.conv_loop, "config": "configs[3]: input [64,32,28,28], weight [64,32,3,3], s1 p1, f32"}))
+        return
 
     if args.detail:
         detail_report(tt, np, args.detail, cpu=not args.no_cpu)
