@@ -22,7 +22,11 @@
  *                         parity is tolerance based.
  *   tto_contiguous        brute force against explicit nested-loop indexing.
  *   tto_conv2d_*          naive 7-deep loop (reference test oracle), adjoint
- *                         identities for the backward pass.
+ *                         identities for the backward pass, and torch's CPU conv2d
+ *                         and its autograd on the shapes of the reference's TT_TORCH
+ *                         tests (tests/test_conv.cpp:147-184,
+ *                         tests/test_conv_autograd.cpp:43-107).
+ *   tto_batched_matmul backward  torch autograd on tests/test_matmul_autograd.cpp:218-262.
  *   tto_pool2d_*          torch.nn.functional max_pool2d / avg_pool2d and their autograd on
  *                         the reference tests' shapes (what tests/test_conv.cpp:186-278 and
  *                         tests/test_conv_autograd.cpp:109-230 compare with), plus a
