@@ -91,7 +91,7 @@ def time_launches(tt, fn, iters, warmup):
 
 
 def detail_report(tt, np, path, cpu=True):
-    """Times every BASELINE configuration (GPU only, inputs resident) and writes a JSON report to `path`.
+    """Times every benchmark configuration (GPU only, inputs resident) and writes a JSON report to `path`.
     Not part of the one-line contract; used to track the small-shape, strided and conv paths."""
     from oracle import tt_oracle as oracle  # seeded input generation only
 
@@ -244,9 +244,9 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="first run one dense 256 MiB copy kernel (known HBM traffic) to scale profiler byte counters")
-    ap.add_argument("--detail", metavar="FILE", help="also time every BASELINE configuration and write a JSON report")
+    ap.add_argument("--detail", metavar="FILE", help="also time every benchmark configuration and write a JSON report")
     ap.add_argument("--conv-loop", type=int, metavar="N", default=0,
-                    help="only run N conv2d forward + backward passes of BASELINE config 4 (a short target for profilers) and exit")
+                    help="only run N conv2d forward + backward passes of benchmark configuration 4 (input [64,32,28,28], weight [64,32,3,3], s1 p1) (a short target for profilers) and exit")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)

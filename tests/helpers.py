@@ -66,7 +66,7 @@ def naive_exact(A, B):
     return full.astype(np.dtype(f"uint{bits}")).view(dt) if dt != np.uint8 else full.astype(np.uint8)
 
 
-# ---- MLP training step of BASELINE config 5, written once over an abstract GEMM --------------------------
+# ---- MLP training step of benchmark configuration 5, written once over an abstract GEMM --------------------------
 def mlp_train_step(X, T, params, mm, mm_bwd, masks=None):
     """One forward + backward of Linear-ReLU-Linear-ReLU-Linear + mse_loss(mean), following the reference's
     op sequence: nn::Linear::forward = matmul + bias.expand (nn/linear.cpp:42-50), relu backward mask

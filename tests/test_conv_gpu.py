@@ -129,7 +129,7 @@ def test_unaligned_window_of_a_larger_image(tt, oracle, dtype):
 
 
 def test_config4_conv_forward_backward(tt, oracle):
-    # BASELINE config 4: input [64,32,28,28], weight [64,32,3,3], stride 1, padding 1, normal(0, 0.1) from a seed.
+    # benchmark configuration 4: input [64,32,28,28], weight [64,32,3,3], stride 1, padding 1, normal(0, 0.1) from a seed.
     x = oracle.Generator(0).normal(0.0, 0.1, (64, 32, 28, 28))
     w = oracle.Generator(1).normal(0.0, 0.1, (64, 32, 3, 3))
     tx, tw = dev(tt, x), dev(tt, w)

@@ -104,7 +104,7 @@ def test_sum_and_full(tt, dtype):
 
 
 def mlp_step_on_device(tt, X, T, params):
-    """The training step of BASELINE config 5 with every op on the device: fused Linear(+bias) GEMMs, relu, mse_loss
+    """The training step of benchmark configuration 5 with every op on the device: fused Linear(+bias) GEMMs, relu, mse_loss
     as pow(y - t, 2).mean(), and the backward pass op for op as the reference's autograd emits it
     (autograd/unary_ops.cpp:568-573, binary_ops.cpp:173-179, reduce_ops.cpp:201-205; bias grads = sum over dim 0)."""
     d = lambda a: tt.Tensor.from_numpy(a)

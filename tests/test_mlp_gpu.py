@@ -1,4 +1,4 @@
-"""BASELINE config 5 on the GPU: one MLP training step (batch 1024, 784 -> 1024 -> 1024 -> 10, ReLU, mse_loss),
+"""Benchmark configuration 5 on the GPU: one MLP training step (batch 1024, 784 -> 1024 -> 1024 -> 10, ReLU, mse_loss),
 every GEMM of the forward and backward pass through the C ABI (nine products, including the skinny N = 10 and
 K = 10 ones and the A.B^T / A^T.B products on permuted views), compared with the same step over the CPU oracle.
 Tolerance: max relative error <= 1e-4 per tensor (f32)."""

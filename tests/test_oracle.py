@@ -173,7 +173,7 @@ def test_matmul_kernel_close_to_high_precision(oracle, dtype, tol):
 
 
 def test_batched_matmul_views_equal_dense_copies(oracle):
-    # BASELINE config 2: B is a transposed view of a [32,128,64] tensor.
+    # benchmark configuration 2: B is a transposed view of a [32,128,64] tensor.
     A = oracle.Generator(0).uniform_real(-1, 1, (32, 128, 64))
     Bsrc = oracle.Generator(1).uniform_real(-1, 1, (32, 128, 64))
     Bv = Bsrc.transpose(0, 2, 1)
