@@ -225,8 +225,8 @@ ttamd_status launch_mfma_typed(const GemmArgs &g, int device, hipStream_t stream
         const double round_time = 2.0 * bm_ * bn_ * static_cast<double>(g.K) * slots / (rate * scale);
         return (rounds + last) * round_time;
     };
-    const double t_small = estimate(TS::SBM, TS::SBN, 4, 119e12);
-    const double t_large = vec ? estimate(TS::LBM, TS::LBN, 2, 133e12) : 1e300;
+    const double t_small = estimate(TS::SBM, TS::SBN, 4, 131e12);
+    const double t_large = vec ? estimate(TS::LBM, TS::LBN, 2, 131e12) : 1e300;
     const double t_xl = (TS::kHasXL && vec) ? estimate(TS::XBM, TS::XBN, 2, 141e12) : 1e300;
     const bool xl = t_xl <= t_large && t_xl <= t_small;
     const bool large = !xl && t_large <= t_small;

@@ -325,6 +325,13 @@ struct TileEngine {
     static constexpr size_t kLdsBytes = 2 * (StA::LDS_ELEMS + StB::LDS_ELEMS) * sizeof(T);
 
     typename M::acc_t acc[NBM][NBN];
+    // The rotated schedule (see step()) pays off for waves with few MFMA blocks (64 x 64 tiles: +9 % at 2048^3).
+    // It keeps one more pair of fragments live across the barrier, which the tiles with 8 or 16 blocks per wave
+    // cannot afford (128 accumulator registers: fp64 spills, fp32 256 x 128 measured 1.5 % slower), so they keep
+    // the plain schedule.
+    static constexpr bool kRotate = NBM * NBN <= 4;
+    FrA last_a;  // fragments of the previous tile's last chunk, multiplied after the barrier
+    FrB last_b;
     int lane, wm0, wn0;
 
     __device__ __forceinline__ void init(int tid) {
@@ -340,8 +347,140 @@ struct TileEngine {
                 for (int e = 0; e < M::NACC; ++e) acc[i][j][e] = T(0);
     }
 
+    // ---- rotated schedule (tiles with at most 4 MFMA blocks per wave) ----
+    __device__ __forceinline__ void read_frags(const T *smem, int buf, int chunk, FrA &fa, FrB &fb) const {
+        fa.read(smem + buf * StA::LDS_ELEMS, wm0, chunk, lane);
+        fb.read(smem + kBOff + buf * StB::LDS_ELEMS, wn0, chunk, lane);
+    }
+    __device__ __forceinline__ void mma_chunk(const FrA &fa, const FrB &fb) {
+#pragma unroll
+        for (int j = 0; j < M::VK; ++j)
+#pragma unroll
+            for (int bm = 0; bm < NBM; ++bm)
+#pragma unroll
+                for (int bn = 0; bn < NBN; ++bn) acc[bm][bn] = M::mma(fa.v[bm][j], fb.v[bn][j], acc[bm][bn]);
+    }
+    // MFMA work of chunks [c0, c1) of the tile in LDS buffer `buf`; chunk 0 takes the fragments in (f0a, f0b),
+    // which were requested earlier.
+    __device__ __forceinline__ void compute_chunks(const T *smem, int buf, int c0, int c1, const FrA &f0a, const FrB &f0b) {
+#pragma unroll
+        for (int c = c0; c < c1; ++c) {
+            if (c == 0) {
+                mma_chunk(f0a, f0b);
+            } else {
+                FrA fa;
+                FrB fb;
+                read_frags(smem, buf, c, fa, fb);
+                mma_chunk(fa, fb);
+            }
+        }
+    }
+
+    // One pipeline step for tile kt.  The loop is rotated so that the barrier sits between reading the last chunk's
+    // fragments and multiplying them:
+    //   on entry the barrier that published tile kt has just been passed and (PENDING) the fragments of the
+    //   previous tile's last chunk wait in registers (last_a, last_b);
+    //   1. request chunk 0 of tile kt from LDS and (LOAD) tile kt + PF from memory into slot kt % PF;
+    //   2. multiply the pending chunk: its MFMAs cover the LDS latency of step 1, which is otherwise exposed after
+    //      every barrier when a SIMD has few waves to run;
+    //   3. multiply chunks 0 .. NC-2 of tile kt; during the last of them read the last chunk's fragments into
+    //      (last_a, last_b) and park tile kt + 1 (slot (kt + 1) % PF) in the other LDS buffer, its stores slotted
+    //      between the MFMAs;
+    //   4. barrier.
+    // The other LDS buffer was last read in part 3 of the previous step (before its barrier), so it may be
+    // overwritten here; tile kt's buffer is only read.
+    template <int S, bool LOAD, bool MASK, bool PENDING>
+    __device__ __forceinline__ void step_rot(StA &sa, StB &sb, T *smem, int K, int kt) {
+        constexpr int PF = StA::kPF;
+        constexpr int NC = BK / kChunk;
+        static_assert(NC >= 2, "a k tile holds at least two chunks");
+        constexpr int kChunkMfmas = M::VK * NBM * NBN;  // MFMAs of one chunk
+        constexpr int kStores = StA::P + StB::P;        // LDS store instructions of one tile (per lane)
+        const int cur = kt & 1;
+        FrA f0a;
+        FrB f0b;
+        read_frags(smem, cur, 0, f0a, f0b);
+        if constexpr (LOAD) {
+            const int k_left = K - (kt + PF) * BK;
+            sa.template load<MASK, S>(k_left);
+            sb.template load<MASK, S>(k_left);
+        }
+        __builtin_amdgcn_sched_barrier(0);  // keep the requests ahead of the MFMA work
+        if constexpr (PENDING) mma_chunk(last_a, last_b);
+        compute_chunks(smem, cur, 0, NC - 2, f0a, f0b);
+        __builtin_amdgcn_sched_barrier(0);
+        compute_chunks(smem, cur, NC - 2, NC - 1, f0a, f0b);
+        read_frags(smem, cur, NC - 1, last_a, last_b);
+        sa.template store<(S + 1) % PF>(smem + (cur ^ 1) * StA::LDS_ELEMS);
+        // Keep A's stores ahead of B's, the order in which their loads were issued: each store then waits only for
+        // the loads up to its own instead of for all of them.
+        asm volatile("" ::: "memory");
+        sb.template store<(S + 1) % PF>(smem + kBOff + (cur ^ 1) * StB::LDS_ELEMS);
+        if constexpr (kChunkMfmas >= 2 * kStores) {
+#pragma unroll
+            for (int i = 0; i < kStores; ++i) {
+                __builtin_amdgcn_sched_group_barrier(0x008, kChunkMfmas / kStores > 2 ? 2 : 1, 0);  // MFMA
+                __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);                                  // DS write
+            }
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        __syncthreads();
+    }
+
+    template <bool LOAD, bool MASK, bool PENDING, int S = 0>
+    __device__ __forceinline__ void step_any_rot(StA &sa, StB &sb, T *smem, int K, int kt, int slot) {
+        if constexpr (S < StA::kPF) {
+            if (slot == S) step_rot<S, LOAD, MASK, PENDING>(sa, sb, smem, K, kt);
+            else step_any_rot<LOAD, MASK, PENDING, S + 1>(sa, sb, smem, K, kt, slot);
+        }
+    }
+
+    __device__ __forceinline__ void run_rot(StA &sa, StB &sb, T *smem, int K, bool unmasked) {
+        constexpr int PF = StA::kPF;
+        constexpr int NC = BK / kChunk;
+        const int KT = (K + BK - 1) / BK;
+        // Prologue: tile 0 goes straight to LDS, tiles 1 .. PF-1 are put in flight.
+        sa.template load<true, 0>(K);
+        sb.template load<true, 0>(K);
+        sa.template store<0>(smem);
+        sb.template store<0>(smem + kBOff);
+        prefetch_rest<1>(sa, sb, K, KT);
+        __syncthreads();
+        // Tiles 0 .. KT-2; the first step has no pending chunk.  While kt + PF < KT a step also issues loads; the
+        // remaining steps only drain the slots.
+        auto pipeline = [&]<bool MASK>() {
+            int kt = 0, slot = 0;
+            auto advance = [&] {
+                ++kt;
+                slot = slot + 1 == PF ? 0 : slot + 1;
+            };
+            if (KT > 1) {
+                if (PF < KT) step_any_rot<true, MASK, false>(sa, sb, smem, K, kt, slot);
+                else step_any_rot<false, MASK, false>(sa, sb, smem, K, kt, slot);
+                advance();
+            }
+            for (; kt + PF < KT; advance()) step_any_rot<true, MASK, true>(sa, sb, smem, K, kt, slot);
+            for (; kt + 1 < KT; advance()) step_any_rot<false, MASK, true>(sa, sb, smem, K, kt, slot);
+        };
+        if (unmasked) {
+            pipeline.template operator()<false>();
+        } else {
+            pipeline.template operator()<true>();
+        }
+        // Last tile: nothing left to request or park.
+        if (KT > 0) {
+            const int cur = (KT - 1) & 1;
+            FrA f0a;
+            FrB f0b;
+            read_frags(smem, cur, 0, f0a, f0b);
+            if (KT > 1) mma_chunk(last_a, last_b);
+            compute_chunks(smem, cur, 0, NC, f0a, f0b);
+        }
+    }
+
+    // ---- plain schedule (tiles with 8 or 16 MFMA blocks per wave) ----
     // MFMA work of chunks [c0, c1) of the tile in LDS buffer `buf`.
-    __device__ __forceinline__ void compute_chunks(const T *smem, int buf, int c0, int c1) {
+    __device__ __forceinline__ void compute_chunks_plain(const T *smem, int buf, int c0, int c1) {
         const T *la = smem + buf * StA::LDS_ELEMS;
         const T *lb = smem + kBOff + buf * StB::LDS_ELEMS;
 #pragma unroll
@@ -358,14 +497,14 @@ struct TileEngine {
                     for (int bn = 0; bn < NBN; ++bn) acc[bm][bn] = M::mma(fa.v[bm][j], fb.v[bn][j], acc[bm][bn]);
         }
     }
-    __device__ __forceinline__ void compute(const T *smem, int buf) { compute_chunks(smem, buf, 0, BK / kChunk); }
+    __device__ __forceinline__ void compute_plain(const T *smem, int buf) { compute_chunks_plain(smem, buf, 0, BK / kChunk); }
 
     // One pipeline step for tile kt, whose register slot arithmetic is static: tile t lives in slot t % PF.
     //   LOAD: issue the global loads of tile kt + PF into slot kt % PF (free: tile kt is already in LDS);
     //   multiply tile kt out of LDS buffer kt & 1; park tile kt + 1 (slot (kt + 1) % PF, loaded PF - 1 steps
     //   ago) in the other LDS buffer, its stores slotted between the MFMAs of the last chunk.
     template <int S, bool LOAD, bool MASK>
-    __device__ __forceinline__ void step(StA &sa, StB &sb, T *smem, int K, int kt) {
+    __device__ __forceinline__ void step_plain(StA &sa, StB &sb, T *smem, int K, int kt) {
         constexpr int PF = StA::kPF;
         constexpr int NC = BK / kChunk;
         constexpr int kLastMfmas = M::VK * NBM * NBN;  // MFMAs of one chunk
@@ -379,13 +518,13 @@ struct TileEngine {
         // Keep the global loads ahead of the MFMA work: left alone, the scheduler sinks them to just before
         // the LDS stores and their latency is exposed on every tile.
         __builtin_amdgcn_sched_barrier(0);
-        compute_chunks(smem, cur, 0, NC - 1);
+        compute_chunks_plain(smem, cur, 0, NC - 1);
         __builtin_amdgcn_sched_barrier(0);
         // Last chunk: its MFMAs run with the LDS stores of the next tile slotted between them.  The other
         // buffer was last read before the previous barrier, so it may be written as soon as the global data
         // has arrived; by the time the last MFMA issues the stores have drained and the barrier costs no
         // pipe time (stores placed after the MFMAs cost ~9 % at 4096^3).
-        compute_chunks(smem, cur, NC - 1, NC);
+        compute_chunks_plain(smem, cur, NC - 1, NC);
         sa.template store<(S + 1) % PF>(smem + (cur ^ 1) * StA::LDS_ELEMS);
         sb.template store<(S + 1) % PF>(smem + kBOff + (cur ^ 1) * StB::LDS_ELEMS);
         if constexpr (kLastMfmas >= 2 * kStores) {
@@ -400,15 +539,15 @@ struct TileEngine {
     }
 
     template <bool LOAD, bool MASK, int S = 0>
-    __device__ __forceinline__ void step_any(StA &sa, StB &sb, T *smem, int K, int kt, int slot) {
+    __device__ __forceinline__ void step_any_plain(StA &sa, StB &sb, T *smem, int K, int kt, int slot) {
         if constexpr (S < StA::kPF) {
-            if (slot == S) step<S, LOAD, MASK>(sa, sb, smem, K, kt);
-            else step_any<LOAD, MASK, S + 1>(sa, sb, smem, K, kt, slot);
+            if (slot == S) step_plain<S, LOAD, MASK>(sa, sb, smem, K, kt);
+            else step_any_plain<LOAD, MASK, S + 1>(sa, sb, smem, K, kt, slot);
         }
     }
 
     // K: reduction length.  `unmasked`: workgroup-uniform promise that every tile is full and interior.
-    __device__ __forceinline__ void run(StA &sa, StB &sb, T *smem, int K, bool unmasked) {
+    __device__ __forceinline__ void run_plain(StA &sa, StB &sb, T *smem, int K, bool unmasked) {
         constexpr int PF = StA::kPF;
         static_assert(StA::kPF == StB::kPF, "both operands use the same prefetch distance");
         const int KT = (K + BK - 1) / BK;
@@ -424,15 +563,15 @@ struct TileEngine {
         auto pipeline = [&]<bool MASK>() {
             int kt = 0;
             if constexpr (PF == 1) {
-                for (; kt + 1 < KT; ++kt) step<0, true, MASK>(sa, sb, smem, K, kt);
+                for (; kt + 1 < KT; ++kt) step_plain<0, true, MASK>(sa, sb, smem, K, kt);
             } else {
                 int slot = 0;
                 for (; kt + PF < KT; ++kt) {
-                    step_any<true, MASK>(sa, sb, smem, K, kt, slot);
+                    step_any_plain<true, MASK>(sa, sb, smem, K, kt, slot);
                     slot = slot + 1 == PF ? 0 : slot + 1;
                 }
                 for (; kt + 1 < KT; ++kt) {
-                    step_any<false, MASK>(sa, sb, smem, K, kt, slot);
+                    step_any_plain<false, MASK>(sa, sb, smem, K, kt, slot);
                     slot = slot + 1 == PF ? 0 : slot + 1;
                 }
             }
@@ -442,7 +581,14 @@ struct TileEngine {
         } else {
             pipeline.template operator()<true>();
         }
-        if (KT > 0) compute(smem, (KT - 1) & 1);
+        if (KT > 0) compute_plain(smem, (KT - 1) & 1);
+    }
+
+    // K: reduction length.  `unmasked`: workgroup-uniform promise that every tile is full and interior.
+    __device__ __forceinline__ void run(StA &sa, StB &sb, T *smem, int K, bool unmasked) {
+        static_assert(StA::kPF == StB::kPF, "both operands use the same prefetch distance");
+        if constexpr (kRotate) run_rot(sa, sb, smem, K, unmasked);
+        else run_plain(sa, sb, smem, K, unmasked);
     }
 
     template <int S>
