@@ -130,6 +130,47 @@ def detail_report(tt, np, path, cpu=True):
                        ("bwd2 dH=dZ.W2^T", H, t(H)), ("bwd2 dW2=H^T.dZ", t(H), H),
                        ("bwd1 dX=dZ.W1^T", H, t(W1)), ("bwd1 dW1=X^T.dZ", t(X), H)):
         gemm_case("cfg5 " + name, a, b)
+    # config 5 as a whole: one training step through the tensor interface (fused Linear GEMMs, relu, mse_loss, the
+    # backward pass op for op; every result is a fresh allocation served by the library's block cache)
+    gp = oracle.Generator(0)
+    Xh, Th = oracle.Generator(0).uniform_real(0.0, 1.0, (1024, 784)), oracle.Generator(1).uniform_real(0.0, 1.0, (1024, 10))
+    params_h = [oracle.linear_init(gp, a, b) for a, b in ((784, 1024), (1024, 1024), (1024, 10))]
+    xs, ts = tt.Tensor.from_numpy(Xh), tt.Tensor.from_numpy(Th)
+    (P1, c1), (P2, c2), (P3, c3) = [(tt.Tensor.from_numpy(W), tt.Tensor.from_numpy(b)) for W, b in params_h]
+
+    def train_step():
+        z1 = tt.linear(xs, P1, c1); a1 = z1.relu(); z2 = tt.linear(a1, P2, c2); a2 = z2.relu(); y = tt.linear(a2, P3, c3)
+        diff = y - ts
+        loss = diff.pow(2.0).mean()
+        gy = tt.full(y.shape, 2.0 / y.numel(), y.dtype) * diff
+        grads = [gy.sum(0)]
+        da2, dW3 = tt.matmul_backward(a2.unsqueeze(0), P3.unsqueeze(0), gy.unsqueeze(0))
+        dz2 = da2.squeeze(0) * tt.where(z2 < 0.0, 0.0, 1.0)
+        da1, dW2 = tt.matmul_backward(a1.unsqueeze(0), P2.unsqueeze(0), dz2.unsqueeze(0))
+        dz1 = da1.squeeze(0) * tt.where(z1 < 0.0, 0.0, 1.0)
+        dX, dW1 = tt.matmul_backward(xs.unsqueeze(0), P1.unsqueeze(0), dz1.unsqueeze(0))
+        grads += [dz2.sum(0), dz1.sum(0), dW3, dW2, dW1, dX]
+        return loss, grads
+
+    for _ in range(5):
+        train_step()
+    be.synchronize(0)
+    t0 = time.perf_counter()
+    for _ in range(30):
+        train_step()
+    be.synchronize(0)
+    step_ms = (time.perf_counter() - t0) / 30 * 1e3
+    step_flop = 2.0 * 1024 * (784 * 1024 + 1024 * 1024 + 1024 * 10) * 3
+    rows.append({"case": "cfg5 whole MLP training step (tensor interface, wall clock incl. host overhead)",
+                 "kernel": "9 GEMMs + 21 streaming launches", "ms": round(step_ms, 4), "GFLOP/s": round(step_flop / step_ms / 1e6, 1)})
+    if cpu:
+        sys.path.insert(0, os.path.join(os.path.dirname(os.path.abspath(__file__)), "tests"))
+        from helpers import mlp_train_step  # the same step written over an abstract GEMM
+        t0 = time.perf_counter()
+        mlp_train_step(Xh, Th, params_h, lambda a, b: oracle.matmul(a, b, "fast"),
+                       lambda a, b, gr: tuple(v[0] for v in oracle.matmul_backward(a[None], b[None], gr[None], "fast")))
+        rows[-1]["cpu_oracle_ms_1core"] = round((time.perf_counter() - t0) * 1e3, 1)
+        rows[-1]["speedup_vs_cpu"] = round(rows[-1]["cpu_oracle_ms_1core"] / step_ms, 1)
     # config 4: conv2d forward / backward, input [64,32,28,28], weight [64,32,3,3], s1 p1
     x = tt.Tensor.from_numpy(oracle.Generator(0).normal(0, 0.1, (64, 32, 28, 28)))
     w = tt.Tensor.from_numpy(oracle.Generator(1).normal(0, 0.1, (64, 32, 3, 3)))

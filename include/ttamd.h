@@ -98,6 +98,15 @@ const char *ttamd_target_arch(void);
 ttamd_status ttamd_malloc(int device, size_t bytes, void **out);
 ttamd_status ttamd_free(int device, void *ptr, size_t bytes);
 ttamd_status ttamd_memory_allocated(int device, uint64_t *current_bytes, uint64_t *total_bytes);
+/* The library keeps freed device blocks (by size class) and hands them out again instead of paying
+ * hipMalloc + hipFree (25-70 us per pair, and a device-wide wait) for every result tensor; the counters above
+ * count what the caller holds, not what is cached.  Reuse follows stream order: safe when one stream carries all
+ * work of a device (the reference's model, cuda/kernel_launch.cuh:19-29); callers with several streams synchronise
+ * before freeing or run with TTAMD_ALLOC_CACHE=0.  ttamd_empty_cache waits for the device and returns every
+ * cached block to the driver; ttamd_memory_cached reports the bytes currently cached.  No counterpart in the
+ * reference, whose DeviceMemory<T> calls cudaMalloc / cudaFree directly (cuda/data_types.cuh:28-101). */
+ttamd_status ttamd_empty_cache(int device);
+ttamd_status ttamd_memory_cached(int device, uint64_t *cached_bytes);
 
 /* Blocking copies: BackendBase::from_vec (backend_base.h:35-48) and to_vec (:55-60). */
 ttamd_status ttamd_memcpy_h2d(int device, void *dst_device, const void *src_host, size_t bytes);

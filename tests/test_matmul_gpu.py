@@ -314,6 +314,35 @@ def test_memory_counters_and_device_errors(tt):
         tt.Tensor.from_numpy(np.zeros(4, dtype=np.float32), tt.Device("amd", be.get_device_count()))
 
 
+def test_freed_blocks_are_cached_and_reused(tt):
+    import ctypes as C
+    lib = tt._capi.lib
+    cached = C.c_uint64()
+
+    def cached_bytes():
+        assert lib.ttamd_memory_cached(0, C.byref(cached)) == 0
+        return cached.value
+
+    assert lib.ttamd_empty_cache(0) == 0 and cached_bytes() == 0
+    p, q = C.c_void_p(), C.c_void_p()
+    assert lib.ttamd_malloc(0, 5000, C.byref(p)) == 0           # size class 5120 (multiples of 512 up to 8 KiB)
+    first = p.value
+    assert lib.ttamd_free(0, p, 5000) == 0
+    assert cached_bytes() == 5120
+    assert lib.ttamd_malloc(0, 4700, C.byref(q)) == 0           # same class: the cached block comes back
+    assert q.value == first and cached_bytes() == 0
+    assert lib.ttamd_malloc(0, 5000, C.byref(p)) == 0 and p.value != first   # the class is empty again: a new block
+    assert lib.ttamd_free(0, p, 5000) == 0 and lib.ttamd_free(0, q, 4700) == 0
+    assert cached_bytes() == 2 * 5120
+    assert lib.ttamd_empty_cache(0) == 0 and cached_bytes() == 0
+    # results stay correct when every temporary of a chain of operations recycles blocks
+    a = np.arange(12, dtype=np.float32).reshape(3, 4)
+    t = tt.Tensor.from_numpy(a)
+    for _ in range(50):
+        t = (t + t) * tt.Tensor.from_numpy(np.full((3, 4), 0.5, np.float32))
+    assert np.array_equal(t.to_numpy(), a)
+
+
 # ----------------------------------------------------------------------------- full-size properties (config 3)
 @pytest.mark.parametrize("dtype", [np.float32, np.float64])
 def test_config3_4096_properties(tt, oracle, dtype):

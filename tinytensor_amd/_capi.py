@@ -40,6 +40,8 @@ def _bind(lib: C.CDLL) -> None:
         "ttamd_malloc": (i, [i, sz, C.POINTER(vp)]),
         "ttamd_free": (i, [i, vp, sz]),
         "ttamd_memory_allocated": (i, [i, C.POINTER(C.c_uint64), C.POINTER(C.c_uint64)]),
+        "ttamd_empty_cache": (i, [i]),
+        "ttamd_memory_cached": (i, [i, C.POINTER(C.c_uint64)]),
         "ttamd_memcpy_h2d": (i, [i, vp, vp, sz]),
         "ttamd_memcpy_d2h": (i, [i, vp, vp, sz]),
         "ttamd_memset_zero": (i, [i, vp, sz, vp]),

@@ -4,9 +4,11 @@
 #include "common.h"
 
 #include <atomic>
+#include <cstdlib>
 #include <cstring>
 #include <map>
 #include <mutex>
+#include <unordered_map>
 #include <utility>
 
 namespace ttamd {
@@ -16,6 +18,47 @@ thread_local char g_error[512] = "no error";
 constexpr int kMaxDevices = 64;
 std::atomic<uint64_t> g_current[kMaxDevices];
 std::atomic<uint64_t> g_total[kMaxDevices];
+
+// Caching allocator.  Every backend operation allocates its result, and hipMalloc + hipFree cost 25-70 us per pair
+// (hipFree also waits for the device), several times the run time of the small kernels between them.  Freed
+// blocks are therefore kept per device, by rounded size, and handed out again; they go back to the driver on
+// ttamd_empty_cache, when an allocation fails, and never otherwise.
+//
+// A reused block may still be read or written by kernels that were enqueued before it was freed.  That is safe
+// when the next user is enqueued on the same stream (stream order), which is the reference's model: all work of a
+// device goes to one stream (cuda/kernel_launch.cuh:19-29) and host copies are ordered against it.  A caller
+// that spreads work over several streams must synchronise them before freeing, or set TTAMD_ALLOC_CACHE=0.
+struct BlockCache {
+    std::mutex mu;
+    std::multimap<size_t, void *> free_blocks;     // rounded size -> block
+    std::unordered_map<void *, size_t> live;        // block -> rounded size
+    uint64_t cached_bytes = 0;
+};
+BlockCache g_cache[kMaxDevices];
+
+bool cache_enabled() {
+    static const bool on = [] {
+        const char *e = std::getenv("TTAMD_ALLOC_CACHE");
+        return !(e && e[0] == '0');
+    }();
+    return on;
+}
+
+// Size classes: multiples of 512 bytes up to 4 KiB, then eight classes per power of two (at most 12.5 % slack).
+size_t round_block(size_t bytes) {
+    if (bytes <= 4096) return (bytes + 511) & ~size_t(511);
+    size_t p = 4096;
+    while (p < bytes) p <<= 1;       // smallest power of two >= bytes
+    const size_t step = p >> 4;      // p/2 < bytes <= p: eight steps of p/16 above p/2
+    return (bytes + step - 1) / step * step;
+}
+
+void release_cached(int device) {
+    BlockCache &c = g_cache[device];
+    for (auto &kv : c.free_blocks) (void)hipFree(kv.second);
+    c.free_blocks.clear();
+    c.cached_bytes = 0;
+}
 }  // namespace
 
 void set_error(const char *fmt, ...) {
@@ -108,11 +151,38 @@ ttamd_status ttamd_malloc(int device, size_t bytes, void **out) {
     if (ttamd_status s = use_device(device)) return s;
     if (bytes == 0) return TTAMD_OK;
     void *p = nullptr;
-    hipError_t e = hipMalloc(&p, bytes);
-    if (e != hipSuccess) {
-        (void)hipGetLastError();
-        set_error("Unable to allocate %zu bytes on AMD device %d: %s", bytes, device, hipGetErrorString(e));
-        return TTAMD_ERR_OUT_OF_MEMORY;
+    const bool cached = cache_enabled();
+    const size_t want = cached ? round_block(bytes) : bytes;
+    BlockCache &c = g_cache[device];
+    if (cached) {
+        std::lock_guard<std::mutex> lock(c.mu);
+        auto it = c.free_blocks.find(want);
+        if (it != c.free_blocks.end()) {
+            p = it->second;
+            c.free_blocks.erase(it);
+            c.cached_bytes -= want;
+            c.live[p] = want;
+        }
+    }
+    if (!p) {
+        hipError_t e = hipMalloc(&p, want);
+        if (e != hipSuccess && cached) {  // give the cached blocks back to the driver and try once more
+            (void)hipGetLastError();
+            {
+                std::lock_guard<std::mutex> lock(c.mu);
+                release_cached(device);
+            }
+            e = hipMalloc(&p, want);
+        }
+        if (e != hipSuccess) {
+            (void)hipGetLastError();
+            set_error("Unable to allocate %zu bytes on AMD device %d: %s", bytes, device, hipGetErrorString(e));
+            return TTAMD_ERR_OUT_OF_MEMORY;
+        }
+        if (cached) {
+            std::lock_guard<std::mutex> lock(c.mu);
+            c.live[p] = want;
+        }
     }
     g_current[device] += bytes;
     g_total[device] += bytes;
@@ -123,8 +193,39 @@ ttamd_status ttamd_malloc(int device, size_t bytes, void **out) {
 ttamd_status ttamd_free(int device, void *ptr, size_t bytes) {
     if (!ptr) return TTAMD_OK;
     if (ttamd_status s = use_device(device)) return s;
-    TTAMD_HIP_CHECK(hipFree(ptr));  // synchronous, like ~DeviceMemory (cuda/data_types.cu:102-116)
+    BlockCache &c = g_cache[device];
+    bool kept = false;
+    {
+        std::lock_guard<std::mutex> lock(c.mu);
+        auto it = c.live.find(ptr);
+        if (it != c.live.end()) {  // a block of the caching allocator: keep it for the next request of its class
+            c.free_blocks.emplace(it->second, ptr);
+            c.cached_bytes += it->second;
+            c.live.erase(it);
+            kept = true;
+        }
+    }
+    if (!kept) TTAMD_HIP_CHECK(hipFree(ptr));  // synchronous, like ~DeviceMemory (cuda/data_types.cu:102-116)
     g_current[device] -= bytes;
+    return TTAMD_OK;
+}
+
+ttamd_status ttamd_empty_cache(int device) {
+    if (ttamd_status s = use_device(device)) return s;
+    TTAMD_HIP_CHECK(hipDeviceSynchronize());  // cached blocks may still be in use by enqueued kernels
+    BlockCache &c = g_cache[device];
+    std::lock_guard<std::mutex> lock(c.mu);
+    release_cached(device);
+    return TTAMD_OK;
+}
+
+ttamd_status ttamd_memory_cached(int device, uint64_t *cached_bytes) {
+    if (ttamd_status s = use_device(device)) return s;
+    if (cached_bytes) {
+        BlockCache &c = g_cache[device];
+        std::lock_guard<std::mutex> lock(c.mu);
+        *cached_bytes = c.cached_bytes;
+    }
     return TTAMD_OK;
 }
 

@@ -439,6 +439,8 @@ public:
         check(ttamd_memory_allocated(device_id, &cur, &tot));
         return tot;
     }
+    // Returns the blocks kept by the library's caching allocator to the driver (waits for the device).
+    void empty_cache(int device_id) const { check(ttamd_empty_cache(device_id)); }
     [[nodiscard]] auto get_device_count() const -> int {
         int n = 0;
         check(ttamd_device_count(&n));
