@@ -5,6 +5,7 @@
 // pooling forward and backward, seeded uniform draws and nn::Linear's default initialisation.
 #include "mini_test.h"
 
+#include <chrono>
 #include <limits>
 
 using namespace tt_amd;
@@ -249,6 +250,76 @@ TEST_CASE("Seeded draws and Linear default init") {
     const Tensor Y = layer.forward(X);
     CHECK(Y.shape() == Shape({8, 64}));
     CHECK(allclose(Y.to_vec<float>(), (matmul(X, layer.weight) + *layer.bias).to_vec<float>(), 1e-5, 1e-6));
+}
+
+namespace {
+struct MlpGrads {
+    Tensor loss, dW1, db1, dW2, db2, dW3, db3, dX;
+};
+// One training step of Linear-ReLU-Linear-ReLU-Linear + mse_loss, op for op as the reference's autograd emits it
+// (nn/linear.cpp:42-50, autograd/unary_ops.cpp:568-573, nn/loss.cpp:69-72, autograd/binary_ops.cpp:173-179).
+MlpGrads mlp_step(const Tensor &x, const Tensor &t, const nn::Linear &l1, const nn::Linear &l2, const nn::Linear &l3) {
+    const Device dev = x.device();
+    const Tensor z1 = l1.forward(x), a1 = relu(z1), z2 = l2.forward(a1), a2 = relu(z2), y = l3.forward(a2);
+    const Tensor diff = y - t;
+    const float n = static_cast<float>(y.numel());
+    MlpGrads g;
+    g.loss = (diff * diff).sum() / full(n, Shape({1}), dev);
+    const Tensor gy = full(1.0f / n * 2.0f, y.shape(), dev) * diff;
+    g.db3 = gy.sum(0);
+    auto [da2, dW3] = matmul_backward(a2.unsqueeze(0), l3.weight.unsqueeze(0), gy.unsqueeze(0));
+    const Tensor zero = full(0.0f, z2.shape(), dev), one = full(1.0f, z2.shape(), dev);
+    const Tensor dz2 = da2.squeeze(0) * where(z2 < zero, zero, one);
+    g.db2 = dz2.sum(0);
+    auto [da1, dW2] = matmul_backward(a1.unsqueeze(0), l2.weight.unsqueeze(0), dz2.unsqueeze(0));
+    const Tensor zero1 = full(0.0f, z1.shape(), dev), one1 = full(1.0f, z1.shape(), dev);
+    const Tensor dz1 = da1.squeeze(0) * where(z1 < zero1, zero1, one1);
+    g.db1 = dz1.sum(0);
+    auto [dX, dW1] = matmul_backward(x.unsqueeze(0), l1.weight.unsqueeze(0), dz1.unsqueeze(0));
+    g.dW3 = dW3.squeeze(0);
+    g.dW2 = dW2.squeeze(0);
+    g.dW1 = dW1.squeeze(0);
+    g.dX = dX.squeeze(0);
+    return g;
+}
+}  // namespace
+
+TEST_CASE("MLP training step") {
+    // small layer sizes against a finite-difference check of the loss, then the benchmark-sized step for its time
+    Generator gen(3);
+    const int B = 16, D0 = 12, D1 = 9, D2 = 7, D3 = 4;
+    const nn::Linear l1(D0, D1, true, gen), l2(D1, D2, true, gen), l3(D2, D3, true, gen);
+    const Tensor x = uniform_real(0.0, 1.0, {B, D0}, gen), t = uniform_real(0.0, 1.0, {B, D3}, gen);
+    const MlpGrads g = mlp_step(x, t, l1, l2, l3);
+    const float loss0 = g.loss.to_vec<float>()[0];
+    CHECK(loss0 > 0.0f);
+    // d loss / d W3[i][j] by central differences on a copy of the weights
+    const auto w3 = l3.weight.to_vec<float>(), dW3 = g.dW3.to_vec<float>();
+    for (int idx : {0, 5, 13, 27}) {
+        auto wp = w3, wm = w3;
+        wp[static_cast<std::size_t>(idx)] += 1e-2f;
+        wm[static_cast<std::size_t>(idx)] -= 1e-2f;
+        const nn::Linear lp(Tensor(wp, {D2, D3}, kAMD), l3.bias), lm(Tensor(wm, {D2, D3}, kAMD), l3.bias);
+        const float fp = mlp_step(x, t, l1, l2, lp).loss.to_vec<float>()[0], fm = mlp_step(x, t, l1, l2, lm).loss.to_vec<float>()[0];
+        CHECK(std::abs((fp - fm) / 2e-2f - dW3[static_cast<std::size_t>(idx)]) < 2e-3f);
+    }
+    // bias gradients are the column sums of the layer's output gradient: db3 = sum over the batch of gy
+    CHECK(g.db3.shape() == Shape({D3}));
+    CHECK(g.dW1.shape() == Shape({D0, D1}));
+    CHECK(g.dX.shape() == Shape({B, D0}));
+    // benchmark size: batch 1024, 784 -> 1024 -> 1024 -> 10
+    Generator gb(0);
+    const nn::Linear b1(784, 1024, true, gb), b2(1024, 1024, true, gb), b3(1024, 10, true, gb);
+    const Tensor X = uniform_real(0.0, 1.0, {1024, 784}, gb), T = uniform_real(0.0, 1.0, {1024, 10}, gb);
+    for (int i = 0; i < 5; ++i) (void)mlp_step(X, T, b1, b2, b3);
+    check(ttamd_device_synchronize(0));
+    const auto t0 = std::chrono::steady_clock::now();
+    const int iters = 30;
+    for (int i = 0; i < iters; ++i) (void)mlp_step(X, T, b1, b2, b3);
+    check(ttamd_device_synchronize(0));
+    const double ms = std::chrono::duration<double, std::milli>(std::chrono::steady_clock::now() - t0).count() / iters;
+    std::printf("  MLP training step 1024 x (784-1024-1024-10), C++ host layer: %.3f ms per step\n", ms);
+    CHECK(ms < 50.0);
 }
 
 int main(int argc, char **argv) { return mini::run_all(argc, argv); }

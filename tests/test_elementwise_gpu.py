@@ -94,12 +94,22 @@ def test_sum_and_full(tt, dtype):
     f = tt.full((3, 4), 7, tt._capi.I32 if dtype == np.int32 else (tt._capi.F32 if dtype == np.float32 else tt._capi.F64))
     assert f.stride == (0, 0) and np.array_equal(f.to_numpy(), np.full((3, 4), 7, dtype))
     if np.issubdtype(dtype, np.floating):
-        x = rng.uniform(-1, 1, (1024, 1000)).astype(dtype)
+        x = rng.uniform(-1, 1, (100, 1000)).astype(dtype)
         seq = np.zeros(1000, dtype=dtype)
         for r in x:                                         # the reference's order: sequential over the reduced dim
             seq = seq + r
         got = dev(tt, x).sum(0).to_numpy()
-        assert np.array_equal(got, seq)                     # same order, same IEEE additions: bit-identical
+        assert np.array_equal(got, seq)                     # short dimension: same order, same IEEE additions
+        # long reduced dimension with few outputs: sliced / wavefront-parallel forms, fixed order but not sequential
+        y = rng.uniform(-1, 1, (1024, 1000)).astype(dtype)
+        tol = (1e-5 if dtype == np.float32 else 1e-13) * 1024
+        assert np.max(np.abs(dev(tt, y).sum(0).to_numpy() - y.sum(0, dtype=np.float64))) <= tol
+        assert np.max(np.abs(dev(tt, y).sum(1).to_numpy() - y.sum(1, dtype=np.float64))) <= tol
+        assert np.max(np.abs(dev(tt, y).permute(1, 0).sum(0).to_numpy() - y.sum(1, dtype=np.float64))) <= tol
+        yi = np.round(y * 8)                                 # multiples of 1/8: exact in any order
+        assert np.array_equal(dev(tt, yi).sum(0).to_numpy(), yi.sum(0))
+        assert np.array_equal(dev(tt, yi).sum(1).to_numpy(), yi.sum(1))
+        assert np.array_equal(dev(tt, yi[:, :7]).sum(0).to_numpy(), yi[:, :7].sum(0))   # fewer outputs than one block
         assert abs(float(dev(tt, x).mean().to_numpy()[0]) - float(x.mean(dtype=np.float64))) <= 1e-5
 
 

@@ -323,6 +323,52 @@ __global__ void __launch_bounds__(256) sum_dim_kernel(const T *__restrict__ a, V
     out[i] = acc;
 }
 
+// Few outputs and a long reduced dimension (a bias gradient: [1024,1024] summed over the batch has 1024 outputs) leave
+// the one-lane-per-output kernel with a handful of workgroups.  Two parallel forms, both with a fixed summation order:
+//  * cols: 64 consecutive outputs x 4 row lanes per workgroup, the reduced dimension cut into slices (grid.y);
+//    partial sums per slice go to scratch and a second sum_dim_kernel adds them in slice order;
+//  * rows (the reduced dimension has unit stride): one wavefront per output, lanes stride the dimension and combine
+//    with a shuffle tree.
+template <typename T>
+__global__ void __launch_bounds__(256) sum_dim_cols_kernel(const T *__restrict__ a, ViewDesc outer, int64_t dim_len, int64_t dim_stride,
+                                                          T *__restrict__ partial, int64_t n_out, int64_t rows_per_slice) {
+    __shared__ T red[4][64];
+    const int ol = threadIdx.x % 64, rl = threadIdx.x / 64;
+    const int64_t o = static_cast<int64_t>(blockIdx.x) * 64 + ol;
+    const int64_t r0 = static_cast<int64_t>(blockIdx.y) * rows_per_slice;
+    const int64_t r1 = r0 + rows_per_slice < dim_len ? r0 + rows_per_slice : dim_len;
+    T acc = T(0);
+    if (o < n_out) {
+        const T *p = a + flat_of(o, outer);
+        for (int64_t r = r0 + rl; r < r1; r += 4) acc = static_cast<T>(acc + p[r * dim_stride]);
+    }
+    red[rl][ol] = acc;
+    __syncthreads();
+    if (rl == 0 && o < n_out)
+        partial[static_cast<int64_t>(blockIdx.y) * n_out + o] =
+            static_cast<T>(static_cast<T>(red[0][ol] + red[1][ol]) + static_cast<T>(red[2][ol] + red[3][ol]));
+}
+
+template <typename T>
+__global__ void __launch_bounds__(256) sum_dim_rows_kernel(const T *__restrict__ a, ViewDesc outer, int64_t dim_len, T *__restrict__ out,
+                                                          int64_t n_out) {
+    __shared__ T red[4][64];
+    const int lane = threadIdx.x % 64, w = threadIdx.x / 64;
+    const int64_t o = static_cast<int64_t>(blockIdx.x) * 4 + w;
+    T acc = T(0);
+    if (o < n_out) {
+        const T *p = a + flat_of(o, outer);
+        for (int64_t j = lane; j < dim_len; j += 64) acc = static_cast<T>(acc + p[j]);
+    }
+    red[w][lane] = acc;
+    __syncthreads();
+    for (int h = 32; h > 0; h >>= 1) {
+        if (lane < h) red[w][lane] = static_cast<T>(red[w][lane] + red[w][lane + h]);
+        __syncthreads();
+    }
+    if (lane == 0 && o < n_out) out[o] = red[w][0];
+}
+
 // sum of everything: per-workgroup partial sums (stage 1) then one workgroup adds the partials (stage 2).
 template <typename T>
 __global__ void __launch_bounds__(256) sum_all_kernel(const T *__restrict__ a, ViewDesc v, bool dense, int64_t numel, T *__restrict__ out) {
@@ -543,6 +589,34 @@ ttamd_status sum_typed(int device, const void *a, const ViewDesc &v, int64_t num
     }
     const int64_t n_out = v.shape[dim] ? numel / v.shape[dim] : 0;
     if (n_out == 0) return TTAMD_OK;
+    const int64_t dim_len = v.shape[dim], dim_stride = v.stride[dim];
+    if (n_out < 32768 && dim_len >= 128) {
+        if (dim_stride == 1) {
+            sum_dim_rows_kernel<T><<<dim3(static_cast<unsigned>((n_out + 3) / 4)), dim3(256), 0, st>>>(src, outer, dim_len, static_cast<T *>(out), n_out);
+            TTAMD_HIP_CHECK(hipGetLastError());
+            return TTAMD_OK;
+        }
+        const int64_t col_blocks = (n_out + 63) / 64;
+        int64_t slices = 1024 / col_blocks;
+        if (slices > dim_len / 32) slices = dim_len / 32;  // at least 32 rows per slice
+        if (slices > 256) slices = 256;
+        if (slices >= 2) {
+            const int64_t rows_per_slice = (dim_len + slices - 1) / slices;
+            slices = (dim_len + rows_per_slice - 1) / rows_per_slice;
+            void *ws = nullptr;
+            if (ttamd_status s = stream_scratch(device, st, static_cast<size_t>(slices) * n_out * sizeof(T), &ws)) return s;
+            sum_dim_cols_kernel<T><<<dim3(static_cast<unsigned>(col_blocks), static_cast<unsigned>(slices)), dim3(256), 0, st>>>(
+                src, outer, dim_len, dim_stride, static_cast<T *>(ws), n_out, rows_per_slice);
+            ViewDesc flat{};
+            flat.ndim = 1;
+            flat.shape[0] = n_out;
+            flat.stride[0] = 1;
+            sum_dim_kernel<T><<<dim3(static_cast<unsigned>((n_out + 255) / 256)), dim3(256), 0, st>>>(static_cast<const T *>(ws), flat, slices, n_out,
+                                                                                                    static_cast<T *>(out), n_out);
+            TTAMD_HIP_CHECK(hipGetLastError());
+            return TTAMD_OK;
+        }
+    }
     sum_dim_kernel<T><<<dim3(static_cast<unsigned>((n_out + 255) / 256)), dim3(256), 0, st>>>(src, outer, v.shape[dim], v.stride[dim],
                                                                                               static_cast<T *>(out), n_out);
     TTAMD_HIP_CHECK(hipGetLastError());
