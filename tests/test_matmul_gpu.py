@@ -232,9 +232,9 @@ def test_variant_selection(tt):
     be = tt.get_backend(tt.kAMD)
     f32 = np.float32
     big = tt.Tensor.empty((1, 4096, 4096), tt._capi.F32)
-    assert be.batched_matmul_variant(big, big) == "mfma_f32_256x128_akc4_bmc4"
-    assert be.batched_matmul_variant(big, big.permute(0, 2, 1)) == "mfma_f32_256x128_akc4_bkc4"
-    assert be.batched_matmul_variant(big.permute(0, 2, 1), big) == "mfma_f32_256x128_amc4_bmc4"
+    assert be.batched_matmul_variant(big, big) == "mfma_f32_256x256_akc4_bmc4"
+    assert be.batched_matmul_variant(big, big.permute(0, 2, 1)) == "mfma_f32_256x256_akc4_bkc4"
+    assert be.batched_matmul_variant(big.permute(0, 2, 1), big) == "mfma_f32_256x256_amc4_bmc4"
     big64 = tt.Tensor.empty((1, 4096, 4096), tt._capi.F64)
     assert be.batched_matmul_variant(big64, big64) == "mfma_f64_128x128_akc2_bmc2"
     small = tt.Tensor.from_numpy(np.zeros((1, 256, 512), f32))

@@ -22,7 +22,7 @@ using namespace mfma;
 // latency, and registers are scarce), more for the 64 x 64 tile whose 16 MFMAs per k tile (~0.45 us) are far
 // shorter than a global load.
 template <typename T, int BM, int BN, int BK, int WGM, int WGN, bool A_KC, int A_VEC, bool B_KC, int B_VEC, int PF>
-__global__ void __launch_bounds__(kThreads, 2)
+__global__ void __launch_bounds__(kThreads, (BM * BN > 256 * 128) ? 1 : 2)  // 256 x 256: one workgroup per CU, accumulators in AGPRs
 gemm_mfma_kernel(GemmArgs g, int tiles_m, int tiles_n, int ksplit, int k_chunk, T *partial) {
     using StA = Stager<T, BM, BK, A_KC, A_VEC, PF>;
     using StB = Stager<T, BN, BK, B_KC, B_VEC, PF>;
@@ -54,7 +54,10 @@ gemm_mfma_kernel(GemmArgs g, int tiles_m, int tiles_n, int ksplit, int k_chunk, 
 
     if (ksplit == 1) {
         T *C = static_cast<T *>(g.C) + static_cast<int64_t>(batch) * g.M * g.N;
-        store_tile_dense<T>(eng, C, g.M, g.N, m0, n0, static_cast<const T *>(g.bias), g.bias_mode, g.relu, g.accumulate);
+        if (g.bias_mode == 0 && !g.relu && !g.accumulate)  // the common case gets a store loop free of epilogue tests
+            store_tile_dense<T>(eng, C, g.M, g.N, m0, n0, static_cast<const T *>(nullptr), 0, 0, 0);
+        else
+            store_tile_dense<T>(eng, C, g.M, g.N, m0, n0, static_cast<const T *>(g.bias), g.bias_mode, g.relu, g.accumulate);
     } else {
         store_tile_dense<T>(eng, partial + static_cast<int64_t>(z) * g.M * g.N, g.M, g.N, m0, n0,
                             static_cast<const T *>(nullptr), 0, 0, 0);
@@ -104,6 +107,7 @@ struct TileShapes;
 template <>
 struct TileShapes<float> {
     static constexpr bool kHasXL = true;
+    static constexpr int YBM = 256, YBN = 256, YBK = 16;  // largest: 4 waves of 128 x 128 (4 x 4 MFMA blocks), one workgroup per CU
     static constexpr int XBM = 256, XBN = 128, XBK = 16;  // extra large: 4 waves of 128 x 64 (4 x 2 MFMA blocks)
     static constexpr int LBM = 128, LBN = 128, LBK = 32;  // large: 4 waves of 64 x 64
     static constexpr int SBM = 64, SBN = 64, SBK = 32;    // small: 4 waves of 32 x 32
@@ -113,6 +117,7 @@ struct TileShapes<float> {
 template <>
 struct TileShapes<double> {
     static constexpr bool kHasXL = false;                  // a 128 x 64 wave tile would need 256 accumulator registers
+    static constexpr int YBM = 128, YBN = 128, YBK = 16;
     static constexpr int XBM = 128, XBN = 128, XBK = 16;
     static constexpr int LBM = 128, LBN = 128, LBK = 16;  // 4 waves of 64 x 64 (4 x 4 blocks of 16 x 16)
     static constexpr int SBM = 64, SBN = 64, SBK = 16;    // 4 waves of 32 x 32
@@ -227,21 +232,23 @@ ttamd_status launch_mfma_typed(const GemmArgs &g, int device, hipStream_t stream
     };
     const double t_small = estimate(TS::SBM, TS::SBN, 4, 131e12);
     const double t_large = vec ? estimate(TS::LBM, TS::LBN, 2, 131e12) : 1e300;
-    const double t_xl = (TS::kHasXL && vec) ? estimate(TS::XBM, TS::XBN, 2, 141e12) : 1e300;
-    const bool xl = t_xl <= t_large && t_xl <= t_small;
-    const bool large = !xl && t_large <= t_small;
-    const int bm = xl ? TS::XBM : (large ? TS::LBM : TS::SBM);
+    const double t_xl = (TS::kHasXL && vec) ? estimate(TS::XBM, TS::XBN, 2, 145e12) : 1e300;
+    const double t_xxl = (TS::kHasXL && vec) ? estimate(TS::YBM, TS::YBN, 1, 147e12) : 1e300;
+    const bool xxl = t_xxl <= t_xl && t_xxl <= t_large && t_xxl <= t_small;
+    const bool xl = !xxl && t_xl <= t_large && t_xl <= t_small;
+    const bool large = !xxl && !xl && t_large <= t_small;
+    const int bm = (xxl || xl) ? TS::XBM : (large ? TS::LBM : TS::SBM);
     // 32-bit buffer addressing: the bytes reachable from a tile's first row must stay below 2^31.
     const int64_t a_reach = (static_cast<int64_t>(bm - 1) * g.a_sm + static_cast<int64_t>(g.K - 1) * g.a_sk + VK) * sizeof(T);
     const int64_t b_reach = (static_cast<int64_t>(bm - 1) * g.b_sn + static_cast<int64_t>(g.K - 1) * g.b_sk + VK) * sizeof(T);
     if (a_reach >= 0x7fffffffLL || b_reach >= 0x7fffffffLL) return TTAMD_OK;
 
-    const SplitPlan sp = (xl || large) ? SplitPlan{1, g.K} : plan_split<T>(g, TS::SBM, TS::SBN, TS::SBK);
+    const SplitPlan sp = (xxl || xl || large) ? SplitPlan{1, g.K} : plan_split<T>(g, TS::SBM, TS::SBN, TS::SBK);
 
     static thread_local char name[112];
     char split_tag[24] = "";
     if (sp.ksplit > 1) snprintf(split_tag, sizeof(split_tag), "_splitk%d", sp.ksplit);
-    snprintf(name, sizeof(name), "%s_%s_a%s%d_b%s%d%s", TS::prefix, xl ? "256x128" : (large ? "128x128" : "64x64"), ca.kc ? "kc" : "mc",
+    snprintf(name, sizeof(name), "%s_%s_a%s%d_b%s%d%s", TS::prefix, xxl ? "256x256" : (xl ? "256x128" : (large ? "128x128" : "64x64")), ca.kc ? "kc" : "mc",
              ca.vec, cb.kc ? "kc" : "mc", cb.vec, split_tag);
     *variant = name;
     *handled = true;
@@ -249,6 +256,7 @@ ttamd_status launch_mfma_typed(const GemmArgs &g, int device, hipStream_t stream
 
     // The large tile exists for 16-byte operands only; the small tile for every mix of 16-byte and element-wise.
     if constexpr (TS::kHasXL) {
+        if (xxl) return launch_layouts<T, TS::YBM, TS::YBN, TS::YBK, 2, 2, VK, VK>(g, ca.kc, cb.kc, sp, device, stream);
         if (xl) return launch_layouts<T, TS::XBM, TS::XBN, TS::XBK, 2, 2, VK, VK>(g, ca.kc, cb.kc, sp, device, stream);
     }
     if (large) return launch_layouts<T, TS::LBM, TS::LBN, TS::LBK, 2, 2, VK, VK>(g, ca.kc, cb.kc, sp, device, stream);

@@ -325,11 +325,13 @@ struct TileEngine {
     static constexpr size_t kLdsBytes = 2 * (StA::LDS_ELEMS + StB::LDS_ELEMS) * sizeof(T);
 
     typename M::acc_t acc[NBM][NBN];
-    // The rotated schedule (see step()) pays off for waves with few MFMA blocks (64 x 64 tiles: +9 % at 2048^3).
-    // It keeps one more pair of fragments live across the barrier, which the tiles with 8 or 16 blocks per wave
-    // cannot afford (128 accumulator registers: fp64 spills, fp32 256 x 128 measured 1.5 % slower), so they keep
-    // the plain schedule.
+    // Three schedules of the main loop, chosen by the number of MFMA blocks a wave owns:
+    //  * rotated (<= 4 blocks: 64 x 64 tiles, fp32 128 x 128, conv tiles) - see step_rot();
+    //  * pipelined (fp32, 8 or 16 blocks: 256 x 128 and 256 x 256) - see step_pipe();
+    //  * plain (fp64 128 x 128: 16 blocks of 16 x 16, 128 accumulator registers leave no room for a second set of
+    //    fragments) - see step_plain().
     static constexpr bool kRotate = NBM * NBN <= 4;
+    static constexpr bool kPipe = !kRotate && sizeof(T) == 4 && BK / kChunk == 2;
     FrA last_a;  // fragments of the previous tile's last chunk, multiplied after the barrier
     FrB last_b;
     int lane, wm0, wn0;
@@ -480,7 +482,107 @@ struct TileEngine {
         }
     }
 
-    // ---- plain schedule (tiles with 8 or 16 MFMA blocks per wave) ----
+    // ---- pipelined schedule (fp32 tiles with 8 or 16 MFMA blocks per wave, two chunks per k tile) ----
+    // With one or two waves per SIMD nothing else hides a wave's own requests, so every load, LDS read and LDS
+    // store of a step is slotted between MFMAs (sched_group_barrier), fragments are double-buffered in registers
+    // and the barrier sits in the middle of chunk 1:
+    //   chunk 0 (fragments f0, read after the previous barrier): its MFMAs carry the global loads of tile kt + 1
+    //     and the LDS reads of chunk 1 (f1);
+    //   chunk 1, first half: its MFMAs carry the LDS stores of tile kt + 1 into the other buffer, finishing a
+    //     quarter of the half early so that the stores have landed when the barrier comes;
+    //   barrier;
+    //   chunk 1, second half: its MFMAs carry the LDS reads of chunk 0 of tile kt + 1 (the next f0).
+    // 4096^3 fp32: 140 -> 145 (256 x 128, two workgroups per CU) / 147 TFLOP/s (256 x 256, one per CU).
+    __device__ __forceinline__ void mma_half(const FrA &fa, const FrB &fb, int j0) {
+#pragma unroll
+        for (int j = j0; j < j0 + M::VK / 2; ++j)
+#pragma unroll
+            for (int bm = 0; bm < NBM; ++bm)
+#pragma unroll
+                for (int bn = 0; bn < NBN; ++bn) acc[bm][bn] = M::mma(fa.v[bm][j], fb.v[bn][j], acc[bm][bn]);
+    }
+
+    template <bool MASK>
+    __device__ __forceinline__ void step_pipe(StA &sa, StB &sb, T *smem, int K, int kt, FrA &f0a, FrB &f0b) {
+        constexpr int kHalf = (M::VK / 2) * NBM * NBN;  // MFMAs of half a chunk
+        constexpr int kLoads = StA::P + StB::P;         // global loads (and LDS stores) of one tile, per lane
+        constexpr int kReads = NBM + NBN;               // LDS read instructions of one chunk's fragments
+        const int cur = kt & 1;
+        FrA f1a;
+        FrB f1b;
+        const int k_left = K - (kt + 1) * BK;
+        sa.template load<MASK, 0>(k_left);
+        sb.template load<MASK, 0>(k_left);
+        read_frags(smem, cur, 1, f1a, f1b);
+        mma_half(f0a, f0b, 0);
+        mma_half(f0a, f0b, M::VK / 2);
+        {
+            constexpr int per = 2 * kHalf / (kLoads + kReads) > 0 ? 2 * kHalf / (kLoads + kReads) : 1;
+#pragma unroll
+            for (int i = 0; i < kLoads; ++i) {
+                __builtin_amdgcn_sched_group_barrier(0x008, per, 0);  // MFMA
+                __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);    // VMEM read
+            }
+#pragma unroll
+            for (int i = 0; i < kReads; ++i) {
+                __builtin_amdgcn_sched_group_barrier(0x008, per, 0);
+                __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);    // DS read
+            }
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        mma_half(f1a, f1b, 0);
+        sa.template store<0>(smem + (cur ^ 1) * StA::LDS_ELEMS);
+        sb.template store<0>(smem + kBOff + (cur ^ 1) * StB::LDS_ELEMS);
+        {
+            constexpr int per = (kHalf - kHalf / 4) / kLoads > 0 ? (kHalf - kHalf / 4) / kLoads : 1;
+#pragma unroll
+            for (int i = 0; i < kLoads; ++i) {
+                __builtin_amdgcn_sched_group_barrier(0x008, per, 0);
+                __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);    // DS write
+            }
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        __syncthreads();
+        read_frags(smem, cur ^ 1, 0, f0a, f0b);
+        mma_half(f1a, f1b, M::VK / 2);
+        {
+            constexpr int per = kHalf / kReads > 0 ? kHalf / kReads : 1;
+#pragma unroll
+            for (int i = 0; i < kReads; ++i) {
+                __builtin_amdgcn_sched_group_barrier(0x008, per, 0);
+                __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+            }
+        }
+        __builtin_amdgcn_sched_barrier(0);
+    }
+
+    __device__ __forceinline__ void run_pipe(StA &sa, StB &sb, T *smem, int K, bool unmasked) {
+        static_assert(StA::kPF == 1 && BK / kChunk == 2, "the pipelined schedule is written for two chunks per k tile");
+        const int KT = (K + BK - 1) / BK;
+        sa.template load<true, 0>(K);
+        sb.template load<true, 0>(K);
+        sa.template store<0>(smem);
+        sb.template store<0>(smem + kBOff);
+        __syncthreads();
+        if (KT > 0) {
+            FrA f0a;
+            FrB f0b;
+            read_frags(smem, 0, 0, f0a, f0b);
+            if (unmasked) {
+                for (int kt = 0; kt + 1 < KT; ++kt) step_pipe<false>(sa, sb, smem, K, kt, f0a, f0b);
+            } else {
+                for (int kt = 0; kt + 1 < KT; ++kt) step_pipe<true>(sa, sb, smem, K, kt, f0a, f0b);
+            }
+            const int cur = (KT - 1) & 1;
+            FrA f1a;
+            FrB f1b;
+            read_frags(smem, cur, 1, f1a, f1b);
+            mma_chunk(f0a, f0b);
+            mma_chunk(f1a, f1b);
+        }
+    }
+
+    // ---- plain schedule (fp64 tiles with 16 MFMA blocks per wave) ----
     // MFMA work of chunks [c0, c1) of the tile in LDS buffer `buf`.
     __device__ __forceinline__ void compute_chunks_plain(const T *smem, int buf, int c0, int c1) {
         const T *la = smem + buf * StA::LDS_ELEMS;
@@ -595,6 +697,7 @@ struct TileEngine {
     __device__ __forceinline__ void run(StA &sa, StB &sb, T *smem, int K, bool unmasked) {
         static_assert(StA::kPF == StB::kPF, "both operands use the same prefetch distance");
         if constexpr (kRotate) run_rot(sa, sb, smem, K, unmasked);
+        else if constexpr (kPipe) run_pipe(sa, sb, smem, K, unmasked);
         else run_plain(sa, sb, smem, K, unmasked);
     }
 
