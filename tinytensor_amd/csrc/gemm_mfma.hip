@@ -109,7 +109,7 @@ struct TileShapes<float> {
     static constexpr bool kHasXL = true;
     static constexpr int YBM = 256, YBN = 256, YBK = 16;  // largest: 4 waves of 128 x 128 (4 x 4 MFMA blocks), one workgroup per CU
     static constexpr int XBM = 256, XBN = 128, XBK = 16;  // extra large: 4 waves of 128 x 64 (4 x 2 MFMA blocks)
-    static constexpr int LBM = 128, LBN = 128, LBK = 32;  // large: 4 waves of 64 x 64
+    static constexpr int LBM = 128, LBN = 128, LBK = 16;  // large: 4 waves of 64 x 64
     static constexpr int SBM = 64, SBN = 64, SBK = 32;    // small: 4 waves of 32 x 32
     static constexpr int SPF = 1;                          // deeper register prefetch measured slower (more registers, same stalls)
     static constexpr const char *prefix = "mfma_f32";
@@ -231,7 +231,7 @@ ttamd_status launch_mfma_typed(const GemmArgs &g, int device, hipStream_t stream
         return (rounds + last) * round_time;
     };
     const double t_small = estimate(TS::SBM, TS::SBN, 4, 131e12);
-    const double t_large = vec ? estimate(TS::LBM, TS::LBN, 2, 131e12) : 1e300;
+    const double t_large = vec ? estimate(TS::LBM, TS::LBN, 2, (sizeof(T) == 4 ? 145e12 : 131e12)) : 1e300;
     const double t_xl = (TS::kHasXL && vec) ? estimate(TS::XBM, TS::XBN, 2, 145e12) : 1e300;
     const double t_xxl = (TS::kHasXL && vec) ? estimate(TS::YBM, TS::YBN, 1, 147e12) : 1e300;
     const bool xxl = t_xxl <= t_xl && t_xxl <= t_large && t_xxl <= t_small;

@@ -326,12 +326,12 @@ struct TileEngine {
 
     typename M::acc_t acc[NBM][NBN];
     // Three schedules of the main loop, chosen by the number of MFMA blocks a wave owns:
-    //  * rotated (<= 4 blocks: 64 x 64 tiles, fp32 128 x 128, conv tiles) - see step_rot();
-    //  * pipelined (fp32, 8 or 16 blocks: 256 x 128 and 256 x 256) - see step_pipe();
+    //  * pipelined (fp32, two chunks per k tile, 4 to 16 blocks: 128 x 128, 256 x 128 and 256 x 256) - see step_pipe();
+    //  * rotated (<= 4 blocks otherwise: 64 x 64 tiles, conv tiles) - see step_rot();
     //  * plain (fp64 128 x 128: 16 blocks of 16 x 16, 128 accumulator registers leave no room for a second set of
     //    fragments) - see step_plain().
-    static constexpr bool kRotate = NBM * NBN <= 4;
-    static constexpr bool kPipe = !kRotate && sizeof(T) == 4 && BK / kChunk == 2;
+    static constexpr bool kPipe = sizeof(T) == 4 && BK / kChunk == 2 && NBM * NBN >= 4;
+    static constexpr bool kRotate = !kPipe && NBM * NBN <= 4;
     FrA last_a;  // fragments of the previous tile's last chunk, multiplied after the barrier
     FrB last_b;
     int lane, wm0, wn0;
@@ -696,8 +696,8 @@ struct TileEngine {
     // K: reduction length.  `unmasked`: workgroup-uniform promise that every tile is full and interior.
     __device__ __forceinline__ void run(StA &sa, StB &sb, T *smem, int K, bool unmasked) {
         static_assert(StA::kPF == StB::kPF, "both operands use the same prefetch distance");
-        if constexpr (kRotate) run_rot(sa, sb, smem, K, unmasked);
-        else if constexpr (kPipe) run_pipe(sa, sb, smem, K, unmasked);
+        if constexpr (kPipe) run_pipe(sa, sb, smem, K, unmasked);
+        else if constexpr (kRotate) run_rot(sa, sb, smem, K, unmasked);
         else run_plain(sa, sb, smem, K, unmasked);
     }
 
