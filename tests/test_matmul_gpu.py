@@ -236,7 +236,7 @@ def test_variant_selection(tt):
     assert be.batched_matmul_variant(big, big.permute(0, 2, 1)) == "mfma_f32_256x256_akc4_bkc4"
     assert be.batched_matmul_variant(big.permute(0, 2, 1), big) == "mfma_f32_256x256_amc4_bmc4"
     big64 = tt.Tensor.empty((1, 4096, 4096), tt._capi.F64)
-    assert be.batched_matmul_variant(big64, big64) == "mfma_f64_128x128_akc2_bmc2"
+    assert be.batched_matmul_variant(big64, big64) == "mfma_f64_256x128_akc2_bmc2"
     small = tt.Tensor.from_numpy(np.zeros((1, 256, 512), f32))
     assert be.batched_matmul_variant(small, small.permute(0, 2, 1)).startswith("mfma_f32_64x64")
     thin = tt.Tensor.from_numpy(np.zeros((1, 512, 10), f32))

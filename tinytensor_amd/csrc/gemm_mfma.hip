@@ -22,7 +22,7 @@ using namespace mfma;
 // latency, and registers are scarce), more for the 64 x 64 tile whose 16 MFMAs per k tile (~0.45 us) are far
 // shorter than a global load.
 template <typename T, int BM, int BN, int BK, int WGM, int WGN, bool A_KC, int A_VEC, bool B_KC, int B_VEC, int PF>
-__global__ void __launch_bounds__(kThreads, (BM * BN > 256 * 128) ? 1 : 2)  // 256 x 256: one workgroup per CU, accumulators in AGPRs
+__global__ void __launch_bounds__(kThreads, (BM * BN * sizeof(T) > 256 * 128 * 4 || (sizeof(T) == 8 && BM * BN >= 128 * 128)) ? 1 : 2)  // 256 x 256 (fp64 128 x 128 and up): one workgroup per CU, accumulators in AGPRs
 gemm_mfma_kernel(GemmArgs g, int tiles_m, int tiles_n, int ksplit, int k_chunk, T *partial) {
     using StA = Stager<T, BM, BK, A_KC, A_VEC, PF>;
     using StB = Stager<T, BN, BK, B_KC, B_VEC, PF>;
@@ -116,9 +116,9 @@ struct TileShapes<float> {
 };
 template <>
 struct TileShapes<double> {
-    static constexpr bool kHasXL = false;                  // a 128 x 64 wave tile would need 256 accumulator registers
-    static constexpr int YBM = 128, YBN = 128, YBK = 16;
-    static constexpr int XBM = 128, XBN = 128, XBK = 16;
+    static constexpr bool kHasXL = true;
+    static constexpr int YBM = 256, YBN = 128, YBK = 16;  // (no larger tile: 128 x 64 per wave already fills 256 accumulator registers)
+    static constexpr int XBM = 256, XBN = 128, XBK = 16;  // 4 waves of 128 x 64 (8 x 4 blocks of 16 x 16), one workgroup per CU
     static constexpr int LBM = 128, LBN = 128, LBK = 16;  // 4 waves of 64 x 64 (4 x 4 blocks of 16 x 16)
     static constexpr int SBM = 64, SBN = 64, SBK = 16;    // 4 waves of 32 x 32
     static constexpr int SPF = 1;
@@ -231,9 +231,10 @@ ttamd_status launch_mfma_typed(const GemmArgs &g, int device, hipStream_t stream
         return (rounds + last) * round_time;
     };
     const double t_small = estimate(TS::SBM, TS::SBN, 4, 131e12);
-    const double t_large = vec ? estimate(TS::LBM, TS::LBN, 2, (sizeof(T) == 4 ? 145e12 : 131e12)) : 1e300;
-    const double t_xl = (TS::kHasXL && vec) ? estimate(TS::XBM, TS::XBN, 2, 145e12) : 1e300;
-    const double t_xxl = (TS::kHasXL && vec) ? estimate(TS::YBM, TS::YBN, 1, 147e12) : 1e300;
+    constexpr bool f32 = sizeof(T) == 4;  // the fp64 big tiles run one workgroup per CU (accumulators in AGPRs)
+    const double t_large = vec ? estimate(TS::LBM, TS::LBN, f32 ? 2 : 1, f32 ? 145e12 : 141e12) : 1e300;
+    const double t_xl = (TS::kHasXL && vec) ? estimate(TS::XBM, TS::XBN, f32 ? 2 : 1, f32 ? 145e12 : 147e12) : 1e300;
+    const double t_xxl = (TS::kHasXL && vec && sizeof(T) == 4) ? estimate(TS::YBM, TS::YBN, 1, 147e12) : 1e300;
     const bool xxl = t_xxl <= t_xl && t_xxl <= t_large && t_xxl <= t_small;
     const bool xl = !xxl && t_xl <= t_large && t_xl <= t_small;
     const bool large = !xxl && !xl && t_large <= t_small;

@@ -330,7 +330,7 @@ struct TileEngine {
     //  * rotated (<= 4 blocks otherwise: 64 x 64 tiles, conv tiles) - see step_rot();
     //  * plain (fp64 128 x 128: 16 blocks of 16 x 16, 128 accumulator registers leave no room for a second set of
     //    fragments) - see step_plain().
-    static constexpr bool kPipe = sizeof(T) == 4 && BK / kChunk == 2 && NBM * NBN >= 4;
+    static constexpr bool kPipe = BK / kChunk == 2 && NBM * NBN >= (sizeof(T) == 4 ? 4 : 16);
     static constexpr bool kRotate = !kPipe && NBM * NBN <= 4;
     FrA last_a;  // fragments of the previous tile's last chunk, multiplied after the barrier
     FrB last_b;
