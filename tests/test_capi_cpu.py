@@ -79,10 +79,13 @@ def test_variant_names_without_gpu(tt):
         return lib.ttamd_batched_matmul_variant(dtype, B, N, K, M, C.byref(a), C.byref(b)).decode()
 
     n = 4096
-    assert variant(capi.F32, 1, n, n, n, (0, n, 1), (0, n, 1)) == "mfma_f32_256x128_akc4_bmc4"
-    assert variant(capi.F32, 1, n, n, n, (0, n, 1), (0, 1, n)) == "mfma_f32_256x128_akc4_bkc4"      # A . B^T
-    assert variant(capi.F32, 1, n, n, n, (0, 1, n), (0, n, 1)) == "mfma_f32_256x128_amc4_bmc4"      # A^T . B
-    assert variant(capi.F64, 1, n, n, n, (0, n, 1), (0, n, 1)) == "mfma_f64_128x128_akc2_bmc2"
+    assert variant(capi.F32, 1, n, n, n, (0, n, 1), (0, n, 1)) == "mfma_f32_256x256_akc4_bmc4"
+    assert variant(capi.F32, 1, n, n, n, (0, n, 1), (0, 1, n)) == "mfma_f32_256x256_akc4_bkc4"      # A . B^T
+    assert variant(capi.F32, 1, n, n, n, (0, 1, n), (0, n, 1)) == "mfma_f32_256x256_amc4_bmc4"      # A^T . B
+    assert variant(capi.F64, 1, n, n, n, (0, n, 1), (0, n, 1)) == "mfma_f64_256x128_akc2_bmc2"
+    assert variant(capi.F32, 1, 6144, 6144, 6144, (0, 6144, 1), (0, 6144, 1)) == "mfma_f32_128x128_akc4_bmc4"
+    # a row of C too long for the 32-bit store offsets of a tile: the vector-ALU kernel takes it
+    assert variant(capi.F32, 1, 64, 64, 1 << 23, (0, 64, 1), (0, 1 << 23, 1)).startswith("simt_f32")
     assert variant(capi.F32, 32, 128, 64, 128, (8192, 64, 1), (8192, 1, 64)) == "mfma_f32_64x64_akc4_bkc4"  # config 2
     assert variant(capi.F32, 1, 256, 512, 256, (0, 512, 1), (0, 256, 1)) == "mfma_f32_64x64_akc4_bmc4_splitk8"  # config 1
     assert variant(capi.F32, 1, 1024, 1024, 10, (0, 1024, 1), (0, 10, 1)) == "mfma_f32_64x64_akc4_bmc1_splitk16"  # skinny N

@@ -461,7 +461,7 @@ conv_fwd_kernel(ConvGeom geo, const T *x, const T *w, const T *bias, T *out, int
     Engine eng;
     eng.init(tid);
     eng.run(sa, sb, smem, K, false);
-    store_tile_dense<T>(eng, out + static_cast<int64_t>(b) * M_ * N_, M_, N_, m0, n0, bias, bias ? 2 : 0, 0, 0);
+    store_tile_dense<T, false>(eng, out + static_cast<int64_t>(b) * M_ * N_, M_, N_, m0, n0, bias, bias ? 2 : 0, 0, 0);
 }
 
 // wt[c][(o, a, b)] = w[o][c][a][b]: the A operand of grad_input with its reduction index contiguous.
@@ -499,7 +499,7 @@ conv_dgrad_kernel(ConvGeom geo, const T *gout, const T *wt, T *gin, int tiles_m,
     Engine eng;
     eng.init(tid);
     eng.run(sa, sb, smem, K, false);
-    store_tile_dense<T>(eng, gin + static_cast<int64_t>(b) * M_ * N_, M_, N_, m0, n0, static_cast<const T *>(nullptr), 0, 0, 0);
+    store_tile_dense<T, true>(eng, gin + static_cast<int64_t>(b) * M_ * N_, M_, N_, m0, n0, static_cast<const T *>(nullptr), 0, 0, 0);
 }
 
 // grad_weight: M = O, N = C*k*k, K = Ho*Wo per image.  Workgroup column `part` = (image group, k slice)
@@ -534,7 +534,7 @@ conv_wgrad_kernel(ConvGeom geo, const T *gout, const T *x, T *partial, int64_t i
         eng.run(sa, sb, smem, k_len, false);
         __syncthreads();  // the next image's prologue overwrites LDS buffer 0
     }
-    store_tile_dense<T>(eng, partial + static_cast<int64_t>(part) * M_ * N_, M_, N_, m0, n0, static_cast<const T *>(nullptr), 0, 0, 0);
+    store_tile_dense<T, true>(eng, partial + static_cast<int64_t>(part) * M_ * N_, M_, N_, m0, n0, static_cast<const T *>(nullptr), 0, 0, 0);
 }
 
 // out[i] = sum over parts of partial[s][i].  A workgroup owns 16 consecutive elements; its 16 lanes per element
@@ -659,6 +659,7 @@ ttamd_status make_plan(const char *who, ttamd_dtype dtype, const ttamd_view4 *in
     const int64_t w_reach = (static_cast<int64_t>(O - 1) * weight->stride[0] + static_cast<int64_t>(C) * k * k) * static_cast<int64_t>(esz);
     const int64_t limit = 0x7fffffffLL;
     if (x_reach >= limit || w_reach >= limit || static_cast<int64_t>(O) * Ho * Wo * static_cast<int64_t>(esz) >= limit ||
+        static_cast<int64_t>(C) * H * W * static_cast<int64_t>(esz) >= limit ||
         static_cast<int64_t>(C) * k * k >= (1 << 24) || static_cast<int64_t>(O) * k * k >= (1 << 24) ||
         static_cast<int64_t>(H) * W >= limit / 8 || input->stride[1] >= limit / 8 || input->stride[2] >= limit / 8 ||
         input->stride[3] >= limit / 8) {

@@ -21,7 +21,12 @@ using namespace mfma;
 // PF = tiles kept in flight in registers: 1 for the big tiles (two workgroups per CU hide each other's load
 // latency, and registers are scarce), more for the 64 x 64 tile whose 16 MFMAs per k tile (~0.45 us) are far
 // shorter than a global load.
-template <typename T, int BM, int BN, int BK, int WGM, int WGN, bool A_KC, int A_VEC, bool B_KC, int B_VEC, int PF>
+// EPI: which epilogues the kernel carries.  kEpiAny tests the epilogue flags at run time and supports split k (the
+// 64 x 64 tile).  The big tiles are compiled twice, kEpiLean (plain store only) and kEpiFull (bias / ReLU /
+// accumulate), and never split k: with both store walks in one kernel the register allocator spills accumulators
+// ahead of the branch for the sake of the heavier walk, and the plain store pays for it.
+constexpr int kEpiAny = 0, kEpiLean = 1, kEpiFull = 2;
+template <typename T, int BM, int BN, int BK, int WGM, int WGN, bool A_KC, int A_VEC, bool B_KC, int B_VEC, int PF, int EPI>
 __global__ void __launch_bounds__(kThreads, (BM * BN * sizeof(T) > 256 * 128 * 4 || (sizeof(T) == 8 && BM * BN >= 128 * 128)) ? 1 : 2)  // 256 x 256 (fp64 128 x 128 and up): one workgroup per CU, accumulators in AGPRs
 gemm_mfma_kernel(GemmArgs g, int tiles_m, int tiles_n, int ksplit, int k_chunk, T *partial) {
     using StA = Stager<T, BM, BK, A_KC, A_VEC, PF>;
@@ -52,15 +57,19 @@ gemm_mfma_kernel(GemmArgs g, int tiles_m, int tiles_n, int ksplit, int k_chunk, 
     eng.init(tid);
     eng.run(sa, sb, smem, Kc, !sa.edge && !sb.edge && Kc % BK == 0);
 
-    if (ksplit == 1) {
-        T *C = static_cast<T *>(g.C) + static_cast<int64_t>(batch) * g.M * g.N;
-        if (g.bias_mode == 0 && !g.relu && !g.accumulate)  // the common case gets a store loop free of epilogue tests
-            store_tile_dense<T>(eng, C, g.M, g.N, m0, n0, static_cast<const T *>(nullptr), 0, 0, 0);
+    T *C = static_cast<T *>(g.C) + static_cast<int64_t>(batch) * g.M * g.N;
+    if constexpr (EPI == kEpiLean) {
+        store_tile_dense<T, true>(eng, C, g.M, g.N, m0, n0, static_cast<const T *>(nullptr), 0, 0, 0);
+    } else if constexpr (EPI == kEpiFull) {
+        store_tile_dense<T, false>(eng, C, g.M, g.N, m0, n0, static_cast<const T *>(g.bias), g.bias_mode, g.relu, g.accumulate);
+    } else if (ksplit == 1) {
+        if (g.bias_mode == 0 && !g.relu && !g.accumulate)  // the common case gets a store loop free of epilogue work
+            store_tile_dense<T, true>(eng, C, g.M, g.N, m0, n0, static_cast<const T *>(nullptr), 0, 0, 0);
         else
-            store_tile_dense<T>(eng, C, g.M, g.N, m0, n0, static_cast<const T *>(g.bias), g.bias_mode, g.relu, g.accumulate);
+            store_tile_dense<T, false>(eng, C, g.M, g.N, m0, n0, static_cast<const T *>(g.bias), g.bias_mode, g.relu, g.accumulate);
     } else {
-        store_tile_dense<T>(eng, partial + static_cast<int64_t>(z) * g.M * g.N, g.M, g.N, m0, n0,
-                            static_cast<const T *>(nullptr), 0, 0, 0);
+        store_tile_dense<T, true>(eng, partial + static_cast<int64_t>(z) * g.M * g.N, g.M, g.N, m0, n0,
+                                  static_cast<const T *>(nullptr), 0, 0, 0);
     }
 }
 
@@ -136,12 +145,20 @@ ttamd_status launch_variant(const GemmArgs &g, const SplitPlan &sp, int device, 
     using StA = Stager<T, BM, BK, A_KC, A_VEC, PF>;
     using StB = Stager<T, BN, BK, B_KC, B_VEC, PF>;
     constexpr size_t lds_bytes = TileEngine<T, BM, BN, BK, WGM, WGN, StA, StB>::kLdsBytes;
-    auto kernel = gemm_mfma_kernel<T, BM, BN, BK, WGM, WGN, A_KC, A_VEC, B_KC, B_VEC, PF>;
-    static bool configured = false;  // raising the dynamic LDS limit is per kernel, once
-    if (!configured && lds_bytes > 48 * 1024) {
+    constexpr bool kTwoKernels = BM * BN >= 128 * 128;
+    const bool lean = g.bias_mode == 0 && !g.relu && !g.accumulate;
+    if (kTwoKernels && sp.ksplit != 1) {
+        set_error("batched_matmul: internal error, split k planned for a %d x %d tile", BM, BN);
+        return TTAMD_ERR_INVALID_ARGUMENT;
+    }
+    constexpr int kEpiA = kTwoKernels ? kEpiLean : kEpiAny, kEpiB = kTwoKernels ? kEpiFull : kEpiAny;
+    auto kernel = lean ? gemm_mfma_kernel<T, BM, BN, BK, WGM, WGN, A_KC, A_VEC, B_KC, B_VEC, PF, kEpiA>
+                       : gemm_mfma_kernel<T, BM, BN, BK, WGM, WGN, A_KC, A_VEC, B_KC, B_VEC, PF, kEpiB>;
+    static bool configured[2] = {false, false};  // raising the dynamic LDS limit is per kernel, once
+    if (!configured[lean] && lds_bytes > 48 * 1024) {
         TTAMD_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
                                             hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_bytes)));
-        configured = true;
+        configured[lean] = true;
     }
     const int tiles_m = (g.M + BM - 1) / BM, tiles_n = (g.N + BN - 1) / BN;
     const int64_t blocks = static_cast<int64_t>(tiles_m) * tiles_n * g.batch * sp.ksplit;
@@ -242,7 +259,8 @@ ttamd_status launch_mfma_typed(const GemmArgs &g, int device, hipStream_t stream
     // 32-bit buffer addressing: the bytes reachable from a tile's first row must stay below 2^31.
     const int64_t a_reach = (static_cast<int64_t>(bm - 1) * g.a_sm + static_cast<int64_t>(g.K - 1) * g.a_sk + VK) * sizeof(T);
     const int64_t b_reach = (static_cast<int64_t>(bm - 1) * g.b_sn + static_cast<int64_t>(g.K - 1) * g.b_sk + VK) * sizeof(T);
-    if (a_reach >= 0x7fffffffLL || b_reach >= 0x7fffffffLL) return TTAMD_OK;
+    const int64_t c_reach = static_cast<int64_t>(g.M < bm ? g.M : bm) * g.N * static_cast<int64_t>(sizeof(T));
+    if (a_reach >= 0x7fffffffLL || b_reach >= 0x7fffffffLL || c_reach >= 0x7fffffffLL) return TTAMD_OK;
 
     const SplitPlan sp = (xxl || xl || large) ? SplitPlan{1, g.K} : plan_split<T>(g, TS::SBM, TS::SBN, TS::SBK);
 

@@ -105,6 +105,22 @@ struct Vec<double, 2> {
     }
 };
 
+// Typed buffer stores of one element or of a pair of neighbouring elements.
+using u32x2 = uint32_t __attribute__((ext_vector_type(2)));
+using u32x4 = uint32_t __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ void buffer_store(__amdgpu_buffer_rsrc_t r, uint32_t off, float v) {
+    __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(uint32_t, v), r, off, 0, 0);
+}
+__device__ __forceinline__ void buffer_store(__amdgpu_buffer_rsrc_t r, uint32_t off, double v) {
+    __builtin_amdgcn_raw_buffer_store_b64(__builtin_bit_cast(u32x2, v), r, off, 0, 0);
+}
+__device__ __forceinline__ void buffer_store(__amdgpu_buffer_rsrc_t r, uint32_t off, f32x2 v) {
+    __builtin_amdgcn_raw_buffer_store_b64(__builtin_bit_cast(u32x2, v), r, off, 0, 0);
+}
+__device__ __forceinline__ void buffer_store(__amdgpu_buffer_rsrc_t r, uint32_t off, f64x2 v) {
+    __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, v), r, off, 0, 0);
+}
+
 template <typename T, int VEC>
 __device__ __forceinline__ void zero_component(typename Vec<T, VEC>::type &v, int j) {
     if constexpr (VEC == 1) {
@@ -314,6 +330,7 @@ template <typename T, int BM, int BN, int BK, int WGM, int WGN, class StA, class
 struct TileEngine {
     using M = Mfma<T>;
     static_assert(WGM * WGN == kWaves, "4 waves per workgroup");
+    static constexpr int kBM = BM, kBN = BN;
     static constexpr int WM = BM / WGM, WN = BN / WGN;
     static constexpr int NBM = WM / M::MB, NBN = WN / M::MB;
     static_assert(WM % M::MB == 0 && WN % M::MB == 0 && BK % kChunk == 0, "tile shape");
@@ -715,72 +732,95 @@ struct TileEngine {
     // Walks the finished tile.  `one(m, n, v)` receives a single element at tile-local (m, n);
     // `two(m, n, v0, v1)` receives columns n and n + 1 of the same row (only called when B is MC/paired and
     // `pairs_ok`); both are expected to do their own bounds checks against the matrix size.
-    template <class One, class Two>
+    // FENCE keeps the scheduler from hoisting the work of later blocks over the stores of earlier ones (an epilogue
+    // that loads per element would otherwise hold a whole tile's loads in flight and spill).
+    template <bool FENCE = false, class One, class Two>
     __device__ __forceinline__ void for_each(bool pairs_ok, One one, Two two) {
         const int jcol = lane % M::MB;
-        if constexpr (FrB::PAIRED) {
-#pragma unroll
-            for (int pr = 0; pr < NBN / 2; ++pr) {
-                const int n = FrB::index_of(wn0, 2 * pr, jcol);  // even column; n + 1 belongs to block 2p+1
-#pragma unroll
-                for (int bm = 0; bm < NBM; ++bm)
-#pragma unroll
-                    for (int e = 0; e < M::NACC; ++e) {
-                        const int m = FrA::index_of(wm0, bm, M::acc_row(e, lane));
-                        if (pairs_ok) {
-                            two(m, n, acc[bm][2 * pr][e], acc[bm][2 * pr + 1][e]);
-                        } else {
-                            one(m, n, acc[bm][2 * pr][e]);
-                            one(m, n + 1, acc[bm][2 * pr + 1][e]);
-                        }
-                    }
-            }
-        } else {
+        auto singles = [&]() {
 #pragma unroll
             for (int bn = 0; bn < NBN; ++bn) {
                 const int n = FrB::index_of(wn0, bn, jcol);
 #pragma unroll
-                for (int bm = 0; bm < NBM; ++bm)
+                for (int bm = 0; bm < NBM; ++bm) {
 #pragma unroll
                     for (int e = 0; e < M::NACC; ++e) one(FrA::index_of(wm0, bm, M::acc_row(e, lane)), n, acc[bm][bn][e]);
+                    if constexpr (FENCE) __builtin_amdgcn_sched_barrier(0);
+                }
             }
+        };
+        if constexpr (FrB::PAIRED) {
+            if (pairs_ok) {
+#pragma unroll
+                for (int pr = 0; pr < NBN / 2; ++pr) {
+                    const int n = FrB::index_of(wn0, 2 * pr, jcol);  // even column; n + 1 belongs to block 2p+1
+#pragma unroll
+                    for (int bm = 0; bm < NBM; ++bm) {
+#pragma unroll
+                        for (int e = 0; e < M::NACC; ++e)
+                            two(FrA::index_of(wm0, bm, M::acc_row(e, lane)), n, acc[bm][2 * pr][e], acc[bm][2 * pr + 1][e]);
+                        if constexpr (FENCE) __builtin_amdgcn_sched_barrier(0);
+                    }
+                }
+            } else {
+                singles();
+            }
+        } else {
+            singles();
         }
     }
 };
 
 // Dense row-major store of a finished tile with the optional bias / ReLU / accumulate epilogue.
 // C points at the matrix (already offset to the batch), M x N its size, (m0, n0) the tile origin.
-template <typename T, class Engine>
+//
+// The tile is written through a buffer descriptor that starts at C[m0][n0] and ends with the last row of the matrix
+// that the tile touches; an element outside the matrix gets the out-of-range offset and the hardware drops its
+// store.  One straight-line path serves interior and edge tiles and an element costs one 32-bit offset.  The host
+// only sends matrices here whose rows under one tile span less than 2^31 bytes (min(BM, M) * N * sizeof(T)).
+// LEAN: no bias, ReLU or accumulation (those arguments are then ignored).
+template <typename T, bool LEAN, class Engine>
 __device__ __forceinline__ void store_tile_dense(Engine &eng, T *__restrict__ C, int M_, int N_, int m0, int n0,
                                                  const T *__restrict__ bias, int bias_mode, int relu, int accumulate) {
     using pair_t = typename Mfma<T>::pair_t;
-    auto finish = [&](T v, int m, int n, int64_t idx) {
-        if (bias_mode == 1) v += bias[n];
-        if (bias_mode == 2) v += bias[m];
-        if (relu) v = v > T(0) ? v : T(0);
-        if (accumulate) v += C[idx];
+    constexpr uint32_t kOob = 0x80000000u;
+    const int rows = M_ - m0 < Engine::kBM ? M_ - m0 : Engine::kBM;
+    const int cols = N_ - n0;
+    const __amdgpu_buffer_rsrc_t out = make_rsrc(C + static_cast<int64_t>(m0) * N_ + n0,
+                                                 (static_cast<int64_t>(rows) * N_ - n0) * static_cast<int64_t>(sizeof(T)));
+    // The epilogue options are uniform run-time flags.  Branching on them per element would put hundreds of branches
+    // into the unrolled walk, so they are folded into data instead: a bias that is absent and a C that is not
+    // accumulated into are read through descriptors of zero length, whose loads return 0 without touching memory.
+    constexpr int64_t kSz = sizeof(T);
+    const __amdgpu_buffer_rsrc_t bias_n = make_rsrc(bias, bias_mode == 1 ? N_ * kSz : 0);
+    const __amdgpu_buffer_rsrc_t bias_m = make_rsrc(bias, bias_mode == 2 ? M_ * kSz : 0);
+    const __amdgpu_buffer_rsrc_t prev = make_rsrc(C + static_cast<int64_t>(m0) * N_ + n0,
+                                                  accumulate ? (static_cast<int64_t>(rows) * N_ - n0) * kSz : 0);
+    auto offset_of = [&](int ml, int nl) {
+        return (ml < rows && nl < cols) ? static_cast<uint32_t>(ml * N_ + nl) * static_cast<uint32_t>(sizeof(T)) : kOob;
+    };
+    auto finish = [&](T v, int ml, int nl, uint32_t off) {
+        if constexpr (LEAN) return v;
+        v += Vec<T, 1>::load(bias_n, static_cast<uint32_t>(n0 + nl) * static_cast<uint32_t>(sizeof(T)));
+        v += Vec<T, 1>::load(bias_m, static_cast<uint32_t>(m0 + ml) * static_cast<uint32_t>(sizeof(T)));
+        v = (v > T(0) || !relu) ? v : T(0);
+        v += Vec<T, 1>::load(prev, off);
         return v;
     };
+    // pairs: n is even and N is even, so n + 1 < N whenever n < N and a wave writes whole row segments
     const bool pairs_ok = (N_ % 2 == 0) && (reinterpret_cast<uintptr_t>(C) % (2 * sizeof(T)) == 0);
-    eng.for_each(
+    eng.template for_each<!LEAN>(
         pairs_ok,
         [&](int ml, int nl, T v) {
-            const int m = m0 + ml, n = n0 + nl;
-            if (m < M_ && n < N_) {
-                const int64_t idx = static_cast<int64_t>(m) * N_ + n;
-                C[idx] = finish(v, m, n, idx);
-            }
+            const uint32_t off = offset_of(ml, nl);
+            buffer_store(out, off, finish(v, ml, nl, off));
         },
         [&](int ml, int nl, T v0, T v1) {
-            // n is even and N_ is even, so n + 1 < N_ whenever n < N_: a wave writes whole row segments
-            const int m = m0 + ml, n = n0 + nl;
-            if (m < M_ && n < N_) {
-                const int64_t idx = static_cast<int64_t>(m) * N_ + n;
-                pair_t out;
-                out[0] = finish(v0, m, n, idx);
-                out[1] = finish(v1, m, n + 1, idx + 1);
-                *reinterpret_cast<pair_t *>(&C[idx]) = out;
-            }
+            const uint32_t off = offset_of(ml, nl);
+            pair_t o;
+            o[0] = finish(v0, ml, nl, off);
+            o[1] = finish(v1, ml, nl + 1, off + static_cast<uint32_t>(sizeof(T)));
+            buffer_store(out, off, o);
         });
 }
 
