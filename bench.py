@@ -21,7 +21,7 @@ PEAK_TFLOPS = {"f32": 157.3, "f64": 78.6}  # MI355X dense matrix peaks
 # FETCH_SIZE / WRITE_SIZE passes summarised in profiles/gemm_4096_f32_f64_mfma.txt (scaled by the same counters'
 # reading for a copy kernel of known size: x2.000 for reads, x1.000 for writes).  Only valid for that exact
 # kernel and size; reported as null otherwise.  Algorithmic bytes are 3 * 4096^2 * 4 = 201.3e6.
-MEASURED_TRAFFIC = {("mfma_f32_256x128_akc4_bmc4", 4096): (339162.2 * 2.0 + 65536.0) * 1024.0}
+MEASURED_TRAFFIC = {("mfma_f32_256x256_akc4_bmc4", 4096): (196856.1 * 2.0 + 65536.0) * 1024.0}
 
 
 def gpu_gemm_timing(tt, np, dtype, n, steps, warmup):
