@@ -290,6 +290,34 @@ def test_epilogue_bias_relu_accumulate(tt, oracle, dtype):
     assert np.array_equal(got, np.maximum(X @ W10 + b10, 0))
 
 
+# The big tiles exist as separate plain-store and full-epilogue kernels; these shapes select them (asserted) with
+# ragged edges in both directions.  Small integers and a short K keep every result exact, so the bar is bit-exact.
+@pytest.mark.parametrize("dtype,N,M,layout,tile", [
+    (np.float32, 3900, 4000, "nn", "256x256"), (np.float32, 3900, 3999, "nt", "256x256"),
+    (np.float32, 3904, 4000, "tn", "256x256"), (np.float32, 3904, 3999, "tt", "256x256"),
+    (np.float32, 6100, 6000, "nn", "128x128"), (np.float32, 6100, 5999, "nt", "128x128"),
+    (np.float64, 3900, 4000, "nn", "256x128"), (np.float64, 3900, 3999, "nt", "256x128"),
+    (np.float64, 3904, 4000, "tn", "256x128"),
+])
+def test_big_tile_epilogues_and_edges(tt, dtype, N, M, layout, tile):
+    K = 40
+    rng = np.random.default_rng(N + M)
+    ints = lambda *shape: rng.integers(-4, 5, shape).astype(dtype)
+    A = ints(1, N, K) if layout[0] == "n" else ints(1, K, N).transpose(0, 2, 1)
+    B = ints(1, K, M) if layout[1] == "n" else ints(1, M, K).transpose(0, 2, 1)
+    tA, tB = to_dev_view(tt, A), to_dev_view(tt, B)
+    be = tt.get_backend(tt.kAMD)
+    assert f"_{tile}_" in be.batched_matmul_variant(tA, tB)
+    want = A[0].astype(np.float64) @ B[0].astype(np.float64)  # exact: |sum| <= 40 * 16
+    assert np.array_equal(be.batched_matmul(tA, tB).to_numpy()[0], want)
+    col_bias, row_bias, prev = ints(M), ints(N), ints(1, N, M)
+    got = be.batched_matmul(tA, tB, bias=dev(tt, col_bias), bias_mode=1, relu=True).to_numpy()[0]
+    assert np.array_equal(got, np.maximum(want + col_bias, 0))
+    acc = dev(tt, prev)
+    be.batched_matmul(tA, tB, out=acc, bias=dev(tt, row_bias), bias_mode=2, accumulate=True)
+    assert np.array_equal(acc.to_numpy()[0], want + row_bias[:, None] + prev[0])
+
+
 def test_contiguous_identity(tt, oracle):
     rng = np.random.default_rng(2)
     for dtype in (np.uint8, np.int16, np.float32, np.float64):
