@@ -18,9 +18,11 @@ using namespace mfma;
 
 // ksplit > 1: the reduction is cut into `ksplit` ranges of `k_chunk` (a multiple of BK); workgroup column z =
 // batch * ksplit + split writes the raw partial tile to `partial[z]` and splitk_reduce_kernel finishes the job.
-// PF = tiles kept in flight in registers: 1 for the big tiles (two workgroups per CU hide each other's load
-// latency, and registers are scarce), more for the 64 x 64 tile whose 16 MFMAs per k tile (~0.45 us) are far
-// shorter than a global load.
+// PF = tiles kept in flight in registers: 1 for the big tiles (a k tile's MFMA work outlasts a global load there,
+// and registers are scarce), 4 for the fp32 64 x 64 tile, whose 16 MFMAs per k tile (~0.43 us) are shorter than a
+// load from L2 under traffic: with one tile in flight a lone workgroup on a CU (1024^3 is 256 tiles) waited for
+// memory in every step.  Measured: 1024 x 784 x 1024 26.2 -> 22.1 us, 1024 x 4096 x 1024 87 -> 78 us, 3072^3 127 -> 131
+// TFLOP/s, although the extra 64 registers halve the resident workgroups per CU.
 // EPI: which epilogues the kernel carries.  kEpiAny tests the epilogue flags at run time and supports split k (the
 // 64 x 64 tile).  The big tiles are compiled twice, kEpiLean (plain store only) and kEpiFull (bias / ReLU /
 // accumulate), and never split k: with both store walks in one kernel the register allocator spills accumulators
@@ -120,7 +122,7 @@ struct TileShapes<float> {
     static constexpr int XBM = 256, XBN = 128, XBK = 16;  // extra large: 4 waves of 128 x 64 (4 x 2 MFMA blocks)
     static constexpr int LBM = 128, LBN = 128, LBK = 16;  // large: 4 waves of 64 x 64
     static constexpr int SBM = 64, SBN = 64, SBK = 32;    // small: 4 waves of 32 x 32
-    static constexpr int SPF = 1;                          // deeper register prefetch measured slower (more registers, same stalls)
+    static constexpr int SPF = 4;                          // k tiles in flight in registers (16-byte operands only)
     static constexpr const char *prefix = "mfma_f32";
 };
 template <>
@@ -130,7 +132,7 @@ struct TileShapes<double> {
     static constexpr int XBM = 256, XBN = 128, XBK = 16;  // 4 waves of 128 x 64 (8 x 4 blocks of 16 x 16), one workgroup per CU
     static constexpr int LBM = 128, LBN = 128, LBK = 16;  // 4 waves of 64 x 64 (4 x 4 blocks of 16 x 16)
     static constexpr int SBM = 64, SBN = 64, SBK = 16;    // 4 waves of 32 x 32
-    static constexpr int SPF = 1;
+    static constexpr int SPF = 4;
     static constexpr const char *prefix = "mfma_f64";
 };
 
@@ -141,7 +143,7 @@ struct SplitPlan {
 
 template <typename T, int BM, int BN, int BK, int WGM, int WGN, bool A_KC, int A_VEC, bool B_KC, int B_VEC>
 ttamd_status launch_variant(const GemmArgs &g, const SplitPlan &sp, int device, hipStream_t stream) {
-    constexpr int PF = (BM <= 64 && BN <= 64) ? TileShapes<T>::SPF : 1;
+    constexpr int PF = (BM <= 64 && BN <= 64 && A_VEC > 1 && B_VEC > 1) ? TileShapes<T>::SPF : 1;  // gathers: registers
     using StA = Stager<T, BM, BK, A_KC, A_VEC, PF>;
     using StB = Stager<T, BN, BK, B_KC, B_VEC, PF>;
     constexpr size_t lds_bytes = TileEngine<T, BM, BN, BK, WGM, WGN, StA, StB>::kLdsBytes;
@@ -235,21 +237,21 @@ ttamd_status launch_mfma_typed(const GemmArgs &g, int device, hipStream_t stream
     // CUs round-robin, so a partial last round costs a whole round as soon as any CU holds a full complement,
     // and a fraction of it when the CUs are thinly populated (a workgroup alone on a CU runs faster).
     const double scale = sizeof(T) == 4 ? 1.0 : 0.5;
-    auto estimate = [&](int bm_, int bn_, int per_cu, double rate) {
+    auto estimate = [&](int bm_, int bn_, int per_cu, double rate, double thin = 0.12) {
         const double tiles = static_cast<double>((g.M + bm_ - 1) / bm_) * ((g.N + bn_ - 1) / bn_) * g.batch;
         const double slots = 256.0 * per_cu;
         const double rounds = std::floor(tiles / slots), frac = tiles / slots - rounds;
         double last = 0.0;
         if (frac > 0.0) {
             const double fill = std::ceil(frac * per_cu - 1e-9) / per_cu;  // busiest CU's share of its slots
-            last = fill >= 1.0 ? 1.0 : 0.12 + 0.88 * fill;
+            last = fill >= 1.0 ? 1.0 : thin + (1.0 - thin) * fill;
         }
         const double round_time = 2.0 * bm_ * bn_ * static_cast<double>(g.K) * slots / (rate * scale);
         return (rounds + last) * round_time;
     };
     const double t_small = estimate(TS::SBM, TS::SBN, 4, 131e12);
     constexpr bool f32 = sizeof(T) == 4;  // the fp64 big tiles run one workgroup per CU (accumulators in AGPRs)
-    const double t_large = vec ? estimate(TS::LBM, TS::LBN, f32 ? 2 : 1, f32 ? 145e12 : 141e12) : 1e300;
+    const double t_large = vec ? estimate(TS::LBM, TS::LBN, f32 ? 2 : 1, f32 ? 145e12 : 141e12, 0.08) : 1e300;
     const double t_xl = (TS::kHasXL && vec) ? estimate(TS::XBM, TS::XBN, f32 ? 2 : 1, f32 ? 145e12 : 147e12) : 1e300;
     const double t_xxl = (TS::kHasXL && vec && sizeof(T) == 4) ? estimate(TS::YBM, TS::YBN, 1, 147e12) : 1e300;
     const bool xxl = t_xxl <= t_xl && t_xxl <= t_large && t_xxl <= t_small;

@@ -456,6 +456,25 @@ struct TileEngine {
         }
     }
 
+    // PF consecutive steps starting at a tile index kt with kt % PF == 1: slots 1, 2, .., PF - 1, 0.
+    template <bool MASK, int I>
+    __device__ __forceinline__ void step_group(StA &sa, StB &sb, T *smem, int K, int kt) {
+        if constexpr (I < StA::kPF) {
+            step_rot<(1 + I) % StA::kPF, true, MASK, true>(sa, sb, smem, K, kt + I);
+            step_group<MASK, I + 1>(sa, sb, smem, K, kt);
+        }
+    }
+    // the last steps (fewer than PF), same slot sequence
+    template <bool MASK, int I>
+    __device__ __forceinline__ void step_tail(StA &sa, StB &sb, T *smem, int K, int kt, int steps) {
+        if constexpr (I < StA::kPF - 1) {
+            if (kt + I < steps) {
+                step_rot<(1 + I) % StA::kPF, true, MASK, true>(sa, sb, smem, K, kt + I);
+                step_tail<MASK, I + 1>(sa, sb, smem, K, kt, steps);
+            }
+        }
+    }
+
     __device__ __forceinline__ void run_rot(StA &sa, StB &sb, T *smem, int K, bool unmasked) {
         constexpr int PF = StA::kPF;
         constexpr int NC = BK / kChunk;
@@ -470,6 +489,19 @@ struct TileEngine {
         // Tiles 0 .. KT-2; the first step has no pending chunk.  While kt + PF < KT a step also issues loads; the
         // remaining steps only drain the slots.
         auto pipeline = [&]<bool MASK>() {
+            if constexpr (PF > 1) {
+                // Register slots are static inside a group of PF steps, so the compiler's wait counters know exactly
+                // which loads a store depends on (a run-time slot switch merges the counters at every branch and
+                // each store then waits for all loads in flight, the newest included).  Every step requests tile
+                // kt + PF; past the end of K those loads come back as zeros (or unused data) and are never parked.
+                const int steps = KT - 1;
+                if (steps <= 0) return;
+                step_rot<0, true, MASK, false>(sa, sb, smem, K, 0);
+                int kt = 1;
+                for (; kt + PF <= steps; kt += PF) step_group<MASK, 0>(sa, sb, smem, K, kt);
+                step_tail<MASK, 0>(sa, sb, smem, K, kt, steps);
+                return;
+            }
             int kt = 0, slot = 0;
             auto advance = [&] {
                 ++kt;
