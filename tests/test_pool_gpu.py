@@ -38,7 +38,9 @@ def test_reference_shape_forward_backward_exact(tt, oracle, op, dtype):
 
 @pytest.mark.parametrize("op", OPS)
 @pytest.mark.parametrize("dtype", ALL_NON_BOOL)
-@pytest.mark.parametrize("geom", [(2, 3, 9, 8, 2, 2, 0), (1, 2, 7, 7, 3, 1, 1), (2, 2, 6, 9, 3, 3, 2), (1, 1, 5, 5, 5, 1, 2), (3, 1, 1, 1, 1, 1, 0)])
+@pytest.mark.parametrize("geom", [(2, 3, 9, 8, 2, 2, 0), (1, 2, 7, 7, 3, 1, 1), (2, 2, 6, 9, 3, 3, 2), (1, 1, 5, 5, 5, 1, 2), (3, 1, 1, 1, 1, 1, 0),
+                                  # non-overlapping windows: odd width (no pair accesses), rows / columns no window reaches
+                                  (2, 3, 9, 7, 2, 2, 0), (1, 2, 10, 11, 3, 3, 0), (2, 2, 8, 8, 4, 4, 0), (1, 3, 64, 66, 2, 2, 0)])
 def test_every_dtype_and_geometry_exact(tt, oracle, op, dtype, geom):
     Bn, Cc, H, W, k, S, P = geom
     rng = np.random.default_rng(sum(geom))
@@ -62,12 +64,13 @@ def test_strided_input_view_empty_batch_and_errors(tt, oracle):
     tx = dev(tt, xs).permute(0, 3, 1, 2)
     assert not tx.is_contiguous()
     for op in OPS:
-        out = forward(tt, op, tx, 3, 2, 1)
-        want = oracle.pool2d_forward(x, op, 3, 2, 1)
-        assert np.array_equal(out.to_numpy(), want)
-        g = rng.normal(size=want.shape).astype(np.float32)
-        gx = tt.pool2d_backward(dev(tt, g), tx, out, op, 3, 2, 1)
-        assert gx.is_contiguous() and np.array_equal(gx.to_numpy(), oracle.pool2d_backward(g, x, want, op, 3, 2, 1))
+        for k, S, P in ((3, 2, 1), (2, 2, 0)):
+            out = forward(tt, op, tx, k, S, P)
+            want = oracle.pool2d_forward(x, op, k, S, P)
+            assert np.array_equal(out.to_numpy(), want)
+            g = rng.normal(size=want.shape).astype(np.float32)
+            gx = tt.pool2d_backward(dev(tt, g), tx, out, op, k, S, P)
+            assert gx.is_contiguous() and np.array_equal(gx.to_numpy(), oracle.pool2d_backward(g, x, want, op, k, S, P))
     empty = tt.Tensor.empty((0, 3, 8, 8), tt._capi.F32)
     assert tt.max_pool2d(empty, 2, 2, 0).shape == (0, 3, 4, 4)
     with pytest.raises(tt.TTException):

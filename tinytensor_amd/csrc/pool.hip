@@ -17,6 +17,12 @@
 // For max / min a first pass over the outputs computes each output's share (gradient / number of window elements
 // equal to the result) into the library's per-stream scratch, so the gather reads two values per covering output
 // instead of recounting its window.
+//
+// Non-overlapping windows without padding (stride == k, padding == 0: the max_pool2d(x, 2, 2, 0) of
+// examples/mnist_cnn_example.cpp:55) take a shorter road: an input element lies in at most one window, so backward
+// is one pass with one lane per output that reads its window once, counts, and writes the window's gradients
+// (plus zeros for rows / columns that no window reaches); with k == 2 and even dense rows both directions move
+// their rows as 2-element vectors, so a wave reads and writes whole contiguous row segments.
 #include "common.h"
 
 #include <cfloat>
@@ -149,6 +155,113 @@ pool_backward_kernel(PoolGeom g, const R *__restrict__ share, const R *__restric
     gin[static_cast<int64_t>(plane) * (g.H * g.W) + pos] = acc;
 }
 
+template <typename T>
+using Pair = T __attribute__((ext_vector_type(2)));
+
+// Forward for k == 2, stride == 2, padding == 0 on rows that can be read as aligned pairs (the host checks).
+// Same visiting order and arithmetic as pool_forward_kernel.
+template <typename T, typename R, int OP>
+__global__ void __launch_bounds__(256) pool_forward_k2_kernel(PoolGeom g, const T *__restrict__ x, R *__restrict__ out) {
+    uint32_t plane, blk;
+    g.d_out_blocks.divmod(blockIdx.x, plane, blk);
+    const uint32_t pos = blk * 256 + threadIdx.x;
+    if (pos >= static_cast<uint32_t>(g.Ho * g.Wo)) return;
+    uint32_t h, w;
+    g.d_Wo.divmod(pos, h, w);
+    const T *src = plane_of(g, x, plane) + static_cast<int64_t>(2 * h) * g.xs_h + 2 * w;
+    const Pair<T> r0 = *reinterpret_cast<const Pair<T> *>(src), r1 = *reinterpret_cast<const Pair<T> *>(src + g.xs_h);
+    const R v[4] = {static_cast<R>(r0[0]), static_cast<R>(r0[1]), static_cast<R>(r1[0]), static_cast<R>(r1[1])};
+    R acc = pool_init<R, OP>();
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        if constexpr (OP == POOL_MAX) acc = (v[i] > acc) ? v[i] : acc;
+        else if constexpr (OP == POOL_MIN) acc = (v[i] < acc) ? v[i] : acc;
+        else acc = (v[i] / R(4)) + acc;
+    }
+    out[static_cast<int64_t>(plane) * (g.Ho * g.Wo) + pos] = acc;
+}
+
+// Backward for non-overlapping windows (stride == k, padding == 0), one lane per output: the window's elements
+// receive grad_out / (number of elements equal to the result) where they equal it (SELECT), or grad_out / k^2
+// each; an element gets its single contribution as 0 + amount, the value the reference's zero-initialised sum
+// ends with.  Input rows and columns beyond the last window are zero-filled by the lanes of the last output row /
+// column.  K2: k == 2 on rows that can be moved as aligned pairs.
+template <typename R, bool SELECT, bool K2>
+__global__ void __launch_bounds__(256)
+pool_backward_window_kernel(PoolGeom g, const R *__restrict__ gout, const R *__restrict__ x, const R *__restrict__ res,
+                            R *__restrict__ gin) {
+    uint32_t plane, blk;
+    g.d_out_blocks.divmod(blockIdx.x, plane, blk);
+    const uint32_t pos = blk * 256 + threadIdx.x;
+    if (pos >= static_cast<uint32_t>(g.Ho * g.Wo)) return;
+    uint32_t h, w;
+    g.d_Wo.divmod(pos, h, w);
+    const int64_t o = static_cast<int64_t>(plane) * (g.Ho * g.Wo) + pos;
+    const int K = K2 ? 2 : g.K;
+    const int y0 = static_cast<int>(h) * K, x0 = static_cast<int>(w) * K;
+    const R *src = plane_of(g, x, plane);
+    R *dst = gin + static_cast<int64_t>(plane) * (g.H * g.W);
+    const R go = gout[o];
+    if constexpr (K2) {
+        Pair<R> d0, d1;
+        if constexpr (SELECT) {
+            const R *s0 = src + static_cast<int64_t>(y0) * g.xs_h + x0;
+            const Pair<R> r0 = *reinterpret_cast<const Pair<R> *>(s0), r1 = *reinterpret_cast<const Pair<R> *>(s0 + g.xs_h);
+            const R target = res[o];
+            const R count = ((r0[0] == target) ? R(1) : R(0)) + ((r0[1] == target) ? R(1) : R(0)) +
+                            ((r1[0] == target) ? R(1) : R(0)) + ((r1[1] == target) ? R(1) : R(0));
+            const R share = go / count;
+            d0[0] = R(0) + ((r0[0] == target) ? share : R(0));
+            d0[1] = R(0) + ((r0[1] == target) ? share : R(0));
+            d1[0] = R(0) + ((r1[0] == target) ? share : R(0));
+            d1[1] = R(0) + ((r1[1] == target) ? share : R(0));
+        } else {
+            const R amount = R(0) + go / R(4);
+            d0[0] = d0[1] = d1[0] = d1[1] = amount;
+        }
+        R *t0 = dst + static_cast<int64_t>(y0) * g.W + x0;
+        *reinterpret_cast<Pair<R> *>(t0) = d0;
+        *reinterpret_cast<Pair<R> *>(t0 + g.W) = d1;
+    } else {
+        R share;
+        R target = R(0);
+        if constexpr (SELECT) {
+            target = res[o];
+            R count = R(0);
+            for (int p = 0; p < K; ++p)
+                for (int q = 0; q < K; ++q)
+                    count += (src[static_cast<int64_t>(y0 + p) * g.xs_h + static_cast<int64_t>(x0 + q) * g.xs_w] == target) ? R(1) : R(0);
+            share = go / count;
+        } else {
+            share = go / static_cast<R>(K * K);
+        }
+        for (int p = 0; p < K; ++p)
+            for (int q = 0; q < K; ++q) {
+                bool take = true;
+                if constexpr (SELECT) take = src[static_cast<int64_t>(y0 + p) * g.xs_h + static_cast<int64_t>(x0 + q) * g.xs_w] == target;
+                dst[static_cast<int64_t>(y0 + p) * g.W + x0 + q] = R(0) + (take ? share : R(0));
+            }
+    }
+    // rows and columns that no window covers
+    const bool last_w = static_cast<int>(w) == g.Wo - 1, last_h = static_cast<int>(h) == g.Ho - 1;
+    if (last_w)
+        for (int p = 0; p < K; ++p)
+            for (int c = g.Wo * K; c < g.W; ++c) dst[static_cast<int64_t>(y0 + p) * g.W + c] = R(0);
+    if (last_h) {
+        const int c_end = last_w ? g.W : x0 + K;
+        for (int r = g.Ho * K; r < g.H; ++r)
+            for (int c = x0; c < c_end; ++c) dst[static_cast<int64_t>(r) * g.W + c] = R(0);
+    }
+}
+
+// Rows of the input (and of a dense tensor of the same shape) can be moved as aligned pairs of T.
+template <typename T>
+bool rows_pair_aligned(const PoolGeom &g, const void *x, const void *dense) {
+    const auto even = [](int64_t v) { return v % 2 == 0; };
+    return g.xs_w == 1 && g.W % 2 == 0 && even(g.xs_h) && even(g.xs_c) && even(g.xs_b) &&
+           reinterpret_cast<uintptr_t>(x) % (2 * sizeof(T)) == 0 && reinterpret_cast<uintptr_t>(dense) % (2 * sizeof(T)) == 0;
+}
+
 ttamd_status make_pool_geom(const char *who, int op, const ttamd_view4 *input, int B, int C, int H, int W, int k, int stride,
                             int padding, PoolGeom *g) {
     if (op < POOL_MAX || op > POOL_AVG) {
@@ -199,7 +312,10 @@ ttamd_status make_pool_geom(const char *who, int op, const ttamd_view4 *input, i
 template <typename T, typename R, int OP>
 ttamd_status launch_forward(const PoolGeom &g, const void *x, void *out, hipStream_t st) {
     const unsigned blocks = static_cast<unsigned>(static_cast<int64_t>(g.B) * g.C * g.out_blocks);
-    pool_forward_kernel<T, R, OP><<<dim3(blocks), dim3(256), 0, st>>>(g, static_cast<const T *>(x), static_cast<R *>(out));
+    if (g.K == 2 && g.S == 2 && g.P == 0 && rows_pair_aligned<T>(g, x, x))
+        pool_forward_k2_kernel<T, R, OP><<<dim3(blocks), dim3(256), 0, st>>>(g, static_cast<const T *>(x), static_cast<R *>(out));
+    else
+        pool_forward_kernel<T, R, OP><<<dim3(blocks), dim3(256), 0, st>>>(g, static_cast<const T *>(x), static_cast<R *>(out));
     TTAMD_HIP_CHECK(hipGetLastError());
     return TTAMD_OK;
 }
@@ -217,7 +333,18 @@ ttamd_status backward_typed(int device, int op, const PoolGeom &g, const void *g
                             hipStream_t st) {
     const int64_t planes = static_cast<int64_t>(g.B) * g.C;
     const dim3 in_grid(static_cast<unsigned>(planes * g.in_blocks)), out_grid(static_cast<unsigned>(planes * g.out_blocks)), block(256);
-    if (op == POOL_AVG) {
+    if (g.S == g.K && g.P == 0 && g.Ho > 0 && g.Wo > 0) {
+        const R *go = static_cast<const R *>(gout), *xi = static_cast<const R *>(x), *rs = static_cast<const R *>(res);
+        R *gi = static_cast<R *>(gin);
+        const bool k2 = g.K == 2 && rows_pair_aligned<R>(g, x, gin);
+        if (op == POOL_AVG) {
+            if (k2) pool_backward_window_kernel<R, false, true><<<out_grid, block, 0, st>>>(g, go, xi, rs, gi);
+            else pool_backward_window_kernel<R, false, false><<<out_grid, block, 0, st>>>(g, go, xi, rs, gi);
+        } else {
+            if (k2) pool_backward_window_kernel<R, true, true><<<out_grid, block, 0, st>>>(g, go, xi, rs, gi);
+            else pool_backward_window_kernel<R, true, false><<<out_grid, block, 0, st>>>(g, go, xi, rs, gi);
+        }
+    } else if (op == POOL_AVG) {
         pool_backward_kernel<R, false><<<in_grid, block, 0, st>>>(g, static_cast<const R *>(gout), static_cast<const R *>(x),
                                                                   static_cast<const R *>(res), static_cast<R *>(gin));
     } else {
