@@ -65,7 +65,9 @@ __device__ __forceinline__ const T *plane_of(const PoolGeom &g, const T *x, uint
     return x + static_cast<int64_t>(b) * g.xs_b + static_cast<int64_t>(c) * g.xs_c;
 }
 
-template <typename T, typename R, int OP>
+// KC: the window size when it is known at compile time (2 or 3), else 0.  With a fixed size the window is unrolled:
+// all of its loads are issued before the first comparison instead of one load per loop iteration.
+template <typename T, typename R, int OP, int KC>
 __global__ void __launch_bounds__(256) pool_forward_kernel(PoolGeom g, const T *__restrict__ x, R *__restrict__ out) {
     uint32_t plane, blk;
     g.d_out_blocks.divmod(blockIdx.x, plane, blk);
@@ -74,17 +76,38 @@ __global__ void __launch_bounds__(256) pool_forward_kernel(PoolGeom g, const T *
     uint32_t h, w;
     g.d_Wo.divmod(pos, h, w);
     const T *src = plane_of(g, x, plane);
-    const R n = static_cast<R>(g.K * g.K);
+    const int K = KC ? KC : g.K;
+    const R n = static_cast<R>(K * K);
     R acc = pool_init<R, OP>();
-    for (int p = 0; p < g.K; ++p) {
-        const int hi = g.S * static_cast<int>(h) + p - g.P;
-        for (int q = 0; q < g.K; ++q) {
-            const int wi = g.S * static_cast<int>(w) + q - g.P;
-            const bool in = !(hi < 0 || wi < 0 || hi >= g.H || wi >= g.W);
-            const R v = in ? static_cast<R>(src[hi * g.xs_h + wi * g.xs_w]) : pool_init<R, OP>();
-            if constexpr (OP == POOL_MAX) acc = (v > acc) ? v : acc;
-            else if constexpr (OP == POOL_MIN) acc = (v < acc) ? v : acc;
-            else acc = (v / n) + acc;
+    auto visit = [&](R v) {
+        if constexpr (OP == POOL_MAX) acc = (v > acc) ? v : acc;
+        else if constexpr (OP == POOL_MIN) acc = (v < acc) ? v : acc;
+        else acc = (v / n) + acc;
+    };
+    const int h0 = g.S * static_cast<int>(h) - g.P, w0 = g.S * static_cast<int>(w) - g.P;
+    if constexpr (KC > 0) {
+        R v[KC * KC];
+#pragma unroll
+        for (int p = 0; p < KC; ++p)
+#pragma unroll
+            for (int q = 0; q < KC; ++q) {
+                const int hi = h0 + p, wi = w0 + q;
+                const bool in = !(hi < 0 || wi < 0 || hi >= g.H || wi >= g.W);
+                // clamped address, so that the load needs no branch; the value is replaced when out of bounds
+                const int hc = hi < 0 ? 0 : (hi >= g.H ? g.H - 1 : hi), wc = wi < 0 ? 0 : (wi >= g.W ? g.W - 1 : wi);
+                const R got = static_cast<R>(src[hc * g.xs_h + wc * g.xs_w]);
+                v[p * KC + q] = in ? got : pool_init<R, OP>();
+            }
+#pragma unroll
+        for (int i = 0; i < KC * KC; ++i) visit(v[i]);
+    } else {
+        for (int p = 0; p < K; ++p) {
+            const int hi = h0 + p;
+            for (int q = 0; q < K; ++q) {
+                const int wi = w0 + q;
+                const bool in = !(hi < 0 || wi < 0 || hi >= g.H || wi >= g.W);
+                visit(in ? static_cast<R>(src[hi * g.xs_h + wi * g.xs_w]) : pool_init<R, OP>());
+            }
         }
     }
     out[static_cast<int64_t>(plane) * (g.Ho * g.Wo) + pos] = acc;
@@ -92,7 +115,7 @@ __global__ void __launch_bounds__(256) pool_forward_kernel(PoolGeom g, const T *
 
 // max / min backward, first pass (one lane per output): share = grad_out / (number of in-bounds window elements
 // equal to the result), the amount each of those elements receives from this output (cpu/kernel/conv.hpp:188-203).
-template <typename R>
+template <typename R, int KC>
 __global__ void __launch_bounds__(256)
 pool_share_kernel(PoolGeom g, const R *__restrict__ gout, const R *__restrict__ x, const R *__restrict__ res, R *__restrict__ share) {
     uint32_t plane, blk;
@@ -104,13 +127,30 @@ pool_share_kernel(PoolGeom g, const R *__restrict__ gout, const R *__restrict__ 
     const R *src = plane_of(g, x, plane);
     const int64_t o = static_cast<int64_t>(plane) * (g.Ho * g.Wo) + pos;
     const R target = res[o];
+    const int h0 = g.S * static_cast<int>(h) - g.P, w0 = g.S * static_cast<int>(w) - g.P;
     R count = R(0);
-    for (int p = 0; p < g.K; ++p)
-        for (int q = 0; q < g.K; ++q) {
-            const int hi = g.S * static_cast<int>(h) + p - g.P, wi = g.S * static_cast<int>(w) + q - g.P;
-            const bool in = !(hi < 0 || wi < 0 || hi >= g.H || wi >= g.W);
-            count += (in && src[hi * g.xs_h + wi * g.xs_w] == target) ? R(1) : R(0);
-        }
+    if constexpr (KC > 0) {  // fixed window: every load issued up front through clamped addresses
+        R v[KC * KC];
+        bool in[KC * KC];
+#pragma unroll
+        for (int p = 0; p < KC; ++p)
+#pragma unroll
+            for (int q = 0; q < KC; ++q) {
+                const int hi = h0 + p, wi = w0 + q;
+                in[p * KC + q] = !(hi < 0 || wi < 0 || hi >= g.H || wi >= g.W);
+                const int hc = hi < 0 ? 0 : (hi >= g.H ? g.H - 1 : hi), wc = wi < 0 ? 0 : (wi >= g.W ? g.W - 1 : wi);
+                v[p * KC + q] = src[hc * g.xs_h + wc * g.xs_w];
+            }
+#pragma unroll
+        for (int i = 0; i < KC * KC; ++i) count += (in[i] && v[i] == target) ? R(1) : R(0);
+    } else {
+        for (int p = 0; p < g.K; ++p)
+            for (int q = 0; q < g.K; ++q) {
+                const int hi = h0 + p, wi = w0 + q;
+                const bool in = !(hi < 0 || wi < 0 || hi >= g.H || wi >= g.W);
+                count += (in && src[hi * g.xs_h + wi * g.xs_w] == target) ? R(1) : R(0);
+            }
+    }
     share[o] = gout[o] / count;
 }
 
@@ -118,7 +158,10 @@ pool_share_kernel(PoolGeom g, const R *__restrict__ gout, const R *__restrict__ 
 // contains the element hands to it.  SELECT: `share` holds the per-output amounts of pool_share_kernel and only
 // outputs whose result equals the element contribute; otherwise `share` is grad_out and every output
 // contributes grad_out / (k*k).
-template <typename R, bool SELECT>
+// NW: compile-time bound on the outputs per axis whose window can contain one element (ceil(k / stride)) when it
+// is 2, else 0 = loop over the run-time range.  With the bound the covering outputs are visited through clamped
+// addresses and predicates, all loads issued up front; an output outside the range adds +0.
+template <typename R, bool SELECT, int NW>
 __global__ void __launch_bounds__(256)
 pool_backward_kernel(PoolGeom g, const R *__restrict__ share, const R *__restrict__ x, const R *__restrict__ res, R *__restrict__ gin) {
     uint32_t plane, blk;
@@ -137,18 +180,37 @@ pool_backward_kernel(PoolGeom g, const R *__restrict__ share, const R *__restric
     h_hi = h_hi >= g.Ho ? g.Ho - 1 : h_hi;
     w_hi = w_hi >= g.Wo ? g.Wo - 1 : w_hi;
     R acc = R(0);
-    if constexpr (SELECT) {
-        const R mine = plane_of(g, x, plane)[static_cast<int64_t>(yh) * g.xs_h + static_cast<int64_t>(xw) * g.xs_w];
-        const R *rplane = res + obase;
+    const R n = static_cast<R>(g.K * g.K);
+    R mine = R(0);
+    const R *rplane = res + obase;
+    if constexpr (SELECT) mine = plane_of(g, x, plane)[static_cast<int64_t>(yh) * g.xs_h + static_cast<int64_t>(xw) * g.xs_w];
+    if constexpr (NW > 0) {
+        R amount[NW * NW], target[NW * NW];
+        bool valid[NW * NW];
+#pragma unroll
+        for (int a = 0; a < NW; ++a)
+#pragma unroll
+            for (int b = 0; b < NW; ++b) {
+                const int h = h_lo + a, w = w_lo + b;
+                valid[a * NW + b] = h <= h_hi && w <= w_hi;
+                const int hc = h > g.Ho - 1 ? g.Ho - 1 : h, wc = w > g.Wo - 1 ? g.Wo - 1 : w;
+                amount[a * NW + b] = splane[hc * g.Wo + wc];
+                if constexpr (SELECT) target[a * NW + b] = rplane[hc * g.Wo + wc];
+            }
+#pragma unroll
+        for (int i = 0; i < NW * NW; ++i) {
+            if constexpr (SELECT) acc += (valid[i] && mine == target[i]) ? amount[i] : R(0);
+            else acc += valid[i] ? amount[i] / n : R(0);
+        }
+    } else if constexpr (SELECT) {
         for (int h = h_lo; h <= h_hi; ++h)
             for (int w = w_lo; w <= w_hi; ++w) {
                 // both loads are issued before the comparison (no dependent second access); an output that does not
                 // select this element adds +0, which leaves the running sum's bits unchanged
-                const R target = rplane[h * g.Wo + w], amount = splane[h * g.Wo + w];
-                acc += (mine == target) ? amount : R(0);
+                const R t = rplane[h * g.Wo + w], amount = splane[h * g.Wo + w];
+                acc += (mine == t) ? amount : R(0);
             }
     } else {
-        const R n = static_cast<R>(g.K * g.K);
         for (int h = h_lo; h <= h_hi; ++h)
             for (int w = w_lo; w <= w_hi; ++w) acc += splane[h * g.Wo + w] / n;
     }
@@ -314,8 +376,12 @@ ttamd_status launch_forward(const PoolGeom &g, const void *x, void *out, hipStre
     const unsigned blocks = static_cast<unsigned>(static_cast<int64_t>(g.B) * g.C * g.out_blocks);
     if (g.K == 2 && g.S == 2 && g.P == 0 && rows_pair_aligned<T>(g, x, x))
         pool_forward_k2_kernel<T, R, OP><<<dim3(blocks), dim3(256), 0, st>>>(g, static_cast<const T *>(x), static_cast<R *>(out));
+    else if (g.K == 3)
+        pool_forward_kernel<T, R, OP, 3><<<dim3(blocks), dim3(256), 0, st>>>(g, static_cast<const T *>(x), static_cast<R *>(out));
+    else if (g.K == 2)
+        pool_forward_kernel<T, R, OP, 2><<<dim3(blocks), dim3(256), 0, st>>>(g, static_cast<const T *>(x), static_cast<R *>(out));
     else
-        pool_forward_kernel<T, R, OP><<<dim3(blocks), dim3(256), 0, st>>>(g, static_cast<const T *>(x), static_cast<R *>(out));
+        pool_forward_kernel<T, R, OP, 0><<<dim3(blocks), dim3(256), 0, st>>>(g, static_cast<const T *>(x), static_cast<R *>(out));
     TTAMD_HIP_CHECK(hipGetLastError());
     return TTAMD_OK;
 }
@@ -344,17 +410,24 @@ ttamd_status backward_typed(int device, int op, const PoolGeom &g, const void *g
             if (k2) pool_backward_window_kernel<R, true, true><<<out_grid, block, 0, st>>>(g, go, xi, rs, gi);
             else pool_backward_window_kernel<R, true, false><<<out_grid, block, 0, st>>>(g, go, xi, rs, gi);
         }
-    } else if (op == POOL_AVG) {
-        pool_backward_kernel<R, false><<<in_grid, block, 0, st>>>(g, static_cast<const R *>(gout), static_cast<const R *>(x),
-                                                                  static_cast<const R *>(res), static_cast<R *>(gin));
     } else {
-        void *share = nullptr;
-        const size_t bytes = static_cast<size_t>(planes) * g.Ho * g.Wo * sizeof(R);
-        if (ttamd_status s = stream_scratch(device, st, bytes ? bytes : sizeof(R), &share)) return s;
-        pool_share_kernel<R><<<out_grid, block, 0, st>>>(g, static_cast<const R *>(gout), static_cast<const R *>(x),
-                                                         static_cast<const R *>(res), static_cast<R *>(share));
-        pool_backward_kernel<R, true><<<in_grid, block, 0, st>>>(g, static_cast<const R *>(share), static_cast<const R *>(x),
-                                                                 static_cast<const R *>(res), static_cast<R *>(gin));
+        const R *go = static_cast<const R *>(gout), *xi = static_cast<const R *>(x), *rs = static_cast<const R *>(res);
+        R *gi = static_cast<R *>(gin);
+        const bool two = (g.K + g.S - 1) / g.S == 2;  // an element lies in at most 2 x 2 windows (k3 s2, k2 s1, k4 s2 ...)
+        if (op == POOL_AVG) {
+            if (two) pool_backward_kernel<R, false, 2><<<in_grid, block, 0, st>>>(g, go, xi, rs, gi);
+            else pool_backward_kernel<R, false, 0><<<in_grid, block, 0, st>>>(g, go, xi, rs, gi);
+        } else {
+            void *ws = nullptr;
+            const size_t bytes = static_cast<size_t>(planes) * g.Ho * g.Wo * sizeof(R);
+            if (ttamd_status s = stream_scratch(device, st, bytes ? bytes : sizeof(R), &ws)) return s;
+            R *share = static_cast<R *>(ws);
+            if (g.K == 3) pool_share_kernel<R, 3><<<out_grid, block, 0, st>>>(g, go, xi, rs, share);
+            else if (g.K == 2) pool_share_kernel<R, 2><<<out_grid, block, 0, st>>>(g, go, xi, rs, share);
+            else pool_share_kernel<R, 0><<<out_grid, block, 0, st>>>(g, go, xi, rs, share);
+            if (two) pool_backward_kernel<R, true, 2><<<in_grid, block, 0, st>>>(g, share, xi, rs, gi);
+            else pool_backward_kernel<R, true, 0><<<in_grid, block, 0, st>>>(g, share, xi, rs, gi);
+        }
     }
     TTAMD_HIP_CHECK(hipGetLastError());
     return TTAMD_OK;
