@@ -68,13 +68,26 @@ __global__ void __launch_bounds__(256) transpose_copy_kernel(const W *__restrict
     }
     const int64_t r0 = static_cast<int64_t>(tr) * 64, c0 = static_cast<int64_t>(tc) * 64;
     const int lane = threadIdx.x % 64, group = threadIdx.x / 64;
+    const W *sp = src + s_off + (r0 + lane) + (c0 + group) * t.src_col_stride;
+    W *dp = dst + d_off + (r0 + group) * t.dst_row_stride + (c0 + lane);
+    if (r0 + 64 <= t.rows && c0 + 64 <= t.cols) {  // interior tile: 16 independent loads per lane, no bounds tests
+        W v[16];
+#pragma unroll
+        for (int i = 0; i < 16; ++i) v[i] = __builtin_nontemporal_load(sp + 4 * i * t.src_col_stride);  // read once
+#pragma unroll
+        for (int i = 0; i < 16; ++i) tile[group + 4 * i][lane] = v[i];
+        __syncthreads();
+#pragma unroll
+        for (int i = 0; i < 16; ++i) dp[4 * i * t.dst_row_stride] = tile[lane][group + 4 * i];
+        return;
+    }
     // read: lanes run along `fast` (unit source stride)
     for (int c = group; c < 64; c += 4)
-        if (r0 + lane < t.rows && c0 + c < t.cols) tile[c][lane] = src[s_off + (r0 + lane) + (c0 + c) * t.src_col_stride];
+        if (r0 + lane < t.rows && c0 + c < t.cols) tile[c][lane] = sp[(c - group) * t.src_col_stride];
     __syncthreads();
     // write: lanes run along the last dimension (unit result stride)
     for (int r = group; r < 64; r += 4)
-        if (r0 + r < t.rows && c0 + lane < t.cols) dst[d_off + (r0 + r) * t.dst_row_stride + (c0 + lane)] = tile[lane][r];
+        if (r0 + r < t.rows && c0 + lane < t.cols) dp[(r - group) * t.dst_row_stride] = tile[lane][r];
 }
 
 template <typename W>
