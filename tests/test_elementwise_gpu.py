@@ -61,6 +61,29 @@ def test_binary_on_strided_and_broadcast_views(tt):
         ta + dev(tt, np.zeros((5,), np.float32))
 
 
+@pytest.mark.parametrize("dtype", [np.float32, np.float64, np.int32, np.uint8])
+@pytest.mark.parametrize("shape", [(1024, 1024), (7, 13), (3,), (257, 5)])
+def test_scalar_operands_take_the_splat_kernels(tt, dtype, shape):
+    # tensor (op) scalar and where(mask, scalar, scalar | tensor): one operand is a single element with every stride 0;
+    # sizes with and without a tail behind the 16-byte vectors
+    rng = np.random.default_rng(sum(shape))
+    a = rng.integers(0, 7, shape).astype(dtype)
+    b = rng.integers(0, 7, shape).astype(dtype)
+    ta, tb = dev(tt, a), dev(tt, b)
+    two = dtype(2)
+    assert np.array_equal((ta + 2).to_numpy(), a + two)
+    assert np.array_equal((ta * 2).to_numpy(), a * two)
+    assert np.array_equal((ta - 2).to_numpy(), (a - two).astype(dtype))
+    assert np.array_equal((ta < 3).to_numpy(), a < 3)
+    mask = ta < 3
+    assert np.array_equal(tt.where(mask, 0, 1).to_numpy(), np.where(a < 3, dtype(0), dtype(1)))
+    assert np.array_equal(tt.where(mask, tb, 5).to_numpy(), np.where(a < 3, b, dtype(5)))
+    assert np.array_equal(tt.where(mask, 5, tb).to_numpy(), np.where(a < 3, dtype(5), b))
+    # scalar on the left of a non-commutative op
+    s = dev(tt, np.full((1,) * len(shape), 9, dtype=dtype)).expand(shape)
+    assert np.array_equal((s - ta).to_numpy(), (dtype(9) - a).astype(dtype))
+
+
 @pytest.mark.parametrize("dtype", [np.float32, np.float64])
 def test_unary_ops(tt, dtype):
     rng = np.random.default_rng(3)

@@ -276,13 +276,18 @@ __device__ __forceinline__ V stream_load(const V *p) {
     return __builtin_nontemporal_load(p);
 }
 
-template <typename T, int OP>
+// SA / SB: the operand is one element broadcast over the shape (every stride 0: `x < 0`, `g * lr`), read once per lane.
+template <typename T, int OP, bool SA = false, bool SB = false>
 __global__ void __launch_bounds__(256) binary_vec_kernel(const T *__restrict__ a, const T *__restrict__ b, void *__restrict__ out, int64_t nvec) {
     constexpr int N = 16 / sizeof(T);
     using R = decltype(binary_apply<T, OP>(T(0), T(0)));
     const int64_t step = static_cast<int64_t>(gridDim.x) * blockDim.x;
+    vec_t<T, N> x, y;
+    if constexpr (SA) x = a[0];
+    if constexpr (SB) y = b[0];
     for (int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < nvec; i += step) {
-        const vec_t<T, N> x = stream_load(reinterpret_cast<const vec_t<T, N> *>(a) + i), y = stream_load(reinterpret_cast<const vec_t<T, N> *>(b) + i);
+        if constexpr (!SA) x = stream_load(reinterpret_cast<const vec_t<T, N> *>(a) + i);
+        if constexpr (!SB) y = stream_load(reinterpret_cast<const vec_t<T, N> *>(b) + i);
         vec_t<R, N> r;
 #pragma unroll
         for (int j = 0; j < N; ++j) r[j] = binary_apply<T, OP>(x[j], y[j]);
@@ -303,14 +308,18 @@ __global__ void __launch_bounds__(256) unary_vec_kernel(const T *__restrict__ a,
     }
 }
 
-template <typename T>
+template <typename T, bool SA = false, bool SB = false>
 __global__ void __launch_bounds__(256) where_vec_kernel(const uint8_t *__restrict__ c, const T *__restrict__ a, const T *__restrict__ b,
                                                        T *__restrict__ out, int64_t nvec) {
     constexpr int N = 16 / sizeof(T);
     const int64_t step = static_cast<int64_t>(gridDim.x) * blockDim.x;
+    vec_t<T, N> x, y;
+    if constexpr (SA) x = a[0];
+    if constexpr (SB) y = b[0];
     for (int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < nvec; i += step) {
         const vec_t<uint8_t, N> m = stream_load(reinterpret_cast<const vec_t<uint8_t, N> *>(c) + i);
-        const vec_t<T, N> x = stream_load(reinterpret_cast<const vec_t<T, N> *>(a) + i), y = stream_load(reinterpret_cast<const vec_t<T, N> *>(b) + i);
+        if constexpr (!SA) x = stream_load(reinterpret_cast<const vec_t<T, N> *>(a) + i);
+        if constexpr (!SB) y = stream_load(reinterpret_cast<const vec_t<T, N> *>(b) + i);
         vec_t<T, N> r;
 #pragma unroll
         for (int j = 0; j < N; ++j) r[j] = m[j] ? x[j] : y[j];
@@ -341,7 +350,15 @@ __global__ void __launch_bounds__(256) sum_dim_kernel(const T *__restrict__ a, V
     if (i >= n_out) return;
     const T *p = a + flat_of(i, outer);
     T acc = T(0);
-    for (int64_t j = 0; j < dim_len; ++j) acc = static_cast<T>(acc + p[j * dim_stride]);
+    int64_t j = 0;
+    for (; j + 8 <= dim_len; j += 8) {  // eight loads in flight, added in index order
+        T v[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) v[u] = p[(j + u) * dim_stride];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) acc = static_cast<T>(acc + v[u]);
+    }
+    for (; j < dim_len; ++j) acc = static_cast<T>(acc + p[j * dim_stride]);
     out[i] = acc;
 }
 
@@ -534,9 +551,41 @@ ttamd_status make_view(const char *who, int ndim, const int64_t *shape, const in
 
 inline bool aligned16(const void *p) { return reinterpret_cast<uintptr_t>(p) % 16 == 0; }
 
+// One element broadcast over the whole shape (more than one element, every extent > 1 has stride 0).
+inline bool is_broadcast_scalar(const ViewDesc &v) {
+    bool any = false;
+    for (int d = 0; d < v.ndim; ++d) {
+        if (v.shape[d] == 1) continue;
+        if (v.stride[d] != 0) return false;
+        any = true;
+    }
+    return any;
+}
+
 template <typename T, int OP>
 ttamd_status launch_binary_op(const void *a, const ViewDesc &va, const void *b, const ViewDesc &vb, void *out, int64_t numel, hipStream_t st) {
-    if (is_dense(va) && is_dense(vb)) {
+    const bool sa = is_broadcast_scalar(va), sb = is_broadcast_scalar(vb);
+    if ((sa != sb) && (sa ? is_dense(vb) : is_dense(va))) {  // tensor (op) scalar: the vector kernel with one operand splat
+        using R = std::conditional_t<(OP >= BIN_LT), uint8_t, T>;
+        constexpr int N = 16 / sizeof(T);
+        const T *pa = static_cast<const T *>(a), *pb = static_cast<const T *>(b);
+        int64_t done = 0;
+        if (aligned16(sa ? b : a) && aligned16(out) && numel >= N) {
+            const int64_t nvec = numel / N;
+            if (sa) binary_vec_kernel<T, OP, true, false><<<dim3(grid_for_vec(nvec)), dim3(256), 0, st>>>(pa, pb, out, nvec);
+            else binary_vec_kernel<T, OP, false, true><<<dim3(grid_for_vec(nvec)), dim3(256), 0, st>>>(pa, pb, out, nvec);
+            done = nvec * N;
+        }
+        if (done < numel) {
+            ViewDesc ta{}, tb{};
+            ta.ndim = tb.ndim = 1;
+            ta.shape[0] = tb.shape[0] = numel - done;
+            ta.stride[0] = sa ? 0 : 1;
+            tb.stride[0] = sb ? 0 : 1;
+            binary_kernel<T, OP, false><<<dim3(grid_for(numel - done)), dim3(256), 0, st>>>(pa + (sa ? 0 : done), ta, pb + (sb ? 0 : done), tb,
+                                                                                        static_cast<R *>(out) + done, numel - done);
+        }
+    } else if (is_dense(va) && is_dense(vb)) {
         using R = std::conditional_t<(OP >= BIN_LT), uint8_t, T>;  // comparisons yield bool bytes
         constexpr int N = 16 / sizeof(T);
         int64_t done = 0;
@@ -906,6 +955,30 @@ ttamd_status ttamd_where(int device, ttamd_dtype dtype, int ndim, const int64_t 
         using T = decltype(tag);
         constexpr int N = 16 / sizeof(T);
         int64_t done = 0;
+        const bool sa = is_broadcast_scalar(va), sb = is_broadcast_scalar(vb);
+        if ((sa || sb) && is_dense(vc) && (sa || is_dense(va)) && (sb || is_dense(vb))) {  // scalar branch values: splat in the vector kernel
+            const T *pa = static_cast<const T *>(a), *pb = static_cast<const T *>(b);
+            if (aligned16(c) && (sa || aligned16(a)) && (sb || aligned16(b)) && aligned16(out) && numel >= N) {
+                const int64_t nvec = numel / N;
+                const dim3 grid(grid_for_vec(nvec)), block(256);
+                if (sa && sb) where_vec_kernel<T, true, true><<<grid, block, 0, st>>>(c, pa, pb, static_cast<T *>(out), nvec);
+                else if (sa) where_vec_kernel<T, true, false><<<grid, block, 0, st>>>(c, pa, pb, static_cast<T *>(out), nvec);
+                else where_vec_kernel<T, false, true><<<grid, block, 0, st>>>(c, pa, pb, static_cast<T *>(out), nvec);
+                done = nvec * N;
+            }
+            if (done < numel) {
+                ViewDesc tc{}, ta{}, tb{};
+                tc.ndim = ta.ndim = tb.ndim = 1;
+                tc.shape[0] = ta.shape[0] = tb.shape[0] = numel - done;
+                tc.stride[0] = 1;
+                ta.stride[0] = sa ? 0 : 1;
+                tb.stride[0] = sb ? 0 : 1;
+                where_kernel<T><<<dim3(grid_for(numel - done)), dim3(256), 0, st>>>(c + done, tc, pa + (sa ? 0 : done), ta, pb + (sb ? 0 : done), tb,
+                                                                                  static_cast<T *>(out) + done, numel - done);
+            }
+            TTAMD_HIP_CHECK(hipGetLastError());
+            return TTAMD_OK;
+        }
         const bool dense = is_dense(vc) && is_dense(va) && is_dense(vb);
         if (dense && aligned16(c) && aligned16(a) && aligned16(b) && aligned16(out) && numel >= N) {
             const int64_t nvec = numel / N;
