@@ -19,10 +19,10 @@ using namespace mfma;
 // ksplit > 1: the reduction is cut into `ksplit` ranges of `k_chunk` (a multiple of BK); workgroup column z =
 // batch * ksplit + split writes the raw partial tile to `partial[z]` and splitk_reduce_kernel finishes the job.
 // PF = tiles kept in flight in registers: 1 for the big tiles (a k tile's MFMA work outlasts a global load there,
-// and registers are scarce), 4 for the fp32 64 x 64 tile, whose 16 MFMAs per k tile (~0.43 us) are shorter than a
+// and registers are scarce), 2 or 4 for the 64 x 64 tile, whose 16 MFMAs per k tile (~0.43 us) are shorter than a
 // load from L2 under traffic: with one tile in flight a lone workgroup on a CU (1024^3 is 256 tiles) waited for
-// memory in every step.  Measured: 1024 x 784 x 1024 26.2 -> 22.1 us, 1024 x 4096 x 1024 87 -> 78 us, 3072^3 127 -> 131
-// TFLOP/s, although the extra 64 registers halve the resident workgroups per CU.
+// memory in every step.  Measured at depth 4: 1024 x 784 x 1024 26.2 -> 22.1 us, 1024 x 4096 x 1024 87 -> 78 us; the
+// host picks the depth per launch (launch_mfma_typed).
 // EPI: which epilogues the kernel carries.  kEpiAny tests the epilogue flags at run time and supports split k (the
 // 64 x 64 tile).  The big tiles are compiled twice, kEpiLean (plain store only) and kEpiFull (bias / ReLU /
 // accumulate), and never split k: with both store walks in one kernel the register allocator spills accumulators
@@ -122,7 +122,7 @@ struct TileShapes<float> {
     static constexpr int XBM = 256, XBN = 128, XBK = 16;  // extra large: 4 waves of 128 x 64 (4 x 2 MFMA blocks)
     static constexpr int LBM = 128, LBN = 128, LBK = 16;  // large: 4 waves of 64 x 64
     static constexpr int SBM = 64, SBN = 64, SBK = 32;    // small: 4 waves of 32 x 32
-    static constexpr int SPF = 4;                          // k tiles in flight in registers (16-byte operands only)
+    static constexpr int SPF = 2, SPF_DEEP = 4;            // k tiles in flight in registers (16-byte operands only)
     static constexpr const char *prefix = "mfma_f32";
 };
 template <>
@@ -132,7 +132,7 @@ struct TileShapes<double> {
     static constexpr int XBM = 256, XBN = 128, XBK = 16;  // 4 waves of 128 x 64 (8 x 4 blocks of 16 x 16), one workgroup per CU
     static constexpr int LBM = 128, LBN = 128, LBK = 16;  // 4 waves of 64 x 64 (4 x 4 blocks of 16 x 16)
     static constexpr int SBM = 64, SBN = 64, SBK = 16;    // 4 waves of 32 x 32
-    static constexpr int SPF = 4;
+    static constexpr int SPF = 2, SPF_DEEP = 4;
     static constexpr const char *prefix = "mfma_f64";
 };
 
@@ -141,9 +141,8 @@ struct SplitPlan {
     int k_chunk = 0;
 };
 
-template <typename T, int BM, int BN, int BK, int WGM, int WGN, bool A_KC, int A_VEC, bool B_KC, int B_VEC>
+template <typename T, int BM, int BN, int BK, int WGM, int WGN, bool A_KC, int A_VEC, bool B_KC, int B_VEC, int PF>
 ttamd_status launch_variant(const GemmArgs &g, const SplitPlan &sp, int device, hipStream_t stream) {
-    constexpr int PF = (BM <= 64 && BN <= 64 && A_VEC > 1 && B_VEC > 1) ? TileShapes<T>::SPF : 1;  // gathers: registers
     using StA = Stager<T, BM, BK, A_KC, A_VEC, PF>;
     using StB = Stager<T, BN, BK, B_KC, B_VEC, PF>;
     constexpr size_t lds_bytes = TileEngine<T, BM, BN, BK, WGM, WGN, StA, StB>::kLdsBytes;
@@ -186,12 +185,12 @@ ttamd_status launch_variant(const GemmArgs &g, const SplitPlan &sp, int device, 
     return TTAMD_OK;
 }
 
-template <typename T, int BM, int BN, int BK, int WGM, int WGN, int A_VEC, int B_VEC>
+template <typename T, int BM, int BN, int BK, int WGM, int WGN, int A_VEC, int B_VEC, int PF = 1>
 ttamd_status launch_layouts(const GemmArgs &g, bool a_kc, bool b_kc, const SplitPlan &sp, int device, hipStream_t stream) {
-    if (a_kc && b_kc) return launch_variant<T, BM, BN, BK, WGM, WGN, true, A_VEC, true, B_VEC>(g, sp, device, stream);
-    if (a_kc && !b_kc) return launch_variant<T, BM, BN, BK, WGM, WGN, true, A_VEC, false, B_VEC>(g, sp, device, stream);
-    if (!a_kc && b_kc) return launch_variant<T, BM, BN, BK, WGM, WGN, false, A_VEC, true, B_VEC>(g, sp, device, stream);
-    return launch_variant<T, BM, BN, BK, WGM, WGN, false, A_VEC, false, B_VEC>(g, sp, device, stream);
+    if (a_kc && b_kc) return launch_variant<T, BM, BN, BK, WGM, WGN, true, A_VEC, true, B_VEC, PF>(g, sp, device, stream);
+    if (a_kc && !b_kc) return launch_variant<T, BM, BN, BK, WGM, WGN, true, A_VEC, false, B_VEC, PF>(g, sp, device, stream);
+    if (!a_kc && b_kc) return launch_variant<T, BM, BN, BK, WGM, WGN, false, A_VEC, true, B_VEC, PF>(g, sp, device, stream);
+    return launch_variant<T, BM, BN, BK, WGM, WGN, false, A_VEC, false, B_VEC, PF>(g, sp, device, stream);
 }
 
 // Split the reduction when the output has too few tiles to fill 256 CUs and K is long enough to share out.
@@ -281,7 +280,16 @@ ttamd_status launch_mfma_typed(const GemmArgs &g, int device, hipStream_t stream
         if (xl) return launch_layouts<T, TS::XBM, TS::XBN, TS::XBK, 2, 2, VK, VK>(g, ca.kc, cb.kc, sp, device, stream);
     }
     if (large) return launch_layouts<T, TS::LBM, TS::LBN, TS::LBK, 2, 2, VK, VK>(g, ca.kc, cb.kc, sp, device, stream);
-    if (ca.vec > 1 && cb.vec > 1) return launch_layouts<T, TS::SBM, TS::SBN, TS::SBK, 2, 2, VK, VK>(g, ca.kc, cb.kc, sp, device, stream);
+    if (ca.vec > 1 && cb.vec > 1) {
+        // Register prefetch depth of the small tile: 4 k tiles in flight when a CU holds at most two workgroups and the
+        // reduction is long (a lone workgroup otherwise waits for memory in every step), else 2, whose smaller register
+        // footprint keeps more workgroups resident (832 tiles with K = 288: 26.5 us against 31.2 us at depth 4).
+        const int64_t wgs = static_cast<int64_t>((g.M + TS::SBM - 1) / TS::SBM) * ((g.N + TS::SBN - 1) / TS::SBN) * g.batch * sp.ksplit;
+        const int k_tiles = ((sp.ksplit > 1 ? sp.k_chunk : g.K) + TS::SBK - 1) / TS::SBK;
+        if (k_tiles >= 16 && wgs <= 512)
+            return launch_layouts<T, TS::SBM, TS::SBN, TS::SBK, 2, 2, VK, VK, TS::SPF_DEEP>(g, ca.kc, cb.kc, sp, device, stream);
+        return launch_layouts<T, TS::SBM, TS::SBN, TS::SBK, 2, 2, VK, VK, TS::SPF>(g, ca.kc, cb.kc, sp, device, stream);
+    }
     if (ca.vec > 1) return launch_layouts<T, TS::SBM, TS::SBN, TS::SBK, 2, 2, VK, 1>(g, ca.kc, cb.kc, sp, device, stream);
     if (cb.vec > 1) return launch_layouts<T, TS::SBM, TS::SBN, TS::SBK, 2, 2, 1, VK>(g, ca.kc, cb.kc, sp, device, stream);
     return launch_layouts<T, TS::SBM, TS::SBN, TS::SBK, 2, 2, 1, 1>(g, ca.kc, cb.kc, sp, device, stream);
