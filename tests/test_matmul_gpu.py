@@ -318,6 +318,24 @@ def test_big_tile_epilogues_and_edges(tt, dtype, N, M, layout, tile):
     assert np.array_equal(acc.to_numpy()[0], want + row_bias[:, None] + prev[0])
 
 
+# Long reductions on few 64 x 64 tiles run with four k tiles in flight (static register slots per group of steps),
+# short or crowded ones with two: both depths, all layouts, k tails and exact multiples, both dtypes.  Small integers
+# keep the sums exact.
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+@pytest.mark.parametrize("layout", LAYOUTS)
+@pytest.mark.parametrize("shape", [(320, 1024, 448), (200, 1000, 260), (64, 4100, 64), (704, 520, 1344), (448, 48, 320)])
+def test_small_tile_prefetch_depths(tt, dtype, layout, shape):
+    N, K, M = shape
+    rng = np.random.default_rng(N + K + M)
+    ints = lambda *sh: rng.integers(-3, 4, sh).astype(dtype)
+    A = ints(2, N, K) if layout[0] == "n" else ints(2, K, N).transpose(0, 2, 1)
+    B = ints(2, K, M) if layout[1] == "n" else ints(2, M, K).transpose(0, 2, 1)
+    tA, tB = to_dev_view(tt, A), to_dev_view(tt, B)
+    assert "_64x64_" in tt.get_backend(tt.kAMD).batched_matmul_variant(tA, tB)
+    got = tt.matmul(tA, tB).to_numpy()
+    assert np.array_equal(got, np.matmul(A.astype(np.float64), B.astype(np.float64)))
+
+
 def test_contiguous_identity(tt, oracle):
     rng = np.random.default_rng(2)
     for dtype in (np.uint8, np.int16, np.float32, np.float64):
