@@ -342,11 +342,10 @@ struct TileEngine {
     static constexpr size_t kLdsBytes = 2 * (StA::LDS_ELEMS + StB::LDS_ELEMS) * sizeof(T);
 
     typename M::acc_t acc[NBM][NBN];
-    // Three schedules of the main loop, chosen by the number of MFMA blocks a wave owns:
-    //  * pipelined (fp32, two chunks per k tile, 4 to 16 blocks: 128 x 128, 256 x 128 and 256 x 256) - see step_pipe();
-    //  * rotated (<= 4 blocks otherwise: 64 x 64 tiles, conv tiles) - see step_rot();
-    //  * plain (fp64 128 x 128: 16 blocks of 16 x 16, 128 accumulator registers leave no room for a second set of
-    //    fragments) - see step_plain().
+    // Two schedules of the main loop, chosen by the number of MFMA blocks a wave owns:
+    //  * pipelined (two chunks per k tile and at least 4 fp32 / 16 fp64 blocks: 128 x 128, 256 x 128, 256 x 256) - see
+    //    step_pipe();
+    //  * rotated (at most 4 blocks: 64 x 64 tiles, conv tiles) - see step_rot().
     static constexpr bool kPipe = BK / kChunk == 2 && NBM * NBN >= (sizeof(T) == 4 ? 4 : 16);
     static constexpr bool kRotate = !kPipe && NBM * NBN <= 4;
     FrA last_a;  // fragments of the previous tile's last chunk, multiplied after the barrier
@@ -631,123 +630,12 @@ struct TileEngine {
         }
     }
 
-    // ---- plain schedule (fp64 tiles with 16 MFMA blocks per wave) ----
-    // MFMA work of chunks [c0, c1) of the tile in LDS buffer `buf`.
-    __device__ __forceinline__ void compute_chunks_plain(const T *smem, int buf, int c0, int c1) {
-        const T *la = smem + buf * StA::LDS_ELEMS;
-        const T *lb = smem + kBOff + buf * StB::LDS_ELEMS;
-#pragma unroll
-        for (int c = c0; c < c1; ++c) {
-            FrA fa;
-            FrB fb;
-            fa.read(la, wm0, c, lane);
-            fb.read(lb, wn0, c, lane);
-#pragma unroll
-            for (int j = 0; j < M::VK; ++j)
-#pragma unroll
-                for (int bm = 0; bm < NBM; ++bm)
-#pragma unroll
-                    for (int bn = 0; bn < NBN; ++bn) acc[bm][bn] = M::mma(fa.v[bm][j], fb.v[bn][j], acc[bm][bn]);
-        }
-    }
-    __device__ __forceinline__ void compute_plain(const T *smem, int buf) { compute_chunks_plain(smem, buf, 0, BK / kChunk); }
-
-    // One pipeline step for tile kt, whose register slot arithmetic is static: tile t lives in slot t % PF.
-    //   LOAD: issue the global loads of tile kt + PF into slot kt % PF (free: tile kt is already in LDS);
-    //   multiply tile kt out of LDS buffer kt & 1; park tile kt + 1 (slot (kt + 1) % PF, loaded PF - 1 steps
-    //   ago) in the other LDS buffer, its stores slotted between the MFMAs of the last chunk.
-    template <int S, bool LOAD, bool MASK>
-    __device__ __forceinline__ void step_plain(StA &sa, StB &sb, T *smem, int K, int kt) {
-        constexpr int PF = StA::kPF;
-        constexpr int NC = BK / kChunk;
-        constexpr int kLastMfmas = M::VK * NBM * NBN;  // MFMAs of one chunk
-        constexpr int kStores = StA::P + StB::P;       // LDS store instructions of one tile (per lane)
-        const int cur = kt & 1;
-        if constexpr (LOAD) {
-            const int k_left = K - (kt + PF) * BK;
-            sa.template load<MASK, S>(k_left);
-            sb.template load<MASK, S>(k_left);
-        }
-        // Keep the global loads ahead of the MFMA work: left alone, the scheduler sinks them to just before
-        // the LDS stores and their latency is exposed on every tile.
-        __builtin_amdgcn_sched_barrier(0);
-        // Raised wave priority while this wave multiplies: the SIMD's other wave, busy with address arithmetic and
-        // loads, then cannot delay the MFMA issue (fp64 128 x 128: +3 %; no gain on the fp32 256 x 128 tile, whose
-        // code is left as it was).
-        if constexpr (sizeof(T) == 8) __builtin_amdgcn_s_setprio(3);
-        compute_chunks_plain(smem, cur, 0, NC - 1);
-        __builtin_amdgcn_sched_barrier(0);
-        // Last chunk: its MFMAs run with the LDS stores of the next tile slotted between them.  The other
-        // buffer was last read before the previous barrier, so it may be written as soon as the global data
-        // has arrived; by the time the last MFMA issues the stores have drained and the barrier costs no
-        // pipe time (stores placed after the MFMAs cost ~9 % at 4096^3).
-        compute_chunks_plain(smem, cur, NC - 1, NC);
-        sa.template store<(S + 1) % PF>(smem + (cur ^ 1) * StA::LDS_ELEMS);
-        sb.template store<(S + 1) % PF>(smem + kBOff + (cur ^ 1) * StB::LDS_ELEMS);
-        if constexpr (kLastMfmas >= 2 * kStores) {
-#pragma unroll
-            for (int i = 0; i < kStores; ++i) {
-                __builtin_amdgcn_sched_group_barrier(0x008, kLastMfmas / kStores > 2 ? 2 : 1, 0);  // MFMA
-                __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);                                 // DS write
-            }
-        }
-        __builtin_amdgcn_sched_barrier(0);
-        if constexpr (sizeof(T) == 8) __builtin_amdgcn_s_setprio(0);
-        __syncthreads();
-    }
-
-    template <bool LOAD, bool MASK, int S = 0>
-    __device__ __forceinline__ void step_any_plain(StA &sa, StB &sb, T *smem, int K, int kt, int slot) {
-        if constexpr (S < StA::kPF) {
-            if (slot == S) step_plain<S, LOAD, MASK>(sa, sb, smem, K, kt);
-            else step_any_plain<LOAD, MASK, S + 1>(sa, sb, smem, K, kt, slot);
-        }
-    }
-
-    // K: reduction length.  `unmasked`: workgroup-uniform promise that every tile is full and interior.
-    __device__ __forceinline__ void run_plain(StA &sa, StB &sb, T *smem, int K, bool unmasked) {
-        constexpr int PF = StA::kPF;
-        static_assert(StA::kPF == StB::kPF, "both operands use the same prefetch distance");
-        const int KT = (K + BK - 1) / BK;
-        // Prologue: tile 0 goes straight to LDS, tiles 1 .. PF-1 are put in flight.
-        sa.template load<true, 0>(K);
-        sb.template load<true, 0>(K);
-        sa.template store<0>(smem);
-        sb.template store<0>(smem + kBOff);
-        prefetch_rest<1>(sa, sb, K, KT);
-        __syncthreads();
-        // Tiles 0 .. KT-2 (the last tile is multiplied after the loop).  While kt + PF < KT every step also
-        // issues loads; the remaining steps only drain the slots.
-        auto pipeline = [&]<bool MASK>() {
-            int kt = 0;
-            if constexpr (PF == 1) {
-                for (; kt + 1 < KT; ++kt) step_plain<0, true, MASK>(sa, sb, smem, K, kt);
-            } else {
-                int slot = 0;
-                for (; kt + PF < KT; ++kt) {
-                    step_any_plain<true, MASK>(sa, sb, smem, K, kt, slot);
-                    slot = slot + 1 == PF ? 0 : slot + 1;
-                }
-                for (; kt + 1 < KT; ++kt) {
-                    step_any_plain<false, MASK>(sa, sb, smem, K, kt, slot);
-                    slot = slot + 1 == PF ? 0 : slot + 1;
-                }
-            }
-        };
-        if (unmasked) {
-            pipeline.template operator()<false>();
-        } else {
-            pipeline.template operator()<true>();
-        }
-        if (KT > 0) compute_plain(smem, (KT - 1) & 1);
-    }
-
     // K: reduction length.  `unmasked`: workgroup-uniform promise that every tile is full and interior.
     __device__ __forceinline__ void run(StA &sa, StB &sb, T *smem, int K, bool unmasked) {
         static_assert(StA::kPF == StB::kPF, "both operands use the same prefetch distance");
+        static_assert(kPipe || kRotate, "no schedule for this tile shape");
         if constexpr (kPipe) run_pipe(sa, sb, smem, K, unmasked);
-        else if constexpr (kRotate) run_rot(sa, sb, smem, K, unmasked);
-        else run_plain(sa, sb, smem, K, unmasked);
+        else run_rot(sa, sb, smem, K, unmasked);
     }
 
     template <int S>
