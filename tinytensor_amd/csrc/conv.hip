@@ -799,12 +799,26 @@ BackwardWorkspace backward_workspace(size_t esz, int B, int C, int H, int W, int
     const int64_t K = static_cast<int64_t>(Ho) * Wo;
     const int64_t k_tiles = (K + bk - 1) / bk;
     const int64_t tiles = static_cast<int64_t>((O + 63) / 64) * ((static_cast<int64_t>(C) * k * k + 63) / 64);
-    int64_t want = 768 / (tiles * w.splits);                      // slices that bring the launch to ~3 workgroups per CU
-    if (want > k_tiles / 4) want = k_tiles / 4;                    // at least 4 k tiles per slice
-    const int64_t room = (64LL << 20) / static_cast<int64_t>(tile ? tile : 1) / w.splits;  // partial tiles <= 64 MiB
-    if (want > room) want = room;
-    if (want < 1) want = 1;
-    const int64_t chunk_tiles = (k_tiles + want - 1) / want;
+    // Slices of the reduction: the launch is as slow as its busiest CU, which runs ceil(workgroups / 256) of them,
+    // each through its k tiles plus about three tiles' worth of prologue and epilogue; every part adds one tile to
+    // the sum that follows.  Costs in microseconds: ~0.6 per k tile of a 64 x 64 workgroup that shares its CU,
+    // ~4 MB per microsecond for the partial tiles.  At least 4 k tiles per slice, partial tiles <= 64 MiB.
+    int64_t max_slices = k_tiles / 4;
+    const int64_t room = (64LL << 20) / static_cast<int64_t>(tile ? tile : 1) / w.splits;
+    if (max_slices > room) max_slices = room;
+    if (max_slices < 1) max_slices = 1;
+    int64_t chunk_tiles = k_tiles > 0 ? k_tiles : 1;
+    double best = 0;
+    for (int64_t want = 1; want <= max_slices; ++want) {
+        const int64_t chunk = (k_tiles + want - 1) / want, slices = (k_tiles + chunk - 1) / chunk;
+        const int64_t parts = slices * w.splits, wgs = tiles * parts;
+        const double cost = static_cast<double>((wgs + 255) / 256) * static_cast<double>(chunk + 3) * 0.6 +
+                            (parts > 1 ? static_cast<double>(parts) * static_cast<double>(tile) / 4e6 : 0.0);
+        if (want == 1 || cost < best) {
+            best = cost;
+            chunk_tiles = chunk;
+        }
+    }
     w.k_chunk = static_cast<int>(chunk_tiles * bk);
     w.kslices = static_cast<int>((k_tiles + chunk_tiles - 1) / chunk_tiles);
     if (w.kslices < 1) w.kslices = 1;
