@@ -296,6 +296,8 @@ def main():
     ap.add_argument("--detail", metavar="FILE", help="also time every benchmark configuration and write a JSON report")
     ap.add_argument("--conv-loop", type=int, metavar="N", default=0,
                     help="only run N conv2d forward + backward passes of benchmark configuration 4 (input [64,32,28,28], weight [64,32,3,3], s1 p1) (a short target for profilers) and exit")
+    ap.add_argument("--conv-shape", metavar="B,C,O,H,W", default="64,32,64,28,28",
+                    help="geometry for --conv-loop (3x3 kernel, stride 1, padding 1); the default is benchmark configuration 4")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
@@ -314,8 +316,9 @@ def main():
     if args.conv_loop:
         be = tt.get_backend(tt.kAMD)
         rng = np.random.default_rng(0)
-        x = tt.Tensor.from_numpy(rng.normal(0, 0.1, (64, 32, 28, 28)).astype(np.float32))
-        w = tt.Tensor.from_numpy(rng.normal(0, 0.1, (64, 32, 3, 3)).astype(np.float32))
+        cb, cc, co, ch, cw = (int(v) for v in args.conv_shape.split(","))
+        x = tt.Tensor.from_numpy(rng.normal(0, 0.1, (cb, cc, ch, cw)).astype(np.float32))
+        w = tt.Tensor.from_numpy(rng.normal(0, 0.1, (co, cc, 3, 3)).astype(np.float32))
         out = be.conv2d(x, w, None, 1, 1)
         go = tt.Tensor.from_numpy(np.ones(out.shape, np.float32))
         be.conv2d_backward(go, x, w, None, 1, 1)
@@ -324,7 +327,7 @@ def main():
             be.conv2d(x, w, None, 1, 1, out=out)
             be.conv2d_backward(go, x, w, None, 1, 1, buffers=bufs)
         be.synchronize(0)
-        print(json.dumps({"conv_loop": args.conv_loop, "config": "configs[3]: input [64,32,28,28], weight [64,32,3,3], s1 p1, f32"}))
+        print(json.dumps({"conv_loop": args.conv_loop, "config": f"input [{cb},{cc},{ch},{cw}], weight [{co},{cc},3,3], s1 p1, f32"}))
         return
 
     if args.detail:
