@@ -40,7 +40,13 @@ def test_reference_shape_forward_backward_exact(tt, oracle, op, dtype):
 @pytest.mark.parametrize("dtype", ALL_NON_BOOL)
 @pytest.mark.parametrize("geom", [(2, 3, 9, 8, 2, 2, 0), (1, 2, 7, 7, 3, 1, 1), (2, 2, 6, 9, 3, 3, 2), (1, 1, 5, 5, 5, 1, 2), (3, 1, 1, 1, 1, 1, 0),
                                   # non-overlapping windows: odd width (no pair accesses), rows / columns no window reaches
-                                  (2, 3, 9, 7, 2, 2, 0), (1, 2, 10, 11, 3, 3, 0), (2, 2, 8, 8, 4, 4, 0), (1, 3, 64, 66, 2, 2, 0)])
+                                  (2, 3, 9, 7, 2, 2, 0), (1, 2, 10, 11, 3, 3, 0), (2, 2, 8, 8, 4, 4, 0), (1, 3, 64, 66, 2, 2, 0),
+                                  # overlapping windows on rows of 4n elements (four elements per lane in backward): three,
+                                  # four and five covering output columns, a single group per row, padding wider than 1
+                                  (2, 3, 9, 8, 3, 2, 1), (1, 2, 7, 12, 2, 1, 0), (2, 2, 10, 16, 4, 2, 1), (1, 2, 6, 8, 2, 1, 1),
+                                  (1, 1, 5, 4, 3, 2, 0), (2, 1, 11, 20, 6, 3, 2), (1, 2, 9, 24, 5, 4, 2),
+                                  # rows longer than a wave's 64 groups of four, and rows that end inside a wave
+                                  (1, 2, 9, 520, 3, 2, 1), (2, 1, 7, 44, 3, 2, 1), (1, 1, 6, 256, 3, 2, 1), (1, 2, 5, 260, 2, 1, 0)])
 def test_every_dtype_and_geometry_exact(tt, oracle, op, dtype, geom):
     Bn, Cc, H, W, k, S, P = geom
     rng = np.random.default_rng(sum(geom))

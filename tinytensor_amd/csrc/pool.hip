@@ -4,7 +4,7 @@
 // (tinytensor/tensor/backend_base.h:286-311; CPU form tinytensor/tensor/backend/cpu/conv.cpp:296-426 over the
 // kernels of tinytensor/tensor/backend/cpu/kernel/conv.hpp:121-275, functors
 // tinytensor/tensor/backend/common/kernel/reduce.hpp:28-140).  Both directions are bandwidth-bound streaming
-// kernels: one lane per output element forward, one lane per input element backward.
+// kernels: one lane per output element forward, one lane per input element (or four) backward.
 //
 // Forward visits the window in the reference's (p, q) order with the reference's arithmetic
 //   max: out = (x > out) ? x : out from lowest();  min: out = (x < out) ? x : out from max();
@@ -17,6 +17,8 @@
 // For max / min a first pass over the outputs computes each output's share (gradient / number of window elements
 // equal to the result) into the library's per-stream scratch, so the gather reads two values per covering output
 // instead of recounting its window.
+// On dense rows of 4n elements with at most 2 x 2 covering windows a lane owns four consecutive elements: it loads
+// the block of covering outputs once and moves the input and the gradient as 16-byte vectors.
 //
 // Non-overlapping windows without padding (stride == k, padding == 0: the max_pool2d(x, 2, 2, 0) of
 // examples/mnist_cnn_example.cpp:55) take a shorter road: an input element lies in at most one window, so backward
@@ -40,7 +42,8 @@ struct PoolGeom {
     // Work is laid out as (plane = b*C + c, block of 256 positions inside the plane) so that every index fits 32
     // bits and is split with exact multiply-shift division instead of 64-bit division.
     int out_blocks, in_blocks;        // blocks of 256 positions per output / input plane
-    FastDiv d_out_blocks, d_in_blocks, d_C, d_Wo, d_W, d_S;
+    int quad_blocks;                  // blocks of 256 groups of four positions per input plane
+    FastDiv d_out_blocks, d_in_blocks, d_quad_blocks, d_C, d_Wo, d_W, d_S;
 };
 
 template <typename R, int OP>
@@ -218,6 +221,74 @@ pool_backward_kernel(PoolGeom g, const R *__restrict__ share, const R *__restric
 }
 
 template <typename T>
+using Quad = T __attribute__((ext_vector_type(4)));
+
+// The same gather for four consecutive elements of one input row per lane (W % 4 == 0, dense aligned rows, an
+// element in at most 2 x 2 windows).  The outputs that cover the four elements form a block of 2 rows x NC columns
+// (NC >= ceil((k + 3) / stride)); their amounts and results are loaded once instead of once per element, the input
+// and the gradient move as one vector each, and every element still adds its own covering outputs in increasing
+// (h, w), so the sums are the ones pool_backward_kernel produces.
+template <typename R, bool SELECT, int NC>
+__global__ void __launch_bounds__(256)
+pool_backward_quad_kernel(PoolGeom g, const R *__restrict__ share, const R *__restrict__ x, const R *__restrict__ res, R *__restrict__ gin) {
+    uint32_t plane, blk;
+    g.d_quad_blocks.divmod(blockIdx.x, plane, blk);
+    const uint32_t pos = (blk * 256 + threadIdx.x) * 4;
+    if (pos >= static_cast<uint32_t>(g.H * g.W)) return;
+    uint32_t yh, xw;
+    g.d_W.divmod(pos, yh, xw);
+    const int64_t obase = static_cast<int64_t>(plane) * (g.Ho * g.Wo);
+    const R *splane = share + obase, *rplane = res + obase;
+    const int ay = static_cast<int>(yh) + g.P, ax0 = static_cast<int>(xw) + g.P;
+    const int h_lo = ay - g.K >= 0 ? static_cast<int>(g.d_S.div(static_cast<uint32_t>(ay - g.K))) + 1 : 0;
+    int h_hi = static_cast<int>(g.d_S.div(static_cast<uint32_t>(ay)));
+    h_hi = h_hi >= g.Ho ? g.Ho - 1 : h_hi;
+    int w_lo[4], w_hi[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const int ax = ax0 + j;
+        w_lo[j] = ax - g.K >= 0 ? static_cast<int>(g.d_S.div(static_cast<uint32_t>(ax - g.K))) + 1 : 0;
+        const int hi = static_cast<int>(g.d_S.div(static_cast<uint32_t>(ax)));
+        w_hi[j] = hi >= g.Wo ? g.Wo - 1 : hi;
+    }
+    const int c_lo = w_lo[0];
+    R amount[2 * NC], target[2 * NC];
+#pragma unroll
+    for (int a = 0; a < 2; ++a)
+#pragma unroll
+        for (int b = 0; b < NC; ++b) {
+            const int h = h_lo + a, w = c_lo + b;
+            const int hc = h > g.Ho - 1 ? g.Ho - 1 : h, wc = w > g.Wo - 1 ? g.Wo - 1 : w;
+            amount[a * NC + b] = splane[hc * g.Wo + wc];
+            if constexpr (SELECT) target[a * NC + b] = rplane[hc * g.Wo + wc];
+        }
+    Quad<R> mine = {R(0), R(0), R(0), R(0)};
+    if constexpr (SELECT)
+        mine = *reinterpret_cast<const Quad<R> *>(plane_of(g, x, plane) + static_cast<int64_t>(yh) * g.xs_h + xw);
+    if constexpr (!SELECT) {  // every covered element receives grad_out / k^2: divide once per output
+        const R n = static_cast<R>(g.K * g.K);
+#pragma unroll
+        for (int i = 0; i < 2 * NC; ++i) amount[i] = amount[i] / n;
+    }
+    Quad<R> acc;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        R sum = R(0);
+#pragma unroll
+        for (int a = 0; a < 2; ++a)
+#pragma unroll
+            for (int b = 0; b < NC; ++b) {
+                const int w = c_lo + b;
+                const bool valid = (h_lo + a <= h_hi) & (w >= w_lo[j]) & (w <= w_hi[j]);
+                if constexpr (SELECT) sum += (valid && mine[j] == target[a * NC + b]) ? amount[a * NC + b] : R(0);
+                else sum += valid ? amount[a * NC + b] : R(0);
+            }
+        acc[j] = sum;
+    }
+    *reinterpret_cast<Quad<R> *>(gin + static_cast<int64_t>(plane) * (g.H * g.W) + pos) = acc;
+}
+
+template <typename T>
 using Pair = T __attribute__((ext_vector_type(2)));
 
 // Forward for k == 2, stride == 2, padding == 0 on rows that can be read as aligned pairs (the host checks).
@@ -324,6 +395,16 @@ bool rows_pair_aligned(const PoolGeom &g, const void *x, const void *dense) {
            reinterpret_cast<uintptr_t>(x) % (2 * sizeof(T)) == 0 && reinterpret_cast<uintptr_t>(dense) % (2 * sizeof(T)) == 0;
 }
 
+// Rows of the input view (when it is read: x != nullptr) and of the dense gradient can be moved as aligned groups of
+// four T.
+template <typename T>
+bool rows_quad_aligned(const PoolGeom &g, const void *x, const void *dense) {
+    const auto by4 = [](int64_t v) { return v % 4 == 0; };
+    if (g.W % 4 != 0 || reinterpret_cast<uintptr_t>(dense) % (4 * sizeof(T)) != 0) return false;
+    if (!x) return true;
+    return g.xs_w == 1 && by4(g.xs_h) && by4(g.xs_c) && by4(g.xs_b) && reinterpret_cast<uintptr_t>(x) % (4 * sizeof(T)) == 0;
+}
+
 ttamd_status make_pool_geom(const char *who, int op, const ttamd_view4 *input, int B, int C, int H, int W, int k, int stride,
                             int padding, PoolGeom *g) {
     if (op < POOL_MAX || op > POOL_AVG) {
@@ -363,6 +444,8 @@ ttamd_status make_pool_geom(const char *who, int op, const ttamd_view4 *input, i
     g->in_blocks = static_cast<int>(in_blocks);
     g->out_blocks = static_cast<int>(out_blocks > 0 ? out_blocks : 1);
     g->d_in_blocks = make_fastdiv(static_cast<uint32_t>(g->in_blocks));
+    g->quad_blocks = static_cast<int>((in_plane / 4 + 255) / 256);
+    g->d_quad_blocks = make_fastdiv(static_cast<uint32_t>(g->quad_blocks > 0 ? g->quad_blocks : 1));
     g->d_out_blocks = make_fastdiv(static_cast<uint32_t>(g->out_blocks));
     g->d_C = make_fastdiv(static_cast<uint32_t>(C));
     g->d_Wo = make_fastdiv(static_cast<uint32_t>(g->Wo > 0 ? g->Wo : 1));
@@ -414,8 +497,13 @@ ttamd_status backward_typed(int device, int op, const PoolGeom &g, const void *g
         const R *go = static_cast<const R *>(gout), *xi = static_cast<const R *>(x), *rs = static_cast<const R *>(res);
         R *gi = static_cast<R *>(gin);
         const bool two = (g.K + g.S - 1) / g.S == 2;  // an element lies in at most 2 x 2 windows (k3 s2, k2 s1, k4 s2 ...)
+        const int cols = (g.K + 3 + g.S - 1) / g.S;   // output columns that can cover four consecutive elements
+        const bool quad = two && cols <= 5 && rows_quad_aligned<R>(g, op == POOL_AVG ? nullptr : x, gin);
+        const dim3 quad_grid(static_cast<unsigned>(planes * g.quad_blocks));
         if (op == POOL_AVG) {
-            if (two) pool_backward_kernel<R, false, 2><<<in_grid, block, 0, st>>>(g, go, xi, rs, gi);
+            if (quad && cols <= 3) pool_backward_quad_kernel<R, false, 3><<<quad_grid, block, 0, st>>>(g, go, xi, rs, gi);
+            else if (quad) pool_backward_quad_kernel<R, false, 5><<<quad_grid, block, 0, st>>>(g, go, xi, rs, gi);
+            else if (two) pool_backward_kernel<R, false, 2><<<in_grid, block, 0, st>>>(g, go, xi, rs, gi);
             else pool_backward_kernel<R, false, 0><<<in_grid, block, 0, st>>>(g, go, xi, rs, gi);
         } else {
             void *ws = nullptr;
@@ -425,7 +513,9 @@ ttamd_status backward_typed(int device, int op, const PoolGeom &g, const void *g
             if (g.K == 3) pool_share_kernel<R, 3><<<out_grid, block, 0, st>>>(g, go, xi, rs, share);
             else if (g.K == 2) pool_share_kernel<R, 2><<<out_grid, block, 0, st>>>(g, go, xi, rs, share);
             else pool_share_kernel<R, 0><<<out_grid, block, 0, st>>>(g, go, xi, rs, share);
-            if (two) pool_backward_kernel<R, true, 2><<<in_grid, block, 0, st>>>(g, share, xi, rs, gi);
+            if (quad && cols <= 3) pool_backward_quad_kernel<R, true, 3><<<quad_grid, block, 0, st>>>(g, share, xi, rs, gi);
+            else if (quad) pool_backward_quad_kernel<R, true, 5><<<quad_grid, block, 0, st>>>(g, share, xi, rs, gi);
+            else if (two) pool_backward_kernel<R, true, 2><<<in_grid, block, 0, st>>>(g, share, xi, rs, gi);
             else pool_backward_kernel<R, true, 0><<<in_grid, block, 0, st>>>(g, share, xi, rs, gi);
         }
     }
