@@ -228,13 +228,13 @@ def detail_report(tt, np, path, cpu=True):
         for op in ("max", "avg"):
             code = cap.POOL[op]
             nonoverlap = S_ == k and P_ == 0
-            fwd_kernel = "pool_forward_k2_kernel" if (nonoverlap and k == 2) else "pool_forward_kernel"
+            fwd_kernel = "pool_forward_k2_kernel" if (nonoverlap and k == 2) else "pool_forward_k3s2_kernel"
             stream_case(f"{op}_pool2d forward k{k} s{S_} p{P_} [64,64,112,112] f32", fwd_kernel, in_b + out_b,
                         lambda: lib.ttamd_pool2d_forward(0, cap.F32, code, C.byref(iv), ptr(Pout), Pb, Pc, Ph, Pw, k, S_, P_, None), 30)
             if nonoverlap:
                 bwd_kernel = "pool_backward_window_kernel"
             else:
-                bwd_kernel = "pool_backward_quad_kernel" if op == "avg" else "pool_share_kernel + pool_backward_quad_kernel"
+                bwd_kernel = "pool_backward_quad_kernel" if op == "avg" else "pool_share_k3s2_kernel + pool_backward_quad_kernel"
             # algorithmic bytes of backward: grad_out and grad_input, plus the input and the result for max / min
             bwd_b = (in_b + out_b) if op == "avg" else (2 * in_b + 2 * out_b)
             stream_case(f"{op}_pool2d backward k{k} s{S_} p{P_} [64,64,112,112] f32", bwd_kernel, bwd_b,

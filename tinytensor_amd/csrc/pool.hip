@@ -43,7 +43,8 @@ struct PoolGeom {
     // bits and is split with exact multiply-shift division instead of 64-bit division.
     int out_blocks, in_blocks;        // blocks of 256 positions per output / input plane
     int quad_blocks;                  // blocks of 256 groups of four positions per input plane
-    FastDiv d_out_blocks, d_in_blocks, d_quad_blocks, d_C, d_Wo, d_W, d_S;
+    int opair_blocks;                 // blocks of 256 pairs of positions per output plane
+    FastDiv d_out_blocks, d_in_blocks, d_quad_blocks, d_opair_blocks, d_C, d_Wo, d_W, d_S;
 };
 
 template <typename R, int OP>
@@ -314,6 +315,102 @@ __global__ void __launch_bounds__(256) pool_forward_k2_kernel(PoolGeom g, const 
     out[static_cast<int64_t>(plane) * (g.Ho * g.Wo) + pos] = acc;
 }
 
+// Forward for k == 3, stride == 2, padding == 1 on dense rows of 4n elements (the host checks): a lane owns the
+// output pair (h, 2m), (h, 2m + 1), whose windows span input columns 4m - 1 .. 4m + 3.  It loads columns
+// 4m .. 4m + 3 of its three rows as one vector each and takes column 4m - 1 from the lane to its left (a wave's
+// first lane loads it), so a wave reads whole contiguous row segments instead of every second element nine times.
+// Same visiting order and arithmetic as pool_forward_kernel.
+template <typename T, typename R, int OP>
+__global__ void __launch_bounds__(256) pool_forward_k3s2_kernel(PoolGeom g, const T *__restrict__ x, R *__restrict__ out) {
+    uint32_t plane, blk;
+    g.d_opair_blocks.divmod(blockIdx.x, plane, blk);
+    const uint32_t pos = (blk * 256 + threadIdx.x) * 2;
+    if (pos >= static_cast<uint32_t>(g.Ho * g.Wo)) return;
+    uint32_t h, w;
+    g.d_Wo.divmod(pos, h, w);
+    const T *src = plane_of(g, x, plane);
+    const int col = 2 * static_cast<int>(w);  // = 4m
+    const bool load_left = threadIdx.x % 64 == 0 && col > 0;
+    R v[3][5];
+    bool rin[3];
+#pragma unroll
+    for (int p = 0; p < 3; ++p) {
+        const int hi = 2 * static_cast<int>(h) - 1 + p;
+        rin[p] = static_cast<unsigned>(hi) < static_cast<unsigned>(g.H);
+        const T *row = src + static_cast<int64_t>(hi < 0 ? 0 : (hi >= g.H ? g.H - 1 : hi)) * g.xs_h + col;
+        const Quad<T> own = *reinterpret_cast<const Quad<T> *>(row);
+        T left = __shfl_up(own[3], 1);
+        if (load_left) left = row[-1];
+        v[p][0] = static_cast<R>(left);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) v[p][1 + j] = static_cast<R>(own[j]);
+    }
+    const R n = R(9);
+    Pair<R> res;
+#pragma unroll
+    for (int o = 0; o < 2; ++o) {
+        R acc = pool_init<R, OP>();
+#pragma unroll
+        for (int p = 0; p < 3; ++p)
+#pragma unroll
+            for (int q = 0; q < 3; ++q) {
+                const bool in = rin[p] && (o == 1 || q > 0 || col > 0);  // only column -1 can be outside (W = 4n)
+                const R e = in ? v[p][2 * o + q] : pool_init<R, OP>();
+                if constexpr (OP == POOL_MAX) acc = (e > acc) ? e : acc;
+                else if constexpr (OP == POOL_MIN) acc = (e < acc) ? e : acc;
+                else acc = (e / n) + acc;
+            }
+        res[o] = acc;
+    }
+    *reinterpret_cast<Pair<R> *>(out + static_cast<int64_t>(plane) * (g.Ho * g.Wo) + pos) = res;
+}
+
+// First pass of max / min backward for the same geometry and row layout, one output pair per lane (same loads as
+// pool_forward_k3s2_kernel): share = grad_out / (number of in-bounds window elements equal to the result).
+template <typename R>
+__global__ void __launch_bounds__(256)
+pool_share_k3s2_kernel(PoolGeom g, const R *__restrict__ gout, const R *__restrict__ x, const R *__restrict__ res, R *__restrict__ share) {
+    uint32_t plane, blk;
+    g.d_opair_blocks.divmod(blockIdx.x, plane, blk);
+    const uint32_t pos = (blk * 256 + threadIdx.x) * 2;
+    if (pos >= static_cast<uint32_t>(g.Ho * g.Wo)) return;
+    uint32_t h, w;
+    g.d_Wo.divmod(pos, h, w);
+    const R *src = plane_of(g, x, plane);
+    const int col = 2 * static_cast<int>(w);
+    const bool load_left = threadIdx.x % 64 == 0 && col > 0;
+    R v[3][5];
+    bool rin[3];
+#pragma unroll
+    for (int p = 0; p < 3; ++p) {
+        const int hi = 2 * static_cast<int>(h) - 1 + p;
+        rin[p] = static_cast<unsigned>(hi) < static_cast<unsigned>(g.H);
+        const R *row = src + static_cast<int64_t>(hi < 0 ? 0 : (hi >= g.H ? g.H - 1 : hi)) * g.xs_h + col;
+        const Quad<R> own = *reinterpret_cast<const Quad<R> *>(row);
+        R left = __shfl_up(own[3], 1);
+        if (load_left) left = row[-1];
+        v[p][0] = left;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) v[p][1 + j] = own[j];
+    }
+    const int64_t o0 = static_cast<int64_t>(plane) * (g.Ho * g.Wo) + pos;
+    const Pair<R> target = *reinterpret_cast<const Pair<R> *>(res + o0), go = *reinterpret_cast<const Pair<R> *>(gout + o0);
+    Pair<R> amount;
+#pragma unroll
+    for (int o = 0; o < 2; ++o) {
+        R count = R(0);
+#pragma unroll
+        for (int p = 0; p < 3; ++p)
+#pragma unroll
+            for (int q = 0; q < 3; ++q) {
+                const bool in = rin[p] && (o == 1 || q > 0 || col > 0);
+                count += (in && v[p][2 * o + q] == target[o]) ? R(1) : R(0);
+            }
+        amount[o] = go[o] / count;
+    }
+    *reinterpret_cast<Pair<R> *>(share + o0) = amount;
+}
+
 // Backward for non-overlapping windows (stride == k, padding == 0), one lane per output: the window's elements
 // receive grad_out / (number of elements equal to the result) where they equal it (SELECT), or grad_out / k^2
 // each; an element gets its single contribution as 0 + amount, the value the reference's zero-initialised sum
@@ -446,6 +543,8 @@ ttamd_status make_pool_geom(const char *who, int op, const ttamd_view4 *input, i
     g->d_in_blocks = make_fastdiv(static_cast<uint32_t>(g->in_blocks));
     g->quad_blocks = static_cast<int>((in_plane / 4 + 255) / 256);
     g->d_quad_blocks = make_fastdiv(static_cast<uint32_t>(g->quad_blocks > 0 ? g->quad_blocks : 1));
+    g->opair_blocks = static_cast<int>((out_plane / 2 + 255) / 256);
+    g->d_opair_blocks = make_fastdiv(static_cast<uint32_t>(g->opair_blocks > 0 ? g->opair_blocks : 1));
     g->d_out_blocks = make_fastdiv(static_cast<uint32_t>(g->out_blocks));
     g->d_C = make_fastdiv(static_cast<uint32_t>(C));
     g->d_Wo = make_fastdiv(static_cast<uint32_t>(g->Wo > 0 ? g->Wo : 1));
@@ -457,7 +556,10 @@ ttamd_status make_pool_geom(const char *who, int op, const ttamd_view4 *input, i
 template <typename T, typename R, int OP>
 ttamd_status launch_forward(const PoolGeom &g, const void *x, void *out, hipStream_t st) {
     const unsigned blocks = static_cast<unsigned>(static_cast<int64_t>(g.B) * g.C * g.out_blocks);
-    if (g.K == 2 && g.S == 2 && g.P == 0 && rows_pair_aligned<T>(g, x, x))
+    if (g.K == 3 && g.S == 2 && g.P == 1 && rows_quad_aligned<T>(g, x, x) && reinterpret_cast<uintptr_t>(out) % (2 * sizeof(R)) == 0) {
+        const unsigned pair_blocks = static_cast<unsigned>(static_cast<int64_t>(g.B) * g.C * g.opair_blocks);
+        pool_forward_k3s2_kernel<T, R, OP><<<dim3(pair_blocks), dim3(256), 0, st>>>(g, static_cast<const T *>(x), static_cast<R *>(out));
+    } else if (g.K == 2 && g.S == 2 && g.P == 0 && rows_pair_aligned<T>(g, x, x))
         pool_forward_k2_kernel<T, R, OP><<<dim3(blocks), dim3(256), 0, st>>>(g, static_cast<const T *>(x), static_cast<R *>(out));
     else if (g.K == 3)
         pool_forward_kernel<T, R, OP, 3><<<dim3(blocks), dim3(256), 0, st>>>(g, static_cast<const T *>(x), static_cast<R *>(out));
@@ -510,7 +612,10 @@ ttamd_status backward_typed(int device, int op, const PoolGeom &g, const void *g
             const size_t bytes = static_cast<size_t>(planes) * g.Ho * g.Wo * sizeof(R);
             if (ttamd_status s = stream_scratch(device, st, bytes ? bytes : sizeof(R), &ws)) return s;
             R *share = static_cast<R *>(ws);
-            if (g.K == 3) pool_share_kernel<R, 3><<<out_grid, block, 0, st>>>(g, go, xi, rs, share);
+            const auto pair_ok = [](const void *p) { return reinterpret_cast<uintptr_t>(p) % (2 * sizeof(R)) == 0; };
+            if (g.K == 3 && g.S == 2 && g.P == 1 && rows_quad_aligned<R>(g, x, x) && pair_ok(gout) && pair_ok(res))
+                pool_share_k3s2_kernel<R><<<dim3(static_cast<unsigned>(planes * g.opair_blocks)), block, 0, st>>>(g, go, xi, rs, share);
+            else if (g.K == 3) pool_share_kernel<R, 3><<<out_grid, block, 0, st>>>(g, go, xi, rs, share);
             else if (g.K == 2) pool_share_kernel<R, 2><<<out_grid, block, 0, st>>>(g, go, xi, rs, share);
             else pool_share_kernel<R, 0><<<out_grid, block, 0, st>>>(g, go, xi, rs, share);
             if (quad && cols <= 3) pool_backward_quad_kernel<R, true, 3><<<quad_grid, block, 0, st>>>(g, share, xi, rs, gi);
