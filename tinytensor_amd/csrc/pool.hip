@@ -222,6 +222,8 @@ pool_backward_kernel(PoolGeom g, const R *__restrict__ share, const R *__restric
 }
 
 template <typename T>
+using Pair = T __attribute__((ext_vector_type(2)));
+template <typename T>
 using Quad = T __attribute__((ext_vector_type(4)));
 
 // The same gather for four consecutive elements of one input row per lane (W % 4 == 0, dense aligned rows, an
@@ -229,7 +231,10 @@ using Quad = T __attribute__((ext_vector_type(4)));
 // (NC >= ceil((k + 3) / stride)); their amounts and results are loaded once instead of once per element, the input
 // and the gradient move as one vector each, and every element still adds its own covering outputs in increasing
 // (h, w), so the sums are the ones pool_backward_kernel produces.
-template <typename R, bool SELECT, int NC>
+// PAIRS (k == 3, stride == 2, padding == 1, NC == 3): the block's first column is even, so columns 0 and 1 of a
+// block row are one aligned pair and column 2 is the first element of the pair that the lane to the right loads (a
+// wave's last lane loads it): a wave reads whole contiguous segments of the output rows.
+template <typename R, bool SELECT, int NC, bool PAIRS = false>
 __global__ void __launch_bounds__(256)
 pool_backward_quad_kernel(PoolGeom g, const R *__restrict__ share, const R *__restrict__ x, const R *__restrict__ res, R *__restrict__ gin) {
     uint32_t plane, blk;
@@ -254,15 +259,39 @@ pool_backward_quad_kernel(PoolGeom g, const R *__restrict__ share, const R *__re
     }
     const int c_lo = w_lo[0];
     R amount[2 * NC], target[2 * NC];
+    if constexpr (PAIRS) {
+        static_assert(NC == 3, "pairs cover a block of three columns");
+        const bool load_right = threadIdx.x % 64 == 63 && c_lo + 2 < g.Wo;
 #pragma unroll
-    for (int a = 0; a < 2; ++a)
-#pragma unroll
-        for (int b = 0; b < NC; ++b) {
-            const int h = h_lo + a, w = c_lo + b;
-            const int hc = h > g.Ho - 1 ? g.Ho - 1 : h, wc = w > g.Wo - 1 ? g.Wo - 1 : w;
-            amount[a * NC + b] = splane[hc * g.Wo + wc];
-            if constexpr (SELECT) target[a * NC + b] = rplane[hc * g.Wo + wc];
+        for (int a = 0; a < 2; ++a) {
+            const int h = h_lo + a;
+            const int row = (h > g.Ho - 1 ? g.Ho - 1 : h) * g.Wo + c_lo;
+            const Pair<R> am = *reinterpret_cast<const Pair<R> *>(splane + row);
+            R am2 = __shfl_down(am[0], 1);
+            if (load_right) am2 = splane[row + 2];
+            amount[a * NC] = am[0];
+            amount[a * NC + 1] = am[1];
+            amount[a * NC + 2] = am2;
+            if constexpr (SELECT) {
+                const Pair<R> tg = *reinterpret_cast<const Pair<R> *>(rplane + row);
+                R tg2 = __shfl_down(tg[0], 1);
+                if (load_right) tg2 = rplane[row + 2];
+                target[a * NC] = tg[0];
+                target[a * NC + 1] = tg[1];
+                target[a * NC + 2] = tg2;
+            }
         }
+    } else {
+#pragma unroll
+        for (int a = 0; a < 2; ++a)
+#pragma unroll
+            for (int b = 0; b < NC; ++b) {
+                const int h = h_lo + a, w = c_lo + b;
+                const int hc = h > g.Ho - 1 ? g.Ho - 1 : h, wc = w > g.Wo - 1 ? g.Wo - 1 : w;
+                amount[a * NC + b] = splane[hc * g.Wo + wc];
+                if constexpr (SELECT) target[a * NC + b] = rplane[hc * g.Wo + wc];
+            }
+    }
     Quad<R> mine = {R(0), R(0), R(0), R(0)};
     if constexpr (SELECT)
         mine = *reinterpret_cast<const Quad<R> *>(plane_of(g, x, plane) + static_cast<int64_t>(yh) * g.xs_h + xw);
@@ -289,8 +318,6 @@ pool_backward_quad_kernel(PoolGeom g, const R *__restrict__ share, const R *__re
     *reinterpret_cast<Quad<R> *>(gin + static_cast<int64_t>(plane) * (g.H * g.W) + pos) = acc;
 }
 
-template <typename T>
-using Pair = T __attribute__((ext_vector_type(2)));
 
 // Forward for k == 2, stride == 2, padding == 0 on rows that can be read as aligned pairs (the host checks).
 // Same visiting order and arithmetic as pool_forward_kernel.
@@ -602,8 +629,11 @@ ttamd_status backward_typed(int device, int op, const PoolGeom &g, const void *g
         const int cols = (g.K + 3 + g.S - 1) / g.S;   // output columns that can cover four consecutive elements
         const bool quad = two && cols <= 5 && rows_quad_aligned<R>(g, op == POOL_AVG ? nullptr : x, gin);
         const dim3 quad_grid(static_cast<unsigned>(planes * g.quad_blocks));
+        const auto pair_ok = [](const void *p) { return reinterpret_cast<uintptr_t>(p) % (2 * sizeof(R)) == 0; };
+        const bool k3s2p1 = g.K == 3 && g.S == 2 && g.P == 1;
         if (op == POOL_AVG) {
-            if (quad && cols <= 3) pool_backward_quad_kernel<R, false, 3><<<quad_grid, block, 0, st>>>(g, go, xi, rs, gi);
+            if (quad && k3s2p1 && pair_ok(gout)) pool_backward_quad_kernel<R, false, 3, true><<<quad_grid, block, 0, st>>>(g, go, xi, rs, gi);
+            else if (quad && cols <= 3) pool_backward_quad_kernel<R, false, 3><<<quad_grid, block, 0, st>>>(g, go, xi, rs, gi);
             else if (quad) pool_backward_quad_kernel<R, false, 5><<<quad_grid, block, 0, st>>>(g, go, xi, rs, gi);
             else if (two) pool_backward_kernel<R, false, 2><<<in_grid, block, 0, st>>>(g, go, xi, rs, gi);
             else pool_backward_kernel<R, false, 0><<<in_grid, block, 0, st>>>(g, go, xi, rs, gi);
@@ -612,13 +642,13 @@ ttamd_status backward_typed(int device, int op, const PoolGeom &g, const void *g
             const size_t bytes = static_cast<size_t>(planes) * g.Ho * g.Wo * sizeof(R);
             if (ttamd_status s = stream_scratch(device, st, bytes ? bytes : sizeof(R), &ws)) return s;
             R *share = static_cast<R *>(ws);
-            const auto pair_ok = [](const void *p) { return reinterpret_cast<uintptr_t>(p) % (2 * sizeof(R)) == 0; };
-            if (g.K == 3 && g.S == 2 && g.P == 1 && rows_quad_aligned<R>(g, x, x) && pair_ok(gout) && pair_ok(res))
+            if (k3s2p1 && rows_quad_aligned<R>(g, x, x) && pair_ok(gout) && pair_ok(res))
                 pool_share_k3s2_kernel<R><<<dim3(static_cast<unsigned>(planes * g.opair_blocks)), block, 0, st>>>(g, go, xi, rs, share);
             else if (g.K == 3) pool_share_kernel<R, 3><<<out_grid, block, 0, st>>>(g, go, xi, rs, share);
             else if (g.K == 2) pool_share_kernel<R, 2><<<out_grid, block, 0, st>>>(g, go, xi, rs, share);
             else pool_share_kernel<R, 0><<<out_grid, block, 0, st>>>(g, go, xi, rs, share);
-            if (quad && cols <= 3) pool_backward_quad_kernel<R, true, 3><<<quad_grid, block, 0, st>>>(g, share, xi, rs, gi);
+            if (quad && k3s2p1 && pair_ok(res)) pool_backward_quad_kernel<R, true, 3, true><<<quad_grid, block, 0, st>>>(g, share, xi, rs, gi);
+            else if (quad && cols <= 3) pool_backward_quad_kernel<R, true, 3><<<quad_grid, block, 0, st>>>(g, share, xi, rs, gi);
             else if (quad) pool_backward_quad_kernel<R, true, 5><<<quad_grid, block, 0, st>>>(g, share, xi, rs, gi);
             else if (two) pool_backward_kernel<R, true, 2><<<in_grid, block, 0, st>>>(g, share, xi, rs, gi);
             else pool_backward_kernel<R, true, 0><<<in_grid, block, 0, st>>>(g, share, xi, rs, gi);
