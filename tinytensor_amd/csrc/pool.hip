@@ -19,6 +19,9 @@
 // instead of recounting its window.
 // On dense rows of 4n elements with at most 2 x 2 covering windows a lane owns four consecutive elements: it loads
 // the block of covering outputs once and moves the input and the gradient as 16-byte vectors.
+// For k == 3, stride == 2, padding == 1 on such rows (tests/test_conv.cpp:186-278) forward and the first backward
+// pass own one output pair per lane and read their three input rows as vectors, the column between two lanes' vectors
+// travelling by wave shuffle.
 //
 // Non-overlapping windows without padding (stride == k, padding == 0: the max_pool2d(x, 2, 2, 0) of
 // examples/mnist_cnn_example.cpp:55) take a shorter road: an input element lies in at most one window, so backward
