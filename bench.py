@@ -163,6 +163,21 @@ def detail_report(tt, np, path, cpu=True):
     step_flop = 2.0 * 1024 * (784 * 1024 + 1024 * 1024 + 1024 * 10) * 3
     rows.append({"case": "cfg5 whole MLP training step (tensor interface, wall clock incl. host overhead)",
                  "kernel": "9 GEMMs + 21 streaming launches", "ms": round(step_ms, 4), "GFLOP/s": round(step_flop / step_ms / 1e6, 1)})
+    # the same step recorded once into a HIP graph and replayed: one launch per step, no per-op host work
+    gstream = tt.graph.Stream()
+    graph = tt.graph.Graph(gstream, train_step)
+    for _ in range(5):
+        graph.launch()
+    gstream.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(30):
+        graph.launch()
+    gstream.synchronize()
+    graph_ms = (time.perf_counter() - t0) / 30 * 1e3
+    rows.append({"case": "cfg5 whole MLP training step replayed from a HIP graph", "kernel": f"{graph.num_nodes()} graph nodes",
+                 "ms": round(graph_ms, 4), "GFLOP/s": round(step_flop / graph_ms / 1e6, 1)})
+    graph.close()
+    gstream.close()
     if cpu:
         sys.path.insert(0, os.path.join(os.path.dirname(os.path.abspath(__file__)), "tests"))
         from helpers import mlp_train_step  # the same step written over an abstract GEMM

@@ -9,3 +9,4 @@ from .tensor import (  # noqa: F401
     matmul, matmul_backward, where, max_pool2d, min_pool2d, avg_pool2d, pool2d_backward,
 )
 from . import _capi  # noqa: F401
+from . import graph  # noqa: F401  (HIP streams and graphs; loads the HIP runtime on first use)

@@ -10,6 +10,7 @@ computes on the host.
 """
 from __future__ import annotations
 
+import contextlib
 import ctypes as C
 from dataclasses import dataclass
 
@@ -256,8 +257,27 @@ class Tensor:
 
 
 # -------------------------------------------------------------------------------------------------
+_STREAM = None  # hipStream_t (an integer handle) that every launch of this module goes to; None = default stream
+
+
+def _stream_arg():
+    return C.c_void_p(_STREAM) if _STREAM else None
+
+
 class BackendAMD:
     """The methods of tinytensor::BackendBase (tensor/backend_base.h:23-322) that the GEMM path uses."""
+
+    @contextlib.contextmanager
+    def on_stream(self, stream: int | None):
+        """Sends every kernel launched inside the block to `stream` (a hipStream_t handle, e.g. one under HIP graph
+        capture).  No counterpart in the reference, whose CUDA backend always uses the default stream
+        (cuda/kernel_launch.cuh:19-29); host copies (to_numpy, from_numpy) stay blocking default-stream copies."""
+        global _STREAM
+        prev, _STREAM = _STREAM, stream
+        try:
+            yield
+        finally:
+            _STREAM = prev
 
     def get_device_count(self) -> int:
         n = C.c_int()
@@ -284,7 +304,7 @@ class BackendAMD:
         shape = (C.c_int64 * max(nd, 1))(*t.shape)
         stride = (C.c_int64 * max(nd, 1))(*t.stride)
         _check(lib.ttamd_contiguous(t.device.id, t.dtype, nd, shape, stride, C.c_void_p(t.storage.ptr), t.offset,
-                                    C.c_void_p(out.storage.ptr), None))
+                                    C.c_void_p(out.storage.ptr), _stream_arg()))
         return out
 
     @staticmethod
@@ -299,14 +319,14 @@ class BackendAMD:
         out = Tensor.empty(lhs.shape, _capi.BOOL if code >= _capi.BIN["lt"] else lhs.dtype, lhs.device)
         _check(lib.ttamd_binary(lhs.device.id, lhs.dtype, code, lhs.dim(), self._i64(lhs.shape), C.c_void_p(lhs.storage.ptr),
                                 lhs.offset, self._i64(lhs.stride), C.c_void_p(rhs.storage.ptr), rhs.offset,
-                                self._i64(rhs.stride), C.c_void_p(out.storage.ptr), None))
+                                self._i64(rhs.stride), C.c_void_p(out.storage.ptr), _stream_arg()))
         return out
 
     def unary(self, t: Tensor, op: str) -> Tensor:
         """BackendBase::relu / negate / abs / sqrt / exp / log / sigmoid / tanh (backend_base.h:136-260)."""
         out = Tensor.empty(t.shape, t.dtype, t.device)
         _check(lib.ttamd_unary(t.device.id, t.dtype, _capi.UN[op], t.dim(), self._i64(t.shape), C.c_void_p(t.storage.ptr),
-                               t.offset, self._i64(t.stride), C.c_void_p(out.storage.ptr), None))
+                               t.offset, self._i64(t.stride), C.c_void_p(out.storage.ptr), _stream_arg()))
         return out
 
     def where(self, cond: Tensor, lhs: Tensor, rhs: Tensor) -> Tensor:
@@ -317,7 +337,7 @@ class BackendAMD:
         _check(lib.ttamd_where(lhs.device.id, lhs.dtype, lhs.dim(), self._i64(lhs.shape), C.c_void_p(cond.storage.ptr),
                                cond.offset, self._i64(cond.stride), C.c_void_p(lhs.storage.ptr), lhs.offset,
                                self._i64(lhs.stride), C.c_void_p(rhs.storage.ptr), rhs.offset, self._i64(rhs.stride),
-                               C.c_void_p(out.storage.ptr), None))
+                               C.c_void_p(out.storage.ptr), _stream_arg()))
         return out
 
     def sum(self, t: Tensor, dim: int | None = None) -> Tensor:
@@ -329,21 +349,21 @@ class BackendAMD:
             d = dim % t.dim()
             out = Tensor.empty(t.shape[:d] + t.shape[d + 1:], t.dtype, t.device)
         _check(lib.ttamd_sum(t.device.id, t.dtype, t.dim(), self._i64(t.shape), C.c_void_p(t.storage.ptr), t.offset,
-                             self._i64(t.stride), d, C.c_void_p(out.storage.ptr), None))
+                             self._i64(t.stride), d, C.c_void_p(out.storage.ptr), _stream_arg()))
         return out
 
     def full(self, value, numel: int, dtype: int, device: Device) -> Tensor:
         """BackendBase::full (backend_base.h:51)."""
         out = Tensor.empty((numel,), dtype, device)
         host = np.array([value], dtype=_NP_OF[dtype])
-        _check(lib.ttamd_full(device.id, dtype, C.c_void_p(host.ctypes.data), numel, C.c_void_p(out.storage.ptr), None))
+        _check(lib.ttamd_full(device.id, dtype, C.c_void_p(host.ctypes.data), numel, C.c_void_p(out.storage.ptr), _stream_arg()))
         return out
 
     def to(self, t: Tensor, dtype: int) -> Tensor:
         """BackendBase::to(tensor, dtype) (backend_base.h:74): element-wise static_cast into dense storage."""
         out = Tensor.empty(t.shape, dtype, t.device)
         _check(lib.ttamd_cast(t.device.id, t.dtype, dtype, t.dim(), self._i64(t.shape), C.c_void_p(t.storage.ptr), t.offset,
-                              self._i64(t.stride), C.c_void_p(out.storage.ptr), None))
+                              self._i64(t.stride), C.c_void_p(out.storage.ptr), _stream_arg()))
         return out
 
     def assign(self, lhs: Tensor, rhs: Tensor) -> None:
@@ -352,7 +372,7 @@ class BackendAMD:
             raise TTException("assign: operands must share shape and dtype")
         _check(lib.ttamd_assign(lhs.device.id, lhs.dtype, lhs.dim(), self._i64(lhs.shape), C.c_void_p(lhs.storage.ptr),
                                 lhs.offset, self._i64(lhs.stride), C.c_void_p(rhs.storage.ptr), rhs.offset,
-                                self._i64(rhs.stride), None))
+                                self._i64(rhs.stride), _stream_arg()))
 
     def pool2d(self, input: Tensor, op: str, kernel_size: int, stride: int, padding: int) -> Tensor:
         """BackendBase::max_pool2d / min_pool2d / avg_pool2d (backend_base.h:286-311)."""
@@ -363,7 +383,7 @@ class BackendAMD:
         out = Tensor.empty((B, Cc, Ho, Wo), rdtype, input.device)
         iv = input.view4()
         _check(lib.ttamd_pool2d_forward(input.device.id, input.dtype, _capi.POOL[op], C.byref(iv), C.c_void_p(out.storage.ptr),
-                                        B, Cc, H, W, kernel_size, stride, padding, None))
+                                        B, Cc, H, W, kernel_size, stride, padding, _stream_arg()))
         return out
 
     def pool2d_backward(self, grad_output: Tensor, input: Tensor, result: Tensor, op: str, kernel_size: int, stride: int,
@@ -376,7 +396,7 @@ class BackendAMD:
         _check(lib.ttamd_pool2d_backward(
             input.device.id, input.dtype, _capi.POOL[op], C.c_void_p(go.storage.ptr + go.offset * go.itemsize), C.byref(iv),
             C.c_void_p(res.storage.ptr + res.offset * res.itemsize), C.c_void_p(gx.storage.ptr), B, Cc, H, W, kernel_size,
-            stride, padding, None))
+            stride, padding, _stream_arg()))
         return gx
 
     def batched_matmul(self, lhs: Tensor, rhs: Tensor, bias: Tensor | None = None, bias_mode: int = 0,
@@ -397,7 +417,7 @@ class BackendAMD:
             ep.accumulate = int(accumulate)
         lv, rv = lhs.view3(), rhs.view3()
         _check(lib.ttamd_batched_matmul(lhs.device.id, lhs.dtype, B, N, K, M, C.byref(lv), C.byref(rv),
-                                        C.c_void_p(out.storage.ptr), C.byref(ep) if ep is not None else None, None))
+                                        C.c_void_p(out.storage.ptr), C.byref(ep) if ep is not None else None, _stream_arg()))
         return out
 
     def batched_matmul_variant(self, lhs: Tensor, rhs: Tensor) -> str:
@@ -421,7 +441,7 @@ class BackendAMD:
             bias = bias.contiguous()
             bptr = C.c_void_p(bias.storage.ptr + bias.offset * bias.itemsize)
         _check(lib.ttamd_conv2d_forward(input.device.id, input.dtype, C.byref(iv), C.byref(wv), bptr,
-                                        C.c_void_p(out.storage.ptr), B, Cc, H, W, O, k, stride, padding, None))
+                                        C.c_void_p(out.storage.ptr), B, Cc, H, W, O, k, stride, padding, _stream_arg()))
         return out
 
     def conv2d_backward(self, grad_output: Tensor, input: Tensor, weight: Tensor, bias: Tensor | None, stride: int,
@@ -448,7 +468,7 @@ class BackendAMD:
             input.device.id, input.dtype, C.c_void_p(go.storage.ptr + go.offset * go.itemsize), C.byref(iv),
             C.byref(wv), C.c_void_p(gx.storage.ptr), C.c_void_p(gw.storage.ptr),
             C.c_void_p(gb.storage.ptr) if gb is not None else None, B, Cc, H, W, O, k, stride, padding,
-            C.c_void_p(ws.ptr), ws.nbytes, None))
+            C.c_void_p(ws.ptr), ws.nbytes, _stream_arg()))
         if buffers is not None:
             return gx, gw, gb
         self.synchronize(input.device.id)  # the workspace is released when this frame returns
@@ -480,7 +500,7 @@ class Generator:
 def _random_fill(shape, dtype, dist, p0, p1, gen: Generator, device: Device) -> Tensor:
     out = Tensor.empty(shape, dtype, device)
     _check(lib.ttamd_random_fill(device.id, dtype, dist, p0, p1, C.byref(gen.state), out.numel(),
-                                 C.c_void_p(out.storage.ptr), None))
+                                 C.c_void_p(out.storage.ptr), _stream_arg()))
     return out
 
 
