@@ -336,6 +336,35 @@ def test_small_tile_prefetch_depths(tt, dtype, layout, shape):
     assert np.array_equal(got, np.matmul(A.astype(np.float64), B.astype(np.float64)))
 
 
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+@pytest.mark.parametrize("layout", LAYOUTS)
+@pytest.mark.parametrize("shape", [(1024, 1024, 1024), (1000, 512, 1001), (784, 1024, 1024), (130, 2048, 70), (1024, 832, 512)])
+def test_two_halves_of_k_in_one_workgroup(tt, dtype, layout, shape):
+    """Launches with at most one 64x64 workgroup per CU and K a whole number of k-tile pairs split the reduction
+    between the two halves of a 512-lane workgroup; exact on integer-valued data, with and without the epilogue,
+    ragged edges included.  (1000 x 512 x 1001 has rows that are not whole 16-byte vectors in some layouts and then
+    takes the ordinary kernels: the assertion on the name only holds where the variant is expected.)"""
+    N, K, M = shape
+    rng = np.random.default_rng(N + K + M)
+    ints = lambda *sh: rng.integers(-3, 4, sh).astype(dtype)
+    A = ints(1, N, K) if layout[0] == "n" else ints(1, K, N).transpose(0, 2, 1)
+    B = ints(1, K, M) if layout[1] == "n" else ints(1, M, K).transpose(0, 2, 1)
+    tA, tB = to_dev_view(tt, A), to_dev_view(tt, B)
+    be = tt.get_backend(tt.kAMD)
+    name = be.batched_matmul_variant(tA, tB)
+    if shape in ((1024, 1024, 1024), (784, 1024, 1024), (1024, 832, 512)):
+        assert name.endswith("_halves"), name
+    want = np.matmul(A.astype(np.float64), B.astype(np.float64))
+    assert np.array_equal(be.batched_matmul(tA, tB).to_numpy(), want)
+    bias = ints(M)
+    got = be.batched_matmul(tA, tB, bias=dev(tt, bias), bias_mode=1, relu=True).to_numpy()
+    assert np.array_equal(got, np.maximum(want + bias, 0))
+    prev = ints(1, N, M)
+    acc = dev(tt, prev)
+    be.batched_matmul(tA, tB, out=acc, accumulate=True)
+    assert np.array_equal(acc.to_numpy(), want + prev)
+
+
 def test_contiguous_identity(tt, oracle):
     rng = np.random.default_rng(2)
     for dtype in (np.uint8, np.int16, np.float32, np.float64):

@@ -75,6 +75,49 @@ gemm_mfma_kernel(GemmArgs g, int tiles_m, int tiles_n, int ksplit, int k_chunk, 
     }
 }
 
+// Two halves of the reduction in one workgroup of 512 lanes: lanes 0-255 multiply k in [0, K/2), lanes 256-511 k in
+// [K/2, K), each half with its own LDS buffers and the same tile and lane layout; the upper half then parks its
+// accumulators in LDS and the lower half adds them and stores.  For launches with at most one workgroup per CU: a
+// SIMD then holds two waves instead of one, and each covers the other's waits (memory, LDS, barrier).  Both halves
+// run the same number of k tiles (the host only launches this when K is a multiple of 2 * BK), so they pass the
+// engine's barriers in step.  The sum is (first half) + (second half), each accumulated in k order: deterministic.
+template <typename T, int BM, int BN, int BK, int WGM, int WGN, bool A_KC, int A_VEC, bool B_KC, int B_VEC, int PF>
+__global__ void __launch_bounds__(2 * kThreads, 1)
+gemm_mfma_dual_kernel(GemmArgs g, int tiles_m, int tiles_n, int k_half) {
+    using StA = Stager<T, BM, BK, A_KC, A_VEC, PF>;
+    using StB = Stager<T, BN, BK, B_KC, B_VEC, PF>;
+    using Engine = TileEngine<T, BM, BN, BK, WGM, WGN, StA, StB>;
+    static_assert(Engine::kAccPerLane * kThreads * sizeof(T) <= Engine::kLdsBytes, "the parked accumulators fit one half's buffers");
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
+    const int half = threadIdx.x / kThreads, tid = threadIdx.x % kThreads;  // wave-uniform
+    T *const smem = reinterpret_cast<T *>(smem_raw + half * Engine::kLdsBytes);
+    int batch, tm, tn;
+    decode_tile(remap_xcd(blockIdx.x, gridDim.x), tiles_m, tiles_n, batch, tm, tn);
+    const int m0 = tm * BM, n0 = tn * BN, k0 = half * k_half;
+    const T *a_base = static_cast<const T *>(g.A) + static_cast<int64_t>(batch) * g.a_sb + static_cast<int64_t>(m0) * g.a_sm +
+                      static_cast<int64_t>(k0) * g.a_sk;
+    const T *b_base = static_cast<const T *>(g.B) + static_cast<int64_t>(batch) * g.b_sb + static_cast<int64_t>(n0) * g.b_sn +
+                      static_cast<int64_t>(k0) * g.b_sk;
+    StA sa;
+    StB sb;
+    sa.init(a_base, tid, g.M - m0, g.a_sm, g.a_sk, k_half);
+    sb.init(b_base, tid, g.N - n0, g.b_sn, g.b_sk, k_half);
+    Engine eng;
+    eng.init(tid);
+    eng.run(sa, sb, smem, k_half, !sa.edge && !sb.edge);
+    __syncthreads();  // every wave is done with its tiles: the lower half's buffers become the exchange area
+    T *const exchange = reinterpret_cast<T *>(smem_raw);
+    if (half == 1) eng.park_acc(exchange, tid);
+    __syncthreads();
+    if (half == 1) return;
+    eng.add_parked_acc(exchange, tid);
+    T *C = static_cast<T *>(g.C) + static_cast<int64_t>(batch) * g.M * g.N;
+    if (g.bias_mode == 0 && !g.relu && !g.accumulate)
+        store_tile_dense<T, true>(eng, C, g.M, g.N, m0, n0, static_cast<const T *>(nullptr), 0, 0, 0);
+    else
+        store_tile_dense<T, false>(eng, C, g.M, g.N, m0, n0, static_cast<const T *>(g.bias), g.bias_mode, g.relu, g.accumulate);
+}
+
 // C[b][i] = epilogue(sum over s of partial[b * ksplit + s][i]), s ascending (deterministic).
 template <typename T>
 __global__ void __launch_bounds__(256) splitk_reduce_kernel(GemmArgs g, const T *__restrict__ partial, int ksplit) {
@@ -185,6 +228,37 @@ ttamd_status launch_variant(const GemmArgs &g, const SplitPlan &sp, int device, 
     return TTAMD_OK;
 }
 
+template <typename T, int BM, int BN, int BK, int WGM, int WGN, bool A_KC, int A_VEC, bool B_KC, int B_VEC, int PF>
+ttamd_status launch_dual_variant(const GemmArgs &g, hipStream_t stream) {
+    using StA = Stager<T, BM, BK, A_KC, A_VEC, PF>;
+    using StB = Stager<T, BN, BK, B_KC, B_VEC, PF>;
+    constexpr size_t lds_bytes = 2 * TileEngine<T, BM, BN, BK, WGM, WGN, StA, StB>::kLdsBytes;
+    auto kernel = gemm_mfma_dual_kernel<T, BM, BN, BK, WGM, WGN, A_KC, A_VEC, B_KC, B_VEC, PF>;
+    static bool configured = false;
+    if (!configured) {
+        TTAMD_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                            static_cast<int>(lds_bytes)));
+        configured = true;
+    }
+    if (g.K % (2 * BK) != 0) {  // the halves must run the same number of k tiles (they share the engine's barriers)
+        set_error("batched_matmul: internal error, two-half kernel planned for K = %d", g.K);
+        return TTAMD_ERR_INVALID_ARGUMENT;
+    }
+    const int tiles_m = (g.M + BM - 1) / BM, tiles_n = (g.N + BN - 1) / BN;
+    const int64_t blocks = static_cast<int64_t>(tiles_m) * tiles_n * g.batch;
+    kernel<<<dim3(static_cast<unsigned>(blocks)), dim3(2 * kThreads), lds_bytes, stream>>>(g, tiles_m, tiles_n, g.K / 2);
+    TTAMD_HIP_CHECK(hipGetLastError());
+    return TTAMD_OK;
+}
+
+template <typename T, int BM, int BN, int BK, int WGM, int WGN, int VEC, int PF>
+ttamd_status launch_dual_layouts(const GemmArgs &g, bool a_kc, bool b_kc, hipStream_t stream) {
+    if (a_kc && b_kc) return launch_dual_variant<T, BM, BN, BK, WGM, WGN, true, VEC, true, VEC, PF>(g, stream);
+    if (a_kc && !b_kc) return launch_dual_variant<T, BM, BN, BK, WGM, WGN, true, VEC, false, VEC, PF>(g, stream);
+    if (!a_kc && b_kc) return launch_dual_variant<T, BM, BN, BK, WGM, WGN, false, VEC, true, VEC, PF>(g, stream);
+    return launch_dual_variant<T, BM, BN, BK, WGM, WGN, false, VEC, false, VEC, PF>(g, stream);
+}
+
 template <typename T, int BM, int BN, int BK, int WGM, int WGN, int A_VEC, int B_VEC, int PF = 1>
 ttamd_status launch_layouts(const GemmArgs &g, bool a_kc, bool b_kc, const SplitPlan &sp, int device, hipStream_t stream) {
     if (a_kc && b_kc) return launch_variant<T, BM, BN, BK, WGM, WGN, true, A_VEC, true, B_VEC, PF>(g, sp, device, stream);
@@ -265,9 +339,15 @@ ttamd_status launch_mfma_typed(const GemmArgs &g, int device, hipStream_t stream
 
     const SplitPlan sp = (xxl || xl || large) ? SplitPlan{1, g.K} : plan_split<T>(g, TS::SBM, TS::SBN, TS::SBK);
 
+    // Small tiles, at most one workgroup per CU and a long reduction: two halves of k in one workgroup of 8 waves.
+    const int64_t small_wgs = static_cast<int64_t>((g.M + TS::SBM - 1) / TS::SBM) * ((g.N + TS::SBN - 1) / TS::SBN) * g.batch;
+    const bool dual = !(xxl || xl || large) && vec && sp.ksplit == 1 && small_wgs <= 256 && g.K % (2 * TS::SBK) == 0 &&
+                      g.K / (2 * TS::SBK) >= 8 && !getenv("TTAMD_NO_DUAL");
+
     static thread_local char name[112];
     char split_tag[24] = "";
     if (sp.ksplit > 1) snprintf(split_tag, sizeof(split_tag), "_splitk%d", sp.ksplit);
+    if (dual) snprintf(split_tag, sizeof(split_tag), "_halves");
     snprintf(name, sizeof(name), "%s_%s_a%s%d_b%s%d%s", TS::prefix, xxl ? "256x256" : (xl ? "256x128" : (large ? "128x128" : "64x64")), ca.kc ? "kc" : "mc",
              ca.vec, cb.kc ? "kc" : "mc", cb.vec, split_tag);
     *variant = name;
@@ -280,6 +360,7 @@ ttamd_status launch_mfma_typed(const GemmArgs &g, int device, hipStream_t stream
         if (xl) return launch_layouts<T, TS::XBM, TS::XBN, TS::XBK, 2, 2, VK, VK>(g, ca.kc, cb.kc, sp, device, stream);
     }
     if (large) return launch_layouts<T, TS::LBM, TS::LBN, TS::LBK, 2, 2, VK, VK>(g, ca.kc, cb.kc, sp, device, stream);
+    if (dual) return launch_dual_layouts<T, TS::SBM, TS::SBN, TS::SBK, 2, 2, VK, TS::SPF_DEEP>(g, ca.kc, cb.kc, stream);
     if (ca.vec > 1 && cb.vec > 1) {
         // Register prefetch depth of the small tile: 4 k tiles in flight when a CU holds at most two workgroups and the
         // reduction is long (a lone workgroup otherwise waits for memory in every step), else 2, whose smaller register

@@ -638,6 +638,26 @@ struct TileEngine {
         else run_rot(sa, sb, smem, K, unmasked);
     }
 
+    // The accumulators of this lane as NBM * NBN * NACC values at lds[i * kThreads + tid]: lets two engines with the
+    // same tile and lane layout (two halves of one reduction) add their results.
+    static constexpr int kAccPerLane = NBM * NBN * M::NACC;
+    __device__ __forceinline__ void park_acc(T *lds, int tid) const {
+#pragma unroll
+        for (int bm = 0; bm < NBM; ++bm)
+#pragma unroll
+            for (int bn = 0; bn < NBN; ++bn)
+#pragma unroll
+                for (int e = 0; e < M::NACC; ++e) lds[((bm * NBN + bn) * M::NACC + e) * kThreads + tid] = acc[bm][bn][e];
+    }
+    __device__ __forceinline__ void add_parked_acc(const T *lds, int tid) {
+#pragma unroll
+        for (int bm = 0; bm < NBM; ++bm)
+#pragma unroll
+            for (int bn = 0; bn < NBN; ++bn)
+#pragma unroll
+                for (int e = 0; e < M::NACC; ++e) acc[bm][bn][e] += lds[((bm * NBN + bn) * M::NACC + e) * kThreads + tid];
+    }
+
     template <int S>
     __device__ __forceinline__ void prefetch_rest(StA &sa, StB &sb, int K, int KT) {
         if constexpr (S < StA::kPF) {
