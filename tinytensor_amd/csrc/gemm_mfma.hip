@@ -342,7 +342,7 @@ ttamd_status launch_mfma_typed(const GemmArgs &g, int device, hipStream_t stream
     // Small tiles, at most one workgroup per CU and a long reduction: two halves of k in one workgroup of 8 waves.
     const int64_t small_wgs = static_cast<int64_t>((g.M + TS::SBM - 1) / TS::SBM) * ((g.N + TS::SBN - 1) / TS::SBN) * g.batch;
     const bool dual = !(xxl || xl || large) && vec && sp.ksplit == 1 && small_wgs <= 256 && g.K % (2 * TS::SBK) == 0 &&
-                      g.K / (2 * TS::SBK) >= 8 && !getenv("TTAMD_NO_DUAL");
+                      g.K / (2 * TS::SBK) >= 8;
 
     static thread_local char name[112];
     char split_tag[24] = "";
