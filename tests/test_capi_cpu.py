@@ -90,7 +90,8 @@ def test_variant_names_without_gpu(tt):
     assert variant(capi.F32, 1, 256, 512, 256, (0, 512, 1), (0, 256, 1)) == "mfma_f32_64x64_akc4_bmc4_splitk8"  # config 1
     assert variant(capi.F32, 1, 1024, 1024, 10, (0, 1024, 1), (0, 10, 1)) == "mfma_f32_64x64_akc4_bmc1_splitk16"  # skinny N
     assert variant(capi.F32, 1, 1024, 1024, 1024, (0, 1024, 1), (0, 1024, 1)) == "mfma_f32_64x64_akc4_bmc4_halves"  # one workgroup per CU: two halves of k
-    assert variant(capi.F32, 1, 1024, 1000, 1024, (0, 1000, 1), (0, 1024, 1)) == "mfma_f32_64x64_akc4_bmc4"     # K not a whole number of tile pairs
+    assert variant(capi.F32, 1, 1024, 784, 1024, (0, 784, 1), (0, 1024, 1)) == "mfma_f32_64x64_akc4_bmc4_halves"  # 392 + 392: 13 k tiles each
+    assert variant(capi.F32, 1, 1024, 516, 1024, (0, 516, 1), (0, 1024, 1)) == "mfma_f32_64x64_akc4_bmc4"     # 260 + 256: 9 and 8 k tiles
     assert variant(capi.F32, 1, 2048, 1024, 1024, (0, 1024, 1), (0, 1024, 1)) == "mfma_f32_64x64_akc4_bmc4"     # two workgroups per CU already
     assert variant(capi.F32, 1, 70, 50, 90, (0, 155, 3), (0, 2, 100)).endswith("_amc1_bkc1") is False
     assert variant(capi.F32, 1, 70, 50, 90, (0, 155, 3), (0, 2, 100)).startswith("mfma_f32_64x64_a")           # gather variant

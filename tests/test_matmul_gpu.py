@@ -338,12 +338,14 @@ def test_small_tile_prefetch_depths(tt, dtype, layout, shape):
 
 @pytest.mark.parametrize("dtype", [np.float32, np.float64])
 @pytest.mark.parametrize("layout", LAYOUTS)
-@pytest.mark.parametrize("shape", [(1024, 1024, 1024), (1000, 512, 1001), (784, 1024, 1024), (130, 2048, 70), (1024, 832, 512)])
+@pytest.mark.parametrize("shape", [(1024, 1024, 1024), (1000, 512, 1001), (784, 1024, 1024), (130, 2048, 70), (1024, 832, 512),
+                                   (1024, 784, 1024), (960, 1000, 1024), (1024, 516, 1024)])
 def test_two_halves_of_k_in_one_workgroup(tt, dtype, layout, shape):
-    """Launches with at most one 64x64 workgroup per CU and K a whole number of k-tile pairs split the reduction
-    between the two halves of a 512-lane workgroup; exact on integer-valued data, with and without the epilogue,
-    ragged edges included.  (1000 x 512 x 1001 has rows that are not whole 16-byte vectors in some layouts and then
-    takes the ordinary kernels: the assertion on the name only holds where the variant is expected.)"""
+    """Launches with at most one 64x64 workgroup per CU split the reduction between the two halves of a 512-lane
+    workgroup when both halves have the same number of k tiles (784 = 392 + 392 and 1000 = 500 + 500 end in partial
+    tiles; 516 = 260 + 256 has unequal tile counts and takes the ordinary kernel); exact on integer-valued data, with
+    and without the epilogue, ragged edges included.  (1000 x 512 x 1001 has rows that are not whole 16-byte vectors
+    in some layouts and then takes the ordinary kernels: the name is only asserted where the variant is expected.)"""
     N, K, M = shape
     rng = np.random.default_rng(N + K + M)
     ints = lambda *sh: rng.integers(-3, 4, sh).astype(dtype)
@@ -352,8 +354,10 @@ def test_two_halves_of_k_in_one_workgroup(tt, dtype, layout, shape):
     tA, tB = to_dev_view(tt, A), to_dev_view(tt, B)
     be = tt.get_backend(tt.kAMD)
     name = be.batched_matmul_variant(tA, tB)
-    if shape in ((1024, 1024, 1024), (784, 1024, 1024), (1024, 832, 512)):
+    if shape in ((1024, 1024, 1024), (784, 1024, 1024), (1024, 832, 512), (1024, 784, 1024), (960, 1000, 1024)):
         assert name.endswith("_halves"), name
+    if shape == (1024, 516, 1024) and dtype == np.float32:  # fp64 (k tile 16): 258 + 258, 17 tiles each
+        assert not name.endswith("_halves"), name
     want = np.matmul(A.astype(np.float64), B.astype(np.float64))
     assert np.array_equal(be.batched_matmul(tA, tB).to_numpy(), want)
     bias = ints(M)

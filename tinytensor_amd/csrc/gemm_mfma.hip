@@ -79,8 +79,9 @@ gemm_mfma_kernel(GemmArgs g, int tiles_m, int tiles_n, int ksplit, int k_chunk, 
 // [K/2, K), each half with its own LDS buffers and the same tile and lane layout; the upper half then parks its
 // accumulators in LDS and the lower half adds them and stores.  For launches with at most one workgroup per CU: a
 // SIMD then holds two waves instead of one, and each covers the other's waits (memory, LDS, barrier).  Both halves
-// run the same number of k tiles (the host only launches this when K is a multiple of 2 * BK), so they pass the
-// engine's barriers in step.  The sum is (first half) + (second half), each accumulated in k order: deterministic.
+// run the same number of k tiles (the host only launches this when ceil(k_half / BK) == ceil((K - k_half) / BK)), so
+// they pass the engine's barriers in step; a half whose length is not a whole number of tiles takes the masked loop,
+// which has the same barriers.  The sum is (first half) + (second half), each accumulated in k order: deterministic.
 template <typename T, int BM, int BN, int BK, int WGM, int WGN, bool A_KC, int A_VEC, bool B_KC, int B_VEC, int PF>
 __global__ void __launch_bounds__(2 * kThreads, 1)
 gemm_mfma_dual_kernel(GemmArgs g, int tiles_m, int tiles_n, int k_half) {
@@ -94,17 +95,18 @@ gemm_mfma_dual_kernel(GemmArgs g, int tiles_m, int tiles_n, int k_half) {
     int batch, tm, tn;
     decode_tile(remap_xcd(blockIdx.x, gridDim.x), tiles_m, tiles_n, batch, tm, tn);
     const int m0 = tm * BM, n0 = tn * BN, k0 = half * k_half;
+    const int Kc = half == 0 ? k_half : g.K - k_half;
     const T *a_base = static_cast<const T *>(g.A) + static_cast<int64_t>(batch) * g.a_sb + static_cast<int64_t>(m0) * g.a_sm +
                       static_cast<int64_t>(k0) * g.a_sk;
     const T *b_base = static_cast<const T *>(g.B) + static_cast<int64_t>(batch) * g.b_sb + static_cast<int64_t>(n0) * g.b_sn +
                       static_cast<int64_t>(k0) * g.b_sk;
     StA sa;
     StB sb;
-    sa.init(a_base, tid, g.M - m0, g.a_sm, g.a_sk, k_half);
-    sb.init(b_base, tid, g.N - n0, g.b_sn, g.b_sk, k_half);
+    sa.init(a_base, tid, g.M - m0, g.a_sm, g.a_sk, Kc);
+    sb.init(b_base, tid, g.N - n0, g.b_sn, g.b_sk, Kc);
     Engine eng;
     eng.init(tid);
-    eng.run(sa, sb, smem, k_half, !sa.edge && !sb.edge);
+    eng.run(sa, sb, smem, Kc, !sa.edge && !sb.edge && Kc % BK == 0);
     __syncthreads();  // every wave is done with its tiles: the lower half's buffers become the exchange area
     T *const exchange = reinterpret_cast<T *>(smem_raw);
     if (half == 1) eng.park_acc(exchange, tid);
@@ -228,6 +230,14 @@ ttamd_status launch_variant(const GemmArgs &g, const SplitPlan &sp, int device, 
     return TTAMD_OK;
 }
 
+// First k of the upper half of a two-half launch: half of K rounded up to a whole 16-byte vector, so that the upper
+// half's operands keep their alignment.
+template <typename T>
+int dual_k_half(int K) {
+    constexpr int VK = Mfma<T>::VK;
+    return ((K + 1) / 2 + VK - 1) / VK * VK;
+}
+
 template <typename T, int BM, int BN, int BK, int WGM, int WGN, bool A_KC, int A_VEC, bool B_KC, int B_VEC, int PF>
 ttamd_status launch_dual_variant(const GemmArgs &g, hipStream_t stream) {
     using StA = Stager<T, BM, BK, A_KC, A_VEC, PF>;
@@ -240,13 +250,14 @@ ttamd_status launch_dual_variant(const GemmArgs &g, hipStream_t stream) {
                                             static_cast<int>(lds_bytes)));
         configured = true;
     }
-    if (g.K % (2 * BK) != 0) {  // the halves must run the same number of k tiles (they share the engine's barriers)
+    const int k_half = dual_k_half<T>(g.K);
+    if (k_half <= 0 || (k_half + BK - 1) / BK != (g.K - k_half + BK - 1) / BK) {  // the halves share the engine's barriers
         set_error("batched_matmul: internal error, two-half kernel planned for K = %d", g.K);
         return TTAMD_ERR_INVALID_ARGUMENT;
     }
     const int tiles_m = (g.M + BM - 1) / BM, tiles_n = (g.N + BN - 1) / BN;
     const int64_t blocks = static_cast<int64_t>(tiles_m) * tiles_n * g.batch;
-    kernel<<<dim3(static_cast<unsigned>(blocks)), dim3(2 * kThreads), lds_bytes, stream>>>(g, tiles_m, tiles_n, g.K / 2);
+    kernel<<<dim3(static_cast<unsigned>(blocks)), dim3(2 * kThreads), lds_bytes, stream>>>(g, tiles_m, tiles_n, k_half);
     TTAMD_HIP_CHECK(hipGetLastError());
     return TTAMD_OK;
 }
@@ -341,8 +352,10 @@ ttamd_status launch_mfma_typed(const GemmArgs &g, int device, hipStream_t stream
 
     // Small tiles, at most one workgroup per CU and a long reduction: two halves of k in one workgroup of 8 waves.
     const int64_t small_wgs = static_cast<int64_t>((g.M + TS::SBM - 1) / TS::SBM) * ((g.N + TS::SBN - 1) / TS::SBN) * g.batch;
-    const bool dual = !(xxl || xl || large) && vec && sp.ksplit == 1 && small_wgs <= 256 && g.K % (2 * TS::SBK) == 0 &&
-                      g.K / (2 * TS::SBK) >= 8;
+    const int k_half = dual_k_half<T>(g.K);
+    const int half_tiles = (k_half + TS::SBK - 1) / TS::SBK;
+    const bool dual = !(xxl || xl || large) && vec && sp.ksplit == 1 && small_wgs <= 256 && half_tiles >= 8 &&
+                      (g.K - k_half + TS::SBK - 1) / TS::SBK == half_tiles;
 
     static thread_local char name[112];
     char split_tag[24] = "";
