@@ -296,6 +296,9 @@ def test_epilogue_bias_relu_accumulate(tt, oracle, dtype):
     (np.float32, 3900, 4000, "nn", "256x256"), (np.float32, 3900, 3999, "nt", "256x256"),
     (np.float32, 3904, 4000, "tn", "256x256"), (np.float32, 3904, 3999, "tt", "256x256"),
     (np.float32, 6100, 6000, "nn", "128x128"), (np.float32, 6100, 5999, "nt", "128x128"),
+    # 192 x 192 (3 x 3 MFMA blocks per wave): only for outputs made of whole tiles
+    (np.float32, 3072, 3072, "nn", "192x192"), (np.float32, 3072, 3072, "nt", "192x192"),
+    (np.float32, 3072, 3072, "tn", "192x192"), (np.float32, 3072, 3072, "tt", "192x192"), (np.float32, 4224, 4224, "nn", "192x192"),
     (np.float64, 3900, 4000, "nn", "256x128"), (np.float64, 3900, 3999, "nt", "256x128"),
     (np.float64, 3904, 4000, "tn", "256x128"),
 ])

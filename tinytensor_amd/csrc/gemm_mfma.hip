@@ -9,6 +9,7 @@
 // kernel entry, the workgroup -> tile mapping and the host-side operand classification.
 #include "mfma_core.h"
 
+#include <algorithm>
 #include <cmath>
 
 namespace ttamd {
@@ -165,6 +166,8 @@ struct TileShapes<float> {
     static constexpr bool kHasXL = true;
     static constexpr int YBM = 256, YBN = 256, YBK = 16;  // largest: 4 waves of 128 x 128 (4 x 4 MFMA blocks), one workgroup per CU
     static constexpr int XBM = 256, XBN = 128, XBK = 16;  // extra large: 4 waves of 128 x 64 (4 x 2 MFMA blocks)
+    static constexpr int MBM = 192, MBN = 192, MBK = 16;  // 4 waves of 96 x 96 (3 x 3 blocks), one workgroup per CU: for outputs
+                                                          // that 256 x 256 tiles cut into an awkward number (3072^2 = 256 of these)
     static constexpr int LBM = 128, LBN = 128, LBK = 16;  // large: 4 waves of 64 x 64
     static constexpr int SBM = 64, SBN = 64, SBK = 32;    // small: 4 waves of 32 x 32
     static constexpr int SPF = 2, SPF_DEEP = 4;            // k tiles in flight in registers (16-byte operands only)
@@ -338,30 +341,35 @@ ttamd_status launch_mfma_typed(const GemmArgs &g, int device, hipStream_t stream
     const double t_large = vec ? estimate(TS::LBM, TS::LBN, f32 ? 2 : 1, f32 ? 145e12 : 141e12, 0.08) : 1e300;
     const double t_xl = (TS::kHasXL && vec) ? estimate(TS::XBM, TS::XBN, f32 ? 2 : 1, f32 ? 145e12 : 147e12) : 1e300;
     const double t_xxl = (TS::kHasXL && vec && sizeof(T) == 4) ? estimate(TS::YBM, TS::YBN, 1, 147e12) : 1e300;
-    const bool xxl = t_xxl <= t_xl && t_xxl <= t_large && t_xxl <= t_small;
-    const bool xl = !xxl && t_xl <= t_large && t_xl <= t_small;
-    const bool large = !xxl && !xl && t_large <= t_small;
-    const int bm = (xxl || xl) ? TS::XBM : (large ? TS::LBM : TS::SBM);
+    double t_mid = 1e300;
+    if constexpr (sizeof(T) == 4)  // whole tiles only: its ragged edge tiles run at two thirds of the rate (5120^3: 2.9 ms against 2.0)
+        if (vec && g.M % TS::MBM == 0 && g.N % TS::MBN == 0) t_mid = estimate(TS::MBM, TS::MBN, 1, 141e12);
+    const double t_best = std::min(std::min(std::min(t_xxl, t_xl), std::min(t_large, t_small)), t_mid);
+    const bool xxl = t_xxl <= t_best;
+    const bool xl = !xxl && t_xl <= t_best;
+    const bool mid = !xxl && !xl && t_mid <= t_best;
+    const bool large = !xxl && !xl && !mid && t_large <= t_best;
+    const int bm = (xxl || xl) ? TS::XBM : (mid ? 192 : (large ? TS::LBM : TS::SBM));
     // 32-bit buffer addressing: the bytes reachable from a tile's first row must stay below 2^31.
     const int64_t a_reach = (static_cast<int64_t>(bm - 1) * g.a_sm + static_cast<int64_t>(g.K - 1) * g.a_sk + VK) * sizeof(T);
     const int64_t b_reach = (static_cast<int64_t>(bm - 1) * g.b_sn + static_cast<int64_t>(g.K - 1) * g.b_sk + VK) * sizeof(T);
     const int64_t c_reach = static_cast<int64_t>(g.M < bm ? g.M : bm) * g.N * static_cast<int64_t>(sizeof(T));
     if (a_reach >= 0x7fffffffLL || b_reach >= 0x7fffffffLL || c_reach >= 0x7fffffffLL) return TTAMD_OK;
 
-    const SplitPlan sp = (xxl || xl || large) ? SplitPlan{1, g.K} : plan_split<T>(g, TS::SBM, TS::SBN, TS::SBK);
+    const SplitPlan sp = (xxl || xl || mid || large) ? SplitPlan{1, g.K} : plan_split<T>(g, TS::SBM, TS::SBN, TS::SBK);
 
     // Small tiles, at most one workgroup per CU and a long reduction: two halves of k in one workgroup of 8 waves.
     const int64_t small_wgs = static_cast<int64_t>((g.M + TS::SBM - 1) / TS::SBM) * ((g.N + TS::SBN - 1) / TS::SBN) * g.batch;
     const int k_half = dual_k_half<T>(g.K);
     const int half_tiles = (k_half + TS::SBK - 1) / TS::SBK;
-    const bool dual = !(xxl || xl || large) && vec && sp.ksplit == 1 && small_wgs <= 256 && half_tiles >= 8 &&
+    const bool dual = !(xxl || xl || mid || large) && vec && sp.ksplit == 1 && small_wgs <= 256 && half_tiles >= 8 &&
                       (g.K - k_half + TS::SBK - 1) / TS::SBK == half_tiles;
 
     static thread_local char name[112];
     char split_tag[24] = "";
     if (sp.ksplit > 1) snprintf(split_tag, sizeof(split_tag), "_splitk%d", sp.ksplit);
     if (dual) snprintf(split_tag, sizeof(split_tag), "_halves");
-    snprintf(name, sizeof(name), "%s_%s_a%s%d_b%s%d%s", TS::prefix, xxl ? "256x256" : (xl ? "256x128" : (large ? "128x128" : "64x64")), ca.kc ? "kc" : "mc",
+    snprintf(name, sizeof(name), "%s_%s_a%s%d_b%s%d%s", TS::prefix, xxl ? "256x256" : (xl ? "256x128" : (mid ? "192x192" : (large ? "128x128" : "64x64"))), ca.kc ? "kc" : "mc",
              ca.vec, cb.kc ? "kc" : "mc", cb.vec, split_tag);
     *variant = name;
     *handled = true;
@@ -372,6 +380,8 @@ ttamd_status launch_mfma_typed(const GemmArgs &g, int device, hipStream_t stream
         if (xxl) return launch_layouts<T, TS::YBM, TS::YBN, TS::YBK, 2, 2, VK, VK>(g, ca.kc, cb.kc, sp, device, stream);
         if (xl) return launch_layouts<T, TS::XBM, TS::XBN, TS::XBK, 2, 2, VK, VK>(g, ca.kc, cb.kc, sp, device, stream);
     }
+    if constexpr (sizeof(T) == 4)
+        if (mid) return launch_layouts<T, TS::MBM, TS::MBN, TS::MBK, 2, 2, VK, VK>(g, ca.kc, cb.kc, sp, device, stream);
     if (large) return launch_layouts<T, TS::LBM, TS::LBN, TS::LBK, 2, 2, VK, VK>(g, ca.kc, cb.kc, sp, device, stream);
     if (dual) return launch_dual_layouts<T, TS::SBM, TS::SBN, TS::SBK, 2, 2, VK, TS::SPF_DEEP>(g, ca.kc, cb.kc, stream);
     if (ca.vec > 1 && cb.vec > 1) {
