@@ -249,18 +249,27 @@ pool_backward_quad_kernel(PoolGeom g, const R *__restrict__ share, const R *__re
     const int64_t obase = static_cast<int64_t>(plane) * (g.Ho * g.Wo);
     const R *splane = share + obase, *rplane = res + obase;
     const int ay = static_cast<int>(yh) + g.P, ax0 = static_cast<int>(xw) + g.P;
-    const int h_lo = ay - g.K >= 0 ? static_cast<int>(g.d_S.div(static_cast<uint32_t>(ay - g.K))) + 1 : 0;
-    int h_hi = static_cast<int>(g.d_S.div(static_cast<uint32_t>(ay)));
-    h_hi = h_hi >= g.Ho ? g.Ho - 1 : h_hi;
-    int w_lo[4], w_hi[4];
+    int h_lo, h_hi, c_lo, w_lo[4], w_hi[4];
+    if constexpr (PAIRS) {
+        // k 3, stride 2, padding 1: row y lies in the windows of output rows y/2 and, for odd y, y/2 + 1; of the four
+        // columns 4m .. 4m + 3 the first lies in output column 2m, the second in 2m and 2m + 1, the third in 2m + 1,
+        // the fourth in 2m + 1 and 2m + 2 (kCovers below).
+        h_lo = static_cast<int>(yh) >> 1;
+        h_hi = (static_cast<int>(yh) + 1) >> 1;
+        c_lo = static_cast<int>(xw) >> 1;
+    } else {
+        h_lo = ay - g.K >= 0 ? static_cast<int>(g.d_S.div(static_cast<uint32_t>(ay - g.K))) + 1 : 0;
+        h_hi = static_cast<int>(g.d_S.div(static_cast<uint32_t>(ay)));
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-        const int ax = ax0 + j;
-        w_lo[j] = ax - g.K >= 0 ? static_cast<int>(g.d_S.div(static_cast<uint32_t>(ax - g.K))) + 1 : 0;
-        const int hi = static_cast<int>(g.d_S.div(static_cast<uint32_t>(ax)));
-        w_hi[j] = hi >= g.Wo ? g.Wo - 1 : hi;
+        for (int j = 0; j < 4; ++j) {
+            const int ax = ax0 + j;
+            w_lo[j] = ax - g.K >= 0 ? static_cast<int>(g.d_S.div(static_cast<uint32_t>(ax - g.K))) + 1 : 0;
+            const int hi = static_cast<int>(g.d_S.div(static_cast<uint32_t>(ax)));
+            w_hi[j] = hi >= g.Wo ? g.Wo - 1 : hi;
+        }
+        c_lo = w_lo[0];
     }
-    const int c_lo = w_lo[0];
+    h_hi = h_hi >= g.Ho ? g.Ho - 1 : h_hi;
     R amount[2 * NC], target[2 * NC];
     if constexpr (PAIRS) {
         static_assert(NC == 3, "pairs cover a block of three columns");
@@ -312,7 +321,14 @@ pool_backward_quad_kernel(PoolGeom g, const R *__restrict__ share, const R *__re
 #pragma unroll
             for (int b = 0; b < NC; ++b) {
                 const int w = c_lo + b;
-                const bool valid = (h_lo + a <= h_hi) & (w >= w_lo[j]) & (w <= w_hi[j]);
+                bool valid;
+                if constexpr (PAIRS) {
+                    constexpr bool kCovers[4][3] = {{true, false, false}, {true, true, false}, {false, true, false}, {false, true, true}};
+                    if (!kCovers[j][b < 3 ? b : 0]) continue;  // (an output that does not cover the element would add +0)
+                    valid = (h_lo + a <= h_hi) & (w < g.Wo);
+                } else {
+                    valid = (h_lo + a <= h_hi) & (w >= w_lo[j]) & (w <= w_hi[j]);
+                }
                 if constexpr (SELECT) sum += (valid && mine[j] == target[a * NC + b]) ? amount[a * NC + b] : R(0);
                 else sum += valid ? amount[a * NC + b] : R(0);
             }
