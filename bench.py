@@ -2,7 +2,10 @@
 
 A "step" is one launch of ttamd_batched_matmul over the workload that the headline metric is quoted on:
 fp32 C[4096,4096] = A[4096,4096] . B[4096,4096], operands uniform(-1,1) from the reference's seeded generator,
-resident in HBM before the timed region.  Prints ONE JSON line (see README / DESIGN for the fields).
+resident in HBM before the timed region.  Prints ONE JSON line: metric / value / unit (GFLOP/s of the whole job),
+ms_per_step, dtype, config.workload and the kernel variant, `roofline` (achieved TFLOP/s of the kernel from HIP events
+on its stream against the fp32 MFMA peak, HBM traffic per launch) and `cpu_baseline` (the CPU oracle on one core over
+a bounded sample of the same workload).
 """
 import argparse
 import ctypes as C
