@@ -96,6 +96,8 @@ def test_backward_exact_on_integer_data_and_adjoints(tt, oracle, dtype):
     (1, 2, 3, 8, 8, 9, 4),     # a whole vector left of the row
     (1, 2, 3, 6, 8, 1, 2),     # padding wider than the kernel
     (3, 70, 66, 6, 4, 3, 1),   # several channel tiles, one vector per row
+    # rows of 2n but not 4n elements: 8-byte gathers (fp32; fp64's 16-byte vector is the pair already)
+    (2, 8, 16, 14, 14, 3, 1), (2, 8, 12, 13, 26, 3, 0), (1, 8, 8, 9, 10, 5, 2), (2, 72, 68, 6, 6, 3, 1), (1, 4, 4, 8, 6, 9, 4),
 ])
 def test_unit_stride_vector_gathers_exact(tt, oracle, dtype, geom):
     Bn, Cc, O, H, W, k, P = geom

@@ -787,6 +787,11 @@ ttamd_status forward_mfma_tile(const ConvPlan &pl, const void *bias, void *out, 
     using VecB = TapStagerMC<T, BN, BK, VK, false, kConvPF>;
     using OneB = Im2colStager<T, BN, BK, kConvPF>;
     if (a_vec && b_vec) return go(conv_fwd_kernel<T, BM, BN, BK, VK, VecB>, conv_lds_bytes<T, BM, BN, VK, VecB>());
+    if constexpr (sizeof(T) == 4) {  // rows of 2n elements: 8-byte gathers
+        using PairB = TapStagerMC<T, BN, BK, 2, false, kConvPF>;
+        if (a_vec && g.S == 1 && g.xs_w == 1 && g.Wo % 2 == 0)
+            return go(conv_fwd_kernel<T, BM, BN, BK, VK, PairB>, conv_lds_bytes<T, BM, BN, VK, PairB>());
+    }
     if (a_vec) return go(conv_fwd_kernel<T, BM, BN, BK, VK, OneB>, conv_lds_bytes<T, BM, BN, VK, OneB>());
     if (b_vec) return go(conv_fwd_kernel<T, BM, BN, BK, 1, VecB>, conv_lds_bytes<T, BM, BN, 1, VecB>());
     return go(conv_fwd_kernel<T, BM, BN, BK, 1, OneB>, conv_lds_bytes<T, BM, BN, 1, OneB>());
@@ -933,6 +938,11 @@ ttamd_status backward_mfma(const ConvPlan &pl, const void *gout, void *gin, void
             using VecB = TapStagerMC<T, BN, BK, VK, true, kConvPF>;
             using OneB = DgradStager<T, BN, BK, kConvPF>;
             if (a_vec && b_vec) return go(conv_dgrad_kernel<T, BM, BN, BK, VK, VecB>, conv_lds_bytes<T, BM, BN, VK, VecB>());
+            if constexpr (sizeof(T) == 4) {
+                using PairB = TapStagerMC<T, BN, BK, 2, true, kConvPF>;
+                if (a_vec && g.S == 1 && g.W % 2 == 0)
+                    return go(conv_dgrad_kernel<T, BM, BN, BK, VK, PairB>, conv_lds_bytes<T, BM, BN, VK, PairB>());
+            }
             if (a_vec) return go(conv_dgrad_kernel<T, BM, BN, BK, VK, OneB>, conv_lds_bytes<T, BM, BN, VK, OneB>());
             if (b_vec) return go(conv_dgrad_kernel<T, BM, BN, BK, 1, VecB>, conv_lds_bytes<T, BM, BN, 1, VecB>());
             return go(conv_dgrad_kernel<T, BM, BN, BK, 1, OneB>, conv_lds_bytes<T, BM, BN, 1, OneB>());
@@ -957,8 +967,17 @@ ttamd_status backward_mfma(const ConvPlan &pl, const void *gout, void *gin, void
         using VecB = TapStagerKC<T, 64, BK, VK, kConvPF>;
         using OneB = Im2colTStager<T, 64, BK, kConvPF>;
         ttamd_status s;
+        bool pair = false;
+        if constexpr (sizeof(T) == 4) pair = a_vec && !b_vec && g.S == 1 && g.xs_w == 1 && g.Wo % 2 == 0;
         if (a_vec && b_vec) s = go(conv_wgrad_kernel<T, BK, VK, VecB>, conv_lds_bytes<T, 64, 64, VK, VecB>());
-        else if (a_vec) s = go(conv_wgrad_kernel<T, BK, VK, OneB>, conv_lds_bytes<T, 64, 64, VK, OneB>());
+        else if (pair) {
+            if constexpr (sizeof(T) == 4) {
+                using PairB = TapStagerKC<T, 64, BK, 2, kConvPF>;
+                s = go(conv_wgrad_kernel<T, BK, VK, PairB>, conv_lds_bytes<T, 64, 64, VK, PairB>());
+            } else {
+                s = TTAMD_OK;
+            }
+        } else if (a_vec) s = go(conv_wgrad_kernel<T, BK, VK, OneB>, conv_lds_bytes<T, 64, 64, VK, OneB>());
         else if (b_vec) s = go(conv_wgrad_kernel<T, BK, 1, VecB>, conv_lds_bytes<T, 64, 64, 1, VecB>());
         else s = go(conv_wgrad_kernel<T, BK, 1, OneB>, conv_lds_bytes<T, 64, 64, 1, OneB>());
         if (s) return s;

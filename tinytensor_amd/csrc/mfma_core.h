@@ -84,6 +84,13 @@ struct Vec<float, 1> {
     }
 };
 template <>
+struct Vec<float, 2> {  // 8-byte gathers of the conv stagers for rows of 2n (but not 4n) elements
+    using type = float __attribute__((ext_vector_type(2)));
+    static __device__ __forceinline__ type load(__amdgpu_buffer_rsrc_t r, uint32_t off) {
+        return __builtin_bit_cast(type, __builtin_amdgcn_raw_buffer_load_b64(r, off, 0, 0));
+    }
+};
+template <>
 struct Vec<float, 4> {
     using type = f32x4;
     static __device__ __forceinline__ type load(__amdgpu_buffer_rsrc_t r, uint32_t off) {
