@@ -42,10 +42,10 @@ def test_forward_reference_pattern_exact(tt, oracle, dtype, S, P):
     (1, 3, 5, 40, 36, 3, 1, 1),    # long reduction per image: grad_weight in several position slices
     (2, 3, 5, 41, 37, 3, 2, 1),    # the same with element-wise gathers
     (2, 40, 48, 10, 12, 3, 1, 1),  # 64x64 tiles with ragged rows in every product
-    # at most four input channels (one channel, 7x7 stem geometry, strides 2 and 3)
+    # at most four input channels: grad_input on the vector ALU (one channel, 7x7 stem geometry, strides 1, 2 and 3,
+    # one to four windows per axis, several workgroups per image); five windows per axis stay on the MFMA kernel
     (2, 1, 8, 28, 28, 3, 1, 0), (1, 3, 16, 31, 29, 7, 2, 3), (2, 2, 4, 10, 9, 3, 3, 1), (3, 4, 6, 9, 9, 4, 2, 0),
-    # ... and large enough that grad_input takes the direct kernel instead of a padded MFMA tile
-    (16, 3, 32, 160, 160, 7, 2, 3), (12, 4, 16, 192, 200, 5, 3, 1),
+    (2, 3, 8, 40, 36, 4, 1, 2), (2, 3, 32, 64, 60, 7, 2, 3), (1, 4, 16, 48, 50, 5, 3, 1), (2, 2, 4, 12, 12, 5, 1, 2),
 ])
 def test_forward_backward_random(tt, oracle, dtype, geom):
     Bn, Cc, O, H, W, k, S, P = geom

@@ -603,46 +603,63 @@ conv_fwd_direct_kernel(ConvGeom geo, const T *__restrict__ x, const T *__restric
 }
 
 // grad_input for layers with at most CMAX input channels (a network's first layer: 1 or 3), where the 32-row MFMA
-// tile of conv_dgrad_kernel would be all but empty (C = 3: 29 of 32 rows multiply zeros).  One lane per input
-// position (b, y, x) accumulates all its channels over (o, p, q) in that order - the order of conv_dgrad_kernel's
-// reduction index - visiting only the taps whose output coordinate is whole: p = (y + P) mod S, + S, ...
-template <typename T, int CMAX>
+// tile of conv_dgrad_kernel would be all but empty (C = 3: 29 of 32 rows multiply zeros) and, with a stride, most of
+// its reduction too (the taps a stride skips).  One lane per input position (b, y, x) accumulates all its channels on
+// the vector ALU, the weights in LDS as [o][p][q][c].  A position lies in at most NP x NP windows per output channel
+// (NP >= ceil(k / S)): slot (i, j) is tap (p0 + i S, q0 + j S), p0 = (y + P) mod S, with output pixel
+// (oh0 - i, ow0 - j).  A lane decodes its slots once; per output channel it then issues all NP * NP loads of grad_out
+// at once (addresses clamped, invalid slots cleared by a select) and reads each slot's CMAX weights as one LDS
+// vector, so the loads overlap instead of forming a dependent chain per tap.  The sum runs over (o, p, q) in that
+// order, the order of conv_dgrad_kernel's reduction index.
+template <typename T, int CMAX, int NP>
 __global__ void __launch_bounds__(256)
-conv_dgrad_direct_kernel(ConvGeom geo, const T *__restrict__ gout, const T *__restrict__ w, T *__restrict__ gin, int64_t total) {
-    const int64_t idx = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
-    if (idx >= total) return;
-    const int HW = geo.H * geo.W, HoWo = geo.Ho * geo.Wo;
-    const int n = static_cast<int>(idx % HW);
-    const int64_t b = idx / HW;
+conv_dgrad_slots_kernel(ConvGeom geo, const T *__restrict__ gout, const T *__restrict__ w, T *__restrict__ gin, int blocks_per_image) {
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
+    T *const wl = reinterpret_cast<T *>(smem_raw);
+    const int kk = geo.k * geo.k, HW = geo.H * geo.W, HoWo = geo.Ho * geo.Wo;
+    for (int i = threadIdx.x; i < geo.O * kk * CMAX; i += 256) {
+        const int c = i % CMAX, t = (i / CMAX) % kk, o = i / (CMAX * kk);
+        wl[i] = c < geo.C ? w[static_cast<int64_t>(o) * geo.w_so + c * kk + t] : T(0);
+    }
+    __syncthreads();
+    const int b = blockIdx.x / blocks_per_image;
+    const int n = (blockIdx.x - b * blocks_per_image) * 256 + threadIdx.x;
+    if (n >= HW) return;
     uint32_t y, x;
     geo.d_W.divmod(static_cast<uint32_t>(n), y, x);
-    const int ay = static_cast<int>(y) + geo.P, ax = static_cast<int>(x) + geo.P;
     uint32_t oh0, p0, ow0, q0;
-    geo.d_S.divmod(static_cast<uint32_t>(ay), oh0, p0);
-    geo.d_S.divmod(static_cast<uint32_t>(ax), ow0, q0);
+    geo.d_S.divmod(y + static_cast<uint32_t>(geo.P), oh0, p0);
+    geo.d_S.divmod(x + static_cast<uint32_t>(geo.P), ow0, q0);
+    int goff[NP * NP], woff[NP * NP];
+    bool ok[NP * NP];
+#pragma unroll
+    for (int i = 0; i < NP; ++i)
+#pragma unroll
+        for (int j = 0; j < NP; ++j) {
+            const int p = static_cast<int>(p0) + i * geo.S, q = static_cast<int>(q0) + j * geo.S;
+            const int oh = static_cast<int>(oh0) - i, ow = static_cast<int>(ow0) - j;
+            const bool v = (p < geo.k) & (q < geo.k) & (oh >= 0) & (oh < geo.Ho) & (ow >= 0) & (ow < geo.Wo);
+            ok[i * NP + j] = v;
+            goff[i * NP + j] = v ? oh * geo.Wo + ow : 0;
+            woff[i * NP + j] = v ? (p * geo.k + q) * CMAX : 0;
+        }
     T acc[CMAX];
 #pragma unroll
     for (int c = 0; c < CMAX; ++c) acc[c] = T(0);
-    const T *gb = gout + b * geo.O * HoWo;
-    const int kk = geo.k * geo.k;
-    for (int o = 0; o < geo.O; ++o) {
-        const T *go = gb + static_cast<int64_t>(o) * HoWo;
-        const T *wo = w + static_cast<int64_t>(o) * geo.w_so;
-        int oh = static_cast<int>(oh0);
-        for (int p = static_cast<int>(p0); p < geo.k && oh >= 0; p += geo.S, --oh) {
-            if (oh >= geo.Ho) continue;
-            int ow = static_cast<int>(ow0);
-            for (int q = static_cast<int>(q0); q < geo.k && ow >= 0; q += geo.S, --ow) {
-                if (ow >= geo.Wo) continue;
-                const T gv = go[oh * geo.Wo + ow];
-                const T *wt = wo + p * geo.k + q;
+    const T *go = gout + static_cast<int64_t>(b) * geo.O * HoWo;
+    const T *wo = wl;
+    for (int o = 0; o < geo.O; ++o, go += HoWo, wo += kk * CMAX) {
+        T gv[NP * NP];
 #pragma unroll
-                for (int c = 0; c < CMAX; ++c)
-                    if (c < geo.C) acc[c] += wt[c * kk] * gv;
-            }
+        for (int t = 0; t < NP * NP; ++t) gv[t] = go[goff[t]];
+#pragma unroll
+        for (int t = 0; t < NP * NP; ++t) {
+            const T v = ok[t] ? gv[t] : T(0);
+#pragma unroll
+            for (int c = 0; c < CMAX; ++c) acc[c] += wo[woff[t] + c] * v;
         }
     }
-    T *dst = gin + b * geo.C * HW + n;
+    T *dst = gin + static_cast<int64_t>(b) * geo.C * HW + n;
 #pragma unroll
     for (int c = 0; c < CMAX; ++c)
         if (c < geo.C) dst[static_cast<int64_t>(c) * HW] = acc[c];
@@ -877,24 +894,10 @@ BackwardWorkspace backward_workspace(size_t esz, int B, int C, int H, int W, int
     return w;
 }
 
-// Layers with at most this many input channels may compute grad_input with conv_dgrad_direct_kernel.
+// Layers with at most this many input channels compute grad_input with conv_dgrad_slots_kernel when a position lies
+// in at most 4 x 4 windows and the weights fit 64 KiB of LDS (7x7 stride-2 RGB stem on 224 x 224, batch 32: 0.3 ms
+// against 7.3 ms on the padded MFMA tile; 3x3 stride-1 first layers of 28 x 28 and 32 x 32 images: 10 - 25 % faster).
 constexpr int kDirectDgradChannels = 4;
-
-// The MFMA grad_input pads the channels to a 32-row tile and multiplies the zeros of the taps that a stride skips;
-// the direct kernel does neither but runs on the vector ALU, one dependent load chain per lane.  Fitted to
-// measurements (microseconds): the MFMA kernel retires ~200 (32 x 128 tile, k tile of 32) steps per microsecond,
-// the direct kernel ~0.6e6 lane-taps per microsecond once it has about half a million lanes.  A 7x7 stride-2 RGB
-// stem on 224 x 224 images (batch 32) takes 7.3 ms one way and 2.0 ms the other; small images and stride 1 stay on
-// the MFMA kernel (batch 64 of 32 x 32 RGB, 3x3: 35 us against 200 us).
-bool direct_dgrad_pays(const ConvGeom &g) {
-    if (g.C > kDirectDgradChannels) return false;
-    const double lanes = static_cast<double>(g.B) * g.H * g.W;
-    const double taps = static_cast<double>((g.k + g.S - 1) / g.S) * ((g.k + g.S - 1) / g.S) * g.O;
-    const double fill = lanes < 524288.0 ? lanes / 524288.0 : 1.0;
-    const double direct_us = lanes * taps / (0.6e6 * fill);
-    const double mfma_us = static_cast<double>(g.B) * ((g.H * g.W + 127) / 128) * ((g.O * g.k * g.k + 31) / 32) / 200.0;
-    return direct_us < mfma_us;
-}
 
 template <typename T>
 ttamd_status backward_mfma(const ConvPlan &pl, const void *gout, void *gin, void *gw, void *gb, void *ws, size_t ws_bytes,
@@ -910,16 +913,21 @@ ttamd_status backward_mfma(const ConvPlan &pl, const void *gout, void *gin, void
     T *const wt = static_cast<T *>(ws);
     T *const partials = reinterpret_cast<T *>(static_cast<char *>(ws) + plan.wt_bytes);
     // grad_input
-    if (direct_dgrad_pays(g)) {
-        const int64_t total = static_cast<int64_t>(g.B) * g.H * g.W;
-        const int64_t blocks = (total + 255) / 256;
-        if (blocks > 0x7fffffff) {
-            set_error("conv2d_backward: too many workgroups");
-            return TTAMD_ERR_INVALID_ARGUMENT;
-        }
-        conv_dgrad_direct_kernel<T, kDirectDgradChannels><<<dim3(static_cast<unsigned>(blocks)), dim3(256), 0, st>>>(
-            g, static_cast<const T *>(gout), static_cast<const T *>(pl.w), static_cast<T *>(gin), total);
-        TTAMD_HIP_CHECK(hipGetLastError());
+    const int np = (g.k + g.S - 1) / g.S;
+    const size_t slots_lds = static_cast<size_t>(g.O) * g.k * g.k * kDirectDgradChannels * sizeof(T);
+    if (g.C <= kDirectDgradChannels && np <= 4 && slots_lds <= 64 * 1024) {
+        const int bpi = (g.H * g.W + 255) / 256;
+        const int64_t blocks = static_cast<int64_t>(g.B) * bpi;
+        auto go = [&](auto kernel) -> ttamd_status {
+            return launch_conv(kernel, slots_lds, blocks, st, g, static_cast<const T *>(gout), static_cast<const T *>(pl.w),
+                               static_cast<T *>(gin), bpi);
+        };
+        ttamd_status rc;
+        if (np == 1) rc = go(conv_dgrad_slots_kernel<T, kDirectDgradChannels, 1>);
+        else if (np == 2) rc = go(conv_dgrad_slots_kernel<T, kDirectDgradChannels, 2>);
+        else if (np == 3) rc = go(conv_dgrad_slots_kernel<T, kDirectDgradChannels, 3>);
+        else rc = go(conv_dgrad_slots_kernel<T, kDirectDgradChannels, 4>);
+        if (rc) return rc;
     } else {
         const int Kd = g.O * g.k * g.k;
         const int total = g.C * Kd;
