@@ -46,6 +46,10 @@ def test_forward_reference_pattern_exact(tt, oracle, dtype, S, P):
     # one to four windows per axis, several workgroups per image); five windows per axis stay on the MFMA kernel
     (2, 1, 8, 28, 28, 3, 1, 0), (1, 3, 16, 31, 29, 7, 2, 3), (2, 2, 4, 10, 9, 3, 3, 1), (3, 4, 6, 9, 9, 4, 2, 0),
     (2, 3, 8, 40, 36, 4, 1, 2), (2, 3, 32, 64, 60, 7, 2, 3), (1, 4, 16, 48, 50, 5, 3, 1), (2, 2, 4, 12, 12, 5, 1, 2),
+    # strided grad_input as S*S dense sub-problems (more than four channels, class rows of 2n elements): strides 2 and
+    # 3, kernels 1 (most classes empty: zeros), 3, 4, 5 and 7, with and without padding, odd heights, several tiles
+    (2, 8, 16, 16, 16, 3, 2, 1), (2, 16, 8, 13, 20, 5, 2, 2), (1, 8, 8, 18, 12, 3, 3, 1), (2, 8, 16, 14, 12, 4, 2, 0),
+    (2, 8, 12, 10, 8, 1, 2, 0), (1, 40, 72, 30, 28, 3, 2, 1), (2, 12, 16, 21, 24, 7, 2, 3), (1, 8, 4, 9, 24, 5, 3, 2),
 ])
 def test_forward_backward_random(tt, oracle, dtype, geom):
     Bn, Cc, O, H, W, k, S, P = geom

@@ -26,6 +26,10 @@ using namespace mfma;
 
 struct ConvGeom {
     int B, C, H, W, O, k, S, P, Ho, Wo;
+    // grad_input's gather alone reads these: the kernel extent and the padding per axis.  They equal (k, k, P, P)
+    // except in the dense sub-problems that a strided grad_input is split into (rectangular kernels, a padding per
+    // axis); d_kk and d_k then divide by kh * kw and kw.
+    int kh, kw, Ph, Pw;
     int64_t xs_b;              // input batch stride (elements)
     int32_t xs_c, xs_h, xs_w;  // input channel / row / column strides (elements)
     int64_t w_so;              // weight stride of the output channel; (c,p,q) are dense behind it
@@ -240,7 +244,7 @@ struct DgradStager : TileLayout<T, ROWS, BK, false> {
 //   FLIP = true:  taps (o, a, b) of grad_out,        positions = input pixels,  dy = P - a  (grad_input)
 template <bool FLIP>
 struct TapView {
-    int taps, positions, src_h, src_w, k, pad;
+    int taps, positions, src_h, src_w, k, pad, pad_h, pad_w;
     int32_t s_ch, s_h;
     FastDiv d_kk, d_k, d_pw;
     __device__ __forceinline__ explicit TapView(const ConvGeom &g) {
@@ -248,8 +252,10 @@ struct TapView {
         pad = g.P;
         d_kk = g.d_kk;
         d_k = g.d_k;
+        pad_h = FLIP ? g.Ph : g.P;
+        pad_w = FLIP ? g.Pw : g.P;
         if constexpr (FLIP) {
-            taps = g.O * g.k * g.k;
+            taps = g.O * g.kh * g.kw;
             positions = g.H * g.W;
             src_h = g.Ho;
             src_w = g.Wo;
@@ -272,8 +278,8 @@ struct TapView {
         d_kk.divmod(t, ch, r);
         d_k.divmod(r, a, b);
         ch_off = static_cast<int32_t>(ch) * s_ch;
-        dy = FLIP ? pad - static_cast<int>(a) : static_cast<int>(a) - pad;
-        dx = FLIP ? pad - static_cast<int>(b) : static_cast<int>(b) - pad;
+        dy = FLIP ? pad_h - static_cast<int>(a) : static_cast<int>(a) - pad_h;
+        dx = FLIP ? pad_w - static_cast<int>(b) : static_cast<int>(b) - pad_w;
     }
 };
 
@@ -477,6 +483,56 @@ __global__ void __launch_bounds__(256) weight_transpose_kernel(ConvGeom geo, con
     wt[idx] = w[static_cast<int64_t>(o) * geo.w_so + c * k2 + r];
 }
 
+// A strided grad_input splits into S*S dense problems.  Input rows y with (y + P) mod S = ry meet only the taps
+// p = ry, ry + S, ... (kp of them), and with y = y0 + S i, p = ry + S pi the output row (y + P - p) / S is
+// i + ay - pi: a unit-stride grad_input with a kp x kq kernel and paddings (ay, ax) over the Hc x Wc positions of the
+// class, which skips the taps that a stride makes zero (three quarters of the reduction at stride 2).
+struct DgradClass {
+    int ry, rx, kp, kq;  // first tap per axis, taps per axis (0: no window reaches these positions)
+    int y0, x0, Hc, Wc;  // first position per axis, positions per axis
+    int ay, ax;          // paddings of the sub-problem
+    int64_t wt_off;      // element offset of the class's packed weight [C, O*kp*kq] in the workspace
+    int64_t tmp_off;     // element offset of the class's dense result [B, C, Hc*Wc]
+};
+constexpr int kMaxDgradStride = 3;
+struct DgradClasses {
+    DgradClass cls[kMaxDgradStride * kMaxDgradStride];
+};
+
+// wtc[c][(o, pi, qi)] = w[o][c][ry + S pi][rx + S qi]
+template <typename T>
+__global__ void __launch_bounds__(256)
+weight_class_pack_kernel(ConvGeom geo, const T *__restrict__ w, T *__restrict__ wtc, DgradClass cl, int total) {
+    const int idx = blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= total) return;
+    const int kpq = cl.kp * cl.kq, row = geo.O * kpq;
+    const int c = idx / row, rem = idx - c * row;
+    const int o = rem / kpq, r = rem - o * kpq;
+    const int pi = r / cl.kq, qi = r - pi * cl.kq;
+    wtc[idx] = w[static_cast<int64_t>(o) * geo.w_so + (c * geo.k + cl.ry + geo.S * pi) * geo.k + cl.rx + geo.S * qi];
+}
+
+// gin[b][c][y][x] = the class result that owns (y, x), or 0 where no window reaches.
+template <typename T>
+__global__ void __launch_bounds__(256)
+dgrad_interleave_kernel(ConvGeom geo, const T *__restrict__ tmp, T *__restrict__ gin, DgradClasses tab, int64_t total) {
+    const int64_t idx = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (idx >= total) return;
+    const int HW = geo.H * geo.W;
+    const int64_t bc = idx / HW;
+    uint32_t y, x, qy, ry, qx, rx;
+    geo.d_W.divmod(static_cast<uint32_t>(idx - bc * HW), y, x);
+    geo.d_S.divmod(y + static_cast<uint32_t>(geo.P), qy, ry);
+    geo.d_S.divmod(x + static_cast<uint32_t>(geo.P), qx, rx);
+    const DgradClass &cl = tab.cls[ry * geo.S + rx];
+    T v = T(0);
+    if (cl.kp > 0 && cl.kq > 0) {
+        const int i = (static_cast<int>(y) - cl.y0) / geo.S, j = (static_cast<int>(x) - cl.x0) / geo.S;
+        v = tmp[cl.tmp_off + bc * (cl.Hc * cl.Wc) + i * cl.Wc + j];
+    }
+    gin[idx] = v;
+}
+
 // grad_input: M = C, N = H*W, K = O*k*k, one GEMM per image.  wt is the transposed weight [C, O*k*k];
 // StB gathers grad_out.
 template <typename T, int BM, int BN, int BK, int A_VEC, class StB>
@@ -490,7 +546,7 @@ conv_dgrad_kernel(ConvGeom geo, const T *gout, const T *wt, T *gin, int tiles_m,
     int b, tm, tn;
     decode_tile(remap_xcd(blockIdx.x, gridDim.x), tiles_m, tiles_n, b, tm, tn);
     const int m0 = tm * BM, n0 = tn * BN;
-    const int M_ = geo.C, N_ = geo.H * geo.W, K = geo.O * geo.k * geo.k;
+    const int M_ = geo.C, N_ = geo.H * geo.W, K = geo.O * geo.kh * geo.kw;
     const int64_t g_image = static_cast<int64_t>(geo.O) * geo.Ho * geo.Wo;
     StA sa;
     StB sb(geo);
@@ -732,6 +788,7 @@ ttamd_status make_plan(const char *who, ttamd_dtype dtype, const ttamd_view4 *in
     ConvGeom &g = plan->geo;
     g = ConvGeom{};
     g.B = B; g.C = C; g.H = H; g.W = W; g.O = O; g.k = k; g.S = stride; g.P = padding; g.Ho = Ho; g.Wo = Wo;
+    g.kh = k; g.kw = k; g.Ph = padding; g.Pw = padding;
     g.xs_b = input->stride[0];
     g.xs_c = static_cast<int32_t>(input->stride[1]);
     g.xs_h = static_cast<int32_t>(input->stride[2]);
@@ -845,11 +902,51 @@ int wgrad_group(size_t esz, int B, int C, int O, int k) {
     return static_cast<int>((B + max_splits - 1) / max_splits);
 }
 
+// The dense sub-problems of a strided grad_input and whether this build takes that road: strides 2 and 3, more
+// channels than the vector-ALU kernel serves, every class's rows made of whole 8-byte (fp32) / 16-byte (fp64) vectors
+// and every packed weight row of whole 16-byte vectors.  Decided by the geometry alone, so that the workspace query and
+// the launch agree.  wt_elems / tmp_elems: workspace elements for the packed weights and the dense class results.
+struct DgradClassPlan {
+    bool use = false;
+    DgradClasses tab{};
+    int64_t wt_elems = 0, tmp_elems = 0;
+};
+
+DgradClassPlan plan_dgrad_classes(size_t esz, int B, int C, int H, int W, int O, int k, int S, int P) {
+    DgradClassPlan pl;
+    if (S < 2 || S > kMaxDgradStride || C <= 4) return pl;
+    const int vk = esz == 4 ? 4 : 2;
+    bool ok = true;
+    for (int ry = 0; ry < S; ++ry)
+        for (int rx = 0; rx < S; ++rx) {
+            DgradClass &c = pl.tab.cls[ry * S + rx];
+            c.ry = ry;
+            c.rx = rx;
+            c.kp = ry < k ? (k - ry + S - 1) / S : 0;
+            c.kq = rx < k ? (k - rx + S - 1) / S : 0;
+            c.y0 = ((ry - P) % S + S) % S;
+            c.x0 = ((rx - P) % S + S) % S;
+            c.Hc = c.y0 < H ? (H - c.y0 + S - 1) / S : 0;
+            c.Wc = c.x0 < W ? (W - c.x0 + S - 1) / S : 0;
+            c.ay = (c.y0 + P - ry) / S;
+            c.ax = (c.x0 + P - rx) / S;
+            c.wt_off = pl.wt_elems;
+            c.tmp_off = pl.tmp_elems;
+            const int64_t kc = static_cast<int64_t>(O) * c.kp * c.kq;
+            pl.wt_elems += (static_cast<int64_t>(C) * kc + vk - 1) / vk * vk;
+            pl.tmp_elems += static_cast<int64_t>(B) * C * c.Hc * c.Wc;
+            if (c.kp > 0 && c.kq > 0 && c.Hc > 0 && c.Wc > 0 && (c.Wc % 2 != 0 || kc % vk != 0)) ok = false;
+        }
+    pl.use = ok;
+    return pl;
+}
+
 // Workspace layout of conv2d_backward: the transposed weight [C, O*k*k] (rounded up to 256 bytes), then, when
 // grad_weight is computed in several parts, `parts` partial [O, C*k*k] tiles.  A part is (group of images,
 // slice of the output positions): enough of them to give every compute unit a few workgroups.
 struct BackwardWorkspace {
-    size_t wt_bytes, partial_bytes;
+    size_t wt_bytes, partial_bytes;  // wt_bytes: the weight area plus, for a strided grad_input in classes, their dense results
+    size_t class_tmp_offset;         // byte offset of those results (0: not used)
     int group, splits;     // images per group, number of groups
     int kslices, k_chunk;  // slices of the Ho*Wo reduction, positions per slice (a multiple of the k tile)
     int parts() const { return splits * kslices; }
@@ -860,6 +957,11 @@ BackwardWorkspace backward_workspace(size_t esz, int B, int C, int H, int W, int
     BackwardWorkspace w{};
     const size_t tile = static_cast<size_t>(O) * C * k * k * esz;
     w.wt_bytes = (tile + 255) & ~static_cast<size_t>(255);
+    if (const DgradClassPlan dc = plan_dgrad_classes(esz, B, C, H, W, O, k, stride, padding); dc.use) {
+        const size_t packed = static_cast<size_t>(dc.wt_elems) * esz;
+        w.class_tmp_offset = ((packed > tile ? packed : tile) + 255) & ~static_cast<size_t>(255);
+        w.wt_bytes = w.class_tmp_offset + ((static_cast<size_t>(dc.tmp_elems) * esz + 255) & ~static_cast<size_t>(255));
+    }
     w.group = wgrad_group(esz, B, C, O, k);
     w.splits = (B + w.group - 1) / w.group;
     const int bk = esz == 4 ? 32 : 16;
@@ -929,11 +1031,14 @@ ttamd_status backward_mfma(const ConvPlan &pl, const void *gout, void *gin, void
         else rc = go(conv_dgrad_slots_kernel<T, kDirectDgradChannels, 4>);
         if (rc) return rc;
     } else {
-        const int Kd = g.O * g.k * g.k;
-        const int total = g.C * Kd;
-        weight_transpose_kernel<T><<<dim3((total + 255) / 256), dim3(256), 0, st>>>(g, static_cast<const T *>(pl.w), wt, total);
-        TTAMD_HIP_CHECK(hipGetLastError());
-        auto run = [&]<int BM, int BN>() -> ttamd_status {
+        // One unit-stride (or, without the class split, strided) grad_input GEMM: geometry gg, transposed weight wts
+        // [C, O*kh*kw], dense result dst [B, C, gg.H*gg.W].
+        auto dgrad_gemm = [&](const ConvGeom &gg, const T *wts, T *dst) -> ttamd_status {
+          const int Kd = gg.O * gg.kh * gg.kw;
+          auto run = [&]<int BM, int BN>() -> ttamd_status {
+            const ConvGeom &g = gg;
+            const T *wt = wts;
+            T *gin = dst;
             const int M_ = g.C, N_ = g.H * g.W;
             const int tiles_m = (M_ + BM - 1) / BM, tiles_n = (N_ + BN - 1) / BN;
             const int64_t blocks = static_cast<int64_t>(tiles_m) * tiles_n * g.B;
@@ -954,9 +1059,47 @@ ttamd_status backward_mfma(const ConvPlan &pl, const void *gout, void *gin, void
             if (a_vec) return go(conv_dgrad_kernel<T, BM, BN, BK, VK, OneB>, conv_lds_bytes<T, BM, BN, VK, OneB>());
             if (b_vec) return go(conv_dgrad_kernel<T, BM, BN, BK, 1, VecB>, conv_lds_bytes<T, BM, BN, 1, VecB>());
             return go(conv_dgrad_kernel<T, BM, BN, BK, 1, OneB>, conv_lds_bytes<T, BM, BN, 1, OneB>());
+          };
+          return gg.C <= 32 ? run.template operator()<32, 128>() : run.template operator()<64, 64>();
         };
-        const ttamd_status s = g.C <= 32 ? run.template operator()<32, 128>() : run.template operator()<64, 64>();
-        if (s) return s;
+        const DgradClassPlan dc = plan_dgrad_classes(sizeof(T), g.B, g.C, g.H, g.W, g.O, g.k, g.S, g.P);
+        if (dc.use && reinterpret_cast<uintptr_t>(ws) % 16 == 0) {  // (the packed weight rows are read as 16-byte vectors)
+            T *const tmp = reinterpret_cast<T *>(static_cast<char *>(ws) + plan.class_tmp_offset);
+            for (int ci = 0; ci < g.S * g.S; ++ci) {
+                const DgradClass &cl = dc.tab.cls[ci];
+                if (cl.kp == 0 || cl.kq == 0 || cl.Hc == 0 || cl.Wc == 0) continue;
+                const int total = g.C * g.O * cl.kp * cl.kq;
+                weight_class_pack_kernel<T><<<dim3((total + 255) / 256), dim3(256), 0, st>>>(g, static_cast<const T *>(pl.w),
+                                                                                             wt + cl.wt_off, cl, total);
+                TTAMD_HIP_CHECK(hipGetLastError());
+                ConvGeom gc = g;  // the class as a unit-stride problem over its own positions
+                gc.H = cl.Hc;
+                gc.W = cl.Wc;
+                gc.S = 1;
+                gc.kh = cl.kp;
+                gc.kw = cl.kq;
+                gc.Ph = cl.ay;
+                gc.Pw = cl.ax;
+                gc.d_kk = make_fastdiv(static_cast<uint32_t>(cl.kp * cl.kq));
+                gc.d_k = make_fastdiv(static_cast<uint32_t>(cl.kq));
+                gc.d_W = make_fastdiv(static_cast<uint32_t>(cl.Wc));
+                gc.d_S = make_fastdiv(1u);
+                if (ttamd_status rc = dgrad_gemm(gc, wt + cl.wt_off, tmp + cl.tmp_off)) return rc;
+            }
+            const int64_t total = static_cast<int64_t>(g.B) * g.C * g.H * g.W;
+            const int64_t blocks = (total + 255) / 256;
+            if (blocks > 0x7fffffff) {
+                set_error("conv2d_backward: too many workgroups");
+                return TTAMD_ERR_INVALID_ARGUMENT;
+            }
+            dgrad_interleave_kernel<T><<<dim3(static_cast<unsigned>(blocks)), dim3(256), 0, st>>>(g, tmp, static_cast<T *>(gin), dc.tab, total);
+            TTAMD_HIP_CHECK(hipGetLastError());
+        } else {
+            const int total = g.C * g.O * g.k * g.k;
+            weight_transpose_kernel<T><<<dim3((total + 255) / 256), dim3(256), 0, st>>>(g, static_cast<const T *>(pl.w), wt, total);
+            TTAMD_HIP_CHECK(hipGetLastError());
+            if (ttamd_status rc = dgrad_gemm(g, wt, static_cast<T *>(gin))) return rc;
+        }
     }
     // grad_weight
     {
