@@ -12,7 +12,9 @@
 //   grad_input   gX[b][c][y][x] = sum_(o,p,q) W[o][c][p][q] * g[b][o][(y+P-p)/S][(x+P-q)/S]   (when divisible, in range)
 //
 // grad_input is the gather form of the reference's col2im scatter-add (conv.hpp:83-118): every output
-// element is owned by one lane, so there is no write race and the result is deterministic.
+// element is owned by one lane, so there is no write race and the result is deterministic.  With a stride it runs as
+// S*S dense unit-stride problems, one per class of input positions (DgradClass); with at most four input channels on
+// the vector ALU (conv_dgrad_slots_kernel).
 // grad_weight reduces over the batch (conv.cpp:239-244): one workgroup column per (group of images, slice of
 // output positions) accumulates in registers, partial tiles go to the caller's workspace and are summed in a
 // fixed order.  Integer dtypes (forward only; autograd never differentiates them) use a direct
