@@ -50,6 +50,8 @@ def test_forward_reference_pattern_exact(tt, oracle, dtype, S, P):
     # 3, kernels 1 (most classes empty: zeros), 3, 4, 5 and 7, with and without padding, odd heights, several tiles
     (2, 8, 16, 16, 16, 3, 2, 1), (2, 16, 8, 13, 20, 5, 2, 2), (1, 8, 8, 18, 12, 3, 3, 1), (2, 8, 16, 14, 12, 4, 2, 0),
     (2, 8, 12, 10, 8, 1, 2, 0), (1, 40, 72, 30, 28, 3, 2, 1), (2, 12, 16, 21, 24, 7, 2, 3), (1, 8, 4, 9, 24, 5, 3, 2),
+    # ... classes with rows of an odd number of elements (element-wise gathers) and weight rows that are not whole vectors
+    (2, 8, 16, 14, 14, 3, 2, 1), (1, 6, 5, 9, 7, 3, 2, 0), (2, 7, 9, 11, 13, 4, 3, 2),
 ])
 def test_forward_backward_random(tt, oracle, dtype, geom):
     Bn, Cc, O, H, W, k, S, P = geom

@@ -198,13 +198,13 @@ struct DgradStager : TileLayout<T, ROWS, BK, false> {
         line0 = __builtin_amdgcn_readfirstlane(tid / ROWS);
         k_next = 0;
         HoWo = geo.Ho * geo.Wo;
-        K = geo.O * geo.k * geo.k;
+        K = geo.O * geo.kh * geo.kw;
         const int n = n0 + n_local;
         n_ok = n < geo.H * geo.W;
         uint32_t y, x;
         geo.d_W.divmod(static_cast<uint32_t>(n_ok ? n : 0), y, x);
-        yP = static_cast<int>(y) + geo.P;
-        xP = static_cast<int>(x) + geo.P;
+        yP = static_cast<int>(y) + geo.Ph;
+        xP = static_cast<int>(x) + geo.Pw;
     }
 
     template <bool MASK, int SLOT = 0>
@@ -905,9 +905,9 @@ int wgrad_group(size_t esz, int B, int C, int O, int k) {
 }
 
 // The dense sub-problems of a strided grad_input and whether this build takes that road: strides 2 and 3, more
-// channels than the vector-ALU kernel serves, every class's rows made of whole 8-byte (fp32) / 16-byte (fp64) vectors
-// and every packed weight row of whole 16-byte vectors.  Decided by the geometry alone, so that the workspace query and
-// the launch agree.  wt_elems / tmp_elems: workspace elements for the packed weights and the dense class results.
+// channels than the vector-ALU kernel serves.  Decided by the geometry alone, so that the workspace query and the
+// launch agree.  (Each class's packed weight starts on a 16-byte boundary; classes whose rows are whole 8- or 16-byte
+// vectors gather with vector loads, the others element by element.)  wt_elems / tmp_elems: workspace elements for the packed weights and the dense class results.
 struct DgradClassPlan {
     bool use = false;
     DgradClasses tab{};
@@ -918,7 +918,6 @@ DgradClassPlan plan_dgrad_classes(size_t esz, int B, int C, int H, int W, int O,
     DgradClassPlan pl;
     if (S < 2 || S > kMaxDgradStride || C <= 4) return pl;
     const int vk = esz == 4 ? 4 : 2;
-    bool ok = true;
     for (int ry = 0; ry < S; ++ry)
         for (int rx = 0; rx < S; ++rx) {
             DgradClass &c = pl.tab.cls[ry * S + rx];
@@ -937,9 +936,8 @@ DgradClassPlan plan_dgrad_classes(size_t esz, int B, int C, int H, int W, int O,
             const int64_t kc = static_cast<int64_t>(O) * c.kp * c.kq;
             pl.wt_elems += (static_cast<int64_t>(C) * kc + vk - 1) / vk * vk;
             pl.tmp_elems += static_cast<int64_t>(B) * C * c.Hc * c.Wc;
-            if (c.kp > 0 && c.kq > 0 && c.Hc > 0 && c.Wc > 0 && (c.Wc % 2 != 0 || kc % vk != 0)) ok = false;
         }
-    pl.use = ok;
+    pl.use = true;
     return pl;
 }
 
@@ -1065,7 +1063,7 @@ ttamd_status backward_mfma(const ConvPlan &pl, const void *gout, void *gin, void
           return gg.C <= 32 ? run.template operator()<32, 128>() : run.template operator()<64, 64>();
         };
         const DgradClassPlan dc = plan_dgrad_classes(sizeof(T), g.B, g.C, g.H, g.W, g.O, g.k, g.S, g.P);
-        if (dc.use && reinterpret_cast<uintptr_t>(ws) % 16 == 0) {  // (the packed weight rows are read as 16-byte vectors)
+        if (dc.use) {
             T *const tmp = reinterpret_cast<T *>(static_cast<char *>(ws) + plan.class_tmp_offset);
             for (int ci = 0; ci < g.S * g.S; ++ci) {
                 const DgradClass &cl = dc.tab.cls[ci];
