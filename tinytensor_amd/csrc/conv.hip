@@ -688,8 +688,13 @@ conv_dgrad_slots_kernel(ConvGeom geo, const T *__restrict__ gout, const T *__res
     uint32_t oh0, p0, ow0, q0;
     geo.d_S.divmod(y + static_cast<uint32_t>(geo.P), oh0, p0);
     geo.d_S.divmod(x + static_cast<uint32_t>(geo.P), ow0, q0);
-    int goff[NP * NP], woff[NP * NP];
-    bool ok[NP * NP];
+    // grad_out of this image through a buffer descriptor: a slot's byte offset inside a channel plane stays in a
+    // register for the whole kernel (invalid slots hold the out-of-range offset, which loads as zero) and the plane
+    // advances through the scalar offset, so a load costs no address arithmetic and no select.
+    const __amdgpu_buffer_rsrc_t grs = make_rsrc(gout + static_cast<int64_t>(b) * geo.O * HoWo,
+                                                 static_cast<int64_t>(geo.O) * HoWo * static_cast<int64_t>(sizeof(T)));
+    uint32_t goff[NP * NP];
+    int woff[NP * NP];
 #pragma unroll
     for (int i = 0; i < NP; ++i)
 #pragma unroll
@@ -697,24 +702,23 @@ conv_dgrad_slots_kernel(ConvGeom geo, const T *__restrict__ gout, const T *__res
             const int p = static_cast<int>(p0) + i * geo.S, q = static_cast<int>(q0) + j * geo.S;
             const int oh = static_cast<int>(oh0) - i, ow = static_cast<int>(ow0) - j;
             const bool v = (p < geo.k) & (q < geo.k) & (oh >= 0) & (oh < geo.Ho) & (ow >= 0) & (ow < geo.Wo);
-            ok[i * NP + j] = v;
-            goff[i * NP + j] = v ? oh * geo.Wo + ow : 0;
+            goff[i * NP + j] = v ? static_cast<uint32_t>(oh * geo.Wo + ow) * static_cast<uint32_t>(sizeof(T)) : kOob;
             woff[i * NP + j] = v ? (p * geo.k + q) * CMAX : 0;
         }
     T acc[CMAX];
 #pragma unroll
     for (int c = 0; c < CMAX; ++c) acc[c] = T(0);
-    const T *go = gout + static_cast<int64_t>(b) * geo.O * HoWo;
     const T *wo = wl;
-    for (int o = 0; o < geo.O; ++o, go += HoWo, wo += kk * CMAX) {
+    const uint32_t plane_bytes = static_cast<uint32_t>(HoWo) * static_cast<uint32_t>(sizeof(T));
+    uint32_t plane = 0;
+    for (int o = 0; o < geo.O; ++o, plane += plane_bytes, wo += kk * CMAX) {
         T gv[NP * NP];
 #pragma unroll
-        for (int t = 0; t < NP * NP; ++t) gv[t] = go[goff[t]];
+        for (int t = 0; t < NP * NP; ++t) gv[t] = Vec<T, 1>::load_at(grs, goff[t], plane);
 #pragma unroll
         for (int t = 0; t < NP * NP; ++t) {
-            const T v = ok[t] ? gv[t] : T(0);
 #pragma unroll
-            for (int c = 0; c < CMAX; ++c) acc[c] += wo[woff[t] + c] * v;
+            for (int c = 0; c < CMAX; ++c) acc[c] += wo[woff[t] + c] * gv[t];
         }
     }
     T *dst = gin + static_cast<int64_t>(b) * geo.C * HW + n;
@@ -1016,7 +1020,7 @@ ttamd_status backward_mfma(const ConvPlan &pl, const void *gout, void *gin, void
     T *const partials = reinterpret_cast<T *>(static_cast<char *>(ws) + plan.wt_bytes);
     // grad_input
     const int np = (g.k + g.S - 1) / g.S;
-    const size_t slots_lds = static_cast<size_t>(g.O) * g.k * g.k * kDirectDgradChannels * sizeof(T);
+    const size_t slots_lds = static_cast<size_t>(g.O) * g.k * g.k * g.C * sizeof(T);
     if (g.C <= kDirectDgradChannels && np <= 4 && slots_lds <= 64 * 1024) {
         const int bpi = (g.H * g.W + 255) / 256;
         const int64_t blocks = static_cast<int64_t>(g.B) * bpi;
@@ -1024,11 +1028,18 @@ ttamd_status backward_mfma(const ConvPlan &pl, const void *gout, void *gin, void
             return launch_conv(kernel, slots_lds, blocks, st, g, static_cast<const T *>(gout), static_cast<const T *>(pl.w),
                                static_cast<T *>(gin), bpi);
         };
+        auto by_windows = [&]<int CMAX>() -> ttamd_status {  // CMAX = C: no padded channel is multiplied
+            if (np == 1) return go(conv_dgrad_slots_kernel<T, CMAX, 1>);
+            if (np == 2) return go(conv_dgrad_slots_kernel<T, CMAX, 2>);
+            if (np == 3) return go(conv_dgrad_slots_kernel<T, CMAX, 3>);
+            return go(conv_dgrad_slots_kernel<T, CMAX, 4>);
+        };
+        static_assert(kDirectDgradChannels == 4, "one instantiation per channel count");
         ttamd_status rc;
-        if (np == 1) rc = go(conv_dgrad_slots_kernel<T, kDirectDgradChannels, 1>);
-        else if (np == 2) rc = go(conv_dgrad_slots_kernel<T, kDirectDgradChannels, 2>);
-        else if (np == 3) rc = go(conv_dgrad_slots_kernel<T, kDirectDgradChannels, 3>);
-        else rc = go(conv_dgrad_slots_kernel<T, kDirectDgradChannels, 4>);
+        if (g.C == 1) rc = by_windows.template operator()<1>();
+        else if (g.C == 2) rc = by_windows.template operator()<2>();
+        else if (g.C == 3) rc = by_windows.template operator()<3>();
+        else rc = by_windows.template operator()<4>();
         if (rc) return rc;
     } else {
         // One unit-stride (or, without the class split, strided) grad_input GEMM: geometry gg, transposed weight wts

@@ -82,6 +82,10 @@ struct Vec<float, 1> {
     static __device__ __forceinline__ type load(__amdgpu_buffer_rsrc_t r, uint32_t off) {
         return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(r, off, 0, 0));
     }
+    // per-lane offset plus a wave-uniform one (the scalar offset operand of the load)
+    static __device__ __forceinline__ type load_at(__amdgpu_buffer_rsrc_t r, uint32_t off, uint32_t uniform_off) {
+        return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(r, off, uniform_off, 0));
+    }
 };
 template <>
 struct Vec<float, 2> {  // 8-byte gathers of the conv stagers for rows of 2n (but not 4n) elements
@@ -102,6 +106,9 @@ struct Vec<double, 1> {
     using type = double;
     static __device__ __forceinline__ type load(__amdgpu_buffer_rsrc_t r, uint32_t off) {
         return __builtin_bit_cast(double, __builtin_amdgcn_raw_buffer_load_b64(r, off, 0, 0));
+    }
+    static __device__ __forceinline__ type load_at(__amdgpu_buffer_rsrc_t r, uint32_t off, uint32_t uniform_off) {
+        return __builtin_bit_cast(double, __builtin_amdgcn_raw_buffer_load_b64(r, off, uniform_off, 0));
     }
 };
 template <>
