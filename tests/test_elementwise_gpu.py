@@ -210,3 +210,17 @@ def test_linear_default_init_on_device_equals_cpu_init(tt, oracle):
         W, b = tt.linear_init(fan_in, fan_out, g_dev)
         Wc, bc = oracle.linear_init(g_cpu, fan_in, fan_out)
         assert np.array_equal(W.to_numpy(), Wc) and np.array_equal(b.to_numpy(), bc)
+
+
+def test_binary_ops_promote_mixed_dtypes(tt):
+    """Binary operators cast their operands to promote_types(lhs, rhs) (tensor/tensor.cpp:2272-2274): the ReLU mask
+    where(z < 0, 0, 1) is f32 by default and multiplies an f64 gradient as f64."""
+    z = np.array([[-1.5, 0.0, 2.25], [3.0, -0.5, 1.0]])
+    tz = tt.Tensor.from_numpy(z)
+    mask = tt.where(tz < 0.0, 0.0, 1.0)
+    assert mask.dtype == tt._capi.F32
+    prod = tz * mask
+    assert prod.dtype == tt._capi.F64 and np.array_equal(prod.to_numpy(), z * (z >= 0))
+    i = tt.Tensor.from_numpy(np.array([1, 2, 3], dtype=np.int32))
+    f = tt.Tensor.from_numpy(np.array([0.5, 0.25, 2.0], dtype=np.float32))
+    assert np.array_equal((i + f).to_numpy(), np.array([1.5, 2.25, 5.0], dtype=np.float32))

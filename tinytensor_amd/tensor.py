@@ -210,7 +210,11 @@ class Tensor:
     def _binary(self, other, op: str) -> "Tensor":
         if not isinstance(other, Tensor):
             other = full(self.shape, other, self.dtype, self.device)
-        a, b = broadcast_tensors(self, other)
+        if other.dtype != self.dtype:  # operands are cast to promote_types(lhs, rhs) (tensor/tensor.cpp:2272-2274)
+            dt = max(self.dtype, other.dtype)
+            a, b = broadcast_tensors(self.to(dt), other.to(dt))
+        else:
+            a, b = broadcast_tensors(self, other)
         return get_backend(self.device).binary(a, b, op)
 
     def __add__(self, o): return self._binary(o, "add")
