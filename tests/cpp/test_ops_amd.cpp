@@ -69,6 +69,13 @@ TEST_CASE("Binary ops with broadcasting") {
             for (int r = 0; r < R; ++r) ok = ok && t[static_cast<std::size_t>(c * R + r)] == static_cast<T>(2 * a[static_cast<std::size_t>(r * Cn + c)]);
         CHECK(ok);
         CHECK_THROWS_AS(std::ignore = A + Tensor(pattern<T>(R, 5, 1), {R}, device), TTException);  // not broadcastable
+        // mixed dtypes are promoted (tensor/tensor.cpp:2272-2274): T with f64 gives f64
+        std::vector<double> bd, mixed;
+        for (int i = 0; i < Cn; ++i) bd.push_back(0.5 + i);
+        for (int i = 0; i < R * Cn; ++i) mixed.push_back(static_cast<double>(a[static_cast<std::size_t>(i)]) + bd[static_cast<std::size_t>(i % Cn)]);
+        const Tensor M = A + Tensor(bd, {Cn}, device);
+        CHECK(M.dtype() == kF64);
+        CHECK(M.template to_vec<double>() == mixed);
     };
     runner_all_except_bool(test);
 }

@@ -561,8 +561,10 @@ inline auto broadcast_tensors(Tensor a, Tensor b) -> std::pair<Tensor, Tensor> {
 }
 #define TT_AMD_FREE_BINARY(NAME)                                                                 \
     inline auto NAME(const Tensor &lhs, const Tensor &rhs) -> Tensor {                           \
-        if (lhs.dtype() != rhs.dtype()) throw TTException(#NAME ": operands must share a dtype"); \
-        const auto [l, r] = broadcast_tensors(lhs, rhs);                                         \
+        /* operands are cast to promote_types(lhs, rhs) (tensor/tensor.cpp:2272-2274) */         \
+        const auto promoted = promote_types(lhs.dtype(), rhs.dtype());                           \
+        const auto [l, r] = broadcast_tensors(lhs.dtype() == promoted ? lhs : lhs.to(promoted),  \
+                                              rhs.dtype() == promoted ? rhs : rhs.to(promoted)); \
         return get_backend(lhs.device())->NAME(l, r);                                            \
     }
 TT_AMD_FREE_BINARY(add)
