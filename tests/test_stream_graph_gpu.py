@@ -1,6 +1,6 @@
 """Every entry point takes the stream it launches on.  These tests run a small Linear training fragment (fused
 bias + ReLU GEMM with a split reduction, GEMMs on transposed views, elementwise kernels, a two-stage sum, conv2d
-forward) on a stream of their own and then inside a HIP graph captured from that stream, and compare every replay
+forward and backward, max pooling forward and backward) on a stream of their own and then inside a HIP graph captured from that stream, and compare every replay
 with the eager result on the same inputs.  The graph is replayed several times with eager work, host copies and
 synchronisation in between: the library only records kernels (its zero fill is a kernel, not a memset node), takes
 its scratch from per-stream buffers that the warm-up run has grown, and allocates nothing while capturing.
@@ -12,7 +12,8 @@ pytestmark = pytest.mark.gpu
 
 
 def fragment(tt, be, x, w1, b1, w2, target, img, filt):
-    """Forward of Linear-ReLU-Linear with a squared-error sum, the two weight gradients' GEMMs, and a conv2d."""
+    """Forward of Linear-ReLU-Linear with a squared-error sum, the two weight gradients' GEMMs, and a conv2d with ReLU
+    and max pooling, forward and backward."""
     h = be.batched_matmul(x, w1, bias=b1, bias_mode=1, relu=True)  # 256x512x256: split reduction + fused epilogue
     y = be.batched_matmul(h, w2)
     d = be.binary(y, target, "sub")
@@ -20,7 +21,11 @@ def fragment(tt, be, x, w1, b1, w2, target, img, filt):
     gw2 = be.batched_matmul(h.permute(0, 2, 1), d)   # A^T . B on a view
     gh = be.batched_matmul(d, w2.permute(0, 2, 1))   # A . B^T on a view
     c = be.conv2d(img, filt, None, 1, 1)
-    return [h, y, loss, gw2, gh, c]
+    a = c.relu()
+    pooled = tt.max_pool2d(a, 2, 2, 0)
+    ga = tt.pool2d_backward(pooled, a, pooled, "max", 2, 2, 0)
+    gimg, gfilt, _ = be.conv2d_backward(ga, img, filt, None, 1, 1)  # workspace from the allocator's cache, no wait
+    return [h, y, loss, gw2, gh, c, pooled, ga, gimg, gfilt]
 
 
 def make_inputs(tt, seed):

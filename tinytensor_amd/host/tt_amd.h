@@ -295,7 +295,7 @@ public:
         const ttamd_view4 iv = view4(input), wv = view4(w);
         check(ttamd_conv2d_backward(dev, dt, go.data_ptr(), &iv, &wv, gx->ptr_, gw->ptr_, gb ? gb->ptr_ : nullptr, B, C, H, W, O, k, stride,
                                     padding, ws.ptr_, ws_bytes, nullptr));
-        check(ttamd_device_synchronize(dev));  // the workspace is released when this scope ends
+        // (no wait for the kernels: the workspace goes back to the allocator in stream order when this scope ends)
         std::optional<Tensor> grad_bias;
         if (gb) grad_bias = Tensor(gb, input.dtype(), Shape({O}), input.device());
         return {Tensor(gx, input.dtype(), input.shape(), input.device()), Tensor(gw, input.dtype(), weight.shape(), input.device()), grad_bias};

@@ -451,8 +451,7 @@ class BackendAMD:
     def conv2d_backward(self, grad_output: Tensor, input: Tensor, weight: Tensor, bias: Tensor | None, stride: int,
                         padding: int, buffers=None):
         """BackendBase::conv2d_backward (backend_base.h:277-284) -> (grad_input, grad_weight, grad_bias|None).
-        `buffers` = (gx, gw, gb, workspace_storage) from an earlier call reuses the results (benchmarks); the call
-        then does not synchronise."""
+        `buffers` = (gx, gw, gb, workspace_storage) from an earlier call reuses the results (benchmarks)."""
         B, Cc, H, W = input.shape
         O, _, k, _ = weight.shape
         go = grad_output.contiguous()
@@ -475,7 +474,7 @@ class BackendAMD:
             C.c_void_p(ws.ptr), ws.nbytes, _stream_arg()))
         if buffers is not None:
             return gx, gw, gb
-        self.synchronize(input.device.id)  # the workspace is released when this frame returns
+        # (no wait for the kernels: like every other temporary, the workspace goes back to the allocator in stream order)
         self.last_conv_buffers = (gx, gw, gb, ws)
         return gx, gw, gb
 
