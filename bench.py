@@ -181,6 +181,53 @@ def detail_report(tt, np, path, cpu=True):
                  "ms": round(graph_ms, 4), "GFLOP/s": round(step_flop / graph_ms / 1e6, 1)})
     graph.close()
     gstream.close()
+    # one training step of the network of the reference's examples/mnist_cnn_example.cpp:31-63 at its batch size of 256
+    # (conv 1->32, ReLU, conv 32->64, ReLU, max-pool, Linear 9216->128, ReLU, Linear 128->10; no dropout; squared error)
+    crng = np.random.default_rng(3)
+    cdev = lambda *shape, scale=0.1: tt.Tensor.from_numpy(crng.normal(0, scale, shape).astype(f32))
+    cx, ct = cdev(256, 1, 28, 28, scale=1.0), cdev(256, 10, scale=1.0)
+    cw1, cb1, cw2, cb2 = cdev(32, 1, 3, 3, scale=0.3), cdev(32), cdev(64, 32, 3, 3, scale=0.06), cdev(64)
+    cW3, cb3, cW4, cb4 = cdev(9216, 128, scale=0.01), cdev(128), cdev(128, 10), cdev(10)
+    mask = lambda z: tt.where(z < 0.0, 0.0, 1.0)
+
+    def cnn_step():
+        z1 = tt.conv2d(cx, cw1, cb1, 1, 0); a1 = z1.relu(); z2 = tt.conv2d(a1, cw2, cb2, 1, 0); a2 = z2.relu()
+        pooled = tt.max_pool2d(a2, 2, 2, 0); flat = pooled.flatten(1)
+        z3 = tt.linear(flat, cW3, cb3); a3 = z3.relu(); y = tt.linear(a3, cW4, cb4)
+        gy = (y - ct) * 2.0
+        da3, dW4 = tt.matmul_backward(a3.unsqueeze(0), cW4.unsqueeze(0), gy.unsqueeze(0))
+        dz3 = da3.squeeze(0) * mask(z3)
+        dflat, dW3 = tt.matmul_backward(flat.unsqueeze(0), cW3.unsqueeze(0), dz3.unsqueeze(0))
+        da2 = tt.pool2d_backward(dflat.squeeze(0).reshape(list(pooled.shape)), a2, pooled, "max", 2, 2, 0)
+        da1, dw2, db2 = tt.conv2d_backward(da2 * mask(z2), a1, cw2, cb2, 1, 0)
+        dx, dw1, db1 = tt.conv2d_backward(da1 * mask(z1), cx, cw1, cb1, 1, 0)
+        return [y, gy.sum(0), dW4, dz3.sum(0), dW3, dw2, db2, dw1, db1, dx]
+
+    for _ in range(3):
+        cnn_step()
+    be.synchronize(0)
+    t0 = time.perf_counter()
+    for _ in range(20):
+        cnn_step()
+    be.synchronize(0)
+    cnn_ms = (time.perf_counter() - t0) / 20 * 1e3
+    cnn_flop = 3 * 2.0 * 256 * (32 * 26 * 26 * 9 + 64 * 24 * 24 * 288 + 9216 * 128 + 128 * 10)
+    rows.append({"case": "mnist_cnn_example network, one training step at batch 256 (tensor interface, wall clock)",
+                 "kernel": "2 conv + 2 Linear layers, pooling, elementwise", "ms": round(cnn_ms, 4), "GFLOP/s": round(cnn_flop / cnn_ms / 1e6, 1)})
+    gstream = tt.graph.Stream()
+    graph = tt.graph.Graph(gstream, cnn_step)
+    for _ in range(3):
+        graph.launch()
+    gstream.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(20):
+        graph.launch()
+    gstream.synchronize()
+    cnn_graph_ms = (time.perf_counter() - t0) / 20 * 1e3
+    rows.append({"case": "mnist_cnn_example network, one training step at batch 256 replayed from a HIP graph",
+                 "kernel": f"{graph.num_nodes()} graph nodes", "ms": round(cnn_graph_ms, 4), "GFLOP/s": round(cnn_flop / cnn_graph_ms / 1e6, 1)})
+    graph.close()
+    gstream.close()
     if cpu:
         sys.path.insert(0, os.path.join(os.path.dirname(os.path.abspath(__file__)), "tests"))
         from helpers import mlp_train_step  # the same step written over an abstract GEMM
