@@ -146,8 +146,8 @@ ttamd_status ttamd_conv2d_forward(int device, ttamd_dtype dtype, const ttamd_vie
  * gather over output positions (no scatter-add, so no write race); grad_weight reduces over
  * the batch inside one GEMM.  `workspace`/`workspace_bytes`: device scratch (never zero bytes
  * for B > 0) holding the weight transposed to [C, O*k*k] for grad_input (for a strided layer:
- * packed per stride class, plus the classes' dense results) and the per-split partial tiles of
- * grad_weight; query the size with ttamd_conv2d_backward_workspace. */
+ * packed per stride class, plus the classes' dense results), the per-split partial tiles of
+ * grad_weight and the per-part sums of grad_bias; query the size with ttamd_conv2d_backward_workspace. */
 ttamd_status ttamd_conv2d_backward_workspace(ttamd_dtype dtype, int B, int C, int H, int W, int O, int k, int stride,
                                              int padding, size_t *bytes);
 ttamd_status ttamd_conv2d_backward(int device, ttamd_dtype dtype, const void *grad_out, const ttamd_view4 *input,

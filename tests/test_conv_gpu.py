@@ -122,6 +122,29 @@ def test_unit_stride_vector_gathers_exact(tt, oracle, dtype, geom):
 
 
 @pytest.mark.parametrize("dtype", [np.float32, np.float64])
+@pytest.mark.parametrize("geom", [
+    # grad_bias is summed in parts of a channel's B * Ho * Wo elements once there are enough of them.
+    # B, C, O, H, W
+    (64, 2, 3, 24, 24),   # 16-byte loads, 18 whole parts (fp32)
+    (33, 2, 5, 23, 21),   # odd rows: element loads, ragged last part
+    (7, 1, 70, 50, 50),   # parts that start and end inside an image
+    (300, 1, 2, 16, 12),  # more images than parts
+    (1, 1, 1, 96, 96),    # one image, one channel
+])
+def test_grad_bias_in_parts_exact(tt, dtype, geom):
+    Bn, Cc, O, H, W = geom
+    rng = np.random.default_rng(sum(geom))
+    x = rng.integers(-2, 3, (Bn, Cc, H, W)).astype(dtype)
+    w = rng.integers(-2, 3, (O, Cc, 1, 1)).astype(dtype)
+    g = rng.integers(-3, 4, (Bn, O, H, W)).astype(dtype)
+    g[:, :, 0, 0] += 5  # a non-zero mean, so that a dropped or doubled part shows
+    gx, gw, gb = tt.conv2d_backward(dev(tt, g), dev(tt, x), dev(tt, w), dev(tt, np.zeros(O, dtype)), 1, 0)
+    assert np.array_equal(gb.to_numpy(), g.astype(np.int64).sum((0, 2, 3)).astype(dtype))  # closed form, exact in both dtypes
+    assert np.array_equal(gw.to_numpy()[:, :, 0, 0], np.einsum("bohw,bchw->oc", g.astype(np.int64), x.astype(np.int64)).astype(dtype))
+    assert np.array_equal(gx.to_numpy(), np.einsum("bohw,oc->bchw", g.astype(np.int64), w[:, :, 0, 0].astype(np.int64)).astype(dtype))
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
 def test_unaligned_window_of_a_larger_image(tt, oracle, dtype):
     # the input is a window [1:9, 3:15] of a stored [2,3,10,20] tensor: rows start at odd element offsets,
     # so every 16-byte gather is unaligned, and the elements around the window are non-zero

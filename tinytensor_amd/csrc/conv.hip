@@ -19,6 +19,8 @@
 // output positions) accumulates in registers, partial tiles go to the caller's workspace and are summed in a
 // fixed order.  Integer dtypes (forward only; autograd never differentiates them) use a direct
 // vector-ALU kernel with wrap-around arithmetic.
+#include <type_traits>
+
 #include "mfma_core.h"
 
 namespace ttamd {
@@ -614,15 +616,26 @@ __global__ void __launch_bounds__(256) reduce_splits_kernel(const T *__restrict_
     if (lane_s == 0 && i < n) out[i] = red[0][e];
 }
 
-// grad_bias[o] = sum over batch and space of grad_out[b][o][.] (cpu/conv.cpp:289).  One workgroup per channel.
-template <typename T>
-__global__ void __launch_bounds__(256) bias_grad_kernel(const T *__restrict__ gout, T *__restrict__ gb, int B, int O, int HoWo) {
+// grad_bias[o] = sum over batch and space of grad_out[b][o][.] (cpu/conv.cpp:289), in two steps so that the launch
+// fills the chip whatever the channel count: workgroup (o, p) adds part p of channel o's B * HoWo elements (taken as
+// vectors V of sizeof(V) / sizeof(T) elements, numbered image by image), and reduce_splits_kernel adds the parts.
+template <typename T, typename V>
+__global__ void __launch_bounds__(256)
+bias_grad_kernel(const T *__restrict__ gout, T *__restrict__ partial, int O, int HoWo, uint32_t total, uint32_t chunk, FastDiv d_per_image) {
+    constexpr int VEC = sizeof(V) / sizeof(T);
     __shared__ T red[256];
     const int o = blockIdx.x;
+    const uint32_t begin = blockIdx.y * chunk, end = begin + chunk < total ? begin + chunk : total;
     T acc = T(0);
-    for (int b = 0; b < B; ++b) {
-        const T *p = gout + (static_cast<int64_t>(b) * O + o) * HoWo;
-        for (int i = threadIdx.x; i < HoWo; i += 256) acc += p[i];
+    for (uint32_t idx = begin + threadIdx.x; idx < end; idx += 256) {
+        uint32_t b, i;
+        d_per_image.divmod(idx, b, i);
+        const V v = *reinterpret_cast<const V *>(gout + (static_cast<int64_t>(b) * O + o) * HoWo + static_cast<int64_t>(i) * VEC);
+        const T *e = reinterpret_cast<const T *>(&v);
+        T s = e[0];
+#pragma unroll
+        for (int j = 1; j < VEC; ++j) s += e[j];
+        acc += s;
     }
     red[threadIdx.x] = acc;
     __syncthreads();
@@ -630,7 +643,7 @@ __global__ void __launch_bounds__(256) bias_grad_kernel(const T *__restrict__ go
         if (static_cast<int>(threadIdx.x) < s) red[threadIdx.x] += red[threadIdx.x + s];
         __syncthreads();
     }
-    if (threadIdx.x == 0) gb[o] = red[0];
+    if (threadIdx.x == 0) partial[static_cast<int64_t>(blockIdx.y) * O + o] = red[0];
 }
 
 // Direct forward for the integer dtypes: one lane per output element, wrap-around arithmetic in unsigned
@@ -953,9 +966,21 @@ struct BackwardWorkspace {
     size_t class_tmp_offset;         // byte offset of those results (0: not used)
     int group, splits;     // images per group, number of groups
     int kslices, k_chunk;  // slices of the Ho*Wo reduction, positions per slice (a multiple of the k tile)
+    size_t bias_bytes;     // per-part sums of grad_bias: kBiasGradParts rows of O elements
     int parts() const { return splits * kslices; }
-    size_t total() const { return wt_bytes + partial_bytes; }
+    size_t total() const { return wt_bytes + partial_bytes + bias_bytes; }
 };
+
+// grad_bias is summed in at most this many parts per channel (about 2048 workgroups per launch, see bias_grad_parts).
+constexpr int kBiasGradParts = 256;
+
+// Number of parts for a channel's `vectors` loads: about 2048 workgroups in all, at least 512 loads per part.
+inline int bias_grad_parts(int O, int64_t vectors) {
+    int64_t parts = (2048 + O - 1) / O;
+    if (parts > vectors / 512) parts = vectors / 512;
+    if (parts > kBiasGradParts) parts = kBiasGradParts;
+    return parts < 1 ? 1 : static_cast<int>(parts);
+}
 
 BackwardWorkspace backward_workspace(size_t esz, int B, int C, int H, int W, int O, int k, int stride, int padding) {
     BackwardWorkspace w{};
@@ -997,6 +1022,8 @@ BackwardWorkspace backward_workspace(size_t esz, int B, int C, int H, int W, int
     w.kslices = static_cast<int>((k_tiles + chunk_tiles - 1) / chunk_tiles);
     if (w.kslices < 1) w.kslices = 1;
     w.partial_bytes = w.parts() > 1 ? static_cast<size_t>(w.parts()) * tile : 0;
+    w.partial_bytes = (w.partial_bytes + 255) & ~static_cast<size_t>(255);
+    w.bias_bytes = static_cast<size_t>(kBiasGradParts) * O * esz;
     return w;
 }
 
@@ -1150,8 +1177,29 @@ ttamd_status backward_mfma(const ConvPlan &pl, const void *gout, void *gin, void
         }
     }
     if (gb) {
-        bias_grad_kernel<T><<<dim3(g.O), dim3(256), 0, st>>>(static_cast<const T *>(gout), static_cast<T *>(gb), g.B, g.O, HoWo);
+        using V = std::conditional_t<sizeof(T) == 4, float4, double2>;
+        const bool vec = rows_vectorizable<T>(gout, HoWo, static_cast<int64_t>(g.O) * HoWo);
+        const int per_image = vec ? HoWo / VK : HoWo;
+        const int64_t total = static_cast<int64_t>(g.B) * per_image;
+        if (total > 0x7fffffff || g.O > 65535) {
+            set_error("conv2d_backward: grad_bias over %lld loads per channel and %d channels exceeds the launch limits",
+                      static_cast<long long>(total), g.O);
+            return TTAMD_ERR_INVALID_ARGUMENT;
+        }
+        const int bparts = bias_grad_parts(g.O, total);
+        const uint32_t chunk = static_cast<uint32_t>((total + bparts - 1) / bparts);
+        T *const sums = bparts > 1 ? reinterpret_cast<T *>(static_cast<char *>(ws) + plan.wt_bytes + plan.partial_bytes) : static_cast<T *>(gb);
+        const dim3 grid(static_cast<unsigned>(g.O), static_cast<unsigned>(bparts));
+        const FastDiv d = make_fastdiv(static_cast<uint32_t>(per_image));
+        if (vec)
+            bias_grad_kernel<T, V><<<grid, dim3(256), 0, st>>>(static_cast<const T *>(gout), sums, g.O, HoWo, static_cast<uint32_t>(total), chunk, d);
+        else
+            bias_grad_kernel<T, T><<<grid, dim3(256), 0, st>>>(static_cast<const T *>(gout), sums, g.O, HoWo, static_cast<uint32_t>(total), chunk, d);
         TTAMD_HIP_CHECK(hipGetLastError());
+        if (bparts > 1) {
+            reduce_splits_kernel<T><<<dim3(static_cast<unsigned>((g.O + 15) / 16)), dim3(256), 0, st>>>(sums, static_cast<T *>(gb), g.O, bparts);
+            TTAMD_HIP_CHECK(hipGetLastError());
+        }
     }
     return TTAMD_OK;
 }
