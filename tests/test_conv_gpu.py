@@ -104,6 +104,10 @@ def test_backward_exact_on_integer_data_and_adjoints(tt, oracle, dtype):
     (3, 70, 66, 6, 4, 3, 1),   # several channel tiles, one vector per row
     # rows of 2n but not 4n elements: 8-byte gathers (fp32; fp64's 16-byte vector is the pair already)
     (2, 8, 16, 14, 14, 3, 1), (2, 8, 12, 13, 26, 3, 0), (1, 8, 8, 9, 10, 5, 2), (2, 72, 68, 6, 6, 3, 1), (1, 4, 4, 8, 6, 9, 4),
+    # rows that are no whole number of 16-byte vectors, numbered over padded rows (the padding columns are dropped on
+    # the way out): odd widths, widths of 4n + 2, several position tiles per image, a tile that ends inside a row
+    (2, 8, 8, 7, 7, 3, 1), (1, 8, 8, 5, 5, 3, 1), (2, 8, 8, 3, 3, 3, 1), (1, 8, 8, 26, 26, 3, 0), (2, 4, 8, 9, 7, 5, 2),
+    (1, 8, 8, 41, 37, 3, 1), (2, 40, 70, 15, 14, 3, 1), (1, 8, 40, 23, 30, 3, 1),
 ])
 def test_unit_stride_vector_gathers_exact(tt, oracle, dtype, geom):
     Bn, Cc, O, H, W, k, P = geom

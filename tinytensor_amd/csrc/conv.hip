@@ -38,6 +38,11 @@ struct ConvGeom {
     int32_t xs_c, xs_h, xs_w;  // input channel / row / column strides (elements)
     int64_t w_so;              // weight stride of the output channel; (c,p,q) are dense behind it
     FastDiv d_kk, d_k, d_Wo, d_W, d_S;
+    // Not 0: the vector-gather kernels of forward and grad_input number their positions over rows of this many
+    // columns, the row width (Wo, or W for grad_input) rounded up to whole 16-byte vectors, so that a vector never
+    // crosses a row although the width is no multiple of it; the columns past the row are computed and dropped.
+    int row_pad;
+    FastDiv d_row_pad;
 };
 
 // ---------------------------------------------------------------------------------------------
@@ -260,20 +265,20 @@ struct TapView {
         pad_w = FLIP ? g.Pw : g.P;
         if constexpr (FLIP) {
             taps = g.O * g.kh * g.kw;
-            positions = g.H * g.W;
+            positions = g.H * (g.row_pad ? g.row_pad : g.W);
             src_h = g.Ho;
             src_w = g.Wo;
             s_ch = g.Ho * g.Wo;
             s_h = g.Wo;
-            d_pw = g.d_W;
+            d_pw = g.row_pad ? g.d_row_pad : g.d_W;
         } else {
             taps = g.C * g.k * g.k;
-            positions = g.Ho * g.Wo;
+            positions = g.Ho * (g.row_pad ? g.row_pad : g.Wo);
             src_h = g.H;
             src_w = g.W;
             s_ch = g.xs_c;
             s_h = g.xs_h;
-            d_pw = g.d_Wo;
+            d_pw = g.row_pad ? g.d_row_pad : g.d_Wo;
         }
     }
     // (channel offset, dy, dx) of tap index t
@@ -451,6 +456,37 @@ constexpr int kConvPF = 2;
 template <typename T, int BM, int BN, int BK, class StA, class StB>
 using ConvEngine = TileEngine<T, BM, BN, BK, BM == 32 ? 1 : 2, BM == 32 ? 4 : 2, StA, StB>;
 
+// Store of a tile whose positions are numbered over padded rows (ConvGeom::row_pad): tile column n = y * row_pad + x
+// goes to C[m][y * w + x] when x < w, C being [M, h * w]; bias (may be null) adds bias[m].  Pairs: n is even, the
+// padded row a multiple of 4 and w even, so x + 1 < w whenever x < w.
+template <typename T, class Engine>
+__device__ __forceinline__ void store_tile_padded_rows(Engine &eng, T *__restrict__ C, int M_, int h, int w, const FastDiv &d_row, int m0,
+                                                       int n0, const T *__restrict__ bias) {
+    using pair_t = typename Mfma<T>::pair_t;
+    constexpr uint32_t kSz = sizeof(T);
+    const int plane = h * w;
+    const int rows = M_ - m0 < Engine::kBM ? M_ - m0 : Engine::kBM;
+    const __amdgpu_buffer_rsrc_t out = make_rsrc(C + static_cast<int64_t>(m0) * plane, static_cast<int64_t>(rows) * plane * kSz);
+    const __amdgpu_buffer_rsrc_t bias_m = make_rsrc(bias, bias ? static_cast<int64_t>(M_) * kSz : 0);  // absent: loads 0
+    auto offset_of = [&](int ml, int nl) {
+        uint32_t y, x;
+        d_row.divmod(static_cast<uint32_t>(n0 + nl), y, x);
+        const bool inside = ml < rows && static_cast<int>(y) < h && static_cast<int>(x) < w;
+        return inside ? static_cast<uint32_t>(ml * plane + static_cast<int>(y) * w + static_cast<int>(x)) * kSz : kOob;
+    };
+    auto bias_of = [&](int ml) { return Vec<T, 1>::load(bias_m, static_cast<uint32_t>(m0 + ml) * kSz); };
+    const bool pairs_ok = (w % 2 == 0) && (reinterpret_cast<uintptr_t>(C) % (2 * sizeof(T)) == 0);
+    eng.template for_each<true>(
+        pairs_ok, [&](int ml, int nl, T v) { buffer_store(out, offset_of(ml, nl), v + bias_of(ml)); },
+        [&](int ml, int nl, T v0, T v1) {
+            const T bv = bias_of(ml);
+            pair_t o;
+            o[0] = v0 + bv;
+            o[1] = v1 + bv;
+            buffer_store(out, offset_of(ml, nl), o);
+        });
+}
+
 // forward: M = O, N = Ho*Wo, K = C*k*k, one GEMM per image.  StB gathers the image.
 template <typename T, int BM, int BN, int BK, int A_VEC, class StB>
 __global__ void __launch_bounds__(kThreads, 2)
@@ -471,7 +507,8 @@ conv_fwd_kernel(ConvGeom geo, const T *x, const T *w, const T *bias, T *out, int
     Engine eng;
     eng.init(tid);
     eng.run(sa, sb, smem, K, false);
-    store_tile_dense<T, false>(eng, out + static_cast<int64_t>(b) * M_ * N_, M_, N_, m0, n0, bias, bias ? 2 : 0, 0, 0);
+    if (geo.row_pad) store_tile_padded_rows<T>(eng, out + static_cast<int64_t>(b) * M_ * N_, M_, geo.Ho, geo.Wo, geo.d_row_pad, m0, n0, bias);
+    else store_tile_dense<T, false>(eng, out + static_cast<int64_t>(b) * M_ * N_, M_, N_, m0, n0, bias, bias ? 2 : 0, 0, 0);
 }
 
 // wt[c][(o, a, b)] = w[o][c][a][b]: the A operand of grad_input with its reduction index contiguous.
@@ -559,7 +596,10 @@ conv_dgrad_kernel(ConvGeom geo, const T *gout, const T *wt, T *gin, int tiles_m,
     Engine eng;
     eng.init(tid);
     eng.run(sa, sb, smem, K, false);
-    store_tile_dense<T, true>(eng, gin + static_cast<int64_t>(b) * M_ * N_, M_, N_, m0, n0, static_cast<const T *>(nullptr), 0, 0, 0);
+    if (geo.row_pad)
+        store_tile_padded_rows<T>(eng, gin + static_cast<int64_t>(b) * M_ * N_, M_, geo.H, geo.W, geo.d_row_pad, m0, n0, static_cast<const T *>(nullptr));
+    else
+        store_tile_dense<T, true>(eng, gin + static_cast<int64_t>(b) * M_ * N_, M_, N_, m0, n0, static_cast<const T *>(nullptr), 0, 0, 0);
 }
 
 // grad_weight: M = O, N = C*k*k, K = Ho*Wo per image.  Workgroup column `part` = (image group, k slice)
@@ -864,15 +904,31 @@ constexpr size_t conv_lds_bytes() {
     return ConvEngine<T, BM, BN, BK, Stager<T, BM, BK, true, A_VEC, kConvPF>, StB>::kLdsBytes;
 }
 
+// Rows of `width` positions that are no whole number of 16-byte vectors: the padded row width with which the
+// 16-byte gathers serve them, or 0 where the narrower gathers stay ahead (the padding columns are wasted work: at
+// most a fifth more of it against the 8-byte gathers of an even width, at most double against element loads).
+template <typename T>
+int padded_row_width(int width) {
+    constexpr int VK = Mfma<T>::VK;
+    if (width % VK == 0) return 0;
+    const int padded = (width + VK - 1) / VK * VK;
+    const bool pairs = sizeof(T) == 4 && width % 2 == 0;
+    return (pairs ? 5 * padded <= 6 * width : padded <= 2 * width) ? padded : 0;
+}
+
 template <typename T, int BM, int BN>
 ttamd_status forward_mfma_tile(const ConvPlan &pl, const void *bias, void *out, hipStream_t st) {
     constexpr int BK = ConvTiles<T>::BK, VK = Mfma<T>::VK;
-    const ConvGeom &g = pl.geo;
-    const int M_ = g.O, N_ = g.Ho * g.Wo;
+    ConvGeom g = pl.geo;
+    const bool a_vec = rows_vectorizable<T>(pl.w, g.w_so, 0);
+    if (a_vec && g.S == 1 && g.xs_w == 1) {
+        g.row_pad = padded_row_width<T>(g.Wo);
+        g.d_row_pad = make_fastdiv(static_cast<uint32_t>(g.row_pad ? g.row_pad : 1));
+    }
+    const int M_ = g.O, N_ = g.Ho * (g.row_pad ? g.row_pad : g.Wo);
     const int tiles_m = (M_ + BM - 1) / BM, tiles_n = (N_ + BN - 1) / BN;
     const int64_t blocks = static_cast<int64_t>(tiles_m) * tiles_n * g.B;
-    const bool a_vec = rows_vectorizable<T>(pl.w, g.w_so, 0);
-    const bool b_vec = g.S == 1 && g.xs_w == 1 && g.Wo % VK == 0;
+    const bool b_vec = g.S == 1 && g.xs_w == 1 && (g.row_pad || g.Wo % VK == 0);
     auto go = [&](auto kernel, size_t lds) {
         return launch_conv(kernel, lds, blocks, st, g, static_cast<const T *>(pl.x), static_cast<const T *>(pl.w),
                            static_cast<const T *>(bias), static_cast<T *>(out), pl.image_bytes, tiles_m, tiles_n);
@@ -1074,14 +1130,18 @@ ttamd_status backward_mfma(const ConvPlan &pl, const void *gout, void *gin, void
         auto dgrad_gemm = [&](const ConvGeom &gg, const T *wts, T *dst) -> ttamd_status {
           const int Kd = gg.O * gg.kh * gg.kw;
           auto run = [&]<int BM, int BN>() -> ttamd_status {
-            const ConvGeom &g = gg;
+            ConvGeom g = gg;
             const T *wt = wts;
             T *gin = dst;
-            const int M_ = g.C, N_ = g.H * g.W;
+            const bool a_vec = rows_vectorizable<T>(wt, Kd, 0);
+            if (a_vec && g.S == 1) {
+                g.row_pad = padded_row_width<T>(g.W);
+                g.d_row_pad = make_fastdiv(static_cast<uint32_t>(g.row_pad ? g.row_pad : 1));
+            }
+            const int M_ = g.C, N_ = g.H * (g.row_pad ? g.row_pad : g.W);
             const int tiles_m = (M_ + BM - 1) / BM, tiles_n = (N_ + BN - 1) / BN;
             const int64_t blocks = static_cast<int64_t>(tiles_m) * tiles_n * g.B;
-            const bool a_vec = rows_vectorizable<T>(wt, Kd, 0);
-            const bool b_vec = g.S == 1 && g.W % VK == 0;
+            const bool b_vec = g.S == 1 && (g.row_pad || g.W % VK == 0);
             auto go = [&](auto kernel, size_t lds) {
                 return launch_conv(kernel, lds, blocks, st, g, static_cast<const T *>(gout), static_cast<const T *>(wt),
                                    static_cast<T *>(gin), tiles_m, tiles_n);
