@@ -254,6 +254,7 @@ struct DgradStager : TileLayout<T, ROWS, BK, false> {
 template <bool FLIP>
 struct TapView {
     int taps, positions, src_h, src_w, k, pad, pad_h, pad_w;
+    int pos_w;  // positions per row that exist (the row may be numbered over more columns, ConvGeom::row_pad)
     int32_t s_ch, s_h;
     FastDiv d_kk, d_k, d_pw;
     __device__ __forceinline__ explicit TapView(const ConvGeom &g) {
@@ -263,6 +264,7 @@ struct TapView {
         d_k = g.d_k;
         pad_h = FLIP ? g.Ph : g.P;
         pad_w = FLIP ? g.Pw : g.P;
+        pos_w = FLIP ? g.W : g.Wo;
         if constexpr (FLIP) {
             taps = g.O * g.kh * g.kw;
             positions = g.H * (g.row_pad ? g.row_pad : g.W);
@@ -377,7 +379,9 @@ struct TapStagerMC : TileLayout<T, ROWS, BK, false> {
 
 // KC layout (reduction index contiguous in LDS), vectors along the positions, which are the reduction
 // index here: B operand of grad_weight.  The tap of each pass is fixed for the whole kernel.
-template <typename T, int ROWS, int BK, int VEC, int PF = 1>
+// PADDED: the positions are numbered over padded rows; the vectors' components in the padding columns are cleared
+// too (grad_out's stager clears its own), so that no value of either operand, finite or not, enters the sum there.
+template <typename T, int ROWS, int BK, int VEC, int PF = 1, bool PADDED = false>
 struct TapStagerKC : TileLayout<T, ROWS, BK, true> {
     using L = TileLayout<T, ROWS, BK, true>;
     using V = typename Vec<T, VEC>::type;
@@ -439,9 +443,73 @@ struct TapStagerKC : TileLayout<T, ROWS, BK, true> {
     template <int SLOT = 0>
     __device__ __forceinline__ void store(T *lds) const {
 #pragma unroll
+        for (int p = 0; p < P; ++p) {
+            V v = clear_outside_row<T, VEC>(reg[SLOT][p], col0[SLOT] + dx[p], tv.src_w);
+            if constexpr (PADDED) v = clear_outside_row<T, VEC>(v, col0[SLOT], tv.pos_w);
+            *reinterpret_cast<V *>(&lds[(p * RPP + row0) * L::LD + k_local]) = v;
+        }
+    }
+};
+
+// A operand of grad_weight when the positions, its reduction index, are numbered over padded rows
+// (ConvGeom::row_pad): row m is channel m0 + m of one image of grad_out [O][Ho * Wo], k = y * row_pad + x.  One vector
+// load fetches columns x .. x + VEC - 1 of row y at any 4-byte alignment; the components in the padding columns
+// (x >= Wo), which hold the next row's first elements, are cleared in store(), so that the gathered input values of
+// those columns never reach the sum.  KC layout, same LDS image as Stager<T, ROWS, BK, true, VEC>.
+template <typename T, int ROWS, int BK, int PF>
+struct PaddedRowsStager : TileLayout<T, ROWS, BK, true> {
+    using L = TileLayout<T, ROWS, BK, true>;
+    static constexpr int VEC = Mfma<T>::VK;
+    using V = typename Vec<T, VEC>::type;
+    static constexpr int kPF = PF;
+    static constexpr int VPL = BK / VEC;
+    static constexpr int RPP = kThreads / VPL;  // rows per pass
+    static constexpr int P = ROWS / RPP;
+    static_assert(BK % VEC == 0 && kThreads % VPL == 0 && ROWS % RPP == 0, "tile must split evenly");
+    V reg[PF][P];
+    int col0[PF];  // column x of the lane's vector in each slot
+    uint32_t row_off[P];
+    __amdgpu_buffer_rsrc_t rsrc;
+    FastDiv d_row;
+    int w, positions, k_local, row0, k_next;
+
+    // base: channel m0 of the image; plane = Ho * Wo; k0: first (padded) position of this workgroup's slice.
+    __device__ __forceinline__ void init(const T *base, int tid, int rows_left, const ConvGeom &geo, int k0) {
+        const int plane = geo.Ho * geo.Wo;
+        const int rows = rows_left < ROWS ? rows_left : ROWS;
+        rsrc = make_rsrc(base, static_cast<int64_t>(rows) * plane * static_cast<int64_t>(sizeof(T)));
+        d_row = geo.d_row_pad;
+        w = geo.Wo;
+        positions = geo.Ho * geo.row_pad;
+        k_local = (tid % VPL) * VEC;
+        row0 = tid / VPL;
+        k_next = k0;
+#pragma unroll
+        for (int p = 0; p < P; ++p) {
+            const int r = p * RPP + row0;
+            row_off[p] = r < rows ? static_cast<uint32_t>(r * plane) * static_cast<uint32_t>(sizeof(T)) : kOob;
+        }
+    }
+
+    template <bool MASK, int SLOT = 0>
+    __device__ __forceinline__ void load(int k_left) {
+        const int n = k_next + k_local;
+        // slices are whole k tiles and the padded rows whole vectors: a vector lies inside the slice or outside it
+        const bool ok = n < positions && k_local < k_left;
+        uint32_t y, x;
+        d_row.divmod(static_cast<uint32_t>(ok ? n : 0), y, x);
+        const uint32_t pos_b = (y * static_cast<uint32_t>(w) + x) * static_cast<uint32_t>(sizeof(T));
+#pragma unroll
+        for (int p = 0; p < P; ++p) reg[SLOT][p] = Vec<T, VEC>::load(rsrc, (ok && row_off[p] != kOob) ? row_off[p] + pos_b : kOob);
+        col0[SLOT] = static_cast<int>(x);
+        k_next += BK;
+    }
+
+    template <int SLOT = 0>
+    __device__ __forceinline__ void store(T *lds) const {
+#pragma unroll
         for (int p = 0; p < P; ++p)
-            *reinterpret_cast<V *>(&lds[(p * RPP + row0) * L::LD + k_local]) =
-                clear_outside_row<T, VEC>(reg[SLOT][p], col0[SLOT] + dx[p], tv.src_w);
+            *reinterpret_cast<V *>(&lds[(p * RPP + row0) * L::LD + k_local]) = clear_outside_row<T, VEC>(reg[SLOT][p], col0[SLOT], w);
     }
 };
 
@@ -605,12 +673,13 @@ conv_dgrad_kernel(ConvGeom geo, const T *gout, const T *wt, T *gin, int tiles_m,
 // grad_weight: M = O, N = C*k*k, K = Ho*Wo per image.  Workgroup column `part` = (image group, k slice)
 // accumulates slice [k0, k0 + k_chunk) of images [grp*group, min(B, (grp+1)*group)) in registers and writes one
 // partial tile; k_chunk is a multiple of BK.
-template <typename T, int BK, int A_VEC, class StB>
+// PADDED: the positions are numbered over padded rows (geo.row_pad != 0), K = Ho * row_pad.
+template <typename T, int BK, int A_VEC, class StB, bool PADDED = false>
 __global__ void __launch_bounds__(kThreads, 2)
 conv_wgrad_kernel(ConvGeom geo, const T *gout, const T *x, T *partial, int64_t image_bytes, int group, int kslices, int k_chunk,
                   int tiles_m, int tiles_n) {
     constexpr int BM = 64, BN = 64;
-    using StA = Stager<T, BM, BK, true, A_VEC, kConvPF>;
+    using StA = std::conditional_t<PADDED, PaddedRowsStager<T, BM, BK, kConvPF>, Stager<T, BM, BK, true, A_VEC, kConvPF>>;
     using Engine = ConvEngine<T, BM, BN, BK, StA, StB>;
     extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
     T *const smem = reinterpret_cast<T *>(smem_raw);
@@ -618,10 +687,11 @@ conv_wgrad_kernel(ConvGeom geo, const T *gout, const T *x, T *partial, int64_t i
     int part, tm, tn;
     decode_tile(remap_xcd(blockIdx.x, gridDim.x), tiles_m, tiles_n, part, tm, tn);
     const int m0 = tm * BM, n0 = tn * BN;
-    const int M_ = geo.O, N_ = geo.C * geo.k * geo.k, K = geo.Ho * geo.Wo;
+    const int plane = geo.Ho * geo.Wo;
+    const int M_ = geo.O, N_ = geo.C * geo.k * geo.k, K = PADDED ? geo.Ho * geo.row_pad : plane;
     const int grp = part / kslices, k0 = (part - grp * kslices) * k_chunk;
     const int k_len = K - k0 < k_chunk ? K - k0 : k_chunk;
-    const int64_t g_image = static_cast<int64_t>(geo.O) * K;
+    const int64_t g_image = static_cast<int64_t>(geo.O) * plane;
     StA sa;
     StB sb(geo);
     sb.init(tid, n0);
@@ -629,7 +699,8 @@ conv_wgrad_kernel(ConvGeom geo, const T *gout, const T *x, T *partial, int64_t i
     eng.init(tid);
     const int b_end = (grp + 1) * group < geo.B ? (grp + 1) * group : geo.B;
     for (int b = grp * group; b < b_end; ++b) {
-        sa.init(gout + b * g_image + static_cast<int64_t>(m0) * K + k0, tid, M_ - m0, K, 1, k_len);
+        if constexpr (PADDED) sa.init(gout + b * g_image + static_cast<int64_t>(m0) * plane, tid, M_ - m0, geo, k0);
+        else sa.init(gout + b * g_image + static_cast<int64_t>(m0) * K + k0, tid, M_ - m0, K, 1, k_len);
         sb.set_image(x + static_cast<int64_t>(b) * geo.xs_b, image_bytes, k0);
         eng.run(sa, sb, smem, k_len, false);
         __syncthreads();  // the next image's prologue overwrites LDS buffer 0
@@ -907,12 +978,11 @@ constexpr size_t conv_lds_bytes() {
 // Rows of `width` positions that are no whole number of 16-byte vectors: the padded row width with which the
 // 16-byte gathers serve them, or 0 where the narrower gathers stay ahead (the padding columns are wasted work: at
 // most a fifth more of it against the 8-byte gathers of an even width, at most double against element loads).
-template <typename T>
-int padded_row_width(int width) {
-    constexpr int VK = Mfma<T>::VK;
+int padded_row_width(size_t esz, int width) {
+    const int VK = static_cast<int>(16 / esz);
     if (width % VK == 0) return 0;
     const int padded = (width + VK - 1) / VK * VK;
-    const bool pairs = sizeof(T) == 4 && width % 2 == 0;
+    const bool pairs = esz == 4 && width % 2 == 0;
     return (pairs ? 5 * padded <= 6 * width : padded <= 2 * width) ? padded : 0;
 }
 
@@ -922,7 +992,7 @@ ttamd_status forward_mfma_tile(const ConvPlan &pl, const void *bias, void *out, 
     ConvGeom g = pl.geo;
     const bool a_vec = rows_vectorizable<T>(pl.w, g.w_so, 0);
     if (a_vec && g.S == 1 && g.xs_w == 1) {
-        g.row_pad = padded_row_width<T>(g.Wo);
+        g.row_pad = padded_row_width(sizeof(T), g.Wo);
         g.d_row_pad = make_fastdiv(static_cast<uint32_t>(g.row_pad ? g.row_pad : 1));
     }
     const int M_ = g.O, N_ = g.Ho * (g.row_pad ? g.row_pad : g.Wo);
@@ -1038,7 +1108,13 @@ inline int bias_grad_parts(int O, int64_t vectors) {
     return parts < 1 ? 1 : static_cast<int>(parts);
 }
 
-BackwardWorkspace backward_workspace(size_t esz, int B, int C, int H, int W, int O, int k, int stride, int padding) {
+// wgrad_padded: grad_weight numbers its reduction over padded rows (wgrad_pads_rows and a unit column stride of the
+// input); the workspace query, which does not see the strides, takes the larger of the two plans.
+bool wgrad_pads_rows(size_t esz, int H, int W, int k, int stride, int padding) {
+    return stride == 1 && padded_row_width(esz, (W + 2 * padding - k) / stride + 1) != 0;
+}
+
+BackwardWorkspace backward_workspace(size_t esz, int B, int C, int H, int W, int O, int k, int stride, int padding, bool wgrad_padded) {
     BackwardWorkspace w{};
     const size_t tile = static_cast<size_t>(O) * C * k * k * esz;
     w.wt_bytes = (tile + 255) & ~static_cast<size_t>(255);
@@ -1051,7 +1127,7 @@ BackwardWorkspace backward_workspace(size_t esz, int B, int C, int H, int W, int
     w.splits = (B + w.group - 1) / w.group;
     const int bk = esz == 4 ? 32 : 16;
     const int Ho = (H + 2 * padding - k) / stride + 1, Wo = (W + 2 * padding - k) / stride + 1;
-    const int64_t K = static_cast<int64_t>(Ho) * Wo;
+    const int64_t K = static_cast<int64_t>(Ho) * (wgrad_padded ? padded_row_width(esz, Wo) : Wo);
     const int64_t k_tiles = (K + bk - 1) / bk;
     const int64_t tiles = static_cast<int64_t>((O + 63) / 64) * ((static_cast<int64_t>(C) * k * k + 63) / 64);
     // Slices of the reduction: the launch is as slow as its busiest CU, which runs ceil(workgroups / 256) of them,
@@ -1094,7 +1170,8 @@ ttamd_status backward_mfma(const ConvPlan &pl, const void *gout, void *gin, void
     constexpr int BK = ConvTiles<T>::BK, VK = Mfma<T>::VK;
     const ConvGeom &g = pl.geo;
     const int HoWo = g.Ho * g.Wo;
-    const BackwardWorkspace plan = backward_workspace(sizeof(T), g.B, g.C, g.H, g.W, g.O, g.k, g.S, g.P);
+    const bool wgrad_padded = g.xs_w == 1 && wgrad_pads_rows(sizeof(T), g.H, g.W, g.k, g.S, g.P);
+    const BackwardWorkspace plan = backward_workspace(sizeof(T), g.B, g.C, g.H, g.W, g.O, g.k, g.S, g.P, wgrad_padded);
     if (!ws || ws_bytes < plan.total()) {
         set_error("conv2d_backward: workspace of %zu bytes is smaller than the %zu bytes required", ws_bytes, plan.total());
         return TTAMD_ERR_INVALID_ARGUMENT;
@@ -1135,7 +1212,7 @@ ttamd_status backward_mfma(const ConvPlan &pl, const void *gout, void *gin, void
             T *gin = dst;
             const bool a_vec = rows_vectorizable<T>(wt, Kd, 0);
             if (a_vec && g.S == 1) {
-                g.row_pad = padded_row_width<T>(g.W);
+                g.row_pad = padded_row_width(sizeof(T), g.W);
                 g.d_row_pad = make_fastdiv(static_cast<uint32_t>(g.row_pad ? g.row_pad : 1));
             }
             const int M_ = g.C, N_ = g.H * (g.row_pad ? g.row_pad : g.W);
@@ -1209,8 +1286,13 @@ ttamd_status backward_mfma(const ConvPlan &pl, const void *gout, void *gin, void
         const int64_t blocks = static_cast<int64_t>(tiles_m) * tiles_n * parts;
         const bool a_vec = rows_vectorizable<T>(gout, HoWo, static_cast<int64_t>(g.O) * HoWo);
         const bool b_vec = g.S == 1 && g.xs_w == 1 && g.Wo % VK == 0;
+        ConvGeom gw_geo = g;
+        if (wgrad_padded) {
+            gw_geo.row_pad = padded_row_width(sizeof(T), g.Wo);
+            gw_geo.d_row_pad = make_fastdiv(static_cast<uint32_t>(gw_geo.row_pad));
+        }
         auto go = [&](auto kernel, size_t lds) {
-            return launch_conv(kernel, lds, blocks, st, g, static_cast<const T *>(gout), static_cast<const T *>(pl.x), partial,
+            return launch_conv(kernel, lds, blocks, st, gw_geo, static_cast<const T *>(gout), static_cast<const T *>(pl.x), partial,
                                pl.image_bytes, plan.group, plan.kslices, plan.k_chunk, tiles_m, tiles_n);
         };
         using VecB = TapStagerKC<T, 64, BK, VK, kConvPF>;
@@ -1218,7 +1300,9 @@ ttamd_status backward_mfma(const ConvPlan &pl, const void *gout, void *gin, void
         ttamd_status s;
         bool pair = false;
         if constexpr (sizeof(T) == 4) pair = a_vec && !b_vec && g.S == 1 && g.xs_w == 1 && g.Wo % 2 == 0;
-        if (a_vec && b_vec) s = go(conv_wgrad_kernel<T, BK, VK, VecB>, conv_lds_bytes<T, 64, 64, VK, VecB>());
+        using PaddedB = TapStagerKC<T, 64, BK, VK, kConvPF, true>;
+        if (wgrad_padded) s = go(conv_wgrad_kernel<T, BK, VK, PaddedB, true>, conv_lds_bytes<T, 64, 64, VK, PaddedB>());
+        else if (a_vec && b_vec) s = go(conv_wgrad_kernel<T, BK, VK, VecB>, conv_lds_bytes<T, 64, 64, VK, VecB>());
         else if (pair) {
             if constexpr (sizeof(T) == 4) {
                 using PairB = TapStagerKC<T, 64, BK, 2, kConvPF>;
@@ -1310,7 +1394,12 @@ ttamd_status ttamd_conv2d_backward_workspace(ttamd_dtype dtype, int B, int C, in
     if (B <= 0 || C <= 0 || O <= 0 || k <= 0 || H <= 0 || W <= 0 || stride <= 0 || padding < 0 || H + 2 * padding < k ||
         W + 2 * padding < k)
         return TTAMD_OK;  // ttamd_conv2d_backward rejects the geometry itself
-    *bytes = backward_workspace(dtype_size(dtype), B, C, H, W, O, k, stride, padding).total();
+    const size_t esz = dtype_size(dtype);
+    *bytes = backward_workspace(esz, B, C, H, W, O, k, stride, padding, false).total();
+    if (wgrad_pads_rows(esz, H, W, k, stride, padding)) {
+        const size_t padded = backward_workspace(esz, B, C, H, W, O, k, stride, padding, true).total();
+        if (padded > *bytes) *bytes = padded;
+    }
     return TTAMD_OK;
 }
 
