@@ -149,6 +149,28 @@ def test_grad_bias_in_parts_exact(tt, dtype, geom):
 
 
 @pytest.mark.parametrize("dtype", [np.float32, np.float64])
+@pytest.mark.parametrize("W", [7, 14])
+def test_padding_columns_of_padded_rows_carry_nothing(tt, oracle, dtype, W):
+    """Rows of 7 or 14 positions are numbered over 8 or 16 columns.  An infinite input value in the last column must
+    reach exactly the sums that the reference's windows give it: a padding column that multiplied it by zero would
+    leave a NaN in a tap whose real windows never touch that pixel."""
+    rng = np.random.default_rng(W)
+    Bn, Cc, O, k = 2, 8, 8, 3
+    x = rng.integers(-2, 3, (Bn, Cc, W + 2, W + 2)).astype(dtype)  # no padding: the output rows have W positions
+    x[0, 1, 3, W + 1] = np.inf
+    w = rng.integers(1, 4, (O, Cc, k, k)).astype(dtype)
+    out = tt.conv2d(dev(tt, x), dev(tt, w), None, 1, 0).to_numpy()
+    want = oracle.conv2d_forward(x, w, None, 1, 0)
+    assert out.shape[3] == W and np.isinf(want).any() and not np.isnan(want).any()
+    assert np.array_equal(out, want)
+    g = rng.integers(1, 4, want.shape).astype(dtype)  # positive: every sum that meets the infinity is +inf, none NaN
+    gx, gw, _ = tt.conv2d_backward(dev(tt, g), dev(tt, x), dev(tt, w), None, 1, 0)
+    wx, ww, _ = oracle.conv2d_backward(g, x, w, False, 1, 0)
+    assert np.isinf(ww).any() and not np.isnan(ww).any() and np.isfinite(ww[:, :, :, :2]).all()
+    assert np.array_equal(gw.to_numpy(), ww) and np.array_equal(gx.to_numpy(), wx)
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
 def test_unaligned_window_of_a_larger_image(tt, oracle, dtype):
     # the input is a window [1:9, 3:15] of a stored [2,3,10,20] tensor: rows start at odd element offsets,
     # so every 16-byte gather is unaligned, and the elements around the window are non-zero
