@@ -108,6 +108,8 @@ def test_backward_exact_on_integer_data_and_adjoints(tt, oracle, dtype):
     # the way out): odd widths, widths of 4n + 2, several position tiles per image, a tile that ends inside a row
     (2, 8, 8, 7, 7, 3, 1), (1, 8, 8, 5, 5, 3, 1), (2, 8, 8, 3, 3, 3, 1), (1, 8, 8, 26, 26, 3, 0), (2, 4, 8, 9, 7, 5, 2),
     (1, 8, 8, 41, 37, 3, 1), (2, 40, 70, 15, 14, 3, 1), (1, 8, 40, 23, 30, 3, 1),
+    # small images: grad_weight runs several of them through one reduction (groups of images, a ragged last group)
+    (40, 70, 66, 6, 4, 3, 1), (13, 70, 66, 7, 7, 3, 1), (9, 8, 8, 10, 10, 3, 1), (5, 72, 8, 8, 8, 3, 1), (21, 66, 70, 5, 5, 3, 1),
 ])
 def test_unit_stride_vector_gathers_exact(tt, oracle, dtype, geom):
     Bn, Cc, O, H, W, k, P = geom

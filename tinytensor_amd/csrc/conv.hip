@@ -398,6 +398,9 @@ struct TapStagerKC : TileLayout<T, ROWS, BK, true> {
     int16_t dy[P], dx[P];
     bool j_ok[P];
     int k_local, row0, k_next;
+    // PADDED only: several images in one reduction.  Every image takes joint_k positions (its own, rounded up to whole
+    // k tiles; 0: one image per run), image_step elements apart; image_base is the current image's element offset.
+    int joint_k, image_step, image_base;
 
     __device__ __forceinline__ explicit TapStagerKC(const ConvGeom &geo) : tv(geo) {}
 
@@ -420,16 +423,34 @@ struct TapStagerKC : TileLayout<T, ROWS, BK, true> {
     __device__ __forceinline__ void set_image(const T *image, int64_t image_bytes, int k0) {
         rsrc = make_rsrc(image, image_bytes);
         k_next = k0;
+        joint_k = 0;
+        image_step = 0;
+        image_base = 0;
+    }
+
+    // The images from `first` on as one reduction: span_bytes covers them all, `step` elements from one to the next.
+    __device__ __forceinline__ void set_images(const T *first, int64_t span_bytes, int positions_per_image, int32_t step) {
+        rsrc = make_rsrc(first, span_bytes);
+        k_next = 0;
+        joint_k = positions_per_image;
+        image_step = step;
+        image_base = 0;
     }
 
     template <bool MASK, int SLOT = 0>
     __device__ __forceinline__ void load(int /*k_left*/) {
+        if constexpr (PADDED) {
+            if (joint_k && k_next >= joint_k) {  // uniform: the next image starts with this tile
+                k_next -= joint_k;
+                image_base += image_step;
+            }
+        }
         const int n = k_next + k_local;
         const bool n_ok = n < tv.positions;
         uint32_t y, x;
         tv.d_pw.divmod(static_cast<uint32_t>(n_ok ? n : 0), y, x);
         const int py = static_cast<int>(y), px0 = static_cast<int>(x);
-        const int32_t base = py * tv.s_h + px0;
+        const int32_t base = (PADDED ? image_base : 0) + py * tv.s_h + px0;
 #pragma unroll
         for (int p = 0; p < P; ++p) {
             const int yy = py + dy[p];
@@ -472,12 +493,20 @@ struct PaddedRowsStager : TileLayout<T, ROWS, BK, true> {
     __amdgpu_buffer_rsrc_t rsrc;
     FastDiv d_row;
     int w, positions, k_local, row0, k_next;
+    int joint_k;                     // several images in one reduction: positions per image (whole k tiles), or 0
+    uint32_t image_step_b, image_b;  // bytes from one image to the next, byte offset of the current image
 
-    // base: channel m0 of the image; plane = Ho * Wo; k0: first (padded) position of this workgroup's slice.
-    __device__ __forceinline__ void init(const T *base, int tid, int rows_left, const ConvGeom &geo, int k0) {
+    // base: channel m0 of the (first) image; k0: first (padded) position of this workgroup's slice.  images > 1 with
+    // positions_per_image (a multiple of BK) runs through that many images in one reduction.
+    __device__ __forceinline__ void init(const T *base, int tid, int rows_left, const ConvGeom &geo, int k0, int images = 1,
+                                         int positions_per_image = 0) {
         const int plane = geo.Ho * geo.Wo;
         const int rows = rows_left < ROWS ? rows_left : ROWS;
-        rsrc = make_rsrc(base, static_cast<int64_t>(rows) * plane * static_cast<int64_t>(sizeof(T)));
+        const int64_t image_elems = static_cast<int64_t>(geo.O) * plane;
+        rsrc = make_rsrc(base, ((images - 1) * image_elems + static_cast<int64_t>(rows) * plane) * static_cast<int64_t>(sizeof(T)));
+        joint_k = positions_per_image;
+        image_step_b = static_cast<uint32_t>(image_elems * static_cast<int64_t>(sizeof(T)));
+        image_b = 0;
         d_row = geo.d_row_pad;
         w = geo.Wo;
         positions = geo.Ho * geo.row_pad;
@@ -493,12 +522,16 @@ struct PaddedRowsStager : TileLayout<T, ROWS, BK, true> {
 
     template <bool MASK, int SLOT = 0>
     __device__ __forceinline__ void load(int k_left) {
+        if (joint_k && k_next >= joint_k) {  // uniform: the next image starts with this tile
+            k_next -= joint_k;
+            image_b += image_step_b;
+        }
         const int n = k_next + k_local;
         // slices are whole k tiles and the padded rows whole vectors: a vector lies inside the slice or outside it
         const bool ok = n < positions && k_local < k_left;
         uint32_t y, x;
         d_row.divmod(static_cast<uint32_t>(ok ? n : 0), y, x);
-        const uint32_t pos_b = (y * static_cast<uint32_t>(w) + x) * static_cast<uint32_t>(sizeof(T));
+        const uint32_t pos_b = image_b + (y * static_cast<uint32_t>(w) + x) * static_cast<uint32_t>(sizeof(T));
 #pragma unroll
         for (int p = 0; p < P; ++p) reg[SLOT][p] = Vec<T, VEC>::load(rsrc, (ok && row_off[p] != kOob) ? row_off[p] + pos_b : kOob);
         col0[SLOT] = static_cast<int>(x);
@@ -673,11 +706,13 @@ conv_dgrad_kernel(ConvGeom geo, const T *gout, const T *wt, T *gin, int tiles_m,
 // grad_weight: M = O, N = C*k*k, K = Ho*Wo per image.  Workgroup column `part` = (image group, k slice)
 // accumulates slice [k0, k0 + k_chunk) of images [grp*group, min(B, (grp+1)*group)) in registers and writes one
 // partial tile; k_chunk is a multiple of BK.
-// PADDED: the positions are numbered over padded rows (geo.row_pad != 0), K = Ho * row_pad.
+// PADDED: the positions are numbered over padded rows (geo.row_pad != 0), K = Ho * row_pad.  With joint_k != 0
+// (PADDED only, kslices = 1) the group's images form one reduction of joint_k positions each, an image's own rounded up
+// to whole k tiles: small images then share one run of the pipeline instead of filling and draining it per image.
 template <typename T, int BK, int A_VEC, class StB, bool PADDED = false>
 __global__ void __launch_bounds__(kThreads, 2)
 conv_wgrad_kernel(ConvGeom geo, const T *gout, const T *x, T *partial, int64_t image_bytes, int group, int kslices, int k_chunk,
-                  int tiles_m, int tiles_n) {
+                  int tiles_m, int tiles_n, int joint_k) {
     constexpr int BM = 64, BN = 64;
     using StA = std::conditional_t<PADDED, PaddedRowsStager<T, BM, BK, kConvPF>, Stager<T, BM, BK, true, A_VEC, kConvPF>>;
     using Engine = ConvEngine<T, BM, BN, BK, StA, StB>;
@@ -698,7 +733,18 @@ conv_wgrad_kernel(ConvGeom geo, const T *gout, const T *x, T *partial, int64_t i
     Engine eng;
     eng.init(tid);
     const int b_end = (grp + 1) * group < geo.B ? (grp + 1) * group : geo.B;
-    for (int b = grp * group; b < b_end; ++b) {
+    bool joint = false;
+    if constexpr (PADDED) {
+        if (joint_k) {
+            joint = true;
+            const int b0 = grp * group, images = b_end - b0;
+            sa.init(gout + b0 * g_image + static_cast<int64_t>(m0) * plane, tid, M_ - m0, geo, 0, images, joint_k);
+            sb.set_images(x + static_cast<int64_t>(b0) * geo.xs_b, (images - 1) * geo.xs_b * static_cast<int64_t>(sizeof(T)) + image_bytes,
+                          joint_k, static_cast<int32_t>(geo.xs_b));
+            eng.run(sa, sb, smem, images * joint_k, false);
+        }
+    }
+    for (int b = grp * group; b < b_end && !joint; ++b) {
         if constexpr (PADDED) sa.init(gout + b * g_image + static_cast<int64_t>(m0) * plane, tid, M_ - m0, geo, k0);
         else sa.init(gout + b * g_image + static_cast<int64_t>(m0) * K + k0, tid, M_ - m0, K, 1, k_len);
         sb.set_image(x + static_cast<int64_t>(b) * geo.xs_b, image_bytes, k0);
@@ -725,6 +771,43 @@ __global__ void __launch_bounds__(256) reduce_splits_kernel(const T *__restrict_
         __syncthreads();
     }
     if (lane_s == 0 && i < n) out[i] = red[0][e];
+}
+
+// The same sum for long outputs: one lane per 16-byte vector of out adds its parts in increasing order, every load a
+// whole coalesced line of the wave (the kernel above reads 64 bytes per part and workgroup, and with few parts most of
+// its lanes have nothing to add).  n is a multiple of the vector length; partial and out are 16-byte aligned.
+template <typename T>
+__global__ void __launch_bounds__(256) reduce_splits_stream_kernel(const T *__restrict__ partial, T *__restrict__ out, int64_t n, int splits) {
+    using V = std::conditional_t<sizeof(T) == 4, float4, double2>;
+    constexpr int VEC = sizeof(V) / sizeof(T);
+    const int64_t i = (static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x) * VEC;
+    if (i >= n) return;
+    V acc = *reinterpret_cast<const V *>(partial + i);
+    T *a = reinterpret_cast<T *>(&acc);
+#pragma unroll 4
+    for (int s = 1; s < splits; ++s) {
+        const V v = *reinterpret_cast<const V *>(partial + static_cast<int64_t>(s) * n + i);
+        const T *e = reinterpret_cast<const T *>(&v);
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) a[j] += e[j];
+    }
+    *reinterpret_cast<V *>(out + i) = acc;
+}
+
+// out[i] = sum over parts of partial[s][i], by whichever of the two kernels suits the shape: the streaming one when
+// there are enough vectors to fill the chip or too few parts to occupy the other's sixteen lanes per element.
+template <typename T>
+ttamd_status launch_reduce_splits(const T *partial, T *out, int64_t n, int splits, hipStream_t st) {
+    constexpr int VEC = 16 / sizeof(T);
+    const bool aligned = n % VEC == 0 && reinterpret_cast<uintptr_t>(partial) % 16 == 0 && reinterpret_cast<uintptr_t>(out) % 16 == 0;
+    if (aligned && (n / VEC >= 65536 || splits <= 8)) {
+        const int64_t blocks = (n / VEC + 255) / 256;
+        reduce_splits_stream_kernel<T><<<dim3(static_cast<unsigned>(blocks)), dim3(256), 0, st>>>(partial, out, n, splits);
+    } else {
+        reduce_splits_kernel<T><<<dim3(static_cast<unsigned>((n + 15) / 16)), dim3(256), 0, st>>>(partial, out, n, splits);
+    }
+    TTAMD_HIP_CHECK(hipGetLastError());
+    return TTAMD_OK;
 }
 
 // grad_bias[o] = sum over batch and space of grad_out[b][o][.] (cpu/conv.cpp:289), in two steps so that the launch
@@ -1114,7 +1197,24 @@ bool wgrad_pads_rows(size_t esz, int H, int W, int k, int stride, int padding) {
     return stride == 1 && padded_row_width(esz, (W + 2 * padding - k) / stride + 1) != 0;
 }
 
-BackwardWorkspace backward_workspace(size_t esz, int B, int C, int H, int W, int O, int k, int stride, int padding, bool wgrad_padded) {
+// Images of at most this many k tiles (their positions numbered over rows of whole vectors) go through grad_weight's
+// reduction several at a time.
+constexpr int kJointTiles = 4;
+
+// Positions per image in that joint reduction (whole k tiles), or 0 where it does not apply.
+int wgrad_joint_positions(size_t esz, int H, int W, int k, int stride, int padding) {
+    if (stride != 1) return 0;
+    const int Ho = H + 2 * padding - k + 1, Wo = W + 2 * padding - k + 1;
+    const int vk = static_cast<int>(16 / esz), bk = esz == 4 ? 32 : 16;
+    const int row = Wo % vk == 0 ? Wo : padded_row_width(esz, Wo);
+    if (row == 0) return 0;
+    const int tiles = (Ho * row + bk - 1) / bk;
+    return tiles <= kJointTiles ? tiles * bk : 0;
+}
+
+// wgrad_mode: 0 positions as they are, 1 over padded rows, 2 over rows of whole vectors with several images per reduction.
+BackwardWorkspace backward_workspace(size_t esz, int B, int C, int H, int W, int O, int k, int stride, int padding, int wgrad_mode) {
+    const bool wgrad_padded = wgrad_mode == 1;
     BackwardWorkspace w{};
     const size_t tile = static_cast<size_t>(O) * C * k * k * esz;
     w.wt_bytes = (tile + 255) & ~static_cast<size_t>(255);
@@ -1153,6 +1253,34 @@ BackwardWorkspace backward_workspace(size_t esz, int B, int C, int H, int W, int
     w.k_chunk = static_cast<int>(chunk_tiles * bk);
     w.kslices = static_cast<int>((k_tiles + chunk_tiles - 1) / chunk_tiles);
     if (w.kslices < 1) w.kslices = 1;
+    if (wgrad_mode == 2) {
+        // Groups of images instead of slices of one: same cost model, a workgroup runs its group's k tiles in one go.
+        // A group's grad_out and (dense) input stay inside the 2 GiB that one buffer descriptor addresses.
+        const int joint_k = wgrad_joint_positions(esz, H, W, k, stride, padding);
+        const int64_t tpi = joint_k / bk;
+        const int64_t image_bytes = static_cast<int64_t>(esz) * (static_cast<int64_t>(O) * Ho * Wo > static_cast<int64_t>(C) * H * W
+                                                                      ? static_cast<int64_t>(O) * Ho * Wo : static_cast<int64_t>(C) * H * W);
+        int64_t max_group = (0x7fffffffLL / (image_bytes ? image_bytes : 1)) - 1;
+        if (max_group < 1) max_group = 1;
+        int64_t max_parts = (64LL << 20) / static_cast<int64_t>(tile ? tile : 1);
+        if (max_parts < 1) max_parts = 1;
+        int best_group = 0;
+        for (int64_t want = 1; want <= B; ++want) {
+            const int64_t group = (B + want - 1) / want, parts = (B + group - 1) / group;
+            if (group > max_group || parts > max_parts) continue;
+            const double cost = static_cast<double>((tiles * parts + 255) / 256) * static_cast<double>(group * tpi + 3) * 0.6 +
+                                (parts > 1 ? static_cast<double>(parts) * static_cast<double>(tile) / 4e6 : 0.0);
+            if (best_group == 0 || cost < best) {
+                best = cost;
+                best_group = static_cast<int>(group);
+            }
+        }
+        if (best_group == 0) best_group = static_cast<int>(max_group < B ? max_group : B);
+        w.group = best_group;
+        w.splits = (B + w.group - 1) / w.group;
+        w.kslices = 1;
+        w.k_chunk = joint_k;
+    }
     w.partial_bytes = w.parts() > 1 ? static_cast<size_t>(w.parts()) * tile : 0;
     w.partial_bytes = (w.partial_bytes + 255) & ~static_cast<size_t>(255);
     w.bias_bytes = static_cast<size_t>(kBiasGradParts) * O * esz;
@@ -1170,8 +1298,15 @@ ttamd_status backward_mfma(const ConvPlan &pl, const void *gout, void *gin, void
     constexpr int BK = ConvTiles<T>::BK, VK = Mfma<T>::VK;
     const ConvGeom &g = pl.geo;
     const int HoWo = g.Ho * g.Wo;
-    const bool wgrad_padded = g.xs_w == 1 && wgrad_pads_rows(sizeof(T), g.H, g.W, g.k, g.S, g.P);
-    const BackwardWorkspace plan = backward_workspace(sizeof(T), g.B, g.C, g.H, g.W, g.O, g.k, g.S, g.P, wgrad_padded);
+    int wgrad_mode = g.xs_w == 1 && wgrad_pads_rows(sizeof(T), g.H, g.W, g.k, g.S, g.P) ? 1 : 0;
+    const int joint_k = g.xs_w == 1 ? wgrad_joint_positions(sizeof(T), g.H, g.W, g.k, g.S, g.P) : 0;
+    if (joint_k) {
+        const BackwardWorkspace jp = backward_workspace(sizeof(T), g.B, g.C, g.H, g.W, g.O, g.k, g.S, g.P, 2);
+        // the group's input images under one descriptor, the image behind the last one addressable too
+        if ((static_cast<int64_t>(jp.group) + 1) * g.xs_b * static_cast<int64_t>(sizeof(T)) < 0x7fffffffLL) wgrad_mode = 2;
+    }
+    const bool wgrad_padded = wgrad_mode != 0;
+    const BackwardWorkspace plan = backward_workspace(sizeof(T), g.B, g.C, g.H, g.W, g.O, g.k, g.S, g.P, wgrad_mode);
     if (!ws || ws_bytes < plan.total()) {
         set_error("conv2d_backward: workspace of %zu bytes is smaller than the %zu bytes required", ws_bytes, plan.total());
         return TTAMD_ERR_INVALID_ARGUMENT;
@@ -1288,12 +1423,12 @@ ttamd_status backward_mfma(const ConvPlan &pl, const void *gout, void *gin, void
         const bool b_vec = g.S == 1 && g.xs_w == 1 && g.Wo % VK == 0;
         ConvGeom gw_geo = g;
         if (wgrad_padded) {
-            gw_geo.row_pad = padded_row_width(sizeof(T), g.Wo);
+            gw_geo.row_pad = g.Wo % VK == 0 ? g.Wo : padded_row_width(sizeof(T), g.Wo);  // whole vectors already: joint mode only
             gw_geo.d_row_pad = make_fastdiv(static_cast<uint32_t>(gw_geo.row_pad));
         }
         auto go = [&](auto kernel, size_t lds) {
             return launch_conv(kernel, lds, blocks, st, gw_geo, static_cast<const T *>(gout), static_cast<const T *>(pl.x), partial,
-                               pl.image_bytes, plan.group, plan.kslices, plan.k_chunk, tiles_m, tiles_n);
+                               pl.image_bytes, plan.group, plan.kslices, plan.k_chunk, tiles_m, tiles_n, wgrad_mode == 2 ? joint_k : 0);
         };
         using VecB = TapStagerKC<T, 64, BK, VK, kConvPF>;
         using OneB = Im2colTStager<T, 64, BK, kConvPF>;
@@ -1314,11 +1449,8 @@ ttamd_status backward_mfma(const ConvPlan &pl, const void *gout, void *gin, void
         else if (b_vec) s = go(conv_wgrad_kernel<T, BK, 1, VecB>, conv_lds_bytes<T, 64, 64, 1, VecB>());
         else s = go(conv_wgrad_kernel<T, BK, 1, OneB>, conv_lds_bytes<T, 64, 64, 1, OneB>());
         if (s) return s;
-        if (parts > 1) {
-            const int64_t rb = (tile_elems + 15) / 16;
-            reduce_splits_kernel<T><<<dim3(static_cast<unsigned>(rb)), dim3(256), 0, st>>>(partial, static_cast<T *>(gw), tile_elems, parts);
-            TTAMD_HIP_CHECK(hipGetLastError());
-        }
+        if (parts > 1)
+            if (ttamd_status rc = launch_reduce_splits<T>(partial, static_cast<T *>(gw), tile_elems, parts, st)) return rc;
     }
     if (gb) {
         using V = std::conditional_t<sizeof(T) == 4, float4, double2>;
@@ -1340,10 +1472,8 @@ ttamd_status backward_mfma(const ConvPlan &pl, const void *gout, void *gin, void
         else
             bias_grad_kernel<T, T><<<grid, dim3(256), 0, st>>>(static_cast<const T *>(gout), sums, g.O, HoWo, static_cast<uint32_t>(total), chunk, d);
         TTAMD_HIP_CHECK(hipGetLastError());
-        if (bparts > 1) {
-            reduce_splits_kernel<T><<<dim3(static_cast<unsigned>((g.O + 15) / 16)), dim3(256), 0, st>>>(sums, static_cast<T *>(gb), g.O, bparts);
-            TTAMD_HIP_CHECK(hipGetLastError());
-        }
+        if (bparts > 1)
+            if (ttamd_status rc = launch_reduce_splits<T>(sums, static_cast<T *>(gb), g.O, bparts, st)) return rc;
     }
     return TTAMD_OK;
 }
@@ -1395,10 +1525,14 @@ ttamd_status ttamd_conv2d_backward_workspace(ttamd_dtype dtype, int B, int C, in
         W + 2 * padding < k)
         return TTAMD_OK;  // ttamd_conv2d_backward rejects the geometry itself
     const size_t esz = dtype_size(dtype);
-    *bytes = backward_workspace(esz, B, C, H, W, O, k, stride, padding, false).total();
+    *bytes = backward_workspace(esz, B, C, H, W, O, k, stride, padding, 0).total();
     if (wgrad_pads_rows(esz, H, W, k, stride, padding)) {
-        const size_t padded = backward_workspace(esz, B, C, H, W, O, k, stride, padding, true).total();
+        const size_t padded = backward_workspace(esz, B, C, H, W, O, k, stride, padding, 1).total();
         if (padded > *bytes) *bytes = padded;
+    }
+    if (wgrad_joint_positions(esz, H, W, k, stride, padding)) {
+        const size_t joint = backward_workspace(esz, B, C, H, W, O, k, stride, padding, 2).total();
+        if (joint > *bytes) *bytes = joint;
     }
     return TTAMD_OK;
 }
