@@ -34,9 +34,13 @@
  *   tto_splitmix64 / xorshift64  published test vectors (Vigna's splitmix64.c
  *                         seed 1234567 stream; xorshift64 13/7/17 closed form).
  *   tto_uniform_real_*    closed form from the bit construction.
- *   tto_normal_*          depends on libm log1p/sin/sqrt: values are generated
- *                         once on the host and handed to both sides; parity
- *                         unpinned across libm versions (statistical checks only).
+ *   tto_normal_*          closed form: every element's (u1, u2) rebuilt from the integer
+ *                         generator and mu + std*sqrt(-2*log1p(-u1))*sin(2*pi*u2) evaluated
+ *                         with 200-bit transcendentals, each step rounded to the type; f32
+ *                         within 2 ulp, f64 within 4 ulp of std*z, with negative controls
+ *                         (cos for sin, u1/u2 swapped, log(u1)) that must miss the bound.
+ *                         The last bits depend on libm's log1p/sin, so inputs drawn from it
+ *                         are generated once on the host and handed to both sides.
  */
 #ifndef TT_ORACLE_H_
 #define TT_ORACLE_H_

@@ -77,12 +77,104 @@ def test_uniform_real_statistics(oracle):
 
 
 def test_normal_statistics(oracle):
-    # Box-Muller values depend on libm; pinned statistically only (parity unpinned at the bit level).
     x = oracle.Generator(0).normal(0.0, 0.1, (200000,), np.float32).astype(np.float64)
     assert abs(x.mean()) < 2e-3 and abs(x.std() - 0.1) < 2e-3
     from scipy import stats
 
     assert stats.kstest(x, "norm", args=(0.0, 0.1)).statistic < 5e-3
+
+
+def _element_uniforms(oracle, seed, n, dtype):
+    """(u1, u2) of every element, rebuilt from the integer generator alone: element i owns a generator seeded with
+    master output i; its first output makes u1 and its second u2 (bit construction of uniform_real_sample with
+    low 0, high 1: r*(1-0)+0 == r exactly)."""
+    import ctypes as C
+
+    master = oracle.Generator(seed)
+    u = np.empty((n, 2), dtype=dtype)
+    for i in range(n):
+        st = C.c_uint64(master())
+        for j in range(2):
+            x = oracle.lib().tto_xorshift64(C.byref(st))
+            if dtype == np.float32:
+                b = np.array([((x & 0xFFFFFFFF) >> 9) | 0x3F800000], dtype=np.uint32).view(np.float32)[0]
+            else:
+                b = np.array([(x >> 12) | 0x3FF0000000000000], dtype=np.uint64).view(np.float64)[0]
+            u[i, j] = dtype(b - dtype(1.0))
+    return u, master.state
+
+
+def _box_muller_model(u1, u2, mu, std, dtype, variant="reference"):
+    """mu + std*sqrt(-2*log1p(-u1))*sin(2*pi*u2) with every transcendental evaluated to 200 bits (mpmath) and each
+    operation's result rounded to `dtype`, as code working in that type does.  Returns (value, std*z) as exact
+    mpmath numbers of dtype-representable values.  The variants are deliberate mistakes (negative controls)."""
+    import mpmath as mp
+
+    mp.mp.prec = 200
+
+    def rnd(v):  # round an mpmath number to dtype (to nearest even), back to mpmath
+        if dtype == np.float64:
+            return mp.mpf(float(v))  # mpf -> float rounds to nearest
+        d = float(v)  # 53-bit first; 200 -> 53 -> 24 double rounding matters only on exact ties of the 53-bit value
+        return mp.mpf(float(np.float32(d)))
+
+    a, b = mp.mpf(float(u1)), mp.mpf(float(u2))
+    if variant == "swapped":
+        a, b = b, a
+    if variant == "log_u1":
+        lg = rnd(mp.log(a)) if a > 0 else mp.mpf("-inf")
+    else:
+        lg = rnd(mp.log1p(-a))
+    r = rnd(mp.sqrt(-2 * lg))
+    two_pi = 2 * rnd(mp.pi)
+    theta = rnd(two_pi * b)
+    trig = rnd(mp.cos(theta)) if variant == "cos" else rnd(mp.sin(theta))
+    z = rnd(r * trig)
+    sz = rnd(mp.mpf(float(std)) * z)
+    return rnd(sz + mp.mpf(float(mu))), sz
+
+
+@pytest.mark.parametrize("dtype,ulps", [(np.float32, 2), (np.float64, 4)])
+def test_normal_closed_form(oracle, dtype, ulps):
+    """Pins tto_normal_* (common/kernel/distribution.hpp:232-246) without libm: the Box-Muller value of every element
+    is rebuilt from the integer generator and 200-bit transcendental evaluations.  A correctly rounded chain and a
+    libm chain (each function within 1 ulp) differ by at most a few units in the last place of std*z; the three
+    plausible slips (cos for sin, u1 and u2 swapped, log(u1) for log1p(-u1)) miss that bound on nearly every element."""
+    n, seed, mu, std = 1000, 11, dtype(0.25), dtype(0.1)
+    g = oracle.Generator(seed)
+    got = g.normal(float(mu), float(std), (n,), dtype)
+    u, master_state = _element_uniforms(oracle, seed, n, dtype)
+    assert g.state == master_state  # n master outputs consumed, nothing else
+
+    def misses(variant):
+        bad = 0
+        for i in range(n):
+            want, sz = _box_muller_model(u[i, 0], u[i, 1], mu, std, dtype, variant)
+            if not np.isfinite(float(want)):
+                bad += 1
+                continue
+            # libm's log1p, sqrt, sin are within 1 ulp each: `ulps` units of std*z cover the chain, plus one unit of
+            # the final sum (an addend that moved by a unit can tip the sum's rounding to the neighbouring value, and
+            # the sum may or may not be contracted into an fma).
+            tol = ulps * float(np.spacing(dtype(abs(float(sz))))) + float(np.spacing(dtype(abs(float(want)))))
+            if abs(float(got[i]) - float(want)) > tol:
+                bad += 1
+        return bad
+
+    assert misses("reference") == 0
+    for wrong in ("cos", "swapped", "log_u1"):
+        assert misses(wrong) > 0.95 * n, wrong
+
+
+def test_normal_zero_mean_keeps_relative_accuracy(oracle):
+    # With mu = 0 (config 4's inputs: normal(0, 0.1)) the value is std*z itself: every element within 4 ulp of the
+    # 200-bit evaluation, including the small ones where sin(theta) is near a zero crossing.
+    n, seed = 500, 0
+    got = oracle.Generator(seed).normal(0.0, 0.1, (n,), np.float32)
+    u, _ = _element_uniforms(oracle, seed, n, np.float32)
+    for i in range(n):
+        want, _sz = _box_muller_model(u[i, 0], u[i, 1], np.float32(0.0), np.float32(0.1), np.float32)
+        assert abs(float(got[i]) - float(want)) <= 4 * float(np.spacing(np.float32(abs(float(want))))), i
 
 
 # ------------------------------------------------------------------------------------------- contiguous
