@@ -19,6 +19,7 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 PEAK_TFLOPS = {"f32": 157.3, "f64": 78.6}  # MI355X dense matrix peaks
+WARMUP_SECONDS = 0.25  # minimum untimed GPU work in front of the timed launches
 
 # Bytes moved between the L2s and the memory fabric per launch of the default workload, from the rocprofv3
 # FETCH_SIZE / WRITE_SIZE passes summarised in profiles/gemm_4096_f32_f64_mfma.txt (scaled by the same counters'
@@ -28,7 +29,7 @@ MEASURED_TRAFFIC = {("mfma_f32_256x256_akc4_bmc4", 4096): (196856.1 * 2.0 + 6553
 
 
 def gpu_gemm_timing(tt, np, dtype, n, steps, warmup):
-    """Returns (wall ms/step, event-timed average kernel ms, variant name, C as numpy)."""
+    """Returns (wall ms/step, event-timed average kernel ms, variant name, (A, B, C), warm-up launches made)."""
     from oracle import tt_oracle as oracle  # input generation only (the reference's RNG restated on the host)
 
     lib = tt._capi.lib
@@ -46,8 +47,15 @@ def gpu_gemm_timing(tt, np, dtype, n, steps, warmup):
         if st != 0:
             raise RuntimeError(tt._capi.last_error())
 
-    for _ in range(warmup):
+    # Untimed warm-up: the requested number of launches and at least WARMUP_SECONDS of GPU work, because the clocks
+    # take on the order of 100 ms of load to settle and a short `--warmup` count would charge the ramp to the timed
+    # launches.  The number of launches actually made is reported as `warmup_effective`.
+    warm, t_end = 0, time.perf_counter() + WARMUP_SECONDS
+    while warm < warmup or time.perf_counter() < t_end:
         step()
+        warm += 1
+        if warm % 8 == 0:
+            be.synchronize(0)
     be.synchronize(0)
     e0, e1 = C.c_void_p(), C.c_void_p()
     lib.ttamd_event_create(0, C.byref(e0))
@@ -63,7 +71,7 @@ def gpu_gemm_timing(tt, np, dtype, n, steps, warmup):
     lib.ttamd_event_elapsed_ms(e0, e1, C.byref(ms))
     lib.ttamd_event_destroy(e0)
     lib.ttamd_event_destroy(e1)
-    return wall_ms, ms.value / steps, variant, (A, B, out)
+    return wall_ms, ms.value / steps, variant, (A, B, out), warm
 
 
 def time_launches(tt, fn, iters, warmup):
@@ -400,7 +408,7 @@ def main():
 
     n = args.n
     flop = 2.0 * n * n * n
-    wall_ms, kern_ms, variant, (A, B, out) = gpu_gemm_timing(tt, np, np.float32, n, args.steps, args.warmup)
+    wall_ms, kern_ms, variant, (A, B, out), warm_eff = gpu_gemm_timing(tt, np, np.float32, n, args.steps, args.warmup)
     gflops = flop / (wall_ms * 1e-3) / 1e9
     achieved_tflops = flop / (kern_ms * 1e-3) / 1e12
 
@@ -413,7 +421,7 @@ def main():
     scale = np.abs(A[rows]).astype(np.float64) @ np.abs(B).astype(np.float64)
     parity = float(np.max(np.abs(Cg[rows].astype(np.float64) - want.astype(np.float64)) / scale))
 
-    wall64, kern64, variant64, _ = gpu_gemm_timing(tt, np, np.float64, n, max(args.steps // 2, 1), args.warmup)
+    wall64, kern64, variant64, _, _ = gpu_gemm_timing(tt, np, np.float64, n, max(args.steps // 2, 1), args.warmup)
     f64_tflops = flop / (kern64 * 1e-3) / 1e12
 
     cpu = None
@@ -434,6 +442,7 @@ def main():
         "n_gpus": 1,
         "steps": args.steps,
         "warmup": args.warmup,
+        "warmup_effective": warm_eff,
         "ms_per_step": round(wall_ms, 4),
         "higher_is_better": True,
         "scaling": "weak",
@@ -445,7 +454,11 @@ def main():
                    "parity_k_scaled_err_rows0_63": parity},
         "roofline": {"bound": "mfma", "achieved": round(achieved_tflops, 2), "peak": PEAK_TFLOPS["f32"],
                      "unit": "TFLOP/s", "frac": round(achieved_tflops / PEAK_TFLOPS["f32"], 4),
-                     "traffic": MEASURED_TRAFFIC.get((variant, n)), "algorithmic_bytes": 3.0 * n * n * 4,
+                     "traffic": MEASURED_TRAFFIC.get((variant, n)),
+                     "traffic_source": ("profiles/gemm_4096_f32_f64_mfma.txt (rocprofv3 FETCH_SIZE / WRITE_SIZE passes of this "
+                                        "kernel and size; a recorded figure, not measured in this run)"
+                                        if (variant, n) in MEASURED_TRAFFIC else None),
+                     "algorithmic_bytes": 3.0 * n * n * 4,
                      "kernel_ms": round(kern_ms, 4)},
         "cpu_baseline": cpu,
         "fp64": {"kernel": variant64, "kernel_ms": round(kern64, 4), "achieved": round(f64_tflops, 2),
