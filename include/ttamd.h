@@ -132,6 +132,19 @@ ttamd_status ttamd_batched_matmul(int device, ttamd_dtype dtype, int B, int N, i
                                   const ttamd_view3 *lhs, const ttamd_view3 *rhs, void *out,
                                   const ttamd_epilogue *epilogue, void *stream);
 
+/* ttamd_batched_matmul for callers that cannot allocate device memory (code under HIP graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  Same arguments, same kernels and
+ * bit-identical results; the difference is where the partial tiles of a split reduction live: in a fixed 8 MiB
+ * array inside the library's code object (one copy per GPU, held until the process ends) instead of the per-stream
+ * buffer that ttamd_batched_matmul grows with hipMalloc.  The call makes no hipMalloc / hipFree.  A product whose
+ * partial tiles exceed the array (possible for some f64 shapes with fewer than 128 output tiles of 64 x 64) is refused
+ * with TTAMD_ERR_INVALID_ARGUMENT and a message naming the sizes.  All calls on one GPU share that GPU's array:
+ * calls that may overlap in time on one GPU (different streams, several threads) race and must be serialised by the
+ * caller.  The first call on a device looks up the array's device address; make that call outside a capture. */
+ttamd_status ttamd_batched_matmul_noalloc(int device, ttamd_dtype dtype, int B, int N, int K, int M,
+                                          const ttamd_view3 *lhs, const ttamd_view3 *rhs, void *out,
+                                          const ttamd_epilogue *epilogue, void *stream);
+
 /* BackendBase::conv2d (backend_base.h:269-275; CPU: cpu/conv.cpp:36-134).  input [B,C,H,W],
  * weight [O,C,k,k] (square kernel), bias [O] or NULL, zero padding; out dense [B,O,Ho,Wo] with
  * Ho = (H + 2*padding - k)/stride + 1.  Implicit GEMM: no im2col buffer is materialised. */

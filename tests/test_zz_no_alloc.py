@@ -1,0 +1,110 @@
+"""ttamd_batched_matmul_noalloc against ttamd_batched_matmul, through the C ABI.
+
+The entry point keeps the partial tiles of a split reduction in a fixed device array of the library instead of a buffer
+obtained with hipMalloc.  Same kernels and the same split plan, so the two entry points must agree bit for bit; the
+array keeps the previous call's contents, hence two calls in a row with the second one smaller.
+"""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+FIXED_SCRATCH_BYTES = 8 << 20
+
+
+def _run(tt, entry, tA, tB, epilogue=None):
+    """out = entry(tA, tB) for 3-D tensors; returns the result as numpy."""
+    capi = tt._capi
+    Bn, N, K = tA.shape
+    M = tB.shape[2]
+    out = tt.Tensor.empty((Bn, N, M), tA.dtype)
+    lv, rv = tA.view3(), tB.view3()
+    st = entry(0, tA.dtype, Bn, N, K, M, C.byref(lv), C.byref(rv), C.c_void_p(out.storage.ptr),
+               C.byref(epilogue) if epilogue is not None else None, None)
+    assert st == capi.OK, capi.last_error()
+    return out.to_numpy()
+
+
+def _pair(rng, dtype, B, N, K, M, integer_valued=False):
+    if integer_valued:
+        a = rng.integers(-4, 5, (B, N, K)).astype(dtype)
+        b = rng.integers(-4, 5, (B, K, M)).astype(dtype)
+    else:
+        a = rng.uniform(-1, 1, (B, N, K)).astype(dtype)
+        b = rng.uniform(-1, 1, (B, K, M)).astype(dtype)
+    return a, b
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+def test_two_calls_in_a_row_match_the_allocating_entry_point(tt, oracle, dtype):
+    lib = tt._capi.lib
+    be = tt.get_backend(tt.kAMD)
+    rng = np.random.default_rng(5)
+    # first a split-k product that fills several MiB of the array, then a smaller split-k product that finds the first
+    # one's partial tiles there, then shapes that use no scratch at all (two halves of k, plain tiles, integers below)
+    # (f64 256 x 512 x 256 splits 16 ways: exactly the 8 MiB the array holds)
+    head = [(3, 320, 1024, 384), (1, 256, 512, 256)] if dtype == np.float32 else [(1, 256, 512, 256), (1, 128, 512, 192)]
+    shapes = head + [(1, 100, 301, 10), (1, 1024, 1024, 1024), (2, 130, 70, 150)]
+    for i, (B, N, K, M) in enumerate(shapes):
+        a, b = _pair(rng, dtype, B, N, K, M)
+        tA, tB = tt.Tensor.from_numpy(a), tt.Tensor.from_numpy(b)
+        variant = be.batched_matmul_variant(tA, tB)
+        if i < 3:
+            assert "splitk" in variant, (variant, (B, N, K, M))
+            ksplit = int(variant.split("splitk")[1])
+            assert ksplit * B * N * M * a.itemsize <= FIXED_SCRATCH_BYTES
+        got = _run(tt, lib.ttamd_batched_matmul_noalloc, tA, tB)
+        want = _run(tt, lib.ttamd_batched_matmul, tA, tB)
+        assert np.array_equal(got, want), (variant, (B, N, K, M))
+        # and against the CPU oracle, K-scaled
+        ref = oracle.batched_matmul(a, b)
+        scale = np.abs(a).astype(np.float64) @ np.abs(b).astype(np.float64)
+        err = np.max(np.abs(got.astype(np.float64) - ref.astype(np.float64)) / np.maximum(scale, 1e-30))
+        assert err <= (1e-4 if dtype == np.float32 else 1e-12), (variant, err)
+
+
+def test_transposed_views_epilogue_and_integers(tt, oracle):
+    capi, lib = tt._capi, tt._capi.lib
+    rng = np.random.default_rng(6)
+    # A^T . B on views (the weight-gradient product of a skinny Linear layer: split k with element-wise B)
+    x, g = rng.integers(-3, 4, (1, 1024, 300)).astype(np.float32), rng.integers(-3, 4, (1, 1024, 10)).astype(np.float32)
+    tX, tG = tt.Tensor.from_numpy(x).permute(0, 2, 1), tt.Tensor.from_numpy(g)
+    got = _run(tt, lib.ttamd_batched_matmul_noalloc, tX, tG)
+    assert np.array_equal(got, _run(tt, lib.ttamd_batched_matmul, tX, tG))
+    assert np.array_equal(got, oracle.batched_matmul(np.ascontiguousarray(x.transpose(0, 2, 1)), g))  # integer-valued: exact
+    # bias + ReLU fused behind a split reduction (applied by the kernel that sums the partial tiles)
+    a, b = _pair(rng, np.float32, 1, 256, 512, 256, integer_valued=True)
+    bias = rng.integers(-50, 50, 256).astype(np.float32)
+    tbias = tt.Tensor.from_numpy(bias)
+    ep = capi.Epilogue(tbias.storage.ptr, 1, 1, 0)
+    tA, tB = tt.Tensor.from_numpy(a), tt.Tensor.from_numpy(b)
+    got = _run(tt, lib.ttamd_batched_matmul_noalloc, tA, tB, ep)
+    assert np.array_equal(got, _run(tt, lib.ttamd_batched_matmul, tA, tB, ep))
+    assert np.array_equal(got[0], np.maximum(oracle.matmul(a[0], b[0]) + bias[None, :], 0))
+    # integer dtypes take the vector-ALU kernel, which has no scratch
+    ai, bi = rng.integers(-100, 100, (2, 70, 90)).astype(np.int32), rng.integers(-100, 100, (2, 90, 50)).astype(np.int32)
+    tA, tB = tt.Tensor.from_numpy(ai), tt.Tensor.from_numpy(bi)
+    assert np.array_equal(_run(tt, lib.ttamd_batched_matmul_noalloc, tA, tB), oracle.batched_matmul(ai, bi))
+
+
+def test_products_beyond_the_fixed_array_are_refused(tt):
+    capi, lib = tt._capi, tt._capi.lib
+    be = tt.get_backend(tt.kAMD)
+    B, N, K, M = 1, 704, 512, 704
+    tA = tt.Tensor.empty((B, N, K), capi.F64)
+    tB = tt.Tensor.empty((B, K, M), capi.F64)
+    variant = be.batched_matmul_variant(tA, tB)
+    ksplit = int(variant.split("splitk")[1])
+    assert ksplit * N * M * 8 > FIXED_SCRATCH_BYTES
+    out = tt.Tensor.empty((B, N, M), capi.F64)
+    lv, rv = tA.view3(), tB.view3()
+    st = lib.ttamd_batched_matmul_noalloc(0, capi.F64, B, N, K, M, C.byref(lv), C.byref(rv), C.c_void_p(out.storage.ptr), None, None)
+    assert st == capi.ERR_INVALID_ARGUMENT
+    msg = capi.last_error()
+    assert "fixed scratch" in msg and str(ksplit * N * M * 8) in msg
+    # the allocating entry point takes the same product
+    st = lib.ttamd_batched_matmul(0, capi.F64, B, N, K, M, C.byref(lv), C.byref(rv), C.c_void_p(out.storage.ptr), None, None)
+    assert st == capi.OK, capi.last_error()
+    be.synchronize(0)

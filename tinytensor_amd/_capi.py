@@ -59,6 +59,7 @@ def _bind(lib: C.CDLL) -> None:
         "ttamd_full": (i, [i, i, vp, C.c_int64, vp, vp]),
         "ttamd_random_fill": (i, [i, i, i, C.c_double, C.c_double, C.POINTER(C.c_uint64), C.c_int64, vp, vp]),
         "ttamd_batched_matmul": (i, [i, i, i, i, i, i, C.POINTER(View3), C.POINTER(View3), vp, C.POINTER(Epilogue), vp]),
+        "ttamd_batched_matmul_noalloc": (i, [i, i, i, i, i, i, C.POINTER(View3), C.POINTER(View3), vp, C.POINTER(Epilogue), vp]),
         "ttamd_batched_matmul_variant": (C.c_char_p, [i, i, i, i, i, C.POINTER(View3), C.POINTER(View3)]),
         "ttamd_conv2d_forward": (i, [i, i, C.POINTER(View4), C.POINTER(View4), vp, vp] + [i] * 8 + [vp]),
         "ttamd_conv2d_backward_workspace": (i, [i] + [i] * 8 + [C.POINTER(sz)]),

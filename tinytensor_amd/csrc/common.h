@@ -15,6 +15,9 @@ namespace ttamd {
 // Thread-local text for ttamd_last_error_string().
 void set_error(const char *fmt, ...) __attribute__((format(printf, 1, 2)));
 
+// Device ids the library's per-device tables are sized for; use_device refuses anything beyond.
+constexpr int kMaxDevices = 64;
+
 // Makes `device` current; TTAMD_ERR_INVALID_DEVICE when the id is out of range.
 ttamd_status use_device(int device);
 
@@ -84,9 +87,11 @@ struct GemmArgs {
 };
 
 // Launchers (defined in gemm_mfma.hip / gemm_simt.hip).  `variant_only`: fill *variant with the
-// kernel name that would run and return without launching.
+// kernel name that would run and return without launching.  `fixed_scratch`: split-k partial tiles go to the
+// library's fixed device array instead of the growing per-stream buffer (nothing is allocated; products whose
+// partial tiles exceed the array are refused).
 ttamd_status launch_gemm_mfma(ttamd_dtype dt, const GemmArgs &g, int device, hipStream_t stream, const char **variant,
-                              bool variant_only, bool *handled);
+                              bool variant_only, bool *handled, bool fixed_scratch = false);
 ttamd_status launch_gemm_simt(ttamd_dtype dt, const GemmArgs &g, hipStream_t stream, const char **variant,
                               bool variant_only);
 

@@ -80,12 +80,8 @@ ttamd_status build_args(ttamd_dtype dtype, int B, int N, int K, int M, const tta
     return TTAMD_OK;
 }
 
-}  // namespace
-
-extern "C" {
-
-ttamd_status ttamd_batched_matmul(int device, ttamd_dtype dtype, int B, int N, int K, int M, const ttamd_view3 *lhs,
-                                  const ttamd_view3 *rhs, void *out, const ttamd_epilogue *epilogue, void *stream) {
+ttamd_status batched_matmul(int device, ttamd_dtype dtype, int B, int N, int K, int M, const ttamd_view3 *lhs,
+                            const ttamd_view3 *rhs, void *out, const ttamd_epilogue *epilogue, void *stream, bool fixed_scratch) {
     GemmArgs g;
     if (ttamd_status s = build_args(dtype, B, N, K, M, lhs, rhs, out, epilogue, &g, true)) return s;
     if (ttamd_status s = use_device(device)) return s;
@@ -94,11 +90,25 @@ ttamd_status ttamd_batched_matmul(int device, ttamd_dtype dtype, int B, int N, i
     const char *variant = nullptr;
     bool handled = false;
     if (K > 0) {
-        if (ttamd_status s = launch_gemm_mfma(dtype, g, device, st, &variant, false, &handled)) return s;
+        if (ttamd_status s = launch_gemm_mfma(dtype, g, device, st, &variant, false, &handled, fixed_scratch)) return s;
         if (handled) return TTAMD_OK;
     }
-    // K == 0 also lands here: the vector-ALU kernel then stores the empty sum (0, + bias).
+    // K == 0 also lands here: the vector-ALU kernel then stores the empty sum (0, + bias).  It uses no scratch.
     return launch_gemm_simt(dtype, g, st, &variant, false);
+}
+
+}  // namespace
+
+extern "C" {
+
+ttamd_status ttamd_batched_matmul(int device, ttamd_dtype dtype, int B, int N, int K, int M, const ttamd_view3 *lhs,
+                                  const ttamd_view3 *rhs, void *out, const ttamd_epilogue *epilogue, void *stream) {
+    return batched_matmul(device, dtype, B, N, K, M, lhs, rhs, out, epilogue, stream, false);
+}
+
+ttamd_status ttamd_batched_matmul_noalloc(int device, ttamd_dtype dtype, int B, int N, int K, int M, const ttamd_view3 *lhs,
+                                          const ttamd_view3 *rhs, void *out, const ttamd_epilogue *epilogue, void *stream) {
+    return batched_matmul(device, dtype, B, N, K, M, lhs, rhs, out, epilogue, stream, true);
 }
 
 const char *ttamd_batched_matmul_variant(ttamd_dtype dtype, int B, int N, int K, int M, const ttamd_view3 *lhs,

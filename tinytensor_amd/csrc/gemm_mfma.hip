@@ -12,10 +12,40 @@
 #include <algorithm>
 #include <cmath>
 
+#include <mutex>
+
 namespace ttamd {
 namespace {
 
 using namespace mfma;
+
+// Partial tiles of split-k launches made through ttamd_batched_matmul_noalloc: a fixed array in the code object
+// instead of the growing per-stream buffer, so that the call never allocates.  Every GPU that loads the library holds
+// its own copy (kFixedScratchBytes of its memory, until the process ends) at its own address; the name below is only
+// the host-side handle of the symbol, the device address comes from hipGetSymbolAddress, once per device.
+constexpr size_t kFixedScratchBytes = size_t(8) << 20;
+static __device__ __align__(256) unsigned char scratch[kFixedScratchBytes];
+
+ttamd_status fixed_scratch_address(int device, void **out) {
+    static std::mutex mu;
+    static void *address[kMaxDevices] = {};
+    if (device < 0 || device >= kMaxDevices) {
+        set_error("batched_matmul_noalloc: device id %d beyond the %d devices the fixed scratch serves", device, kMaxDevices);
+        return TTAMD_ERR_INVALID_DEVICE;
+    }
+    std::lock_guard<std::mutex> lock(mu);
+    if (!address[device]) {  // the caller has made `device` current (use_device)
+        void *p = nullptr;
+        TTAMD_HIP_CHECK(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+        if (!p) {
+            set_error("batched_matmul_noalloc: the scratch symbol has no address on device %d", device);
+            return TTAMD_ERR_LAUNCH;
+        }
+        address[device] = p;
+    }
+    *out = address[device];
+    return TTAMD_OK;
+}
 
 // ksplit > 1: the reduction is cut into `ksplit` ranges of `k_chunk` (a multiple of BK); workgroup column z =
 // batch * ksplit + split writes the raw partial tile to `partial[z]` and splitk_reduce_kernel finishes the job.
@@ -187,6 +217,7 @@ struct TileShapes<double> {
 struct SplitPlan {
     int ksplit = 1;
     int k_chunk = 0;
+    bool fixed_scratch = false;  // partial tiles go to the library's fixed array (the call must not allocate)
 };
 
 template <typename T, int BM, int BN, int BK, int WGM, int WGN, bool A_KC, int A_VEC, bool B_KC, int B_VEC, int PF>
@@ -203,11 +234,12 @@ ttamd_status launch_variant(const GemmArgs &g, const SplitPlan &sp, int device, 
     constexpr int kEpiA = kTwoKernels ? kEpiLean : kEpiAny, kEpiB = kTwoKernels ? kEpiFull : kEpiAny;
     auto kernel = lean ? gemm_mfma_kernel<T, BM, BN, BK, WGM, WGN, A_KC, A_VEC, B_KC, B_VEC, PF, kEpiA>
                        : gemm_mfma_kernel<T, BM, BN, BK, WGM, WGN, A_KC, A_VEC, B_KC, B_VEC, PF, kEpiB>;
-    static bool configured[2] = {false, false};  // raising the dynamic LDS limit is per kernel, once
-    if (!configured[lean] && lds_bytes > 48 * 1024) {
+    static bool configured[kMaxDevices][2] = {};  // raising the dynamic LDS limit: once per kernel and device
+    const int slot = device >= 0 && device < kMaxDevices ? device : 0;
+    if ((!configured[slot][lean] || slot != device) && lds_bytes > 48 * 1024) {
         TTAMD_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
                                             hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_bytes)));
-        configured[lean] = true;
+        configured[slot][lean] = true;
     }
     const int tiles_m = (g.M + BM - 1) / BM, tiles_n = (g.N + BN - 1) / BN;
     const int64_t blocks = static_cast<int64_t>(tiles_m) * tiles_n * g.batch * sp.ksplit;
@@ -219,7 +251,16 @@ ttamd_status launch_variant(const GemmArgs &g, const SplitPlan &sp, int device, 
     if (sp.ksplit > 1) {
         void *ws = nullptr;
         const size_t bytes = static_cast<size_t>(sp.ksplit) * g.batch * g.M * g.N * sizeof(T);
-        if (ttamd_status st = stream_scratch(device, stream, bytes, &ws)) return st;
+        if (sp.fixed_scratch) {
+            if (bytes > kFixedScratchBytes) {
+                set_error("batched_matmul_noalloc: this product splits its reduction %d ways and needs %zu bytes of partial "
+                          "tiles; the fixed scratch holds %zu (use ttamd_batched_matmul)", sp.ksplit, bytes, kFixedScratchBytes);
+                return TTAMD_ERR_INVALID_ARGUMENT;
+            }
+            if (ttamd_status st = fixed_scratch_address(device, &ws)) return st;
+        } else if (ttamd_status st = stream_scratch(device, stream, bytes, &ws)) {
+            return st;
+        }
         partial = static_cast<T *>(ws);
     }
     kernel<<<dim3(static_cast<unsigned>(blocks)), dim3(kThreads), lds_bytes, stream>>>(g, tiles_m, tiles_n, sp.ksplit,
@@ -242,16 +283,17 @@ int dual_k_half(int K) {
 }
 
 template <typename T, int BM, int BN, int BK, int WGM, int WGN, bool A_KC, int A_VEC, bool B_KC, int B_VEC, int PF>
-ttamd_status launch_dual_variant(const GemmArgs &g, hipStream_t stream) {
+ttamd_status launch_dual_variant(const GemmArgs &g, int device, hipStream_t stream) {
     using StA = Stager<T, BM, BK, A_KC, A_VEC, PF>;
     using StB = Stager<T, BN, BK, B_KC, B_VEC, PF>;
     constexpr size_t lds_bytes = 2 * TileEngine<T, BM, BN, BK, WGM, WGN, StA, StB>::kLdsBytes;
     auto kernel = gemm_mfma_dual_kernel<T, BM, BN, BK, WGM, WGN, A_KC, A_VEC, B_KC, B_VEC, PF>;
-    static bool configured = false;
-    if (!configured) {
+    static bool configured[kMaxDevices] = {};  // once per kernel and device
+    const int slot = device >= 0 && device < kMaxDevices ? device : 0;
+    if (!configured[slot] || slot != device) {
         TTAMD_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
                                             static_cast<int>(lds_bytes)));
-        configured = true;
+        configured[slot] = true;
     }
     const int k_half = dual_k_half<T>(g.K);
     if (k_half <= 0 || (k_half + BK - 1) / BK != (g.K - k_half + BK - 1) / BK) {  // the halves share the engine's barriers
@@ -266,11 +308,11 @@ ttamd_status launch_dual_variant(const GemmArgs &g, hipStream_t stream) {
 }
 
 template <typename T, int BM, int BN, int BK, int WGM, int WGN, int VEC, int PF>
-ttamd_status launch_dual_layouts(const GemmArgs &g, bool a_kc, bool b_kc, hipStream_t stream) {
-    if (a_kc && b_kc) return launch_dual_variant<T, BM, BN, BK, WGM, WGN, true, VEC, true, VEC, PF>(g, stream);
-    if (a_kc && !b_kc) return launch_dual_variant<T, BM, BN, BK, WGM, WGN, true, VEC, false, VEC, PF>(g, stream);
-    if (!a_kc && b_kc) return launch_dual_variant<T, BM, BN, BK, WGM, WGN, false, VEC, true, VEC, PF>(g, stream);
-    return launch_dual_variant<T, BM, BN, BK, WGM, WGN, false, VEC, false, VEC, PF>(g, stream);
+ttamd_status launch_dual_layouts(const GemmArgs &g, bool a_kc, bool b_kc, int device, hipStream_t stream) {
+    if (a_kc && b_kc) return launch_dual_variant<T, BM, BN, BK, WGM, WGN, true, VEC, true, VEC, PF>(g, device, stream);
+    if (a_kc && !b_kc) return launch_dual_variant<T, BM, BN, BK, WGM, WGN, true, VEC, false, VEC, PF>(g, device, stream);
+    if (!a_kc && b_kc) return launch_dual_variant<T, BM, BN, BK, WGM, WGN, false, VEC, true, VEC, PF>(g, device, stream);
+    return launch_dual_variant<T, BM, BN, BK, WGM, WGN, false, VEC, false, VEC, PF>(g, device, stream);
 }
 
 template <typename T, int BM, int BN, int BK, int WGM, int WGN, int A_VEC, int B_VEC, int PF = 1>
@@ -310,7 +352,7 @@ SplitPlan plan_split(const GemmArgs &g, int bm, int bn, int bk) {
 
 template <typename T>
 ttamd_status launch_mfma_typed(const GemmArgs &g, int device, hipStream_t stream, const char **variant, bool variant_only,
-                               bool *handled) {
+                               bool *handled, bool fixed_scratch) {
     using TS = TileShapes<T>;
     constexpr int VK = Mfma<T>::VK;
     *handled = false;
@@ -356,7 +398,8 @@ ttamd_status launch_mfma_typed(const GemmArgs &g, int device, hipStream_t stream
     const int64_t c_reach = static_cast<int64_t>(g.M < bm ? g.M : bm) * g.N * static_cast<int64_t>(sizeof(T));
     if (a_reach >= 0x7fffffffLL || b_reach >= 0x7fffffffLL || c_reach >= 0x7fffffffLL) return TTAMD_OK;
 
-    const SplitPlan sp = (xxl || xl || mid || large) ? SplitPlan{1, g.K} : plan_split<T>(g, TS::SBM, TS::SBN, TS::SBK);
+    SplitPlan sp = (xxl || xl || mid || large) ? SplitPlan{1, g.K} : plan_split<T>(g, TS::SBM, TS::SBN, TS::SBK);
+    sp.fixed_scratch = fixed_scratch;
 
     // Small tiles, at most one workgroup per CU and a long reduction: two halves of k in one workgroup of 8 waves.
     const int64_t small_wgs = static_cast<int64_t>((g.M + TS::SBM - 1) / TS::SBM) * ((g.N + TS::SBN - 1) / TS::SBN) * g.batch;
@@ -383,7 +426,7 @@ ttamd_status launch_mfma_typed(const GemmArgs &g, int device, hipStream_t stream
     if constexpr (sizeof(T) == 4)
         if (mid) return launch_layouts<T, TS::MBM, TS::MBN, TS::MBK, 2, 2, VK, VK>(g, ca.kc, cb.kc, sp, device, stream);
     if (large) return launch_layouts<T, TS::LBM, TS::LBN, TS::LBK, 2, 2, VK, VK>(g, ca.kc, cb.kc, sp, device, stream);
-    if (dual) return launch_dual_layouts<T, TS::SBM, TS::SBN, TS::SBK, 2, 2, VK, TS::SPF_DEEP>(g, ca.kc, cb.kc, stream);
+    if (dual) return launch_dual_layouts<T, TS::SBM, TS::SBN, TS::SBK, 2, 2, VK, TS::SPF_DEEP>(g, ca.kc, cb.kc, device, stream);
     if (ca.vec > 1 && cb.vec > 1) {
         // Register prefetch depth of the small tile: 4 k tiles in flight when a CU holds at most two workgroups and the
         // reduction is long (a lone workgroup otherwise waits for memory in every step), else 2, whose smaller register
@@ -402,10 +445,10 @@ ttamd_status launch_mfma_typed(const GemmArgs &g, int device, hipStream_t stream
 }  // namespace
 
 ttamd_status launch_gemm_mfma(ttamd_dtype dt, const GemmArgs &g, int device, hipStream_t stream, const char **variant,
-                              bool variant_only, bool *handled) {
+                              bool variant_only, bool *handled, bool fixed_scratch) {
     *handled = false;
-    if (dt == TTAMD_F32) return launch_mfma_typed<float>(g, device, stream, variant, variant_only, handled);
-    if (dt == TTAMD_F64) return launch_mfma_typed<double>(g, device, stream, variant, variant_only, handled);
+    if (dt == TTAMD_F32) return launch_mfma_typed<float>(g, device, stream, variant, variant_only, handled, fixed_scratch);
+    if (dt == TTAMD_F64) return launch_mfma_typed<double>(g, device, stream, variant, variant_only, handled, fixed_scratch);
     return TTAMD_OK;
 }
 

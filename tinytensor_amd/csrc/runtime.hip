@@ -15,7 +15,6 @@ namespace ttamd {
 
 namespace {
 thread_local char g_error[512] = "no error";
-constexpr int kMaxDevices = 64;
 std::atomic<uint64_t> g_current[kMaxDevices];
 std::atomic<uint64_t> g_total[kMaxDevices];
 
