@@ -252,8 +252,7 @@ def detail_report(tt, np, path, cpu=True):
     ms = time_launches(tt, lambda: be.conv2d(x, w, None, 1, 1, out=out), 100, 10)
     rows.append({"case": "cfg4 conv2d forward", "kernel": "conv_fwd_kernel (implicit GEMM)", "ms": round(ms, 5),
                  "GFLOP/s": round(1.850e9 / ms / 1e6, 1)})
-    be.conv2d_backward(go, x, w, None, 1, 1)
-    bufs = be.last_conv_buffers
+    bufs = be.conv2d_backward(go, x, w, None, 1, 1, return_buffers=True)
     ms = time_launches(tt, lambda: be.conv2d_backward(go, x, w, None, 1, 1, buffers=bufs), 50, 5)
     rows.append({"case": "cfg4 conv2d backward (grad_input + grad_weight)", "kernel": "conv_dgrad_kernel + conv_wgrad_kernel + reduce",
                  "ms": round(ms, 5), "GFLOP/s": round(3.700e9 / ms / 1e6, 1)})
@@ -394,8 +393,7 @@ def main():
         w = tt.Tensor.from_numpy(rng.normal(0, 0.1, (co, cc, 3, 3)).astype(np.float32))
         out = be.conv2d(x, w, None, 1, 1)
         go = tt.Tensor.from_numpy(np.ones(out.shape, np.float32))
-        be.conv2d_backward(go, x, w, None, 1, 1)
-        bufs = be.last_conv_buffers
+        bufs = be.conv2d_backward(go, x, w, None, 1, 1, return_buffers=True)
         for _ in range(args.conv_loop):
             be.conv2d(x, w, None, 1, 1, out=out)
             be.conv2d_backward(go, x, w, None, 1, 1, buffers=bufs)

@@ -217,7 +217,9 @@ ttamd_status ttamd_where(int device, ttamd_dtype dtype, int ndim, const int64_t 
                          int64_t cond_offset, const int64_t *cond_stride, const void *lhs, int64_t lhs_offset,
                          const int64_t *lhs_stride, const void *rhs, int64_t rhs_offset, const int64_t *rhs_stride,
                          void *out, void *stream);
-/* BackendBase::sum(tensor) (dim = -1, one element out) and sum(tensor, dim) (that dimension removed). */
+/* BackendBase::sum(tensor) (dim = -1, one element out) and sum(tensor, dim) (that dimension removed).  The result has
+ * the operand's dtype for f32 / f64; bool and every integer dtype are summed in 64 bits and the result is I64
+ * (common/reduce.h:56-61, cpu/reduce.cpp:38-54), so `out` holds 8 bytes per element for them. */
 ttamd_status ttamd_sum(int device, ttamd_dtype dtype, int ndim, const int64_t *shape, const void *src, int64_t offset,
                        const int64_t *stride, int dim, void *out, void *stream);
 /* BackendBase::full (backend_base.h:51): `value` points at one host scalar of `dtype`. */
@@ -230,6 +232,14 @@ ttamd_status ttamd_full(int device, ttamd_dtype dtype, const void *value, int64_
  * backend does (cuda/distribution.cu:32-99), so uniform values are bit-identical to the CPU backend's. */
 ttamd_status ttamd_random_fill(int device, ttamd_dtype dtype, int dist, double p0, double p1, uint64_t *master_state,
                                int64_t numel, void *out, void *stream);
+/* The same draws written in place through a strided view (ndim <= 8, element strides >= 0), as the CPU backend's
+ * in-place kernel does (cpu/distribution.cpp:96-139, cpu/kernel/distribution.hpp:28-32): element i of the view, i
+ * its row-major rank over `shape`, takes the i-th master output as its state and lands at
+ * data[offset + sum(index[d] * stride[d])] (common/util.h:18-34).  nn::Conv2d initialises its weight through
+ * weight->permute({1,0,2,3}) (nn/conv2d.cpp:56), so the draw order runs over [C,O,k,k] while the storage is [O,C,k,k]. */
+ttamd_status ttamd_random_fill_view(int device, ttamd_dtype dtype, int dist, double p0, double p1, uint64_t *master_state,
+                                    int ndim, const int64_t *shape, const int64_t *stride, void *data, int64_t offset,
+                                    void *stream);
 
 /* ---- timing (no reference counterpart: the reference has no timers; used by the benchmark
  * to bracket kernels with HIP events on the stream they run on) ------------------------ */

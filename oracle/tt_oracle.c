@@ -119,6 +119,28 @@ static inline int to_flat_index(int rank, int ndim, const int *shape, const int 
     }
     return flat;
 }
+
+/* In-place draws through a strided view (cpu/distribution.cpp:96-139 with cpu/kernel/distribution.hpp:28-32):
+ * element i of the view (row-major rank over `shape`) takes master output i as its state and is written at
+ * to_flat_index(i).  nn::Conv2d initialises its weight through weight->permute({1,0,2,3}) (nn/conv2d.cpp:56). */
+void tto_uniform_real_view_f32(uint64_t *state, float low, float high, float *data, int ndim, const int *shape,
+                               const int *stride, int offset) {
+    int n = 1;
+    for (int d = 0; d < ndim; ++d) n *= shape[d];
+    for (int i = 0; i < n; ++i) {
+        uint64_t st = tto_xorshift64(state);
+        data[to_flat_index(i, ndim, shape, stride, offset)] = uniform_sample_f32(low, high, &st);
+    }
+}
+void tto_uniform_real_view_f64(uint64_t *state, double low, double high, double *data, int ndim, const int *shape,
+                               const int *stride, int offset) {
+    int n = 1;
+    for (int d = 0; d < ndim; ++d) n *= shape[d];
+    for (int i = 0; i < n; ++i) {
+        uint64_t st = tto_xorshift64(state);
+        data[to_flat_index(i, ndim, shape, stride, offset)] = uniform_sample_f64(low, high, &st);
+    }
+}
 /* identity op into a dense result (cpu/unary.cpp:26-58) */
 void tto_contiguous(const void *src, void *dst, int elem_size, int ndim, const int *shape, const int *stride,
                     int offset) {

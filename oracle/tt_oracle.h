@@ -34,6 +34,9 @@
  *   tto_splitmix64 / xorshift64  published test vectors (Vigna's splitmix64.c
  *                         seed 1234567 stream; xorshift64 13/7/17 closed form).
  *   tto_uniform_real_*    closed form from the bit construction.
+ *   tto_uniform_real_view_*  the dense draw in the view's order scattered by explicit index loops
+ *                         (brute force), and numpy's transposition of the dense draw for the
+ *                         permuted view that nn::Conv2d's initialisation uses.
  *   tto_normal_*          closed form: every element's (u1, u2) rebuilt from the integer
  *                         generator and mu + std*sqrt(-2*log1p(-u1))*sin(2*pi*u2) evaluated
  *                         with 200-bit transcendentals, each step rounded to the type; f32
@@ -75,6 +78,14 @@ void tto_uniform_real_f32(uint64_t *state, float low, float high, float *out, in
 void tto_uniform_real_f64(uint64_t *state, double low, double high, double *out, int64_t n);
 void tto_normal_f32(uint64_t *state, float mu, float std, float *out, int64_t n);
 void tto_normal_f64(uint64_t *state, double mu, double std, double *out, int64_t n);
+
+/* In-place uniform draws through a strided view (cpu/distribution.cpp:96-139, cpu/kernel/distribution.hpp:28-32):
+ * the i-th element of the view in row-major order of `shape` takes the i-th master output as its state and lands
+ * at data[offset + sum(index[d]*stride[d])].  Strides and offset in elements. */
+void tto_uniform_real_view_f32(uint64_t *state, float low, float high, float *data, int ndim, const int *shape,
+                               const int *stride, int offset);
+void tto_uniform_real_view_f64(uint64_t *state, double low, double high, double *data, int ndim, const int *shape,
+                               const int *stride, int offset);
 
 /* ---- strided view -> dense copy (Tensor::contiguous via the identity op:
  * cpu/unary.cpp:26-58 with common/util.h:18-34) ---- */

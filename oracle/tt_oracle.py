@@ -53,7 +53,10 @@ def _load(flavour: str) -> C.CDLL:
     lib.tto_uniform_real_f64.argtypes = [u64p, C.c_double, C.c_double, vp, i64]
     lib.tto_normal_f32.argtypes = [u64p, C.c_float, C.c_float, vp, i64]
     lib.tto_normal_f64.argtypes = [u64p, C.c_double, C.c_double, vp, i64]
-    for f in ("tto_uniform_real_f32", "tto_uniform_real_f64", "tto_normal_f32", "tto_normal_f64"):
+    lib.tto_uniform_real_view_f32.argtypes = [u64p, C.c_float, C.c_float, vp, i32, ip, ip, i32]
+    lib.tto_uniform_real_view_f64.argtypes = [u64p, C.c_double, C.c_double, vp, i32, ip, ip, i32]
+    for f in ("tto_uniform_real_f32", "tto_uniform_real_f64", "tto_normal_f32", "tto_normal_f64", "tto_uniform_real_view_f32",
+              "tto_uniform_real_view_f64"):
         getattr(lib, f).restype = None
     lib.tto_contiguous.restype = None
     lib.tto_contiguous.argtypes = [vp, vp, i32, i32, ip, ip, i32]
@@ -121,6 +124,13 @@ class Generator:
         fn = lib().tto_uniform_real_f32 if out.dtype == np.float32 else lib().tto_uniform_real_f64
         fn(C.byref(self._state), low, high, _ptr(out), out.size)
         return out.reshape(shape)
+
+    def uniform_real_(self, view: np.ndarray, low: float, high: float) -> None:
+        """Tensor::uniform_real_ on a strided view, in place (cpu/distribution.cpp:96-139): `view` is any numpy view
+        with non-negative strides; its elements are drawn in the view's own row-major order."""
+        base, offset = view_base(view)
+        fn = lib().tto_uniform_real_view_f32 if view.dtype == np.float32 else lib().tto_uniform_real_view_f64
+        fn(C.byref(self._state), low, high, _ptr(base), view.ndim, _ints(view.shape), _ints(elem_strides(view)), offset)
 
     def normal(self, mu: float, std: float, shape, dtype=np.float32) -> np.ndarray:
         out = np.empty(int(np.prod(shape)), dtype=dtype)
@@ -299,4 +309,19 @@ def linear_init(gen: Generator, in_features: int, out_features: int, dtype=np.fl
     W = gen.uniform_real(-bound_w, bound_w, (in_features, out_features), dtype)
     bound_b = 1.0 / np.sqrt(fan)
     b = gen.uniform_real(-bound_b, bound_b, (out_features,), dtype)
+    return W, b
+
+
+def conv2d_init(gen: Generator, in_channels: int, out_channels: int, kernel_size: int, bias: bool = True, dtype=np.float32):
+    """nn::Conv2d default init (nn/conv2d.cpp:20-66): weight [O,C,k,k] drawn IN PLACE through the view
+    weight.permute(1,0,2,3) by kaiming_uniform_ (fan = view.size(0)*k*k = C*k*k, nn/init.cpp:30-52,106-112), then bias
+    ~ U(+-1/sqrt(fan)) with fan = calc_fan_in_out(weight) = O*k*k."""
+    k = kernel_size
+    W = np.zeros((out_channels, in_channels, k, k), dtype=dtype)
+    bound_w = np.sqrt(3.0) * (1.0 / np.sqrt(float(in_channels * k * k)))
+    gen.uniform_real_(W.transpose(1, 0, 2, 3), -bound_w, bound_w)
+    b = None
+    if bias:
+        bound_b = 1.0 / np.sqrt(float(out_channels * k * k))
+        b = gen.uniform_real(-bound_b, bound_b, (out_channels,), dtype)
     return W, b

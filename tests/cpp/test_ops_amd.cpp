@@ -259,6 +259,65 @@ TEST_CASE("Seeded draws and Linear default init") {
     CHECK(allclose(Y.to_vec<float>(), (matmul(X, layer.weight) + *layer.bias).to_vec<float>(), 1e-5, 1e-6));
 }
 
+TEST_CASE("Conv2d default init through the permuted view") {
+    // nn::Conv2d (nn/conv2d.cpp:20-66): kaiming_uniform_ on weight.permute({1,0,2,3}) -- the draws run over [in,out,k,k]
+    // with fan = in*k*k -- then the bias with fan = out*k*k.  Stated independently: a dense draw of [in,out,k,k],
+    // permuted back and made contiguous.
+    const int in = 5, out = 12, k = 3;
+    Generator gl(11), gr(11);
+    const nn::Conv2d layer(in, out, k, 1, 1, true, gl);
+    CHECK(layer.weight.shape() == Shape({out, in, k, k}));
+    CHECK(layer.weight.is_contiguous());
+    const double bw = std::sqrt(3.0) * (1.0 / std::sqrt(static_cast<double>(in * k * k))), bb = 1.0 / std::sqrt(static_cast<double>(out * k * k));
+    const Tensor dense = uniform_real(-bw, bw, {in, out, k, k}, gr);
+    CHECK(layer.weight.to_vec<float>() == dense.permute({1, 0, 2, 3}).to_vec<float>());
+    CHECK(layer.weight.to_vec<float>() != dense.to_vec<float>());
+    CHECK(layer.bias->to_vec<float>() == uniform_real(-bb, bb, {out}, gr).to_vec<float>());
+    CHECK(gl.state == gr.state);
+    // in-place draws through a view leave the rest of the storage alone
+    Tensor base = full(-7.0f, Shape({4, 6}), kAMD).contiguous();
+    Generator g1(5), g2(5);
+    Tensor cols = base.permute({1, 0});  // [6,4] view with strides (1,6)
+    cols.uniform_real_(0.0, 1.0, g1);
+    CHECK(base.to_vec<float>() == uniform_real(0.0, 1.0, {6, 4}, g2).permute({1, 0}).to_vec<float>());
+    // forward = conv2d with the layer's stride and padding
+    const Tensor x = uniform_real(-1.0, 1.0, {2, in, 9, 9}, gr);
+    const Tensor y = layer.forward(x);
+    CHECK(y.shape() == Shape({2, out, 9, 9}));
+    CHECK(y.to_vec<float>() == conv2d(x, layer.weight, layer.bias, 1, 1).to_vec<float>());
+    CHECK_THROWS_AS(std::ignore = layer.forward(uniform_real(-1.0, 1.0, {2, in + 1, 9, 9}, gr)), TTException);
+    CHECK_THROWS_AS(nn::Conv2d(0, 4, 3, 1, 0, true, gl), TTException);
+    CHECK_THROWS_AS(nn::Conv2d(4, 4, 3, 0, 0, true, gl), TTException);
+    CHECK_THROWS_AS(nn::Conv2d(4, 4, 3, 1, -1, true, gl), TTException);
+}
+
+TEST_CASE("Integer sums are 64-bit") {
+    // common/reduce.h:56-61: sums of bool and integer tensors accumulate in int64 and return an i64 tensor
+    auto test = []<typename T>(Device device) {
+        if constexpr (std::is_integral_v<T>) {
+            const int N = 60000;
+            std::vector<T> a;
+            int64_t total = 0;
+            for (int i = 0; i < N; ++i) {
+                a.push_back(static_cast<T>(100 + i % 27));
+                total += 100 + i % 27;
+            }
+            const Tensor A(a, {600, 100}, device);
+            CHECK(A.sum().dtype() == kI64);
+            CHECK(A.sum().template to_vec<int64_t>() == std::vector<int64_t>{total});  // 6.7e6: beyond u8 and i16
+            std::vector<int64_t> cols(100, 0);
+            for (int i = 0; i < N; ++i) cols[static_cast<std::size_t>(i % 100)] += static_cast<int64_t>(a[static_cast<std::size_t>(i)]);
+            CHECK(A.sum(0).template to_vec<int64_t>() == cols);
+        }
+    };
+    runner_all_except_bool(test);
+    std::vector<bool> m;
+    for (int i = 0; i < 1000; ++i) m.push_back(i % 3 == 0);
+    const Tensor M(m, {10, 100}, kAMD);
+    CHECK(M.sum().dtype() == kI64);
+    CHECK(M.sum().to_vec<int64_t>() == std::vector<int64_t>{334});
+}
+
 namespace {
 struct MlpGrads {
     Tensor loss, dW1, db1, dW2, db2, dW3, db3, dX;

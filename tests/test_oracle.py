@@ -410,3 +410,47 @@ def test_linear_default_init(oracle):
     W2 = g2.uniform_real(-bw, bw, (784, 16))
     assert np.array_equal(W, W2)
     assert abs(W.astype(np.float64).var() - bw * bw / 3) < 2e-5
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+def test_in_place_draw_through_a_view_brute_force(oracle, dtype):
+    # Tensor::uniform_real_ on a view (cpu/kernel/distribution.hpp:28-32): the i-th element in the view's row-major
+    # order takes the i-th draw.  Independent statement: the dense draw of the same generator, scattered by explicit
+    # index loops over the view's shape -- for a permuted view with an offset, and for a sliced (strided) one.
+    base = np.full((5, 4, 3, 6), -7.0, dtype=dtype)
+    view = base.transpose(1, 0, 2, 3)[1:, :, :, 2:5]  # shape [3,5,3,3], offset and non-dense strides
+    g = oracle.Generator(9)
+    g.uniform_real_(view, -0.5, 0.25)
+    dense = oracle.Generator(9).uniform_real(-0.5, 0.25, (view.size,), dtype)
+    want = np.full((5, 4, 3, 6), -7.0, dtype=dtype)
+    i = 0
+    for a in range(3):
+        for b in range(5):
+            for c in range(3):
+                for d in range(3):
+                    want[b, a + 1, c, d + 2] = dense[i]
+                    i += 1
+    assert np.array_equal(base, want)  # the drawn elements AND the untouched ones
+    g2 = oracle.Generator(9)
+    g2.uniform_real(-0.5, 0.25, (view.size,), dtype)
+    assert g.state == g2.state  # one master output per element, nothing else
+
+
+def test_conv2d_default_init(oracle):
+    # nn::Conv2d(3, 8, 5): weight [8,3,5,5] drawn through permute(1,0,2,3) with fan = 3*25 (the VIEW's size(0)), then
+    # bias with fan = 8*25 (the weight's size(0)).  Independent statement: draw [3,8,5,5] densely, transpose with numpy.
+    C_, O_, k = 3, 8, 5
+    W, b = oracle.conv2d_init(oracle.Generator(4), C_, O_, k)
+    assert W.shape == (O_, C_, k, k) and b.shape == (O_,)
+    g = oracle.Generator(4)
+    bw = np.sqrt(3.0) / np.sqrt(C_ * k * k)
+    dense = g.uniform_real(-bw, bw, (C_, O_, k, k))
+    assert np.array_equal(W, dense.transpose(1, 0, 2, 3))
+    assert not np.array_equal(W, dense.reshape(O_, C_, k, k))  # a dense draw in storage order is a different tensor
+    bb = 1.0 / np.sqrt(O_ * k * k)
+    assert np.array_equal(b, g.uniform_real(-bb, bb, (O_,)))
+    assert np.abs(W).max() < bw and np.abs(W).max() > 0.95 * bw and np.abs(b).max() < bb
+    # the bias bound uses the out-channel fan: with the in-channel fan (1/sqrt(75) = 0.115) values up to that would appear
+    assert bb < 0.0708 and np.abs(b).max() > 0.5 * bb
+    Wn, bn = oracle.conv2d_init(oracle.Generator(4), C_, O_, k, bias=False)
+    assert bn is None and np.array_equal(Wn, W)

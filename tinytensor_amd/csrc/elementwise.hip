@@ -341,24 +341,28 @@ __global__ void __launch_bounds__(256) full_kernel(T *__restrict__ out, T value,
     for (int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < numel; i += step) out[i] = value;
 }
 
+// Sums read elements of type T and accumulate in A: A = T for the float types; every integer type (and bool) is summed
+// into int64, which is also the result's type (common/reduce.h:56-61: "sum reductions on low width int types get cast to
+// larger width to circumvent overflows"; cpu/reduce.cpp:38-54 allocates the result as that type).
+//
 // sum over one dimension: one lane per output element walks the reduced dimension in index order, which is
 // the order of the reference's reduce_dim_kernel (cpu/kernel/reduce.hpp:15-32).  `outer` = view without `dim`.
-template <typename T>
+template <typename T, typename A>
 __global__ void __launch_bounds__(256) sum_dim_kernel(const T *__restrict__ a, ViewDesc outer, int64_t dim_len, int64_t dim_stride,
-                                                     T *__restrict__ out, int64_t n_out) {
+                                                     A *__restrict__ out, int64_t n_out) {
     const int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
     if (i >= n_out) return;
     const T *p = a + flat_of(i, outer);
-    T acc = T(0);
+    A acc = A(0);
     int64_t j = 0;
     for (; j + 8 <= dim_len; j += 8) {  // eight loads in flight, added in index order
         T v[8];
 #pragma unroll
         for (int u = 0; u < 8; ++u) v[u] = p[(j + u) * dim_stride];
 #pragma unroll
-        for (int u = 0; u < 8; ++u) acc = static_cast<T>(acc + v[u]);
+        for (int u = 0; u < 8; ++u) acc = static_cast<A>(acc + static_cast<A>(v[u]));
     }
-    for (; j < dim_len; ++j) acc = static_cast<T>(acc + p[j * dim_stride]);
+    for (; j < dim_len; ++j) acc = static_cast<A>(acc + static_cast<A>(p[j * dim_stride]));
     out[i] = acc;
 }
 
@@ -368,51 +372,51 @@ __global__ void __launch_bounds__(256) sum_dim_kernel(const T *__restrict__ a, V
 //    partial sums per slice go to scratch and a second sum_dim_kernel adds them in slice order;
 //  * rows (the reduced dimension has unit stride): one wavefront per output, lanes stride the dimension and combine
 //    with a shuffle tree.
-template <typename T>
+template <typename T, typename A>
 __global__ void __launch_bounds__(256) sum_dim_cols_kernel(const T *__restrict__ a, ViewDesc outer, int64_t dim_len, int64_t dim_stride,
-                                                          T *__restrict__ partial, int64_t n_out, int64_t rows_per_slice) {
-    __shared__ T red[4][64];
+                                                          A *__restrict__ partial, int64_t n_out, int64_t rows_per_slice) {
+    __shared__ A red[4][64];
     const int ol = threadIdx.x % 64, rl = threadIdx.x / 64;
     const int64_t o = static_cast<int64_t>(blockIdx.x) * 64 + ol;
     const int64_t r0 = static_cast<int64_t>(blockIdx.y) * rows_per_slice;
     const int64_t r1 = r0 + rows_per_slice < dim_len ? r0 + rows_per_slice : dim_len;
-    T acc = T(0);
+    A acc = A(0);
     if (o < n_out) {
         const T *p = a + flat_of(o, outer);
-        for (int64_t r = r0 + rl; r < r1; r += 4) acc = static_cast<T>(acc + p[r * dim_stride]);
+        for (int64_t r = r0 + rl; r < r1; r += 4) acc = static_cast<A>(acc + static_cast<A>(p[r * dim_stride]));
     }
     red[rl][ol] = acc;
     __syncthreads();
     if (rl == 0 && o < n_out)
         partial[static_cast<int64_t>(blockIdx.y) * n_out + o] =
-            static_cast<T>(static_cast<T>(red[0][ol] + red[1][ol]) + static_cast<T>(red[2][ol] + red[3][ol]));
+            static_cast<A>(static_cast<A>(red[0][ol] + red[1][ol]) + static_cast<A>(red[2][ol] + red[3][ol]));
 }
 
-template <typename T>
-__global__ void __launch_bounds__(256) sum_dim_rows_kernel(const T *__restrict__ a, ViewDesc outer, int64_t dim_len, T *__restrict__ out,
+template <typename T, typename A>
+__global__ void __launch_bounds__(256) sum_dim_rows_kernel(const T *__restrict__ a, ViewDesc outer, int64_t dim_len, A *__restrict__ out,
                                                           int64_t n_out) {
-    __shared__ T red[4][64];
+    __shared__ A red[4][64];
     const int lane = threadIdx.x % 64, w = threadIdx.x / 64;
     const int64_t o = static_cast<int64_t>(blockIdx.x) * 4 + w;
-    T acc = T(0);
+    A acc = A(0);
     if (o < n_out) {
         const T *p = a + flat_of(o, outer);
-        for (int64_t j = lane; j < dim_len; j += 64) acc = static_cast<T>(acc + p[j]);
+        for (int64_t j = lane; j < dim_len; j += 64) acc = static_cast<A>(acc + static_cast<A>(p[j]));
     }
     red[w][lane] = acc;
     __syncthreads();
     for (int h = 32; h > 0; h >>= 1) {
-        if (lane < h) red[w][lane] = static_cast<T>(red[w][lane] + red[w][lane + h]);
+        if (lane < h) red[w][lane] = static_cast<A>(red[w][lane] + red[w][lane + h]);
         __syncthreads();
     }
     if (lane == 0 && o < n_out) out[o] = red[w][0];
 }
 
 // sum of everything: per-workgroup partial sums (stage 1) then one workgroup adds the partials (stage 2).
-template <typename T>
-__global__ void __launch_bounds__(256) sum_all_kernel(const T *__restrict__ a, ViewDesc v, bool dense, int64_t numel, T *__restrict__ out) {
-    __shared__ T red[256];
-    T acc = T(0);
+template <typename T, typename A>
+__global__ void __launch_bounds__(256) sum_all_kernel(const T *__restrict__ a, ViewDesc v, bool dense, int64_t numel, A *__restrict__ out) {
+    __shared__ A red[256];
+    A acc = A(0);
     const int64_t step = static_cast<int64_t>(gridDim.x) * blockDim.x;
     int64_t first = 0;  // elements [0, first) are covered by 16-byte loads
     if (dense && reinterpret_cast<uintptr_t>(a) % 16 == 0) {
@@ -421,16 +425,16 @@ __global__ void __launch_bounds__(256) sum_all_kernel(const T *__restrict__ a, V
         for (int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < nvec; i += step) {
             const vec_t<T, N> x = stream_load(reinterpret_cast<const vec_t<T, N> *>(a) + i);
 #pragma unroll
-            for (int j = 0; j < N; ++j) acc = static_cast<T>(acc + x[j]);
+            for (int j = 0; j < N; ++j) acc = static_cast<A>(acc + static_cast<A>(x[j]));
         }
         first = nvec * N;
     }
     for (int64_t i = first + static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < numel; i += step)
-        acc = static_cast<T>(acc + (dense ? a[i] : a[flat_of(i, v)]));
+        acc = static_cast<A>(acc + static_cast<A>(dense ? a[i] : a[flat_of(i, v)]));
     red[threadIdx.x] = acc;
     __syncthreads();
     for (int s = 128; s > 0; s >>= 1) {
-        if (static_cast<int>(threadIdx.x) < s) red[threadIdx.x] = static_cast<T>(red[threadIdx.x] + red[threadIdx.x + s]);
+        if (static_cast<int>(threadIdx.x) < s) red[threadIdx.x] = static_cast<A>(red[threadIdx.x] + red[threadIdx.x + s]);
         __syncthreads();
     }
     if (threadIdx.x == 0) out[blockIdx.x] = red[0];
@@ -451,16 +455,20 @@ __device__ __forceinline__ float unit_sample(uint64_t &st, float) {
 __device__ __forceinline__ double unit_sample(uint64_t &st, double) {
     return __builtin_bit_cast(double, (xorshift64(st) >> 12) | 0x3FF0000000000000ull) - 1.0;
 }
+// Element i of the view (row-major rank over its shape) takes state i and is written at the view's address of that
+// rank, as the in-place kernel of the CPU backend does (cpu/kernel/distribution.hpp:28-32 with common/util.h:18-34).
 template <typename T>
-__global__ void __launch_bounds__(256) uniform_real_kernel(const uint64_t *__restrict__ states, T low, T high, T *__restrict__ out, int64_t n) {
+__global__ void __launch_bounds__(256) uniform_real_kernel(const uint64_t *__restrict__ states, T low, T high, T *__restrict__ out, ViewDesc v,
+                                                          bool dense, int64_t n) {
     const int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
     if (i >= n) return;
     uint64_t st = states[i];
     const T r = unit_sample(st, T(0));
-    out[i] = fma(r, high - low, low);  // r * (high - low) + low, contracted as the fma flavour of the host build does
+    out[dense ? i : flat_of(i, v)] = fma(r, high - low, low);  // r * (high - low) + low, contracted as the fma flavour of the host build does
 }
 template <typename T>
-__global__ void __launch_bounds__(256) normal_kernel(const uint64_t *__restrict__ states, T mu, T stddev, T *__restrict__ out, int64_t n) {
+__global__ void __launch_bounds__(256) normal_kernel(const uint64_t *__restrict__ states, T mu, T stddev, T *__restrict__ out, ViewDesc v,
+                                                    bool dense, int64_t n) {
     const int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
     if (i >= n) return;
     uint64_t st = states[i];
@@ -468,7 +476,7 @@ __global__ void __launch_bounds__(256) normal_kernel(const uint64_t *__restrict_
     const T u2 = unit_sample(st, T(0));
     const T r = sqrt(T(-2) * log1p(-u1));
     const T theta = T(2) * T(3.14159265358979323846) * u2;
-    out[i] = stddev * (r * sin(theta)) + mu;
+    out[dense ? i : flat_of(i, v)] = stddev * (r * sin(theta)) + mu;
 }
 
 // to(dtype): out[i] = static_cast<R>(view[i]) (tinytensor/tensor/backend/cpu/cast.cpp:27-34; bool keeps C++'s
@@ -641,20 +649,21 @@ ttamd_status dispatch_unary(int op, const void *a, const ViewDesc &va, void *out
 
 template <typename T>
 ttamd_status sum_typed(int device, const void *a, const ViewDesc &v, int64_t numel, int dim, void *out, hipStream_t st) {
+    using A = std::conditional_t<std::is_floating_point_v<T>, T, int64_t>;  // accumulator and result type
     const T *src = static_cast<const T *>(a);
     if (dim < 0) {
         const unsigned blocks = numel > (1 << 22) ? 2048 : (numel > 256 * 64 ? 256 : 1);
         if (blocks == 1) {
-            sum_all_kernel<T><<<dim3(1), dim3(256), 0, st>>>(src, v, is_dense(v), numel, static_cast<T *>(out));
+            sum_all_kernel<T, A><<<dim3(1), dim3(256), 0, st>>>(src, v, is_dense(v), numel, static_cast<A *>(out));
         } else {
             void *ws = nullptr;
-            if (ttamd_status s = stream_scratch(device, st, blocks * sizeof(T), &ws)) return s;
-            sum_all_kernel<T><<<dim3(blocks), dim3(256), 0, st>>>(src, v, is_dense(v), numel, static_cast<T *>(ws));
+            if (ttamd_status s = stream_scratch(device, st, blocks * sizeof(A), &ws)) return s;
+            sum_all_kernel<T, A><<<dim3(blocks), dim3(256), 0, st>>>(src, v, is_dense(v), numel, static_cast<A *>(ws));
             ViewDesc pv{};
             pv.ndim = 1;
             pv.shape[0] = blocks;
             pv.stride[0] = 1;
-            sum_all_kernel<T><<<dim3(1), dim3(256), 0, st>>>(static_cast<const T *>(ws), pv, true, blocks, static_cast<T *>(out));
+            sum_all_kernel<A, A><<<dim3(1), dim3(256), 0, st>>>(static_cast<const A *>(ws), pv, true, blocks, static_cast<A *>(out));
         }
         TTAMD_HIP_CHECK(hipGetLastError());
         return TTAMD_OK;
@@ -671,7 +680,7 @@ ttamd_status sum_typed(int device, const void *a, const ViewDesc &v, int64_t num
     const int64_t dim_len = v.shape[dim], dim_stride = v.stride[dim];
     if (n_out < 32768 && dim_len >= 128) {
         if (dim_stride == 1) {
-            sum_dim_rows_kernel<T><<<dim3(static_cast<unsigned>((n_out + 3) / 4)), dim3(256), 0, st>>>(src, outer, dim_len, static_cast<T *>(out), n_out);
+            sum_dim_rows_kernel<T, A><<<dim3(static_cast<unsigned>((n_out + 3) / 4)), dim3(256), 0, st>>>(src, outer, dim_len, static_cast<A *>(out), n_out);
             TTAMD_HIP_CHECK(hipGetLastError());
             return TTAMD_OK;
         }
@@ -683,21 +692,21 @@ ttamd_status sum_typed(int device, const void *a, const ViewDesc &v, int64_t num
             const int64_t rows_per_slice = (dim_len + slices - 1) / slices;
             slices = (dim_len + rows_per_slice - 1) / rows_per_slice;
             void *ws = nullptr;
-            if (ttamd_status s = stream_scratch(device, st, static_cast<size_t>(slices) * n_out * sizeof(T), &ws)) return s;
-            sum_dim_cols_kernel<T><<<dim3(static_cast<unsigned>(col_blocks), static_cast<unsigned>(slices)), dim3(256), 0, st>>>(
-                src, outer, dim_len, dim_stride, static_cast<T *>(ws), n_out, rows_per_slice);
+            if (ttamd_status s = stream_scratch(device, st, static_cast<size_t>(slices) * n_out * sizeof(A), &ws)) return s;
+            sum_dim_cols_kernel<T, A><<<dim3(static_cast<unsigned>(col_blocks), static_cast<unsigned>(slices)), dim3(256), 0, st>>>(
+                src, outer, dim_len, dim_stride, static_cast<A *>(ws), n_out, rows_per_slice);
             ViewDesc flat{};
             flat.ndim = 1;
             flat.shape[0] = n_out;
             flat.stride[0] = 1;
-            sum_dim_kernel<T><<<dim3(static_cast<unsigned>((n_out + 255) / 256)), dim3(256), 0, st>>>(static_cast<const T *>(ws), flat, slices, n_out,
-                                                                                                    static_cast<T *>(out), n_out);
+            sum_dim_kernel<A, A><<<dim3(static_cast<unsigned>((n_out + 255) / 256)), dim3(256), 0, st>>>(static_cast<const A *>(ws), flat, slices, n_out,
+                                                                                                       static_cast<A *>(out), n_out);
             TTAMD_HIP_CHECK(hipGetLastError());
             return TTAMD_OK;
         }
     }
-    sum_dim_kernel<T><<<dim3(static_cast<unsigned>((n_out + 255) / 256)), dim3(256), 0, st>>>(src, outer, v.shape[dim], v.stride[dim],
-                                                                                              static_cast<T *>(out), n_out);
+    sum_dim_kernel<T, A><<<dim3(static_cast<unsigned>((n_out + 255) / 256)), dim3(256), 0, st>>>(src, outer, v.shape[dim], v.stride[dim],
+                                                                                                 static_cast<A *>(out), n_out);
     TTAMD_HIP_CHECK(hipGetLastError());
     return TTAMD_OK;
 }
@@ -1005,7 +1014,7 @@ ttamd_status ttamd_sum(int device, ttamd_dtype dtype, int ndim, const int64_t *s
     int64_t numel = 0;
     if (ttamd_status s = make_view("sum", ndim, shape, stride, &va, &numel)) return s;
     const size_t esz = dtype_size(dtype);
-    if (dtype <= TTAMD_BOOL || dtype > TTAMD_F64 || esz == 0) {
+    if (dtype < TTAMD_BOOL || dtype > TTAMD_F64 || esz == 0) {
         set_error("sum: unsupported dtype code %d", static_cast<int>(dtype));
         return TTAMD_ERR_UNSUPPORTED_DTYPE;
     }
@@ -1020,6 +1029,7 @@ ttamd_status ttamd_sum(int device, ttamd_dtype dtype, int ndim, const int64_t *s
     }
     const void *a = static_cast<const char *>(src) + offset * static_cast<int64_t>(esz);
     hipStream_t st = static_cast<hipStream_t>(stream);
+    if (dtype == TTAMD_BOOL) return sum_typed<uint8_t>(device, a, va, numel, dim, out, st);  // one byte holding 0 or 1
     TTAMD_DISPATCH_DTYPE(dtype, (sum_typed<T_>(device, a, va, numel, dim, out, st)))
     return TTAMD_ERR_UNSUPPORTED_DTYPE;
 }
@@ -1059,23 +1069,28 @@ ttamd_status ttamd_full(int device, ttamd_dtype dtype, const void *value, int64_
 
 
 // dist: 0 = uniform_real(low = p0, high = p1), 1 = normal(mu = p0, std = p1).  *master_state is the host-side master
-// generator state (Generator::state); it advances by n outputs.
-ttamd_status ttamd_random_fill(int device, ttamd_dtype dtype, int dist, double p0, double p1, uint64_t *master_state, int64_t numel,
-                               void *out, void *stream) {
+// generator state (Generator::state); it advances by one output per element of the view.
+ttamd_status ttamd_random_fill_view(int device, ttamd_dtype dtype, int dist, double p0, double p1, uint64_t *master_state, int ndim,
+                                    const int64_t *shape, const int64_t *stride, void *data, int64_t offset, void *stream) {
     if (dtype != TTAMD_F32 && dtype != TTAMD_F64) {
         set_error("random_fill: floating point dtypes only");
         return TTAMD_ERR_UNSUPPORTED_DTYPE;
     }
-    if (!master_state || numel < 0 || (dist != 0 && dist != 1) || (dist == 0 && !(p0 < p1))) {
+    if (!master_state || offset < 0 || (dist != 0 && dist != 1) || (dist == 0 && !(p0 < p1))) {
         set_error("random_fill: invalid arguments (Expected low < high for uniform_real)");
         return TTAMD_ERR_INVALID_ARGUMENT;
     }
+    ViewDesc v;
+    int64_t numel = 0;
+    if (ttamd_status s = make_view("random_fill", ndim, shape, stride, &v, &numel)) return s;
     if (ttamd_status s = use_device(device)) return s;
     if (numel == 0) return TTAMD_OK;
-    if (!out) {
-        set_error("random_fill: out is NULL");
+    if (!data) {
+        set_error("random_fill: data is NULL");
         return TTAMD_ERR_INVALID_ARGUMENT;
     }
+    const bool dense = is_dense(v);
+    void *out = static_cast<char *>(data) + offset * static_cast<int64_t>(dtype_size(dtype));
     hipStream_t st = static_cast<hipStream_t>(stream);
     // per-element generator states, produced on the host in order (cpu/distribution.cpp:31-38)
     uint64_t *host_states = nullptr;
@@ -1107,11 +1122,11 @@ ttamd_status ttamd_random_fill(int device, ttamd_dtype dtype, int dist, double p
         const unsigned blocks = static_cast<unsigned>((numel + 255) / 256);
         const uint64_t *sp = static_cast<const uint64_t *>(dev_states);
         if (dtype == TTAMD_F32) {
-            if (dist == 0) uniform_real_kernel<float><<<dim3(blocks), dim3(256), 0, st>>>(sp, static_cast<float>(p0), static_cast<float>(p1), static_cast<float *>(out), numel);
-            else normal_kernel<float><<<dim3(blocks), dim3(256), 0, st>>>(sp, static_cast<float>(p0), static_cast<float>(p1), static_cast<float *>(out), numel);
+            if (dist == 0) uniform_real_kernel<float><<<dim3(blocks), dim3(256), 0, st>>>(sp, static_cast<float>(p0), static_cast<float>(p1), static_cast<float *>(out), v, dense, numel);
+            else normal_kernel<float><<<dim3(blocks), dim3(256), 0, st>>>(sp, static_cast<float>(p0), static_cast<float>(p1), static_cast<float *>(out), v, dense, numel);
         } else {
-            if (dist == 0) uniform_real_kernel<double><<<dim3(blocks), dim3(256), 0, st>>>(sp, p0, p1, static_cast<double *>(out), numel);
-            else normal_kernel<double><<<dim3(blocks), dim3(256), 0, st>>>(sp, p0, p1, static_cast<double *>(out), numel);
+            if (dist == 0) uniform_real_kernel<double><<<dim3(blocks), dim3(256), 0, st>>>(sp, p0, p1, static_cast<double *>(out), v, dense, numel);
+            else normal_kernel<double><<<dim3(blocks), dim3(256), 0, st>>>(sp, p0, p1, static_cast<double *>(out), v, dense, numel);
         }
         if ((e = hipGetLastError()) != hipSuccess) fail(e, "kernel launch");
     }
@@ -1120,6 +1135,17 @@ ttamd_status ttamd_random_fill(int device, ttamd_dtype dtype, int dist, double p
     (void)hipFree(dev_states);
     (void)hipHostFree(host_states);
     return rc;
+}
+
+// The dense case of ttamd_random_fill_view: `out` is a dense tensor of numel elements.
+ttamd_status ttamd_random_fill(int device, ttamd_dtype dtype, int dist, double p0, double p1, uint64_t *master_state, int64_t numel,
+                               void *out, void *stream) {
+    if (numel < 0) {
+        set_error("random_fill: negative element count");
+        return TTAMD_ERR_INVALID_ARGUMENT;
+    }
+    const int64_t shape[1] = {numel}, stride[1] = {1};
+    return ttamd_random_fill_view(device, dtype, dist, p0, p1, master_state, 1, shape, stride, out, 0, stream);
 }
 
 }  // extern "C"

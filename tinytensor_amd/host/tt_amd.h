@@ -110,6 +110,18 @@ private:
     std::vector<int> dims_;
 };
 
+// Element count of a result, computed in 64 bits: a tensor's numel and every index the library uses fit an int
+// (include/tt/shape.h:122), so anything beyond is refused instead of wrapping around into a tiny allocation.
+inline auto checked_numel(std::initializer_list<int64_t> extents) -> std::size_t {
+    int64_t n = 1;
+    for (int64_t e : extents) {
+        if (e < 0) throw TTException("negative extent");
+        n *= e;
+        if (n > static_cast<int64_t>(INT32_MAX)) throw TTException("tensor has more than 2^31 - 1 elements");
+    }
+    return static_cast<std::size_t>(n);
+}
+
 // Owning device allocation (peer of the reference's DeviceMemory<T>, cuda/data_types.cuh:28-101).
 class StorageAMD {
 public:
@@ -220,6 +232,17 @@ public:
     [[nodiscard]] auto sum() const -> Tensor;
     [[nodiscard]] auto sum(int dim) const -> Tensor;
     auto assign(const Tensor &rhs) -> Tensor &;  // writes rhs's elements through this view
+    // Tensor::uniform_real_(low, high, gen) / normal_(mu, std, gen) (tensor.cpp:1783-1801): in place, through this view
+    template <typename Gen> auto uniform_real_(double low, double high, Gen &gen) -> Tensor &;
+    template <typename Gen> auto normal_(double mu, double std, Gen &gen) -> Tensor &;
+    // an uninitialised dense tensor (the layers below overwrite every element; the reference starts from zeros())
+    static auto empty(const Shape &shape, ScalarType dtype, Device device) -> Tensor {
+        std::vector<int64_t> ext(shape.to_vec().begin(), shape.to_vec().end());
+        int64_t n = 1;
+        for (int64_t e : ext) n *= e;
+        if (n < 0 || n > static_cast<int64_t>(INT32_MAX)) throw TTException("tensor has more than 2^31 - 1 elements");
+        return {std::make_shared<StorageAMD>(static_cast<std::size_t>(n) * dtype_size(dtype), device.id), dtype, shape, device};
+    }
 
     static auto dense_stride(const Shape &shape) -> Shape {
         std::vector<int> st(static_cast<std::size_t>(shape.ndim()), 1);
@@ -263,7 +286,7 @@ public:
     [[nodiscard]] auto batched_matmul(const Tensor &lhs, const Tensor &rhs, const ttamd_epilogue *epilogue = nullptr) const -> Tensor {
         const int B = lhs.size(0), N = lhs.size(1), K = lhs.size(2), M = rhs.size(2);
         const ttamd_view3 l = view3(lhs), r = view3(rhs);
-        auto out = std::make_shared<StorageAMD>(static_cast<std::size_t>(B) * N * M * dtype_size(lhs.dtype()), lhs.device().id);
+        auto out = std::make_shared<StorageAMD>(checked_numel({B, N, M}) * dtype_size(lhs.dtype()), lhs.device().id);
         check(ttamd_batched_matmul(lhs.device().id, static_cast<ttamd_dtype>(lhs.dtype()), B, N, K, M, &l, &r, out->ptr_, epilogue, nullptr));
         return {out, lhs.dtype(), Shape({B, N, M}), lhs.device()};
     }
@@ -274,7 +297,9 @@ public:
         const Tensor w = weight.contiguous();  // used as the matrix [O, C*k*k], as cpu/conv.cpp:69 reshapes it
         const std::optional<Tensor> b = bias ? std::optional<Tensor>(bias->contiguous()) : std::nullopt;
         const ttamd_view4 iv = view4(input), wv = view4(w);
-        auto out = std::make_shared<StorageAMD>(static_cast<std::size_t>(std::max(B * O * Ho * Wo, 0)) * dtype_size(input.dtype()), input.device().id);
+        if (Ho <= 0 || Wo <= 0) throw TTException("conv2d: the kernel does not fit the padded input");
+        checked_numel({B, C, H, W});
+        auto out = std::make_shared<StorageAMD>(checked_numel({B, O, Ho, Wo}) * dtype_size(input.dtype()), input.device().id);
         check(ttamd_conv2d_forward(input.device().id, static_cast<ttamd_dtype>(input.dtype()), &iv, &wv, b ? b->data_ptr() : nullptr, out->ptr_,
                                    B, C, H, W, O, k, stride, padding, nullptr));
         return {out, input.dtype(), Shape({B, O, Ho, Wo}), input.device()};
@@ -286,8 +311,8 @@ public:
         const auto dt = static_cast<ttamd_dtype>(input.dtype());
         const std::size_t esz = dtype_size(input.dtype());
         const Tensor go = grad_output.contiguous(), w = weight.contiguous();
-        auto gx = std::make_shared<StorageAMD>(static_cast<std::size_t>(input.numel()) * esz, dev);
-        auto gw = std::make_shared<StorageAMD>(static_cast<std::size_t>(weight.numel()) * esz, dev);
+        auto gx = std::make_shared<StorageAMD>(checked_numel({B, C, H, W}) * esz, dev);
+        auto gw = std::make_shared<StorageAMD>(checked_numel({O, C, k, k}) * esz, dev);
         std::shared_ptr<StorageAMD> gb = bias ? std::make_shared<StorageAMD>(static_cast<std::size_t>(O) * esz, dev) : nullptr;
         std::size_t ws_bytes = 0;
         check(ttamd_conv2d_backward_workspace(dt, B, C, H, W, O, k, stride, padding, &ws_bytes));
@@ -354,19 +379,21 @@ public:
                           nullptr));
         return {out, lhs.dtype(), lhs.shape(), lhs.device()};
     }
-    // sum(tensor) -> one element; sum(tensor, dim) -> that dimension removed (backend_base.h:148-149)
+    // sum(tensor) -> one element; sum(tensor, dim) -> that dimension removed (backend_base.h:148-149).  bool and the
+    // integer dtypes are summed in 64 bits and the result is i64 (common/reduce.h:56-61).
     [[nodiscard]] auto sum(const Tensor &t, int dim = -1) const -> Tensor {
+        const ScalarType rt = (t.dtype() == kF32 || t.dtype() == kF64) ? t.dtype() : kI64;
         std::vector<int> osh;
         if (dim < 0) osh = {1};
         else
             for (int d = 0; d < t.dim(); ++d)
                 if (d != dim) osh.push_back(t.size(d));
         const Shape out_shape{osh};
-        auto out = std::make_shared<StorageAMD>(static_cast<std::size_t>(out_shape.numel()) * dtype_size(t.dtype()), t.device().id);
+        auto out = std::make_shared<StorageAMD>(static_cast<std::size_t>(out_shape.numel()) * dtype_size(rt), t.device().id);
         const auto sh = i64(t.shape()), st = i64(t.stride());
         check(ttamd_sum(t.device().id, static_cast<ttamd_dtype>(t.dtype()), t.dim(), sh.data(), t.storage()->ptr_, t.offset(), st.data(), dim,
                         out->ptr_, nullptr));
-        return {out, t.dtype(), out_shape, t.device()};
+        return {out, rt, out_shape, t.device()};
     }
     template <typename T>
     [[nodiscard]] auto full(T value, int numel, Device device) const -> Tensor {  // backend_base.h:51
@@ -395,7 +422,8 @@ public:
         const int Ho = (H + 2 * padding - kernel_size) / stride + 1, Wo = (W + 2 * padding - kernel_size) / stride + 1;
         const bool is_float = input.dtype() == kF32 || input.dtype() == kF64;
         const ScalarType rt = (op == TTAMD_POOL_AVG && !is_float) ? kF32 : input.dtype();  // common/reduce.h:63-69
-        auto out = std::make_shared<StorageAMD>(static_cast<std::size_t>(std::max(B * C * Ho * Wo, 0)) * dtype_size(rt), input.device().id);
+        if (Ho <= 0 || Wo <= 0) throw TTException("pool2d: the window does not fit the padded input");
+        auto out = std::make_shared<StorageAMD>(checked_numel({B, C, Ho, Wo}) * dtype_size(rt), input.device().id);
         const ttamd_view4 iv = view4(input);
         check(ttamd_pool2d_forward(input.device().id, static_cast<ttamd_dtype>(input.dtype()), op, &iv, out->ptr_, B, C, H, W, kernel_size,
                                    stride, padding, nullptr));
@@ -428,6 +456,13 @@ public:
         auto out = std::make_shared<StorageAMD>(static_cast<std::size_t>(shape.numel()) * dtype_size(dtype), device.id);
         check(ttamd_random_fill(device.id, static_cast<ttamd_dtype>(dtype), dist, p0, p1, &generator_state, shape.numel(), out->ptr_, nullptr));
         return {out, dtype, shape, device};
+    }
+    // BackendBase::uniform_real_ / normal_ (backend_base.h:96-103), scalar parameters: written in place through the
+    // view `t`; element i of the view takes the i-th draw (cpu/kernel/distribution.hpp:28-32).
+    void random_fill_(const Tensor &t, int dist, double p0, double p1, uint64_t &generator_state) const {
+        const auto sh = i64(t.shape()), st = i64(t.stride());
+        check(ttamd_random_fill_view(t.device().id, static_cast<ttamd_dtype>(t.dtype()), dist, p0, p1, &generator_state, t.dim(), sh.data(),
+                                     st.data(), t.storage()->ptr_, t.offset(), nullptr));
     }
     [[nodiscard]] auto current_memory_allocated(int device_id) const -> uint64_t {
         uint64_t cur = 0, tot = 0;
@@ -641,7 +676,73 @@ inline auto normal(double mu, double std, const Shape &shape, Generator &gen, Sc
     return get_backend(device)->random_fill(1, mu, std, shape, gen.state, dtype, device);
 }
 
+template <typename Gen>
+auto Tensor::uniform_real_(double low, double high, Gen &gen) -> Tensor & {
+    if (dtype_ != kF32 && dtype_ != kF64) throw TTException("uniform_real_ expects a floating point tensor");
+    if (!(low < high)) throw TTException("Expected low < high. At least one element violates this.");
+    get_backend(device_)->random_fill_(*this, 0, low, high, gen.state);
+    return *this;
+}
+template <typename Gen>
+auto Tensor::normal_(double mu, double std, Gen &gen) -> Tensor & {
+    if (dtype_ != kF32 && dtype_ != kF64) throw TTException("normal_ expects a floating point tensor");
+    get_backend(device_)->random_fill_(*this, 1, mu, std, gen.state);
+    return *this;
+}
+
 namespace nn {
+// nn::calc_fan_in_out (nn/init.cpp:30-52): both fans are size(0) times the receptive field (the sizes beyond dim 1).
+inline auto calc_fan_in_out(const Tensor &tensor) -> std::tuple<double, double> {
+    if (tensor.dim() < 2) throw TTException("Unable to calculate fan in and fan out for tensors with dimensions fewer than 2");
+    int field = 1;
+    for (int i = 2; i < tensor.dim(); ++i) field *= tensor.size(i);
+    const double fan = static_cast<double>(tensor.size(0) * field);
+    return {fan, fan};
+}
+// nn::kaiming_uniform_ (nn/init.cpp:106-112), fan_in mode: U(+-sqrt(3) * gain / sqrt(fan)), drawn in place.
+inline void kaiming_uniform_(Tensor tensor, Generator &gen, double gain = 1.0) {
+    const auto [fan_in, fan_out] = calc_fan_in_out(tensor);
+    (void)fan_out;
+    const double bound = std::sqrt(3.0) * (gain / std::sqrt(fan_in));
+    tensor.uniform_real_(-bound, bound, gen);
+}
+
+// nn::Conv2d (nn/conv2d.cpp:20-81, include/tt/nn/conv2d.h:35-44): weight [out, in, k, k] initialised through the view
+// weight.permute({1,0,2,3}) (conv2d.cpp:56) -- the draws run in that view's row-major order and its fan is in*k*k --
+// then bias ~ U(+-1/sqrt(out*k*k)) (calc_fan_in_out of the weight itself, conv2d.cpp:60-62); forward = conv2d.
+class Conv2d {
+public:
+    Conv2d(int in_channels, int out_channels, int kernel_size, int stride, int padding, bool with_bias, Generator &gen,
+           ScalarType dtype = kF32, Device device = kAMD)
+        : stride_(stride), padding_(padding) {
+        if (in_channels <= 0) throw TTException("Expected in_channels > 0, given in_channels=" + std::to_string(in_channels));
+        if (out_channels <= 0) throw TTException("Expected out_channels > 0, given out_channels=" + std::to_string(out_channels));
+        if (kernel_size <= 0) throw TTException("Expected kernel_size > 0, given kernel_size=" + std::to_string(kernel_size));
+        if (stride <= 0) throw TTException("Expected stride > 0, given stride=" + std::to_string(stride));
+        if (padding < 0) throw TTException("Expected padding >= 0, given padding=" + std::to_string(padding));
+        weight = Tensor::empty(Shape({out_channels, in_channels, kernel_size, kernel_size}), dtype, device);
+        kaiming_uniform_(weight.permute({1, 0, 2, 3}), gen);
+        if (with_bias) {
+            bias = Tensor::empty(Shape({out_channels}), dtype, device);
+            const auto [fan_in, fan_out] = calc_fan_in_out(weight);
+            (void)fan_out;
+            const double bound = 1.0 / std::sqrt(fan_in);
+            bias->uniform_real_(-bound, bound, gen);
+        }
+    }
+    [[nodiscard]] auto forward(const Tensor &input) const -> Tensor {
+        if (input.dim() == 4 && input.size(1) != weight.size(1))
+            throw TTException("Input channels " + std::to_string(input.size(1)) + " does not match layer input channels " +
+                              std::to_string(weight.size(1)));
+        return conv2d(input, weight, bias, stride_, padding_);
+    }
+    Tensor weight;
+    std::optional<Tensor> bias;
+
+private:
+    int stride_, padding_;
+};
+
 // nn::Linear (nn/linear.cpp:20-50): weight is [in_features, out_features]; forward = matmul + bias.  The bias add
 // (and an optional ReLU that follows it) is fused into the GEMM's store phase.
 class Linear {

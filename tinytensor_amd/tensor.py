@@ -12,6 +12,7 @@ from __future__ import annotations
 
 import contextlib
 import ctypes as C
+import math
 from dataclasses import dataclass
 
 import numpy as np
@@ -243,6 +244,23 @@ class Tensor:
     def item(self):
         return self.to_numpy().reshape(-1)[0]
 
+    def uniform_real_(self, low: float, high: float, gen: "Generator") -> "Tensor":
+        """Tensor::uniform_real_(low, high, gen) (tensor/tensor.cpp:1783-1801) -> BackendBase::uniform_real_: in place,
+        through this tensor's view (element i of the view takes the i-th draw, cpu/kernel/distribution.hpp:28-32)."""
+        if self.dtype not in (_capi.F32, _capi.F64):
+            raise TTException("uniform_real_ expects a floating point tensor")
+        if not low < high:
+            raise TTException("Expected low < high. At least one element violates this.")
+        get_backend(self.device).random_fill_(self, 0, low, high, gen)
+        return self
+
+    def normal_(self, mu: float, std: float, gen: "Generator") -> "Tensor":
+        """Tensor::normal_(mu, std, gen) -> BackendBase::normal_, in place through this tensor's view."""
+        if self.dtype not in (_capi.F32, _capi.F64):
+            raise TTException("normal_ expects a floating point tensor")
+        get_backend(self.device).random_fill_(self, 1, mu, std, gen)
+        return self
+
     def view3(self) -> _capi.View3:
         v = _capi.View3()
         v.data = self.storage.ptr
@@ -345,13 +363,15 @@ class BackendAMD:
         return out
 
     def sum(self, t: Tensor, dim: int | None = None) -> Tensor:
-        """BackendBase::sum(tensor) / sum(tensor, dim) (backend_base.h:148-149)."""
+        """BackendBase::sum(tensor) / sum(tensor, dim) (backend_base.h:148-149).  bool and integer tensors are summed
+        in 64 bits into an I64 result (common/reduce.h:56-61)."""
+        rdtype = t.dtype if t.dtype in (_capi.F32, _capi.F64) else _capi.I64
         if dim is None:
-            out = Tensor.empty((1,), t.dtype, t.device)
+            out = Tensor.empty((1,), rdtype, t.device)
             d = -1
         else:
             d = dim % t.dim()
-            out = Tensor.empty(t.shape[:d] + t.shape[d + 1:], t.dtype, t.device)
+            out = Tensor.empty(t.shape[:d] + t.shape[d + 1:], rdtype, t.device)
         _check(lib.ttamd_sum(t.device.id, t.dtype, t.dim(), self._i64(t.shape), C.c_void_p(t.storage.ptr), t.offset,
                              self._i64(t.stride), d, C.c_void_p(out.storage.ptr), _stream_arg()))
         return out
@@ -362,6 +382,12 @@ class BackendAMD:
         host = np.array([value], dtype=_NP_OF[dtype])
         _check(lib.ttamd_full(device.id, dtype, C.c_void_p(host.ctypes.data), numel, C.c_void_p(out.storage.ptr), _stream_arg()))
         return out
+
+    def random_fill_(self, t: Tensor, dist: int, p0: float, p1: float, gen: "Generator") -> None:
+        """BackendBase::uniform_real_ / normal_ (backend_base.h:96-103) with scalar parameters, written through the
+        view `t` in place; `gen` advances by t.numel() outputs."""
+        _check(lib.ttamd_random_fill_view(t.device.id, t.dtype, dist, p0, p1, C.byref(gen.state), t.dim(), self._i64(t.shape),
+                                          self._i64(t.stride), C.c_void_p(t.storage.ptr), t.offset, _stream_arg()))
 
     def to(self, t: Tensor, dtype: int) -> Tensor:
         """BackendBase::to(tensor, dtype) (backend_base.h:74): element-wise static_cast into dense storage."""
@@ -449,9 +475,10 @@ class BackendAMD:
         return out
 
     def conv2d_backward(self, grad_output: Tensor, input: Tensor, weight: Tensor, bias: Tensor | None, stride: int,
-                        padding: int, buffers=None):
+                        padding: int, buffers=None, return_buffers: bool = False):
         """BackendBase::conv2d_backward (backend_base.h:277-284) -> (grad_input, grad_weight, grad_bias|None).
-        `buffers` = (gx, gw, gb, workspace_storage) from an earlier call reuses the results (benchmarks)."""
+        `return_buffers`: return (gx, gw, gb, workspace_storage) instead, a tuple that a later call takes as `buffers`
+        to write into the same results and workspace (benchmarks: no allocation inside a timed loop)."""
         B, Cc, H, W = input.shape
         O, _, k, _ = weight.shape
         go = grad_output.contiguous()
@@ -472,10 +499,9 @@ class BackendAMD:
             C.byref(wv), C.c_void_p(gx.storage.ptr), C.c_void_p(gw.storage.ptr),
             C.c_void_p(gb.storage.ptr) if gb is not None else None, B, Cc, H, W, O, k, stride, padding,
             C.c_void_p(ws.ptr), ws.nbytes, _stream_arg()))
-        if buffers is not None:
-            return gx, gw, gb
+        if return_buffers:
+            return gx, gw, gb, ws
         # (no wait for the kernels: like every other temporary, the workspace goes back to the allocator in stream order)
-        self.last_conv_buffers = (gx, gw, gb, ws)
         return gx, gw, gb
 
 
@@ -498,6 +524,19 @@ class Generator:
         r = ((r ^ (r >> 30)) * 0xBF58476D1CE4E5B9) & m
         r = ((r ^ (r >> 27)) * 0x94D049BB133111EB) & m
         self.state = C.c_uint64(r ^ (r >> 31))
+
+
+_DEFAULT_GENERATOR = Generator(0)
+
+
+def default_generator() -> Generator:
+    """get_default_generator() (tensor/random.cpp:69-90): the generator that draws without an explicit one use."""
+    return _DEFAULT_GENERATOR
+
+
+def set_default_generator_seed(seed: int) -> None:
+    """set_default_generator_seed (tensor/random.cpp:84-86)."""
+    _DEFAULT_GENERATOR.state = Generator(seed).state
 
 
 def _random_fill(shape, dtype, dist, p0, p1, gen: Generator, device: Device) -> Tensor:
@@ -527,6 +566,85 @@ def linear_init(in_features: int, out_features: int, gen: Generator, dtype: int 
     bound_b = 1.0 / fan ** 0.5
     b = uniform_real(-bound_b, bound_b, (out_features,), gen, dtype, device)
     return W, b
+
+
+def calc_fan_in_out(t: Tensor):
+    """nn::calc_fan_in_out (nn/init.cpp:30-52): BOTH fans are size(0) times the receptive field (sizes beyond dim 1)."""
+    if t.dim() < 2:
+        raise TTException(f"Unable to calculate fan in and fan out for tensors with dimensions fewer than 2. Given tensor "
+                          f"with {t.dim()} dimensions")
+    field = 1
+    for d in range(2, t.dim()):
+        field *= t.size(d)
+    return float(t.size(0) * field), float(t.size(0) * field)
+
+
+def kaiming_uniform_(t: Tensor, gen: Generator, gain: float = 1.0) -> None:
+    """nn::kaiming_uniform_ (nn/init.cpp:106-112), fan_in mode: U(+-sqrt(3) * gain / sqrt(fan)) drawn in place."""
+    fan, _ = calc_fan_in_out(t)
+    bound = math.sqrt(3.0) * (gain / math.sqrt(fan))
+    t.uniform_real_(-bound, bound, gen)
+
+
+class Conv2d:
+    """nn::Conv2d (nn/conv2d.cpp:20-81, include/tt/nn/conv2d.h:35-44).  weight [out,in,k,k] is initialised through the
+    view weight.permute(1,0,2,3) (conv2d.cpp:56): the draws run over [in,out,k,k] in row-major order of that view and
+    its fan is in_channels*k*k; the bias bound comes from calc_fan_in_out(weight) = out_channels*k*k (conv2d.cpp:60-62).
+    Both are drawn from `gen` (the reference uses the thread's default generator) in that order."""
+
+    def __init__(self, in_channels: int, out_channels: int, kernel_size: int, stride: int, padding: int, bias: bool = True,
+                 dtype: int = _capi.F32, device: Device = kAMD, gen: Generator | None = None):
+        for name, v, ok in (("in_channels", in_channels, in_channels > 0), ("out_channels", out_channels, out_channels > 0),
+                            ("kernel_size", kernel_size, kernel_size > 0), ("stride", stride, stride > 0)):
+            if not ok:
+                raise TTException(f"Expected {name} > 0, given {name}={v}")
+        if padding < 0:
+            raise TTException(f"Expected padding >= 0, given padding={padding}")
+        gen = gen if gen is not None else default_generator()
+        self.stride, self.padding = stride, padding
+        self.weight = Tensor.empty((out_channels, in_channels, kernel_size, kernel_size), dtype, device)
+        kaiming_uniform_(self.weight.permute(1, 0, 2, 3), gen)
+        self.bias = None
+        if bias:
+            self.bias = Tensor.empty((out_channels,), dtype, device)
+            fan_in, _ = calc_fan_in_out(self.weight)
+            bound = 1.0 / math.sqrt(fan_in)
+            self.bias.uniform_real_(-bound, bound, gen)
+
+    def parameters(self):
+        return [self.weight] + ([self.bias] if self.bias is not None else [])
+
+    def forward(self, input: Tensor) -> Tensor:
+        if input.dim() == 4 and input.size(1) != self.weight.size(1):
+            raise TTException(f"Input channels {input.size(1)} does not match layer input channels {self.weight.size(1)}")
+        return conv2d(input, self.weight, self.bias, self.stride, self.padding)
+
+    __call__ = forward
+
+
+class Linear:
+    """nn::Linear (nn/linear.cpp:20-50): weight [in,out] by kaiming_uniform_, bias ~ U(+-1/sqrt(in)), forward
+    matmul(input, weight) + bias with the bias add fused into the GEMM's epilogue."""
+
+    def __init__(self, in_features: int, out_features: int, bias: bool = True, dtype: int = _capi.F32, device: Device = kAMD,
+                 gen: Generator | None = None):
+        gen = gen if gen is not None else default_generator()
+        self.weight = Tensor.empty((in_features, out_features), dtype, device)
+        kaiming_uniform_(self.weight, gen)
+        self.bias = None
+        if bias:
+            self.bias = Tensor.empty((out_features,), dtype, device)
+            fan_in, _ = calc_fan_in_out(self.weight)
+            bound = 1.0 / math.sqrt(fan_in)
+            self.bias.uniform_real_(-bound, bound, gen)
+
+    def parameters(self):
+        return [self.weight] + ([self.bias] if self.bias is not None else [])
+
+    def forward(self, input: Tensor) -> Tensor:
+        return linear(input, self.weight, self.bias)
+
+    __call__ = forward
 
 
 def full(shape, value, dtype: int = _capi.F32, device: Device = kAMD) -> Tensor:
