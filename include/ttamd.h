@@ -100,11 +100,18 @@ ttamd_status ttamd_free(int device, void *ptr, size_t bytes);
 ttamd_status ttamd_memory_allocated(int device, uint64_t *current_bytes, uint64_t *total_bytes);
 /* The library keeps freed device blocks (by size class) and hands them out again instead of paying
  * hipMalloc + hipFree (25-70 us per pair, and a device-wide wait) for every result tensor; the counters above
- * count what the caller holds, not what is cached.  Reuse follows stream order: safe when one stream carries all
- * work of a device (the reference's model, cuda/kernel_launch.cuh:19-29); callers with several streams synchronise
- * before freeing or run with TTAMD_ALLOC_CACHE=0.  ttamd_empty_cache waits for the device and returns every
- * cached block to the driver; ttamd_memory_cached reports the bytes currently cached.  No counterpart in the
- * reference, whose DeviceMemory<T> calls cudaMalloc / cudaFree directly (cuda/data_types.cuh:28-101). */
+ * count what the caller holds, not what is cached.  A cached block may still be in use by kernels enqueued before
+ * its free, so the cache follows streams: ttamd_malloc_on_stream / ttamd_free_on_stream name the stream the block
+ * is about to be used on / was last used on (ttamd_malloc / ttamd_free mean the default stream, the reference's
+ * model: cuda/kernel_launch.cuh:19-29).  A block goes back out at once to a request for a stream it was allocated
+ * or freed for (stream order), to a request for another stream only after events recorded on its own streams have
+ * completed, and to anyone after ttamd_device_synchronize.  A caller that uses a block on a third stream
+ * synchronises that stream before the free.  TTAMD_ALLOC_CACHE=0 switches the cache off.  ttamd_empty_cache waits
+ * for the device and returns every cached block to the driver; ttamd_memory_cached reports the bytes currently
+ * cached.  No counterpart in the reference, whose DeviceMemory<T> calls cudaMalloc / cudaFree directly
+ * (cuda/data_types.cuh:28-101). */
+ttamd_status ttamd_malloc_on_stream(int device, size_t bytes, void *stream, void **out);
+ttamd_status ttamd_free_on_stream(int device, void *ptr, size_t bytes, void *stream);
 ttamd_status ttamd_empty_cache(int device);
 ttamd_status ttamd_memory_cached(int device, uint64_t *cached_bytes);
 

@@ -86,3 +86,108 @@ def test_captured_graph_replays_match_eager(tt):
         if graph is not None:
             graph.close()
         stream.close()
+
+
+def test_blocks_allocated_between_replays_are_not_overwritten(tt):
+    """Temporaries of the captured function are freed when it returns; their blocks must stay the graph's own, or a
+    tensor allocated afterwards in the same size class would be overwritten by the next replay."""
+    be = tt.get_backend(tt.kAMD)
+    stream = tt.graph.Stream()
+    graph = None
+    try:
+        host = make_inputs(tt, 2)
+        dev = {k: tt.Tensor.from_numpy(v) for k, v in host.items()}
+        graph = tt.graph.Graph(stream, lambda: fragment(tt, be, **dev))
+        graph.launch()
+        stream.synchronize()
+        first = [t.to_numpy() for t in graph.outputs]
+        # fresh tensors in the size classes of the fragment's temporaries and results (d, a, the conv workspace, ...)
+        rng = np.random.default_rng(7)
+        guards = []
+        for shape in ((1, 256, 64), (4, 16, 12, 12), (1, 256, 256), (4, 16, 6, 6), (16, 8, 3, 3), (4, 8, 12, 12), (1, 64, 256)) * 3:
+            h = rng.normal(0, 1, shape).astype(np.float32)
+            guards.append((h, tt.Tensor.from_numpy(h)))
+        for _ in range(2):
+            graph.launch()
+            stream.synchronize()
+        for h, t in guards:
+            assert np.array_equal(t.to_numpy(), h)
+        for g, w in zip(graph.outputs, first):
+            assert np.array_equal(g.to_numpy(), w)
+    finally:
+        if graph is not None:
+            graph.close()
+        stream.close()
+
+
+def test_scratch_growth_after_a_capture_keeps_the_recorded_buffer(tt):
+    """A captured split-k product has its scratch address recorded; a later, larger split-k product on the same stream
+    grows the scratch.  The outgrown buffer must stay valid for the replays."""
+    be = tt.get_backend(tt.kAMD)
+    stream = tt.graph.Stream()
+    graph = None
+    try:
+        rng = np.random.default_rng(3)
+        a = tt.Tensor.from_numpy(rng.integers(-3, 4, (1, 256, 512)).astype(np.float32))
+        b = tt.Tensor.from_numpy(rng.integers(-3, 4, (1, 512, 256)).astype(np.float32))
+        assert "splitk" in be.batched_matmul_variant(a, b)
+        graph = tt.graph.Graph(stream, lambda: [be.batched_matmul(a, b)])
+        graph.launch()
+        stream.synchronize()
+        want = graph.outputs[0].to_numpy()
+        assert np.array_equal(want[0], (a.to_numpy()[0].astype(np.float64) @ b.to_numpy()[0]).astype(np.float32))
+        # 3 x 320 x 1024 x 384 splits three ways: 4.2 MiB of partial tiles, more than the stream's first 4 MiB buffer
+        big_a = tt.Tensor.from_numpy(rng.integers(-3, 4, (3, 320, 1024)).astype(np.float32))
+        big_b = tt.Tensor.from_numpy(rng.integers(-3, 4, (3, 1024, 384)).astype(np.float32))
+        assert "splitk3" in be.batched_matmul_variant(big_a, big_b)
+        big = stream.run(lambda: be.batched_matmul(big_a, big_b))
+        stream.synchronize()
+        assert np.array_equal(big.to_numpy(), np.matmul(big_a.to_numpy().astype(np.float64), big_b.to_numpy()).astype(np.float32))
+        for _ in range(2):
+            graph.launch()
+            stream.synchronize()
+            assert np.array_equal(graph.outputs[0].to_numpy(), want)
+    finally:
+        if graph is not None:
+            graph.close()
+        stream.close()
+
+
+def test_block_freed_on_one_stream_is_not_reused_on_another_while_in_flight(tt):
+    """A tensor is released right after work that reads it has been enqueued on a (non-blocking) stream; an allocation
+    of the same size for the default stream, made while that work is still running, must not receive its block."""
+    be = tt.get_backend(tt.kAMD)
+    assert tt._capi.lib.ttamd_empty_cache(0) == 0  # so that the block released below is the only cached one of its size
+    stream = tt.graph.Stream(non_blocking=True)
+    try:
+        n = 2048
+        rng = np.random.default_rng(4)
+        a_h = rng.integers(-2, 3, (1, n, n)).astype(np.float32)
+        b_h = rng.integers(-2, 3, (1, n, n)).astype(np.float32)
+        b = tt.Tensor.from_numpy(b_h)
+        outs = [tt.Tensor.empty((1, n, n), tt._capi.F32) for _ in range(4)]
+        want = (a_h[0].astype(np.float64) @ b_h[0]).astype(np.float32)  # small integers: exact in any order
+        be.synchronize(0)
+
+        def enqueue():
+            a = tt.Tensor.from_numpy(a_h)          # allocated for `stream` (the upload itself is a blocking copy)
+            for _ in range(60):                    # tens of milliseconds of GEMMs that read `a`
+                for o in outs:
+                    be.batched_matmul(a, b, out=o)
+            return a.storage.ptr                   # `a` is released here, with the work still queued
+
+        freed_ptr = stream.run(enqueue)
+        # default stream, same size class, while the GEMMs run: other data
+        other_h = np.full((1, n, n), 7.0, np.float32)
+        other = tt.Tensor.from_numpy(other_h)
+        in_flight_reuse = other.storage.ptr == freed_ptr
+        stream.synchronize()
+        for o in outs:
+            assert np.array_equal(o.to_numpy()[0], want)
+        assert np.array_equal(other.to_numpy(), other_h)
+        assert not in_flight_reuse
+        # once the stream is idle the block serves any stream again
+        again = tt.Tensor.empty((1, n, n), tt._capi.F32)
+        assert again.storage.ptr == freed_ptr
+    finally:
+        stream.close()

@@ -69,7 +69,8 @@ inline FastDiv make_fastdiv(uint32_t d) {
 
 // Device scratch owned by the library, one growing buffer per (device, stream): kernels enqueued on one stream
 // run in order, so consecutive calls on that stream may share it; calls on different streams get different
-// buffers.  Growing allocates (hipMalloc) and frees the old buffer (hipFree, which waits for the device).
+// buffers.  Growing allocates (hipMalloc, at least double the size); the outgrown buffer is kept until the process
+// ends, because kernels in flight and captured graphs may still refer to it.
 ttamd_status stream_scratch(int device, hipStream_t stream, size_t bytes, void **out);
 
 // One GEMM problem as the kernels see it.  Conventional letters inside the kernels:

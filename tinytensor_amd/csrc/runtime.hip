@@ -10,6 +10,7 @@
 #include <mutex>
 #include <unordered_map>
 #include <utility>
+#include <vector>
 
 namespace ttamd {
 
@@ -23,15 +24,36 @@ std::atomic<uint64_t> g_total[kMaxDevices];
 // blocks are therefore kept per device, by rounded size, and handed out again; they go back to the driver on
 // ttamd_empty_cache, when an allocation fails, and never otherwise.
 //
-// A reused block may still be read or written by kernels that were enqueued before it was freed.  That is safe
-// when the next user is enqueued on the same stream (stream order), which is the reference's model: all work of a
-// device goes to one stream (cuda/kernel_launch.cuh:19-29) and host copies are ordered against it.  A caller
-// that spreads work over several streams must synchronise them before freeing, or set TTAMD_ALLOC_CACHE=0.
+// A cached block may still be read or written by kernels that were enqueued before it was freed.  Each block
+// therefore remembers the streams it was used on -- the one it was allocated for and the one it was freed for -- and
+// is handed out again
+//   * to a request for one of those streams at once (stream order makes that safe; the reference's model, where one
+//     stream carries all work of a device, cuda/kernel_launch.cuh:19-29, only ever takes this road),
+//   * to a request for another stream only after an event recorded on each of its streams has completed (the event is
+//     recorded when the block is first considered for such a request, which is later than the free and so covers it),
+//   * to anyone once the whole device has been synchronised after the free (ttamd_device_synchronize,
+//     ttamd_empty_cache).
+// While the requesting stream is being captured into a graph only the first and the last road are open: no events
+// are recorded or queried during a capture.
+struct CachedBlock {
+    void *ptr = nullptr;
+    int n_streams = 0;
+    hipStream_t stream[2] = {nullptr, nullptr};
+    hipEvent_t event[2] = {nullptr, nullptr};  // recorded lazily, see above
+    uint64_t epoch = 0;                        // the device's synchronisation count when the block was freed
+};
+struct LiveBlock {
+    size_t rounded = 0;
+    hipStream_t stream = nullptr;  // the stream the block was allocated for
+};
 struct BlockCache {
     std::mutex mu;
-    std::multimap<size_t, void *> free_blocks;     // rounded size -> block
-    std::unordered_map<void *, size_t> live;        // block -> rounded size
+    std::multimap<size_t, CachedBlock> free_blocks;  // rounded size -> block
+    std::unordered_map<void *, LiveBlock> live;       // block -> rounded size, allocation stream
     uint64_t cached_bytes = 0;
+    std::atomic<uint64_t> epoch{0};                   // bumped when a whole-device synchronisation starts
+    std::atomic<uint64_t> synced{0};                  // blocks freed at an epoch below this are idle: a synchronisation
+                                                      // that started after their free has completed
 };
 BlockCache g_cache[kMaxDevices];
 
@@ -52,11 +74,60 @@ size_t round_block(size_t bytes) {
     return (bytes + step - 1) / step * step;
 }
 
+void drop_events(CachedBlock &b) {
+    for (int i = 0; i < 2; ++i)
+        if (b.event[i]) {
+            (void)hipEventDestroy(b.event[i]);
+            b.event[i] = nullptr;
+        }
+}
+
 void release_cached(int device) {
     BlockCache &c = g_cache[device];
-    for (auto &kv : c.free_blocks) (void)hipFree(kv.second);
+    for (auto &kv : c.free_blocks) {
+        drop_events(kv.second);
+        (void)hipFree(kv.second.ptr);
+    }
     c.free_blocks.clear();
     c.cached_bytes = 0;
+}
+
+bool is_capturing(hipStream_t stream) {
+    hipStreamCaptureStatus status = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(stream, &status) != hipSuccess) {
+        (void)hipGetLastError();
+        return true;  // an unusable stream handle: take the conservative road
+    }
+    return status != hipStreamCaptureStatusNone;
+}
+
+// May the cached block be handed to a request for `stream` now?  `may_use_events`: the requesting stream is not under
+// capture, so events on the block's other streams may be recorded and queried.
+bool reusable(CachedBlock &b, hipStream_t stream, uint64_t synced_epoch, bool may_use_events) {
+    if (b.epoch < synced_epoch) return true;  // the device has been synchronised since the free
+    for (int i = 0; i < b.n_streams; ++i) {
+        if (b.stream[i] == stream) continue;  // stream order
+        if (!may_use_events) return false;
+        if (!b.event[i]) {
+            if (is_capturing(b.stream[i])) return false;  // an event recorded there would become a graph node
+            hipEvent_t ev = nullptr;
+            if (hipEventCreateWithFlags(&ev, hipEventDisableTiming) != hipSuccess) {
+                (void)hipGetLastError();
+                return false;
+            }
+            if (hipEventRecord(ev, b.stream[i]) != hipSuccess) {  // e.g. the stream has been destroyed since
+                (void)hipGetLastError();
+                (void)hipEventDestroy(ev);
+                return false;  // only a whole-device synchronisation releases this block
+            }
+            b.event[i] = ev;
+        }
+        if (hipEventQuery(b.event[i]) != hipSuccess) {
+            (void)hipGetLastError();  // hipErrorNotReady: work enqueued before the free may still be running
+            return false;
+        }
+    }
+    return true;
 }
 }  // namespace
 
@@ -88,10 +159,12 @@ ttamd_status stream_scratch(int device, hipStream_t stream, size_t bytes, void *
     };
     static std::mutex mu;
     static std::map<std::pair<int, hipStream_t>, Buf> bufs;  // lives until the process ends
+    static std::vector<void *> retired;                       // outgrown buffers, see below
     std::lock_guard<std::mutex> lock(mu);
     Buf &b = bufs[{device, stream}];
     if (b.bytes < bytes) {
         size_t want = bytes < (size_t(4) << 20) ? (size_t(4) << 20) : bytes;
+        if (want < 2 * b.bytes) want = 2 * b.bytes;
         want = (want + 255) & ~size_t(255);
         void *p = nullptr;
         hipError_t e = hipMalloc(&p, want);
@@ -100,7 +173,10 @@ ttamd_status stream_scratch(int device, hipStream_t stream, size_t bytes, void *
             set_error("Unable to allocate %zu bytes of scratch on AMD device %d: %s", want, device, hipGetErrorString(e));
             return TTAMD_ERR_OUT_OF_MEMORY;
         }
-        if (b.ptr) TTAMD_HIP_CHECK(hipFree(b.ptr));  // waits for kernels that may still read the old buffer
+        // The old buffer is kept until the process ends: kernels in flight may still use it, and a captured graph has
+        // its address baked in and may be replayed at any time.  Growth at least doubles the size, so all retired
+        // buffers of a stream together stay below its current one.
+        if (b.ptr) retired.push_back(b.ptr);
         b.ptr = p;
         b.bytes = want;
     }
@@ -141,7 +217,7 @@ const char *ttamd_last_error_string(void) { return g_error; }
 
 const char *ttamd_target_arch(void) { return "gfx950"; }
 
-ttamd_status ttamd_malloc(int device, size_t bytes, void **out) {
+ttamd_status ttamd_malloc_on_stream(int device, size_t bytes, void *stream, void **out) {
     if (!out) {
         set_error("ttamd_malloc: out is NULL");
         return TTAMD_ERR_INVALID_ARGUMENT;
@@ -149,25 +225,36 @@ ttamd_status ttamd_malloc(int device, size_t bytes, void **out) {
     *out = nullptr;
     if (ttamd_status s = use_device(device)) return s;
     if (bytes == 0) return TTAMD_OK;
+    hipStream_t st = static_cast<hipStream_t>(stream);
     void *p = nullptr;
     const bool cached = cache_enabled();
     const size_t want = cached ? round_block(bytes) : bytes;
     BlockCache &c = g_cache[device];
     if (cached) {
         std::lock_guard<std::mutex> lock(c.mu);
-        auto it = c.free_blocks.find(want);
-        if (it != c.free_blocks.end()) {
-            p = it->second;
-            c.free_blocks.erase(it);
-            c.cached_bytes -= want;
-            c.live[p] = want;
+        const auto range = c.free_blocks.equal_range(want);
+        if (range.first != range.second) {
+            const uint64_t epoch = c.synced.load();
+            auto hit = range.second;
+            for (auto it = range.first; it != range.second && hit == range.second; ++it)  // stream order or synchronised: no HIP calls
+                if (reusable(it->second, st, epoch, false)) hit = it;
+            if (hit == range.second && !is_capturing(st))
+                for (auto it = range.first; it != range.second && hit == range.second; ++it)
+                    if (reusable(it->second, st, epoch, true)) hit = it;
+            if (hit != range.second) {
+                p = hit->second.ptr;
+                drop_events(hit->second);
+                c.free_blocks.erase(hit);
+                c.cached_bytes -= want;
+                c.live[p] = LiveBlock{want, st};
+            }
         }
     }
     if (!p) {
         hipError_t e = hipMalloc(&p, want);
         if (e != hipSuccess && cached) {  // give the cached blocks back to the driver and try once more
             (void)hipGetLastError();
-            {
+            if (hipDeviceSynchronize() == hipSuccess) {  // cached blocks may still be in use by enqueued kernels
                 std::lock_guard<std::mutex> lock(c.mu);
                 release_cached(device);
             }
@@ -180,7 +267,7 @@ ttamd_status ttamd_malloc(int device, size_t bytes, void **out) {
         }
         if (cached) {
             std::lock_guard<std::mutex> lock(c.mu);
-            c.live[p] = want;
+            c.live[p] = LiveBlock{want, st};
         }
     }
     g_current[device] += bytes;
@@ -189,7 +276,7 @@ ttamd_status ttamd_malloc(int device, size_t bytes, void **out) {
     return TTAMD_OK;
 }
 
-ttamd_status ttamd_free(int device, void *ptr, size_t bytes) {
+ttamd_status ttamd_free_on_stream(int device, void *ptr, size_t bytes, void *stream) {
     if (!ptr) return TTAMD_OK;
     if (ttamd_status s = use_device(device)) return s;
     BlockCache &c = g_cache[device];
@@ -198,8 +285,13 @@ ttamd_status ttamd_free(int device, void *ptr, size_t bytes) {
         std::lock_guard<std::mutex> lock(c.mu);
         auto it = c.live.find(ptr);
         if (it != c.live.end()) {  // a block of the caching allocator: keep it for the next request of its class
-            c.free_blocks.emplace(it->second, ptr);
-            c.cached_bytes += it->second;
+            CachedBlock b;
+            b.ptr = ptr;
+            b.stream[b.n_streams++] = it->second.stream;
+            if (static_cast<hipStream_t>(stream) != it->second.stream) b.stream[b.n_streams++] = static_cast<hipStream_t>(stream);
+            b.epoch = c.epoch.load();
+            c.cached_bytes += it->second.rounded;
+            c.free_blocks.emplace(it->second.rounded, b);
             c.live.erase(it);
             kept = true;
         }
@@ -209,9 +301,13 @@ ttamd_status ttamd_free(int device, void *ptr, size_t bytes) {
     return TTAMD_OK;
 }
 
+ttamd_status ttamd_malloc(int device, size_t bytes, void **out) { return ttamd_malloc_on_stream(device, bytes, nullptr, out); }
+
+ttamd_status ttamd_free(int device, void *ptr, size_t bytes) { return ttamd_free_on_stream(device, ptr, bytes, nullptr); }
+
 ttamd_status ttamd_empty_cache(int device) {
     if (ttamd_status s = use_device(device)) return s;
-    TTAMD_HIP_CHECK(hipDeviceSynchronize());  // cached blocks may still be in use by enqueued kernels
+    if (ttamd_status s = ttamd_device_synchronize(device)) return s;  // cached blocks may still be in use by enqueued kernels
     BlockCache &c = g_cache[device];
     std::lock_guard<std::mutex> lock(c.mu);
     release_cached(device);
@@ -281,7 +377,14 @@ ttamd_status ttamd_memset_zero(int device, void *dst_device, size_t bytes, void 
 
 ttamd_status ttamd_device_synchronize(int device) {
     if (ttamd_status s = use_device(device)) return s;
+    // Blocks freed before this point are idle afterwards, whatever stream used them.  The epoch moves on before the
+    // wait, so a block freed while the wait is in progress carries the new epoch and is not released by it.
+    BlockCache &c = g_cache[device];
+    const uint64_t mine = ++c.epoch;
     TTAMD_HIP_CHECK(hipDeviceSynchronize());
+    uint64_t seen = c.synced.load();
+    while (seen < mine && !c.synced.compare_exchange_weak(seen, mine)) {
+    }
     return TTAMD_OK;
 }
 

@@ -5,9 +5,10 @@ No counterpart in the reference (its CUDA backend launches everything on the def
 tinytensor/tensor/backend/cuda/kernel_launch.cuh:19-29).  Every entry point of the C ABI takes the stream it
 launches on and only records kernels (no memset or copy nodes), so a step that has run once on the stream — which
 sets the kernels' attributes, grows the per-stream scratch and leaves its result blocks in the allocator's cache —
-can be captured without allocating.  The tensors a captured function returns, and those it reads, keep their
-addresses inside the graph: refresh inputs in place (Graph.copy_in) and keep the outputs referenced while the graph
-lives.
+can be captured without allocating.  The graph replays with the addresses it was recorded with: the tensors the
+captured function reads are refreshed in place (Graph.copy_in), and every block the function allocated while it was
+being recorded -- results and temporaries alike -- stays pinned to the Graph object until Graph.close(), so that no
+later allocation can receive a block that a replay still writes.
 """
 from __future__ import annotations
 
@@ -16,7 +17,7 @@ import ctypes as C
 import numpy as np
 
 from . import _capi
-from .tensor import Tensor, TTException, get_backend, kAMD
+from .tensor import Tensor, TTException, get_backend, kAMD, pin_allocations
 
 _hip = None
 
@@ -27,7 +28,8 @@ def _runtime():
         lib = C.CDLL("libamdhip64.so")
         vp = C.c_void_p
         for name, args in {
-            "hipStreamCreate": [C.POINTER(vp)], "hipStreamSynchronize": [vp], "hipStreamDestroy": [vp],
+            "hipStreamCreate": [C.POINTER(vp)], "hipStreamCreateWithFlags": [C.POINTER(vp), C.c_uint],
+            "hipStreamSynchronize": [vp], "hipStreamDestroy": [vp],
             "hipStreamBeginCapture": [vp, C.c_int], "hipStreamEndCapture": [vp, C.POINTER(vp)],
             "hipGraphInstantiate": [C.POINTER(vp), vp, C.POINTER(vp), C.c_char_p, C.c_size_t],
             "hipGraphLaunch": [vp, vp], "hipGraphExecDestroy": [vp], "hipGraphDestroy": [vp],
@@ -46,11 +48,15 @@ def _call(name: str, *args) -> None:
 
 
 class Stream:
-    """A HIP stream at the default priority."""
+    """A HIP stream at the default priority.  `non_blocking`: the stream does not synchronise implicitly with the
+    default stream (hipStreamNonBlocking), so work on the two may overlap."""
 
-    def __init__(self):
+    def __init__(self, non_blocking: bool = False):
         self._h = C.c_void_p()
-        _call("hipStreamCreate", C.byref(self._h))
+        if non_blocking:
+            _call("hipStreamCreateWithFlags", C.byref(self._h), 1)  # hipStreamNonBlocking
+        else:
+            _call("hipStreamCreate", C.byref(self._h))
 
     @property
     def handle(self) -> int:
@@ -65,7 +71,10 @@ class Stream:
             return fn()
 
     def close(self) -> None:
+        """Waits for the stream's work, then destroys it (blocks freed for this stream stay in the allocator's cache
+        under its handle; they are idle once the stream is)."""
         if self._h.value:
+            _call("hipStreamSynchronize", self._h)
             _call("hipStreamDestroy", self._h)
             self._h = C.c_void_p()
 
@@ -76,14 +85,24 @@ class Graph:
     def __init__(self, stream: Stream, fn, warmup: int = 2):
         self.stream = stream
         self._graph, self._exec = C.c_void_p(), C.c_void_p()
+        # The warm-up runs keep their allocations until they end, as the recorded run will: afterwards the allocator's
+        # cache holds one block for every tensor the function creates, temporaries included, and the capture below
+        # finds them all there.
         for _ in range(warmup):
-            stream.run(fn)
+            keep: list = []
+            with pin_allocations(keep):
+                stream.run(fn)
+            stream.synchronize()
+            with get_backend(kAMD).on_stream(stream.handle):
+                del keep[:]  # returned for this stream
         stream.synchronize()
         # Global capture mode: an allocation or a blocking call anywhere in the process would invalidate the capture,
         # which is the guarantee wanted here.
+        self._pinned: list = []  # every storage allocated during the capture, held until close()
         _call("hipStreamBeginCapture", stream._h, 0)
         try:
-            self.outputs = stream.run(fn)
+            with pin_allocations(self._pinned):
+                self.outputs = stream.run(fn)
         finally:
             rc = _runtime().hipStreamEndCapture(stream._h, C.byref(self._graph))
         if rc != 0 or not self._graph.value:
@@ -115,3 +134,4 @@ class Graph:
         if self._graph.value:
             _call("hipGraphDestroy", self._graph)
             self._graph = C.c_void_p()
+        self._pinned = []  # the blocks go back to the allocator (for the stream current now)

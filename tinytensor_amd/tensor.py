@@ -53,19 +53,26 @@ def _check(status: int) -> None:
     raise TTException(msg)
 
 
+_PINNED = None  # while a HIP graph is being captured: the list that keeps every storage allocated meanwhile alive
+
+
 class _Storage:
-    """Owning device allocation (peer of DeviceMemory<T>, cuda/data_types.cuh:28-101)."""
+    """Owning device allocation (peer of DeviceMemory<T>, cuda/data_types.cuh:28-101).  The block is requested for the
+    stream that launches go to at that moment and returned for the one current at its release, so that the library's
+    block cache never hands it to another stream while kernels of those two may still use it."""
 
     def __init__(self, nbytes: int, device: Device):
         self.nbytes = int(nbytes)
         self.device = device
         p = C.c_void_p()
-        _check(lib.ttamd_malloc(device.id, self.nbytes, C.byref(p)))
+        _check(lib.ttamd_malloc_on_stream(device.id, self.nbytes, _stream_arg(), C.byref(p)))
         self.ptr = p.value or 0
+        if _PINNED is not None:
+            _PINNED.append(self)
 
     def __del__(self):
         if getattr(self, "ptr", 0):
-            lib.ttamd_free(self.device.id, C.c_void_p(self.ptr), self.nbytes)
+            lib.ttamd_free_on_stream(self.device.id, C.c_void_p(self.ptr), self.nbytes, _stream_arg())
             self.ptr = 0
 
 
@@ -284,6 +291,19 @@ _STREAM = None  # hipStream_t (an integer handle) that every launch of this modu
 
 def _stream_arg():
     return C.c_void_p(_STREAM) if _STREAM else None
+
+
+@contextlib.contextmanager
+def pin_allocations(keep: list):
+    """Every storage allocated inside the block is appended to `keep`, which the caller holds for as long as the
+    addresses must stay the allocation's own (a captured HIP graph replays with the addresses it was recorded with:
+    a temporary that went back to the block cache could be handed to an unrelated tensor and overwritten by a replay)."""
+    global _PINNED
+    prev, _PINNED = _PINNED, keep
+    try:
+        yield keep
+    finally:
+        _PINNED = prev
 
 
 class BackendAMD:
