@@ -368,6 +368,10 @@ def main():
     ap.add_argument("--detail", metavar="FILE", help="also time every benchmark configuration and write a JSON report")
     ap.add_argument("--conv-loop", type=int, metavar="N", default=0,
                     help="only run N conv2d forward + backward passes of benchmark configuration 4 (input [64,32,28,28], weight [64,32,3,3], s1 p1) (a short target for profilers) and exit")
+    ap.add_argument("--mlp-loop", type=int, metavar="N", default=0,
+                    help="only run N training steps of benchmark configuration 5 (batch 1024, 784-1024-1024-10, mse_loss) from the fused "
+                         "forms (a short target for profilers), print the wall-clock time per step and exit")
+    ap.add_argument("--mlp-ops", action="store_true", help="with --mlp-loop: the step op by op (unfused) instead")
     ap.add_argument("--conv-shape", metavar="B,C,O,H,W", default="64,32,64,28,28",
                     help="geometry for --conv-loop (3x3 kernel, stride 1, padding 1); the default is benchmark configuration 4")
     args = ap.parse_args()
@@ -399,6 +403,53 @@ def main():
             be.conv2d_backward(go, x, w, None, 1, 1, buffers=bufs)
         be.synchronize(0)
         print(json.dumps({"conv_loop": args.conv_loop, "config": f"input [{cb},{cc},{ch},{cw}], weight [{co},{cc},3,3], s1 p1, f32"}))
+        return
+
+    if args.mlp_loop:
+        from oracle import tt_oracle as oracle  # seeded inputs and default init (host restatement of the reference's RNG)
+
+        be = tt.get_backend(tt.kAMD)
+        gp = oracle.Generator(0)
+        xs = tt.Tensor.from_numpy(oracle.Generator(0).uniform_real(0.0, 1.0, (1024, 784)))
+        ts = tt.Tensor.from_numpy(oracle.Generator(1).uniform_real(0.0, 1.0, (1024, 10)))
+        (P1, c1), (P2, c2), (P3, c3) = [tuple(tt.Tensor.from_numpy(v) for v in oracle.linear_init(gp, a, b))
+                                        for a, b in ((784, 1024), (1024, 1024), (1024, 10))]
+
+        def fused_step():
+            z1, a1 = tt.linear_relu(xs, P1, c1); z2, a2 = tt.linear_relu(a1, P2, c2); y = tt.linear(a2, P3, c3)
+            loss, gy, db3 = tt.mse_loss(y, ts, grad=True, bias_grad=True)
+            dz2, dW3, db2 = tt.linear_backward(gy, a2, P3, relu_input=z2)
+            dz1, dW2, db1 = tt.linear_backward(dz2, a1, P2, relu_input=z1)
+            dX, dW1, _ = tt.linear_backward(dz1, xs, P1, bias_grad=False)
+            return [loss, dW1, db1, dW2, db2, dW3, db3, dX]
+
+        def ops_step():
+            z1 = tt.linear(xs, P1, c1); a1 = z1.relu(); z2 = tt.linear(a1, P2, c2); a2 = z2.relu(); y = tt.linear(a2, P3, c3)
+            diff = y - ts
+            loss = diff.pow(2.0).mean()
+            gy = tt.full(y.shape, 2.0 / y.numel(), y.dtype) * diff
+            da2, dW3 = tt.matmul_backward(a2.unsqueeze(0), P3.unsqueeze(0), gy.unsqueeze(0))
+            dz2 = da2.squeeze(0) * tt.where(z2 < 0.0, 0.0, 1.0)
+            da1, dW2 = tt.matmul_backward(a1.unsqueeze(0), P2.unsqueeze(0), dz2.unsqueeze(0))
+            dz1 = da1.squeeze(0) * tt.where(z1 < 0.0, 0.0, 1.0)
+            dX, dW1 = tt.matmul_backward(xs.unsqueeze(0), P1.unsqueeze(0), dz1.unsqueeze(0))
+            return [loss, gy.sum(0), dz2.sum(0), dz1.sum(0), dW3, dW2, dW1, dX]
+
+        step = ops_step if args.mlp_ops else fused_step
+        stream = tt.graph.Stream()
+        graph = tt.graph.Graph(stream, step)  # replayed from a HIP graph: the kernels' own time, no per-op host work
+        for _ in range(20):
+            graph.launch()
+        stream.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.mlp_loop):
+            graph.launch()
+        stream.synchronize()
+        ms = (time.perf_counter() - t0) / args.mlp_loop * 1e3
+        print(json.dumps({"mlp_loop": args.mlp_loop, "form": "op by op" if args.mlp_ops else "fused", "graph_nodes": graph.num_nodes(),
+                          "ms_per_step": round(ms, 4), "config": "batch 1024, 784-1024-1024-10, f32, forward + backward"}))
+        graph.close()
+        stream.close()
         return
 
     if args.detail:

@@ -71,12 +71,29 @@ typedef struct ttamd_view4 {
 /* Epilogue fused into the GEMM's store phase.  All fields 0/NULL = plain C = A.B, which is
  * what BackendBase::batched_matmul computes.  The other modes serve the callers either side
  * of the GEMM: nn::Linear's `+ bias->expand()` (tinytensor/nn/linear.cpp:45-48), the ReLU
- * that follows it in an MLP, and conv2d's per-channel bias (cpu/conv.cpp:115-124). */
+ * that follows it in an MLP, conv2d's per-channel bias (cpu/conv.cpp:115-124), and the
+ * element-wise steps that autograd places around the backward GEMMs of a Linear layer.
+ * Order of application to each element v of A.B:
+ *   v += bias;  v = 0 where relu_grad_input < 0;  v = max(v, 0) if relu;  v += out if accumulate;
+ *   out = v;  relu_out = max(v, 0);  colsum_out[column] += v. */
 typedef struct ttamd_epilogue {
     const void *bias; /* device pointer, same dtype as the GEMM, or NULL                      */
     int32_t bias_mode;/* 0 none, 1 = bias[column] (Linear), 2 = bias[row] (conv channel)      */
     int32_t relu;     /* 1: out = max(out, 0) after the bias                                  */
     int32_t accumulate;/* 1: out += result instead of out = result (grad accumulation)        */
+    int32_t reserved; /* 0                                                                    */
+    /* Linear followed by ReLU in one launch: `out` keeps the Linear result, which autograd saves as the ReLU's
+     * input (autograd/unary_ops.cpp:562-567), and relu_out (dense [B,N,M] like out, or NULL) receives max(out, 0).
+     * Not together with `relu`. */
+    void *relu_out;
+    /* TensorRelu::backward (autograd/unary_ops.cpp:568-573: grad_output * where(input < 0, 0, 1)) applied by the
+     * GEMM that computes grad_output: dense [B,N,M] like out, the ReLU's saved input, or NULL. */
+    const void *relu_grad_input;
+    /* Sum of `out` over its rows, [B,M] (or NULL): the gradient of a Linear layer's bias, which nn/linear.cpp:45-48
+     * adds as an expanded view, so its gradient sums the batch dimension.  Per-tile partial sums are added in a fixed
+     * order by a second small kernel (deterministic; not the reference's row-by-row order).  f32/f64 on the
+     * matrix-core kernels only; not together with `accumulate`. */
+    void *colsum_out;
 } ttamd_epilogue;
 
 /* ---- library / device ------------------------------------------------------------------ */
@@ -231,6 +248,17 @@ ttamd_status ttamd_sum(int device, ttamd_dtype dtype, int ndim, const int64_t *s
                        const int64_t *stride, int dim, void *out, void *stream);
 /* BackendBase::full (backend_base.h:51): `value` points at one host scalar of `dtype`. */
 ttamd_status ttamd_full(int device, ttamd_dtype dtype, const void *value, int64_t numel, void *out, void *stream);
+
+/* nn::mse_loss(input, target, ReductionMode::mean) (nn/loss.cpp:69-72) and its backward in one pass over dense
+ * [rows, cols] operands (f32 / f64).  What the reference computes op by op -- pow(input - target, 2), mean as
+ * (x / numel).sum() (autograd/reduce_ops.cpp:195-205), and backward grad_input = (1 / numel) * 2 * (input - target)
+ * (autograd/binary_ops.cpp:153-159) -- as one streaming kernel plus a one-workgroup finish: loss_out [1];
+ * grad_input_out [rows, cols] or NULL; grad_colsum_out [cols] or NULL = grad_input summed over the rows (the bias
+ * gradient of the Linear layer that produced `input`; cols <= 64 only, wider matrices sum with ttamd_sum).
+ * Sums run in a fixed order (deterministic), not in the reference's element order. */
+ttamd_status ttamd_mse_loss(int device, ttamd_dtype dtype, int64_t rows, int64_t cols, const void *input,
+                            const void *target, void *loss_out, void *grad_input_out, void *grad_colsum_out,
+                            void *stream);
 
 /* BackendBase::uniform_real_ / normal_ (backend_base.h:96-103) for a dense float tensor with scalar parameters, as
  * nn::Linear's default initialisation calls them (nn/init.cpp:30-52,106-112).  dist 0 = uniform_real(low = p0,

@@ -348,6 +348,27 @@ MlpGrads mlp_step(const Tensor &x, const Tensor &t, const nn::Linear &l1, const 
     g.dX = dX.squeeze(0);
     return g;
 }
+// The same step from the fused forms: Linear + ReLU in one launch, the loss with its gradient and the head's bias
+// gradient in one, and per layer one GEMM for dx (ReLU mask and bias gradient in its store) and one for dW.
+MlpGrads mlp_step_fused(const Tensor &x, const Tensor &t, const nn::Linear &l1, const nn::Linear &l2, const nn::Linear &l3) {
+    const auto [z1, a1] = l1.forward_relu(x);
+    const auto [z2, a2] = l2.forward_relu(a1);
+    const Tensor y = l3.forward(a2);
+    const nn::MseLoss loss = nn::mse_loss(y, t, true);
+    const nn::LinearGrads g3 = nn::linear_backward(loss.grad_input, a2, l3.weight, &z2, true);
+    const nn::LinearGrads g2 = nn::linear_backward(g3.dx, a1, l2.weight, &z1, true);
+    const nn::LinearGrads g1 = nn::linear_backward(g2.dx, x, l1.weight);
+    MlpGrads g;
+    g.loss = loss.loss;
+    g.db3 = *loss.grad_colsum;
+    g.dW3 = g3.dW;
+    g.db2 = *g3.db_prev;
+    g.dW2 = g2.dW;
+    g.db1 = *g2.db_prev;
+    g.dW1 = g1.dW;
+    g.dX = g1.dx;
+    return g;
+}
 }  // namespace
 
 TEST_CASE("MLP training step") {
@@ -384,8 +405,35 @@ TEST_CASE("MLP training step") {
     for (int i = 0; i < iters; ++i) (void)mlp_step(X, T, b1, b2, b3);
     check(ttamd_device_synchronize(0));
     const double ms = std::chrono::duration<double, std::milli>(std::chrono::steady_clock::now() - t0).count() / iters;
-    std::printf("  MLP training step 1024 x (784-1024-1024-10), C++ host layer: %.3f ms per step\n", ms);
+    std::printf("  MLP training step 1024 x (784-1024-1024-10), C++ host layer, op by op: %.3f ms per step\n", ms);
     CHECK(ms < 50.0);
+    // the same step from the fused forms (at most 15 launches); every result against the op-by-op step
+    const MlpGrads ref = mlp_step(X, T, b1, b2, b3), fused = mlp_step_fused(X, T, b1, b2, b3);
+    auto close = [](const Tensor &a, const Tensor &b) {
+        const auto va = a.to_vec<float>(), vb = b.to_vec<float>();
+        float big = 0.0f, err = 0.0f;
+        for (std::size_t i = 0; i < va.size(); ++i) {
+            big = std::max(big, std::abs(vb[i]));
+            err = std::max(err, std::abs(va[i] - vb[i]));
+        }
+        return va.size() == vb.size() && err <= 1e-5f * big;
+    };
+    CHECK(close(fused.loss, ref.loss));
+    CHECK(close(fused.dW1, ref.dW1));
+    CHECK(close(fused.db1, ref.db1));
+    CHECK(close(fused.dW2, ref.dW2));
+    CHECK(close(fused.db2, ref.db2));
+    CHECK(close(fused.dW3, ref.dW3));
+    CHECK(close(fused.db3, ref.db3));
+    CHECK(close(fused.dX, ref.dX));
+    for (int i = 0; i < 5; ++i) (void)mlp_step_fused(X, T, b1, b2, b3);
+    check(ttamd_device_synchronize(0));
+    const auto t1 = std::chrono::steady_clock::now();
+    for (int i = 0; i < iters; ++i) (void)mlp_step_fused(X, T, b1, b2, b3);
+    check(ttamd_device_synchronize(0));
+    const double ms_fused = std::chrono::duration<double, std::milli>(std::chrono::steady_clock::now() - t1).count() / iters;
+    std::printf("  the same step from the fused forms (14 launches): %.3f ms per step\n", ms_fused);
+    CHECK(ms_fused < 50.0);
 }
 
 int main(int argc, char **argv) { return mini::run_all(argc, argv); }

@@ -1,0 +1,149 @@
+"""The fused forms around a Linear layer's GEMMs: second output max(out, 0) (Linear + ReLU), the ReLU-backward mask and
+the bias gradient's column sums in the store of the GEMM that computes grad_output, mse_loss with its backward in one
+pass, and the whole MLP training step of benchmark configuration 5 built from them.  Each piece is compared with numpy on
+integer-valued data (exact in any summation order) for every kernel family that can carry it, then the whole step with
+the CPU oracle at the benchmark's size."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+from helpers import max_rel_error, mlp_train_step
+
+pytestmark = pytest.mark.gpu
+
+# (B, N, K, M): small-tile plain, ragged with odd M (no paired stores), two halves of k, split k, 128 x 128, 192 x 192,
+# 256 x 256 / 256 x 128 tiles, K = 10 (the skinny backward product of configuration 5), element-wise gathers
+SHAPES = [(1, 200, 96, 136), (2, 130, 70, 151), (1, 1024, 1024, 1024), (1, 256, 512, 256), (1, 2048, 64, 2048),
+          (1, 3072, 32, 3072), (1, 4096, 32, 4096), (1, 1024, 10, 1024), (3, 70, 50, 90)]
+
+
+def _variant(tt, a, b):
+    return tt.get_backend(tt.kAMD).batched_matmul_variant(a, b)
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+@pytest.mark.parametrize("shape", SHAPES)
+def test_store_extensions_match_numpy(tt, dtype, shape):
+    B, N, K, M = shape
+    rng = np.random.default_rng(N + K + M)
+    a = rng.integers(-3, 4, (B, N, K)).astype(dtype)
+    b = rng.integers(-3, 4, (B, K, M)).astype(dtype)
+    bias = rng.integers(-5, 6, (M,)).astype(dtype)
+    z = rng.integers(-2, 3, (B, N, M)).astype(dtype)           # the saved input of a ReLU: negatives, zeros, positives
+    be = tt.get_backend(tt.kAMD)
+    ta, tb, tbias, tz = (tt.Tensor.from_numpy(v) for v in (a, b, bias, z))
+    prod = np.matmul(a.astype(np.float64), b.astype(np.float64))
+    # 1. Linear + ReLU: out keeps the value before the ReLU, relu_out its positive part
+    act = tt.Tensor.empty((B, N, M), ta.dtype)
+    out = be.batched_matmul(ta, tb, bias=tbias, bias_mode=1, relu_out=act)
+    want = (prod + bias).astype(dtype)
+    assert np.array_equal(out.to_numpy(), want), _variant(tt, ta, tb)
+    assert np.array_equal(act.to_numpy(), np.maximum(want, 0))
+    # 2. ReLU backward mask and column sums in one store
+    cs = tt.Tensor.empty((B, M), ta.dtype)
+    dz = be.batched_matmul(ta, tb, relu_grad_input=tz, colsum_out=cs)
+    want_dz = (prod * np.where(z < 0, 0.0, 1.0)).astype(dtype)
+    assert np.array_equal(dz.to_numpy(), want_dz)
+    assert np.array_equal(cs.to_numpy(), want_dz.sum(axis=1).astype(dtype))
+    # 3. column sums alone, on transposed views (the operands of a backward GEMM)
+    at = tt.Tensor.from_numpy(np.ascontiguousarray(a.transpose(0, 2, 1))).permute(0, 2, 1)
+    bt = tt.Tensor.from_numpy(np.ascontiguousarray(b.transpose(0, 2, 1))).permute(0, 2, 1)
+    cs2 = tt.Tensor.empty((B, M), ta.dtype)
+    out2 = be.batched_matmul(at, bt, colsum_out=cs2)
+    assert np.array_equal(out2.to_numpy(), prod.astype(dtype))
+    assert np.array_equal(cs2.to_numpy(), prod.sum(axis=1).astype(dtype))
+    # the plain call is untouched by the extensions
+    assert np.array_equal(be.batched_matmul(ta, tb).to_numpy(), prod.astype(dtype))
+
+
+def test_store_extension_argument_checks(tt):
+    be = tt.get_backend(tt.kAMD)
+    a = tt.Tensor.from_numpy(np.ones((1, 8, 8), np.float32))
+    good = tt.Tensor.empty((1, 8, 8), tt._capi.F32)
+    with pytest.raises(tt.TTException):
+        be.batched_matmul(a, a, relu=True, relu_out=good)              # relu_out excludes relu
+    with pytest.raises(tt.TTException):
+        be.batched_matmul(a, a, accumulate=True, out=good, colsum_out=tt.Tensor.empty((1, 8), tt._capi.F32))
+    with pytest.raises(tt.TTException):
+        be.batched_matmul(a, a, relu_out=tt.Tensor.empty((1, 8, 4), tt._capi.F32))
+    i = tt.Tensor.from_numpy(np.ones((1, 8, 8), np.int32))
+    with pytest.raises(tt.TTException):
+        be.batched_matmul(i, i, colsum_out=tt.Tensor.empty((1, 8), tt._capi.I32))
+    # integer operands do carry the mask and the second output (vector-ALU kernel)
+    zi = tt.Tensor.from_numpy(np.array([[[-1, 0, 1, 2, -3, 4, 5, -6]] * 8], np.int32))
+    acti = tt.Tensor.empty((1, 8, 8), tt._capi.I32)
+    got = be.batched_matmul(i, i, relu_grad_input=zi, relu_out=acti).to_numpy()
+    assert np.array_equal(got[0], np.where(zi.to_numpy()[0] < 0, 0, 8)) and np.array_equal(acti.to_numpy(), got)
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+@pytest.mark.parametrize("shape", [(1024, 10), (7, 3), (50000, 64), (300, 1000), (1, 1), (4096, 33)])
+def test_mse_loss_forward_and_backward(tt, dtype, shape):
+    rng = np.random.default_rng(shape[0])
+    y = rng.uniform(-1, 1, shape).astype(dtype)
+    t = rng.uniform(-1, 1, shape).astype(dtype)
+    narrow = shape[1] <= 64
+    loss, g, cs = tt.mse_loss(tt.Tensor.from_numpy(y), tt.Tensor.from_numpy(t), grad=True, bias_grad=narrow)
+    d = y.astype(np.float64) - t
+    tol = 1e-5 if dtype == np.float32 else 1e-13
+    assert abs(float(loss.to_numpy()[0]) - np.mean(d * d)) <= tol * np.mean(d * d)
+    want_g = (dtype(1) / dtype(y.size) * dtype(2)) * (y - t)       # ((1/N) * 2) * (y - t), the reference's rounding
+    assert np.array_equal(g.to_numpy(), want_g)
+    if narrow:
+        assert np.max(np.abs(cs.to_numpy() - want_g.astype(np.float64).sum(0))) <= tol * np.abs(want_g).sum(0).max()
+    else:
+        with pytest.raises(tt.TTException):
+            tt.mse_loss(tt.Tensor.from_numpy(y), tt.Tensor.from_numpy(t), grad=True, bias_grad=True)
+    only_loss, none_g, none_cs = tt.mse_loss(tt.Tensor.from_numpy(y), tt.Tensor.from_numpy(t), grad=False)
+    assert none_g is None and none_cs is None and only_loss.to_numpy()[0] == loss.to_numpy()[0]
+
+
+def fused_mlp_step(tt, x, t, params):
+    """The training step of benchmark configuration 5 from the fused forms: 3 forward launches (+ the split reduction's
+    sum for the 10-column head), the loss with its gradient and the head's bias gradient in one, and per layer one GEMM
+    for dx (mask and bias gradient in its store, + the sum of the partial rows) and one for dW."""
+    (W1, b1), (W2, b2), (W3, b3) = params
+    z1, a1 = tt.linear_relu(x, W1, b1)
+    z2, a2 = tt.linear_relu(a1, W2, b2)
+    y = tt.linear(a2, W3, b3)
+    loss, gy, db3 = tt.mse_loss(y, t, grad=True, bias_grad=True)
+    dz2, dW3, db2 = tt.linear_backward(gy, a2, W3, relu_input=z2)
+    dz1, dW2, db1 = tt.linear_backward(dz2, a1, W2, relu_input=z1)
+    dX, dW1, _ = tt.linear_backward(dz1, x, W1, bias_grad=False)
+    return dict(y=y, loss=loss, dW1=dW1, db1=db1, dW2=dW2, db2=db2, dW3=dW3, db3=db3, dX=dX, z1=z1, z2=z2)
+
+
+def test_fused_mlp_training_step_matches_the_oracle_and_fits_15_launches(tt, oracle):
+    X = oracle.Generator(0).uniform_real(0.0, 1.0, (1024, 784))
+    T = oracle.Generator(1).uniform_real(0.0, 1.0, (1024, 10))
+    g = oracle.Generator(0)
+    params_h = [oracle.linear_init(g, a, b) for a, b in ((784, 1024), (1024, 1024), (1024, 10))]
+    d = tt.Tensor.from_numpy
+    x, t = d(X), d(T)
+    params = [(d(W), d(b)) for W, b in params_h]
+    got = {k: v.to_numpy() for k, v in fused_mlp_step(tt, x, t, params).items()}
+    masks = (np.where(got["z1"] < 0, np.float32(0), np.float32(1)), np.where(got["z2"] < 0, np.float32(0), np.float32(1)))
+    want = mlp_train_step(X, T, params_h, lambda a, b: oracle.matmul(a, b),
+                          lambda a, b, gr: tuple(v[0] for v in oracle.matmul_backward(a[None], b[None], gr[None])), masks=masks)
+    own = mlp_train_step(X, T, params_h, lambda a, b: oracle.matmul(a, b),
+                         lambda a, b, gr: tuple(v[0] for v in oracle.matmul_backward(a[None], b[None], gr[None])))
+    assert sum(int(np.sum(a != b)) for a, b in zip(masks, own["masks"])) <= 8   # z within rounding of 0
+    for key in ("y", "dW1", "db1", "dW2", "db2", "dW3", "db3", "dX"):
+        assert got[key].shape == want[key].shape, key
+        assert max_rel_error(got[key], want[key]) <= 1e-4, key
+    assert abs(float(got["loss"][0]) - float(want["loss"])) <= 1e-4 * abs(float(want["loss"]))
+    # launches: record the step into a HIP graph and count its kernel nodes
+    stream = tt.graph.Stream()
+    graph = None
+    try:
+        graph = tt.graph.Graph(stream, lambda: list(fused_mlp_step(tt, x, t, params).values()))
+        assert graph.num_nodes() <= 15, graph.num_nodes()
+        graph.launch()
+        stream.synchronize()
+        for k, v in zip(("y", "loss", "dW1", "db1", "dW2", "db2", "dW3", "db3", "dX"), graph.outputs):
+            assert np.array_equal(v.to_numpy(), got[k]), k   # same kernels, same inputs
+    finally:
+        if graph is not None:
+            graph.close()
+        stream.close()

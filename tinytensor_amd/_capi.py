@@ -28,7 +28,8 @@ class View4(C.Structure):
 
 
 class Epilogue(C.Structure):
-    _fields_ = [("bias", C.c_void_p), ("bias_mode", C.c_int32), ("relu", C.c_int32), ("accumulate", C.c_int32)]
+    _fields_ = [("bias", C.c_void_p), ("bias_mode", C.c_int32), ("relu", C.c_int32), ("accumulate", C.c_int32),
+                ("reserved", C.c_int32), ("relu_out", C.c_void_p), ("relu_grad_input", C.c_void_p), ("colsum_out", C.c_void_p)]
 
 
 def _bind(lib: C.CDLL) -> None:
@@ -60,6 +61,7 @@ def _bind(lib: C.CDLL) -> None:
         "ttamd_sum": (i, [i, i, i, C.POINTER(C.c_int64), vp, C.c_int64, C.POINTER(C.c_int64), i, vp, vp]),
         "ttamd_full": (i, [i, i, vp, C.c_int64, vp, vp]),
         "ttamd_random_fill": (i, [i, i, i, C.c_double, C.c_double, C.POINTER(C.c_uint64), C.c_int64, vp, vp]),
+        "ttamd_mse_loss": (i, [i, i, C.c_int64, C.c_int64, vp, vp, vp, vp, vp, vp]),
         "ttamd_random_fill_view": (i, [i, i, i, C.c_double, C.c_double, C.POINTER(C.c_uint64), i, C.POINTER(C.c_int64),
                                        C.POINTER(C.c_int64), vp, C.c_int64, vp]),
         "ttamd_batched_matmul": (i, [i, i, i, i, i, i, C.POINTER(View3), C.POINTER(View3), vp, C.POINTER(Epilogue), vp]),

@@ -85,6 +85,12 @@ struct GemmArgs {
     int M, N, K, batch;
     const void *bias;
     int bias_mode, relu, accumulate;
+    // extensions of the store (mfma::EpilogueExt): second output max(value, 0); mask "0 where zmask < 0"; column sums
+    void *relu_out;
+    const void *zmask;
+    void *colsum_out;      // [batch, N], written by the kernel that adds the partial rows
+    void *colsum_partial;  // [batch, colsum_rows, N] partial sums, filled in by the launcher (scratch)
+    int colsum_rows;
 };
 
 // Launchers (defined in gemm_mfma.hip / gemm_simt.hip).  `variant_only`: fill *variant with the

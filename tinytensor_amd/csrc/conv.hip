@@ -578,8 +578,8 @@ __device__ __forceinline__ void store_tile_padded_rows(Engine &eng, T *__restric
     auto bias_of = [&](int ml) { return Vec<T, 1>::load(bias_m, static_cast<uint32_t>(m0 + ml) * kSz); };
     const bool pairs_ok = (w % 2 == 0) && (reinterpret_cast<uintptr_t>(C) % (2 * sizeof(T)) == 0);
     eng.template for_each<true>(
-        pairs_ok, [&](int ml, int nl, T v) { buffer_store(out, offset_of(ml, nl), v + bias_of(ml)); },
-        [&](int ml, int nl, T v0, T v1) {
+        pairs_ok, [&](int ml, int nl, T v, int) { buffer_store(out, offset_of(ml, nl), v + bias_of(ml)); },
+        [&](int ml, int nl, T v0, T v1, int) {
             const T bv = bias_of(ml);
             pair_t o;
             o[0] = v0 + bv;

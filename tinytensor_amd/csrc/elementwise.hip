@@ -763,6 +763,104 @@ ttamd_status cast_from(ttamd_dtype to, const void *a, const ViewDesc &va, void *
     default: break;                                            \
     }
 
+// nn::mse_loss with mean reduction (nn/loss.cpp:69-72: pow(input - target, 2).mean(), the mean being
+// (x / numel).sum(), autograd/reduce_ops.cpp:195-200) together with its backward (grad_output / numel from the mean,
+// times 2 * (input - target) from pow: autograd/reduce_ops.cpp:201-205, binary_ops.cpp:153-159) and, for narrow
+// matrices, the column sums of that gradient (the bias gradient of the Linear layer that produced `input`).
+// Lane layout: CP column lanes (a power of two >= cols, at most 64) by 256 / CP row lanes; a lane walks its column
+// down the rows in steps of (row lanes * blocks).  Sums are folded over the row lanes in a fixed tree, per-block
+// partials ([blocks][cols + 1]: column sums, then the loss) are added by block index: deterministic.
+template <typename T, int CP>
+__global__ void __launch_bounds__(256) mse_loss_kernel(const T *__restrict__ y, const T *__restrict__ t, int64_t rows, int cols, T inv_n,
+                                                      T *__restrict__ grad, T *__restrict__ partial, T *__restrict__ loss,
+                                                      T *__restrict__ colsum) {
+    constexpr int RL = 256 / CP;
+    __shared__ T red[RL][CP + 1];
+    __shared__ T red_loss[256];
+    const int cl = threadIdx.x % CP, rl = threadIdx.x / CP;
+    const T scale = inv_n * T(2);
+    T csum = T(0), lsum = T(0);
+    if (cl < cols) {
+        for (int64_t r = static_cast<int64_t>(blockIdx.x) * RL + rl; r < rows; r += static_cast<int64_t>(gridDim.x) * RL) {
+            const int64_t i = r * cols + cl;
+            const T d = y[i] - t[i];
+            lsum += d * d * inv_n;
+            const T g = scale * d;
+            if (grad) grad[i] = g;
+            csum += g;
+        }
+    }
+    red[rl][cl] = csum;
+    red_loss[threadIdx.x] = lsum;
+    __syncthreads();
+    for (int h = RL / 2; h > 0; h >>= 1) {
+        if (rl < h) red[rl][cl] += red[rl + h][cl];
+        __syncthreads();
+    }
+    for (int h = 128; h > 0; h >>= 1) {
+        if (static_cast<int>(threadIdx.x) < h) red_loss[threadIdx.x] += red_loss[threadIdx.x + h];
+        __syncthreads();
+    }
+    if (gridDim.x == 1) {  // a single workgroup holds the final sums: no partials, no finishing kernel
+        if (rl == 0 && cl < cols && colsum) colsum[cl] = red[0][cl];
+        if (threadIdx.x == 0) loss[0] = red_loss[0];
+        return;
+    }
+    T *p = partial + static_cast<int64_t>(blockIdx.x) * (cols + 1);
+    if (rl == 0 && cl < cols) p[cl] = red[0][cl];
+    if (threadIdx.x == 0) p[cols] = red_loss[0];
+}
+
+// out[j] = sum over blocks b (ascending) of partial[b][j], j < cols + 1; column sums to colsum (may be null), the
+// last entry to loss.
+template <typename T>
+__global__ void __launch_bounds__(256) mse_loss_finish_kernel(const T *__restrict__ partial, int blocks, int cols, T *__restrict__ loss,
+                                                             T *__restrict__ colsum) {
+    const int j = blockIdx.x * blockDim.x + threadIdx.x;
+    if (j > cols) return;
+    T v = T(0);
+    for (int b = 0; b < blocks; ++b) v += partial[static_cast<int64_t>(b) * (cols + 1) + j];
+    if (j == cols) loss[0] = v;
+    else if (colsum) colsum[j] = v;
+}
+
+template <typename T>
+ttamd_status launch_mse_loss(int device, int64_t rows, int64_t cols, const void *y, const void *t, void *loss, void *grad, void *colsum,
+                             hipStream_t st) {
+    // wide matrices (no column sums there): one flat column of rows * cols elements
+    if (cols > 64) {
+        rows *= cols;
+        cols = 1;
+    }
+    int cp = 1;
+    while (cp < cols) cp *= 2;
+    const int rl = 256 / cp;
+    int64_t blocks = (rows + static_cast<int64_t>(rl) * 8 - 1) / (static_cast<int64_t>(rl) * 8);  // about 8 rows per lane: a lane's
+                                                                                                 // loads are one dependent chain
+    if (blocks > 1024) blocks = 1024;
+    if (blocks < 1) blocks = 1;
+    void *ws = nullptr;
+    if (blocks > 1)
+        if (ttamd_status s = stream_scratch(device, st, static_cast<size_t>(blocks) * (cols + 1) * sizeof(T), &ws)) return s;
+    const T inv_n = T(1) / static_cast<T>(rows * cols);
+    const T *yp = static_cast<const T *>(y), *tp = static_cast<const T *>(t);
+    T *gp = static_cast<T *>(grad), *pp = static_cast<T *>(ws), *lp = static_cast<T *>(loss), *cs = static_cast<T *>(colsum);
+    const dim3 grid(static_cast<unsigned>(blocks)), block(256);
+    const int c = static_cast<int>(cols);
+    switch (cp) {
+    case 1: mse_loss_kernel<T, 1><<<grid, block, 0, st>>>(yp, tp, rows, c, inv_n, gp, pp, lp, cs); break;
+    case 2: mse_loss_kernel<T, 2><<<grid, block, 0, st>>>(yp, tp, rows, c, inv_n, gp, pp, lp, cs); break;
+    case 4: mse_loss_kernel<T, 4><<<grid, block, 0, st>>>(yp, tp, rows, c, inv_n, gp, pp, lp, cs); break;
+    case 8: mse_loss_kernel<T, 8><<<grid, block, 0, st>>>(yp, tp, rows, c, inv_n, gp, pp, lp, cs); break;
+    case 16: mse_loss_kernel<T, 16><<<grid, block, 0, st>>>(yp, tp, rows, c, inv_n, gp, pp, lp, cs); break;
+    case 32: mse_loss_kernel<T, 32><<<grid, block, 0, st>>>(yp, tp, rows, c, inv_n, gp, pp, lp, cs); break;
+    default: mse_loss_kernel<T, 64><<<grid, block, 0, st>>>(yp, tp, rows, c, inv_n, gp, pp, lp, cs); break;
+    }
+    if (blocks > 1) mse_loss_finish_kernel<T><<<dim3(1), dim3(256), 0, st>>>(pp, static_cast<int>(blocks), c, lp, cs);
+    TTAMD_HIP_CHECK(hipGetLastError());
+    return TTAMD_OK;
+}
+
 }  // namespace
 }  // namespace ttamd
 
@@ -1146,6 +1244,31 @@ ttamd_status ttamd_random_fill(int device, ttamd_dtype dtype, int dist, double p
     }
     const int64_t shape[1] = {numel}, stride[1] = {1};
     return ttamd_random_fill_view(device, dtype, dist, p0, p1, master_state, 1, shape, stride, out, 0, stream);
+}
+
+ttamd_status ttamd_mse_loss(int device, ttamd_dtype dtype, int64_t rows, int64_t cols, const void *input, const void *target,
+                            void *loss_out, void *grad_input_out, void *grad_colsum_out, void *stream) {
+    if (dtype != TTAMD_F32 && dtype != TTAMD_F64) {
+        set_error("mse_loss: floating point dtypes only");
+        return TTAMD_ERR_UNSUPPORTED_DTYPE;
+    }
+    if (rows < 0 || cols < 0 || rows * cols > 0x7fffffffLL) {
+        set_error("mse_loss: invalid shape [%lld, %lld]", static_cast<long long>(rows), static_cast<long long>(cols));
+        return TTAMD_ERR_INVALID_ARGUMENT;
+    }
+    if (grad_colsum_out && cols > 64) {
+        set_error("mse_loss: the fused column sums serve at most 64 columns (given %lld); sum the gradient with ttamd_sum",
+                  static_cast<long long>(cols));
+        return TTAMD_ERR_INVALID_ARGUMENT;
+    }
+    if (ttamd_status s = use_device(device)) return s;
+    if (!loss_out || (rows * cols > 0 && (!input || !target))) {
+        set_error("mse_loss: NULL data pointer");
+        return TTAMD_ERR_INVALID_ARGUMENT;
+    }
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    if (dtype == TTAMD_F32) return launch_mse_loss<float>(device, rows, cols, input, target, loss_out, grad_input_out, grad_colsum_out, st);
+    return launch_mse_loss<double>(device, rows, cols, input, target, loss_out, grad_input_out, grad_colsum_out, st);
 }
 
 }  // extern "C"

@@ -59,6 +59,19 @@ ttamd_status build_args(ttamd_dtype dtype, int B, int N, int K, int M, const tta
             set_error("batched_matmul: invalid epilogue (bias_mode=%d, bias=%p)", ep->bias_mode, ep->bias);
             return TTAMD_ERR_INVALID_ARGUMENT;
         }
+        if ((ep->relu_out && ep->relu) || (ep->colsum_out && ep->accumulate)) {
+            set_error("batched_matmul: invalid epilogue (relu_out excludes relu, colsum_out excludes accumulate)");
+            return TTAMD_ERR_INVALID_ARGUMENT;
+        }
+        if (ep->colsum_out && dtype != TTAMD_F32 && dtype != TTAMD_F64) {
+            set_error("batched_matmul: colsum_out is implemented for f32 and f64");
+            return TTAMD_ERR_UNSUPPORTED_DTYPE;
+        }
+        if (reinterpret_cast<uintptr_t>(ep->relu_out) % esz != 0 || reinterpret_cast<uintptr_t>(ep->relu_grad_input) % esz != 0 ||
+            reinterpret_cast<uintptr_t>(ep->colsum_out) % esz != 0) {
+            set_error("batched_matmul: epilogue pointers must be aligned to the element size");
+            return TTAMD_ERR_INVALID_ARGUMENT;
+        }
     }
     g->A = static_cast<const char *>(lhs->data) + lhs->offset * static_cast<int64_t>(esz);
     g->B = static_cast<const char *>(rhs->data) + rhs->offset * static_cast<int64_t>(esz);
@@ -77,6 +90,11 @@ ttamd_status build_args(ttamd_dtype dtype, int B, int N, int K, int M, const tta
     g->bias_mode = ep ? ep->bias_mode : 0;
     g->relu = ep ? ep->relu : 0;
     g->accumulate = ep ? ep->accumulate : 0;
+    g->relu_out = ep ? ep->relu_out : nullptr;
+    g->zmask = ep ? ep->relu_grad_input : nullptr;
+    g->colsum_out = ep ? ep->colsum_out : nullptr;
+    g->colsum_partial = nullptr;
+    g->colsum_rows = 0;
     return TTAMD_OK;
 }
 
@@ -94,6 +112,10 @@ ttamd_status batched_matmul(int device, ttamd_dtype dtype, int B, int N, int K, 
         if (handled) return TTAMD_OK;
     }
     // K == 0 also lands here: the vector-ALU kernel then stores the empty sum (0, + bias).  It uses no scratch.
+    if (g.colsum_out) {
+        set_error("batched_matmul: colsum_out needs the matrix-core kernels (K > 0, rows under a tile below 2 GiB)");
+        return TTAMD_ERR_INVALID_ARGUMENT;
+    }
     return launch_gemm_simt(dtype, g, st, &variant, false);
 }
 

@@ -55,10 +55,27 @@ ttamd_status fixed_scratch_address(int device, void **out) {
 // memory in every step.  Measured at depth 4: 1024 x 784 x 1024 26.2 -> 22.1 us, 1024 x 4096 x 1024 87 -> 78 us; the
 // host picks the depth per launch (launch_mfma_typed).
 // EPI: which epilogues the kernel carries.  kEpiAny tests the epilogue flags at run time and supports split k (the
-// 64 x 64 tile).  The big tiles are compiled twice, kEpiLean (plain store only) and kEpiFull (bias / ReLU /
-// accumulate), and never split k: with both store walks in one kernel the register allocator spills accumulators
-// ahead of the branch for the sake of the heavier walk, and the plain store pays for it.
-constexpr int kEpiAny = 0, kEpiLean = 1, kEpiFull = 2;
+// 64 x 64 tile).  The big tiles are compiled three times, kEpiLean (plain store only), kEpiFull (bias / ReLU /
+// accumulate) and kEpiExt (those plus second output, mask and column sums), and never split k: with several store
+// walks in one kernel the register allocator spills accumulators ahead of the branch for the sake of the heaviest
+// walk, and the plain store pays for it.
+constexpr int kEpiAny = 0, kEpiLean = 1, kEpiFull = 2, kEpiExt = 3;
+
+// The store's extensions for one workgroup: pointers moved to the batch, partial column sums to this tile row's rows.
+template <typename T>
+__device__ __forceinline__ EpilogueExt<T> make_ext(const GemmArgs &g, int batch, int tm, int wgm) {
+    const int64_t mn = static_cast<int64_t>(g.M) * g.N;
+    EpilogueExt<T> e;
+    e.relu_out = g.relu_out ? static_cast<T *>(g.relu_out) + batch * mn : nullptr;
+    e.zmask = g.zmask ? static_cast<const T *>(g.zmask) + batch * mn : nullptr;
+    e.colsum = g.colsum_partial ? static_cast<T *>(g.colsum_partial) + static_cast<int64_t>(batch) * g.colsum_rows * g.N : nullptr;
+    e.colsum_row0 = tm * wgm;
+    return e;
+}
+__host__ __device__ inline bool ext_store(const GemmArgs &g) { return g.relu_out || g.zmask || g.colsum_out; }
+__host__ __device__ inline bool plain_store(const GemmArgs &g) {
+    return g.bias_mode == 0 && !g.relu && !g.accumulate && !ext_store(g);
+}
 template <typename T, int BM, int BN, int BK, int WGM, int WGN, bool A_KC, int A_VEC, bool B_KC, int B_VEC, int PF, int EPI>
 __global__ void __launch_bounds__(kThreads, (BM * BN * sizeof(T) > 256 * 128 * 4 || (sizeof(T) == 8 && BM * BN >= 128 * 128)) ? 1 : 2)  // 256 x 256 (fp64 128 x 128 and up): one workgroup per CU, accumulators in AGPRs
 gemm_mfma_kernel(GemmArgs g, int tiles_m, int tiles_n, int ksplit, int k_chunk, T *partial) {
@@ -88,18 +105,24 @@ gemm_mfma_kernel(GemmArgs g, int tiles_m, int tiles_n, int ksplit, int k_chunk, 
 
     Engine eng;
     eng.init(tid);
-    eng.run(sa, sb, smem, Kc, !sa.edge && !sb.edge && Kc % BK == 0);
+    eng.run(sa, sb, smem, Kc, !sa.row_mask && !sb.row_mask);
 
     T *C = static_cast<T *>(g.C) + static_cast<int64_t>(batch) * g.M * g.N;
     if constexpr (EPI == kEpiLean) {
         store_tile_dense<T, true>(eng, C, g.M, g.N, m0, n0, static_cast<const T *>(nullptr), 0, 0, 0);
     } else if constexpr (EPI == kEpiFull) {
         store_tile_dense<T, false>(eng, C, g.M, g.N, m0, n0, static_cast<const T *>(g.bias), g.bias_mode, g.relu, g.accumulate);
+    } else if constexpr (EPI == kEpiExt) {
+        store_tile_dense<T, false, true>(eng, C, g.M, g.N, m0, n0, static_cast<const T *>(g.bias), g.bias_mode, g.relu, g.accumulate,
+                                         make_ext<T>(g, batch, tm, WGM));
     } else if (ksplit == 1) {
-        if (g.bias_mode == 0 && !g.relu && !g.accumulate)  // the common case gets a store loop free of epilogue work
+        if (plain_store(g))  // the common case gets a store loop free of epilogue work
             store_tile_dense<T, true>(eng, C, g.M, g.N, m0, n0, static_cast<const T *>(nullptr), 0, 0, 0);
-        else
+        else if (!ext_store(g))
             store_tile_dense<T, false>(eng, C, g.M, g.N, m0, n0, static_cast<const T *>(g.bias), g.bias_mode, g.relu, g.accumulate);
+        else
+            store_tile_dense<T, false, true>(eng, C, g.M, g.N, m0, n0, static_cast<const T *>(g.bias), g.bias_mode, g.relu, g.accumulate,
+                                             make_ext<T>(g, batch, tm, WGM));
     } else {
         store_tile_dense<T, true>(eng, partial + static_cast<int64_t>(z) * g.M * g.N, g.M, g.N, m0, n0,
                                   static_cast<const T *>(nullptr), 0, 0, 0);
@@ -137,7 +160,7 @@ gemm_mfma_dual_kernel(GemmArgs g, int tiles_m, int tiles_n, int k_half) {
     sb.init(b_base, tid, g.N - n0, g.b_sn, g.b_sk, Kc);
     Engine eng;
     eng.init(tid);
-    eng.run(sa, sb, smem, Kc, !sa.edge && !sb.edge && Kc % BK == 0);
+    eng.run(sa, sb, smem, Kc, !sa.row_mask && !sb.row_mask);
     __syncthreads();  // every wave is done with its tiles: the lower half's buffers become the exchange area
     T *const exchange = reinterpret_cast<T *>(smem_raw);
     if (half == 1) eng.park_acc(exchange, tid);
@@ -145,10 +168,13 @@ gemm_mfma_dual_kernel(GemmArgs g, int tiles_m, int tiles_n, int k_half) {
     if (half == 1) return;
     eng.add_parked_acc(exchange, tid);
     T *C = static_cast<T *>(g.C) + static_cast<int64_t>(batch) * g.M * g.N;
-    if (g.bias_mode == 0 && !g.relu && !g.accumulate)
+    if (plain_store(g))
         store_tile_dense<T, true>(eng, C, g.M, g.N, m0, n0, static_cast<const T *>(nullptr), 0, 0, 0);
-    else
+    else if (!ext_store(g))
         store_tile_dense<T, false>(eng, C, g.M, g.N, m0, n0, static_cast<const T *>(g.bias), g.bias_mode, g.relu, g.accumulate);
+    else
+        store_tile_dense<T, false, true>(eng, C, g.M, g.N, m0, n0, static_cast<const T *>(g.bias), g.bias_mode, g.relu, g.accumulate,
+                                         make_ext<T>(g, batch, tm, WGM));
 }
 
 // C[b][i] = epilogue(sum over s of partial[b * ksplit + s][i]), s ascending (deterministic).
@@ -164,11 +190,35 @@ __global__ void __launch_bounds__(256) splitk_reduce_kernel(GemmArgs g, const T 
     const T *bias = static_cast<const T *>(g.bias);
     if (g.bias_mode == 1) v += bias[i % g.N];
     if (g.bias_mode == 2) v += bias[i / g.N];
+    if (g.zmask && static_cast<const T *>(g.zmask)[static_cast<int64_t>(batch) * mn + i] < T(0)) v = T(0);
     if (g.relu) v = v > T(0) ? v : T(0);
     T *C = static_cast<T *>(g.C) + static_cast<int64_t>(batch) * mn;
     if (g.accumulate) v += C[i];
     C[i] = v;
+    if (g.relu_out) static_cast<T *>(g.relu_out)[static_cast<int64_t>(batch) * mn + i] = v > T(0) ? v : T(0);
 }
+
+// colsum[b][n] = sum over r of partial[b][r][n], r ascending (deterministic).
+template <typename T>
+__global__ void __launch_bounds__(256) colsum_reduce_kernel(const T *__restrict__ partial, int rows, int N, T *__restrict__ out) {
+    const int n = blockIdx.x * blockDim.x + threadIdx.x;
+    if (n >= N) return;
+    const T *p = partial + static_cast<int64_t>(blockIdx.y) * rows * N + n;
+    T v = T(0);
+    int r = 0;
+    for (; r + 8 <= rows; r += 8) {  // eight loads in flight, added in row order
+        T x[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) x[u] = p[static_cast<int64_t>(r + u) * N];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) v += x[u];
+    }
+    for (; r < rows; ++r) v += p[static_cast<int64_t>(r) * N];
+    out[static_cast<int64_t>(blockIdx.y) * N + n] = v;
+}
+
+// Scratch of a launch: the library's fixed array (calls that must not allocate) or the stream's growing buffer.
+ttamd_status launch_scratch(int device, hipStream_t stream, size_t bytes, bool fixed, void **out);
 
 // ---------------------------------------------------------------------------------------------
 // Host side: operand classification and variant table.
@@ -220,26 +270,59 @@ struct SplitPlan {
     bool fixed_scratch = false;  // partial tiles go to the library's fixed array (the call must not allocate)
 };
 
+ttamd_status launch_scratch(int device, hipStream_t stream, size_t bytes, bool fixed, void **out) {
+    if (!fixed) return stream_scratch(device, stream, bytes, out);
+    if (bytes > kFixedScratchBytes) {
+        set_error("batched_matmul_noalloc: this product needs %zu bytes of partial results (a split reduction's tiles or "
+                  "the column sums' rows); the fixed scratch holds %zu (use ttamd_batched_matmul)", bytes, kFixedScratchBytes);
+        return TTAMD_ERR_INVALID_ARGUMENT;
+    }
+    return fixed_scratch_address(device, out);
+}
+
+// Column sums: `rows` partial rows per batch item go to scratch, finish_colsum adds them up after the GEMM.
+template <typename T>
+ttamd_status prepare_colsum(GemmArgs &g, int rows, int device, hipStream_t stream, bool fixed) {
+    if (!g.colsum_out) return TTAMD_OK;
+    void *ws = nullptr;
+    const size_t bytes = static_cast<size_t>(g.batch) * rows * g.N * sizeof(T);
+    if (ttamd_status st = launch_scratch(device, stream, bytes, fixed, &ws)) return st;
+    g.colsum_partial = ws;
+    g.colsum_rows = rows;
+    return TTAMD_OK;
+}
+template <typename T>
+ttamd_status finish_colsum(const GemmArgs &g, hipStream_t stream) {
+    if (!g.colsum_out) return TTAMD_OK;
+    colsum_reduce_kernel<T><<<dim3(static_cast<unsigned>((g.N + 63) / 64), g.batch), dim3(64), 0, stream>>>(
+        static_cast<const T *>(g.colsum_partial), g.colsum_rows, g.N, static_cast<T *>(g.colsum_out));
+    TTAMD_HIP_CHECK(hipGetLastError());
+    return TTAMD_OK;
+}
+
 template <typename T, int BM, int BN, int BK, int WGM, int WGN, bool A_KC, int A_VEC, bool B_KC, int B_VEC, int PF>
 ttamd_status launch_variant(const GemmArgs &g, const SplitPlan &sp, int device, hipStream_t stream) {
     using StA = Stager<T, BM, BK, A_KC, A_VEC, PF>;
     using StB = Stager<T, BN, BK, B_KC, B_VEC, PF>;
     constexpr size_t lds_bytes = TileEngine<T, BM, BN, BK, WGM, WGN, StA, StB>::kLdsBytes;
     constexpr bool kTwoKernels = BM * BN >= 128 * 128;
-    const bool lean = g.bias_mode == 0 && !g.relu && !g.accumulate;
+    const bool lean = plain_store(g);
     if (kTwoKernels && sp.ksplit != 1) {
         set_error("batched_matmul: internal error, split k planned for a %d x %d tile", BM, BN);
         return TTAMD_ERR_INVALID_ARGUMENT;
     }
-    constexpr int kEpiA = kTwoKernels ? kEpiLean : kEpiAny, kEpiB = kTwoKernels ? kEpiFull : kEpiAny;
-    auto kernel = lean ? gemm_mfma_kernel<T, BM, BN, BK, WGM, WGN, A_KC, A_VEC, B_KC, B_VEC, PF, kEpiA>
-                       : gemm_mfma_kernel<T, BM, BN, BK, WGM, WGN, A_KC, A_VEC, B_KC, B_VEC, PF, kEpiB>;
-    static bool configured[kMaxDevices][2] = {};  // raising the dynamic LDS limit: once per kernel and device
+    constexpr int kEpiA = kTwoKernels ? kEpiLean : kEpiAny, kEpiB = kTwoKernels ? kEpiFull : kEpiAny,
+                  kEpiC = kTwoKernels ? kEpiExt : kEpiAny;
+    const int which = lean ? 0 : (ext_store(g) ? 2 : 1);
+    auto kernel = which == 0   ? gemm_mfma_kernel<T, BM, BN, BK, WGM, WGN, A_KC, A_VEC, B_KC, B_VEC, PF, kEpiA>
+                  : which == 1 ? gemm_mfma_kernel<T, BM, BN, BK, WGM, WGN, A_KC, A_VEC, B_KC, B_VEC, PF, kEpiB>
+                               : gemm_mfma_kernel<T, BM, BN, BK, WGM, WGN, A_KC, A_VEC, B_KC, B_VEC, PF, kEpiC>;
+    static bool configured[kMaxDevices][3] = {};  // raising the dynamic LDS limit: once per kernel and device
     const int slot = device >= 0 && device < kMaxDevices ? device : 0;
-    if ((!configured[slot][lean] || slot != device) && lds_bytes > 48 * 1024) {
+    if ((!configured[slot][which] || slot != device) && lds_bytes > 48 * 1024) {
         TTAMD_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
                                             hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_bytes)));
-        configured[slot][lean] = true;
+        configured[slot][which] = true;
     }
     const int tiles_m = (g.M + BM - 1) / BM, tiles_n = (g.N + BN - 1) / BN;
     const int64_t blocks = static_cast<int64_t>(tiles_m) * tiles_n * g.batch * sp.ksplit;
@@ -248,22 +331,16 @@ ttamd_status launch_variant(const GemmArgs &g, const SplitPlan &sp, int device, 
         return TTAMD_ERR_INVALID_ARGUMENT;
     }
     T *partial = nullptr;
-    if (sp.ksplit > 1) {
+    GemmArgs ga = g;
+    if (sp.ksplit > 1) {  // (never together with column sums: the planner does not split then)
         void *ws = nullptr;
         const size_t bytes = static_cast<size_t>(sp.ksplit) * g.batch * g.M * g.N * sizeof(T);
-        if (sp.fixed_scratch) {
-            if (bytes > kFixedScratchBytes) {
-                set_error("batched_matmul_noalloc: this product splits its reduction %d ways and needs %zu bytes of partial "
-                          "tiles; the fixed scratch holds %zu (use ttamd_batched_matmul)", sp.ksplit, bytes, kFixedScratchBytes);
-                return TTAMD_ERR_INVALID_ARGUMENT;
-            }
-            if (ttamd_status st = fixed_scratch_address(device, &ws)) return st;
-        } else if (ttamd_status st = stream_scratch(device, stream, bytes, &ws)) {
-            return st;
-        }
+        if (ttamd_status st = launch_scratch(device, stream, bytes, sp.fixed_scratch, &ws)) return st;
         partial = static_cast<T *>(ws);
+    } else if (ttamd_status st = prepare_colsum<T>(ga, tiles_m * WGM, device, stream, sp.fixed_scratch)) {
+        return st;
     }
-    kernel<<<dim3(static_cast<unsigned>(blocks)), dim3(kThreads), lds_bytes, stream>>>(g, tiles_m, tiles_n, sp.ksplit,
+    kernel<<<dim3(static_cast<unsigned>(blocks)), dim3(kThreads), lds_bytes, stream>>>(ga, tiles_m, tiles_n, sp.ksplit,
                                                                                       sp.ksplit > 1 ? sp.k_chunk : g.K, partial);
     TTAMD_HIP_CHECK(hipGetLastError());
     if (sp.ksplit > 1) {
@@ -271,7 +348,7 @@ ttamd_status launch_variant(const GemmArgs &g, const SplitPlan &sp, int device, 
         splitk_reduce_kernel<T><<<dim3(static_cast<unsigned>((mn + 255) / 256), g.batch), dim3(256), 0, stream>>>(g, partial, sp.ksplit);
         TTAMD_HIP_CHECK(hipGetLastError());
     }
-    return TTAMD_OK;
+    return finish_colsum<T>(ga, stream);
 }
 
 // First k of the upper half of a two-half launch: half of K rounded up to a whole 16-byte vector, so that the upper
@@ -283,7 +360,7 @@ int dual_k_half(int K) {
 }
 
 template <typename T, int BM, int BN, int BK, int WGM, int WGN, bool A_KC, int A_VEC, bool B_KC, int B_VEC, int PF>
-ttamd_status launch_dual_variant(const GemmArgs &g, int device, hipStream_t stream) {
+ttamd_status launch_dual_variant(const GemmArgs &g, int device, hipStream_t stream, bool fixed_scratch) {
     using StA = Stager<T, BM, BK, A_KC, A_VEC, PF>;
     using StB = Stager<T, BN, BK, B_KC, B_VEC, PF>;
     constexpr size_t lds_bytes = 2 * TileEngine<T, BM, BN, BK, WGM, WGN, StA, StB>::kLdsBytes;
@@ -302,17 +379,19 @@ ttamd_status launch_dual_variant(const GemmArgs &g, int device, hipStream_t stre
     }
     const int tiles_m = (g.M + BM - 1) / BM, tiles_n = (g.N + BN - 1) / BN;
     const int64_t blocks = static_cast<int64_t>(tiles_m) * tiles_n * g.batch;
-    kernel<<<dim3(static_cast<unsigned>(blocks)), dim3(2 * kThreads), lds_bytes, stream>>>(g, tiles_m, tiles_n, k_half);
+    GemmArgs ga = g;
+    if (ttamd_status st = prepare_colsum<T>(ga, tiles_m * WGM, device, stream, fixed_scratch)) return st;
+    kernel<<<dim3(static_cast<unsigned>(blocks)), dim3(2 * kThreads), lds_bytes, stream>>>(ga, tiles_m, tiles_n, k_half);
     TTAMD_HIP_CHECK(hipGetLastError());
-    return TTAMD_OK;
+    return finish_colsum<T>(ga, stream);
 }
 
 template <typename T, int BM, int BN, int BK, int WGM, int WGN, int VEC, int PF>
-ttamd_status launch_dual_layouts(const GemmArgs &g, bool a_kc, bool b_kc, int device, hipStream_t stream) {
-    if (a_kc && b_kc) return launch_dual_variant<T, BM, BN, BK, WGM, WGN, true, VEC, true, VEC, PF>(g, device, stream);
-    if (a_kc && !b_kc) return launch_dual_variant<T, BM, BN, BK, WGM, WGN, true, VEC, false, VEC, PF>(g, device, stream);
-    if (!a_kc && b_kc) return launch_dual_variant<T, BM, BN, BK, WGM, WGN, false, VEC, true, VEC, PF>(g, device, stream);
-    return launch_dual_variant<T, BM, BN, BK, WGM, WGN, false, VEC, false, VEC, PF>(g, device, stream);
+ttamd_status launch_dual_layouts(const GemmArgs &g, bool a_kc, bool b_kc, int device, hipStream_t stream, bool fixed_scratch) {
+    if (a_kc && b_kc) return launch_dual_variant<T, BM, BN, BK, WGM, WGN, true, VEC, true, VEC, PF>(g, device, stream, fixed_scratch);
+    if (a_kc && !b_kc) return launch_dual_variant<T, BM, BN, BK, WGM, WGN, true, VEC, false, VEC, PF>(g, device, stream, fixed_scratch);
+    if (!a_kc && b_kc) return launch_dual_variant<T, BM, BN, BK, WGM, WGN, false, VEC, true, VEC, PF>(g, device, stream, fixed_scratch);
+    return launch_dual_variant<T, BM, BN, BK, WGM, WGN, false, VEC, false, VEC, PF>(g, device, stream, fixed_scratch);
 }
 
 template <typename T, int BM, int BN, int BK, int WGM, int WGN, int A_VEC, int B_VEC, int PF = 1>
@@ -331,7 +410,7 @@ SplitPlan plan_split(const GemmArgs &g, int bm, int bn, int bk) {
     sp.k_chunk = g.K;
     const int64_t tiles = static_cast<int64_t>((g.M + bm - 1) / bm) * ((g.N + bn - 1) / bn) * g.batch;
     const int k_tiles = (g.K + bk - 1) / bk;
-    if (tiles >= 128 || k_tiles < 4 || g.batch > 65535) return sp;
+    if (tiles >= 128 || k_tiles < 4 || g.batch > 65535 || g.colsum_out) return sp;  // (column sums come from whole tiles)
     int want = static_cast<int>((256 + tiles - 1) / tiles);
     const int max_by_k = k_tiles / 2;  // at least two k tiles per split
     if (want > max_by_k) want = max_by_k;
@@ -426,7 +505,7 @@ ttamd_status launch_mfma_typed(const GemmArgs &g, int device, hipStream_t stream
     if constexpr (sizeof(T) == 4)
         if (mid) return launch_layouts<T, TS::MBM, TS::MBN, TS::MBK, 2, 2, VK, VK>(g, ca.kc, cb.kc, sp, device, stream);
     if (large) return launch_layouts<T, TS::LBM, TS::LBN, TS::LBK, 2, 2, VK, VK>(g, ca.kc, cb.kc, sp, device, stream);
-    if (dual) return launch_dual_layouts<T, TS::SBM, TS::SBN, TS::SBK, 2, 2, VK, TS::SPF_DEEP>(g, ca.kc, cb.kc, device, stream);
+    if (dual) return launch_dual_layouts<T, TS::SBM, TS::SBN, TS::SBK, 2, 2, VK, TS::SPF_DEEP>(g, ca.kc, cb.kc, device, stream, fixed_scratch);
     if (ca.vec > 1 && cb.vec > 1) {
         // Register prefetch depth of the small tile: 4 k tiles in flight when a CU holds at most two workgroups and the
         // reduction is long (a lone workgroup otherwise waits for memory in every step), else 2, whose smaller register

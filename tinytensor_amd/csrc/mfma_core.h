@@ -189,6 +189,7 @@ struct Stager : TileLayout<T, ROWS, BK, KC> {
     uint32_t k_step_b;
     int tid;
     bool edge;
+    bool row_mask;  // some vector of this tile holds rows both inside and outside the matrix: loads must mask
 
     // line/column coordinates of pass p for this lane
     static __device__ __forceinline__ int line_of(int p, int tid) { return (p * kThreads + tid) / VPL; }
@@ -199,6 +200,9 @@ struct Stager : TileLayout<T, ROWS, BK, KC> {
     __device__ __forceinline__ void init(const T *base, int tid_, int rows_left, int64_t s_row, int64_t s_k, int K) {
         tid = tid_;
         edge = rows_left < ROWS;
+        // KC vectors run along k and element-wise loads fetch one row: a row outside the matrix costs only its offset
+        // (out of range, the load returns 0).  MC vectors hold VEC consecutive rows.
+        row_mask = !KC && VEC > 1 && edge && rows_left % VEC != 0;
         int64_t ext = (static_cast<int64_t>(rows_left - 1) * s_row + static_cast<int64_t>(K - 1) * s_k + 1) * sizeof(T);
         // With 16-byte loads the extent is rounded up to the vector size: the base is 16-byte aligned, so the
         // last vector stays inside the allocation's final 16-byte block and its tail is masked anyway.
@@ -477,18 +481,21 @@ struct TileEngine {
             step_group<MASK, I + 1>(sa, sb, smem, K, kt);
         }
     }
-    // the last steps (fewer than PF), same slot sequence
-    template <bool MASK, int I>
-    __device__ __forceinline__ void step_tail(StA &sa, StB &sb, T *smem, int K, int kt, int steps) {
-        if constexpr (I < StA::kPF - 1) {
+    // Up to PF steps from kt (kt % PF == 1) while kt + I < steps, same slot sequence as step_group; the step that
+    // requests tile `first_partial` (the one k tile that reaches past K) takes the masked body, the others the
+    // unmasked one.  first_partial < 0: every step masked.
+    template <int I>
+    __device__ __forceinline__ void step_group_tail(StA &sa, StB &sb, T *smem, int K, int kt, int steps, int first_partial) {
+        if constexpr (I < StA::kPF) {
             if (kt + I < steps) {
-                step_rot<(1 + I) % StA::kPF, true, MASK, true>(sa, sb, smem, K, kt + I);
-                step_tail<MASK, I + 1>(sa, sb, smem, K, kt, steps);
+                if (first_partial < 0 || kt + I + StA::kPF == first_partial) step_rot<(1 + I) % StA::kPF, true, true, true>(sa, sb, smem, K, kt + I);
+                else step_rot<(1 + I) % StA::kPF, true, false, true>(sa, sb, smem, K, kt + I);
+                step_group_tail<I + 1>(sa, sb, smem, K, kt, steps, first_partial);
             }
         }
     }
 
-    __device__ __forceinline__ void run_rot(StA &sa, StB &sb, T *smem, int K, bool unmasked) {
+    __device__ __forceinline__ void run_rot(StA &sa, StB &sb, T *smem, int K, bool rows_ok) {
         constexpr int PF = StA::kPF;
         constexpr int NC = BK / kChunk;
         const int KT = (K + BK - 1) / BK;
@@ -501,37 +508,50 @@ struct TileEngine {
         __syncthreads();
         // Tiles 0 .. KT-2; the first step has no pending chunk.  While kt + PF < KT a step also issues loads; the
         // remaining steps only drain the slots.
-        auto pipeline = [&]<bool MASK>() {
-            if constexpr (PF > 1) {
-                // Register slots are static inside a group of PF steps, so the compiler's wait counters know exactly
-                // which loads a store depends on (a run-time slot switch merges the counters at every branch and
-                // each store then waits for all loads in flight, the newest included).  Every step requests tile
-                // kt + PF; past the end of K those loads come back as zeros (or unused data) and are never parked.
-                const int steps = KT - 1;
-                if (steps <= 0) return;
-                step_rot<0, true, MASK, false>(sa, sb, smem, K, 0);
+        // `rows_ok` (workgroup-uniform): no load of this workgroup needs a row mask, so only a k tile that reaches
+        // past K needs masks.  That can only be the last tile, KT - 1, which is requested by step KT - 1 - PF: that
+        // one step takes the masked body, every other one the unmasked body (straight-line loads slotted between the
+        // MFMAs; requests past the end of K come back as zeros or unused data and are never parked).
+        const int first_partial = (K % BK == 0) ? (KT + 2 * PF) : (KT - 1);  // first tile whose load needs a k mask
+        if constexpr (PF > 1) {
+            // Register slots are static inside a group of PF steps, so the compiler's wait counters know exactly
+            // which loads a store depends on (a run-time slot switch merges the counters at every branch and
+            // each store then waits for all loads in flight, the newest included).  Every step requests tile
+            // kt + PF.
+            const int steps = KT - 1;
+            if (steps > 0) {
+                if (rows_ok && PF != first_partial) step_rot<0, true, false, false>(sa, sb, smem, K, 0);
+                else step_rot<0, true, true, false>(sa, sb, smem, K, 0);
                 int kt = 1;
-                for (; kt + PF <= steps; kt += PF) step_group<MASK, 0>(sa, sb, smem, K, kt);
-                step_tail<MASK, 0>(sa, sb, smem, K, kt, steps);
-                return;
+                if (rows_ok) {
+                    for (; kt + PF <= steps && kt + 2 * PF - 1 < first_partial; kt += PF) step_group<false, 0>(sa, sb, smem, K, kt);
+                    for (; kt + PF <= steps; kt += PF) step_group_tail<0>(sa, sb, smem, K, kt, steps, first_partial);
+                    step_group_tail<0>(sa, sb, smem, K, kt, steps, first_partial);
+                } else {
+                    for (; kt + PF <= steps; kt += PF) step_group<true, 0>(sa, sb, smem, K, kt);
+                    step_group_tail<0>(sa, sb, smem, K, kt, steps, -PF);  // (every step masked)
+                }
             }
-            int kt = 0, slot = 0;
-            auto advance = [&] {
-                ++kt;
-                slot = slot + 1 == PF ? 0 : slot + 1;
-            };
-            if (KT > 1) {
-                if (PF < KT) step_any_rot<true, MASK, false>(sa, sb, smem, K, kt, slot);
-                else step_any_rot<false, MASK, false>(sa, sb, smem, K, kt, slot);
-                advance();
-            }
-            for (; kt + PF < KT; advance()) step_any_rot<true, MASK, true>(sa, sb, smem, K, kt, slot);
-            for (; kt + 1 < KT; advance()) step_any_rot<false, MASK, true>(sa, sb, smem, K, kt, slot);
-        };
-        if (unmasked) {
-            pipeline.template operator()<false>();
         } else {
-            pipeline.template operator()<true>();
+            auto pipeline = [&]<bool MASK>() {
+                int kt = 0, slot = 0;
+                auto advance = [&] {
+                    ++kt;
+                    slot = slot + 1 == PF ? 0 : slot + 1;
+                };
+                if (KT > 1) {
+                    if (PF < KT) step_any_rot<true, MASK, false>(sa, sb, smem, K, kt, slot);
+                    else step_any_rot<false, MASK, false>(sa, sb, smem, K, kt, slot);
+                    advance();
+                }
+                for (; kt + PF < KT; advance()) step_any_rot<true, MASK, true>(sa, sb, smem, K, kt, slot);
+                for (; kt + 1 < KT; advance()) step_any_rot<false, MASK, true>(sa, sb, smem, K, kt, slot);
+            };
+            if (rows_ok && K % BK == 0) {
+                pipeline.template operator()<false>();
+            } else {
+                pipeline.template operator()<true>();
+            }
         }
         // Last tile: nothing left to request or park.
         if (KT > 0) {
@@ -644,12 +664,13 @@ struct TileEngine {
         }
     }
 
-    // K: reduction length.  `unmasked`: workgroup-uniform promise that every tile is full and interior.
-    __device__ __forceinline__ void run(StA &sa, StB &sb, T *smem, int K, bool unmasked) {
+    // K: reduction length.  `rows_ok`: workgroup-uniform promise that every row of both operand tiles is inside
+    // the matrix (a k tile that reaches past K is dealt with here).
+    __device__ __forceinline__ void run(StA &sa, StB &sb, T *smem, int K, bool rows_ok) {
         static_assert(StA::kPF == StB::kPF, "both operands use the same prefetch distance");
         static_assert(kPipe || kRotate, "no schedule for this tile shape");
-        if constexpr (kPipe) run_pipe(sa, sb, smem, K, unmasked);
-        else run_rot(sa, sb, smem, K, unmasked);
+        if constexpr (kPipe) run_pipe(sa, sb, smem, K, rows_ok && K % BK == 0);
+        else run_rot(sa, sb, smem, K, rows_ok);
     }
 
     // The accumulators of this lane as NBM * NBN * NACC values at lds[i * kThreads + tid]: lets two engines with the
@@ -683,9 +704,11 @@ struct TileEngine {
         }
     }
 
-    // Walks the finished tile.  `one(m, n, v)` receives a single element at tile-local (m, n);
-    // `two(m, n, v0, v1)` receives columns n and n + 1 of the same row (only called when B is MC/paired and
-    // `pairs_ok`); both are expected to do their own bounds checks against the matrix size.
+    // Walks the finished tile.  `one(m, n, v, bn)` receives a single element at tile-local (m, n);
+    // `two(m, n, v0, v1, bn)` receives columns n and n + 1 of the same row (only called when B is MC/paired and
+    // `pairs_ok`); both are expected to do their own bounds checks against the matrix size.  bn (a compile-time
+    // constant after unrolling) numbers the lane's columns: a lane meets NBN distinct columns, column slot bn for
+    // `one`, slots bn and bn + 1 for `two`.
     // FENCE keeps the scheduler from hoisting the work of later blocks over the stores of earlier ones (an epilogue
     // that loads per element would otherwise hold a whole tile's loads in flight and spill).
     template <bool FENCE = false, class One, class Two>
@@ -698,7 +721,7 @@ struct TileEngine {
 #pragma unroll
                 for (int bm = 0; bm < NBM; ++bm) {
 #pragma unroll
-                    for (int e = 0; e < M::NACC; ++e) one(FrA::index_of(wm0, bm, M::acc_row(e, lane)), n, acc[bm][bn][e]);
+                    for (int e = 0; e < M::NACC; ++e) one(FrA::index_of(wm0, bm, M::acc_row(e, lane)), n, acc[bm][bn][e], bn);
                     if constexpr (FENCE) __builtin_amdgcn_sched_barrier(0);
                 }
             }
@@ -712,7 +735,7 @@ struct TileEngine {
                     for (int bm = 0; bm < NBM; ++bm) {
 #pragma unroll
                         for (int e = 0; e < M::NACC; ++e)
-                            two(FrA::index_of(wm0, bm, M::acc_row(e, lane)), n, acc[bm][2 * pr][e], acc[bm][2 * pr + 1][e]);
+                            two(FrA::index_of(wm0, bm, M::acc_row(e, lane)), n, acc[bm][2 * pr][e], acc[bm][2 * pr + 1][e], 2 * pr);
                         if constexpr (FENCE) __builtin_amdgcn_sched_barrier(0);
                     }
                 }
@@ -725,6 +748,25 @@ struct TileEngine {
     }
 };
 
+// What the store of a tile can do beyond bias / ReLU / accumulate; every pointer may be null.  All three serve the
+// callers either side of a Linear layer's GEMMs in a training step:
+//   relu_out   dense like C: C keeps the value before the ReLU (what autograd saves as the ReLU's input,
+//              autograd/unary_ops.cpp:562-567) and relu_out receives max(value, 0) -- Linear + ReLU in one launch;
+//   zmask      dense like C: the value is replaced by 0 where zmask < 0 -- TensorRelu::backward's
+//              grad_output * where(input < 0, 0, 1) (autograd/unary_ops.cpp:568-573) applied by the GEMM that
+//              computes grad_output;
+//   colsum     [rows of partial sums][N]: row (colsum_row0 + the wave's row index in the workgroup) receives the sums
+//              over this wave's rows of what is stored to C, per column -- the bias gradient's sum over the batch
+//              (nn/linear.cpp:45-48: the bias is an expanded view, its gradient sums the broadcast dimension); a
+//              second kernel adds the partial rows in order.
+template <typename T>
+struct EpilogueExt {
+    T *relu_out = nullptr;
+    const T *zmask = nullptr;
+    T *colsum = nullptr;
+    int colsum_row0 = 0;
+};
+
 // Dense row-major store of a finished tile with the optional bias / ReLU / accumulate epilogue.
 // C points at the matrix (already offset to the batch), M x N its size, (m0, n0) the tile origin.
 //
@@ -732,50 +774,110 @@ struct TileEngine {
 // that the tile touches; an element outside the matrix gets the out-of-range offset and the hardware drops its
 // store.  One straight-line path serves interior and edge tiles and an element costs one 32-bit offset.  The host
 // only sends matrices here whose rows under one tile span less than 2^31 bytes (min(BM, M) * N * sizeof(T)).
-// LEAN: no bias, ReLU or accumulation (those arguments are then ignored).
-template <typename T, bool LEAN, class Engine>
+// LEAN: no bias, ReLU, accumulation or extensions (those arguments are then ignored).  EXT: the walk also serves
+// `ext` (a separate instantiation, because its extra loads, second store and column sums cost the big tiles registers
+// that the plain bias / ReLU / accumulate walk should not pay for).
+template <typename T, bool LEAN, bool EXT = false, class Engine>
 __device__ __forceinline__ void store_tile_dense(Engine &eng, T *__restrict__ C, int M_, int N_, int m0, int n0,
-                                                 const T *__restrict__ bias, int bias_mode, int relu, int accumulate) {
+                                                 const T *__restrict__ bias, int bias_mode, int relu, int accumulate,
+                                                 const EpilogueExt<T> &ext = EpilogueExt<T>{}) {
     using pair_t = typename Mfma<T>::pair_t;
+    using MI = Mfma<T>;
     constexpr uint32_t kOob = 0x80000000u;
     const int rows = M_ - m0 < Engine::kBM ? M_ - m0 : Engine::kBM;
     const int cols = N_ - n0;
-    const __amdgpu_buffer_rsrc_t out = make_rsrc(C + static_cast<int64_t>(m0) * N_ + n0,
-                                                 (static_cast<int64_t>(rows) * N_ - n0) * static_cast<int64_t>(sizeof(T)));
+    const int64_t tile_bytes = (static_cast<int64_t>(rows) * N_ - n0) * static_cast<int64_t>(sizeof(T));
+    const int64_t tile_first = static_cast<int64_t>(m0) * N_ + n0;
+    const __amdgpu_buffer_rsrc_t out = make_rsrc(C + tile_first, tile_bytes);
     // The epilogue options are uniform run-time flags.  Branching on them per element would put hundreds of branches
-    // into the unrolled walk, so they are folded into data instead: a bias that is absent and a C that is not
-    // accumulated into are read through descriptors of zero length, whose loads return 0 without touching memory.
+    // into the unrolled walk, so they are folded into data instead: a bias that is absent, a C that is not
+    // accumulated into and a mask that is not asked for are read through descriptors of zero length, whose loads
+    // return 0 without touching memory, and a second output that is not asked for is written through one, whose
+    // stores the hardware drops.
     constexpr int64_t kSz = sizeof(T);
     const __amdgpu_buffer_rsrc_t bias_n = make_rsrc(bias, bias_mode == 1 ? N_ * kSz : 0);
     const __amdgpu_buffer_rsrc_t bias_m = make_rsrc(bias, bias_mode == 2 ? M_ * kSz : 0);
-    const __amdgpu_buffer_rsrc_t prev = make_rsrc(C + static_cast<int64_t>(m0) * N_ + n0,
-                                                  accumulate ? (static_cast<int64_t>(rows) * N_ - n0) * kSz : 0);
+    const __amdgpu_buffer_rsrc_t prev = make_rsrc(C + tile_first, accumulate ? tile_bytes : 0);
+    static_assert(!(LEAN && EXT), "the lean walk has no extensions");
+    const __amdgpu_buffer_rsrc_t zmask = make_rsrc(ext.zmask ? ext.zmask + tile_first : ext.zmask, (EXT && ext.zmask) ? tile_bytes : 0);
+    const __amdgpu_buffer_rsrc_t second =
+        make_rsrc(ext.relu_out ? ext.relu_out + tile_first : ext.relu_out, (EXT && ext.relu_out) ? tile_bytes : 0);
     auto offset_of = [&](int ml, int nl) {
         return (ml < rows && nl < cols) ? static_cast<uint32_t>(ml * N_ + nl) * static_cast<uint32_t>(sizeof(T)) : kOob;
     };
-    auto finish = [&](T v, int ml, int nl, uint32_t off) {
+    T csum[Engine::NBN];  // sums of what this lane stores, per column slot
+#pragma unroll
+    for (int i = 0; i < Engine::NBN; ++i) csum[i] = T(0);
+    auto finish = [&](T v, int ml, int nl, uint32_t off, int slot, bool valid) {
         if constexpr (LEAN) return v;
         v += Vec<T, 1>::load(bias_n, static_cast<uint32_t>(n0 + nl) * static_cast<uint32_t>(sizeof(T)));
         v += Vec<T, 1>::load(bias_m, static_cast<uint32_t>(m0 + ml) * static_cast<uint32_t>(sizeof(T)));
+        if constexpr (EXT) v = Vec<T, 1>::load(zmask, off) < T(0) ? T(0) : v;  // absent mask: compares 0 < 0
         v = (v > T(0) || !relu) ? v : T(0);
         v += Vec<T, 1>::load(prev, off);
+        if constexpr (EXT) csum[slot] += valid ? v : T(0);
         return v;
     };
+    auto positive = [](T v) { return v > T(0) ? v : T(0); };
     // pairs: n is even and N is even, so n + 1 < N whenever n < N and a wave writes whole row segments
-    const bool pairs_ok = (N_ % 2 == 0) && (reinterpret_cast<uintptr_t>(C) % (2 * sizeof(T)) == 0);
+    const bool pairs_ok = (N_ % 2 == 0) && (reinterpret_cast<uintptr_t>(C) % (2 * sizeof(T)) == 0) &&
+                          (!EXT || (reinterpret_cast<uintptr_t>(ext.relu_out) % (2 * sizeof(T)) == 0 &&
+                                    reinterpret_cast<uintptr_t>(ext.zmask) % (2 * sizeof(T)) == 0));
     eng.template for_each<!LEAN>(
         pairs_ok,
-        [&](int ml, int nl, T v) {
+        [&](int ml, int nl, T v, int slot) {
             const uint32_t off = offset_of(ml, nl);
-            buffer_store(out, off, finish(v, ml, nl, off));
+            const T o = finish(v, ml, nl, off, slot, off != kOob);
+            buffer_store(out, off, o);
+            if constexpr (EXT) buffer_store(second, off, positive(o));
         },
-        [&](int ml, int nl, T v0, T v1) {
+        [&](int ml, int nl, T v0, T v1, int slot) {
             const uint32_t off = offset_of(ml, nl);
             pair_t o;
-            o[0] = finish(v0, ml, nl, off);
-            o[1] = finish(v1, ml, nl + 1, off + static_cast<uint32_t>(sizeof(T)));
+            if constexpr (EXT) {  // the same steps as finish(), the mask and the old value fetched as pairs
+                const pair_t zz = Vec<T, 2>::load(zmask, off), pp = Vec<T, 2>::load(prev, off);
+                const T bm = Vec<T, 1>::load(bias_m, static_cast<uint32_t>(m0 + ml) * static_cast<uint32_t>(sizeof(T)));
+                const T in[2] = {v0, v1};
+#pragma unroll
+                for (int j = 0; j < 2; ++j) {
+                    T v = in[j] + Vec<T, 1>::load(bias_n, static_cast<uint32_t>(n0 + nl + j) * static_cast<uint32_t>(sizeof(T))) + bm;
+                    v = zz[j] < T(0) ? T(0) : v;
+                    v = (v > T(0) || !relu) ? v : T(0);
+                    v += pp[j];
+                    csum[slot + j] += off != kOob ? v : T(0);
+                    o[j] = v;
+                }
+            } else {
+                o[0] = finish(v0, ml, nl, off, slot, off != kOob);
+                o[1] = finish(v1, ml, nl + 1, off + static_cast<uint32_t>(sizeof(T)), slot + 1, off != kOob);
+            }
             buffer_store(out, off, o);
+            if constexpr (EXT) {
+                pair_t r;
+                r[0] = positive(o[0]);
+                r[1] = positive(o[1]);
+                buffer_store(second, off, r);
+            }
         });
+    if constexpr (EXT) {
+        if (ext.colsum) {  // workgroup-uniform
+            // Lanes l, l + MB, ... of a wave hold the same columns and different rows: fold them, then lanes 0 .. MB-1
+            // write the wave's sums.  Column of slot s: the walk's own numbering (for_each).
+            const int jcol = eng.lane % MI::MB;
+            const bool paired = Engine::FrB::PAIRED && pairs_ok;
+            T *row = ext.colsum + static_cast<int64_t>(ext.colsum_row0 + eng.wm0 / Engine::WM) * N_;
+#pragma unroll
+            for (int s = 0; s < Engine::NBN; ++s) {
+                T v = csum[s];
+#pragma unroll
+                for (int d = MI::MB; d < 64; d *= 2) v += __shfl_xor(v, d, 64);
+                int nl;
+                if (paired) nl = Engine::FrB::index_of(eng.wn0, s & ~1, jcol) + (s & 1);
+                else nl = Engine::FrB::index_of(eng.wn0, s, jcol);
+                if (eng.lane < MI::MB && nl < cols) row[n0 + nl] = v;
+            }
+        }
+    }
 }
 
 }  // namespace mfma

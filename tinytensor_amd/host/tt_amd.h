@@ -775,9 +775,74 @@ public:
         sh.back() = weight.size(1);
         return out.reshape(Shape(sh));
     }
+    // forward followed by relu() in ONE launch -> {z, a}: z = input . weight + bias is what autograd saves as the
+    // ReLU's input (autograd/unary_ops.cpp:562-567), a = max(z, 0) what the next layer reads.
+    [[nodiscard]] auto forward_relu(const Tensor &input) const -> std::pair<Tensor, Tensor> {
+        const Tensor x2 = input.dim() == 2 ? input : input.flatten(0, -2);
+        if (x2.size(1) != weight.size(0)) throw TTException("Invalid shape for matrix multiplication");
+        if (x2.dtype() != weight.dtype() || x2.dtype() == kBool) throw TTException("Linear: operands must share one non-bool dtype");
+        auto sh = input.shape().to_vec();
+        sh.back() = weight.size(1);
+        const Tensor act = Tensor::empty(Shape(sh), x2.dtype(), input.device());
+        ttamd_epilogue ep{};
+        std::optional<Tensor> b = bias ? std::optional<Tensor>(bias->contiguous()) : std::nullopt;
+        ep.bias = b ? b->data_ptr() : nullptr;
+        ep.bias_mode = b ? 1 : 0;
+        ep.relu_out = act.data_ptr();
+        const Tensor out = get_backend(input.device())->batched_matmul(x2.unsqueeze(0), weight.unsqueeze(0), &ep);
+        return {out.reshape(Shape(sh)), act};
+    }
     Tensor weight;
     std::optional<Tensor> bias;
 };
+
+// Backward of y = x . W (+ b) for 2-D operands, as autograd emits it (TensorBatchedMatmul::backward on permute views,
+// autograd/binary_ops.cpp:173-179) with the element-wise steps that follow dx fused into its GEMM's store:
+//   dx = dy . W^T;  when x = relu(*relu_input): dx *= where(relu_input < 0, 0, 1) (autograd/unary_ops.cpp:568-573);
+//   when bias_grad: db_prev = dx.sum(0), the bias gradient of the Linear layer that produced relu_input;
+//   dW = x^T . dy.
+struct LinearGrads {
+    Tensor dx, dW;
+    std::optional<Tensor> db_prev;
+};
+inline auto linear_backward(const Tensor &grad_output, const Tensor &input, const Tensor &weight, const Tensor *relu_input = nullptr,
+                            bool bias_grad = false) -> LinearGrads {
+    const auto *be = get_backend(grad_output.device());
+    LinearGrads g;
+    ttamd_epilogue ep{};
+    std::optional<Tensor> z;
+    if (relu_input) {
+        if (!(relu_input->shape() == input.shape()) || relu_input->dtype() != input.dtype()) throw TTException("linear_backward: relu_input must match input");
+        z = relu_input->contiguous();
+        ep.relu_grad_input = z->data_ptr();
+    }
+    if (bias_grad) {
+        g.db_prev = Tensor::empty(Shape({input.size(1)}), input.dtype(), input.device());
+        ep.colsum_out = g.db_prev->data_ptr();
+    }
+    g.dx = be->batched_matmul(grad_output.unsqueeze(0), weight.unsqueeze(0).permute({0, 2, 1}), &ep).squeeze(0);
+    g.dW = be->batched_matmul(input.unsqueeze(0).permute({0, 2, 1}), grad_output.unsqueeze(0)).squeeze(0);
+    return g;
+}
+
+// nn::mse_loss(input, target) with mean reduction (nn/loss.cpp:69-72) and its backward in the same pass:
+// loss [1], grad_input (1 / numel) * 2 * (input - target), and (bias_grad, at most 64 columns) grad_input.sum(0).
+struct MseLoss {
+    Tensor loss, grad_input;
+    std::optional<Tensor> grad_colsum;
+};
+inline auto mse_loss(const Tensor &input, const Tensor &target, bool bias_grad = false) -> MseLoss {
+    if (!(input.shape() == target.shape()) || input.dtype() != target.dtype() || input.dim() != 2)
+        throw TTException("mse_loss: input and target must be 2-D tensors of one shape and dtype");
+    const Tensor y = input.contiguous(), t = target.contiguous();
+    MseLoss r;
+    r.loss = Tensor::empty(Shape({1}), y.dtype(), y.device());
+    r.grad_input = Tensor::empty(y.shape(), y.dtype(), y.device());
+    if (bias_grad) r.grad_colsum = Tensor::empty(Shape({y.size(1)}), y.dtype(), y.device());
+    check(ttamd_mse_loss(y.device().id, static_cast<ttamd_dtype>(y.dtype()), y.size(0), y.size(1), y.data_ptr(), t.data_ptr(), r.loss.data_ptr(),
+                         r.grad_input.data_ptr(), r.grad_colsum ? r.grad_colsum->data_ptr() : nullptr, nullptr));
+    return r;
+}
 }  // namespace nn
 
 }  // namespace tt_amd

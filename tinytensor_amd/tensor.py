@@ -450,21 +450,34 @@ class BackendAMD:
         return gx
 
     def batched_matmul(self, lhs: Tensor, rhs: Tensor, bias: Tensor | None = None, bias_mode: int = 0,
-                       relu: bool = False, out: Tensor | None = None, accumulate: bool = False) -> Tensor:
+                       relu: bool = False, out: Tensor | None = None, accumulate: bool = False,
+                       relu_out: Tensor | None = None, relu_grad_input: Tensor | None = None,
+                       colsum_out: Tensor | None = None) -> Tensor:
         """BackendBase::batched_matmul (backend_base.h:130).  The keyword arguments select the fused
-        epilogue of ttamd_batched_matmul; with the defaults this is the reference call exactly."""
+        epilogue of ttamd_batched_matmul; with the defaults this is the reference call exactly.
+        relu_out: dense [B,N,M] tensor that receives max(out, 0) while `out` keeps the value before the ReLU;
+        relu_grad_input: dense [B,N,M] saved input z of a ReLU, out = result * (z < 0 ? 0 : 1);
+        colsum_out: dense [B,M] tensor that receives out summed over its rows."""
         assert lhs.dim() == 3 and rhs.dim() == 3 and lhs.size(2) == rhs.size(1)
         B, N, K = lhs.shape
         M = rhs.size(2)
         if out is None:
             out = Tensor.empty((B, N, M), lhs.dtype, lhs.device)
         ep = None
-        if bias is not None or relu or accumulate:
+        if bias is not None or relu or accumulate or relu_out is not None or relu_grad_input is not None or colsum_out is not None:
             ep = _capi.Epilogue()
             ep.bias = (bias.storage.ptr + bias.offset * bias.itemsize) if bias is not None else None
             ep.bias_mode = bias_mode if bias is not None else 0
             ep.relu = int(relu)
             ep.accumulate = int(accumulate)
+            for name, t in (("relu_out", relu_out), ("relu_grad_input", relu_grad_input), ("colsum_out", colsum_out)):
+                if t is None:
+                    continue
+                want = (B, M) if name == "colsum_out" else (B, N, M)
+                dense = all(n == 1 or st == d for n, st, d in zip(t.shape, t.stride, _dense_strides(t.shape)))
+                if not dense or t.numel() != int(np.prod(want)) or t.dtype != lhs.dtype:
+                    raise TTException(f"batched_matmul: {name} must be a dense tensor of {want} elements of the operands' dtype")
+                setattr(ep, name, t.storage.ptr + t.offset * t.itemsize)
         lv, rv = lhs.view3(), rhs.view3()
         _check(lib.ttamd_batched_matmul(lhs.device.id, lhs.dtype, B, N, K, M, C.byref(lv), C.byref(rv),
                                         C.c_void_p(out.storage.ptr), C.byref(ep) if ep is not None else None, _stream_arg()))
@@ -758,6 +771,56 @@ def linear(input: Tensor, weight: Tensor, bias: Tensor | None = None, relu: bool
     out = get_backend(input.device).batched_matmul(x2.unsqueeze(0), weight.unsqueeze(0), bias=bias, bias_mode=1,
                                                    relu=relu)
     return out.reshape(list(input.shape[:-1]) + [weight.size(1)])
+
+
+def linear_relu(input: Tensor, weight: Tensor, bias: Tensor | None = None):
+    """nn::Linear::forward followed by relu() in one launch -> (z, a): z = input . weight + bias is what autograd saves
+    as the ReLU's input (autograd/unary_ops.cpp:562-567), a = max(z, 0) what the next layer reads."""
+    x2 = input.flatten(0, -2) if input.dim() != 2 else input
+    if x2.size(1) != weight.size(0):
+        raise TTException(f"Invalid shape for matrix multiplication. LHS={x2.shape} and RHS={weight.shape}")
+    x2, weight = _promote(x2, weight)
+    if bias is not None:
+        bias = bias.to(x2.dtype)
+    a = Tensor.empty((1, x2.size(0), weight.size(1)), x2.dtype, x2.device)
+    z = get_backend(input.device).batched_matmul(x2.unsqueeze(0), weight.unsqueeze(0), bias=bias, bias_mode=1, relu_out=a)
+    shape = list(input.shape[:-1]) + [weight.size(1)]
+    return z.reshape(shape), a.reshape(shape)
+
+
+def linear_backward(grad_output: Tensor, input: Tensor, weight: Tensor, relu_input: Tensor | None = None,
+                    bias_grad: bool = True):
+    """Backward of y = x . W (+ b) for 2-D operands dy = grad_output [n, out], x = input [n, in], W = weight [in, out],
+    as autograd emits it (TensorBatchedMatmul::backward on permute views, autograd/binary_ops.cpp:173-179) with the
+    element-wise steps that follow dx fused into its GEMM:
+        dx = dy . W^T;
+        when x = relu(relu_input): dx *= where(relu_input < 0, 0, 1)   (TensorRelu::backward, unary_ops.cpp:568-573);
+        when bias_grad: db_prev = dx.sum(0), the bias gradient of the Linear layer that produced relu_input;
+        dW = x^T . dy.
+    Returns (dx, dW, db_prev | None)."""
+    be = get_backend(grad_output.device)
+    n, fin = input.shape
+    db = Tensor.empty((1, fin), grad_output.dtype, grad_output.device) if bias_grad else None
+    dx = be.batched_matmul(grad_output.unsqueeze(0), weight.unsqueeze(0).permute(0, 2, 1),
+                           relu_grad_input=relu_input.unsqueeze(0) if relu_input is not None else None, colsum_out=db)
+    dW = be.batched_matmul(input.unsqueeze(0).permute(0, 2, 1), grad_output.unsqueeze(0))
+    return dx.squeeze(0), dW.squeeze(0), (db.reshape([fin]) if db is not None else None)
+
+
+def mse_loss(input: Tensor, target: Tensor, grad: bool = True, bias_grad: bool = False):
+    """nn::mse_loss(input, target) with mean reduction (nn/loss.cpp:69-72) and, when `grad`, its backward in the same
+    pass -> (loss [1], grad_input | None, grad_input.sum(0) | None).  2-D dense operands of one float dtype."""
+    if input.shape != target.shape or input.dtype != target.dtype or input.dim() != 2:
+        raise TTException("mse_loss: input and target must be 2-D tensors of one shape and dtype")
+    input, target = input.contiguous(), target.contiguous()
+    rows, cols = input.shape
+    loss = Tensor.empty((1,), input.dtype, input.device)
+    g = Tensor.empty(input.shape, input.dtype, input.device) if grad else None
+    cs = Tensor.empty((cols,), input.dtype, input.device) if (grad and bias_grad) else None
+    ptr = lambda t: C.c_void_p(t.storage.ptr + t.offset * t.itemsize) if t is not None else None
+    _check(lib.ttamd_mse_loss(input.device.id, input.dtype, rows, cols, ptr(input), ptr(target), ptr(loss), ptr(g), ptr(cs),
+                              _stream_arg()))
+    return loss, g, cs
 
 
 def conv2d(input: Tensor, weight: Tensor, bias: Tensor | None = None, stride: int = 1, padding: int = 0) -> Tensor:
