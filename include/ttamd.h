@@ -275,6 +275,12 @@ ttamd_status ttamd_random_fill(int device, ttamd_dtype dtype, int dist, double p
 ttamd_status ttamd_random_fill_view(int device, ttamd_dtype dtype, int dist, double p0, double p1, uint64_t *master_state,
                                     int ndim, const int64_t *shape, const int64_t *stride, void *data, int64_t offset,
                                     void *stream);
+/* The same with the per-element generator states supplied by the caller (host array, one per element of the view in
+ * its row-major order): what an adapter inside the reference passes, whose Generator (include/tt/random.h:17-42)
+ * hands out states only through operator() -- create_gen_states, cpu/distribution.cpp:31-38, draws them exactly so. */
+ttamd_status ttamd_random_fill_states(int device, ttamd_dtype dtype, int dist, double p0, double p1, const uint64_t *states,
+                                      int ndim, const int64_t *shape, const int64_t *stride, void *data, int64_t offset,
+                                      void *stream);
 
 /* ---- timing (no reference counterpart: the reference has no timers; used by the benchmark
  * to bracket kernels with HIP events on the stream they run on) ------------------------ */

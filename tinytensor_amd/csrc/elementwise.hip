@@ -5,6 +5,7 @@
 // grad_output) and moves raw bytes, so one kernel per element size serves every dtype.
 #include "common.h"
 
+#include <cstdlib>
 #include <cstring>
 #include <type_traits>
 
@@ -1166,15 +1167,16 @@ ttamd_status ttamd_full(int device, ttamd_dtype dtype, const void *value, int64_
 }
 
 
-// dist: 0 = uniform_real(low = p0, high = p1), 1 = normal(mu = p0, std = p1).  *master_state is the host-side master
-// generator state (Generator::state); it advances by one output per element of the view.
-ttamd_status ttamd_random_fill_view(int device, ttamd_dtype dtype, int dist, double p0, double p1, uint64_t *master_state, int ndim,
-                                    const int64_t *shape, const int64_t *stride, void *data, int64_t offset, void *stream) {
+// dist: 0 = uniform_real(low = p0, high = p1), 1 = normal(mu = p0, std = p1).  `states`: one generator state per element
+// of the view, in the view's row-major order, produced on the host (cpu/distribution.cpp:31-38 draws them from the
+// caller's Generator one by one; the reference's GPU backend uploads them the same way, cuda/distribution.cu:32-99).
+ttamd_status ttamd_random_fill_states(int device, ttamd_dtype dtype, int dist, double p0, double p1, const uint64_t *states, int ndim,
+                                      const int64_t *shape, const int64_t *stride, void *data, int64_t offset, void *stream) {
     if (dtype != TTAMD_F32 && dtype != TTAMD_F64) {
         set_error("random_fill: floating point dtypes only");
         return TTAMD_ERR_UNSUPPORTED_DTYPE;
     }
-    if (!master_state || offset < 0 || (dist != 0 && dist != 1) || (dist == 0 && !(p0 < p1))) {
+    if (offset < 0 || (dist != 0 && dist != 1) || (dist == 0 && !(p0 < p1))) {
         set_error("random_fill: invalid arguments (Expected low < high for uniform_real)");
         return TTAMD_ERR_INVALID_ARGUMENT;
     }
@@ -1183,26 +1185,21 @@ ttamd_status ttamd_random_fill_view(int device, ttamd_dtype dtype, int dist, dou
     if (ttamd_status s = make_view("random_fill", ndim, shape, stride, &v, &numel)) return s;
     if (ttamd_status s = use_device(device)) return s;
     if (numel == 0) return TTAMD_OK;
-    if (!data) {
-        set_error("random_fill: data is NULL");
+    if (!data || !states) {
+        set_error("random_fill: NULL data or states pointer");
         return TTAMD_ERR_INVALID_ARGUMENT;
     }
     const bool dense = is_dense(v);
     void *out = static_cast<char *>(data) + offset * static_cast<int64_t>(dtype_size(dtype));
     hipStream_t st = static_cast<hipStream_t>(stream);
-    // per-element generator states, produced on the host in order (cpu/distribution.cpp:31-38)
+    const size_t state_bytes = static_cast<size_t>(numel) * sizeof(uint64_t);
+    // staging: pinned host copy (the caller's array may be pageable and may go away when this call returns) and a
+    // device copy; both are released once the stream has consumed them
     uint64_t *host_states = nullptr;
-    TTAMD_HIP_CHECK(hipHostMalloc(reinterpret_cast<void **>(&host_states), static_cast<size_t>(numel) * sizeof(uint64_t), hipHostMallocDefault));
-    uint64_t x = *master_state;
-    for (int64_t i = 0; i < numel; ++i) {
-        x ^= x << 13;
-        x ^= x >> 7;
-        x ^= x << 17;
-        host_states[i] = x;
-    }
-    *master_state = x;
+    TTAMD_HIP_CHECK(hipHostMalloc(reinterpret_cast<void **>(&host_states), state_bytes, hipHostMallocDefault));
+    memcpy(host_states, states, state_bytes);
     void *dev_states = nullptr;
-    hipError_t e = hipMalloc(&dev_states, static_cast<size_t>(numel) * sizeof(uint64_t));
+    hipError_t e = hipMalloc(&dev_states, state_bytes);
     if (e != hipSuccess) {
         (void)hipGetLastError();
         (void)hipHostFree(host_states);
@@ -1214,8 +1211,7 @@ ttamd_status ttamd_random_fill_view(int device, ttamd_dtype dtype, int dist, dou
         set_error("%s failed: %s", what, hipGetErrorString(err));
         rc = TTAMD_ERR_LAUNCH;
     };
-    if ((e = hipMemcpyAsync(dev_states, host_states, static_cast<size_t>(numel) * sizeof(uint64_t), hipMemcpyHostToDevice, st)) != hipSuccess)
-        fail(e, "hipMemcpyAsync");
+    if ((e = hipMemcpyAsync(dev_states, host_states, state_bytes, hipMemcpyHostToDevice, st)) != hipSuccess) fail(e, "hipMemcpyAsync");
     if (rc == TTAMD_OK) {
         const unsigned blocks = static_cast<unsigned>((numel + 255) / 256);
         const uint64_t *sp = static_cast<const uint64_t *>(dev_states);
@@ -1228,10 +1224,38 @@ ttamd_status ttamd_random_fill_view(int device, ttamd_dtype dtype, int dist, dou
         }
         if ((e = hipGetLastError()) != hipSuccess) fail(e, "kernel launch");
     }
-    // the staging buffers are released after the stream has consumed them
     if ((e = hipStreamSynchronize(st)) != hipSuccess && rc == TTAMD_OK) fail(e, "hipStreamSynchronize");
     (void)hipFree(dev_states);
     (void)hipHostFree(host_states);
+    return rc;
+}
+
+// The same with the states drawn here: *master_state is the caller's master generator state (Generator::state, xorshift64
+// with shifts 13, 7, 17: tensor/random.cpp:36-43); it advances by one output per element of the view.
+ttamd_status ttamd_random_fill_view(int device, ttamd_dtype dtype, int dist, double p0, double p1, uint64_t *master_state, int ndim,
+                                    const int64_t *shape, const int64_t *stride, void *data, int64_t offset, void *stream) {
+    if (!master_state) {
+        set_error("random_fill: master_state is NULL");
+        return TTAMD_ERR_INVALID_ARGUMENT;
+    }
+    ViewDesc v;
+    int64_t numel = 0;
+    if (ttamd_status s = make_view("random_fill", ndim, shape, stride, &v, &numel)) return s;
+    uint64_t *states = static_cast<uint64_t *>(malloc(static_cast<size_t>(numel > 0 ? numel : 1) * sizeof(uint64_t)));
+    if (!states) {
+        set_error("random_fill: unable to allocate %lld generator states on the host", static_cast<long long>(numel));
+        return TTAMD_ERR_OUT_OF_MEMORY;
+    }
+    uint64_t x = *master_state;
+    for (int64_t i = 0; i < numel; ++i) {
+        x ^= x << 13;
+        x ^= x >> 7;
+        x ^= x << 17;
+        states[i] = x;
+    }
+    const ttamd_status rc = ttamd_random_fill_states(device, dtype, dist, p0, p1, states, ndim, shape, stride, data, offset, stream);
+    free(states);
+    if (rc == TTAMD_OK) *master_state = x;
     return rc;
 }
 
