@@ -102,6 +102,28 @@ ttamd_status launch_gemm_mfma(ttamd_dtype dt, const GemmArgs &g, int device, hip
 ttamd_status launch_gemm_simt(ttamd_dtype dt, const GemmArgs &g, hipStream_t stream, const char **variant,
                               bool variant_only);
 
+// Stride-1 fp32 convolution served by conv_patch.hip (weights resident in LDS, input rows staged once per tile).
+// The caller fills the first block; launch_conv_patch_f32 derives the rest and reports through *handled whether the
+// geometry fits (otherwise nothing was launched and the caller takes its general kernels).
+struct ConvPatchArgs {
+    const float *x;        // input [B,C,H,W]: column stride 1, the other strides below (elements)
+    const float *w;        // weight: tap t of (row, reduction channel) at element row * w_row + red * w_red + t
+    const float *bias;     // [O] or null
+    float *out;            // dense [B,O,Ho,Wo]
+    int B, C, H, W, O, k, P, Ho, Wo;  // C: reduction channels (the input's), O: rows of the result
+    int64_t xs_b;
+    int32_t xs_c, xs_h;
+    int64_t w_row, w_red;
+    int w_flip;            // taps used in reverse order (gradient with respect to the input)
+    int w_rows_fast;       // lanes of the weight loader run along the rows (the axis whose stride is k*k) instead of the channels
+    int64_t image_bytes, weight_bytes;  // bytes reachable from an image's / the weight's first element
+    // derived
+    int K, lda, cpad, R, pitch, vecs_per_row, xh, last_vecs, n_items, stage_slots, cl_shift, tiles_m, tiles_n;
+    int n_seg, seg_len, segs_per_pass, n_fast, n_wvec, w_dense, w_pass_vecs;
+    FastDiv d_wfast, d_segv, d_k, d_ngrp, d_xh, d_R, d_cpad4, d_2P, d_P, d_Wo, d_tiles_n;
+};
+ttamd_status launch_conv_patch_f32(ConvPatchArgs a, hipStream_t stream, bool *handled);
+
 }  // namespace ttamd
 
 #endif  // TTAMD_CSRC_COMMON_H_

@@ -19,6 +19,7 @@
 // output positions) accumulates in registers, partial tiles go to the caller's workspace and are summed in a
 // fixed order.  Integer dtypes (forward only; autograd never differentiates them) use a direct
 // vector-ALU kernel with wrap-around arithmetic.
+#include <cstdlib>
 #include <type_traits>
 
 #include "mfma_core.h"
@@ -1027,6 +1028,15 @@ ttamd_status set_lds(Kernel kernel, size_t lds_bytes) {
     return TTAMD_OK;
 }
 
+// TTAMD_CONV_PATCH=0 keeps every convolution on the implicit-GEMM kernels of this file (for comparisons).
+inline bool patch_kernel_enabled() {
+    static const bool on = [] {
+        const char *e = std::getenv("TTAMD_CONV_PATCH");
+        return !(e && e[0] == '0');
+    }();
+    return on;
+}
+
 template <typename T>
 struct ConvTiles {
     static constexpr int BK = sizeof(T) == 4 ? 32 : 16;
@@ -1101,6 +1111,25 @@ ttamd_status forward_mfma_tile(const ConvPlan &pl, const void *bias, void *out, 
 
 template <typename T>
 ttamd_status forward_mfma(const ConvPlan &pl, const void *bias, void *out, hipStream_t st) {
+    if constexpr (std::is_same_v<T, float>) {
+        // unit stride, dense rows and a weight block that fits in LDS: the persistent kernel of conv_patch.hip
+        const ConvGeom &g = pl.geo;
+        if (g.S == 1 && g.xs_w == 1 && patch_kernel_enabled()) {
+            ConvPatchArgs a{};
+            a.x = static_cast<const float *>(pl.x);
+            a.w = static_cast<const float *>(pl.w);
+            a.bias = static_cast<const float *>(bias);
+            a.out = static_cast<float *>(out);
+            a.B = g.B; a.C = g.C; a.H = g.H; a.W = g.W; a.O = g.O; a.k = g.k; a.P = g.P; a.Ho = g.Ho; a.Wo = g.Wo;
+            a.xs_b = g.xs_b; a.xs_c = g.xs_c; a.xs_h = g.xs_h;
+            a.w_row = g.w_so; a.w_red = static_cast<int64_t>(g.k) * g.k;  // lanes along the input channels
+            a.image_bytes = pl.image_bytes;
+            a.weight_bytes = pl.weight_bytes;
+            bool handled = false;
+            if (ttamd_status s = launch_conv_patch_f32(a, st, &handled)) return s;
+            if (handled) return TTAMD_OK;
+        }
+    }
     if (pl.geo.O <= 32) return forward_mfma_tile<T, 32, 128>(pl, bias, out, st);
     return forward_mfma_tile<T, 64, 64>(pl, bias, out, st);
 }
