@@ -91,6 +91,77 @@ def test_backward_exact_on_integer_data_and_adjoints(tt, oracle, dtype):
     assert lhs == np.sum(gx.to_numpy().astype(np.float64) * x) == np.sum(gw.to_numpy().astype(np.float64) * w)
 
 
+def _last_kernel(which):
+    from tinytensor_amd import _capi
+    return _capi.lib.ttamd_conv2d_last_kernel(which)
+
+
+@pytest.mark.parametrize("geom", [
+    # fp32, unit stride: the persistent kernel that keeps the weight block in LDS, forward (input channels 8n, rows
+    # of whole 16-byte vectors) and grad_input (output channels 8n, output rows of whole vectors).
+    # B, C, O, H, W, k, P, forward on it, grad_input on it
+    (3, 32, 64, 28, 28, 3, 1, True, True),     # benchmark geometry: 8 waves forward, one patch buffer for grad_input
+    (2, 8, 8, 8, 8, 3, 1, True, True),         # 8 channels per staging item, an image smaller than a tile (idle waves)
+    (2, 24, 40, 12, 12, 3, 1, True, False),    # channel counts 8 (2n + 1); result rows beyond the last channel; grad_input's patch
+                                                # of 14 rows x 40 channels is more than a lane's 16 loads
+    (2, 24, 40, 12, 32, 3, 1, True, True),     # the same with rows of 8 vectors
+    (5, 16, 32, 20, 20, 5, 2, True, True),     # 5 x 5 taps, at most 32 result rows
+    (2, 16, 16, 9, 16, 1, 0, True, True),      # 1 x 1
+    (2, 8, 16, 10, 12, 2, 1, True, False),     # even kernel; Wo = 13: grad_input on the implicit-GEMM kernel
+    (2, 32, 96, 14, 36, 3, 0, True, False),    # no padding, a second half-empty row block, 9 vectors per row; Wo = 34
+    (70, 32, 64, 6, 4, 3, 1, True, False),     # many small images, one vector per row (grad_input: a tile's rows of 64
+                                                # channels are more than a lane's 16 loads)
+    (2, 64, 32, 28, 28, 3, 1, True, True),     # 64 channels in: 16 loads per lane and tile, one patch buffer
+    (2, 16, 24, 8, 8, 3, 2, True, False),      # padding 2 with k = 3; Wo = 10
+    (2, 48, 64, 8, 8, 3, 1, True, False),      # a weight block that passes through LDS in several passes of row-wise loads
+    (1, 128, 16, 8, 8, 3, 1, False, True),     # forward: the weight block does not fit; grad_input (16 channels in): it does
+    (3, 32, 64, 7, 28, 3, 1, True, True),      # tiles that start and end inside rows, images of 196 positions
+])
+def test_lds_resident_kernel_exact(tt, oracle, geom):
+    Bn, Cc, O, H, W, k, P, fwd_on, dgrad_on = geom
+    rng = np.random.default_rng(sum(geom[:7]))
+    x = rng.integers(-3, 4, (Bn, Cc, H, W)).astype(np.float32)
+    w = rng.integers(-3, 4, (O, Cc, k, k)).astype(np.float32)
+    b = rng.integers(-3, 4, (O,)).astype(np.float32)
+    out = tt.conv2d(dev(tt, x), dev(tt, w), dev(tt, b), 1, P).to_numpy()
+    assert (_last_kernel(0) & 0xF00 == 0x200) == fwd_on, hex(_last_kernel(0))
+    want = oracle.conv2d_forward(x, w, b, 1, P)
+    assert np.array_equal(out, want)
+    assert np.array_equal(want - b[None, :, None, None], oracle.conv2d_naive(x, w, 1, P))
+    g = rng.integers(-3, 4, want.shape).astype(np.float32)
+    gx, gw, gb = tt.conv2d_backward(dev(tt, g), dev(tt, x), dev(tt, w), dev(tt, b), 1, P)
+    assert (_last_kernel(1) & 0xF00 == 0x200) == dgrad_on, hex(_last_kernel(1))
+    wx, ww, wb = oracle.conv2d_backward(g, x, w, True, 1, P)
+    assert np.array_equal(gx.to_numpy(), wx) and np.array_equal(gw.to_numpy(), ww) and np.array_equal(gb.to_numpy(), wb)
+
+
+def test_lds_resident_kernel_on_views(tt, oracle):
+    # an input window of a larger tensor (row stride 16, 16-byte aligned start) and, through the C ABI, a weight whose
+    # output-channel stride is larger than C k k (the row-wise weight loads)
+    from tinytensor_amd import _capi
+    import ctypes as C
+    rng = np.random.default_rng(77)
+    big = rng.integers(-3, 4, (2, 16, 12, 16)).astype(np.float32)
+    wbig = rng.integers(-3, 4, (24, 20, 3, 3)).astype(np.float32)
+    x, w = np.ascontiguousarray(big[:, :, 2:10, 4:12]), np.ascontiguousarray(wbig[:, :16])
+    tb = dev(tt, big)
+    tx = tt.Tensor(tb.storage, tb.dtype, (2, 16, 8, 8), (16 * 12 * 16, 12 * 16, 16, 1), 2 * 16 + 4)
+    assert not tx.is_contiguous()
+    got = tt.conv2d(tx, dev(tt, w), None, 1, 1).to_numpy()
+    assert _last_kernel(0) & 0xF00 == 0x200
+    want = oracle.conv2d_forward(x, w, None, 1, 1)
+    assert np.array_equal(got, want)
+    twb = dev(tt, wbig)
+    tw = tt.Tensor(twb.storage, twb.dtype, (24, 16, 3, 3), (20 * 9, 9, 3, 1), 0)
+    out = tt.Tensor.empty(want.shape, _capi.F32, tx.device)
+    iv, wv = tx.view4(), tw.view4()
+    rc = _capi.lib.ttamd_conv2d_forward(0, _capi.F32, C.byref(iv), C.byref(wv), None, C.c_void_p(out.storage.ptr),
+                                        2, 16, 8, 8, 24, 3, 1, 1, None)
+    assert rc == 0, _capi.last_error()
+    assert _last_kernel(0) & 0xF00 == 0x200
+    assert np.array_equal(out.to_numpy(), want)
+
+
 @pytest.mark.parametrize("dtype", [np.float32, np.float64])
 @pytest.mark.parametrize("geom", [
     # unit stride with rows that are a whole number of 16-byte vectors: the vector-gather kernels.

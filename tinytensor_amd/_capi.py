@@ -71,6 +71,7 @@ def _bind(lib: C.CDLL) -> None:
         "ttamd_batched_matmul_variant": (C.c_char_p, [i, i, i, i, i, C.POINTER(View3), C.POINTER(View3)]),
         "ttamd_conv2d_forward": (i, [i, i, C.POINTER(View4), C.POINTER(View4), vp, vp] + [i] * 8 + [vp]),
         "ttamd_conv2d_backward_workspace": (i, [i] + [i] * 8 + [C.POINTER(sz)]),
+        "ttamd_conv2d_last_kernel": (i, [i]),
         "ttamd_conv2d_backward": (i, [i, i, vp, C.POINTER(View4), C.POINTER(View4), vp, vp, vp] + [i] * 8 + [vp, sz, vp]),
         "ttamd_pool2d_forward": (i, [i, i, i, C.POINTER(View4), vp] + [i] * 7 + [vp]),
         "ttamd_pool2d_backward": (i, [i, i, i, vp, C.POINTER(View4), vp, vp] + [i] * 7 + [vp]),

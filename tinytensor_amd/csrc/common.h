@@ -119,10 +119,10 @@ struct ConvPatchArgs {
     int64_t image_bytes, weight_bytes;  // bytes reachable from an image's / the weight's first element
     // derived
     int K, lda, cpad, R, pitch, vecs_per_row, xh, last_vecs, n_items, stage_slots, cl_shift, tiles_m, tiles_n;
-    int n_seg, seg_len, segs_per_pass, n_fast, n_wvec, w_dense, w_pass_vecs;
+    int n_seg, seg_len, segs_per_pass, n_fast, n_wvec, w_dense, w_pass_vecs, n_buf;
     FastDiv d_wfast, d_segv, d_k, d_ngrp, d_xh, d_R, d_cpad4, d_2P, d_P, d_Wo, d_tiles_n;
 };
-ttamd_status launch_conv_patch_f32(ConvPatchArgs a, hipStream_t stream, bool *handled);
+ttamd_status launch_conv_patch_f32(ConvPatchArgs a, hipStream_t stream, int *variant);
 
 }  // namespace ttamd
 

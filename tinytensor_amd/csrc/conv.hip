@@ -1028,6 +1028,11 @@ ttamd_status set_lds(Kernel kernel, size_t lds_bytes) {
     return TTAMD_OK;
 }
 
+// Which kernel family the calling thread's last forward ([0]) and grad_input ([1]) launches took: 0x100 the
+// implicit-GEMM kernels of this file, 0x200 + 16 * waves + patch buffers the persistent kernel of conv_patch.hip,
+// 0 anything else.  Read through ttamd_conv2d_last_kernel by the tests that mean to cover a particular kernel.
+thread_local int t_last_kernel[2] = {0, 0};
+
 // TTAMD_CONV_PATCH=0 keeps every convolution on the implicit-GEMM kernels of this file (for comparisons).
 inline bool patch_kernel_enabled() {
     static const bool on = [] {
@@ -1125,11 +1130,15 @@ ttamd_status forward_mfma(const ConvPlan &pl, const void *bias, void *out, hipSt
             a.w_row = g.w_so; a.w_red = static_cast<int64_t>(g.k) * g.k;  // lanes along the input channels
             a.image_bytes = pl.image_bytes;
             a.weight_bytes = pl.weight_bytes;
-            bool handled = false;
-            if (ttamd_status s = launch_conv_patch_f32(a, st, &handled)) return s;
-            if (handled) return TTAMD_OK;
+            int variant = 0;
+            if (ttamd_status s = launch_conv_patch_f32(a, st, &variant)) return s;
+            if (variant) {
+                t_last_kernel[0] = 0x200 + variant;
+                return TTAMD_OK;
+            }
         }
     }
+    t_last_kernel[0] = 0x100;
     if (pl.geo.O <= 32) return forward_mfma_tile<T, 32, 128>(pl, bias, out, st);
     return forward_mfma_tile<T, 64, 64>(pl, bias, out, st);
 }
@@ -1343,6 +1352,7 @@ ttamd_status backward_mfma(const ConvPlan &pl, const void *gout, void *gin, void
     T *const wt = static_cast<T *>(ws);
     T *const partials = reinterpret_cast<T *>(static_cast<char *>(ws) + plan.wt_bytes);
     // grad_input
+    t_last_kernel[1] = 0;
     const int np = (g.k + g.S - 1) / g.S;
     const size_t slots_lds = static_cast<size_t>(g.O) * g.k * g.k * g.C * sizeof(T);
     if (g.C <= kDirectDgradChannels && np <= 4 && slots_lds <= 64 * 1024) {
@@ -1401,6 +1411,7 @@ ttamd_status backward_mfma(const ConvPlan &pl, const void *gout, void *gin, void
           };
           return gg.C <= 32 ? run.template operator()<32, 128>() : run.template operator()<64, 64>();
         };
+        t_last_kernel[1] = 0x100;
         const DgradClassPlan dc = plan_dgrad_classes(sizeof(T), g.B, g.C, g.H, g.W, g.O, g.k, g.S, g.P);
         if (dc.use) {
             T *const tmp = reinterpret_cast<T *>(static_cast<char *>(ws) + plan.class_tmp_offset);
@@ -1434,10 +1445,34 @@ ttamd_status backward_mfma(const ConvPlan &pl, const void *gout, void *gin, void
             dgrad_interleave_kernel<T><<<dim3(static_cast<unsigned>(blocks)), dim3(256), 0, st>>>(g, tmp, static_cast<T *>(gin), dc.tab, total);
             TTAMD_HIP_CHECK(hipGetLastError());
         } else {
-            const int total = g.C * g.O * g.k * g.k;
-            weight_transpose_kernel<T><<<dim3((total + 255) / 256), dim3(256), 0, st>>>(g, static_cast<const T *>(pl.w), wt, total);
-            TTAMD_HIP_CHECK(hipGetLastError());
-            if (ttamd_status rc = dgrad_gemm(g, wt, static_cast<T *>(gin))) return rc;
+            bool handled = false;
+            if constexpr (std::is_same_v<T, float>) {
+                // unit stride: grad_input is the convolution of grad_out with the reversed taps, padding k - 1 - P and
+                // the weight's two channel axes exchanged -- the persistent kernel of conv_patch.hip reads the weight
+                // in that order itself (no transposed copy)
+                if (g.S == 1 && g.kh == g.k && g.kw == g.k && g.P < g.k && patch_kernel_enabled()) {
+                    ConvPatchArgs a{};
+                    a.x = static_cast<const float *>(gout);
+                    a.w = static_cast<const float *>(pl.w);
+                    a.bias = nullptr;
+                    a.out = static_cast<float *>(gin);
+                    a.B = g.B; a.C = g.O; a.H = g.Ho; a.W = g.Wo; a.O = g.C; a.k = g.k; a.P = g.k - 1 - g.P; a.Ho = g.H; a.Wo = g.W;
+                    a.xs_b = static_cast<int64_t>(g.O) * HoWo; a.xs_c = HoWo; a.xs_h = g.Wo;
+                    a.w_row = static_cast<int64_t>(g.k) * g.k; a.w_red = g.w_so; a.w_flip = 1; a.w_rows_fast = 1;
+                    a.image_bytes = static_cast<int64_t>(g.O) * HoWo * 4;
+                    a.weight_bytes = pl.weight_bytes;
+                    int variant = 0;
+                    if (ttamd_status rc = launch_conv_patch_f32(a, st, &variant)) return rc;
+                    handled = variant != 0;
+                    if (handled) t_last_kernel[1] = 0x200 + variant;
+                }
+            }
+            if (!handled) {
+                const int total = g.C * g.O * g.k * g.k;
+                weight_transpose_kernel<T><<<dim3((total + 255) / 256), dim3(256), 0, st>>>(g, static_cast<const T *>(pl.w), wt, total);
+                TTAMD_HIP_CHECK(hipGetLastError());
+                if (ttamd_status rc = dgrad_gemm(g, wt, static_cast<T *>(gin))) return rc;
+            }
         }
     }
     // grad_weight
@@ -1514,12 +1549,15 @@ using namespace ttamd;
 
 extern "C" {
 
+int ttamd_conv2d_last_kernel(int which) { return which == 0 || which == 1 ? ttamd::t_last_kernel[which] : 0; }
+
 ttamd_status ttamd_conv2d_forward(int device, ttamd_dtype dtype, const ttamd_view4 *input, const ttamd_view4 *weight,
                                   const void *bias, void *out, int B, int C, int H, int W, int O, int k, int stride,
                                   int padding, void *stream) {
     ConvPlan pl;
     if (ttamd_status s = make_plan("conv2d", dtype, input, weight, B, C, H, W, O, k, stride, padding, &pl)) return s;
     if (ttamd_status s = use_device(device)) return s;
+    t_last_kernel[0] = 0;
     if (B == 0) return TTAMD_OK;
     if (!input->data || !weight->data || !out) {
         set_error("conv2d: NULL data pointer");

@@ -32,24 +32,12 @@ namespace {
 
 using namespace mfma;
 
-constexpr int kStageLoads = 32;   // 16-byte loads per tile and lane, times the waves of the workgroup
+constexpr int kStageLoads = 64;   // most 16-byte loads per tile and lane, times the waves of the workgroup
 constexpr int kWeightLoads = 80;  // likewise for the loads in flight while the weights are brought in
 constexpr int kLdsBytes = 160 * 1024;  // per workgroup on gfx950
 constexpr int kPairs = 4;        // (row, channel) pairs of the weight a lane moves together
 
 __device__ __forceinline__ f32x4 lds_load4(const float *p) { return *reinterpret_cast<const f32x4 *>(p); }
-
-#ifdef TTAMD_PATCH_TRACE  // development builds: cycle stamps of workgroup 0's waves at the phase boundaries
-__device__ uint64_t g_patch_trace[8 * 64];
-#define PATCH_STAMP(slot)                                                                               \
-    do {                                                                                                \
-        if (blockIdx.x == 0 && lane == 0 && (slot) < 64) g_patch_trace[wave * 64 + (slot)] = clock64(); \
-    } while (0)
-#else
-#define PATCH_STAMP(slot) \
-    do {                  \
-    } while (0)
-#endif
 
 // Issue order of one group: an LDS read after every second MFMA (2 CC reads, 4 CC MFMAs).  Left to itself the
 // scheduler sinks each read down to the MFMA that consumes it, which exposes the LDS latency once per chunk.
@@ -65,15 +53,16 @@ __device__ __forceinline__ void interleave_reads() {
 // WGM x WGN waves of one 32 x 32 MFMA block each: output tile (32 WGM) channels x (32 WGN) positions.
 // CC: chunks of 8 reduction indices (8 channels of one tap) that are read and multiplied as one straight-line group;
 // C / 8 is a multiple of it.
-template <int WGM, int WGN, int CC>
+// MAXS: staging slots (16-byte loads per lane and tile).
+template <int WGM, int WGN, int CC, int MAXS>
 __global__ void __launch_bounds__(64 * WGM * WGN, 1) conv_patch_kernel(ConvPatchArgs a) {
     constexpr int NW = WGM * WGN, NT = 64 * NW;  // 4 waves (one per SIMD) or 8
     static_assert(NW == 4 || NW == 8, "4 or 8 waves");
-    constexpr int MAXS = kStageLoads / NW, WVECS = kWeightLoads / NW;
+    constexpr int WVECS = kWeightLoads / NW;
     constexpr int BM = 32 * WGM, BN = 32 * WGN;
     extern __shared__ __attribute__((aligned(16))) float smem_patch[];
     float *const A = smem_patch;                   // [BM][lda], k' = tap * C + c
-    float *const patch = smem_patch + BM * a.lda;  // [2][R][pitch][cpad], then a few floats nobody reads
+    float *const patch = smem_patch + BM * a.lda;  // [1 or 2][R][pitch][cpad]
     const int tid = threadIdx.x, lane = tid % 64;
     const int wave = __builtin_amdgcn_readfirstlane(tid / 64);
     const int wm = wave / WGN, wn = wave % WGN;
@@ -86,8 +75,6 @@ __global__ void __launch_bounds__(64 * WGM * WGN, 1) conv_patch_kernel(ConvPatch
     const int mblk = blockIdx.x % a.tiles_m, gi = blockIdx.x / a.tiles_m;
     const int m0 = mblk * BM;
     const int n_tiles = a.B * a.tiles_n;
-
-    PATCH_STAMP(0);
     const int n_groups = K / (8 * CC);
     const float *const ap = A + (wm * 32 + li) * a.lda + 4 * kg;
     const int HoWo = a.Ho * a.Wo;
@@ -181,7 +168,6 @@ __global__ void __launch_bounds__(64 * WGM * WGN, 1) conv_patch_kernel(ConvPatch
             for (int i = 0; i < WVECS; ++i)
                 if (i < a.n_wvec) wv[i] = Vec<float, 4>::load(wsrc, static_cast<uint32_t>(tid + i * NT) * 16u);
         }
-        PATCH_STAMP(56);
         auto pair_of = [&](int v, int s0, const float *&src, float *&dst) {
             uint32_t slow, fast;
             a.d_wfast.divmod(static_cast<uint32_t>(v), slow, fast);
@@ -226,9 +212,7 @@ __global__ void __launch_bounds__(64 * WGM * WGN, 1) conv_patch_kernel(ConvPatch
                         if (v0 + i * NT < v_hi) *reinterpret_cast<f32x4 *>(patch + 4 * (v0 + i * NT - v_lo)) = part[i];
                 }
             }
-            PATCH_STAMP(57 + (s0 > 0 ? 3 : 0));
             __syncthreads();
-            PATCH_STAMP(58 + (s0 > 0 ? 3 : 0));
             const int n_pairs = (s1 - s0) * a.n_fast;
             if (k2 == 9) {
 #pragma unroll 1
@@ -257,15 +241,12 @@ __global__ void __launch_bounds__(64 * WGM * WGN, 1) conv_patch_kernel(ConvPatch
                     for (int t = 0; t < k2; ++t) dst[t * step] = src[t];
                 }
             }
-            PATCH_STAMP(59 + (s0 > 0 ? 3 : 0));
         }
     }
-    PATCH_STAMP(1);
     __syncthreads();  // the weights have left the patch area
-    PATCH_STAMP(2);
     // the halo columns of both patch buffers stay zero from here on; every other cell is rewritten for each tile
     {
-        const int halo_cells = 2 * a.R * 2 * a.P;  // (buffer, row, side, column)
+        const int halo_cells = a.n_buf * a.R * 2 * a.P;  // (buffer, row, side, column)
 #pragma unroll 1
         for (int v = tid; v < halo_cells * (cpad / 4); v += NT) {
             uint32_t cell, c4, br, sp, side, pc;
@@ -276,20 +257,15 @@ __global__ void __launch_bounds__(64 * WGM * WGN, 1) conv_patch_kernel(ConvPatch
             *reinterpret_cast<f32x4 *>(patch + (static_cast<int>(br) * pitch + x) * cpad + 4 * static_cast<int>(c4)) = f32x4{0.f, 0.f, 0.f, 0.f};
         }
     }
-    PATCH_STAMP(3);
     if (j < n_tiles) park(0);
-    PATCH_STAMP(5);
     __syncthreads();
-    PATCH_STAMP(6);
-    int stamp = 8;
 
     // The reduction in groups of CC chunks: group g covers tap g / ngrp, channels (g % ngrp) * 8 CC ..., i.e. k' from
     // 8 CC g on.  The fragments of the next group are requested from LDS before the MFMAs of the current one (two
     // register sets, no copies), so a wave's own LDS latency hides behind its MFMA work: with one wave per SIMD
     // nothing else would hide it.
-    for (int cur = 0; j < n_tiles; j += groups, cur ^= 1) {
+    for (int cur = 0; j < n_tiles; j += groups, cur ^= a.n_buf - 1) {
         const int jn = j + groups;
-        PATCH_STAMP(stamp);
         const int b = tile_b, n0 = tile_n * BN, h_first = tile_h;
         if (jn < n_tiles) {  // the next tile's rows are in flight during this tile's MFMA work
             tile_n += static_cast<int>(step_n);
@@ -327,7 +303,6 @@ __global__ void __launch_bounds__(64 * WGM * WGN, 1) conv_patch_kernel(ConvPatch
                 for (int t = 0; t < 4; ++t) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[i][t], fb[i][t], acc, 0, 0, 0);
         };
         f32x4 fa0[CC], fa1[CC], fb0[CC], fb1[CC];
-        PATCH_STAMP(stamp + 1);
         if (wave_active) fetch(0, fa0, fb0);
         int g = wave_active ? 0 : n_groups;
         for (; g + 1 < n_groups; g += 2) {
@@ -339,10 +314,9 @@ __global__ void __launch_bounds__(64 * WGM * WGN, 1) conv_patch_kernel(ConvPatch
             interleave_reads<4 * CC>();
         }
         if (g < n_groups) multiply(fa0, fb0);
-        PATCH_STAMP(stamp + 2);
 
-        if (jn < n_tiles) park(cur ^ 1);  // the loads were issued a whole tile ago
-        PATCH_STAMP(stamp + 3);
+        if (a.n_buf == 1) __syncthreads();  // one patch buffer: every wave has left it
+        if (jn < n_tiles) park(cur ^ (a.n_buf - 1));  // the loads were issued a whole tile ago
 
         // store: out[b][o][n] (+ bias[o]); positions outside the result are dropped by the buffer store
         if (wave_active) {
@@ -367,15 +341,12 @@ __global__ void __launch_bounds__(64 * WGM * WGN, 1) conv_patch_kernel(ConvPatch
                 }
             }
         }
-        PATCH_STAMP(stamp + 4);
         __syncthreads();
-        PATCH_STAMP(stamp + 5);
-        stamp += 8;
     }
 }
 
 // Derived geometry for tiles of BM x BN computed by `waves` waves; false when this kernel does not apply.
-bool plan_patch(ConvPatchArgs &a, int BM, int BN, int waves, size_t *lds_bytes) {
+bool plan_patch(ConvPatchArgs &a, int BM, int BN, int waves, int n_buf, size_t *lds_bytes) {
     const int k = a.k, threads = 64 * waves;
     const int HoWo = a.Ho * a.Wo;
     a.K = a.C * k * k;
@@ -393,7 +364,8 @@ bool plan_patch(ConvPatchArgs &a, int BM, int BN, int waves, size_t *lds_bytes) 
     a.tiles_m = (a.O + BM - 1) / BM;
     a.tiles_n = (HoWo + BN - 1) / BN;
     const int64_t patch_elems = static_cast<int64_t>(a.R) * a.pitch * a.cpad;
-    int64_t lds_floats = static_cast<int64_t>(BM) * a.lda + 2 * patch_elems;
+    a.n_buf = n_buf;
+    int64_t lds_floats = static_cast<int64_t>(BM) * a.lda + n_buf * patch_elems;
     if (a.stage_slots > kStageLoads / waves || lds_floats * 4 > kLdsBytes) return false;
     if (static_cast<int64_t>(a.B) * a.tiles_n > 0x7fffffff || static_cast<int64_t>(a.O) * HoWo * 4 >= 0x7fffffff) return false;
     if (static_cast<int64_t>(a.C) * a.xs_c * 4 + static_cast<int64_t>(a.R) * a.xs_h * 4 >= 0x7fffffff) return false;
@@ -428,14 +400,14 @@ bool plan_patch(ConvPatchArgs &a, int BM, int BN, int waves, size_t *lds_bytes) 
     return true;
 }
 
-template <int WGM, int WGN, int CC>
+template <int WGM, int WGN, int CC, int MAXS>
 ttamd_status launch_patch(ConvPatchArgs a, hipStream_t st, size_t lds) {
     const int64_t n_tiles = static_cast<int64_t>(a.B) * a.tiles_n;
     int64_t groups = 256 / a.tiles_m;
     if (groups < 1) groups = 1;
     if (groups > n_tiles) groups = n_tiles;
     a.d_ngrp = make_fastdiv(static_cast<uint32_t>(a.C / (8 * CC)));
-    auto kernel = conv_patch_kernel<WGM, WGN, CC>;
+    auto kernel = conv_patch_kernel<WGM, WGN, CC, MAXS>;
     TTAMD_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds)));
     kernel<<<dim3(static_cast<unsigned>(groups * a.tiles_m)), dim3(64 * WGM * WGN), lds, st>>>(a);
     TTAMD_HIP_CHECK(hipGetLastError());
@@ -444,27 +416,21 @@ ttamd_status launch_patch(ConvPatchArgs a, hipStream_t st, size_t lds) {
 
 template <int WGM, int WGN>
 ttamd_status launch_patch_cc(const ConvPatchArgs &a, hipStream_t st, size_t lds) {
-    const int c_chunks = a.C / 8;
-    if (c_chunks % 4 == 0) return launch_patch<WGM, WGN, 4>(a, st, lds);
-    if (c_chunks % 2 == 0) return launch_patch<WGM, WGN, 2>(a, st, lds);
-    return launch_patch<WGM, WGN, 1>(a, st, lds);
+    constexpr int S1 = kStageLoads / (WGM * WGN), S0 = S1 / 2;  // slot counts compiled for
+    const bool few = a.stage_slots <= S0;
+    if (a.C % 32 == 0) return few ? launch_patch<WGM, WGN, 4, S0>(a, st, lds) : launch_patch<WGM, WGN, 4, S1>(a, st, lds);
+    return few ? launch_patch<WGM, WGN, 1, S0>(a, st, lds) : launch_patch<WGM, WGN, 1, S1>(a, st, lds);
 }
 
 }  // namespace
 
-#ifdef TTAMD_PATCH_TRACE
-extern "C" int ttamd_debug_patch_trace(uint64_t *host_out) {
-    return static_cast<int>(hipMemcpyFromSymbol(host_out, HIP_SYMBOL(g_patch_trace), sizeof(uint64_t) * 4 * 64));
-}
-#endif
-
-// Launches when the geometry fits this kernel: *handled says whether it did.  Expects in `a`: the tensors and their
+// Launches when the geometry fits this kernel: *variant is 0 when it does not, else 16 * waves + patch buffers.  Expects in `a`: the tensors and their
 // strides, B C H W O k P Ho Wo, and the weight access (w_row, w_red, w_flip, w_rows_fast): tap t of (row, reduction
 // channel) is at element  row * w_row + red * w_red + t  of the weight and is used as tap k*k - 1 - t when w_flip is
 // set.  Eight waves (two per SIMD, which hide each other's staging and store latencies) where their larger patch
-// fits in LDS, four otherwise.
-ttamd_status launch_conv_patch_f32(ConvPatchArgs a, hipStream_t st, bool *handled) {
-    *handled = false;
+// fits in LDS, four otherwise; two patch buffers where they fit, one otherwise.
+ttamd_status launch_conv_patch_f32(ConvPatchArgs a, hipStream_t st, int *variant) {
+    *variant = 0;
     const int k = a.k;
     if (a.B <= 0 || k < 1 || a.P >= k || a.C % 8 != 0 || a.W % 4 != 0) return TTAMD_OK;
     if (a.xs_h % 4 != 0 || a.xs_c % 4 != 0 || a.xs_b % 4 != 0 || reinterpret_cast<uintptr_t>(a.x) % 16 != 0) return TTAMD_OK;
@@ -473,13 +439,15 @@ ttamd_status launch_conv_patch_f32(ConvPatchArgs a, hipStream_t st, bool *handle
     const bool narrow = a.O <= 32;
     size_t lds = 0;
     static const bool wide_ok = std::getenv("TTAMD_CONV_PATCH_WAVES") == nullptr || std::atoi(std::getenv("TTAMD_CONV_PATCH_WAVES")) != 4;
-    if (wide_ok && plan_patch(a, narrow ? 32 : 64, narrow ? 256 : 128, 8, &lds)) {
-        *handled = true;
-        return narrow ? launch_patch_cc<1, 8>(a, st, lds) : launch_patch_cc<2, 4>(a, st, lds);
-    }
-    if (plan_patch(a, narrow ? 32 : 64, narrow ? 128 : 64, 4, &lds)) {
-        *handled = true;
-        return narrow ? launch_patch_cc<1, 4>(a, st, lds) : launch_patch_cc<2, 2>(a, st, lds);
+    for (int n_buf = 2; n_buf >= 1; --n_buf) {  // one patch buffer (a second barrier per tile) when two do not fit
+        if (wide_ok && plan_patch(a, narrow ? 32 : 64, narrow ? 256 : 128, 8, n_buf, &lds)) {
+            *variant = 8 * 16 + n_buf;
+            return narrow ? launch_patch_cc<1, 8>(a, st, lds) : launch_patch_cc<2, 4>(a, st, lds);
+        }
+        if (plan_patch(a, narrow ? 32 : 64, narrow ? 128 : 64, 4, n_buf, &lds)) {
+            *variant = 4 * 16 + n_buf;
+            return narrow ? launch_patch_cc<1, 4>(a, st, lds) : launch_patch_cc<2, 2>(a, st, lds);
+        }
     }
     return TTAMD_OK;
 }
