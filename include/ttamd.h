@@ -129,6 +129,12 @@ ttamd_status ttamd_memory_allocated(int device, uint64_t *current_bytes, uint64_
  * (cuda/data_types.cuh:28-101). */
 ttamd_status ttamd_malloc_on_stream(int device, size_t bytes, void *stream, void **out);
 ttamd_status ttamd_free_on_stream(int device, void *ptr, size_t bytes, void *stream);
+
+/* No counterpart in the reference.  Call before destroying a stream that was ever passed to ttamd_malloc_on_stream or
+ * ttamd_free_on_stream: waits for the stream's work (hipStreamSynchronize) and removes the handle from the allocator's
+ * books, so that no later request records or queries an event on a stream that no longer exists.  Blocks allocated
+ * for the stream stay valid. */
+ttamd_status ttamd_stream_release(int device, void *stream);
 ttamd_status ttamd_empty_cache(int device);
 ttamd_status ttamd_memory_cached(int device, uint64_t *cached_bytes);
 

@@ -191,3 +191,30 @@ def test_block_freed_on_one_stream_is_not_reused_on_another_while_in_flight(tt):
         assert again.storage.ptr == freed_ptr
     finally:
         stream.close()
+
+
+def test_blocks_of_a_closed_stream_serve_later_requests(tt):
+    """Blocks allocated and freed for a stream stay in the cache under its handle; once the stream has been closed
+    (Stream.close releases the handle first) a request for another stream takes such a block without touching the
+    stream that no longer exists, and a block that outlives its allocation stream is freed and reused as well."""
+    assert tt._capi.lib.ttamd_empty_cache(0) == 0
+    stream = tt.graph.Stream()
+    kept = stream.run(lambda: tt.Tensor.from_numpy(np.arange(3000, dtype=np.float32)))      # outlives the stream
+    freed_ptr = stream.run(lambda: tt.Tensor.from_numpy(np.ones(5000, np.float32)).storage.ptr)  # freed for the stream
+    stream.close()
+    again = tt.Tensor.from_numpy(np.full(5000, 2.0, np.float32))  # default stream, the cached block's size class
+    assert again.storage.ptr == freed_ptr
+    assert np.array_equal(again.to_numpy(), np.full(5000, 2.0, np.float32))
+    assert np.array_equal(kept.to_numpy(), np.arange(3000, dtype=np.float32))
+    del kept                                                       # freed for the default stream, allocated for the closed one
+    other = tt.graph.Stream()
+    try:
+        # (whether this request gets that block depends on whether the event it records on the default stream has
+        # already completed; either way it must not touch the closed stream)
+        reuse = other.run(lambda: tt.Tensor.from_numpy(np.full(3000, 5.0, np.float32)))
+        other.synchronize()
+        assert np.array_equal(reuse.to_numpy(), np.full(3000, 5.0, np.float32))
+        del reuse
+        assert tt._capi.lib.ttamd_device_synchronize(0) == 0
+    finally:
+        other.close()

@@ -42,6 +42,7 @@ def _bind(lib: C.CDLL) -> None:
         "ttamd_free": (i, [i, vp, sz]),
         "ttamd_malloc_on_stream": (i, [i, sz, vp, C.POINTER(vp)]),
         "ttamd_free_on_stream": (i, [i, vp, sz, vp]),
+        "ttamd_stream_release": (i, [i, vp]),
         "ttamd_memory_allocated": (i, [i, C.POINTER(C.c_uint64), C.POINTER(C.c_uint64)]),
         "ttamd_empty_cache": (i, [i]),
         "ttamd_memory_cached": (i, [i, C.POINTER(C.c_uint64)]),

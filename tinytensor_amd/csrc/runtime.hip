@@ -46,6 +46,8 @@ struct LiveBlock {
     size_t rounded = 0;
     hipStream_t stream = nullptr;  // the stream the block was allocated for
 };
+// Tag of a live block whose allocation stream has been released (ttamd_stream_release) in the meantime.
+const hipStream_t kNoStream = reinterpret_cast<hipStream_t>(static_cast<uintptr_t>(1));
 struct BlockCache {
     std::mutex mu;
     std::multimap<size_t, CachedBlock> free_blocks;  // rounded size -> block
@@ -287,7 +289,7 @@ ttamd_status ttamd_free_on_stream(int device, void *ptr, size_t bytes, void *str
         if (it != c.live.end()) {  // a block of the caching allocator: keep it for the next request of its class
             CachedBlock b;
             b.ptr = ptr;
-            b.stream[b.n_streams++] = it->second.stream;
+            if (it->second.stream != kNoStream) b.stream[b.n_streams++] = it->second.stream;  // (released since: nothing pending there)
             if (static_cast<hipStream_t>(stream) != it->second.stream) b.stream[b.n_streams++] = static_cast<hipStream_t>(stream);
             b.epoch = c.epoch.load();
             c.cached_bytes += it->second.rounded;
@@ -298,6 +300,36 @@ ttamd_status ttamd_free_on_stream(int device, void *ptr, size_t bytes, void *str
     }
     if (!kept) TTAMD_HIP_CHECK(hipFree(ptr));  // synchronous, like ~DeviceMemory (cuda/data_types.cu:102-116)
     g_current[device] -= bytes;
+    return TTAMD_OK;
+}
+
+ttamd_status ttamd_stream_release(int device, void *stream) {
+    if (ttamd_status s = use_device(device)) return s;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    if (!st) return TTAMD_OK;  // the default stream is never destroyed
+    TTAMD_HIP_CHECK(hipStreamSynchronize(st));
+    // Nothing of this stream's is pending any more: forget the handle, so that no later request touches it (it is about
+    // to be destroyed).  Live blocks allocated for it count as allocated for no stream from here on; cached blocks
+    // lose it from their list of streams to wait for.
+    BlockCache &c = g_cache[device];
+    std::lock_guard<std::mutex> lock(c.mu);
+    for (auto &kv : c.live)
+        if (kv.second.stream == st) kv.second.stream = kNoStream;
+    for (auto &kv : c.free_blocks) {
+        CachedBlock &b = kv.second;
+        int n = 0;
+        for (int i = 0; i < b.n_streams; ++i) {
+            if (b.stream[i] == st) {
+                if (b.event[i]) (void)hipEventDestroy(b.event[i]);
+                continue;
+            }
+            b.stream[n] = b.stream[i];
+            b.event[n] = b.event[i];
+            ++n;
+        }
+        for (int i = n; i < 2; ++i) b.stream[i] = nullptr, b.event[i] = nullptr;
+        b.n_streams = n;
+    }
     return TTAMD_OK;
 }
 

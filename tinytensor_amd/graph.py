@@ -71,10 +71,12 @@ class Stream:
             return fn()
 
     def close(self) -> None:
-        """Waits for the stream's work, then destroys it (blocks freed for this stream stay in the allocator's cache
-        under its handle; they are idle once the stream is)."""
+        """Waits for the stream's work and takes the handle off the allocator's books (blocks allocated or freed for
+        this stream stay usable; nothing will wait on the stream again), then destroys it."""
         if self._h.value:
-            _call("hipStreamSynchronize", self._h)
+            rc = _capi.lib.ttamd_stream_release(kAMD.id, self._h)
+            if rc != 0:
+                raise TTException(_capi.lib.ttamd_last_error_string().decode())
             _call("hipStreamDestroy", self._h)
             self._h = C.c_void_p()
 
