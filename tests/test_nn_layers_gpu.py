@@ -103,3 +103,32 @@ def test_integer_and_bool_sums_are_64_bit(tt):
     assert np.array_equal(tm.permute(1, 0).sum(0).to_numpy(), m.sum(axis=1).astype(np.int64))   # strided view
     f = tt.Tensor.from_numpy(np.ones((4, 5), np.float32))
     assert f.sum().dtype == tt._capi.F32 and f.sum(1).dtype == tt._capi.F32
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+def test_draws_from_caller_supplied_states(tt, oracle, dtype):
+    """ttamd_random_fill_states: the caller draws one generator state per element (cpu/distribution.cpp:31-38) and the
+    device writes element i of the view from state i -- the same values as the call that draws the states itself."""
+    import ctypes as C
+    code = tt._capi.F32 if dtype == np.float32 else tt._capi.F64
+    lib = tt._capi.lib
+    shape, stride, offset = (3, 5, 2), (2, 6, 1), 1           # a permuted view with an offset into 31 stored elements
+    n = int(np.prod(shape))
+    for dist, p0, p1 in ((0, -0.5, 0.25), (1, 0.0, 0.1)):
+        gen = oracle.Generator(11)
+        states = (C.c_uint64 * n)(*[gen() for _ in range(n)])  # Generator::operator(), element order = the view's row-major order
+        by_states = tt.Tensor.from_numpy(np.full(31, -7.0, dtype=dtype))
+        rc = lib.ttamd_random_fill_states(0, code, dist, p0, p1, states, 3, (C.c_int64 * 3)(*shape), (C.c_int64 * 3)(*stride),
+                                          C.c_void_p(by_states.storage.ptr), offset, None)
+        assert rc == 0, tt._capi.last_error()
+        by_master = tt.Tensor.from_numpy(np.full(31, -7.0, dtype=dtype))
+        view = tt.Tensor(by_master.storage, code, shape, stride, offset)
+        g_dev = tt.Generator(11)
+        (view.uniform_real_ if dist == 0 else view.normal_)(p0, p1, g_dev)
+        assert g_dev.state.value == gen.state                  # both consumed n outputs
+        assert np.array_equal(by_states.to_numpy(), by_master.to_numpy())
+        assert np.count_nonzero(by_states.to_numpy() != -7.0) == n
+    if dtype == np.float32:
+        rc = lib.ttamd_random_fill_states(0, tt._capi.I32, 0, 0.0, 1.0, states, 3, (C.c_int64 * 3)(*shape), (C.c_int64 * 3)(*stride),
+                                          C.c_void_p(by_states.storage.ptr), offset, None)
+        assert rc != 0                                          # floating point dtypes only
