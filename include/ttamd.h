@@ -199,10 +199,11 @@ ttamd_status ttamd_conv2d_backward(int device, ttamd_dtype dtype, const void *gr
                                    size_t workspace_bytes, void *stream);
 
 /* No counterpart in the reference: which kernel family the calling thread's last ttamd_conv2d_forward (which = 0) or
- * the grad_input part of its last ttamd_conv2d_backward (which = 1) launched.  0x100: the implicit-GEMM MFMA kernels;
- * 0x200 + 16 * waves + patch buffers: the persistent kernel that keeps the weight block in LDS (fp32, unit stride,
- * channel counts that are multiples of 8, rows of whole 16-byte vectors); 0: neither (another dtype, a direct
- * kernel) or no call yet.  For tests and profiles that mean to cover a particular kernel. */
+ * the grad_input (which = 1) or grad_weight (which = 2) part of its last ttamd_conv2d_backward launched.  0x100: the
+ * implicit-GEMM MFMA kernels; 0x200 + 16 * waves + patch buffers: the persistent kernel that keeps the weight block in
+ * LDS (fp32, unit stride, channel counts that are multiples of 8, rows of whole 16-byte vectors), 0x200 for
+ * grad_weight: the kernel that stages both operands in LDS; 0: neither (another dtype, a direct kernel) or no call
+ * yet.  For tests and profiles that mean to cover a particular kernel. */
 int ttamd_conv2d_last_kernel(int which);
 
 /* BackendBase::max_pool2d / min_pool2d / avg_pool2d (backend_base.h:286-311; CPU: cpu/conv.cpp:296-349 over

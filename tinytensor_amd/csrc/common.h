@@ -124,6 +124,30 @@ struct ConvPatchArgs {
 };
 ttamd_status launch_conv_patch_f32(ConvPatchArgs a, hipStream_t stream, int *variant);
 
+// grad_weight with both operands staged in LDS (conv_wgrad_patch.hip).  The plan depends on the shape alone.
+struct ConvWgradPatchPlan {
+    bool use;
+    int RS, SPI;          // output rows per stage, stages per image
+    int n_stages;         // B * SPI
+    int workgroups;       // = partial tiles written
+    int blocks_per_wave;
+    size_t lds_bytes;
+};
+ConvWgradPatchPlan plan_conv_wgrad_patch(int B, int C, int H, int W, int O, int k, int S, int P);
+struct ConvWgradPatchArgs {
+    const float *gout;     // dense [B,O,Ho,Wo]
+    const float *x;        // input [B,C,H,W]: column stride 1, the other strides below (elements)
+    float *partial;        // [workgroups][O][C k k]
+    int B, C, H, W, O, k, P, Ho, Wo;
+    int64_t xs_b;
+    int32_t xs_c, xs_h;
+    int64_t image_bytes;   // bytes reachable from an image's first element
+    // derived
+    int RS, SPI, n_stages, R, pitch, plane, pitch_a, waves_per_ob, col_blocks, blocks_per_wave;
+    FastDiv d_cblocks, d_k, d_2P, d_P, d_R, d_spi, d_avecs, d_xvecs, d_vw, d_kvecs;
+};
+ttamd_status launch_conv_wgrad_patch_f32(ConvWgradPatchArgs a, const ConvWgradPatchPlan &plan, hipStream_t stream, bool *handled);
+
 }  // namespace ttamd
 
 #endif  // TTAMD_CSRC_COMMON_H_

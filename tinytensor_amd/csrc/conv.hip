@@ -795,7 +795,34 @@ __global__ void __launch_bounds__(256) reduce_splits_stream_kernel(const T *__re
     *reinterpret_cast<V *>(out + i) = acc;
 }
 
-// out[i] = sum over parts of partial[s][i], by whichever of the two kernels suits the shape: the streaming one when
+// The same sum for many parts of a tile of middling length (grad_weight's one partial tile per workgroup): a workgroup
+// owns 64 consecutive elements, each of its four waves adds a contiguous quarter of the parts in increasing order --
+// every load a whole coalesced line of the wave, eight in flight -- and the four sums are added in order.
+template <typename T>
+__global__ void __launch_bounds__(256) reduce_splits_ranges_kernel(const T *__restrict__ partial, T *__restrict__ out, int64_t n, int splits) {
+    __shared__ T red[4][64];
+    const int lane = threadIdx.x % 64, w = threadIdx.x / 64;
+    const int64_t i = static_cast<int64_t>(blockIdx.x) * 64 + lane;
+    const int per = (splits + 3) / 4;
+    const int s0 = w * per, s1 = s0 + per < splits ? s0 + per : splits;
+    T acc = T(0);
+    if (i < n) {
+        int s = s0;
+        for (; s + 8 <= s1; s += 8) {
+            T v[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) v[u] = partial[static_cast<int64_t>(s + u) * n + i];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) acc += v[u];
+        }
+        for (; s < s1; ++s) acc += partial[static_cast<int64_t>(s) * n + i];
+    }
+    red[w][lane] = acc;
+    __syncthreads();
+    if (w == 0 && i < n) out[i] = ((red[0][lane] + red[1][lane]) + red[2][lane]) + red[3][lane];
+}
+
+// out[i] = sum over parts of partial[s][i], by whichever of the kernels suits the shape: the streaming one when
 // there are enough vectors to fill the chip or too few parts to occupy the other's sixteen lanes per element.
 template <typename T>
 ttamd_status launch_reduce_splits(const T *partial, T *out, int64_t n, int splits, hipStream_t st) {
@@ -804,6 +831,8 @@ ttamd_status launch_reduce_splits(const T *partial, T *out, int64_t n, int split
     if (aligned && (n / VEC >= 65536 || splits <= 8)) {
         const int64_t blocks = (n / VEC + 255) / 256;
         reduce_splits_stream_kernel<T><<<dim3(static_cast<unsigned>(blocks)), dim3(256), 0, st>>>(partial, out, n, splits);
+    } else if (splits >= 32 && n >= 4096) {
+        reduce_splits_ranges_kernel<T><<<dim3(static_cast<unsigned>((n + 63) / 64)), dim3(256), 0, st>>>(partial, out, n, splits);
     } else {
         reduce_splits_kernel<T><<<dim3(static_cast<unsigned>((n + 15) / 16)), dim3(256), 0, st>>>(partial, out, n, splits);
     }
@@ -1028,10 +1057,10 @@ ttamd_status set_lds(Kernel kernel, size_t lds_bytes) {
     return TTAMD_OK;
 }
 
-// Which kernel family the calling thread's last forward ([0]) and grad_input ([1]) launches took: 0x100 the
+// Which kernel family the calling thread's last forward ([0]), grad_input ([1]) and grad_weight ([2]) launches took: 0x100 the
 // implicit-GEMM kernels of this file, 0x200 + 16 * waves + patch buffers the persistent kernel of conv_patch.hip,
 // 0 anything else.  Read through ttamd_conv2d_last_kernel by the tests that mean to cover a particular kernel.
-thread_local int t_last_kernel[2] = {0, 0};
+thread_local int t_last_kernel[3] = {0, 0, 0};
 
 // TTAMD_CONV_PATCH=0 keeps every convolution on the implicit-GEMM kernels of this file (for comparisons).
 inline bool patch_kernel_enabled() {
@@ -1320,6 +1349,10 @@ BackwardWorkspace backward_workspace(size_t esz, int B, int C, int H, int W, int
         w.k_chunk = joint_k;
     }
     w.partial_bytes = w.parts() > 1 ? static_cast<size_t>(w.parts()) * tile : 0;
+    if (esz == 4) {  // the LDS-staged grad_weight kernel writes one partial tile per workgroup
+        const ConvWgradPatchPlan pp = plan_conv_wgrad_patch(B, C, H, W, O, k, stride, padding);
+        if (pp.use && pp.workgroups > 1 && static_cast<size_t>(pp.workgroups) * tile > w.partial_bytes) w.partial_bytes = static_cast<size_t>(pp.workgroups) * tile;
+    }
     w.partial_bytes = (w.partial_bytes + 255) & ~static_cast<size_t>(255);
     w.bias_bytes = static_cast<size_t>(kBiasGradParts) * O * esz;
     return w;
@@ -1479,6 +1512,27 @@ ttamd_status backward_mfma(const ConvPlan &pl, const void *gout, void *gin, void
     {
         const int M_ = g.O, N_ = g.C * g.k * g.k;
         const int64_t tile_elems = static_cast<int64_t>(M_) * N_;
+        bool staged = false;
+        if constexpr (std::is_same_v<T, float>) {
+            // unit stride, channel counts that are multiples of 32, rows of whole vectors: both operands staged in LDS
+            if (g.xs_w == 1 && patch_kernel_enabled()) {
+                const ConvWgradPatchPlan pp = plan_conv_wgrad_patch(g.B, g.C, g.H, g.W, g.O, g.k, g.S, g.P);
+                if (pp.use) {
+                    ConvWgradPatchArgs a{};
+                    a.gout = static_cast<const float *>(gout);
+                    a.x = static_cast<const float *>(pl.x);
+                    a.partial = pp.workgroups > 1 ? partials : static_cast<float *>(gw);
+                    a.B = g.B; a.C = g.C; a.H = g.H; a.W = g.W; a.O = g.O; a.k = g.k; a.P = g.P; a.Ho = g.Ho; a.Wo = g.Wo;
+                    a.xs_b = g.xs_b; a.xs_c = g.xs_c; a.xs_h = g.xs_h;
+                    a.image_bytes = pl.image_bytes;
+                    if (ttamd_status rc = launch_conv_wgrad_patch_f32(a, pp, st, &staged)) return rc;
+                    if (staged && pp.workgroups > 1)
+                        if (ttamd_status rc = launch_reduce_splits<T>(partials, static_cast<T *>(gw), tile_elems, pp.workgroups, st)) return rc;
+                }
+            }
+        }
+        t_last_kernel[2] = staged ? 0x200 : 0x100;
+        if (!staged) {
         const int parts = plan.parts();
         T *const partial = parts > 1 ? partials : static_cast<T *>(gw);
         const int tiles_m = (M_ + 63) / 64, tiles_n = (N_ + 63) / 64;
@@ -1515,6 +1569,7 @@ ttamd_status backward_mfma(const ConvPlan &pl, const void *gout, void *gin, void
         if (s) return s;
         if (parts > 1)
             if (ttamd_status rc = launch_reduce_splits<T>(partial, static_cast<T *>(gw), tile_elems, parts, st)) return rc;
+        }
     }
     if (gb) {
         using V = std::conditional_t<sizeof(T) == 4, float4, double2>;
@@ -1549,7 +1604,7 @@ using namespace ttamd;
 
 extern "C" {
 
-int ttamd_conv2d_last_kernel(int which) { return which == 0 || which == 1 ? ttamd::t_last_kernel[which] : 0; }
+int ttamd_conv2d_last_kernel(int which) { return which >= 0 && which <= 2 ? ttamd::t_last_kernel[which] : 0; }
 
 ttamd_status ttamd_conv2d_forward(int device, ttamd_dtype dtype, const ttamd_view4 *input, const ttamd_view4 *weight,
                                   const void *bias, void *out, int B, int C, int H, int W, int O, int k, int stride,
