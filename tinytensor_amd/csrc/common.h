@@ -143,8 +143,8 @@ struct ConvWgradPatchArgs {
     int32_t xs_c, xs_h;
     int64_t image_bytes;   // bytes reachable from an image's first element
     // derived
-    int RS, SPI, n_stages, R, pitch, plane, pitch_a, waves_per_ob, col_blocks, blocks_per_wave;
-    FastDiv d_cblocks, d_k, d_2P, d_P, d_R, d_spi, d_avecs, d_xvecs, d_vw, d_kvecs;
+    int RS, SPI, n_stages, R, pitch, plane, pitch_a, waves_per_ob, col_blocks, blocks_per_wave, rows_per_load;
+    FastDiv d_cblocks, d_k, d_2P, d_P, d_R, d_spi, d_vw;
 };
 ttamd_status launch_conv_wgrad_patch_f32(ConvWgradPatchArgs a, const ConvWgradPatchPlan &plan, hipStream_t stream, bool *handled);
 

@@ -21,9 +21,21 @@ namespace {
 
 using namespace mfma;
 
+// Issue order of a chunk: the next chunk's 16-byte A read first, then a pair of 4-byte B reads behind every second
+// MFMA of the current chunk.  Left to itself the scheduler sinks every read down to the MFMA that consumes it.
+template <int N, int I = 0>
+__device__ __forceinline__ void interleave_reads() {
+    if constexpr (I == 0) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+    if constexpr (I < N) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        if constexpr (I % 2 == 0) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // (the compiler pairs the 4-byte reads)
+        interleave_reads<N, I + 1>();
+    }
+}
+
 constexpr int kMaxBlocks = 5;        // 32 x 32 result blocks per wave (80 accumulator registers)
 constexpr int kLdsBytes = 160 * 1024;
-constexpr int kBatchA = 14, kBatchX = 8;  // 16-byte loads per lane and round of the staging: grad_out rows, input rows
+constexpr int kBatchA = 16, kBatchX = 8;  // 16-byte loads per lane and round of the staging: grad_out rows, input rows
 
 // NB: blocks per wave compiled for (the wave's actual count may be lower).
 template <int NB>
@@ -68,8 +80,14 @@ __global__ void __launch_bounds__(kThreads, 1) conv_wgrad_patch_kernel(ConvWgrad
         patch[static_cast<int>(c) * plane + static_cast<int>(r) * pitch + (side ? a.P + a.W + static_cast<int>(pc) : static_cast<int>(pc))] = 0.f;
     }
 
+    // the lane's part of an input load: row x_lane_r of the item's row group, vector x_lane_v of that row
+    uint32_t xr, xv;
+    a.d_vw.divmod(static_cast<uint32_t>(lane), xr, xv);
+    const int x_lane_r = static_cast<int>(xr);
+    const bool x_lane_ok = x_lane_r < a.rows_per_load;
+    const uint32_t x_lane_goff = static_cast<uint32_t>((x_lane_r * a.xs_h + 4 * static_cast<int>(xv)) * 4);
+    const int x_lane_lds = x_lane_r * pitch + a.P + 4 * static_cast<int>(xv);
     const int a_vecs = pitch_a / 4;            // 16-byte vectors per staged grad_out row (the tail beyond the stage: zeros)
-    const int x_vecs = a.R * (a.W / 4);        // vectors per channel of the patch
     const int HoWo = a.Ho * Wo;
     const float *const ap = gy + (ob * 32 + li) * pitch_a + 4 * kg;
 
@@ -81,45 +99,57 @@ __global__ void __launch_bounds__(kThreads, 1) conv_wgrad_patch_kernel(ConvWgrad
         const int np = rows * Wo;  // positions of this stage (a multiple of 4)
         // ---- stage: grad_out rows [O][np] (zeros behind np), input rows r0 - P .. r0 - P + R - 1 of every channel
         {
-            // all loads of a round are issued before the first LDS write, so that a round costs one memory latency
+            // Row-wise: an instruction of a wave loads 64 vectors of one grad_out row, or rows_per_load input rows of
+            // one channel; which row or channel is wave-uniform and rides in the load's scalar offset, the lane's part
+            // of the address is fixed for the whole kernel.  All loads of a round are issued before its first LDS
+            // write, so a round costs one memory latency.
             const float *gbase = a.gout + (static_cast<int64_t>(b) * a.O) * HoWo + static_cast<int64_t>(r0) * Wo;
             const __amdgpu_buffer_rsrc_t gsrc = make_rsrc(gbase, (static_cast<int64_t>(a.O) * HoWo - static_cast<int64_t>(r0) * Wo) * 4);
             const int y0 = r0 - a.P;
             const int64_t first_x = static_cast<int64_t>(b) * a.xs_b + static_cast<int64_t>(y0) * a.xs_h;
             const __amdgpu_buffer_rsrc_t xsrc = make_rsrc(a.x + first_x, a.image_bytes - static_cast<int64_t>(y0) * a.xs_h * 4);
-            const int n_a = a.O * a_vecs, n_x = a.C * x_vecs;
-            for (int va = tid, vx = tid; va < n_a || vx < n_x; va += kThreads * kBatchA, vx += kThreads * kBatchX) {
+            // grad_out: wave w loads rows w, w + 4, ... (64 vectors of a row per instruction); input: channels w, w + 4,
+            // ... (rows_per_load patch rows per instruction).  The usual stage is one round of each.
+            const int a_groups = (a_vecs + 63) / 64, x_groups = (a.R + a.rows_per_load - 1) / a.rows_per_load;
+            const int a_rounds = (a.O + kWaves * kBatchA - 1) / (kWaves * kBatchA) * a_groups;
+            const int x_rounds = (a.C + kWaves * kBatchX - 1) / (kWaves * kBatchX) * x_groups;
+            for (int round = 0; round < a_rounds || round < x_rounds; ++round) {
                 f32x4 da[kBatchA], dx[kBatchX];
-                int la[kBatchA], lx[kBatchX];
+                const int vg = round % a_groups, o0 = wave + (round / a_groups) * (kWaves * kBatchA);
+                const int rg = round % x_groups, c0 = wave + (round / x_groups) * (kWaves * kBatchX);
+                const int ax = vg * 64 + lane;                              // this lane's vector of a grad_out row
+                const int xr = x_lane_r + rg * a.rows_per_load;             // this lane's patch row
+                const uint32_t a_voff = round < a_rounds && 4 * ax < np ? static_cast<uint32_t>(ax) * 16u : kOob;
+                const bool x_in = round < x_rounds && x_lane_ok && xr < a.R;
+                const uint32_t x_voff = x_in && static_cast<unsigned>(y0 + xr) < static_cast<unsigned>(a.H) ? x_lane_goff : kOob;
+                const uint32_t x_soff = static_cast<uint32_t>(rg * a.rows_per_load * a.xs_h * 4);
 #pragma unroll
                 for (int i = 0; i < kBatchA; ++i) {
-                    const int v = va + i * kThreads;
-                    uint32_t o, x;
-                    a.d_avecs.divmod(static_cast<uint32_t>(v), o, x);
-                    const bool ok = v < n_a && static_cast<int>(4 * x) < np;
-                    da[i] = Vec<float, 4>::load(gsrc, ok ? (o * static_cast<uint32_t>(HoWo) + 4 * x) * 4u : kOob);
-                    la[i] = v < n_a ? static_cast<int>(o) * pitch_a + 4 * static_cast<int>(x) : -1;
+                    const int o = o0 + i * kWaves;
+                    da[i] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(gsrc, o < a.O ? a_voff : kOob, static_cast<uint32_t>(o) * static_cast<uint32_t>(HoWo) * 4u, 0));
                 }
 #pragma unroll
                 for (int i = 0; i < kBatchX; ++i) {
-                    const int v = vx + i * kThreads;
-                    uint32_t c, rem, r, xv;
-                    a.d_xvecs.divmod(static_cast<uint32_t>(v), c, rem);
-                    a.d_vw.divmod(rem, r, xv);
-                    const bool ok = v < n_x && static_cast<unsigned>(y0 + static_cast<int>(r)) < static_cast<unsigned>(a.H);
-                    dx[i] = Vec<float, 4>::load(
-                        xsrc, ok ? static_cast<uint32_t>((static_cast<int32_t>(c) * a.xs_c + static_cast<int32_t>(r) * a.xs_h + 4 * static_cast<int32_t>(xv)) * 4) : kOob);
-                    lx[i] = v < n_x ? static_cast<int>(c) * plane + static_cast<int>(r) * pitch + a.P + 4 * static_cast<int>(xv) : -1;
+                    const int c = c0 + i * kWaves;
+                    dx[i] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(xsrc, c < a.C ? x_voff : kOob, x_soff + static_cast<uint32_t>(c * a.xs_c * 4), 0));
                 }
+                if (round < a_rounds && ax < a_vecs) {  // (vectors behind np: the zeros the loads returned)
+                    float *dst = gy + 4 * ax;
 #pragma unroll
-                for (int i = 0; i < kBatchA; ++i)
-                    if (la[i] >= 0) *reinterpret_cast<f32x4 *>(gy + la[i]) = da[i];
+                    for (int i = 0; i < kBatchA; ++i) {
+                        const int o = o0 + i * kWaves;
+                        if (o < a.O) *reinterpret_cast<f32x4 *>(dst + o * pitch_a) = da[i];
+                    }
+                }
+                if (x_in) {
+                    float *dst = patch + rg * a.rows_per_load * pitch + x_lane_lds;
 #pragma unroll
-                for (int i = 0; i < kBatchX; ++i) {
-                    if (lx[i] >= 0) {
-                        float *dst = patch + lx[i];
+                    for (int i = 0; i < kBatchX; ++i) {
+                        const int c = c0 + i * kWaves;
+                        if (c < a.C) {
 #pragma unroll
-                        for (int e = 0; e < 4; ++e) dst[e] = dx[i][e];  // (the plane pitch is odd: no 16-byte alignment here)
+                            for (int e = 0; e < 4; ++e) dst[c * plane + e] = dx[i][e];  // (the plane pitch is odd: no 16-byte alignment here)
+                        }
                     }
                 }
             }
@@ -127,7 +157,7 @@ __global__ void __launch_bounds__(kThreads, 1) conv_wgrad_patch_kernel(ConvWgrad
         __syncthreads();
 
         // ---- multiply: chunks of 8 positions; lane (li, kg) takes positions 8 ch + 4 kg .. + 3 of the chunk
-        if (nb > 0) {
+        {
             const int chunks = (np + 7) / 8;
             const int last_off = (rows - 1) * pitch + Wo - 4;  // patch offset of the stage's last four positions
             int x = 4 * kg, off = 4 * kg, pos = 4 * kg;        // this lane's column, patch offset and position in the current chunk
@@ -150,11 +180,12 @@ __global__ void __launch_bounds__(kThreads, 1) conv_wgrad_patch_kernel(ConvWgrad
                 off += wrap ? 8 + pitch - Wo : 8;
             };
             auto multiply = [&](const f32x4 &fa, const float(&fb)[NB][4]) {
+                // (a wave with fewer than NB blocks multiplies its first block again in the spare slots and drops the
+                // result: the workgroup is as slow as its busiest wave either way, and the loop stays one basic block)
 #pragma unroll
                 for (int i = 0; i < NB; ++i)
-                    if (i < nb)  // uniform
 #pragma unroll
-                        for (int t = 0; t < 4; ++t) acc[i] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[t], fb[i][t], acc[i], 0, 0, 0);
+                    for (int t = 0; t < 4; ++t) acc[i] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[t], fb[i][t], acc[i], 0, 0, 0);
             };
             f32x4 fa0, fa1;
             float fb0[NB][4], fb1[NB][4];
@@ -163,8 +194,10 @@ __global__ void __launch_bounds__(kThreads, 1) conv_wgrad_patch_kernel(ConvWgrad
             for (; ch + 1 < chunks; ch += 2) {
                 fetch(ch + 1, fa1, fb1);
                 multiply(fa0, fb0);
+                interleave_reads<4 * NB>();
                 fetch(ch + 2 < chunks ? ch + 2 : chunks - 1, fa0, fb0);  // (past the end: fetched and not used)
                 multiply(fa1, fb1);
+                interleave_reads<4 * NB>();
             }
             if (ch < chunks) multiply(fa0, fb0);
         }
@@ -186,11 +219,9 @@ __global__ void __launch_bounds__(kThreads, 1) conv_wgrad_patch_kernel(ConvWgrad
     }
     __syncthreads();
     float *const out = a.partial + static_cast<int64_t>(blockIdx.x) * a.O * K;
-    for (int v = tid; v < a.O * (K / 4); v += kThreads) {
-        uint32_t o, x;
-        a.d_kvecs.divmod(static_cast<uint32_t>(v), o, x);
-        *reinterpret_cast<f32x4 *>(out + static_cast<int64_t>(o) * K + 4 * x) = *reinterpret_cast<const f32x4 *>(tile + static_cast<int>(o) * tp + 4 * static_cast<int>(x));
-    }
+    for (int o = wave; o < a.O; o += kWaves)  // a row per wave and step, 64 vectors per instruction
+        for (int x = lane; x < K / 4; x += 64)
+            *reinterpret_cast<f32x4 *>(out + static_cast<int64_t>(o) * K + 4 * x) = *reinterpret_cast<const f32x4 *>(tile + o * tp + 4 * x);
 }
 
 }  // namespace
@@ -201,7 +232,7 @@ __global__ void __launch_bounds__(kThreads, 1) conv_wgrad_patch_kernel(ConvWgrad
 ConvWgradPatchPlan plan_conv_wgrad_patch(int B, int C, int H, int W, int O, int k, int S, int P) {
     ConvWgradPatchPlan pl{};
     const int Ho = H + 2 * P - k + 1, Wo = W + 2 * P - k + 1;
-    if (S != 1 || B <= 0 || k < 1 || P >= k || C % 32 != 0 || O % 32 != 0 || W % 4 != 0 || Ho < 1 || Wo < 8 || Wo % 4 != 0) return pl;
+    if (S != 1 || B <= 0 || k < 1 || P >= k || C % 32 != 0 || O % 32 != 0 || W % 4 != 0 || W > 256 || Ho < 1 || Wo < 8 || Wo % 4 != 0) return pl;
     const int n_ob = O / 32;
     if (n_ob != 1 && n_ob != 2 && n_ob != 4) return pl;
     const int waves_per_ob = kWaves / n_ob;
@@ -267,10 +298,8 @@ ttamd_status launch_conv_wgrad_patch_f32(ConvWgradPatchArgs a, const ConvWgradPa
     a.d_P = make_fastdiv(static_cast<uint32_t>(a.P > 0 ? a.P : 1));
     a.d_R = make_fastdiv(static_cast<uint32_t>(a.R));
     a.d_spi = make_fastdiv(static_cast<uint32_t>(a.SPI));
-    a.d_avecs = make_fastdiv(static_cast<uint32_t>(a.pitch_a / 4));
-    a.d_xvecs = make_fastdiv(static_cast<uint32_t>(a.R * (a.W / 4)));
+    a.rows_per_load = 64 / (a.W / 4);  // input rows one load instruction of a wave covers
     a.d_vw = make_fastdiv(static_cast<uint32_t>(a.W / 4));
-    a.d_kvecs = make_fastdiv(static_cast<uint32_t>(a.C * k * k / 4));
     auto go = [&](auto kernel) -> ttamd_status {
         TTAMD_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(pl.lds_bytes)));
         kernel<<<dim3(static_cast<unsigned>(pl.workgroups)), dim3(kThreads), pl.lds_bytes, st>>>(a);
