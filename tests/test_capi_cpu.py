@@ -61,12 +61,14 @@ def test_validation_without_gpu(tt):
     sz = C.c_size_t(1)
     assert lib.ttamd_conv2d_backward_workspace(capi.I32, 4, 3, 8, 8, 4, 3, 1, 0, C.byref(sz)) == capi.ERR_UNSUPPORTED_DTYPE
     assert lib.ttamd_conv2d_backward_workspace(capi.F32, 64, 32, 28, 28, 64, 3, 1, 1, C.byref(sz)) == capi.OK
-    # the transposed weight, one partial grad_weight tile per workgroup of the LDS-staged kernel (256: a quarter image
-    # each), 256 rows of grad_bias sums
+    # the transposed weight, one partial grad_weight tile per (image, half of the positions), 256 rows of grad_bias sums
     tile = 64 * 32 * 9 * 4
-    assert sz.value == tile + 256 * tile + 256 * 64 * 4
-    # one image: a workgroup (and a partial tile) per output row
-    assert lib.ttamd_conv2d_backward_workspace(capi.F32, 1, 32, 28, 28, 64, 3, 1, 1, C.byref(sz)) == capi.OK and sz.value == tile + 28 * tile + 256 * 64 * 4
+    assert sz.value == tile + 128 * tile + 256 * 64 * 4
+    assert lib.ttamd_conv2d_backward_workspace(capi.F32, 1, 32, 28, 28, 64, 3, 1, 1, C.byref(sz)) == capi.OK and sz.value == tile + 5 * tile + 256 * 64 * 4
+    # 32 output channels: grad_weight by the kernel that stages both operands in LDS, one partial tile per workgroup
+    # (256 workgroups of a quarter image each)
+    half = 32 * 32 * 9 * 4
+    assert lib.ttamd_conv2d_backward_workspace(capi.F32, 64, 32, 28, 28, 32, 3, 1, 1, C.byref(sz)) == capi.OK and sz.value == half + 256 * half + 256 * 32 * 4
     assert lib.ttamd_conv2d_backward_workspace(capi.F64, 1, 3, 8, 8, 5, 3, 1, 1, C.byref(sz)) == capi.OK
     assert sz.value == 1280 + 256 * 5 * 8  # 5*3*9*8 = 1080 bytes rounded up to 256, plus the grad_bias sums
 

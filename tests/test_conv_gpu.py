@@ -135,6 +135,34 @@ def test_lds_resident_kernel_exact(tt, oracle, geom):
     assert np.array_equal(gx.to_numpy(), wx) and np.array_equal(gw.to_numpy(), ww) and np.array_equal(gb.to_numpy(), wb)
 
 
+@pytest.mark.parametrize("geom", [
+    # fp32, unit stride, 32 output channels, input channels 32 n, rows of whole vectors with at least 8 outputs:
+    # grad_weight by the kernel that stages grad_out's and the input's rows in LDS.  B, C, H, W, k, P
+    (3, 32, 28, 28, 3, 1),     # 9 blocks of 32 x 32 over the four waves (3, 3, 3, 0)
+    (2, 64, 12, 16, 3, 1),     # 18 blocks (5, 5, 5, 3)
+    (5, 32, 9, 12, 1, 0),      # 1 x 1: one block, three idle waves
+    (2, 32, 20, 20, 5, 2),     # 5 x 5 taps: 25 blocks is more than a wave's five -> the implicit-GEMM kernel
+    (2, 32, 10, 12, 3, 0),     # no padding (Wo = 10: not whole vectors -> the implicit-GEMM kernel)
+    (300, 32, 8, 8, 3, 1),     # more units than workgroups: several stages per workgroup, added up in registers
+    (7, 32, 11, 16, 3, 1),     # units of unequal height (the last unit of an image is short), a ragged last chunk
+    (2, 32, 6, 44, 3, 1),      # wide rows: 11 vectors per row, 5 input rows per load instruction
+])
+def test_lds_staged_grad_weight_exact(tt, oracle, geom):
+    Bn, Cc, H, W, k, P = geom
+    O = 32
+    rng = np.random.default_rng(sum(geom))
+    x = rng.integers(-3, 4, (Bn, Cc, H, W)).astype(np.float32)
+    w = rng.integers(-3, 4, (O, Cc, k, k)).astype(np.float32)
+    Ho, Wo = H + 2 * P - k + 1, W + 2 * P - k + 1
+    g = rng.integers(-3, 4, (Bn, O, Ho, Wo)).astype(np.float32)
+    gx, gw, gb = tt.conv2d_backward(dev(tt, g), dev(tt, x), dev(tt, w), dev(tt, np.zeros(O, np.float32)), 1, P)
+    staged = Wo % 4 == 0 and Wo >= 8 and k * k * (Cc // 32) <= 20
+    assert (_last_kernel(2) == 0x200) == staged, hex(_last_kernel(2))
+    wx, ww, wb = oracle.conv2d_backward(g, x, w, True, 1, P)
+    assert np.array_equal(gw.to_numpy(), ww)
+    assert np.array_equal(gx.to_numpy(), wx) and np.array_equal(gb.to_numpy(), wb)
+
+
 def test_lds_resident_kernel_on_views(tt, oracle):
     # an input window of a larger tensor (row stride 16, 16-byte aligned start) and, through the C ABI, a weight whose
     # output-channel stride is larger than C k k (the row-wise weight loads)

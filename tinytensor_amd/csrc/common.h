@@ -127,8 +127,9 @@ ttamd_status launch_conv_patch_f32(ConvPatchArgs a, hipStream_t stream, int *var
 // grad_weight with both operands staged in LDS (conv_wgrad_patch.hip).  The plan depends on the shape alone.
 struct ConvWgradPatchPlan {
     bool use;
-    int RS, SPI;          // output rows per stage, stages per image
-    int n_stages;         // B * SPI
+    int RS, SPI;          // output rows per unit, units per image
+    int RSS, n_sub;       // a unit is cut into n_sub stages of RSS rows
+    int n_units;          // B * SPI
     int workgroups;       // = partial tiles written
     int blocks_per_wave;
     size_t lds_bytes;
@@ -143,8 +144,8 @@ struct ConvWgradPatchArgs {
     int32_t xs_c, xs_h;
     int64_t image_bytes;   // bytes reachable from an image's first element
     // derived
-    int RS, SPI, n_stages, R, pitch, plane, pitch_a, waves_per_ob, col_blocks, blocks_per_wave, rows_per_load;
-    FastDiv d_cblocks, d_k, d_2P, d_P, d_R, d_spi, d_vw;
+    int RS, SPI, RSS, n_sub, n_units, R, pitch, plane, pitch_a, waves_per_ob, col_blocks, blocks_per_wave;
+    FastDiv d_cblocks, d_k, d_2P, d_P, d_R, d_C, d_spi, d_vw;
 };
 ttamd_status launch_conv_wgrad_patch_f32(ConvWgradPatchArgs a, const ConvWgradPatchPlan &plan, hipStream_t stream, bool *handled);
 

@@ -35,33 +35,34 @@ __device__ __forceinline__ void interleave_reads() {
 
 constexpr int kMaxBlocks = 5;        // 32 x 32 result blocks per wave (80 accumulator registers)
 constexpr int kLdsBytes = 160 * 1024;
-constexpr int kBatchA = 16, kBatchX = 8;  // 16-byte loads per lane and round of the staging: grad_out rows, input rows
+constexpr int kBatchA = 16, kBatchX = 16;  // most 16-byte loads per lane and stage: grad_out rows, input channels (O, C <= 64)
 
 // NB: blocks per wave compiled for (the wave's actual count may be lower).
 template <int NB>
 __global__ void __launch_bounds__(kThreads, 1) conv_wgrad_patch_kernel(ConvWgradPatchArgs a) {
     extern __shared__ __attribute__((aligned(16))) float smem_wg[];
-    float *const gy = smem_wg;                      // [O][pitch_a]: grad_out rows of the stage
-    float *const patch = smem_wg + a.O * a.pitch_a;  // [C][plane]: input rows of the stage, halo columns zero
+    // two stage buffers, each [O][pitch_a] grad_out rows + [C][plane] input rows (halo columns zero)
+    const int buf_floats = a.O * a.pitch_a + a.C * a.plane;
     const int tid = threadIdx.x, lane = tid % 64;
     const int wave = __builtin_amdgcn_readfirstlane(tid / 64);
     const int li = lane % 32, kg = lane / 32;
     const int Wo = a.Wo, pitch = a.pitch, plane = a.plane, pitch_a = a.pitch_a;
     const int K = a.C * a.k * a.k;
+    const int HoWo = a.Ho * Wo;
 
     // this wave's blocks: output-channel block ob, column blocks first .. first + nb - 1 (column block = tap * C/32 + cb)
     const int ob = wave / a.waves_per_ob;
     const int first = (wave % a.waves_per_ob) * a.blocks_per_wave;
     int nb = a.col_blocks - first;
     nb = nb < 0 ? 0 : (nb > a.blocks_per_wave ? a.blocks_per_wave : nb);
-    int block_base[NB];  // float offset in the patch of (channel of this lane, tap) for position 0
-    int block_col[NB];   // first result column (c k k + tap) of the block's channel 0 ... see the store
+    int block_base[NB];  // float offset in a patch of (channel of this lane, tap) for position 0
+    int block_col[NB];   // result column (c k k + tap) of the block's channel 0
 #pragma unroll
     for (int i = 0; i < NB; ++i) {
         uint32_t tap, cb, p, q;
         a.d_cblocks.divmod(static_cast<uint32_t>(first + (i < nb ? i : 0)), tap, cb);
         a.d_k.divmod(tap, p, q);
-        block_base[i] = (static_cast<int>(cb) * 32 + li) * plane + static_cast<int>(p) * pitch + static_cast<int>(q);
+        block_base[i] = a.O * pitch_a + (static_cast<int>(cb) * 32 + li) * plane + static_cast<int>(p) * pitch + static_cast<int>(q);
         block_col[i] = static_cast<int>(cb) * 32 * a.k * a.k + static_cast<int>(tap);
     }
     f32x16 acc[NB];
@@ -70,94 +71,104 @@ __global__ void __launch_bounds__(kThreads, 1) conv_wgrad_patch_kernel(ConvWgrad
 #pragma unroll
         for (int e = 0; e < 16; ++e) acc[i][e] = 0.f;
 
-    // halo columns of the patch: zero for the whole kernel (the staging below never writes them)
-    for (int v = tid; v < a.C * a.R * 2 * a.P; v += kThreads) {
-        uint32_t row, sp, side, pc;
-        a.d_2P.divmod(static_cast<uint32_t>(v), row, sp);  // row = c * R + r
+    // halo columns of both patches: zero for the whole kernel (the staging below never writes them)
+    for (int v = tid; v < 2 * a.C * a.R * 2 * a.P; v += kThreads) {
+        uint32_t row, sp, side, pc, bc, r, bf, c;
+        a.d_2P.divmod(static_cast<uint32_t>(v), row, sp);  // row = (buffer * C + c) * R + r
         a.d_P.divmod(sp, side, pc);
-        uint32_t c, r;
-        a.d_R.divmod(row, c, r);
-        patch[static_cast<int>(c) * plane + static_cast<int>(r) * pitch + (side ? a.P + a.W + static_cast<int>(pc) : static_cast<int>(pc))] = 0.f;
+        a.d_R.divmod(row, bc, r);
+        a.d_C.divmod(bc, bf, c);
+        smem_wg[static_cast<int>(bf) * buf_floats + a.O * pitch_a + static_cast<int>(c) * plane + static_cast<int>(r) * pitch +
+                (side ? a.P + a.W + static_cast<int>(pc) : static_cast<int>(pc))] = 0.f;
     }
 
-    // the lane's part of an input load: row x_lane_r of the item's row group, vector x_lane_v of that row
+    // The lane's part of the staging: vector `lane` of a grad_out row (an instruction of a wave loads one row); row
+    // x_lane_r, vector x_lane_v of a channel's patch (an instruction loads a channel's R rows).  Which row or channel
+    // is wave-uniform and rides in the load's scalar offset.
+    const int a_vecs = pitch_a / 4;  // 16-byte vectors per staged grad_out row (behind the stage's positions: zeros)
     uint32_t xr, xv;
     a.d_vw.divmod(static_cast<uint32_t>(lane), xr, xv);
     const int x_lane_r = static_cast<int>(xr);
-    const bool x_lane_ok = x_lane_r < a.rows_per_load;
+    const bool x_lane_ok = x_lane_r < a.R;
     const uint32_t x_lane_goff = static_cast<uint32_t>((x_lane_r * a.xs_h + 4 * static_cast<int>(xv)) * 4);
-    const int x_lane_lds = x_lane_r * pitch + a.P + 4 * static_cast<int>(xv);
-    const int a_vecs = pitch_a / 4;            // 16-byte vectors per staged grad_out row (the tail beyond the stage: zeros)
-    const int HoWo = a.Ho * Wo;
-    const float *const ap = gy + (ob * 32 + li) * pitch_a + 4 * kg;
+    const int x_lane_lds = a.O * pitch_a + x_lane_r * pitch + a.P + 4 * static_cast<int>(xv);
 
-    for (int s = blockIdx.x; s < a.n_stages; s += gridDim.x) {
-        uint32_t b, si;
-        a.d_spi.divmod(static_cast<uint32_t>(s), b, si);
-        const int r0 = static_cast<int>(si) * a.RS;
-        const int rows = a.Ho - r0 < a.RS ? a.Ho - r0 : a.RS;
-        const int np = rows * Wo;  // positions of this stage (a multiple of 4)
-        // ---- stage: grad_out rows [O][np] (zeros behind np), input rows r0 - P .. r0 - P + R - 1 of every channel
-        {
-            // Row-wise: an instruction of a wave loads 64 vectors of one grad_out row, or rows_per_load input rows of
-            // one channel; which row or channel is wave-uniform and rides in the load's scalar offset, the lane's part
-            // of the address is fixed for the whole kernel.  All loads of a round are issued before its first LDS
-            // write, so a round costs one memory latency.
-            const float *gbase = a.gout + (static_cast<int64_t>(b) * a.O) * HoWo + static_cast<int64_t>(r0) * Wo;
-            const __amdgpu_buffer_rsrc_t gsrc = make_rsrc(gbase, (static_cast<int64_t>(a.O) * HoWo - static_cast<int64_t>(r0) * Wo) * 4);
-            const int y0 = r0 - a.P;
-            const int64_t first_x = static_cast<int64_t>(b) * a.xs_b + static_cast<int64_t>(y0) * a.xs_h;
-            const __amdgpu_buffer_rsrc_t xsrc = make_rsrc(a.x + first_x, a.image_bytes - static_cast<int64_t>(y0) * a.xs_h * 4);
-            // grad_out: wave w loads rows w, w + 4, ... (64 vectors of a row per instruction); input: channels w, w + 4,
-            // ... (rows_per_load patch rows per instruction).  The usual stage is one round of each.
-            const int a_groups = (a_vecs + 63) / 64, x_groups = (a.R + a.rows_per_load - 1) / a.rows_per_load;
-            const int a_rounds = (a.O + kWaves * kBatchA - 1) / (kWaves * kBatchA) * a_groups;
-            const int x_rounds = (a.C + kWaves * kBatchX - 1) / (kWaves * kBatchX) * x_groups;
-            for (int round = 0; round < a_rounds || round < x_rounds; ++round) {
-                f32x4 da[kBatchA], dx[kBatchX];
-                const int vg = round % a_groups, o0 = wave + (round / a_groups) * (kWaves * kBatchA);
-                const int rg = round % x_groups, c0 = wave + (round / x_groups) * (kWaves * kBatchX);
-                const int ax = vg * 64 + lane;                              // this lane's vector of a grad_out row
-                const int xr = x_lane_r + rg * a.rows_per_load;             // this lane's patch row
-                const uint32_t a_voff = round < a_rounds && 4 * ax < np ? static_cast<uint32_t>(ax) * 16u : kOob;
-                const bool x_in = round < x_rounds && x_lane_ok && xr < a.R;
-                const uint32_t x_voff = x_in && static_cast<unsigned>(y0 + xr) < static_cast<unsigned>(a.H) ? x_lane_goff : kOob;
-                const uint32_t x_soff = static_cast<uint32_t>(rg * a.rows_per_load * a.xs_h * 4);
+    // This workgroup's stages: units blockIdx.x, blockIdx.x + gridDim.x, ... (a unit: RS output rows of one image),
+    // each cut into n_sub stages of RSS rows; stage t + 1 is loaded while stage t is multiplied.
+    const int n_units = (a.n_units - static_cast<int>(blockIdx.x) + static_cast<int>(gridDim.x) - 1) / static_cast<int>(gridDim.x);
+    const int n_t = n_units * a.n_sub;
+    auto stage_at = [&](int t, int &b, int &r0, int &rows) {
+        const int j = t / a.n_sub, sub = t - j * a.n_sub;  // (n_sub is 1 or 2)
+        uint32_t bi, si;
+        a.d_spi.divmod(static_cast<uint32_t>(static_cast<int>(blockIdx.x) + j * static_cast<int>(gridDim.x)), bi, si);
+        const int ur0 = static_cast<int>(si) * a.RS;
+        const int urows = a.Ho - ur0 < a.RS ? a.Ho - ur0 : a.RS;
+        b = static_cast<int>(bi);
+        r0 = ur0 + sub * a.RSS;
+        rows = urows - sub * a.RSS;
+        rows = rows < 0 ? 0 : (rows > a.RSS ? a.RSS : rows);
+    };
+    f32x4 da[kBatchA], dx[kBatchX];
+    auto request = [&](int t) {  // global -> registers: all loads of a stage in flight together
+        int b, r0, rows;
+        stage_at(t, b, r0, rows);
+        const int np = rows * Wo;
+        const float *gbase = a.gout + (static_cast<int64_t>(b) * a.O) * HoWo + static_cast<int64_t>(r0) * Wo;
+        const __amdgpu_buffer_rsrc_t gsrc = make_rsrc(gbase, (static_cast<int64_t>(a.O) * HoWo - static_cast<int64_t>(r0) * Wo) * 4);
+        const int y0 = r0 - a.P;
+        const int64_t first_x = static_cast<int64_t>(b) * a.xs_b + static_cast<int64_t>(y0) * a.xs_h;
+        const __amdgpu_buffer_rsrc_t xsrc = make_rsrc(a.x + first_x, a.image_bytes - static_cast<int64_t>(y0) * a.xs_h * 4);
+        const uint32_t a_voff = 4 * lane < np ? static_cast<uint32_t>(lane) * 16u : kOob;
+        const uint32_t x_voff = x_lane_ok && static_cast<unsigned>(y0 + x_lane_r) < static_cast<unsigned>(a.H) ? x_lane_goff : kOob;
 #pragma unroll
-                for (int i = 0; i < kBatchA; ++i) {
-                    const int o = o0 + i * kWaves;
-                    da[i] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(gsrc, o < a.O ? a_voff : kOob, static_cast<uint32_t>(o) * static_cast<uint32_t>(HoWo) * 4u, 0));
-                }
+        for (int i = 0; i < kBatchA; ++i) {
+            const int o = wave + i * kWaves;
+            da[i] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(gsrc, o < a.O ? a_voff : kOob, static_cast<uint32_t>(o) * static_cast<uint32_t>(HoWo) * 4u, 0));
+        }
 #pragma unroll
-                for (int i = 0; i < kBatchX; ++i) {
-                    const int c = c0 + i * kWaves;
-                    dx[i] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(xsrc, c < a.C ? x_voff : kOob, x_soff + static_cast<uint32_t>(c * a.xs_c * 4), 0));
-                }
-                if (round < a_rounds && ax < a_vecs) {  // (vectors behind np: the zeros the loads returned)
-                    float *dst = gy + 4 * ax;
+        for (int i = 0; i < kBatchX; ++i) {
+            const int c = wave + i * kWaves;
+            dx[i] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(xsrc, c < a.C ? x_voff : kOob, static_cast<uint32_t>(c * a.xs_c * 4), 0));
+        }
+    };
+    auto park = [&](int buf) {  // registers -> stage buffer `buf`
+        float *base = smem_wg + buf * buf_floats;
+        if (lane < a_vecs) {  // (vectors behind the stage's positions: the zeros the loads returned)
+            float *dst = base + 4 * lane;
 #pragma unroll
-                    for (int i = 0; i < kBatchA; ++i) {
-                        const int o = o0 + i * kWaves;
-                        if (o < a.O) *reinterpret_cast<f32x4 *>(dst + o * pitch_a) = da[i];
-                    }
-                }
-                if (x_in) {
-                    float *dst = patch + rg * a.rows_per_load * pitch + x_lane_lds;
+            for (int i = 0; i < kBatchA; ++i) {
+                const int o = wave + i * kWaves;
+                if (o < a.O) *reinterpret_cast<f32x4 *>(dst + o * pitch_a) = da[i];
+            }
+        }
+        if (x_lane_ok) {
+            float *dst = base + x_lane_lds;
 #pragma unroll
-                    for (int i = 0; i < kBatchX; ++i) {
-                        const int c = c0 + i * kWaves;
-                        if (c < a.C) {
+            for (int i = 0; i < kBatchX; ++i) {
+                const int c = wave + i * kWaves;
+                if (c < a.C) {
 #pragma unroll
-                            for (int e = 0; e < 4; ++e) dst[c * plane + e] = dx[i][e];  // (the plane pitch is odd: no 16-byte alignment here)
-                        }
-                    }
+                    for (int e = 0; e < 4; ++e) dst[c * plane + e] = dx[i][e];  // (the plane pitch is odd: no 16-byte alignment here)
                 }
             }
         }
-        __syncthreads();
+    };
 
+    if (n_t > 0) {
+        request(0);
+        park(0);
+    }
+    __syncthreads();
+    for (int t = 0; t < n_t; ++t) {
+        const int cur = t & 1;
+        if (t + 1 < n_t) request(t + 1);
+        int b_, r0_, rows;
+        stage_at(t, b_, r0_, rows);
+        const int np = rows * Wo;  // positions of this stage (a multiple of 4)
         // ---- multiply: chunks of 8 positions; lane (li, kg) takes positions 8 ch + 4 kg .. + 3 of the chunk
         {
+            const float *const stage = smem_wg + cur * buf_floats;
+            const float *const ap = stage + (ob * 32 + li) * pitch_a + 4 * kg;
             const int chunks = (np + 7) / 8;
             const int last_off = (rows - 1) * pitch + Wo - 4;  // patch offset of the stage's last four positions
             int x = 4 * kg, off = 4 * kg, pos = 4 * kg;        // this lane's column, patch offset and position in the current chunk
@@ -168,9 +179,9 @@ __global__ void __launch_bounds__(kThreads, 1) conv_wgrad_patch_kernel(ConvWgrad
                 const int o = pos < np ? off : last_off;
 #pragma unroll
                 for (int i = 0; i < NB; ++i) {
-                    const float *bp = patch + block_base[i] + o;
+                    const float *bp = stage + block_base[i] + o;
 #pragma unroll
-                    for (int t = 0; t < 4; ++t) fb[i][t] = bp[t];
+                    for (int t4 = 0; t4 < 4; ++t4) fb[i][t4] = bp[t4];
                 }
                 // next chunk: 8 positions on, wrapping into the next row (Wo >= 8: at most one wrap)
                 pos += 8;
@@ -185,23 +196,26 @@ __global__ void __launch_bounds__(kThreads, 1) conv_wgrad_patch_kernel(ConvWgrad
 #pragma unroll
                 for (int i = 0; i < NB; ++i)
 #pragma unroll
-                    for (int t = 0; t < 4; ++t) acc[i] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[t], fb[i][t], acc[i], 0, 0, 0);
+                    for (int t4 = 0; t4 < 4; ++t4) acc[i] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[t4], fb[i][t4], acc[i], 0, 0, 0);
             };
-            f32x4 fa0, fa1;
-            float fb0[NB][4], fb1[NB][4];
-            fetch(0, fa0, fb0);
-            int ch = 0;
-            for (; ch + 1 < chunks; ch += 2) {
-                fetch(ch + 1, fa1, fb1);
-                multiply(fa0, fb0);
-                interleave_reads<4 * NB>();
-                fetch(ch + 2 < chunks ? ch + 2 : chunks - 1, fa0, fb0);  // (past the end: fetched and not used)
-                multiply(fa1, fb1);
-                interleave_reads<4 * NB>();
+            if (chunks > 0) {
+                f32x4 fa0, fa1;
+                float fb0[NB][4], fb1[NB][4];
+                fetch(0, fa0, fb0);
+                int ch = 0;
+                for (; ch + 1 < chunks; ch += 2) {
+                    fetch(ch + 1, fa1, fb1);
+                    multiply(fa0, fb0);
+                    interleave_reads<4 * NB>();
+                    fetch(ch + 2 < chunks ? ch + 2 : chunks - 1, fa0, fb0);  // (past the end: fetched and not used)
+                    multiply(fa1, fb1);
+                    interleave_reads<4 * NB>();
+                }
+                if (ch < chunks) multiply(fa0, fb0);
             }
-            if (ch < chunks) multiply(fa0, fb0);
         }
-        __syncthreads();  // every wave has left the stage's buffers
+        if (t + 1 < n_t) park(cur ^ 1);  // (the other buffer: last read before the previous barrier)
+        __syncthreads();
     }
 
     // ---- partial tile of this workgroup, [O][C k k] as grad_weight is laid out: through LDS, so that the copy to
@@ -232,41 +246,54 @@ __global__ void __launch_bounds__(kThreads, 1) conv_wgrad_patch_kernel(ConvWgrad
 ConvWgradPatchPlan plan_conv_wgrad_patch(int B, int C, int H, int W, int O, int k, int S, int P) {
     ConvWgradPatchPlan pl{};
     const int Ho = H + 2 * P - k + 1, Wo = W + 2 * P - k + 1;
-    if (S != 1 || B <= 0 || k < 1 || P >= k || C % 32 != 0 || O % 32 != 0 || W % 4 != 0 || W > 256 || Ho < 1 || Wo < 8 || Wo % 4 != 0) return pl;
+    // (Output-channel counts above 32: measured on a par with the implicit-GEMM kernel, whose 64-row tile is full there
+    // -- 30.0 + 5.8 us against 31.1 + 4.7 us for [64,32,28,28] x [64,32,3,3] -- so that one keeps them.)
+    if (S != 1 || B <= 0 || k < 1 || P >= k || C % 32 != 0 || O != 32 || W % 4 != 0 || W > 256 || Ho < 1 || Wo < 8 || Wo % 4 != 0) return pl;
     const int n_ob = O / 32;
     if (n_ob != 1 && n_ob != 2 && n_ob != 4) return pl;
     const int waves_per_ob = kWaves / n_ob;
     const int col_blocks = k * k * (C / 32);
     const int blocks_per_wave = (col_blocks + waves_per_ob - 1) / waves_per_ob;
     if (blocks_per_wave > kMaxBlocks) return pl;
+    if (O > kWaves * kBatchA || C > kWaves * kBatchX) return pl;  // a wave stages O / 4 rows and C / 4 channels per stage
     const int pitch = W + 2 * P;
     const int64_t K = static_cast<int64_t>(C) * k * k;
-    auto lds_floats = [&](int rs) {
-        const int64_t pitch_a = 4 * ((((static_cast<int64_t>(rs) * Wo + 7) / 8 * 8) / 4) | 1);  // whole chunks, 4 (2 n + 1) floats
-        const int64_t plane = (static_cast<int64_t>(rs + k - 1) * pitch) | 1;
-        const int64_t stage = O * pitch_a + C * plane;
-        const int64_t tile = O * (K + 4);
-        return stage > tile ? stage : tile;
+    const int64_t tile = O * (K + 4);
+    if (tile * 4 > kLdsBytes) return pl;
+    // a stage of rss output rows: floats of one stage buffer, or 0 when a wave's load instructions do not cover it
+    auto stage_floats = [&](int rss) -> int64_t {
+        const int64_t pitch_a = 4 * ((((static_cast<int64_t>(rss) * Wo + 7) / 8 * 8) / 4) | 1);  // whole chunks, 4 (2 n + 1) floats
+        if (pitch_a / 4 > 64 || rss + k - 1 > 64 / (W / 4)) return 0;  // one instruction per grad_out row / per channel
+        const int64_t plane = (static_cast<int64_t>(rss + k - 1) * pitch) | 1;
+        return O * pitch_a + C * plane;
     };
-    int rs_max = 0;
-    for (int rs = 1; rs <= Ho; ++rs)
-        if (lds_floats(rs) * 4 <= kLdsBytes) rs_max = rs;
-    if (rs_max < 1 || static_cast<int64_t>(O) * (K + 4) * 4 > kLdsBytes) return pl;
+    // Units of rs = ceil(Ho / spi) rows, one or more per workgroup: the split that gives the busiest of the 256
+    // workgroups the least to do.  A unit is one stage: cutting it into two double-buffered stages was measured and
+    // gains nothing (the loads that arrive during the MFMA loop slow it by as much as the load phase they hide:
+    // 94 against 74 cycles per MFMA), so n_sub stays 1; the kernel keeps the general form.
     int best_spi = 0;
     int64_t best_cost = 0;
-    for (int spi = (Ho + rs_max - 1) / rs_max; spi <= Ho; ++spi) {
+    for (int spi = 1; spi <= Ho; ++spi) {
         const int rs = (Ho + spi - 1) / spi;
-        const int64_t stages = static_cast<int64_t>(B) * spi;
-        const int64_t cost = ((stages + 255) / 256) * (rs * Wo + 64);  // positions of the busiest workgroup, plus a stage's fixed cost
+        if ((Ho + rs - 1) / rs != spi) continue;  // (the same rs as a smaller spi)
+        const int n_sub = 1, rss = (rs + n_sub - 1) / n_sub;
+        const int64_t sf = stage_floats(rss);
+        if (sf == 0 || 2 * sf * 4 > kLdsBytes) continue;
+        const int64_t units = static_cast<int64_t>(B) * spi;
+        const int64_t cost = ((units + 255) / 256) * (static_cast<int64_t>(rs) * Wo + 48 * n_sub + 64);  // positions, plus fixed costs per stage and unit
         if (best_spi == 0 || cost < best_cost) best_spi = spi, best_cost = cost;
     }
+    if (best_spi == 0) return pl;
+    pl.SPI = best_spi;
     pl.RS = (Ho + best_spi - 1) / best_spi;
-    pl.SPI = (Ho + pl.RS - 1) / pl.RS;
-    const int64_t stages = static_cast<int64_t>(B) * pl.SPI;
-    if (stages > 0x7fffffff) return pl;
-    pl.n_stages = static_cast<int>(stages);
-    pl.workgroups = stages < 256 ? pl.n_stages : 256;
-    pl.lds_bytes = static_cast<size_t>(lds_floats(pl.RS)) * 4;
+    pl.n_sub = 1;
+    pl.RSS = (pl.RS + pl.n_sub - 1) / pl.n_sub;
+    const int64_t units = static_cast<int64_t>(B) * pl.SPI;
+    if (units > 0x7fffffff) return pl;
+    pl.n_units = static_cast<int>(units);
+    pl.workgroups = units < 256 ? pl.n_units : 256;
+    const int64_t lds_floats = 2 * stage_floats(pl.RSS) > tile ? 2 * stage_floats(pl.RSS) : tile;
+    pl.lds_bytes = static_cast<size_t>(lds_floats) * 4;
     pl.blocks_per_wave = blocks_per_wave;
     pl.use = true;
     return pl;
@@ -284,11 +311,13 @@ ttamd_status launch_conv_wgrad_patch_f32(ConvWgradPatchArgs a, const ConvWgradPa
     if (a.O * HoWo * 4 >= 0x7fffffff || static_cast<int64_t>(a.C) * a.xs_c * 4 + static_cast<int64_t>(a.H + 2 * k) * a.xs_h * 4 >= 0x7fffffff) return TTAMD_OK;
     a.RS = pl.RS;
     a.SPI = pl.SPI;
-    a.n_stages = pl.n_stages;
-    a.R = a.RS + k - 1;
+    a.RSS = pl.RSS;
+    a.n_sub = pl.n_sub;
+    a.n_units = pl.n_units;
+    a.R = a.RSS + k - 1;
     a.pitch = a.W + 2 * a.P;
     a.plane = (a.R * a.pitch) | 1;
-    a.pitch_a = 4 * ((((a.RS * a.Wo + 7) / 8 * 8) / 4) | 1);
+    a.pitch_a = 4 * ((((a.RSS * a.Wo + 7) / 8 * 8) / 4) | 1);
     a.waves_per_ob = kWaves / (a.O / 32);
     a.col_blocks = k * k * (a.C / 32);
     a.blocks_per_wave = pl.blocks_per_wave;
@@ -298,7 +327,7 @@ ttamd_status launch_conv_wgrad_patch_f32(ConvWgradPatchArgs a, const ConvWgradPa
     a.d_P = make_fastdiv(static_cast<uint32_t>(a.P > 0 ? a.P : 1));
     a.d_R = make_fastdiv(static_cast<uint32_t>(a.R));
     a.d_spi = make_fastdiv(static_cast<uint32_t>(a.SPI));
-    a.rows_per_load = 64 / (a.W / 4);  // input rows one load instruction of a wave covers
+    a.d_C = make_fastdiv(static_cast<uint32_t>(a.C));
     a.d_vw = make_fastdiv(static_cast<uint32_t>(a.W / 4));
     auto go = [&](auto kernel) -> ttamd_status {
         TTAMD_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(pl.lds_bytes)));
