@@ -54,10 +54,13 @@ __device__ __forceinline__ void interleave_reads() {
 // CC: chunks of 8 reduction indices (8 channels of one tap) that are read and multiplied as one straight-line group;
 // C / 8 is a multiple of it.
 // MAXS: staging slots (16-byte loads per lane and tile).
-template <int WGM, int WGN, int CC, int MAXS>
-__global__ void __launch_bounds__(64 * WGM * WGN, 1) conv_patch_kernel(ConvPatchArgs a) {
-    constexpr int NW = WGM * WGN, NT = 64 * NW;  // 4 waves (one per SIMD) or 8
+// KS: 1, or 2 sets of WGM x WGN waves that each take half of the reduction groups of the same tile (a second wave per
+// SIMD where a wider tile's patch would not fit in LDS); the upper set hands its accumulators over through LDS.
+template <int WGM, int WGN, int CC, int MAXS, int KS = 1>
+__global__ void __launch_bounds__(64 * WGM * WGN * KS, 1) conv_patch_kernel(ConvPatchArgs a) {
+    constexpr int NW = WGM * WGN * KS, NT = 64 * NW;  // 4 waves (one per SIMD) or 8
     static_assert(NW == 4 || NW == 8, "4 or 8 waves");
+    static_assert(KS == 1 || KS == 2, "one or two halves of the reduction");
     constexpr int WVECS = kWeightLoads / NW;
     constexpr int BM = 32 * WGM, BN = 32 * WGN;
     extern __shared__ __attribute__((aligned(16))) float smem_patch[];
@@ -65,7 +68,8 @@ __global__ void __launch_bounds__(64 * WGM * WGN, 1) conv_patch_kernel(ConvPatch
     float *const patch = smem_patch + BM * a.lda;  // [1 or 2][R][pitch][cpad]
     const int tid = threadIdx.x, lane = tid % 64;
     const int wave = __builtin_amdgcn_readfirstlane(tid / 64);
-    const int wm = wave / WGN, wn = wave % WGN;
+    const int ks = wave / (WGM * WGN), wtile = wave % (WGM * WGN);
+    const int wm = wtile / WGN, wn = wtile % WGN;
     const int li = lane % 32, kg = lane / 32;
     const int C = a.C, K = a.K, pitch = a.pitch, cpad = a.cpad;
     const int patch_elems = a.R * pitch * cpad;
@@ -303,23 +307,43 @@ __global__ void __launch_bounds__(64 * WGM * WGN, 1) conv_patch_kernel(ConvPatch
                 for (int t = 0; t < 4; ++t) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[i][t], fb[i][t], acc, 0, 0, 0);
         };
         f32x4 fa0[CC], fa1[CC], fb0[CC], fb1[CC];
-        if (wave_active) fetch(0, fa0, fb0);
-        int g = wave_active ? 0 : n_groups;
-        for (; g + 1 < n_groups; g += 2) {
+        const int g_end = KS == 1 ? n_groups : (ks + 1) * (n_groups / KS);  // this wave set's share of the groups
+        int g = wave_active ? (KS == 1 ? 0 : ks * (n_groups / KS)) : g_end;
+        if (wave_active) fetch(g, fa0, fb0);
+        for (; g + 1 < g_end; g += 2) {
             fetch(g + 1, fa1, fb1);
             multiply(fa0, fb0);
             interleave_reads<4 * CC>();
-            fetch(g + 2 < n_groups ? g + 2 : n_groups - 1, fa0, fb0);  // (past the end: a harmless repeat)
+            fetch(g + 2 < g_end ? g + 2 : g_end - 1, fa0, fb0);  // (past the end: a harmless repeat)
             multiply(fa1, fb1);
             interleave_reads<4 * CC>();
         }
-        if (g < n_groups) multiply(fa0, fb0);
+        if (g < g_end) multiply(fa0, fb0);
 
-        if (a.n_buf == 1) __syncthreads();  // one patch buffer: every wave has left it
+        if constexpr (KS == 2) {
+            // the upper set's sums go to the lower set through LDS (behind the patch buffers), added as
+            // (lower half of the groups) + (upper half): a fixed order
+            float *const exch = patch + a.n_buf * patch_elems + (wtile * 64 + lane) * 16;
+            if (ks == 1) {
+#pragma unroll
+                for (int e = 0; e < 16; e += 4) *reinterpret_cast<f32x4 *>(exch + e) = f32x4{acc[e], acc[e + 1], acc[e + 2], acc[e + 3]};
+            }
+            __syncthreads();  // (also: every wave has left the patch buffer)
+            if (ks == 0) {
+#pragma unroll
+                for (int e = 0; e < 16; e += 4) {
+                    const f32x4 v = *reinterpret_cast<const f32x4 *>(exch + e);
+#pragma unroll
+                    for (int t = 0; t < 4; ++t) acc[e + t] += v[t];
+                }
+            }
+        } else {
+            if (a.n_buf == 1) __syncthreads();  // one patch buffer: every wave has left it
+        }
         if (jn < n_tiles) park(cur ^ (a.n_buf - 1));  // the loads were issued a whole tile ago
 
         // store: out[b][o][n] (+ bias[o]); positions outside the result are dropped by the buffer store
-        if (wave_active) {
+        if (wave_active && ks == 0) {
             float *ob = a.out + static_cast<int64_t>(b) * a.O * HoWo;
             const __amdgpu_buffer_rsrc_t osrc = make_rsrc(ob, static_cast<int64_t>(a.O) * HoWo * 4);
             if (full_rows) {
@@ -346,7 +370,7 @@ __global__ void __launch_bounds__(64 * WGM * WGN, 1) conv_patch_kernel(ConvPatch
 }
 
 // Derived geometry for tiles of BM x BN computed by `waves` waves; false when this kernel does not apply.
-bool plan_patch(ConvPatchArgs &a, int BM, int BN, int waves, int n_buf, size_t *lds_bytes) {
+bool plan_patch(ConvPatchArgs &a, int BM, int BN, int waves, int n_buf, size_t *lds_bytes, int halves = 1) {
     const int k = a.k, threads = 64 * waves;
     const int HoWo = a.Ho * a.Wo;
     a.K = a.C * k * k;
@@ -365,7 +389,8 @@ bool plan_patch(ConvPatchArgs &a, int BM, int BN, int waves, int n_buf, size_t *
     a.tiles_n = (HoWo + BN - 1) / BN;
     const int64_t patch_elems = static_cast<int64_t>(a.R) * a.pitch * a.cpad;
     a.n_buf = n_buf;
-    int64_t lds_floats = static_cast<int64_t>(BM) * a.lda + n_buf * patch_elems;
+    int64_t lds_floats = static_cast<int64_t>(BM) * a.lda + n_buf * patch_elems + (halves == 2 ? waves / 2 * 64 * 16 : 0);
+    if (halves == 2 && (a.C % 32 != 0 || (static_cast<int64_t>(a.C) / 32 * k * k) % 2 != 0)) return false;  // an even number of 32-channel groups
     if (a.stage_slots > kStageLoads / waves || lds_floats * 4 > kLdsBytes) return false;
     if (static_cast<int64_t>(a.B) * a.tiles_n > 0x7fffffff || static_cast<int64_t>(a.O) * HoWo * 4 >= 0x7fffffff) return false;
     if (static_cast<int64_t>(a.C) * a.xs_c * 4 + static_cast<int64_t>(a.R) * a.xs_h * 4 >= 0x7fffffff) return false;
@@ -400,26 +425,30 @@ bool plan_patch(ConvPatchArgs &a, int BM, int BN, int waves, int n_buf, size_t *
     return true;
 }
 
-template <int WGM, int WGN, int CC, int MAXS>
+template <int WGM, int WGN, int CC, int MAXS, int KS = 1>
 ttamd_status launch_patch(ConvPatchArgs a, hipStream_t st, size_t lds) {
     const int64_t n_tiles = static_cast<int64_t>(a.B) * a.tiles_n;
     int64_t groups = 256 / a.tiles_m;
     if (groups < 1) groups = 1;
     if (groups > n_tiles) groups = n_tiles;
     a.d_ngrp = make_fastdiv(static_cast<uint32_t>(a.C / (8 * CC)));
-    auto kernel = conv_patch_kernel<WGM, WGN, CC, MAXS>;
+    auto kernel = conv_patch_kernel<WGM, WGN, CC, MAXS, KS>;
     TTAMD_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds)));
-    kernel<<<dim3(static_cast<unsigned>(groups * a.tiles_m)), dim3(64 * WGM * WGN), lds, st>>>(a);
+    kernel<<<dim3(static_cast<unsigned>(groups * a.tiles_m)), dim3(64 * WGM * WGN * KS), lds, st>>>(a);
     TTAMD_HIP_CHECK(hipGetLastError());
     return TTAMD_OK;
 }
 
-template <int WGM, int WGN>
+template <int WGM, int WGN, int KS = 1>
 ttamd_status launch_patch_cc(const ConvPatchArgs &a, hipStream_t st, size_t lds) {
-    constexpr int S1 = kStageLoads / (WGM * WGN), S0 = S1 / 2;  // slot counts compiled for
+    constexpr int S1 = kStageLoads / (WGM * WGN * KS), S0 = S1 / 2;  // slot counts compiled for
     const bool few = a.stage_slots <= S0;
-    if (a.C % 32 == 0) return few ? launch_patch<WGM, WGN, 4, S0>(a, st, lds) : launch_patch<WGM, WGN, 4, S1>(a, st, lds);
-    return few ? launch_patch<WGM, WGN, 1, S0>(a, st, lds) : launch_patch<WGM, WGN, 1, S1>(a, st, lds);
+    if constexpr (KS == 2) {  // (only with 32-channel groups, of which each set takes half)
+        return few ? launch_patch<WGM, WGN, 4, S0, 2>(a, st, lds) : launch_patch<WGM, WGN, 4, S1, 2>(a, st, lds);
+    } else {
+        if (a.C % 32 == 0) return few ? launch_patch<WGM, WGN, 4, S0>(a, st, lds) : launch_patch<WGM, WGN, 4, S1>(a, st, lds);
+        return few ? launch_patch<WGM, WGN, 1, S0>(a, st, lds) : launch_patch<WGM, WGN, 1, S1>(a, st, lds);
+    }
 }
 
 }  // namespace
@@ -443,6 +472,11 @@ ttamd_status launch_conv_patch_f32(ConvPatchArgs a, hipStream_t st, int *variant
         if (wide_ok && plan_patch(a, narrow ? 32 : 64, narrow ? 256 : 128, 8, n_buf, &lds)) {
             *variant = 8 * 16 + n_buf;
             return narrow ? launch_patch_cc<1, 8>(a, st, lds) : launch_patch_cc<2, 4>(a, st, lds);
+        }
+        // the four-wave tile with a second set of waves on the other half of the reduction
+        if (wide_ok && plan_patch(a, narrow ? 32 : 64, narrow ? 128 : 64, 8, n_buf, &lds, 2)) {
+            *variant = 8 * 16 + n_buf;
+            return narrow ? launch_patch_cc<1, 4, 2>(a, st, lds) : launch_patch_cc<2, 2, 2>(a, st, lds);
         }
         if (plan_patch(a, narrow ? 32 : 64, narrow ? 128 : 64, 4, n_buf, &lds)) {
             *variant = 4 * 16 + n_buf;
