@@ -331,15 +331,24 @@ __device__ __forceinline__ int remap_xcd(int pid, int total) {
 // Logical workgroup id -> (batch, tile row, tile column); tiles are walked in groups of 8 tile rows so that
 // the workgroups resident on one XCD share operand panels through its L2.
 __device__ __forceinline__ void decode_tile(int pid, int tiles_m, int tiles_n, int &batch, int &tm, int &tn) {
+    // (All values are workgroup-uniform; an integer division is some forty scalar instructions in a kernel's first
+    // microsecond, so the common cases -- one batch item, a full group of eight tile rows -- go without.)
     const int tiles = tiles_m * tiles_n;
-    batch = pid / tiles;
+    batch = pid < tiles ? 0 : pid / tiles;
     pid -= batch * tiles;
     constexpr int GROUP = 8;
     const int group_sz = GROUP * tiles_n;
-    const int first_m = (pid / group_sz) * GROUP;
+    const int group = pid < group_sz ? 0 : pid / group_sz;
+    const int first_m = group * GROUP;
+    const int in_group = pid - group * group_sz;
     const int gm = (tiles_m - first_m) < GROUP ? (tiles_m - first_m) : GROUP;
-    tm = first_m + (pid % group_sz) % gm;
-    tn = (pid % group_sz) / gm;
+    if (gm == GROUP) {
+        tm = first_m + in_group % GROUP;
+        tn = in_group / GROUP;
+    } else {
+        tm = first_m + in_group % gm;
+        tn = in_group / gm;
+    }
 }
 
 // ---------------------------------------------------------------------------------------------
