@@ -78,7 +78,8 @@ def test_store_extension_argument_checks(tt):
 
 
 @pytest.mark.parametrize("dtype", [np.float32, np.float64])
-@pytest.mark.parametrize("shape", [(1024, 10), (7, 3), (50000, 64), (300, 1000), (1, 1), (4096, 33)])
+@pytest.mark.parametrize("shape", [(1024, 10), (7, 3), (50000, 64), (300, 1000), (1, 1), (4096, 33),
+                                   (16384, 1), (16385, 1), (256, 64), (257, 64), (1000, 5)])
 def test_mse_loss_forward_and_backward(tt, dtype, shape):
     rng = np.random.default_rng(shape[0])
     y = rng.uniform(-1, 1, shape).astype(dtype)

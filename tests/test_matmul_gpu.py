@@ -98,6 +98,74 @@ def test_batched_reference_pattern_exact(tt, dtype):
     assert np.array_equal(got, want)
 
 
+# ----------------------------------------------------------------------------- at most 16 columns
+# (B, N rows, K, M columns): the MLP head of benchmark configuration 5 and its weight gradient's shape, ragged rows,
+# k that ends inside a wave's chunk / inside a 16-byte vector / before most waves get any, one column, 16 columns, batches
+THIN_SHAPES = [(1, 1024, 1024, 10), (1, 1000, 784, 10), (2, 37, 333, 7), (1, 16, 64, 16), (3, 50, 130, 1), (1, 5, 2050, 16),
+               (1, 300, 65, 3)]
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+@pytest.mark.parametrize("layout", ["plain", "a_transposed", "b_transposed", "a_row_slice"])
+@pytest.mark.parametrize("shape", THIN_SHAPES)
+def test_products_of_at_most_16_columns(tt, oracle, dtype, layout, shape):
+    B, N, K, M = shape
+    rng = np.random.default_rng(N * 7 + K + M)
+    a = rng.integers(-4, 5, (B, N, K)).astype(dtype)
+    b = rng.integers(-4, 5, (B, K, M)).astype(dtype)
+    be = tt.get_backend(tt.kAMD)
+    ta, tb = dev(tt, a), dev(tt, b)
+    if layout == "a_transposed":      # h^T . dy: A is a permuted view, k-major
+        ta = dev(tt, np.ascontiguousarray(a.transpose(0, 2, 1))).permute(0, 2, 1)
+    elif layout == "b_transposed":
+        tb = dev(tt, np.ascontiguousarray(b.transpose(0, 2, 1))).permute(0, 2, 1)
+    elif layout == "a_row_slice":     # rows of a wider matrix: row stride above K, the start not 16-byte aligned for odd offsets
+        wide = np.zeros((B, N, K + 5), dtype)
+        wide[:, :, 3:3 + K] = a
+        tw = dev(tt, wide)
+        ta = tt.Tensor(tw.storage, tw.dtype, (B, N, K), (N * (K + 5), K + 5, 1), 3)
+    variant = be.batched_matmul_variant(ta, tb)
+    assert variant.startswith("thin_f32" if dtype == np.float32 else "thin_f64"), variant
+    if layout == "plain" and K % (4 if dtype == np.float32 else 2) == 0:
+        assert "vec" in variant
+    if layout in ("a_transposed", "a_row_slice"):
+        assert "vec" not in variant
+    want = np.matmul(a.astype(np.float64), b.astype(np.float64))
+    assert np.array_equal(be.batched_matmul(ta, tb).to_numpy(), want.astype(dtype)), variant
+    # the store's steps: bias per column with ReLU and second output, bias per row accumulated onto the old values,
+    # the ReLU-backward mask
+    bias_n, bias_m = rng.integers(-5, 6, (M,)).astype(dtype), rng.integers(-5, 6, (N,)).astype(dtype)
+    act = tt.Tensor.empty((B, N, M), ta.dtype)
+    got = be.batched_matmul(ta, tb, bias=dev(tt, bias_n), bias_mode=1, relu_out=act).to_numpy()
+    assert np.array_equal(got, (want + bias_n).astype(dtype)) and np.array_equal(act.to_numpy(), np.maximum(got, 0))
+    old = rng.integers(-9, 10, (B, N, M)).astype(dtype)
+    acc = dev(tt, old)
+    be.batched_matmul(ta, tb, bias=dev(tt, bias_m), bias_mode=2, relu=True, accumulate=True, out=acc)
+    assert np.array_equal(acc.to_numpy(), (np.maximum(want + bias_m[None, :, None], 0) + old).astype(dtype))
+    z = rng.integers(-2, 3, (B, N, M)).astype(dtype)
+    got = be.batched_matmul(ta, tb, relu_grad_input=dev(tt, z)).to_numpy()
+    assert np.array_equal(got, (want * np.where(z < 0, 0.0, 1.0)).astype(dtype))
+    # uniform data against the oracle, at the tolerance of the other products
+    if layout == "plain":
+        A = rng.uniform(-1, 1, (B, N, K)).astype(dtype)
+        Bm = rng.uniform(-1, 1, (B, K, M)).astype(dtype)
+        got = be.batched_matmul(dev(tt, A), dev(tt, Bm)).to_numpy()
+        for i in range(B):
+            check_close(got[i], oracle.matmul(A[i], Bm[i]), A[i], Bm[i], dtype)
+
+
+def test_operands_beyond_k_do_not_leak_into_thin_products(tt):
+    """The chunk of k that crosses K reads stand-in elements (the row's element at k = 0); an infinity there must reach
+    the sum once, from k = 0 itself, and not a second time as inf * 0 = NaN."""
+    be = tt.get_backend(tt.kAMD)
+    for K in (70, 72):           # element-wise loads, 16-byte loads
+        a = np.ones((1, 20, K), np.float32)
+        a[0, :, 0] = np.inf
+        b = np.ones((1, K, 10), np.float32)
+        got = be.batched_matmul(dev(tt, a), dev(tt, b)).to_numpy()
+        assert np.all(np.isposinf(got)), K
+
+
 # ----------------------------------------------------------------------------- benchmark configurations
 def test_config1_single_f32(tt, oracle):
     A = oracle.Generator(0).uniform_real(-1, 1, (256, 512))
@@ -240,7 +308,10 @@ def test_variant_selection(tt):
     small = tt.Tensor.from_numpy(np.zeros((1, 256, 512), f32))
     assert be.batched_matmul_variant(small, small.permute(0, 2, 1)).startswith("mfma_f32_64x64")
     thin = tt.Tensor.from_numpy(np.zeros((1, 512, 10), f32))
-    assert be.batched_matmul_variant(small, thin).startswith("mfma_f32_64x64_akc4_bmc1_splitk")  # few tiles, long K
+    assert be.batched_matmul_variant(small, thin) == "thin_f32_16rows_vec4"          # at most 16 columns, long K
+    assert be.batched_matmul_variant(small.permute(0, 2, 1), tt.Tensor.empty((1, 256, 10), tt._capi.F32)) == "thin_f32_16rows"
+    short = tt.Tensor.from_numpy(np.zeros((1, 256, 48), f32))
+    assert be.batched_matmul_variant(short, tt.Tensor.empty((1, 48, 10), tt._capi.F32)).startswith("mfma_f32_64x64")  # short K
     thin_i = tt.Tensor.from_numpy(np.zeros((1, 512, 10), np.int32))
     small_i = tt.Tensor.from_numpy(np.zeros((1, 256, 512), np.int32))
     assert be.batched_matmul_variant(small_i, thin_i) == "simt_i32_128x16"

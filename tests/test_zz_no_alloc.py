@@ -43,7 +43,8 @@ def test_two_calls_in_a_row_match_the_allocating_entry_point(tt, oracle, dtype):
     be = tt.get_backend(tt.kAMD)
     rng = np.random.default_rng(5)
     # first a split-k product that fills several MiB of the array, then a smaller split-k product that finds the first
-    # one's partial tiles there, then shapes that use no scratch at all (two halves of k, plain tiles, integers below)
+    # one's partial tiles there, then shapes that use no scratch at all (10 columns, two halves of k, plain tiles,
+    # integers below)
     # (f64 256 x 512 x 256 splits 16 ways: exactly the 8 MiB the array holds)
     head = [(3, 320, 1024, 384), (1, 256, 512, 256)] if dtype == np.float32 else [(1, 256, 512, 256), (1, 128, 512, 192)]
     shapes = head + [(1, 100, 301, 10), (1, 1024, 1024, 1024), (2, 130, 70, 150)]
@@ -51,7 +52,7 @@ def test_two_calls_in_a_row_match_the_allocating_entry_point(tt, oracle, dtype):
         a, b = _pair(rng, dtype, B, N, K, M)
         tA, tB = tt.Tensor.from_numpy(a), tt.Tensor.from_numpy(b)
         variant = be.batched_matmul_variant(tA, tB)
-        if i < 3:
+        if i < 2:
             assert "splitk" in variant, (variant, (B, N, K, M))
             ksplit = int(variant.split("splitk")[1])
             assert ksplit * B * N * M * a.itemsize <= FIXED_SCRATCH_BYTES

@@ -101,6 +101,10 @@ ttamd_status launch_gemm_mfma(ttamd_dtype dt, const GemmArgs &g, int device, hip
                               bool variant_only, bool *handled, bool fixed_scratch = false);
 ttamd_status launch_gemm_simt(ttamd_dtype dt, const GemmArgs &g, hipStream_t stream, const char **variant,
                               bool variant_only);
+// Products of at most 16 columns and a reduction long enough to share out (gemm_thin.hip): one launch, no scratch.
+// *handled says whether the product is one of them (nothing is launched otherwise).
+ttamd_status launch_gemm_thin(ttamd_dtype dt, const GemmArgs &g, hipStream_t stream, const char **variant, bool variant_only,
+                              bool *handled);
 
 // Stride-1 fp32 convolution served by conv_patch.hip (weights resident in LDS, input rows staged once per tile).
 // The caller fills the first block; launch_conv_patch_f32 derives the rest and reports through *handled whether the

@@ -768,27 +768,42 @@ ttamd_status cast_from(ttamd_dtype to, const void *a, const ViewDesc &va, void *
 // (x / numel).sum(), autograd/reduce_ops.cpp:195-200) together with its backward (grad_output / numel from the mean,
 // times 2 * (input - target) from pow: autograd/reduce_ops.cpp:201-205, binary_ops.cpp:153-159) and, for narrow
 // matrices, the column sums of that gradient (the bias gradient of the Linear layer that produced `input`).
-// Lane layout: CP column lanes (a power of two >= cols, at most 64) by 256 / CP row lanes; a lane walks its column
-// down the rows in steps of (row lanes * blocks).  Sums are folded over the row lanes in a fixed tree, per-block
-// partials ([blocks][cols + 1]: column sums, then the loss) are added by block index: deterministic.
-template <typename T, int CP>
-__global__ void __launch_bounds__(256) mse_loss_kernel(const T *__restrict__ y, const T *__restrict__ t, int64_t rows, int cols, T inv_n,
-                                                      T *__restrict__ grad, T *__restrict__ partial, T *__restrict__ loss,
-                                                      T *__restrict__ colsum) {
-    constexpr int RL = 256 / CP;
+// Lane layout: CP column lanes (a power of two >= cols, at most 64) by THREADS / CP row lanes; a lane walks its column
+// down the rows in steps of (row lanes * blocks), U rows to a batch whose loads are all issued before the first is
+// used (a small matrix is one memory round trip away, not one per row).  Sums are folded over the row lanes in a fixed
+// tree, per-block partials ([blocks][cols + 1]: column sums, then the loss) are added by block index: deterministic.
+// THREADS = 1024 with U = 16 is the form for a matrix that a single workgroup takes in one batch: no partials, no
+// finishing kernel.
+template <typename T, int CP, int THREADS, int U>
+__global__ void __launch_bounds__(THREADS) mse_loss_kernel(const T *__restrict__ y, const T *__restrict__ t, int64_t rows, int cols,
+                                                          T inv_n, T *__restrict__ grad, T *__restrict__ partial,
+                                                          T *__restrict__ loss, T *__restrict__ colsum) {
+    constexpr int RL = THREADS / CP;
     __shared__ T red[RL][CP + 1];
-    __shared__ T red_loss[256];
+    __shared__ T red_loss[THREADS];
     const int cl = threadIdx.x % CP, rl = threadIdx.x / CP;
     const T scale = inv_n * T(2);
     T csum = T(0), lsum = T(0);
     if (cl < cols) {
-        for (int64_t r = static_cast<int64_t>(blockIdx.x) * RL + rl; r < rows; r += static_cast<int64_t>(gridDim.x) * RL) {
-            const int64_t i = r * cols + cl;
-            const T d = y[i] - t[i];
-            lsum += d * d * inv_n;
-            const T g = scale * d;
-            if (grad) grad[i] = g;
-            csum += g;
+        const int64_t step = static_cast<int64_t>(gridDim.x) * RL;
+        for (int64_t r0 = static_cast<int64_t>(blockIdx.x) * RL + rl; r0 < rows; r0 += step * U) {
+            T yv[U], tv[U];
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                const int64_t r = r0 + u * step;
+                const int64_t i = (r < rows ? r : rows - 1) * cols + cl;  // no branch around a load: they all go out together
+                yv[u] = y[i];
+                tv[u] = t[i];
+            }
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                const int64_t r = r0 + u * step;
+                const T d = r < rows ? yv[u] - tv[u] : T(0);
+                lsum += d * d * inv_n;
+                const T g = scale * d;
+                if (grad && r < rows) grad[r * cols + cl] = g;
+                csum += g;
+            }
         }
     }
     red[rl][cl] = csum;
@@ -798,7 +813,7 @@ __global__ void __launch_bounds__(256) mse_loss_kernel(const T *__restrict__ y, 
         if (rl < h) red[rl][cl] += red[rl + h][cl];
         __syncthreads();
     }
-    for (int h = 128; h > 0; h >>= 1) {
+    for (int h = THREADS / 2; h > 0; h >>= 1) {
         if (static_cast<int>(threadIdx.x) < h) red_loss[threadIdx.x] += red_loss[threadIdx.x + h];
         __syncthreads();
     }
@@ -835,28 +850,37 @@ ttamd_status launch_mse_loss(int device, int64_t rows, int64_t cols, const void 
     }
     int cp = 1;
     while (cp < cols) cp *= 2;
+    const bool small = rows * cp <= 1024 * 16;  // one workgroup of 1024 lanes, at most 16 rows to a lane: a single batch
     const int rl = 256 / cp;
-    int64_t blocks = (rows + static_cast<int64_t>(rl) * 8 - 1) / (static_cast<int64_t>(rl) * 8);  // about 8 rows per lane: a lane's
-                                                                                                 // loads are one dependent chain
+    int64_t blocks = (rows + static_cast<int64_t>(rl) * 8 - 1) / (static_cast<int64_t>(rl) * 8);  // about 8 rows per lane
     if (blocks > 1024) blocks = 1024;
-    if (blocks < 1) blocks = 1;
+    if (blocks < 1 || small) blocks = 1;
     void *ws = nullptr;
     if (blocks > 1)
         if (ttamd_status s = stream_scratch(device, st, static_cast<size_t>(blocks) * (cols + 1) * sizeof(T), &ws)) return s;
     const T inv_n = T(1) / static_cast<T>(rows * cols);
     const T *yp = static_cast<const T *>(y), *tp = static_cast<const T *>(t);
     T *gp = static_cast<T *>(grad), *pp = static_cast<T *>(ws), *lp = static_cast<T *>(loss), *cs = static_cast<T *>(colsum);
-    const dim3 grid(static_cast<unsigned>(blocks)), block(256);
+    const dim3 grid(static_cast<unsigned>(blocks));
     const int c = static_cast<int>(cols);
+#define TTAMD_MSE_CASE(CP)                                                                                        \
+    case CP:                                                                                                      \
+        if (small) mse_loss_kernel<T, CP, 1024, 16><<<grid, dim3(1024), 0, st>>>(yp, tp, rows, c, inv_n, gp, pp, lp, cs); \
+        else mse_loss_kernel<T, CP, 256, 8><<<grid, dim3(256), 0, st>>>(yp, tp, rows, c, inv_n, gp, pp, lp, cs);   \
+        break;
     switch (cp) {
-    case 1: mse_loss_kernel<T, 1><<<grid, block, 0, st>>>(yp, tp, rows, c, inv_n, gp, pp, lp, cs); break;
-    case 2: mse_loss_kernel<T, 2><<<grid, block, 0, st>>>(yp, tp, rows, c, inv_n, gp, pp, lp, cs); break;
-    case 4: mse_loss_kernel<T, 4><<<grid, block, 0, st>>>(yp, tp, rows, c, inv_n, gp, pp, lp, cs); break;
-    case 8: mse_loss_kernel<T, 8><<<grid, block, 0, st>>>(yp, tp, rows, c, inv_n, gp, pp, lp, cs); break;
-    case 16: mse_loss_kernel<T, 16><<<grid, block, 0, st>>>(yp, tp, rows, c, inv_n, gp, pp, lp, cs); break;
-    case 32: mse_loss_kernel<T, 32><<<grid, block, 0, st>>>(yp, tp, rows, c, inv_n, gp, pp, lp, cs); break;
-    default: mse_loss_kernel<T, 64><<<grid, block, 0, st>>>(yp, tp, rows, c, inv_n, gp, pp, lp, cs); break;
+        TTAMD_MSE_CASE(1)
+        TTAMD_MSE_CASE(2)
+        TTAMD_MSE_CASE(4)
+        TTAMD_MSE_CASE(8)
+        TTAMD_MSE_CASE(16)
+        TTAMD_MSE_CASE(32)
+    default:
+        if (small) mse_loss_kernel<T, 64, 1024, 16><<<grid, dim3(1024), 0, st>>>(yp, tp, rows, c, inv_n, gp, pp, lp, cs);
+        else mse_loss_kernel<T, 64, 256, 8><<<grid, dim3(256), 0, st>>>(yp, tp, rows, c, inv_n, gp, pp, lp, cs);
+        break;
     }
+#undef TTAMD_MSE_CASE
     if (blocks > 1) mse_loss_finish_kernel<T><<<dim3(1), dim3(256), 0, st>>>(pp, static_cast<int>(blocks), c, lp, cs);
     TTAMD_HIP_CHECK(hipGetLastError());
     return TTAMD_OK;
