@@ -310,6 +310,10 @@ def test_variant_selection(tt):
     thin = tt.Tensor.from_numpy(np.zeros((1, 512, 10), f32))
     assert be.batched_matmul_variant(small, thin) == "thin_f32_16rows_vec4"          # at most 16 columns, long K
     assert be.batched_matmul_variant(small.permute(0, 2, 1), tt.Tensor.empty((1, 256, 10), tt._capi.F32)) == "thin_f32_16rows"
+    assert be.batched_matmul_variant(tt.Tensor.empty((1, 1024, 10), tt._capi.F32),
+                                     tt.Tensor.empty((1, 10, 1024), tt._capi.F32)) == "thin_f32_k16"  # reduction of at most 16
+    assert be.batched_matmul_variant(tt.Tensor.empty((1, 32, 10), tt._capi.F64), tt.Tensor.empty((1, 10, 32), tt._capi.F64)) \
+        .startswith("mfma_f64")                                                                        # ... of a small output
     short = tt.Tensor.from_numpy(np.zeros((1, 256, 48), f32))
     assert be.batched_matmul_variant(short, tt.Tensor.empty((1, 48, 10), tt._capi.F32)).startswith("mfma_f32_64x64")  # short K
     thin_i = tt.Tensor.from_numpy(np.zeros((1, 512, 10), np.int32))

@@ -57,7 +57,7 @@ def test_config5_mlp_training_step(tt, oracle):
     assert any(v.startswith("mfma_f32") and "akc4_bmc4" in v for v in variants)
     assert any(v.startswith("mfma_f32") and "akc4_bkc4" in v for v in variants)  # dC . B^T
     assert any(v.startswith("mfma_f32") and "amc4_bmc4" in v for v in variants)  # A^T . dC
-    assert sum(v.startswith("thin_f32") for v in variants) == 2                  # N = 10: y and dW3
+    assert sum(v.startswith("thin_f32") for v in variants) == 3                  # N = 10 (y, dW3) and K = 10 (dz2)
 
 
 def test_fused_linear_relu_matches_unfused(tt, oracle):

@@ -101,10 +101,15 @@ ttamd_status launch_gemm_mfma(ttamd_dtype dt, const GemmArgs &g, int device, hip
                               bool variant_only, bool *handled, bool fixed_scratch = false);
 ttamd_status launch_gemm_simt(ttamd_dtype dt, const GemmArgs &g, hipStream_t stream, const char **variant,
                               bool variant_only);
-// Products of at most 16 columns and a reduction long enough to share out (gemm_thin.hip): one launch, no scratch.
+// Products of at most 16 columns and a reduction long enough to share out, and products with a reduction of at most
+// 16 (gemm_thin.hip): one launch; only the column sums of the second kind may take scratch.
 // *handled says whether the product is one of them (nothing is launched otherwise).
-ttamd_status launch_gemm_thin(ttamd_dtype dt, const GemmArgs &g, hipStream_t stream, const char **variant, bool variant_only,
-                              bool *handled);
+ttamd_status launch_gemm_thin(ttamd_dtype dt, const GemmArgs &g, int device, hipStream_t stream, const char **variant,
+                              bool variant_only, bool *handled, bool fixed_scratch = false);
+// The GEMM launchers' scratch (the stream's growing buffer, or the library's fixed array when `fixed`) and the kernel
+// that adds `rows` partial rows of column sums: out[b][n] = sum over r of partial[b][r][n], r ascending.
+ttamd_status gemm_scratch(int device, hipStream_t stream, size_t bytes, bool fixed, void **out);
+ttamd_status launch_colsum_reduce(ttamd_dtype dt, const void *partial, int rows, int N, int batch, void *out, hipStream_t stream);
 
 // Stride-1 fp32 convolution served by conv_patch.hip (weights resident in LDS, input rows staged once per tile).
 // The caller fills the first block; launch_conv_patch_f32 derives the rest and reports through *handled whether the

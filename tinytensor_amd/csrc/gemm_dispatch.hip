@@ -108,7 +108,7 @@ ttamd_status batched_matmul(int device, ttamd_dtype dtype, int B, int N, int K, 
     const char *variant = nullptr;
     bool handled = false;
     if (K > 0) {
-        if (ttamd_status s = launch_gemm_thin(dtype, g, st, &variant, false, &handled)) return s;
+        if (ttamd_status s = launch_gemm_thin(dtype, g, device, st, &variant, false, &handled, fixed_scratch)) return s;
         if (handled) return TTAMD_OK;
         if (ttamd_status s = launch_gemm_mfma(dtype, g, device, st, &variant, false, &handled, fixed_scratch)) return s;
         if (handled) return TTAMD_OK;
@@ -143,7 +143,7 @@ const char *ttamd_batched_matmul_variant(ttamd_dtype dtype, int B, int N, int K,
     const char *variant = "none";
     bool handled = false;
     if (K > 0) {
-        if (launch_gemm_thin(dtype, g, nullptr, &variant, true, &handled) != TTAMD_OK) return "invalid";
+        if (launch_gemm_thin(dtype, g, 0, nullptr, &variant, true, &handled) != TTAMD_OK) return "invalid";
         if (handled) return variant;
         if (launch_gemm_mfma(dtype, g, 0, nullptr, &variant, true, &handled) != TTAMD_OK) return "invalid";
         if (handled) return variant;

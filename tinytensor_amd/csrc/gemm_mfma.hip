@@ -523,6 +523,20 @@ ttamd_status launch_mfma_typed(const GemmArgs &g, int device, hipStream_t stream
 
 }  // namespace
 
+ttamd_status gemm_scratch(int device, hipStream_t stream, size_t bytes, bool fixed, void **out) {
+    return launch_scratch(device, stream, bytes, fixed, out);
+}
+
+ttamd_status launch_colsum_reduce(ttamd_dtype dt, const void *partial, int rows, int N, int batch, void *out, hipStream_t stream) {
+    const dim3 grid(static_cast<unsigned>((N + 63) / 64), static_cast<unsigned>(batch));
+    if (dt == TTAMD_F32)
+        colsum_reduce_kernel<float><<<grid, dim3(64), 0, stream>>>(static_cast<const float *>(partial), rows, N, static_cast<float *>(out));
+    else
+        colsum_reduce_kernel<double><<<grid, dim3(64), 0, stream>>>(static_cast<const double *>(partial), rows, N, static_cast<double *>(out));
+    TTAMD_HIP_CHECK(hipGetLastError());
+    return TTAMD_OK;
+}
+
 ttamd_status launch_gemm_mfma(ttamd_dtype dt, const GemmArgs &g, int device, hipStream_t stream, const char **variant,
                               bool variant_only, bool *handled, bool fixed_scratch) {
     *handled = false;

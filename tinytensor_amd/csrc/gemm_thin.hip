@@ -9,6 +9,12 @@
 // registers (each element of A is read exactly once by the whole grid, B is small and comes from L2), and the waves'
 // 16 x 16 partial results are added through LDS in wave order.  One launch, one memory round trip per chunk.
 //
+// The second kernel here is for a reduction of at most 16 (dz = (dy . W^T) * mask with 10 classes: the product that
+// carries the gradient back through the head): four MFMA steps make a 16 x 16 tile, so the kernel is a stream of
+// tiles bounded by the mask it reads and the result it writes.  A workgroup owns a strip of 16 columns and up to 1024
+// rows of it; B's 16 x 16 corner stays in registers, every wave issues the loads of all its tiles before the first
+// MFMA, and a workgroup that owns all the rows of its strip finishes the bias gradient's column sums by itself.
+//
 // MFMA operand lanes (both dtypes): lane l supplies A[l % 16][l / 16] and B[l / 16][l % 16] of a 16 x 4 by 4 x 16
 // step.  Which k a step's four slices stand for is free as long as A and B agree, so a lane that loads a 16-byte
 // vector of its row uses the vector's elements in consecutive steps.
@@ -41,8 +47,17 @@ struct ThinMma<double> {
     static __device__ __forceinline__ int acc_row(int e, int lane) { return 4 * e + lane / 16; }
 };
 
+// The loaded value is needed here, whatever is done with it afterwards.  Without this the compiler turns "load a
+// stand-in, then select zero" into a branch around the load and waits for each such load by itself; with it, a run of
+// loads followed by a run of keep() calls is a run of loads in flight together.
+template <typename V>
+__device__ __forceinline__ void keep(V &v) {
+    asm volatile("" : "+v"(v));
+}
+
 constexpr int kThinWaves = 16;
 constexpr int kThinMinK = 64;  // below this most waves would have nothing to do
+constexpr int64_t kThinKMinOutput = 64 * 64;  // smaller outputs of a short reduction: a single tile of the general kernels
 
 // VECA: A's rows are contiguous in k, 16-byte aligned, and K is a whole number of 16-byte vectors.
 template <typename T, bool VECA>
@@ -117,6 +132,225 @@ __global__ void __launch_bounds__(64 * kThinWaves) gemm_thin_kernel(GemmArgs g) 
     if (g.relu_out) static_cast<T *>(g.relu_out)[idx] = v > T(0) ? v : T(0);
 }
 
+// ---------------------------------------------------------------------------------------------------------------
+// K <= 16.  Where a lane's four accumulator elements sit in the 16 x 16 tile decides how it stores them:
+//   f32, computed as the transposed tile (B's slice as the first operand): row l % 16, columns 4 * (l / 16) + e --
+//        four consecutive columns, one 16-byte store when the row length allows;
+//   f64: rows 4 * e + l / 16, column l % 16 -- 16 lanes write 128 contiguous bytes of a row.
+template <typename T>
+struct ThinTile;
+template <>
+struct ThinTile<float> {
+    static constexpr bool kTransposed = true;
+    static __device__ __forceinline__ int row(int e, int lane) { return lane % 16; }
+    static __device__ __forceinline__ int col(int e, int lane) { return 4 * (lane / 16) + e; }
+};
+template <>
+struct ThinTile<double> {
+    static constexpr bool kTransposed = false;
+    static __device__ __forceinline__ int row(int e, int lane) { return 4 * e + lane / 16; }
+    static __device__ __forceinline__ int col(int e, int lane) { return lane % 16; }
+};
+
+// TPW tiles per wave; a workgroup's 16 waves take the 16 * TPW row tiles of its block in turn (tile = u * 16 + wave,
+// rotated by the strip's number).
+// colsum_dst: [batch][gridDim.y][N] -- the launcher passes the final array when gridDim.y == 1.
+template <typename T, int TPW>
+__global__ void __launch_bounds__(64 * kThinWaves) gemm_thin_k_kernel(GemmArgs g, T *__restrict__ colsum_dst, int vec_rows) {
+    using MI = ThinMma<T>;
+    using TL = ThinTile<T>;
+    using acc_t = typename MI::acc_t;
+    __shared__ T red[kThinWaves][16];
+    const int tid = threadIdx.x, wave = tid / 64, lane = tid % 64;
+    const int li = lane % 16, q = lane / 16;
+    const int n0 = blockIdx.x * 16, batch = blockIdx.z;
+    const int m_block = blockIdx.y * (256 * TPW);
+    // Neighbouring strips start at different row tiles: rows are a multiple of the memory channels' interleave apart
+    // when N is a power of two, and strips that walked the rows in step would all queue at the same channels.
+    const int rot = blockIdx.x % (kThinWaves * TPW);
+    const T *__restrict__ A = static_cast<const T *>(g.A) + static_cast<int64_t>(batch) * g.a_sb;
+    const T *__restrict__ B = static_cast<const T *>(g.B) + static_cast<int64_t>(batch) * g.b_sb;
+    const T *__restrict__ Z = g.zmask ? static_cast<const T *>(g.zmask) + static_cast<int64_t>(batch) * g.M * g.N : nullptr;
+    T *__restrict__ C = static_cast<T *>(g.C) + static_cast<int64_t>(batch) * g.M * g.N;
+    T *__restrict__ R = g.relu_out ? static_cast<T *>(g.relu_out) + static_cast<int64_t>(batch) * g.M * g.N : nullptr;
+    // Step s of a tile multiplies slice k = 4 s + q.  Beyond K, M or N the loads read a valid stand-in element and the
+    // value is zeroed (beyond K on both sides, so that no stand-in infinity meets a zero).
+    // Every load of the wave's tiles goes out before the first value is looked at.
+    T bop[4], aop[TPW][4], zv[TPW][4];
+    acc_t zvec[TPW];
+    const bool vec = TL::kTransposed && vec_rows;  // (then N is a multiple of 4: a lane's four columns are in range together)
+    {
+        const int n = n0 + li < g.N ? n0 + li : g.N - 1;
+#pragma unroll
+        for (int s = 0; s < 4; ++s) {
+            const int k = 4 * s + q;
+            bop[s] = B[static_cast<int64_t>(k < g.K ? k : 0) * g.b_sk + static_cast<int64_t>(n) * g.b_sn];
+        }
+    }
+#pragma unroll
+    for (int u = 0; u < TPW; ++u) {
+        const int m0 = m_block + ((u * kThinWaves + wave + rot) % (kThinWaves * TPW)) * 16;
+        const int m = m0 + li < g.M ? m0 + li : g.M - 1;
+#pragma unroll
+        for (int s = 0; s < 4; ++s) {
+            const int k = 4 * s + q;
+            aop[u][s] = A[static_cast<int64_t>(m) * g.a_sm + static_cast<int64_t>(k < g.K ? k : 0) * g.a_sk];
+        }
+    }
+    if (Z && vec) {  // workgroup-uniform
+#pragma unroll
+        for (int u = 0; u < TPW; ++u) {
+            const int m0 = m_block + ((u * kThinWaves + wave + rot) % (kThinWaves * TPW)) * 16;
+            const int zr = m0 + TL::row(0, lane) < g.M ? m0 + TL::row(0, lane) : g.M - 1;
+            const int zc = n0 + TL::col(0, lane) < g.N ? n0 + TL::col(0, lane) : 0;
+            zvec[u] = *reinterpret_cast<const acc_t *>(Z + static_cast<int64_t>(zr) * g.N + zc);
+        }
+#pragma unroll
+        for (int u = 0; u < TPW; ++u) keep(zvec[u]);
+#pragma unroll
+        for (int u = 0; u < TPW; ++u) {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) zv[u][e] = zvec[u][e];
+        }
+    } else if (Z) {
+#pragma unroll
+        for (int u = 0; u < TPW; ++u) {
+            const int m0 = m_block + ((u * kThinWaves + wave + rot) % (kThinWaves * TPW)) * 16;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const int r = m0 + TL::row(e, lane) < g.M ? m0 + TL::row(e, lane) : g.M - 1;
+                const int c = n0 + TL::col(e, lane) < g.N ? n0 + TL::col(e, lane) : g.N - 1;
+                zv[u][e] = Z[static_cast<int64_t>(r) * g.N + c];
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < TPW; ++u) {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) keep(zv[u][e]);
+        }
+    } else {
+#pragma unroll
+        for (int u = 0; u < TPW; ++u) {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) zv[u][e] = T(0);
+        }
+    }
+#pragma unroll
+    for (int s = 0; s < 4; ++s) {
+        keep(bop[s]);
+        bop[s] = 4 * s + q < g.K && n0 + li < g.N ? bop[s] : T(0);
+    }
+#pragma unroll
+    for (int u = 0; u < TPW; ++u) {
+#pragma unroll
+        for (int s = 0; s < 4; ++s) {
+            keep(aop[u][s]);
+            aop[u][s] = 4 * s + q < g.K ? aop[u][s] : T(0);
+        }
+    }
+    const T *bias = static_cast<const T *>(g.bias);
+    T csum[4] = {T(0), T(0), T(0), T(0)};
+#pragma unroll
+    for (int u = 0; u < TPW; ++u) {
+        const int m0 = m_block + ((u * kThinWaves + wave + rot) % (kThinWaves * TPW)) * 16;
+        acc_t acc = {};
+#pragma unroll
+        for (int s = 0; s < 4; ++s) acc = TL::kTransposed ? MI::mma(bop[s], aop[u][s], acc) : MI::mma(aop[u][s], bop[s], acc);
+        T out[4];
+        bool in[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {  // bias, ReLU-backward mask, ReLU, accumulate: the order of the general kernels
+            const int m = m0 + TL::row(e, lane), n = n0 + TL::col(e, lane);
+            in[e] = m < g.M && n < g.N;
+            T v = acc[e];
+            if (g.bias_mode == 1 && in[e]) v += bias[n];
+            if (g.bias_mode == 2 && in[e]) v += bias[m];
+            if (zv[u][e] < T(0)) v = T(0);
+            if (g.relu) v = v > T(0) ? v : T(0);
+            if (g.accumulate && in[e]) v += C[static_cast<int64_t>(m) * g.N + n];
+            out[e] = v;
+            csum[e] += in[e] ? v : T(0);
+        }
+        if (TL::kTransposed && vec_rows) {
+            if (in[0]) {  // a lane's four columns are in range together
+                const int64_t idx = static_cast<int64_t>(m0 + TL::row(0, lane)) * g.N + n0 + TL::col(0, lane);
+                acc_t o, r;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    o[e] = out[e];
+                    r[e] = out[e] > T(0) ? out[e] : T(0);
+                }
+                *reinterpret_cast<acc_t *>(C + idx) = o;
+                if (R) *reinterpret_cast<acc_t *>(R + idx) = r;
+            }
+        } else {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                if (!in[e]) continue;
+                const int64_t idx = static_cast<int64_t>(m0 + TL::row(e, lane)) * g.N + n0 + TL::col(e, lane);
+                C[idx] = out[e];
+                if (R) R[idx] = out[e] > T(0) ? out[e] : T(0);
+            }
+        }
+    }
+    if (!colsum_dst) return;  // workgroup-uniform
+    // Column sums of the block's rows: over a wave's lanes first, then over the waves in wave order.
+    if (TL::kTransposed) {  // lanes of one q hold 16 rows of columns 4 q + e
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+#pragma unroll
+            for (int d = 1; d < 16; d *= 2) csum[e] += __shfl_xor(csum[e], d, 64);
+        }
+        if (li == 0) {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) red[wave][4 * q + e] = csum[e];
+        }
+    } else {  // a lane holds four rows of column l % 16; the other twelve are in the lanes 16, 32, 48 further on
+        T v = (csum[0] + csum[1]) + (csum[2] + csum[3]);
+        v += __shfl_xor(v, 16, 64);
+        v += __shfl_xor(v, 32, 64);
+        if (lane < 16) red[wave][lane] = v;
+    }
+    __syncthreads();
+    if (tid < 16 && n0 + tid < g.N) {
+        T v = T(0);
+#pragma unroll
+        for (int w = 0; w < kThinWaves; ++w) v += red[w][tid];
+        colsum_dst[(static_cast<int64_t>(batch) * gridDim.y + blockIdx.y) * g.N + n0 + tid] = v;
+    }
+}
+
+template <typename T>
+ttamd_status launch_thin_k_typed(ttamd_dtype dt, const GemmArgs &g, int device, hipStream_t stream, bool fixed_scratch) {
+    const int strips = (g.N + 15) / 16;
+    // With column sums: 1024 rows to a workgroup, so that up to 1024 rows finish their sums inside the kernel and longer
+    // matrices leave few partial rows; fewer rows when the matrix is shorter.  Without: 256 rows, the most workgroups
+    // (measured at 1024 x 10 x 1024: 6.3 us against 8.9).
+    int tpw = g.colsum_out ? 4 : 1;
+    while (tpw > 1 && g.M <= 256 * (tpw / 2)) tpw /= 2;
+    const int row_blocks = (g.M + 256 * tpw - 1) / (256 * tpw);
+    if (row_blocks > 65535 || g.batch > 65535) {
+        set_error("batched_matmul: %d row blocks by %d batch items exceed the grid limit", row_blocks, g.batch);
+        return TTAMD_ERR_INVALID_ARGUMENT;
+    }
+    T *colsum_dst = static_cast<T *>(g.colsum_out);
+    if (g.colsum_out && row_blocks > 1) {  // partial rows now, colsum_reduce adds them
+        void *ws = nullptr;
+        const size_t bytes = static_cast<size_t>(g.batch) * row_blocks * g.N * sizeof(T);
+        if (ttamd_status st = gemm_scratch(device, stream, bytes, fixed_scratch, &ws)) return st;
+        colsum_dst = static_cast<T *>(ws);
+    }
+    auto aligned = [](const void *p) { return reinterpret_cast<uintptr_t>(p) % 16 == 0; };
+    const int vec_rows = g.N % 4 == 0 && aligned(g.C) && aligned(g.zmask) && aligned(g.relu_out) ? 1 : 0;
+    const dim3 grid(static_cast<unsigned>(strips), static_cast<unsigned>(row_blocks), static_cast<unsigned>(g.batch)), block(64 * kThinWaves);
+    if (tpw == 4) gemm_thin_k_kernel<T, 4><<<grid, block, 0, stream>>>(g, colsum_dst, vec_rows);
+    else if (tpw == 2) gemm_thin_k_kernel<T, 2><<<grid, block, 0, stream>>>(g, colsum_dst, vec_rows);
+    else gemm_thin_k_kernel<T, 1><<<grid, block, 0, stream>>>(g, colsum_dst, vec_rows);
+    TTAMD_HIP_CHECK(hipGetLastError());
+    if (g.colsum_out && row_blocks > 1) return launch_colsum_reduce(dt, colsum_dst, row_blocks, g.N, g.batch, g.colsum_out, stream);
+    return TTAMD_OK;
+}
+
 template <typename T>
 ttamd_status launch_thin_typed(const GemmArgs &g, hipStream_t stream, const char **variant, bool variant_only, const char *name_vec,
                                const char *name_any) {
@@ -134,9 +368,16 @@ ttamd_status launch_thin_typed(const GemmArgs &g, hipStream_t stream, const char
 
 }  // namespace
 
-ttamd_status launch_gemm_thin(ttamd_dtype dt, const GemmArgs &g, hipStream_t stream, const char **variant, bool variant_only,
-                              bool *handled) {
+ttamd_status launch_gemm_thin(ttamd_dtype dt, const GemmArgs &g, int device, hipStream_t stream, const char **variant,
+                              bool variant_only, bool *handled, bool fixed_scratch) {
     *handled = false;
+    if ((dt == TTAMD_F32 || dt == TTAMD_F64) && g.K <= 16 && g.N >= 16 && static_cast<int64_t>(g.M) * g.N >= kThinKMinOutput) {
+        *handled = true;
+        *variant = dt == TTAMD_F32 ? "thin_f32_k16" : "thin_f64_k16";
+        if (variant_only) return TTAMD_OK;
+        return dt == TTAMD_F32 ? launch_thin_k_typed<float>(dt, g, device, stream, fixed_scratch)
+                               : launch_thin_k_typed<double>(dt, g, device, stream, fixed_scratch);
+    }
     if ((dt != TTAMD_F32 && dt != TTAMD_F64) || g.N > 16 || g.K < kThinMinK || g.colsum_out || g.batch > 65535) return TTAMD_OK;
     *handled = true;
     if (dt == TTAMD_F32) return launch_thin_typed<float>(g, stream, variant, variant_only, "thin_f32_16rows_vec4", "thin_f32_16rows");
