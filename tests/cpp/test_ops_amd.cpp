@@ -432,7 +432,7 @@ TEST_CASE("MLP training step") {
     for (int i = 0; i < iters; ++i) (void)mlp_step_fused(X, T, b1, b2, b3);
     check(ttamd_device_synchronize(0));
     const double ms_fused = std::chrono::duration<double, std::milli>(std::chrono::steady_clock::now() - t1).count() / iters;
-    std::printf("  the same step from the fused forms (14 launches): %.3f ms per step\n", ms_fused);
+    std::printf("  the same step from the fused forms (11 launches): %.3f ms per step\n", ms_fused);
     CHECK(ms_fused < 50.0);
 }
 
