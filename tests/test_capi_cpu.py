@@ -95,7 +95,7 @@ def test_variant_names_without_gpu(tt):
     # a row of C too long for the 32-bit store offsets of a tile: the vector-ALU kernel takes it
     assert variant(capi.F32, 1, 64, 64, 1 << 23, (0, 64, 1), (0, 1 << 23, 1)).startswith("simt_f32")
     assert variant(capi.F32, 32, 128, 64, 128, (8192, 64, 1), (8192, 1, 64)) == "mfma_f32_64x64_akc4_bkc4"  # config 2
-    assert variant(capi.F32, 1, 256, 512, 256, (0, 512, 1), (0, 256, 1)) == "mfma_f32_64x64_akc4_bmc4_splitk8"  # config 1
+    assert variant(capi.F32, 1, 256, 512, 256, (0, 512, 1), (0, 256, 1)) == "small_f32_16x16_vec4"  # config 1
     assert variant(capi.F32, 1, 1024, 1024, 10, (0, 1024, 1), (0, 10, 1)) == "thin_f32_16rows_vec4"  # skinny N
     assert variant(capi.F32, 1, 1024, 1024, 1024, (0, 1024, 1), (0, 1024, 1)) == "mfma_f32_64x64_akc4_bmc4_halves"  # one workgroup per CU: two halves of k
     assert variant(capi.F32, 1, 1024, 784, 1024, (0, 784, 1), (0, 1024, 1)) == "mfma_f32_64x64_akc4_bmc4_halves"  # 392 + 392: 13 k tiles each

@@ -12,9 +12,9 @@ from helpers import max_rel_error, mlp_train_step
 
 pytestmark = pytest.mark.gpu
 
-# (B, N, K, M): small-tile plain, ragged with odd M (no paired stores), two halves of k, split k, 128 x 128, 192 x 192,
+# (B, N, K, M): small-tile plain, ragged with odd M (no paired stores), two halves of k, a small output, split k, 128 x 128, 192 x 192,
 # 256 x 256 / 256 x 128 tiles, K = 10 (the skinny backward product of configuration 5), element-wise gathers
-SHAPES = [(1, 200, 96, 136), (2, 130, 70, 151), (1, 1024, 1024, 1024), (1, 256, 512, 256), (1, 2048, 64, 2048),
+SHAPES = [(1, 200, 96, 136), (2, 130, 70, 151), (1, 1024, 1024, 1024), (1, 256, 512, 256), (1, 320, 512, 416), (1, 2048, 64, 2048),
           (1, 3072, 32, 3072), (1, 4096, 32, 4096), (1, 1024, 10, 1024), (3, 70, 50, 90),
           # reductions of at most 16 (their own kernel): ragged rows and columns, rows of 4n and of odd length, one to four
           # tiles per wave, several row blocks (the column sums then come from partial rows), batches, k = 1 and k = 16

@@ -101,14 +101,17 @@ def test_batched_reference_pattern_exact(tt, dtype):
 # ----------------------------------------------------------------------------- at most 16 columns
 # (B, N rows, K, M columns): the MLP head of benchmark configuration 5 and its weight gradient's shape, ragged rows,
 # k that ends inside a wave's chunk / inside a 16-byte vector / before most waves get any, one column, 16 columns, batches
-THIN_SHAPES = [(1, 1024, 1024, 10), (1, 1000, 784, 10), (2, 37, 333, 7), (1, 16, 64, 16), (3, 50, 130, 1), (1, 5, 2050, 16),
+THIN_SHAPES = [(1, 1024, 1024, 10), (1, 1000, 784, 10), (2, 37, 333, 7), (1, 16, 64, 16), (3, 50, 130, 1), (1, 5, 1022, 16),
                (1, 300, 65, 3)]
+# small outputs of a long reduction (the same kernel over a grid of 16 x 16 blocks): benchmark configuration 1, ragged
+# blocks in both directions, batches, one block row
+SMALL_SHAPES = [(1, 256, 512, 256), (2, 100, 300, 50), (1, 37, 129, 333), (4, 128, 256, 128), (1, 17, 1024, 17)]
 
 
 @pytest.mark.parametrize("dtype", [np.float32, np.float64])
 @pytest.mark.parametrize("layout", ["plain", "a_transposed", "b_transposed", "a_row_slice"])
-@pytest.mark.parametrize("shape", THIN_SHAPES)
-def test_products_of_at_most_16_columns(tt, oracle, dtype, layout, shape):
+@pytest.mark.parametrize("shape", THIN_SHAPES + SMALL_SHAPES)
+def test_products_of_at_most_16_columns_and_small_outputs(tt, oracle, dtype, layout, shape):
     B, N, K, M = shape
     rng = np.random.default_rng(N * 7 + K + M)
     a = rng.integers(-4, 5, (B, N, K)).astype(dtype)
@@ -125,7 +128,7 @@ def test_products_of_at_most_16_columns(tt, oracle, dtype, layout, shape):
         tw = dev(tt, wide)
         ta = tt.Tensor(tw.storage, tw.dtype, (B, N, K), (N * (K + 5), K + 5, 1), 3)
     variant = be.batched_matmul_variant(ta, tb)
-    assert variant.startswith("thin_f32" if dtype == np.float32 else "thin_f64"), variant
+    assert variant.startswith(("thin_" if M <= 16 else "small_") + ("f32" if dtype == np.float32 else "f64")), variant
     if layout == "plain" and K % (4 if dtype == np.float32 else 2) == 0:
         assert "vec" in variant
     if layout in ("a_transposed", "a_row_slice"):
@@ -306,7 +309,11 @@ def test_variant_selection(tt):
     big64 = tt.Tensor.empty((1, 4096, 4096), tt._capi.F64)
     assert be.batched_matmul_variant(big64, big64) == "mfma_f64_256x128_akc2_bmc2"
     small = tt.Tensor.from_numpy(np.zeros((1, 256, 512), f32))
-    assert be.batched_matmul_variant(small, small.permute(0, 2, 1)).startswith("mfma_f32_64x64")
+    assert be.batched_matmul_variant(small, small.permute(0, 2, 1)) == "small_f32_16x16_vec4"  # 16 tiles of 64 x 64, long K
+    mid = tt.Tensor.empty((1, 512, 512), tt._capi.F32)
+    assert be.batched_matmul_variant(mid, mid).startswith("mfma_f32_64x64_akc4_bmc4_splitk")  # more blocks than one round
+    deep = tt.Tensor.empty((1, 256, 8192), tt._capi.F32)
+    assert be.batched_matmul_variant(deep, deep.permute(0, 2, 1)).startswith("mfma_f32_64x64_akc4_bkc4_splitk")  # too long a k
     thin = tt.Tensor.from_numpy(np.zeros((1, 512, 10), f32))
     assert be.batched_matmul_variant(small, thin) == "thin_f32_16rows_vec4"          # at most 16 columns, long K
     assert be.batched_matmul_variant(small.permute(0, 2, 1), tt.Tensor.empty((1, 256, 10), tt._capi.F32)) == "thin_f32_16rows"
@@ -401,7 +408,7 @@ def test_big_tile_epilogues_and_edges(tt, dtype, N, M, layout, tile):
 # keep the sums exact.
 @pytest.mark.parametrize("dtype", [np.float32, np.float64])
 @pytest.mark.parametrize("layout", LAYOUTS)
-@pytest.mark.parametrize("shape", [(320, 1024, 448), (200, 1000, 260), (64, 4100, 64), (704, 520, 1344), (448, 48, 320)])
+@pytest.mark.parametrize("shape", [(320, 1024, 448), (200, 1000, 420), (64, 4100, 64), (704, 520, 1344), (448, 48, 320)])
 def test_small_tile_prefetch_depths(tt, dtype, layout, shape):
     N, K, M = shape
     rng = np.random.default_rng(N + K + M)

@@ -14,8 +14,8 @@ pytestmark = pytest.mark.gpu
 def fragment(tt, be, x, w1, b1, w2, target, img, filt):
     """Forward of Linear-ReLU-Linear with a squared-error sum, the two weight gradients' GEMMs, and a conv2d with ReLU
     and max pooling, forward and backward."""
-    h = be.batched_matmul(x, w1, bias=b1, bias_mode=1, relu=True)  # 256x512x256: split reduction + fused epilogue
-    y = be.batched_matmul(h, w2)
+    h = be.batched_matmul(x, w1, bias=b1, bias_mode=1, relu=True)  # 320x512x416: split reduction + fused epilogue
+    y = be.batched_matmul(h, w2)                     # 320x416x64: the kernel for small outputs
     d = be.binary(y, target, "sub")
     loss = be.sum(be.binary(d, d, "mul"))
     gw2 = be.batched_matmul(h.permute(0, 2, 1), d)   # A^T . B on a view
@@ -31,9 +31,9 @@ def fragment(tt, be, x, w1, b1, w2, target, img, filt):
 def make_inputs(tt, seed):
     rng = np.random.default_rng(seed)
     f = np.float32
-    host = dict(x=rng.uniform(-1, 1, (1, 256, 512)).astype(f), w1=rng.uniform(-0.1, 0.1, (1, 512, 256)).astype(f),
-                b1=rng.uniform(-1, 1, (256,)).astype(f), w2=rng.uniform(-0.1, 0.1, (1, 256, 64)).astype(f),
-                target=rng.uniform(-1, 1, (1, 256, 64)).astype(f), img=rng.normal(0, 1, (4, 8, 12, 12)).astype(f),
+    host = dict(x=rng.uniform(-1, 1, (1, 320, 512)).astype(f), w1=rng.uniform(-0.1, 0.1, (1, 512, 416)).astype(f),
+                b1=rng.uniform(-1, 1, (416,)).astype(f), w2=rng.uniform(-0.1, 0.1, (1, 416, 64)).astype(f),
+                target=rng.uniform(-1, 1, (1, 320, 64)).astype(f), img=rng.normal(0, 1, (4, 8, 12, 12)).astype(f),
                 filt=rng.normal(0, 0.2, (16, 8, 3, 3)).astype(f))
     return host
 
@@ -128,8 +128,8 @@ def test_scratch_growth_after_a_capture_keeps_the_recorded_buffer(tt):
     graph = None
     try:
         rng = np.random.default_rng(3)
-        a = tt.Tensor.from_numpy(rng.integers(-3, 4, (1, 256, 512)).astype(np.float32))
-        b = tt.Tensor.from_numpy(rng.integers(-3, 4, (1, 512, 256)).astype(np.float32))
+        a = tt.Tensor.from_numpy(rng.integers(-3, 4, (1, 320, 512)).astype(np.float32))
+        b = tt.Tensor.from_numpy(rng.integers(-3, 4, (1, 512, 416)).astype(np.float32))
         assert "splitk" in be.batched_matmul_variant(a, b)
         graph = tt.graph.Graph(stream, lambda: [be.batched_matmul(a, b)])
         graph.launch()

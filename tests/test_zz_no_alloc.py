@@ -45,8 +45,8 @@ def test_two_calls_in_a_row_match_the_allocating_entry_point(tt, oracle, dtype):
     # first a split-k product that fills several MiB of the array, then a smaller split-k product that finds the first
     # one's partial tiles there, then shapes that use no scratch at all (10 columns, two halves of k, plain tiles,
     # integers below)
-    # (f64 256 x 512 x 256 splits 16 ways: exactly the 8 MiB the array holds)
-    head = [(3, 320, 1024, 384), (1, 256, 512, 256)] if dtype == np.float32 else [(1, 256, 512, 256), (1, 128, 512, 192)]
+    # (small outputs with a moderate k, like 256 x 512 x 256, take a kernel without scratch: not what this test is after)
+    head = [(3, 320, 1024, 384), (1, 320, 512, 416)] if dtype == np.float32 else [(1, 64, 4096, 128), (1, 64, 8192, 64)]
     shapes = head + [(1, 100, 301, 10), (1, 1024, 1024, 1024), (2, 130, 70, 150)]
     for i, (B, N, K, M) in enumerate(shapes):
         a, b = _pair(rng, dtype, B, N, K, M)
@@ -70,14 +70,14 @@ def test_transposed_views_epilogue_and_integers(tt, oracle):
     capi, lib = tt._capi, tt._capi.lib
     rng = np.random.default_rng(6)
     # A^T . B on views (the weight-gradient product of a skinny Linear layer: split k with element-wise B)
-    x, g = rng.integers(-3, 4, (1, 1024, 300)).astype(np.float32), rng.integers(-3, 4, (1, 1024, 10)).astype(np.float32)
+    x, g = rng.integers(-3, 4, (1, 4096, 300)).astype(np.float32), rng.integers(-3, 4, (1, 4096, 10)).astype(np.float32)
     tX, tG = tt.Tensor.from_numpy(x).permute(0, 2, 1), tt.Tensor.from_numpy(g)
     got = _run(tt, lib.ttamd_batched_matmul_noalloc, tX, tG)
     assert np.array_equal(got, _run(tt, lib.ttamd_batched_matmul, tX, tG))
     assert np.array_equal(got, oracle.batched_matmul(np.ascontiguousarray(x.transpose(0, 2, 1)), g))  # integer-valued: exact
     # bias + ReLU fused behind a split reduction (applied by the kernel that sums the partial tiles)
-    a, b = _pair(rng, np.float32, 1, 256, 512, 256, integer_valued=True)
-    bias = rng.integers(-50, 50, 256).astype(np.float32)
+    a, b = _pair(rng, np.float32, 1, 320, 512, 416, integer_valued=True)
+    bias = rng.integers(-50, 50, 416).astype(np.float32)
     tbias = tt.Tensor.from_numpy(bias)
     ep = capi.Epilogue(tbias.storage.ptr, 1, 1, 0)
     tA, tB = tt.Tensor.from_numpy(a), tt.Tensor.from_numpy(b)

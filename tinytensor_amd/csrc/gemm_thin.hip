@@ -57,6 +57,8 @@ __device__ __forceinline__ void keep(V &v) {
 
 constexpr int kThinWaves = 16;
 constexpr int kThinMinK = 64;  // below this most waves would have nothing to do
+constexpr int kSmallMinK = 128;
+constexpr int64_t kSmallMaxBlocks = 512;
 constexpr int64_t kThinKMinOutput = 64 * 64;  // smaller outputs of a short reduction: a single tile of the general kernels
 
 // VECA: A's rows are contiguous in k, 16-byte aligned, and K is a whole number of 16-byte vectors.
@@ -70,12 +72,12 @@ __global__ void __launch_bounds__(64 * kThinWaves) gemm_thin_kernel(GemmArgs g) 
     __shared__ T red[kThinWaves][256];
     const int tid = threadIdx.x, wave = tid / 64, lane = tid % 64;
     const int li = lane % 16, q = lane / 16;
-    const int batch = blockIdx.y, m0 = blockIdx.x * 16;
+    const int batch = blockIdx.z, m0 = blockIdx.x * 16, n0 = blockIdx.y * 16;
     // Rows beyond M and columns beyond N read a valid element (row M-1, column N-1): a row's garbage stays in that
     // row, which is not stored; the columns' B values are zeroed.  Beyond K both operands are zeroed.
     const int row = m0 + li < g.M ? m0 + li : g.M - 1;
-    const int col = li < g.N ? li : g.N - 1;
-    const bool col_ok = li < g.N;
+    const int col = n0 + li < g.N ? n0 + li : g.N - 1;
+    const bool col_ok = n0 + li < g.N;
     const T *__restrict__ A = static_cast<const T *>(g.A) + static_cast<int64_t>(batch) * g.a_sb + static_cast<int64_t>(row) * g.a_sm;
     const T *__restrict__ B = static_cast<const T *>(g.B) + static_cast<int64_t>(batch) * g.b_sb + static_cast<int64_t>(col) * g.b_sn;
     acc_t acc0 = {}, acc1 = {};
@@ -117,7 +119,7 @@ __global__ void __launch_bounds__(64 * kThinWaves) gemm_thin_kernel(GemmArgs g) 
 #pragma unroll
     for (int w = 0; w < kThinWaves; ++w) v += red[w][tid];  // wave order: deterministic
     const int e = tid / 64, l = tid % 64;
-    const int m = m0 + MI::acc_row(e, l), n = l % 16;
+    const int m = m0 + MI::acc_row(e, l), n = n0 + l % 16;
     if (m >= g.M || n >= g.N) return;
     // The store's steps in the order of the general kernels: bias, ReLU-backward mask, ReLU, accumulate, second output.
     const int64_t idx = (static_cast<int64_t>(batch) * g.M + m) * g.N + n;
@@ -359,7 +361,8 @@ ttamd_status launch_thin_typed(const GemmArgs &g, hipStream_t stream, const char
                      (variant_only || reinterpret_cast<uintptr_t>(g.A) % 16 == 0);
     *variant = vec ? name_vec : name_any;
     if (variant_only) return TTAMD_OK;
-    const dim3 grid(static_cast<unsigned>((g.M + 15) / 16), static_cast<unsigned>(g.batch)), block(64 * kThinWaves);
+    const dim3 grid(static_cast<unsigned>((g.M + 15) / 16), static_cast<unsigned>((g.N + 15) / 16), static_cast<unsigned>(g.batch));
+    const dim3 block(64 * kThinWaves);
     if (vec) gemm_thin_kernel<T, true><<<grid, block, 0, stream>>>(g);
     else gemm_thin_kernel<T, false><<<grid, block, 0, stream>>>(g);
     TTAMD_HIP_CHECK(hipGetLastError());
@@ -378,10 +381,25 @@ ttamd_status launch_gemm_thin(ttamd_dtype dt, const GemmArgs &g, int device, hip
         return dt == TTAMD_F32 ? launch_thin_k_typed<float>(dt, g, device, stream, fixed_scratch)
                                : launch_thin_k_typed<double>(dt, g, device, stream, fixed_scratch);
     }
-    if ((dt != TTAMD_F32 && dt != TTAMD_F64) || g.N > 16 || g.K < kThinMinK || g.colsum_out || g.batch > 65535) return TTAMD_OK;
+    if ((dt != TTAMD_F32 && dt != TTAMD_F64) || g.colsum_out || g.batch > 65535) return TTAMD_OK;
+    const int64_t blocks = static_cast<int64_t>((g.M + 15) / 16) * ((g.N + 15) / 16) * g.batch;
+    // A wave's share of k is a chain of memory round trips, one per chunk: beyond four chunks per wave (two when A's
+    // rows cannot be read as vectors) the tiles with their reduction split over workgroups are faster again
+    // (measured at 1024 x K x 10, f32: 12.2 against 14.9 us at K = 4096, 23.7 against 21.5 at K = 8192).
+    const int vec_len = dt == TTAMD_F32 ? 4 : 2;
+    const bool rows_vec = g.a_sk == 1 && g.K % vec_len == 0 && g.a_sm % vec_len == 0 && g.a_sb % vec_len == 0;
+    const int max_k = (rows_vec ? 4 : 2) * kThinWaves * 16 * vec_len;
+    const bool thin = g.N <= 16 && g.K >= kThinMinK && g.K <= max_k;
+    // A small output with a long reduction: on 64 x 64 tiles it would have a few tiles, split k over workgroups and add
+    // the parts in a second kernel.  As 16 x 16 blocks it fills the chip in one round of workgroups (two fit a CU).
+    const bool small = g.N > 16 && g.K >= kSmallMinK && g.K <= max_k && blocks <= kSmallMaxBlocks;
+    if (!thin && !small) return TTAMD_OK;
     *handled = true;
-    if (dt == TTAMD_F32) return launch_thin_typed<float>(g, stream, variant, variant_only, "thin_f32_16rows_vec4", "thin_f32_16rows");
-    return launch_thin_typed<double>(g, stream, variant, variant_only, "thin_f64_16rows_vec2", "thin_f64_16rows");
+    if (dt == TTAMD_F32)
+        return thin ? launch_thin_typed<float>(g, stream, variant, variant_only, "thin_f32_16rows_vec4", "thin_f32_16rows")
+                    : launch_thin_typed<float>(g, stream, variant, variant_only, "small_f32_16x16_vec4", "small_f32_16x16");
+    return thin ? launch_thin_typed<double>(g, stream, variant, variant_only, "thin_f64_16rows_vec2", "thin_f64_16rows")
+                : launch_thin_typed<double>(g, stream, variant, variant_only, "small_f64_16x16_vec2", "small_f64_16x16");
 }
 
 }  // namespace ttamd
