@@ -313,7 +313,7 @@ def detail_report(tt, np, path, cpu=True):
             if nonoverlap:
                 bwd_kernel = "pool_backward_window_kernel"
             else:
-                bwd_kernel = "pool_backward_quad_kernel" if op == "avg" else "pool_share_k3s2_kernel + pool_backward_quad_kernel"
+                bwd_kernel = "pool_backward_quad_kernel" if op == "avg" else "pool_backward_k3s2_tile_kernel"
             # algorithmic bytes of backward: grad_out and grad_input, plus the input and the result for max / min
             bwd_b = (in_b + out_b) if op == "avg" else (2 * in_b + 2 * out_b)
             stream_case(f"{op}_pool2d backward k{k} s{S_} p{P_} [64,64,112,112] f32", bwd_kernel, bwd_b,

@@ -46,7 +46,9 @@ def test_reference_shape_forward_backward_exact(tt, oracle, op, dtype):
                                   (2, 3, 9, 8, 3, 2, 1), (1, 2, 7, 12, 2, 1, 0), (2, 2, 10, 16, 4, 2, 1), (1, 2, 6, 8, 2, 1, 1),
                                   (1, 1, 5, 4, 3, 2, 0), (2, 1, 11, 20, 6, 3, 2), (1, 2, 9, 24, 5, 4, 2),
                                   # rows longer than a wave's 64 groups of four, and rows that end inside a wave
-                                  (1, 2, 9, 520, 3, 2, 1), (2, 1, 7, 44, 3, 2, 1), (1, 1, 6, 256, 3, 2, 1), (1, 2, 5, 260, 2, 1, 0)])
+                                  (1, 2, 9, 520, 3, 2, 1), (2, 1, 7, 44, 3, 2, 1), (1, 1, 6, 256, 3, 2, 1), (1, 2, 5, 260, 2, 1, 0),
+                                  # two and three input rows (every window hangs over an edge), a single group of four
+                                  (1, 2, 2, 4, 3, 2, 1), (2, 1, 2, 8, 3, 2, 1), (1, 1, 3, 4, 3, 2, 1)])
 def test_every_dtype_and_geometry_exact(tt, oracle, op, dtype, geom):
     Bn, Cc, H, W, k, S, P = geom
     rng = np.random.default_rng(sum(geom))

@@ -374,7 +374,8 @@ ttamd_status launch_thin_typed(const GemmArgs &g, hipStream_t stream, const char
 ttamd_status launch_gemm_thin(ttamd_dtype dt, const GemmArgs &g, int device, hipStream_t stream, const char **variant,
                               bool variant_only, bool *handled, bool fixed_scratch) {
     *handled = false;
-    if ((dt == TTAMD_F32 || dt == TTAMD_F64) && g.K <= 16 && g.N >= 16 && static_cast<int64_t>(g.M) * g.N >= kThinKMinOutput) {
+    if ((dt == TTAMD_F32 || dt == TTAMD_F64) && g.K <= 16 && g.N >= 16 && static_cast<int64_t>(g.M) * g.N >= kThinKMinOutput &&
+        g.batch <= 65535 && (g.M + 255) / 256 <= 65535) {  // (grid limits: anything beyond goes to the general kernels)
         *handled = true;
         *variant = dt == TTAMD_F32 ? "thin_f32_k16" : "thin_f64_k16";
         if (variant_only) return TTAMD_OK;

@@ -457,6 +457,116 @@ pool_share_k3s2_kernel(PoolGeom g, const R *__restrict__ gout, const R *__restri
     *reinterpret_cast<Pair<R> *>(share + o0) = amount;
 }
 
+// max / min backward for k == 3, stride == 2, padding == 1 on dense rows of 4n elements (at most kTileMaxWo output
+// columns) in ONE launch: a workgroup owns kTileRows output rows h0 .. of one plane and the 2 * kTileRows input rows
+// 2 h0 .. that receive from them.  First its lanes compute the shares of output rows h0 .. h0 + kTileRows (one more
+// row than it owns: the last input row also receives from the row below), one output pair per lane with the loads of
+// pool_share_k3s2_kernel, into LDS together with the results; after a barrier the lanes take the input rows four
+// elements at a time and add the shares of the covering outputs from LDS, in increasing (h, w).  Shares and sums are
+// formed exactly as the two kernels form them, but the shares never travel through memory (two launches move 870 MB
+// for a [64,64,112,112] f32 input, the input, result and both gradients are 514 MB), and the input rows the second
+// step reads were read by the first a moment ago.  (Counting the windows again in every lane that gathers -- no LDS,
+// no barrier -- is no faster than the two launches: each share is then computed by some 4.5 lanes and the kernel is
+// bound by its comparisons.)
+constexpr int kTileRows = 8, kTileMaxWo = 256;
+
+template <typename R>
+__global__ void __launch_bounds__(256)
+pool_backward_k3s2_tile_kernel(PoolGeom g, int tiles, FastDiv d_tiles, const R *__restrict__ gout, const R *__restrict__ x,
+                               const R *__restrict__ res, R *__restrict__ gin) {
+    __shared__ R s_share[(kTileRows + 1) * kTileMaxWo], s_target[(kTileRows + 1) * kTileMaxWo];
+    uint32_t plane, tile;
+    d_tiles.divmod(blockIdx.x, plane, tile);
+    const int h0 = static_cast<int>(tile) * kTileRows;
+    const R *src = plane_of(g, x, plane);
+    const int64_t obase = static_cast<int64_t>(plane) * (g.Ho * g.Wo);
+    // 1. shares of output rows h0 .. h0 + kTileRows (those that exist), one pair of outputs per lane and round
+    const int out_rows = g.Ho - h0 < kTileRows + 1 ? g.Ho - h0 : kTileRows + 1;
+    const uint32_t n_out = static_cast<uint32_t>(out_rows * g.Wo);
+    for (uint32_t first = 0; first < n_out; first += 512) {  // (workgroup-uniform bound: every lane shuffles)
+        const uint32_t want = first + threadIdx.x * 2;
+        const bool live = want < n_out;
+        const uint32_t pos = live ? want : n_out - 2;  // a lane beyond the end recomputes the last pair and drops it
+        uint32_t hr, w;
+        g.d_Wo.divmod(pos, hr, w);
+        const int h = h0 + static_cast<int>(hr), col = 2 * static_cast<int>(w);  // col = 4m
+        const bool load_left = threadIdx.x % 64 == 0 && col > 0;
+        R v[3][5];
+        bool rin[3];
+#pragma unroll
+        for (int p = 0; p < 3; ++p) {
+            const int hi = 2 * h - 1 + p;
+            rin[p] = static_cast<unsigned>(hi) < static_cast<unsigned>(g.H);
+            const R *row = src + static_cast<int64_t>(hi < 0 ? 0 : (hi >= g.H ? g.H - 1 : hi)) * g.xs_h + col;
+            const Quad<R> own = *reinterpret_cast<const Quad<R> *>(row);
+            R left = __shfl_up(own[3], 1);
+            if (load_left) left = row[-1];
+            v[p][0] = left;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) v[p][1 + j] = own[j];
+        }
+        const int64_t o0 = obase + static_cast<int64_t>(h) * g.Wo + w;
+        const Pair<R> target = *reinterpret_cast<const Pair<R> *>(res + o0), go = *reinterpret_cast<const Pair<R> *>(gout + o0);
+#pragma unroll
+        for (int o = 0; o < 2; ++o) {
+            R count = R(0);
+#pragma unroll
+            for (int p = 0; p < 3; ++p)
+#pragma unroll
+                for (int q = 0; q < 3; ++q) {
+                    const bool in = rin[p] && (o == 1 || q > 0 || col > 0);  // only column -1 can be outside (W = 4n)
+                    count += (in && v[p][2 * o + q] == target[o]) ? R(1) : R(0);
+                }
+            if (live) {
+                s_share[hr * kTileMaxWo + w + o] = go[o] / count;
+                s_target[hr * kTileMaxWo + w + o] = target[o];
+            }
+        }
+    }
+    __syncthreads();
+    // 2. input rows 2 h0 .. 2 h0 + 2 kTileRows - 1 (those that exist), four elements per lane and round
+    const int y0 = 2 * h0;
+    const int in_rows = g.H - y0 < 2 * kTileRows ? g.H - y0 : 2 * kTileRows;
+    const uint32_t n_in = static_cast<uint32_t>(in_rows * g.W);
+    for (uint32_t pos = threadIdx.x * 4; pos < n_in; pos += 1024) {
+        uint32_t yr, xw;
+        g.d_W.divmod(pos, yr, xw);
+        const int y = y0 + static_cast<int>(yr);
+        const Quad<R> mine = *reinterpret_cast<const Quad<R> *>(src + static_cast<int64_t>(y) * g.xs_h + xw);
+        // row y lies in the windows of output rows y / 2 and, for odd y, y / 2 + 1; the four columns in those of
+        // output columns 2m, 2m + 1, 2m + 2 (kCovers below)
+        const int hr_lo = static_cast<int>(yr) >> 1, c_lo = static_cast<int>(xw) >> 1;
+        int h_hi = (y + 1) >> 1;
+        h_hi = h_hi >= g.Ho ? g.Ho - 1 : h_hi;
+        const int n_rows = h_hi - (y >> 1) + 1;  // 1 or 2 covering output rows
+        R amount[6], target[6];
+#pragma unroll
+        for (int a = 0; a < 2; ++a)
+#pragma unroll
+            for (int b = 0; b < 3; ++b) {
+                const int c = c_lo + b < g.Wo ? c_lo + b : g.Wo - 1;  // (row hr_lo + 1 of the arrays always exists)
+                amount[a * 3 + b] = s_share[(hr_lo + a) * kTileMaxWo + c];
+                target[a * 3 + b] = s_target[(hr_lo + a) * kTileMaxWo + c];
+            }
+        Quad<R> acc;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            constexpr bool kCovers[4][3] = {{true, false, false}, {true, true, false}, {false, true, false}, {false, true, true}};
+            R sum = R(0);
+#pragma unroll
+            for (int a = 0; a < 2; ++a)
+#pragma unroll
+                for (int b = 0; b < 3; ++b) {
+                    if (!kCovers[j][b]) continue;  // (an output that does not cover the element would add +0)
+                    const bool valid = (a < n_rows) & (c_lo + b < g.Wo);
+                    sum += (valid && mine[j] == target[a * 3 + b]) ? amount[a * 3 + b] : R(0);
+                }
+            acc[j] = sum;
+        }
+        *reinterpret_cast<Quad<R> *>(gin + static_cast<int64_t>(plane) * (g.H * g.W) + static_cast<int64_t>(y) * g.W + xw) = acc;
+    }
+}
+
 // Backward for non-overlapping windows (stride == k, padding == 0), one lane per output: the window's elements
 // receive grad_out / (number of elements equal to the result) where they equal it (SELECT), or grad_out / k^2
 // each; an element gets its single contribution as 0 + amount, the value the reference's zero-initialised sum
@@ -657,6 +767,14 @@ ttamd_status backward_typed(int device, int op, const PoolGeom &g, const void *g
             else if (two) pool_backward_kernel<R, false, 2><<<in_grid, block, 0, st>>>(g, go, xi, rs, gi);
             else pool_backward_kernel<R, false, 0><<<in_grid, block, 0, st>>>(g, go, xi, rs, gi);
         } else {
+            const int64_t tiles = (g.Ho + kTileRows - 1) / kTileRows;
+            if (quad && k3s2p1 && pair_ok(gout) && pair_ok(res) && g.Wo <= kTileMaxWo && planes * tiles <= 0x7fffffff) {
+                // one launch, the shares stay in LDS
+                pool_backward_k3s2_tile_kernel<R><<<dim3(static_cast<unsigned>(planes * tiles)), block, 0, st>>>(
+                    g, static_cast<int>(tiles), make_fastdiv(static_cast<uint32_t>(tiles)), go, xi, rs, gi);
+                TTAMD_HIP_CHECK(hipGetLastError());
+                return TTAMD_OK;
+            }
             void *ws = nullptr;
             const size_t bytes = static_cast<size_t>(planes) * g.Ho * g.Wo * sizeof(R);
             if (ttamd_status s = stream_scratch(device, st, bytes ? bytes : sizeof(R), &ws)) return s;
