@@ -906,17 +906,22 @@ conv_fwd_direct_kernel(ConvGeom geo, const T *__restrict__ x, const T *__restric
 // at once (addresses clamped, invalid slots cleared by a select) and reads each slot's CMAX weights as one LDS
 // vector, so the loads overlap instead of forming a dependent chain per tap.  The sum runs over (o, p, q) in that
 // order, the order of conv_dgrad_kernel's reduction index.
-template <typename T, int CMAX, int NP>
+// UNIT (stride 1, NP == k): slot (i, j) is tap (i, j) for every lane, so a weight is the same for the whole wave: it
+// is read through the scalar cache straight from the weight tensor and multiplied as a scalar operand -- no LDS copy,
+// no per-lane LDS read per product.
+template <typename T, int CMAX, int NP, bool UNIT = false>
 __global__ void __launch_bounds__(256)
 conv_dgrad_slots_kernel(ConvGeom geo, const T *__restrict__ gout, const T *__restrict__ w, T *__restrict__ gin, int blocks_per_image) {
     extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
     T *const wl = reinterpret_cast<T *>(smem_raw);
     const int kk = geo.k * geo.k, HW = geo.H * geo.W, HoWo = geo.Ho * geo.Wo;
-    for (int i = threadIdx.x; i < geo.O * kk * CMAX; i += 256) {
-        const int c = i % CMAX, t = (i / CMAX) % kk, o = i / (CMAX * kk);
-        wl[i] = c < geo.C ? w[static_cast<int64_t>(o) * geo.w_so + c * kk + t] : T(0);
+    if constexpr (!UNIT) {
+        for (int i = threadIdx.x; i < geo.O * kk * CMAX; i += 256) {
+            const int c = i % CMAX, t = (i / CMAX) % kk, o = i / (CMAX * kk);
+            wl[i] = c < geo.C ? w[static_cast<int64_t>(o) * geo.w_so + c * kk + t] : T(0);
+        }
+        __syncthreads();
     }
-    __syncthreads();
     const int b = blockIdx.x / blocks_per_image;
     const int n = (blockIdx.x - b * blocks_per_image) * 256 + threadIdx.x;
     if (n >= HW) return;
@@ -948,14 +953,40 @@ conv_dgrad_slots_kernel(ConvGeom geo, const T *__restrict__ gout, const T *__res
     const T *wo = wl;
     const uint32_t plane_bytes = static_cast<uint32_t>(HoWo) * static_cast<uint32_t>(sizeof(T));
     uint32_t plane = 0;
-    for (int o = 0; o < geo.O; ++o, plane += plane_bytes, wo += kk * CMAX) {
+    // kOU output channels to a round, their NP * NP * kOU loads in flight together; the sum still runs over (o, p, q)
+    // in order.  (First layer of the MNIST example network, 1 -> 32 channels at batch 256: 28.7 us with one channel
+    // per round and the weights in LDS, 27.5 with four, 24.5 with four and scalar weights -- what is left is the
+    // 288 single-element loads per lane.)
+    constexpr int kOU = 4;
+    int o = 0;
+    for (; o + kOU <= geo.O; o += kOU, plane += kOU * plane_bytes, wo += kOU * kk * CMAX) {
+        T gv[kOU][NP * NP];
+#pragma unroll
+        for (int u = 0; u < kOU; ++u)
+#pragma unroll
+            for (int t = 0; t < NP * NP; ++t) gv[u][t] = Vec<T, 1>::load_at(grs, goff[t], plane + u * plane_bytes);
+#pragma unroll
+        for (int u = 0; u < kOU; ++u)
+#pragma unroll
+            for (int t = 0; t < NP * NP; ++t) {
+#pragma unroll
+                for (int c = 0; c < CMAX; ++c) {
+                    if constexpr (UNIT) acc[c] += w[static_cast<int64_t>(o + u) * geo.w_so + c * kk + (t / NP) * geo.k + t % NP] * gv[u][t];
+                    else acc[c] += wo[u * kk * CMAX + woff[t] + c] * gv[u][t];
+                }
+            }
+    }
+    for (; o < geo.O; ++o, plane += plane_bytes, wo += kk * CMAX) {
         T gv[NP * NP];
 #pragma unroll
         for (int t = 0; t < NP * NP; ++t) gv[t] = Vec<T, 1>::load_at(grs, goff[t], plane);
 #pragma unroll
         for (int t = 0; t < NP * NP; ++t) {
 #pragma unroll
-            for (int c = 0; c < CMAX; ++c) acc[c] += wo[woff[t] + c] * gv[t];
+            for (int c = 0; c < CMAX; ++c) {
+                if constexpr (UNIT) acc[c] += w[static_cast<int64_t>(o) * geo.w_so + c * kk + (t / NP) * geo.k + t % NP] * gv[t];
+                else acc[c] += wo[woff[t] + c] * gv[t];
+            }
         }
     }
     T *dst = gin + static_cast<int64_t>(b) * geo.C * HW + n;
@@ -1396,6 +1427,16 @@ ttamd_status backward_mfma(const ConvPlan &pl, const void *gout, void *gin, void
                                static_cast<T *>(gin), bpi);
         };
         auto by_windows = [&]<int CMAX>() -> ttamd_status {  // CMAX = C: no padded channel is multiplied
+            if (g.S == 1) {  // np == k: the weights are wave-uniform scalars, no LDS copy
+                auto unit = [&](auto kernel) -> ttamd_status {
+                    return launch_conv(kernel, 0, blocks, st, g, static_cast<const T *>(gout), static_cast<const T *>(pl.w),
+                                       static_cast<T *>(gin), bpi);
+                };
+                if (np == 1) return unit(conv_dgrad_slots_kernel<T, CMAX, 1, true>);
+                if (np == 2) return unit(conv_dgrad_slots_kernel<T, CMAX, 2, true>);
+                if (np == 3) return unit(conv_dgrad_slots_kernel<T, CMAX, 3, true>);
+                return unit(conv_dgrad_slots_kernel<T, CMAX, 4, true>);
+            }
             if (np == 1) return go(conv_dgrad_slots_kernel<T, CMAX, 1>);
             if (np == 2) return go(conv_dgrad_slots_kernel<T, CMAX, 2>);
             if (np == 3) return go(conv_dgrad_slots_kernel<T, CMAX, 3>);
