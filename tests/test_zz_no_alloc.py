@@ -84,6 +84,19 @@ def test_transposed_views_epilogue_and_integers(tt, oracle):
     got = _run(tt, lib.ttamd_batched_matmul_noalloc, tA, tB, ep)
     assert np.array_equal(got, _run(tt, lib.ttamd_batched_matmul, tA, tB, ep))
     assert np.array_equal(got[0], np.maximum(oracle.matmul(a[0], b[0]) + bias[None, :], 0))
+    # column sums: partial rows in the fixed array, of the tiles (1024 x 1024 x 1024) and of the short-reduction kernel
+    # on a matrix taller than one workgroup's rows (2500 x 10 x 1024)
+    for (N, K, M) in ((1024, 1024, 1024), (2500, 10, 1024)):
+        a, b = _pair(rng, np.float32, 1, N, K, M, integer_valued=True)
+        tA, tB = tt.Tensor.from_numpy(a), tt.Tensor.from_numpy(b)
+        sums = [tt.Tensor.empty((1, M), capi.F32) for _ in range(2)]
+        outs = []
+        for entry, cs in zip((lib.ttamd_batched_matmul_noalloc, lib.ttamd_batched_matmul), sums):
+            outs.append(_run(tt, entry, tA, tB, capi.Epilogue(None, 0, 0, 0, 0, None, None, cs.storage.ptr)))
+        want = oracle.matmul(a[0], b[0])
+        assert np.array_equal(outs[0], outs[1]) and np.array_equal(outs[0][0], want)
+        assert np.array_equal(sums[0].to_numpy(), sums[1].to_numpy())
+        assert np.array_equal(sums[0].to_numpy()[0], want.astype(np.float64).sum(0).astype(np.float32))  # integers: exact
     # integer dtypes take the vector-ALU kernel, which has no scratch
     ai, bi = rng.integers(-100, 100, (2, 70, 90)).astype(np.int32), rng.integers(-100, 100, (2, 90, 50)).astype(np.int32)
     tA, tB = tt.Tensor.from_numpy(ai), tt.Tensor.from_numpy(bi)
