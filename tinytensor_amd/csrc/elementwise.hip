@@ -493,7 +493,10 @@ __global__ void __launch_bounds__(256) cast_kernel(const T *__restrict__ a, View
 
 template <typename T, typename R>
 __global__ void __launch_bounds__(256) cast_vec_kernel(const T *__restrict__ a, R *__restrict__ out, int64_t nvec) {
-    constexpr int N = 16 / sizeof(T);
+    // 16 bytes of the wider side per lane: a widening cast then stores one vector per lane, so a wave's store covers
+    // contiguous memory (with 16 bytes of the input per lane a lane wrote two vectors 32 bytes apart from its
+    // neighbour's, every store instruction touching half of each line).
+    constexpr int N = 16 / (sizeof(T) > sizeof(R) ? sizeof(T) : sizeof(R));
     const int64_t step = static_cast<int64_t>(gridDim.x) * blockDim.x;
     for (int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < nvec; i += step) {
         const vec_t<T, N> x = stream_load(reinterpret_cast<const vec_t<T, N> *>(a) + i);
@@ -722,7 +725,7 @@ struct BoolByte {
 
 template <typename T, typename R>
 ttamd_status launch_cast(const void *a, const ViewDesc &va, void *out, int64_t numel, hipStream_t st) {
-    constexpr int N = 16 / sizeof(T);
+    constexpr int N = 16 / (sizeof(T) > sizeof(R) ? sizeof(T) : sizeof(R));  // (cast_vec_kernel's vector length)
     const bool dense = is_dense(va);
     int64_t done = 0;
     if (dense && aligned16(a) && aligned16(out) && numel >= N) {
