@@ -424,7 +424,9 @@ def test_small_tile_prefetch_depths(tt, dtype, layout, shape):
 @pytest.mark.parametrize("dtype", [np.float32, np.float64])
 @pytest.mark.parametrize("layout", LAYOUTS)
 @pytest.mark.parametrize("shape", [(1024, 1024, 1024), (1000, 512, 1001), (784, 1024, 1024), (130, 2048, 70), (1024, 832, 512),
-                                   (1024, 784, 1024), (960, 1000, 1024), (1024, 516, 1024)])
+                                   (1024, 784, 1024), (960, 1000, 1024), (1024, 516, 1024),
+                                   # the 128 x 128 tile (fp32) with a reduction of 2048 or more: whole and ragged tiles
+                                   (2048, 2048, 2048), (1900, 2056, 1988)])
 def test_two_halves_of_k_in_one_workgroup(tt, dtype, layout, shape):
     """Launches with at most one 64x64 workgroup per CU split the reduction between the two halves of a 512-lane
     workgroup when both halves have the same number of k tiles (784 = 392 + 392 and 1000 = 500 + 500 end in partial
@@ -441,6 +443,8 @@ def test_two_halves_of_k_in_one_workgroup(tt, dtype, layout, shape):
     name = be.batched_matmul_variant(tA, tB)
     if shape in ((1024, 1024, 1024), (784, 1024, 1024), (1024, 832, 512), (1024, 784, 1024), (960, 1000, 1024)):
         assert name.endswith("_halves"), name
+    if shape[1] >= 2048 and shape[0] > 1024 and dtype == np.float32:
+        assert name.startswith("mfma_f32_128x128") and name.endswith("_halves"), name
     if shape == (1024, 516, 1024) and dtype == np.float32:  # fp64 (k tile 16): 258 + 258, 17 tiles each
         assert not name.endswith("_halves"), name
     want = np.matmul(A.astype(np.float64), B.astype(np.float64))

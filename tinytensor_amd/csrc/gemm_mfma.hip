@@ -142,7 +142,7 @@ gemm_mfma_dual_kernel(GemmArgs g, int tiles_m, int tiles_n, int k_half) {
     using StA = Stager<T, BM, BK, A_KC, A_VEC, PF>;
     using StB = Stager<T, BN, BK, B_KC, B_VEC, PF>;
     using Engine = TileEngine<T, BM, BN, BK, WGM, WGN, StA, StB>;
-    static_assert(Engine::kAccPerLane * kThreads * sizeof(T) <= Engine::kLdsBytes, "the parked accumulators fit one half's buffers");
+    static_assert(Engine::kAccPerLane * kThreads * sizeof(T) <= 2 * Engine::kLdsBytes, "the parked accumulators fit the two halves' buffers");
     extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
     const int half = threadIdx.x / kThreads, tid = threadIdx.x % kThreads;  // wave-uniform
     T *const smem = reinterpret_cast<T *>(smem_raw + half * Engine::kLdsBytes);
@@ -509,10 +509,17 @@ ttamd_status launch_mfma_typed(const GemmArgs &g, int device, hipStream_t stream
     const bool dual = !(xxl || xl || mid || large) && vec && sp.ksplit == 1 && small_wgs <= 256 && half_tiles >= 8 &&
                       (g.K - k_half + TS::SBK - 1) / TS::SBK == half_tiles;
 
+    // The 128 x 128 tile (fp32) with at most one workgroup per CU and a reduction of 2048 or more: the same two halves
+    // (2048^3: 128.4 -> 126.5 us, 2048 x 4096 x 2048: 250.3 -> 244.6; shorter reductions lose: K = 784 53.8 -> 60.9).
+    const int64_t large_wgs = static_cast<int64_t>((g.M + TS::LBM - 1) / TS::LBM) * ((g.N + TS::LBN - 1) / TS::LBN) * g.batch;
+    const int large_half_tiles = (k_half + TS::LBK - 1) / TS::LBK;
+    const bool dual_large = sizeof(T) == 4 && large && large_wgs <= 256 && large_half_tiles >= 64 &&
+                            (g.K - k_half + TS::LBK - 1) / TS::LBK == large_half_tiles;
+
     static thread_local char name[112];
     char split_tag[24] = "";
     if (sp.ksplit > 1) snprintf(split_tag, sizeof(split_tag), "_splitk%d", sp.ksplit);
-    if (dual) snprintf(split_tag, sizeof(split_tag), "_halves");
+    if (dual || dual_large) snprintf(split_tag, sizeof(split_tag), "_halves");
     snprintf(name, sizeof(name), "%s_%s_a%s%d_b%s%d%s", TS::prefix, xxl ? "256x256" : (xl ? "256x128" : (mid ? "192x192" : (large ? "128x128" : "64x64"))), ca.kc ? "kc" : "mc",
              ca.vec, cb.kc ? "kc" : "mc", cb.vec, split_tag);
     *variant = name;
@@ -526,6 +533,7 @@ ttamd_status launch_mfma_typed(const GemmArgs &g, int device, hipStream_t stream
     }
     if constexpr (sizeof(T) == 4)
         if (mid) return launch_layouts<T, TS::MBM, TS::MBN, TS::MBK, 2, 2, VK, VK>(g, ca.kc, cb.kc, sp, device, stream);
+    if (dual_large) return launch_dual_layouts<T, TS::LBM, TS::LBN, TS::LBK, 2, 2, VK, 1>(g, ca.kc, cb.kc, device, stream, fixed_scratch);
     if (large) return launch_layouts<T, TS::LBM, TS::LBN, TS::LBK, 2, 2, VK, VK>(g, ca.kc, cb.kc, sp, device, stream);
     if (dual) return launch_dual_layouts<T, TS::SBM, TS::SBN, TS::SBK, 2, 2, VK, TS::SPF_DEEP>(g, ca.kc, cb.kc, device, stream, fixed_scratch);
     if (ca.vec > 1 && cb.vec > 1) {
