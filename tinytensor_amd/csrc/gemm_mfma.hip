@@ -533,7 +533,8 @@ ttamd_status launch_mfma_typed(const GemmArgs &g, int device, hipStream_t stream
     }
     if constexpr (sizeof(T) == 4)
         if (mid) return launch_layouts<T, TS::MBM, TS::MBN, TS::MBK, 2, 2, VK, VK>(g, ca.kc, cb.kc, sp, device, stream);
-    if (dual_large) return launch_dual_layouts<T, TS::LBM, TS::LBN, TS::LBK, 2, 2, VK, 1>(g, ca.kc, cb.kc, device, stream, fixed_scratch);
+    if constexpr (sizeof(T) == 4)
+        if (dual_large) return launch_dual_layouts<T, TS::LBM, TS::LBN, TS::LBK, 2, 2, VK, 1>(g, ca.kc, cb.kc, device, stream, fixed_scratch);
     if (large) return launch_layouts<T, TS::LBM, TS::LBN, TS::LBK, 2, 2, VK, VK>(g, ca.kc, cb.kc, sp, device, stream);
     if (dual) return launch_dual_layouts<T, TS::SBM, TS::SBN, TS::SBK, 2, 2, VK, TS::SPF_DEEP>(g, ca.kc, cb.kc, device, stream, fixed_scratch);
     if (ca.vec > 1 && cb.vec > 1) {

@@ -100,6 +100,9 @@ struct Vec<float, 4> {
     static __device__ __forceinline__ type load(__amdgpu_buffer_rsrc_t r, uint32_t off) {
         return __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(r, off, 0, 0));
     }
+    static __device__ __forceinline__ type load_at(__amdgpu_buffer_rsrc_t r, uint32_t off, uint32_t uniform_off) {
+        return __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(r, off, uniform_off, 0));
+    }
 };
 template <>
 struct Vec<double, 1> {
@@ -116,6 +119,9 @@ struct Vec<double, 2> {
     using type = f64x2;
     static __device__ __forceinline__ type load(__amdgpu_buffer_rsrc_t r, uint32_t off) {
         return __builtin_bit_cast(f64x2, __builtin_amdgcn_raw_buffer_load_b128(r, off, 0, 0));
+    }
+    static __device__ __forceinline__ type load_at(__amdgpu_buffer_rsrc_t r, uint32_t off, uint32_t uniform_off) {
+        return __builtin_bit_cast(f64x2, __builtin_amdgcn_raw_buffer_load_b128(r, off, uniform_off, 0));
     }
 };
 
@@ -187,6 +193,7 @@ struct Stager : TileLayout<T, ROWS, BK, KC> {
     int nval[P];  // MC only: valid components of the vector along the row dimension
     __amdgpu_buffer_rsrc_t rsrc;
     uint32_t k_step_b;
+    uint32_t k_off;  // wave-uniform part of the walk along k (see load)
     int tid;
     bool edge;
     bool row_mask;  // some vector of this tile holds rows both inside and outside the matrix: loads must mask
@@ -210,6 +217,7 @@ struct Stager : TileLayout<T, ROWS, BK, KC> {
         rsrc = make_rsrc(base, ext);
         const uint32_t s_row_b = static_cast<uint32_t>(s_row * sizeof(T)), s_k_b = static_cast<uint32_t>(s_k * sizeof(T));
         k_step_b = s_k_b * BK;
+        k_off = 0;
 #pragma unroll
         for (int p = 0; p < P; ++p) {
             const int line = line_of(p, tid), col = col_of(p, tid);
@@ -227,13 +235,23 @@ struct Stager : TileLayout<T, ROWS, BK, KC> {
 
     // Fetches the next tile into register slot SLOT; k_left = K - (first k of that tile).  MASK = false is
     // the steady state (full k tile, interior rows): loads only, no selects.
-    template <bool MASK, int SLOT = 0>
+    // UNIFORM_K: the step along k is kept in a scalar register and handed to the load as its scalar offset, so the
+    // walk costs one scalar add per tile instead of a vector add per load.  The hardware does not range-check the
+    // scalar offset: only for loads whose tile lies inside K (rows outside the matrix still have their out-of-range
+    // per-lane offset and load zeros).  The two forms may be mixed: the address is always voff + k_off.
+    template <bool MASK, int SLOT = 0, bool UNIFORM_K = false>
     __device__ __forceinline__ void load(int k_left) {
+        static_assert(!(MASK && UNIFORM_K), "a masked load relies on the range check of its whole offset");
         const bool k_tail = k_left < BK;
 #pragma unroll
         for (int p = 0; p < P; ++p) {
-            V v = Vec<T, VEC>::load(rsrc, voff[p]);
-            voff[p] += k_step_b;
+            V v;
+            if constexpr (UNIFORM_K) {
+                v = Vec<T, VEC>::load_at(rsrc, voff[p], k_off);
+            } else {
+                v = Vec<T, VEC>::load(rsrc, voff[p] + k_off);
+                voff[p] += k_step_b;
+            }
             if constexpr (!MASK) {
                 reg[SLOT][p] = v;
                 continue;
@@ -260,6 +278,7 @@ struct Stager : TileLayout<T, ROWS, BK, KC> {
             }
             reg[SLOT][p] = v;
         }
+        if constexpr (UNIFORM_K) k_off += k_step_b;
     }
 
     template <int SLOT = 0>
@@ -593,17 +612,20 @@ struct TileEngine {
                 for (int bn = 0; bn < NBN; ++bn) acc[bm][bn] = M::mma(fa.v[bm][j], fb.v[bn][j], acc[bm][bn]);
     }
 
-    template <bool MASK>
+    // CUR = kt & 1, the LDS buffer that holds tile kt: a template parameter in the unmasked loop, so that every LDS
+    // address of the step is a per-lane base (the same in every step) plus an immediate offset; -1 = taken from kt at
+    // run time (the masked loop, whose selects need the registers that two unrolled steps would take).
+    template <bool MASK, int CUR = -1>
     __device__ __forceinline__ void step_pipe(StA &sa, StB &sb, T *smem, int K, int kt, FrA &f0a, FrB &f0b) {
         constexpr int kHalf = (M::VK / 2) * NBM * NBN;  // MFMAs of half a chunk
         constexpr int kLoads = StA::P + StB::P;         // global loads (and LDS stores) of one tile, per lane
         constexpr int kReads = NBM + NBN;               // LDS read instructions of one chunk's fragments
-        const int cur = kt & 1;
+        const int cur = CUR >= 0 ? CUR : (kt & 1);
         FrA f1a;
         FrB f1b;
         const int k_left = K - (kt + 1) * BK;
-        sa.template load<MASK, 0>(k_left);
-        sb.template load<MASK, 0>(k_left);
+        sa.template load<MASK, 0, !MASK>(k_left);  // (the unmasked loop only requests tiles inside K)
+        sb.template load<MASK, 0, !MASK>(k_left);
         read_frags(smem, cur, 1, f1a, f1b);
         mma_half(f0a, f0b, 0);
         mma_half(f0a, f0b, M::VK / 2);
@@ -659,10 +681,15 @@ struct TileEngine {
             FrA f0a;
             FrB f0b;
             read_frags(smem, 0, 0, f0a, f0b);
+            int kt = 0;  // two steps to a round: the buffers alternate at compile time
             if (unmasked) {
-                for (int kt = 0; kt + 1 < KT; ++kt) step_pipe<false>(sa, sb, smem, K, kt, f0a, f0b);
+                for (; kt + 2 < KT; kt += 2) {
+                    step_pipe<false, 0>(sa, sb, smem, K, kt, f0a, f0b);
+                    step_pipe<false, 1>(sa, sb, smem, K, kt + 1, f0a, f0b);
+                }
+                if (kt + 1 < KT) step_pipe<false, 0>(sa, sb, smem, K, kt, f0a, f0b);
             } else {
-                for (int kt = 0; kt + 1 < KT; ++kt) step_pipe<true>(sa, sb, smem, K, kt, f0a, f0b);
+                for (; kt + 1 < KT; ++kt) step_pipe<true>(sa, sb, smem, K, kt, f0a, f0b);
             }
             const int cur = (KT - 1) & 1;
             FrA f1a;
