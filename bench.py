@@ -25,7 +25,7 @@ WARMUP_SECONDS = 0.25  # minimum untimed GPU work in front of the timed launches
 # FETCH_SIZE / WRITE_SIZE passes summarised in profiles/gemm_4096_f32_f64_mfma.txt (scaled by the same counters'
 # reading for a copy kernel of known size: x2.000 for reads, x1.000 for writes).  Only valid for that exact
 # kernel and size; reported as null otherwise.  Algorithmic bytes are 3 * 4096^2 * 4 = 201.3e6.
-MEASURED_TRAFFIC = {("mfma_f32_256x256_akc4_bmc4", 4096): (196856.1 * 2.0 + 65536.0) * 1024.0}
+MEASURED_TRAFFIC = {("mfma_f32_256x256_akc4_bmc4", 4096): (196783.0 * 2.0 + 65536.0) * 1024.0}
 
 
 def gpu_gemm_timing(tt, np, dtype, n, steps, warmup):

@@ -88,7 +88,8 @@ def test_variant_names_without_gpu(tt):
     assert variant(capi.F32, 1, n, n, n, (0, n, 1), (0, 1, n)) == "mfma_f32_256x256_akc4_bkc4"      # A . B^T
     assert variant(capi.F32, 1, n, n, n, (0, 1, n), (0, n, 1)) == "mfma_f32_256x256_amc4_bmc4"      # A^T . B
     assert variant(capi.F64, 1, n, n, n, (0, n, 1), (0, n, 1)) == "mfma_f64_256x128_akc2_bmc2"
-    assert variant(capi.F32, 1, 6144, 6144, 6144, (0, 6144, 1), (0, 6144, 1)) == "mfma_f32_128x128_akc4_bmc4"
+    assert variant(capi.F32, 1, 6144, 6144, 6144, (0, 6144, 1), (0, 6144, 1)) == "mfma_f32_192x192_akc4_bmc4"   # 1024 whole tiles: four rounds
+    assert variant(capi.F32, 1, 2816, 2816, 2816, (0, 2816, 1), (0, 2816, 1)) == "mfma_f32_128x128_akc4_bmc4"   # 484 tiles: one round at two per CU
     assert variant(capi.F32, 1, 3072, 3072, 3072, (0, 3072, 1), (0, 3072, 1)) == "mfma_f32_192x192_akc4_bmc4"  # 256 whole tiles of 192 x 192
     assert variant(capi.F32, 1, 3000, 3000, 3000, (0, 3000, 1), (0, 3000, 1)) == "mfma_f32_64x64_akc4_bmc4"    # ragged: no 192 x 192
     assert variant(capi.F64, 1, 3072, 3072, 3072, (0, 3072, 1), (0, 3072, 1)) == "mfma_f64_64x64_akc2_bmc2"    # fp32 only

@@ -60,6 +60,9 @@ ttamd_status fixed_scratch_address(int device, void **out) {
 // walks in one kernel the register allocator spills accumulators ahead of the branch for the sake of the heaviest
 // walk, and the plain store pays for it.
 constexpr int kEpiAny = 0, kEpiLean = 1, kEpiFull = 2, kEpiExt = 3;
+// kEpiLean for a problem made of whole tiles (M, N, K multiples of BM, BN, BK): no masked loop in the kernel, whose
+// registers otherwise cost the plain kernel of the biggest tiles 228 bytes of scratch per lane.
+constexpr int kEpiLeanWhole = 4;
 
 // The store's extensions for one workgroup: pointers moved to the batch, partial column sums to this tile row's rows.
 template <typename T>
@@ -105,10 +108,10 @@ gemm_mfma_kernel(GemmArgs g, int tiles_m, int tiles_n, int ksplit, int k_chunk, 
 
     Engine eng;
     eng.init(tid);
-    eng.run(sa, sb, smem, Kc, !sa.row_mask && !sb.row_mask);
+    eng.template run<EPI == kEpiLeanWhole>(sa, sb, smem, Kc, !sa.row_mask && !sb.row_mask);
 
     T *C = static_cast<T *>(g.C) + static_cast<int64_t>(batch) * g.M * g.N;
-    if constexpr (EPI == kEpiLean) {
+    if constexpr (EPI == kEpiLean || EPI == kEpiLeanWhole) {
         store_tile_dense<T, true>(eng, C, g.M, g.N, m0, n0, static_cast<const T *>(nullptr), 0, 0, 0);
     } else if constexpr (EPI == kEpiFull) {
         store_tile_dense<T, false>(eng, C, g.M, g.N, m0, n0, static_cast<const T *>(g.bias), g.bias_mode, g.relu, g.accumulate);
@@ -332,11 +335,17 @@ ttamd_status launch_variant(const GemmArgs &g, const SplitPlan &sp, int device, 
     }
     constexpr int kEpiA = kTwoKernels ? kEpiLean : kEpiAny, kEpiB = kTwoKernels ? kEpiFull : kEpiAny,
                   kEpiC = kTwoKernels ? kEpiExt : kEpiAny;
-    const int which = lean ? 0 : (ext_store(g) ? 2 : 1);
+    // the biggest tiles (one workgroup per CU, every register taken) have a kernel for problems of whole tiles
+    // (fp32 256 x 256 only: the fp64 256 x 128 kernel has no scratch with its masked loop and 460 bytes without)
+    constexpr bool kHasWhole = sizeof(T) == 4 && BM * BN >= 256 * 256 && A_VEC > 1 && B_VEC > 1;
+    constexpr int kEpiD = kHasWhole ? kEpiLeanWhole : kEpiA;
+    const bool whole = kHasWhole && lean && sp.ksplit == 1 && g.M % BM == 0 && g.N % BN == 0 && g.K % BK == 0 && g.K > 0;
+    const int which = whole ? 3 : (lean ? 0 : (ext_store(g) ? 2 : 1));
     auto kernel = which == 0   ? gemm_mfma_kernel<T, BM, BN, BK, WGM, WGN, A_KC, A_VEC, B_KC, B_VEC, PF, kEpiA>
                   : which == 1 ? gemm_mfma_kernel<T, BM, BN, BK, WGM, WGN, A_KC, A_VEC, B_KC, B_VEC, PF, kEpiB>
-                               : gemm_mfma_kernel<T, BM, BN, BK, WGM, WGN, A_KC, A_VEC, B_KC, B_VEC, PF, kEpiC>;
-    static bool configured[kMaxDevices][3] = {};  // raising the dynamic LDS limit: once per kernel and device
+                  : which == 2 ? gemm_mfma_kernel<T, BM, BN, BK, WGM, WGN, A_KC, A_VEC, B_KC, B_VEC, PF, kEpiC>
+                               : gemm_mfma_kernel<T, BM, BN, BK, WGM, WGN, A_KC, A_VEC, B_KC, B_VEC, PF, kEpiD>;
+    static bool configured[kMaxDevices][4] = {};  // raising the dynamic LDS limit: once per kernel and device
     const int slot = device >= 0 && device < kMaxDevices ? device : 0;
     if ((!configured[slot][which] || slot != device) && lds_bytes > 48 * 1024) {
         TTAMD_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
@@ -479,14 +488,18 @@ ttamd_status launch_mfma_typed(const GemmArgs &g, int device, hipStream_t stream
         const double round_time = 2.0 * bm_ * bn_ * static_cast<double>(g.K) * slots / (rate * scale);
         return (rounds + last) * round_time;
     };
-    const double t_small = estimate(TS::SBM, TS::SBN, 4, 131e12);
+    // The small tile sustains 139 TFLOP/s once several rounds overlap each other's first loads and stores (5120^3:
+    // 1.92 ms in 6.25 rounds); a launch pays for that ramp once, about 6 % of a round (2048^3 in exactly one round:
+    // 130 us, 132 TFLOP/s).
+    const double t_small = estimate(TS::SBM, TS::SBN, 4, 139e12) +
+                           0.06 * 2.0 * TS::SBM * TS::SBN * static_cast<double>(g.K) * 1024.0 / (139e12 * scale);
     constexpr bool f32 = sizeof(T) == 4;  // the fp64 big tiles run one workgroup per CU (accumulators in AGPRs)
-    const double t_large = vec ? estimate(TS::LBM, TS::LBN, f32 ? 2 : 1, f32 ? 145e12 : 141e12, 0.08) : 1e300;
-    const double t_xl = (TS::kHasXL && vec) ? estimate(TS::XBM, TS::XBN, f32 ? 2 : 1, f32 ? 145e12 : 147e12) : 1e300;
-    const double t_xxl = (TS::kHasXL && vec && sizeof(T) == 4) ? estimate(TS::YBM, TS::YBN, 1, 147e12) : 1e300;
+    const double t_large = vec ? estimate(TS::LBM, TS::LBN, f32 ? 2 : 1, f32 ? 150e12 : 148e12, 0.08) : 1e300;
+    const double t_xl = (TS::kHasXL && vec) ? estimate(TS::XBM, TS::XBN, f32 ? 2 : 1, f32 ? 149e12 : 152e12) : 1e300;
+    const double t_xxl = (TS::kHasXL && vec && sizeof(T) == 4) ? estimate(TS::YBM, TS::YBN, 1, 151e12) : 1e300;
     double t_mid = 1e300;
     if constexpr (sizeof(T) == 4)  // whole tiles only: its ragged edge tiles run at two thirds of the rate (5120^3: 2.9 ms against 2.0)
-        if (vec && g.M % TS::MBM == 0 && g.N % TS::MBN == 0) t_mid = estimate(TS::MBM, TS::MBN, 1, 141e12);
+        if (vec && g.M % TS::MBM == 0 && g.N % TS::MBN == 0) t_mid = estimate(TS::MBM, TS::MBN, 1, 149e12);
     const double t_best = std::min(std::min(std::min(t_xxl, t_xl), std::min(t_large, t_small)), t_mid);
     const bool xxl = t_xxl <= t_best;
     const bool xl = !xxl && t_xl <= t_best;

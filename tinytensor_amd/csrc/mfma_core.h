@@ -669,11 +669,14 @@ struct TileEngine {
         __builtin_amdgcn_sched_barrier(0);
     }
 
+    // WHOLE: the caller promises at compile time what `unmasked` says at run time (and that K > 0), so the masked loop
+    // and its registers are not part of the kernel at all.
+    template <bool WHOLE>
     __device__ __forceinline__ void run_pipe(StA &sa, StB &sb, T *smem, int K, bool unmasked) {
         static_assert(StA::kPF == 1 && BK / kChunk == 2, "the pipelined schedule is written for two chunks per k tile");
         const int KT = (K + BK - 1) / BK;
-        sa.template load<true, 0>(K);
-        sb.template load<true, 0>(K);
+        sa.template load<!WHOLE, 0>(K);
+        sb.template load<!WHOLE, 0>(K);
         sa.template store<0>(smem);
         sb.template store<0>(smem + kBOff);
         __syncthreads();
@@ -682,7 +685,7 @@ struct TileEngine {
             FrB f0b;
             read_frags(smem, 0, 0, f0a, f0b);
             int kt = 0;  // two steps to a round: the buffers alternate at compile time
-            if (unmasked) {
+            if (WHOLE || unmasked) {
                 for (; kt + 2 < KT; kt += 2) {
                     step_pipe<false, 0>(sa, sb, smem, K, kt, f0a, f0b);
                     step_pipe<false, 1>(sa, sb, smem, K, kt + 1, f0a, f0b);
@@ -702,10 +705,13 @@ struct TileEngine {
 
     // K: reduction length.  `rows_ok`: workgroup-uniform promise that every row of both operand tiles is inside
     // the matrix (a k tile that reaches past K is dealt with here).
+    // WHOLE (pipelined schedule only): rows_ok and K % BK == 0 hold for every workgroup of the launch.
+    template <bool WHOLE = false>
     __device__ __forceinline__ void run(StA &sa, StB &sb, T *smem, int K, bool rows_ok) {
         static_assert(StA::kPF == StB::kPF, "both operands use the same prefetch distance");
         static_assert(kPipe || kRotate, "no schedule for this tile shape");
-        if constexpr (kPipe) run_pipe(sa, sb, smem, K, rows_ok && K % BK == 0);
+        static_assert(!WHOLE || kPipe, "only the pipelined schedule has a form without masks");
+        if constexpr (kPipe) run_pipe<WHOLE>(sa, sb, smem, K, rows_ok && K % BK == 0);
         else run_rot(sa, sb, smem, K, rows_ok);
     }
 
