@@ -218,3 +218,32 @@ def test_blocks_of_a_closed_stream_serve_later_requests(tt):
         assert tt._capi.lib.ttamd_device_synchronize(0) == 0
     finally:
         other.close()
+
+
+def test_scalar_operands_are_filled_once(tt):
+    """A scalar operand of an element-wise call is a stride-0 view of a one-element tensor that is kept per value: the
+    recorded graph of a function that has run before holds no fill kernels, 0.0 and -0.0 are different constants, and
+    full() still hands out storage of its own."""
+    x = tt.Tensor.from_numpy(np.array([[-1.5, 2.0, 0.0, 3.0]], np.float32))
+    stream = tt.graph.Stream()
+    graph = None
+    try:
+        graph = tt.graph.Graph(stream, lambda: [x * 2.0, tt.where(x < 0.0, 0.0, 1.0), x * 2.0])
+        assert graph.num_nodes() == 4   # mul, lt, where, mul: no fills
+        graph.launch()
+        stream.synchronize()
+        assert np.array_equal(graph.outputs[0].to_numpy(), x.to_numpy() * 2)
+        assert np.array_equal(graph.outputs[1].to_numpy(), np.where(x.to_numpy() < 0, 0, 1).astype(np.float32))
+        assert np.array_equal(graph.outputs[2].to_numpy(), x.to_numpy() * 2)
+    finally:
+        if graph is not None:
+            graph.close()
+        stream.close()
+    pos, neg = (x * 0.0).to_numpy(), (x * -0.0).to_numpy()
+    assert np.array_equal(np.signbit(pos), np.signbit(x.to_numpy() * np.float32(0.0)))
+    assert np.array_equal(np.signbit(neg), np.signbit(x.to_numpy() * np.float32(-0.0)))
+    a, b = tt.full((2, 2), 7.0), tt.full((2, 2), 7.0)
+    assert a.storage is not b.storage and np.array_equal(a.to_numpy(), np.full((2, 2), 7, np.float32))
+    ints = tt.Tensor.from_numpy(np.arange(6, dtype=np.int32))
+    assert np.array_equal((ints * 3).to_numpy(), np.arange(6) * 3) and np.array_equal((ints * 3).to_numpy(), np.arange(6) * 3)
+

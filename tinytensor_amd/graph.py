@@ -34,6 +34,7 @@ def _runtime():
             "hipGraphInstantiate": [C.POINTER(vp), vp, C.POINTER(vp), C.c_char_p, C.c_size_t],
             "hipGraphLaunch": [vp, vp], "hipGraphExecDestroy": [vp], "hipGraphDestroy": [vp],
             "hipGraphGetNodes": [vp, C.POINTER(vp), C.POINTER(C.c_size_t)],
+            "hipStreamIsCapturing": [vp, C.POINTER(C.c_int)],
         }.items():
             fn = getattr(lib, name)
             fn.argtypes, fn.restype = args, C.c_int
@@ -45,6 +46,15 @@ def _call(name: str, *args) -> None:
     rc = getattr(_runtime(), name)(*args)
     if rc != 0:
         raise TTException(f"{name} failed with HIP error {rc}")
+
+
+def stream_is_capturing(handle) -> bool:
+    """Whether the stream with this hipStream_t handle (None or 0: the default stream) is recording a graph."""
+    if not handle:
+        return False
+    status = C.c_int(0)
+    _call("hipStreamIsCapturing", C.c_void_p(handle), C.byref(status))
+    return status.value != 0  # hipStreamCaptureStatusNone == 0
 
 
 class Stream:

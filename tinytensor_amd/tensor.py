@@ -217,7 +217,7 @@ class Tensor:
     # ---- elementwise ops around the GEMMs (frontend broadcasting, then one backend call) ----------
     def _binary(self, other, op: str) -> "Tensor":
         if not isinstance(other, Tensor):
-            other = full(self.shape, other, self.dtype, self.device)
+            other = _constant(self.shape, other, self.dtype, self.device)
         if other.dtype != self.dtype:  # operands are cast to promote_types(lhs, rhs) (tensor/tensor.cpp:2272-2274)
             dt = max(self.dtype, other.dtype)
             a, b = broadcast_tensors(self.to(dt), other.to(dt))
@@ -687,6 +687,30 @@ def full(shape, value, dtype: int = _capi.F32, device: Device = kAMD) -> Tensor:
     return Tensor(one.storage, dtype, shape, (0,) * len(shape), 0)
 
 
+_CONSTANTS: dict = {}  # (bytes of the value in its dtype, dtype, device id) -> one-element tensor
+
+
+def _constant(shape, value, dtype: int, device: Device) -> Tensor:
+    """A scalar operand of an element-wise call (`t * 2.0`, `where(c, 0.0, 1.0)`) as a stride-0 view of a one-element
+    tensor that is kept for the next call with the same value: such operands are only ever read, so one launch fills
+    the element the first time and later calls launch nothing (a training step written op by op issues ten of these
+    fills).  The element is filled on the current stream and the device synchronised before it goes into the table, so
+    that any stream may read it afterwards; a first use inside a stream capture cannot wait and stays a one-off
+    (the warm-up runs that precede a capture have normally met the value already).  `full()` itself never shares."""
+    shape = tuple(shape)
+    key = (np.array(value).astype(_NP_OF[dtype]).tobytes(), dtype, device.id)
+    one = _CONSTANTS.get(key)
+    if one is None:
+        one = get_backend(device).full(value, 1, dtype, device)
+        from .graph import stream_is_capturing
+        if not stream_is_capturing(_STREAM):
+            get_backend(device).synchronize(device.id)
+            if len(_CONSTANTS) >= 256:
+                _CONSTANTS.pop(next(iter(_CONSTANTS)))
+            _CONSTANTS[key] = one
+    return Tensor(one.storage, dtype, shape, (0,) * len(shape), 0)
+
+
 def broadcast_tensors(a: Tensor, b: Tensor):
     """Right-aligned broadcasting through unsqueeze + expand views (no data movement)."""
     while a.dim() < b.dim():
@@ -704,9 +728,9 @@ def broadcast_tensors(a: Tensor, b: Tensor):
 def where(cond: Tensor, lhs, rhs) -> Tensor:
     """tinytensor::where with scalar or tensor branches."""
     if not isinstance(lhs, Tensor):
-        lhs = full(cond.shape, lhs, rhs.dtype if isinstance(rhs, Tensor) else _capi.F32, cond.device)
+        lhs = _constant(cond.shape, lhs, rhs.dtype if isinstance(rhs, Tensor) else _capi.F32, cond.device)
     if not isinstance(rhs, Tensor):
-        rhs = full(cond.shape, rhs, lhs.dtype, cond.device)
+        rhs = _constant(cond.shape, rhs, lhs.dtype, cond.device)
     lhs, rhs = broadcast_tensors(lhs, rhs)
     cond, lhs = broadcast_tensors(cond, lhs)
     cond, rhs = broadcast_tensors(cond, rhs)
