@@ -299,6 +299,31 @@ def test_unaligned_views_fall_back_to_elementwise_loads(tt, oracle, dtype):
     check_close(got, oracle.matmul(A, B), A, B, dtype)
 
 
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+@pytest.mark.parametrize("N,Kp,M", [(130, 72, 150), (384, 256, 384), (1024, 1024, 1024), (320, 1000, 448)])
+def test_vectors_that_straddle_the_end_of_k_are_cut(tt, dtype, N, Kp, M):
+    """Rows padded to a whole number of 16-byte vectors, K one to three elements short of the pitch: the last vector of
+    a row holds elements on both sides of K.  The padding holds NaN, so a single element taken from beyond K (in either
+    operand: A's rows run along k, and so do the rows of B's storage, read as B^T) shows in every sum it reaches."""
+    rng = np.random.default_rng(N + Kp)
+    code = tt._capi.F32 if dtype == np.float32 else tt._capi.F64
+    vec = 16 // np.dtype(dtype).itemsize
+    be = tt.get_backend(tt.kAMD)
+    for short in range(1, vec):
+        K = Kp - short
+        baseA = rng.integers(-4, 5, size=(N, Kp)).astype(dtype)
+        baseBt = rng.integers(-4, 5, size=(M, Kp)).astype(dtype)
+        A, Bt = baseA[:, :K].copy(), baseBt[:, :K].copy()
+        baseA[:, K:] = np.nan
+        baseBt[:, K:] = np.nan
+        tA = tt.Tensor(tt.Tensor.from_numpy(baseA.ravel()).storage, code, (1, N, K), (N * Kp, Kp, 1), 0)
+        tB = tt.Tensor(tt.Tensor.from_numpy(baseBt.ravel()).storage, code, (1, K, M), (M * Kp, 1, Kp), 0)
+        variant = be.batched_matmul_variant(tA, tB)
+        assert f"akc{vec}_bkc{vec}" in variant, variant
+        got = be.batched_matmul(tA, tB).to_numpy()[0]
+        assert np.array_equal(got, naive_exact(A, np.ascontiguousarray(Bt.T))), (K, variant)
+
+
 def test_variant_selection(tt):
     be = tt.get_backend(tt.kAMD)
     f32 = np.float32

@@ -147,7 +147,12 @@ gemm_mfma_dual_kernel(GemmArgs g, int tiles_m, int tiles_n, int k_half) {
     using Engine = TileEngine<T, BM, BN, BK, WGM, WGN, StA, StB>;
     static_assert(Engine::kAccPerLane * kThreads * sizeof(T) <= 2 * Engine::kLdsBytes, "the parked accumulators fit the two halves' buffers");
     extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
-    const int half = threadIdx.x / kThreads, tid = threadIdx.x % kThreads;  // wave-uniform
+    // The half is the same for every lane of a wave.  Said through readfirstlane so that the compiler keeps it, and the
+    // half's length, k tile count and every loop condition and mask decision derived from it, in scalar registers
+    // (left as a function of threadIdx.x they are per-lane values: compares on the vector ALU, loops and branches by
+    // execution mask).
+    const int half = __builtin_amdgcn_readfirstlane(static_cast<int>(threadIdx.x / kThreads));
+    const int tid = threadIdx.x % kThreads;
     T *const smem = reinterpret_cast<T *>(smem_raw + half * Engine::kLdsBytes);
     int batch, tm, tn;
     decode_tile(remap_xcd(blockIdx.x, gridDim.x), tiles_m, tiles_n, batch, tm, tn);

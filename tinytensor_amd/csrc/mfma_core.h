@@ -242,38 +242,39 @@ struct Stager : TileLayout<T, ROWS, BK, KC> {
     template <bool MASK, int SLOT = 0, bool UNIFORM_K = false>
     __device__ __forceinline__ void load(int k_left) {
         static_assert(!(MASK && UNIFORM_K), "a masked load relies on the range check of its whole offset");
-        const bool k_tail = k_left < BK;
+        // A vector that lies wholly beyond K (or wholly in rows outside the matrix: init) is requested at the
+        // out-of-range offset and comes back as zeros.  Only a vector that straddles the edge needs a select on the
+        // loaded data, and a select makes the wave wait for its load on the spot, a full memory round trip per load
+        // with nothing else in flight: that is left to the layouts that can have such vectors (a k extent that is
+        // not a multiple of the vector, rows_left not a multiple of it), under a workgroup-uniform condition.
+        const bool k_straddle = KC && VEC > 1 && k_left > 0 && k_left < BK && k_left % VEC != 0;
 #pragma unroll
         for (int p = 0; p < P; ++p) {
             V v;
             if constexpr (UNIFORM_K) {
                 v = Vec<T, VEC>::load_at(rsrc, voff[p], k_off);
             } else {
-                v = Vec<T, VEC>::load(rsrc, voff[p] + k_off);
+                uint32_t off = voff[p] + k_off;
+                if constexpr (MASK) {
+                    if ((KC ? col_of(p, tid) : line_of(p, tid)) >= k_left) off = kOob;
+                }
+                v = Vec<T, VEC>::load(rsrc, off);
                 voff[p] += k_step_b;
             }
-            if constexpr (!MASK) {
-                reg[SLOT][p] = v;
-                continue;
-            }
-            if constexpr (KC) {
-                if (k_tail) {
-                    const int col = col_of(p, tid);
+            if constexpr (MASK && VEC > 1) {
+                if constexpr (KC) {
+                    if (k_straddle) {
+                        const int col = col_of(p, tid);
 #pragma unroll
-                    for (int j = 0; j < VEC; ++j)
-                        if (col + j >= k_left) zero_component<T, VEC>(v, j);
-                }
-            } else {
-                if (k_tail) {
-                    if (line_of(p, tid) >= k_left) {
-#pragma unroll
-                        for (int j = 0; j < VEC; ++j) zero_component<T, VEC>(v, j);
+                        for (int j = 0; j < VEC; ++j)
+                            if (col + j >= k_left) zero_component<T, VEC>(v, j);
                     }
-                }
-                if (VEC > 1 && edge) {
+                } else {
+                    if (row_mask) {
 #pragma unroll
-                    for (int j = 0; j < VEC; ++j)
-                        if (j >= nval[p]) zero_component<T, VEC>(v, j);
+                        for (int j = 0; j < VEC; ++j)
+                            if (j >= nval[p]) zero_component<T, VEC>(v, j);
+                    }
                 }
             }
             reg[SLOT][p] = v;
@@ -527,12 +528,14 @@ struct TileEngine {
         constexpr int PF = StA::kPF;
         constexpr int NC = BK / kChunk;
         const int KT = (K + BK - 1) / BK;
-        // Prologue: tile 0 goes straight to LDS, tiles 1 .. PF-1 are put in flight.
+        // Prologue: tiles 0 .. PF-1 are requested together, so that the first requests of a workgroup (the slowest
+        // it makes: nothing of its operands is in a cache yet) overlap instead of queueing behind tile 0's round
+        // trip; tile 0 then goes straight to LDS.
         sa.template load<true, 0>(K);
         sb.template load<true, 0>(K);
+        prefetch_rest<1>(sa, sb, K, KT);
         sa.template store<0>(smem);
         sb.template store<0>(smem + kBOff);
-        prefetch_rest<1>(sa, sb, K, KT);
         __syncthreads();
         // Tiles 0 .. KT-2; the first step has no pending chunk.  While kt + PF < KT a step also issues loads; the
         // remaining steps only drain the slots.
@@ -738,10 +741,10 @@ struct TileEngine {
     template <int S>
     __device__ __forceinline__ void prefetch_rest(StA &sa, StB &sb, int K, int KT) {
         if constexpr (S < StA::kPF) {
-            if (S < KT) {
-                sa.template load<true, S>(K - S * BK);
-                sb.template load<true, S>(K - S * BK);
-            }
+            // (unconditional: a tile beyond K is requested at out-of-range offsets and costs next to nothing, and
+            // without a branch the wait counters of the stores that follow are exact)
+            sa.template load<true, S>(K - S * BK);
+            sb.template load<true, S>(K - S * BK);
             prefetch_rest<S + 1>(sa, sb, K, KT);
         }
     }
