@@ -578,14 +578,22 @@ __device__ __forceinline__ void store_tile_padded_rows(Engine &eng, T *__restric
     };
     auto bias_of = [&](int ml) { return Vec<T, 1>::load(bias_m, static_cast<uint32_t>(m0 + ml) * kSz); };
     const bool pairs_ok = (w % 2 == 0) && (reinterpret_cast<uintptr_t>(C) % (2 * sizeof(T)) == 0);
-    eng.template for_each<true>(
-        pairs_ok, [&](int ml, int nl, T v, int) { buffer_store(out, offset_of(ml, nl), v + bias_of(ml)); },
-        [&](int ml, int nl, T v0, T v1, int) {
-            const T bv = bias_of(ml);
-            pair_t o;
-            o[0] = v0 + bv;
-            o[1] = v1 + bv;
-            buffer_store(out, offset_of(ml, nl), o);
+    // (phased walk: a block's bias loads go out together, then its stores)
+    T bv[Mfma<T>::NACC];
+    eng.template for_each<true, true>(
+        pairs_ok,
+        [&]<int PHASE>(int ml, int nl, T v, int, int e) {
+            if constexpr (PHASE != 1) bv[e] = bias_of(ml);
+            if constexpr (PHASE != 0) buffer_store(out, offset_of(ml, nl), v + bv[e]);
+        },
+        [&]<int PHASE>(int ml, int nl, T v0, T v1, int, int e) {
+            if constexpr (PHASE != 1) bv[e] = bias_of(ml);
+            if constexpr (PHASE != 0) {
+                pair_t o;
+                o[0] = v0 + bv[e];
+                o[1] = v1 + bv[e];
+                buffer_store(out, offset_of(ml, nl), o);
+            }
         });
 }
 

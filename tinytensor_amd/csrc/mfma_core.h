@@ -756,7 +756,14 @@ struct TileEngine {
     // `one`, slots bn and bn + 1 for `two`.
     // FENCE keeps the scheduler from hoisting the work of later blocks over the stores of earlier ones (an epilogue
     // that loads per element would otherwise hold a whole tile's loads in flight and spill).
-    template <bool FENCE = false, class One, class Two>
+    //
+    // The callbacks are templates over a phase and also receive e, the element's number inside its MFMA block (a
+    // compile-time constant after unrolling).  PHASED = false: one call per element, phase 2 (everything).  PHASED =
+    // true: a block's elements are walked twice, phase 0 (requests: the callback keeps what it loads in arrays indexed
+    // by e) and then phase 1 (arithmetic and stores).  A store followed by a load through another descriptor cannot be
+    // reordered by the compiler (they might alias), so a walk that loads and stores element by element is a chain of
+    // memory round trips, one per element; in two phases a block's loads are in flight together.
+    template <bool FENCE = false, bool PHASED = false, class One, class Two>
     __device__ __forceinline__ void for_each(bool pairs_ok, One one, Two two) {
         const int jcol = lane % M::MB;
         auto singles = [&]() {
@@ -765,8 +772,18 @@ struct TileEngine {
                 const int n = FrB::index_of(wn0, bn, jcol);
 #pragma unroll
                 for (int bm = 0; bm < NBM; ++bm) {
+                    if constexpr (PHASED) {
 #pragma unroll
-                    for (int e = 0; e < M::NACC; ++e) one(FrA::index_of(wm0, bm, M::acc_row(e, lane)), n, acc[bm][bn][e], bn);
+                        for (int e = 0; e < M::NACC; ++e)
+                            one.template operator()<0>(FrA::index_of(wm0, bm, M::acc_row(e, lane)), n, acc[bm][bn][e], bn, e);
+#pragma unroll
+                        for (int e = 0; e < M::NACC; ++e)
+                            one.template operator()<1>(FrA::index_of(wm0, bm, M::acc_row(e, lane)), n, acc[bm][bn][e], bn, e);
+                    } else {
+#pragma unroll
+                        for (int e = 0; e < M::NACC; ++e)
+                            one.template operator()<2>(FrA::index_of(wm0, bm, M::acc_row(e, lane)), n, acc[bm][bn][e], bn, e);
+                    }
                     if constexpr (FENCE) __builtin_amdgcn_sched_barrier(0);
                 }
             }
@@ -778,9 +795,21 @@ struct TileEngine {
                     const int n = FrB::index_of(wn0, 2 * pr, jcol);  // even column; n + 1 belongs to block 2p+1
 #pragma unroll
                     for (int bm = 0; bm < NBM; ++bm) {
+                        if constexpr (PHASED) {
 #pragma unroll
-                        for (int e = 0; e < M::NACC; ++e)
-                            two(FrA::index_of(wm0, bm, M::acc_row(e, lane)), n, acc[bm][2 * pr][e], acc[bm][2 * pr + 1][e], 2 * pr);
+                            for (int e = 0; e < M::NACC; ++e)
+                                two.template operator()<0>(FrA::index_of(wm0, bm, M::acc_row(e, lane)), n, acc[bm][2 * pr][e],
+                                                           acc[bm][2 * pr + 1][e], 2 * pr, e);
+#pragma unroll
+                            for (int e = 0; e < M::NACC; ++e)
+                                two.template operator()<1>(FrA::index_of(wm0, bm, M::acc_row(e, lane)), n, acc[bm][2 * pr][e],
+                                                           acc[bm][2 * pr + 1][e], 2 * pr, e);
+                        } else {
+#pragma unroll
+                            for (int e = 0; e < M::NACC; ++e)
+                                two.template operator()<2>(FrA::index_of(wm0, bm, M::acc_row(e, lane)), n, acc[bm][2 * pr][e],
+                                                           acc[bm][2 * pr + 1][e], 2 * pr, e);
+                        }
                         if constexpr (FENCE) __builtin_amdgcn_sched_barrier(0);
                     }
                 }
@@ -853,56 +882,79 @@ __device__ __forceinline__ void store_tile_dense(Engine &eng, T *__restrict__ C,
     T csum[Engine::NBN];  // sums of what this lane stores, per column slot
 #pragma unroll
     for (int i = 0; i < Engine::NBN; ++i) csum[i] = T(0);
-    auto finish = [&](T v, int ml, int nl, uint32_t off, int slot, bool valid) {
-        if constexpr (LEAN) return v;
-        v += Vec<T, 1>::load(bias_n, static_cast<uint32_t>(n0 + nl) * static_cast<uint32_t>(sizeof(T)));
-        v += Vec<T, 1>::load(bias_m, static_cast<uint32_t>(m0 + ml) * static_cast<uint32_t>(sizeof(T)));
-        if constexpr (EXT) v = Vec<T, 1>::load(zmask, off) < T(0) ? T(0) : v;  // absent mask: compares 0 < 0
-        v = (v > T(0) || !relu) ? v : T(0);
-        v += Vec<T, 1>::load(prev, off);
-        if constexpr (EXT) csum[slot] += valid ? v : T(0);
-        return v;
-    };
     auto positive = [](T v) { return v > T(0) ? v : T(0); };
     // pairs: n is even and N is even, so n + 1 < N whenever n < N and a wave writes whole row segments
     const bool pairs_ok = (N_ % 2 == 0) && (reinterpret_cast<uintptr_t>(C) % (2 * sizeof(T)) == 0) &&
                           (!EXT || (reinterpret_cast<uintptr_t>(ext.relu_out) % (2 * sizeof(T)) == 0 &&
                                     reinterpret_cast<uintptr_t>(ext.zmask) % (2 * sizeof(T)) == 0));
-    eng.template for_each<!LEAN>(
-        pairs_ok,
-        [&](int ml, int nl, T v, int slot) {
-            const uint32_t off = offset_of(ml, nl);
-            const T o = finish(v, ml, nl, off, slot, off != kOob);
-            buffer_store(out, off, o);
-            if constexpr (EXT) buffer_store(second, off, positive(o));
-        },
-        [&](int ml, int nl, T v0, T v1, int slot) {
-            const uint32_t off = offset_of(ml, nl);
-            pair_t o;
-            if constexpr (EXT) {  // the same steps as finish(), the mask and the old value fetched as pairs
-                const pair_t zz = Vec<T, 2>::load(zmask, off), pp = Vec<T, 2>::load(prev, off);
-                const T bm = Vec<T, 1>::load(bias_m, static_cast<uint32_t>(m0 + ml) * static_cast<uint32_t>(sizeof(T)));
-                const T in[2] = {v0, v1};
+    // What the walk loads for the elements of one MFMA block (see for_each: phase 0 requests, phase 1 uses).  Two phases
+    // for tiles with up to 64 accumulators per lane; the big tiles have no registers to spare for a block's loads and
+    // keep the element-by-element walk.
+    constexpr bool kPhased = !LEAN && Engine::kAccPerLane <= 64;
+    constexpr int NA = MI::NACC;
+    uint32_t offs[NA];
+    T l_bn[NA][2], l_bm[NA];
+    pair_t l_z[NA], l_p[NA];
+    constexpr uint32_t kSzU = static_cast<uint32_t>(sizeof(T));
+    // W = 1: a single element (component 0 of the pairs); W = 2: columns n and n + 1.  The arithmetic per element, in
+    // this order: + bias[n], + bias[m], mask, ReLU, + old value.
+    auto element = [&]<int PHASE, int W>(int ml, int nl, const T (&in)[W], int slot, int e) {
+        if constexpr (PHASE != 1) {
+            offs[e] = offset_of(ml, nl);
+            if constexpr (!LEAN) {
 #pragma unroll
-                for (int j = 0; j < 2; ++j) {
-                    T v = in[j] + Vec<T, 1>::load(bias_n, static_cast<uint32_t>(n0 + nl + j) * static_cast<uint32_t>(sizeof(T))) + bm;
-                    v = zz[j] < T(0) ? T(0) : v;
+                for (int j = 0; j < W; ++j) l_bn[e][j] = Vec<T, 1>::load(bias_n, static_cast<uint32_t>(n0 + nl + j) * kSzU);
+                l_bm[e] = Vec<T, 1>::load(bias_m, static_cast<uint32_t>(m0 + ml) * kSzU);
+                if constexpr (W == 2) {
+                    if constexpr (EXT) l_z[e] = Vec<T, 2>::load(zmask, offs[e]);  // (absent mask: zeros)
+                    l_p[e] = Vec<T, 2>::load(prev, offs[e]);
+                } else {
+                    if constexpr (EXT) l_z[e][0] = Vec<T, 1>::load(zmask, offs[e]);
+                    l_p[e][0] = Vec<T, 1>::load(prev, offs[e]);
+                }
+            }
+        }
+        if constexpr (PHASE != 0) {
+            const uint32_t off = offs[e];
+            T o[W];
+#pragma unroll
+            for (int j = 0; j < W; ++j) {
+                T v = in[j];
+                if constexpr (!LEAN) {
+                    v += l_bn[e][j];
+                    v += l_bm[e];
+                    if constexpr (EXT) v = l_z[e][j] < T(0) ? T(0) : v;
                     v = (v > T(0) || !relu) ? v : T(0);
-                    v += pp[j];
-                    csum[slot + j] += off != kOob ? v : T(0);
-                    o[j] = v;
+                    v += l_p[e][j];
+                    if constexpr (EXT) csum[slot + j] += off != kOob ? v : T(0);
+                }
+                o[j] = v;
+            }
+            if constexpr (W == 2) {
+                pair_t ov, rv;
+                ov[0] = o[0];
+                ov[1] = o[1];
+                buffer_store(out, off, ov);
+                if constexpr (EXT) {
+                    rv[0] = positive(o[0]);
+                    rv[1] = positive(o[1]);
+                    buffer_store(second, off, rv);
                 }
             } else {
-                o[0] = finish(v0, ml, nl, off, slot, off != kOob);
-                o[1] = finish(v1, ml, nl + 1, off + static_cast<uint32_t>(sizeof(T)), slot + 1, off != kOob);
+                buffer_store(out, off, o[0]);
+                if constexpr (EXT) buffer_store(second, off, positive(o[0]));
             }
-            buffer_store(out, off, o);
-            if constexpr (EXT) {
-                pair_t r;
-                r[0] = positive(o[0]);
-                r[1] = positive(o[1]);
-                buffer_store(second, off, r);
-            }
+        }
+    };
+    eng.template for_each<!LEAN, kPhased>(
+        pairs_ok,
+        [&]<int PHASE>(int ml, int nl, T v, int slot, int e) {
+            const T in[1] = {v};
+            element.template operator()<PHASE, 1>(ml, nl, in, slot, e);
+        },
+        [&]<int PHASE>(int ml, int nl, T v0, T v1, int slot, int e) {
+            const T in[2] = {v0, v1};
+            element.template operator()<PHASE, 2>(ml, nl, in, slot, e);
         });
     if constexpr (EXT) {
         if (ext.colsum) {  // workgroup-uniform
