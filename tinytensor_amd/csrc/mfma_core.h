@@ -460,36 +460,70 @@ struct TileEngine {
         constexpr int NC = BK / kChunk;
         static_assert(NC >= 2, "a k tile holds at least two chunks");
         constexpr int kChunkMfmas = M::VK * NBM * NBN;  // MFMAs of one chunk
-        constexpr int kStores = StA::P + StB::P;        // LDS store instructions of one tile (per lane)
+        constexpr int kStores = StA::P + StB::P;        // LDS store instructions (and global loads) of one tile, per lane
+        constexpr int kAllReads = 64;                   // "every LDS read of the region" for a scheduling group
         const int cur = kt & 1;
-        FrA f0a;
-        FrB f0b;
-        read_frags(smem, cur, 0, f0a, f0b);
+        // Fragments are double-buffered in registers: chunk c + 1 is requested from LDS before chunk c is multiplied,
+        // so a read has a chunk's MFMAs to arrive in (requested just in time it stalls the wave for the LDS latency,
+        // several times per step).
+        FrA fa[2];
+        FrB fb[2];
+        read_frags(smem, cur, 0, fa[0], fb[0]);
         if constexpr (LOAD) {
             const int k_left = K - (kt + PF) * BK;
             sa.template load<MASK, S>(k_left);
             sb.template load<MASK, S>(k_left);
         }
-        __builtin_amdgcn_sched_barrier(0);  // keep the requests ahead of the MFMA work
-        __builtin_amdgcn_s_setprio(3);  // multiply ahead of the other waves' address arithmetic (+1 % at 2048^3)
-        if constexpr (PENDING) mma_chunk(last_a, last_b);
-        compute_chunks(smem, cur, 0, NC - 2, f0a, f0b);
-        __builtin_amdgcn_sched_barrier(0);
-        compute_chunks(smem, cur, NC - 2, NC - 1, f0a, f0b);
-        read_frags(smem, cur, NC - 1, last_a, last_b);
-        sa.template store<(S + 1) % PF>(smem + (cur ^ 1) * StA::LDS_ELEMS);
-        // Keep A's stores ahead of B's, the order in which their loads were issued: each store then waits only for
-        // the loads up to its own instead of for all of them.
-        asm volatile("" ::: "memory");
-        sb.template store<(S + 1) % PF>(smem + kBOff + (cur ^ 1) * StB::LDS_ELEMS);
-        if constexpr (kChunkMfmas >= 2 * kStores) {
+        if constexpr (PENDING && !MASK && LOAD && kChunkMfmas >= 2) {
+            // The pending chunk's operands are in registers: its first MFMA goes out right after the barrier and the
+            // requests follow in its shadow (LDS reads first, they are needed first), instead of the matrix pipe
+            // idling while every wave of the workgroup issues its requests at the same moment.
+            __builtin_amdgcn_s_setprio(3);
+            mma_chunk(last_a, last_b);
+            constexpr int kGaps = kChunkMfmas - 1;
+            constexpr int kPerGap = (kStores + kGaps - 1) / kGaps;
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);          // MFMA
+            __builtin_amdgcn_sched_group_barrier(0x100, kAllReads, 0);  // DS read
 #pragma unroll
-            for (int i = 0; i < kStores; ++i) {
-                __builtin_amdgcn_sched_group_barrier(0x008, kChunkMfmas / kStores > 2 ? 2 : 1, 0);  // MFMA
-                __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);                                  // DS write
+            for (int i = 0; i < kGaps; ++i) {
+                __builtin_amdgcn_sched_group_barrier(0x020, kPerGap, 0);  // VMEM read
+                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
             }
+            __builtin_amdgcn_sched_barrier(0);
+        } else {
+            __builtin_amdgcn_sched_barrier(0);  // keep the requests ahead of the MFMA work
+            __builtin_amdgcn_s_setprio(3);      // multiply ahead of the other waves' address arithmetic (+1 % at 2048^3)
+            if constexpr (PENDING) mma_chunk(last_a, last_b);
         }
-        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int c = 0; c < NC - 1; ++c) {
+            // Request chunk c + 1 (the tile's last chunk goes to the registers that wait across the barrier), then
+            // multiply chunk c; the last multiplied chunk also parks tile kt + 1 in the other LDS buffer, its stores
+            // slotted between the MFMAs.
+            if (c + 1 < NC - 1) read_frags(smem, cur, c + 1, fa[(c + 1) & 1], fb[(c + 1) & 1]);
+            else read_frags(smem, cur, NC - 1, last_a, last_b);
+            if (c == NC - 2) {
+                sa.template store<(S + 1) % PF>(smem + (cur ^ 1) * StA::LDS_ELEMS);
+                // Keep A's stores ahead of B's, the order in which their loads were issued: each store then waits only
+                // for the loads up to its own instead of for all of them.
+                asm volatile("" ::: "memory");
+                sb.template store<(S + 1) % PF>(smem + kBOff + (cur ^ 1) * StB::LDS_ELEMS);
+            }
+            mma_chunk(fa[c & 1], fb[c & 1]);
+            __builtin_amdgcn_sched_group_barrier(0x100, kAllReads, 0);
+            if (c == NC - 2) {
+                if constexpr (kChunkMfmas >= 2 * kStores) {
+#pragma unroll
+                    for (int i = 0; i < kStores; ++i) {
+                        __builtin_amdgcn_sched_group_barrier(0x008, kChunkMfmas / kStores > 2 ? 2 : 1, 0);  // MFMA
+                        __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);                                  // DS write
+                    }
+                }
+            } else {
+                __builtin_amdgcn_sched_group_barrier(0x008, kChunkMfmas, 0);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
         __builtin_amdgcn_s_setprio(0);
         __syncthreads();
     }
