@@ -425,22 +425,6 @@ struct TileEngine {
 #pragma unroll
                 for (int bn = 0; bn < NBN; ++bn) acc[bm][bn] = M::mma(fa.v[bm][j], fb.v[bn][j], acc[bm][bn]);
     }
-    // MFMA work of chunks [c0, c1) of the tile in LDS buffer `buf`; chunk 0 takes the fragments in (f0a, f0b),
-    // which were requested earlier.
-    __device__ __forceinline__ void compute_chunks(const T *smem, int buf, int c0, int c1, const FrA &f0a, const FrB &f0b) {
-#pragma unroll
-        for (int c = c0; c < c1; ++c) {
-            if (c == 0) {
-                mma_chunk(f0a, f0b);
-            } else {
-                FrA fa;
-                FrB fb;
-                read_frags(smem, buf, c, fa, fb);
-                mma_chunk(fa, fb);
-            }
-        }
-    }
-
     // One pipeline step for tile kt.  The loop is rotated so that the barrier sits between reading the last chunk's
     // fragments and multiplying them:
     //   on entry the barrier that published tile kt has just been passed and (PENDING) the fragments of the
@@ -468,17 +452,20 @@ struct TileEngine {
         // several times per step).
         FrA fa[2];
         FrB fb[2];
+        constexpr bool kMfmaFirst = PENDING && !MASK && LOAD && kChunkMfmas >= 2;
+        // (s_setprio is a fixed point for the instruction scheduler: where the requests are to be moved behind the
+        // first MFMA it has to come before them)
+        if constexpr (kMfmaFirst) __builtin_amdgcn_s_setprio(3);
         read_frags(smem, cur, 0, fa[0], fb[0]);
         if constexpr (LOAD) {
             const int k_left = K - (kt + PF) * BK;
             sa.template load<MASK, S>(k_left);
             sb.template load<MASK, S>(k_left);
         }
-        if constexpr (PENDING && !MASK && LOAD && kChunkMfmas >= 2) {
+        if constexpr (kMfmaFirst) {
             // The pending chunk's operands are in registers: its first MFMA goes out right after the barrier and the
             // requests follow in its shadow (LDS reads first, they are needed first), instead of the matrix pipe
             // idling while every wave of the workgroup issues its requests at the same moment.
-            __builtin_amdgcn_s_setprio(3);
             mma_chunk(last_a, last_b);
             constexpr int kGaps = kChunkMfmas - 1;
             constexpr int kPerGap = (kStores + kGaps - 1) / kGaps;
@@ -625,7 +612,19 @@ struct TileEngine {
             FrB f0b;
             read_frags(smem, cur, 0, f0a, f0b);
             if (KT > 1) mma_chunk(last_a, last_b);
-            compute_chunks(smem, cur, 0, NC, f0a, f0b);
+            // Only the chunks that hold some k below K: the rest of a partial tile is zeros (K = 392 = 12 tiles + 8
+            // spends one chunk on its last tile instead of four).
+            const int chunks = (K - (KT - 1) * BK + kChunk - 1) / kChunk;
+            mma_chunk(f0a, f0b);
+#pragma unroll
+            for (int c = 1; c < NC; ++c) {
+                if (c < chunks) {  // workgroup-uniform
+                    FrA fa;
+                    FrB fb;
+                    read_frags(smem, cur, c, fa, fb);
+                    mma_chunk(fa, fb);
+                }
+            }
         }
     }
 
