@@ -154,11 +154,41 @@ __global__ void __launch_bounds__(64 * WGM * WGN * KS, 1) conv_patch_kernel(Conv
         }
     }
 
-    // ---- once per workgroup: the weight block.  It is copied through the still unused patch area with 16-byte
-    // vectors, segment by segment (one output row's [C][k k] in the forward layout), and moved from there to A in
-    // the order k' = tap * C + c: per (row, reduction channel) pair k*k reads a float apart and k*k writes C floats
-    // apart, the lanes along the axis in which pairs lie k*k floats apart.
-    {
+    // ---- once per workgroup: the weight block, into A in the order k' = tap * C + c.
+    // 3 x 3 kernels: a lane takes (row, reduction channel) pairs, reads the pair's nine taps (consecutive floats in
+    // memory in both weight layouts) straight from memory, every load of its pairs in flight together, and writes them
+    // C floats apart; the lanes run along the axis in which pairs lie nine floats apart, so a load instruction covers
+    // a contiguous stretch of the weight and a store instruction consecutive floats of A.
+    // Other kernel sizes: the block is copied through the still unused patch area with 16-byte vectors, segment by
+    // segment (one output row's [C][k k] in the forward layout), and moved from there to A, per pair k*k reads a float
+    // apart and k*k writes C floats apart.
+    if (a.k == 3) {
+        const int step = a.w_flip ? -C : C;
+        const __amdgpu_buffer_rsrc_t wsrc = make_rsrc(a.w, a.weight_bytes);
+        const int n_pairs = a.n_seg * a.n_fast;
+#pragma unroll 1
+        for (int v = tid; v < n_pairs; v += kPairs * NT) {
+            float *dst[kPairs];
+            float taps[kPairs][9];
+#pragma unroll
+            for (int i = 0; i < kPairs; ++i) {
+                const int vv = v + i * NT < n_pairs ? v + i * NT : v;  // (beyond the end: the first one again)
+                uint32_t slow, fast;
+                a.d_wfast.divmod(static_cast<uint32_t>(vv), slow, fast);
+                const int row = a.w_rows_fast ? static_cast<int>(fast) : static_cast<int>(slow);
+                const int red = a.w_rows_fast ? static_cast<int>(slow) : static_cast<int>(fast);
+                // rows beyond the last output channel are requested out of range and arrive as zeros
+                const uint32_t off = m0 + row < a.O ? static_cast<uint32_t>((m0 + row) * a.w_row + red * a.w_red) * 4u : kOob;
+                dst[i] = A + row * a.lda + red + (a.w_flip ? 8 * C : 0);
+#pragma unroll
+                for (int u = 0; u < 9; ++u) taps[i][u] = Vec<float, 1>::load(wsrc, off + 4u * u);
+            }
+#pragma unroll
+            for (int i = 0; i < kPairs; ++i)
+#pragma unroll
+                for (int u = 0; u < 9; ++u) dst[i][u * step] = taps[i][u];
+        }
+    } else {
         const int k2 = a.k * a.k;
         const int seg_vecs = a.seg_len / 4;
         const int step = a.w_flip ? -C : C;
@@ -218,32 +248,13 @@ __global__ void __launch_bounds__(64 * WGM * WGN * KS, 1) conv_patch_kernel(Conv
             }
             __syncthreads();
             const int n_pairs = (s1 - s0) * a.n_fast;
-            if (k2 == 9) {
 #pragma unroll 1
-                for (int v = tid; v < n_pairs; v += kPairs * NT) {  // kPairs pairs per step: their LDS latencies overlap
-                    const float *src[kPairs];
-                    float *dst[kPairs];
-                    float taps[kPairs][9];
-#pragma unroll
-                    for (int i = 0; i < kPairs; ++i) {
-                        pair_of(v + i * NT < n_pairs ? v + i * NT : v, s0, src[i], dst[i]);  // (beyond the end: the first one again)
-#pragma unroll
-                        for (int u = 0; u < 9; ++u) taps[i][u] = src[i][u];
-                    }
-#pragma unroll
-                    for (int i = 0; i < kPairs; ++i)
-#pragma unroll
-                        for (int u = 0; u < 9; ++u) dst[i][u * step] = taps[i][u];
-                }
-            } else {
+            for (int v = tid; v < n_pairs; v += NT) {
+                const float *src;
+                float *dst;
+                pair_of(v, s0, src, dst);
 #pragma unroll 1
-                for (int v = tid; v < n_pairs; v += NT) {
-                    const float *src;
-                    float *dst;
-                    pair_of(v, s0, src, dst);
-#pragma unroll 1
-                    for (int t = 0; t < k2; ++t) dst[t * step] = src[t];
-                }
+                for (int t = 0; t < k2; ++t) dst[t * step] = src[t];
             }
         }
     }
