@@ -805,7 +805,7 @@ __global__ void __launch_bounds__(256) reduce_splits_stream_kernel(const T *__re
 
 // The same sum for many parts of a tile of middling length (grad_weight's one partial tile per workgroup): a workgroup
 // owns 64 consecutive elements, each of its four waves adds a contiguous quarter of the parts in increasing order --
-// every load a whole coalesced line of the wave, eight in flight -- and the four sums are added in order.
+// every load a whole coalesced line of the wave, up to sixteen in flight -- and the four sums are added in order.
 template <typename T>
 __global__ void __launch_bounds__(256) reduce_splits_ranges_kernel(const T *__restrict__ partial, T *__restrict__ out, int64_t n, int splits) {
     __shared__ T red[4][64];
@@ -816,6 +816,13 @@ __global__ void __launch_bounds__(256) reduce_splits_ranges_kernel(const T *__re
     T acc = T(0);
     if (i < n) {
         int s = s0;
+        for (; s + 16 <= s1; s += 16) {  // (sixteen in flight: a quarter of 128 parts is two round trips, not four)
+            T v[16];
+#pragma unroll
+            for (int u = 0; u < 16; ++u) v[u] = partial[static_cast<int64_t>(s + u) * n + i];
+#pragma unroll
+            for (int u = 0; u < 16; ++u) acc += v[u];
+        }
         for (; s + 8 <= s1; s += 8) {
             T v[8];
 #pragma unroll
