@@ -429,14 +429,16 @@ struct TileEngine {
     // fragments and multiplying them:
     //   on entry the barrier that published tile kt has just been passed and (PENDING) the fragments of the
     //   previous tile's last chunk wait in registers (last_a, last_b);
-    //   1. request chunk 0 of tile kt from LDS and (LOAD) tile kt + PF from memory into slot kt % PF;
-    //   2. multiply the pending chunk: its MFMAs cover the LDS latency of step 1, which is otherwise exposed after
-    //      every barrier when a SIMD has few waves to run;
-    //   3. multiply chunks 0 .. NC-2 of tile kt; during the last of them read the last chunk's fragments into
-    //      (last_a, last_b) and park tile kt + 1 (slot (kt + 1) % PF) in the other LDS buffer, its stores slotted
-    //      between the MFMAs;
+    //   1. request chunk 0 of tile kt from LDS and (LOAD) tile kt + PF from memory into slot kt % PF, and multiply
+    //      the pending chunk: its MFMAs cover the LDS latency of the request, which is otherwise exposed after every
+    //      barrier when a SIMD has few waves to run; in the unmasked loop the first of them is issued ahead of the
+    //      requests;
+    //   2. for c = 0 .. NC-2: request chunk c + 1 of tile kt from LDS (the last chunk's fragments go to (last_a,
+    //      last_b)), then multiply chunk c;
+    //   3. the last multiplied chunk also parks tile kt + 1 (slot (kt + 1) % PF) in the other LDS buffer, its stores
+    //      slotted between the MFMAs;
     //   4. barrier.
-    // The other LDS buffer was last read in part 3 of the previous step (before its barrier), so it may be
+    // The other LDS buffer was last read in part 2 of the previous step (before its barrier), so it may be
     // overwritten here; tile kt's buffer is only read.
     template <int S, bool LOAD, bool MASK, bool PENDING>
     __device__ __forceinline__ void step_rot(StA &sa, StB &sb, T *smem, int K, int kt) {
