@@ -804,37 +804,44 @@ __global__ void __launch_bounds__(256) reduce_splits_stream_kernel(const T *__re
 }
 
 // The same sum for many parts of a tile of middling length (grad_weight's one partial tile per workgroup): a workgroup
-// owns 64 consecutive elements, each of its four waves adds a contiguous quarter of the parts in increasing order --
-// every load a whole coalesced line of the wave, up to sixteen in flight -- and the four sums are added in order.
+// owns 64 consecutive elements, each of its eight waves adds a contiguous eighth of the parts in increasing order --
+// every load a whole coalesced line of the wave, up to sixteen in flight (128 parts: one round trip per wave) -- and
+// the eight sums are added in order.
 template <typename T>
-__global__ void __launch_bounds__(256) reduce_splits_ranges_kernel(const T *__restrict__ partial, T *__restrict__ out, int64_t n, int splits) {
-    __shared__ T red[4][64];
+__global__ void __launch_bounds__(512) reduce_splits_ranges_kernel(const T *__restrict__ partial, T *__restrict__ out, int64_t n, int splits) {
+    constexpr int kWaves = 8;
+    __shared__ T red[kWaves][64];
     const int lane = threadIdx.x % 64, w = threadIdx.x / 64;
     const int64_t i = static_cast<int64_t>(blockIdx.x) * 64 + lane;
-    const int per = (splits + 3) / 4;
+    const int per = (splits + kWaves - 1) / kWaves;
     const int s0 = w * per, s1 = s0 + per < splits ? s0 + per : splits;
     T acc = T(0);
     if (i < n) {
         int s = s0;
-        for (; s + 16 <= s1; s += 16) {  // (sixteen in flight: a quarter of 128 parts is two round trips, not four)
+        for (; s + 16 <= s1; s += 16) {
             T v[16];
 #pragma unroll
             for (int u = 0; u < 16; ++u) v[u] = partial[static_cast<int64_t>(s + u) * n + i];
 #pragma unroll
             for (int u = 0; u < 16; ++u) acc += v[u];
         }
-        for (; s + 8 <= s1; s += 8) {
-            T v[8];
+        for (; s + 4 <= s1; s += 4) {
+            T v[4];
 #pragma unroll
-            for (int u = 0; u < 8; ++u) v[u] = partial[static_cast<int64_t>(s + u) * n + i];
+            for (int u = 0; u < 4; ++u) v[u] = partial[static_cast<int64_t>(s + u) * n + i];
 #pragma unroll
-            for (int u = 0; u < 8; ++u) acc += v[u];
+            for (int u = 0; u < 4; ++u) acc += v[u];
         }
         for (; s < s1; ++s) acc += partial[static_cast<int64_t>(s) * n + i];
     }
     red[w][lane] = acc;
     __syncthreads();
-    if (w == 0 && i < n) out[i] = ((red[0][lane] + red[1][lane]) + red[2][lane]) + red[3][lane];
+    if (w == 0 && i < n) {
+        T v = red[0][lane];
+#pragma unroll
+        for (int k = 1; k < kWaves; ++k) v += red[k][lane];
+        out[i] = v;
+    }
 }
 
 // out[i] = sum over parts of partial[s][i], by whichever of the kernels suits the shape: the streaming one when
@@ -847,7 +854,7 @@ ttamd_status launch_reduce_splits(const T *partial, T *out, int64_t n, int split
         const int64_t blocks = (n / VEC + 255) / 256;
         reduce_splits_stream_kernel<T><<<dim3(static_cast<unsigned>(blocks)), dim3(256), 0, st>>>(partial, out, n, splits);
     } else if (splits >= 32 && n >= 4096) {
-        reduce_splits_ranges_kernel<T><<<dim3(static_cast<unsigned>((n + 63) / 64)), dim3(256), 0, st>>>(partial, out, n, splits);
+        reduce_splits_ranges_kernel<T><<<dim3(static_cast<unsigned>((n + 63) / 64)), dim3(512), 0, st>>>(partial, out, n, splits);
     } else {
         reduce_splits_kernel<T><<<dim3(static_cast<unsigned>((n + 15) / 16)), dim3(256), 0, st>>>(partial, out, n, splits);
     }
