@@ -425,9 +425,10 @@ def main():
         def fused_step():
             z1, a1 = tt.linear_relu(xs, P1, c1); z2, a2 = tt.linear_relu(a1, P2, c2); y = tt.linear(a2, P3, c3)
             loss, gy, db3 = tt.mse_loss(y, ts, grad=True, bias_grad=True)
-            dz2, dW3, db2 = tt.linear_backward(gy, a2, P3, relu_input=z2)
-            dz1, dW2, db1 = tt.linear_backward(dz2, a1, P2, relu_input=z1)
-            dX, dW1, _ = tt.linear_backward(dz1, xs, P1, bias_grad=False)
+            # (bias gradients of layers 1 and 2 from the vectors of dz that the weight-gradient products stage)
+            dz2, dW3, _ = tt.linear_backward(gy, a2, P3, relu_input=z2, bias_grad=False)
+            dz1, dW2, db2 = tt.linear_backward(dz2, a1, P2, relu_input=z1, bias_grad="own")
+            dX, dW1, db1 = tt.linear_backward(dz1, xs, P1, bias_grad="own")
             return [loss, dW1, db1, dW2, db2, dW3, db3, dX]
 
         def ops_step():

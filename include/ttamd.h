@@ -75,7 +75,8 @@ typedef struct ttamd_view4 {
  * element-wise steps that autograd places around the backward GEMMs of a Linear layer.
  * Order of application to each element v of A.B:
  *   v += bias;  v = 0 where relu_grad_input < 0;  v = max(v, 0) if relu;  v += out if accumulate;
- *   out = v;  relu_out = max(v, 0);  colsum_out[column] += v. */
+ *   out = v;  relu_out = max(v, 0);  colsum_out[column] += v.
+ * rhs_colsum_out does not depend on the product. */
 typedef struct ttamd_epilogue {
     const void *bias; /* device pointer, same dtype as the GEMM, or NULL                      */
     int32_t bias_mode;/* 0 none, 1 = bias[column] (Linear), 2 = bias[row] (conv channel)      */
@@ -94,6 +95,12 @@ typedef struct ttamd_epilogue {
      * order by a second small kernel (deterministic; not the reference's row-by-row order).  f32/f64 on the
      * matrix-core kernels only; not together with `accumulate`. */
     void *colsum_out;
+    /* Sum of the right operand over its rows (k), [B,M] (or NULL): when the product is a Linear layer's weight
+     * gradient x^T . dy (TensorBatchedMatmul::backward, autograd/binary_ops.cpp:173-179), the right operand is dy and
+     * its column sums are the bias gradient (nn/linear.cpp:45-48), taken from the vectors the product stages anyway
+     * where its kernel can, else by a launch of its own.  The right operand must be dense row-major; f32/f64.  Added
+     * in a fixed order (deterministic; not the reference's row-by-row order). */
+    void *rhs_colsum_out;
 } ttamd_epilogue;
 
 /* ---- library / device ------------------------------------------------------------------ */

@@ -53,6 +53,16 @@ def test_validation_without_gpu(tt):
     v.stride[1] = -1
     assert lib.ttamd_batched_matmul(0, capi.F32, 1, 2, 2, 2, C.byref(v), C.byref(v), None, None, None) == capi.ERR_INVALID_ARGUMENT
     assert lib.ttamd_batched_matmul(0, capi.F32, 1, 2, 2, 2, None, None, None, None, None) == capi.ERR_INVALID_ARGUMENT
+    # the right operand's column sums: f32 / f64 and a dense row-major right operand (checked before any device work)
+    a, b, ep = capi.View3(), capi.View3(), capi.Epilogue()
+    a.data = b.data = 256
+    ep.rhs_colsum_out = 512
+    for i, (sa, sb) in enumerate(zip((4, 2, 1), (4, 1, 2))):   # rhs as a transposed view
+        a.stride[i], b.stride[i] = sa, sb
+    assert lib.ttamd_batched_matmul(0, capi.F32, 1, 2, 2, 2, C.byref(a), C.byref(b), C.c_void_p(1024), C.byref(ep), None) == capi.ERR_INVALID_ARGUMENT
+    assert b"dense row-major" in lib.ttamd_last_error_string()
+    b.stride[1], b.stride[2] = 2, 1
+    assert lib.ttamd_batched_matmul(0, capi.I32, 1, 2, 2, 2, C.byref(a), C.byref(b), C.c_void_p(1024), C.byref(ep), None) == capi.ERR_UNSUPPORTED_DTYPE
     # conv geometry errors
     v4 = capi.View4()
     assert lib.ttamd_conv2d_forward(0, capi.F32, C.byref(v4), C.byref(v4), None, None, 1, 3, 8, 8, 4, 3, 0, 0, None) == capi.ERR_INVALID_ARGUMENT

@@ -103,22 +103,69 @@ def test_mse_loss_forward_and_backward(tt, dtype, shape):
     assert none_g is None and none_cs is None and only_loss.to_numpy()[0] == loss.to_numpy()[0]
 
 
-def fused_mlp_step(tt, x, t, params):
-    """The training step of benchmark configuration 5 from the fused forms: 3 forward launches (+ the split reduction's
-    sum for the 10-column head), the loss with its gradient and the head's bias gradient in one, and per layer one GEMM
-    for dx (mask and bias gradient in its store, + the sum of the partial rows) and one for dW."""
+def fused_mlp_step(tt, x, t, params, own=False):
+    """The training step of benchmark configuration 5 from the fused forms: 3 forward launches, the loss with its
+    gradient and the head's bias gradient in one, and per layer one GEMM for dx (the ReLU-backward mask in its store) and
+    one for dW.  The bias gradients of layers 1 and 2 are column sums of dz: taken in the store of the GEMM that writes
+    dz (+ the sum of the partial rows), or (`own`) from the vectors of dz that the layer's dW GEMM stages."""
     (W1, b1), (W2, b2), (W3, b3) = params
     z1, a1 = tt.linear_relu(x, W1, b1)
     z2, a2 = tt.linear_relu(a1, W2, b2)
     y = tt.linear(a2, W3, b3)
     loss, gy, db3 = tt.mse_loss(y, t, grad=True, bias_grad=True)
-    dz2, dW3, db2 = tt.linear_backward(gy, a2, W3, relu_input=z2)
-    dz1, dW2, db1 = tt.linear_backward(dz2, a1, W2, relu_input=z1)
-    dX, dW1, _ = tt.linear_backward(dz1, x, W1, bias_grad=False)
+    if own:
+        dz2, dW3, _ = tt.linear_backward(gy, a2, W3, relu_input=z2, bias_grad=False)
+        dz1, dW2, db2 = tt.linear_backward(dz2, a1, W2, relu_input=z1, bias_grad="own")
+        dX, dW1, db1 = tt.linear_backward(dz1, x, W1, bias_grad="own")
+    else:
+        dz2, dW3, db2 = tt.linear_backward(gy, a2, W3, relu_input=z2)
+        dz1, dW2, db1 = tt.linear_backward(dz2, a1, W2, relu_input=z1)
+        dX, dW1, _ = tt.linear_backward(dz1, x, W1, bias_grad=False)
     return dict(y=y, loss=loss, dW1=dW1, db1=db1, dW2=dW2, db2=db2, dW3=dW3, db3=db3, dX=dX, z1=z1, z2=z2)
 
 
-def test_fused_mlp_training_step_matches_the_oracle_and_fits_15_launches(tt, oracle):
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+@pytest.mark.parametrize("a_transposed", [False, True])
+@pytest.mark.parametrize("shape", [(1, 1024, 1024, 1024), (1, 784, 1024, 1024), (1, 1024, 1000, 1000), (2, 512, 832, 520), (1, 960, 516, 1024),
+                                   (1, 1024, 1024, 10), (1, 200, 96, 136), (2, 130, 70, 151), (1, 2048, 64, 2048), (1, 300, 7, 52),
+                                   (1, 256, 512, 256), (1, 64, 1, 64)])
+def test_right_operand_column_sums(tt, dtype, a_transposed, shape):
+    """rhs_colsum_out = the right operand summed over k, whichever kernel takes the product: the two-half kernel adds
+    up the vectors it stages (the first four shapes, a Linear layer's weight gradient x^T . dy among them: ragged
+    columns, a partial last k tile, batches), every other kernel leaves it to a launch of its own.  Exact on
+    integer-valued data; the product itself is not affected."""
+    B, N, K, M = shape
+    rng = np.random.default_rng(N + 3 * K + M)
+    a = rng.integers(-3, 4, (B, N, K)).astype(dtype)
+    b = rng.integers(-3, 4, (B, K, M)).astype(dtype)
+    be = tt.get_backend(tt.kAMD)
+    ta = tt.Tensor.from_numpy(np.ascontiguousarray(a.transpose(0, 2, 1))).permute(0, 2, 1) if a_transposed else tt.Tensor.from_numpy(a)
+    tb = tt.Tensor.from_numpy(b)
+    sums = tt.Tensor.from_numpy(np.full((B, M), 77, dtype))
+    got = be.batched_matmul(ta, tb, rhs_colsum_out=sums).to_numpy()
+    assert np.array_equal(got, np.matmul(a.astype(np.float64), b.astype(np.float64)).astype(dtype))
+    assert np.array_equal(sums.to_numpy(), b.sum(axis=1)), _variant(tt, ta, tb)
+    # with the other options of the store in the same call
+    bias = rng.integers(-5, 6, (M,)).astype(dtype)
+    sums2 = tt.Tensor.from_numpy(np.zeros((B, M), dtype))
+    got = be.batched_matmul(ta, tb, bias=tt.Tensor.from_numpy(bias), bias_mode=1, relu=True, rhs_colsum_out=sums2).to_numpy()
+    assert np.array_equal(got, np.maximum(np.matmul(a.astype(np.float64), b.astype(np.float64)) + bias, 0).astype(dtype))
+    assert np.array_equal(sums2.to_numpy(), b.sum(axis=1))
+
+
+def test_right_operand_column_sums_need_a_dense_operand(tt):
+    be = tt.get_backend(tt.kAMD)
+    a = tt.Tensor.from_numpy(np.ones((1, 64, 64), np.float32))
+    bt = tt.Tensor.from_numpy(np.ones((1, 64, 64), np.float32)).permute(0, 2, 1)
+    with pytest.raises(tt.TTException):
+        be.batched_matmul(a, bt, rhs_colsum_out=tt.Tensor.from_numpy(np.zeros((1, 64), np.float32)))
+    ai = tt.Tensor.from_numpy(np.ones((1, 64, 64), np.int32))
+    with pytest.raises(tt.TTException):
+        be.batched_matmul(ai, ai, rhs_colsum_out=tt.Tensor.from_numpy(np.zeros((1, 64), np.int32)))
+
+
+@pytest.mark.parametrize("own", [False, True])
+def test_fused_mlp_training_step_matches_the_oracle_and_fits_15_launches(tt, oracle, own):
     X = oracle.Generator(0).uniform_real(0.0, 1.0, (1024, 784))
     T = oracle.Generator(1).uniform_real(0.0, 1.0, (1024, 10))
     g = oracle.Generator(0)
@@ -126,13 +173,13 @@ def test_fused_mlp_training_step_matches_the_oracle_and_fits_15_launches(tt, ora
     d = tt.Tensor.from_numpy
     x, t = d(X), d(T)
     params = [(d(W), d(b)) for W, b in params_h]
-    got = {k: v.to_numpy() for k, v in fused_mlp_step(tt, x, t, params).items()}
+    got = {k: v.to_numpy() for k, v in fused_mlp_step(tt, x, t, params, own).items()}
     masks = (np.where(got["z1"] < 0, np.float32(0), np.float32(1)), np.where(got["z2"] < 0, np.float32(0), np.float32(1)))
     want = mlp_train_step(X, T, params_h, lambda a, b: oracle.matmul(a, b),
                           lambda a, b, gr: tuple(v[0] for v in oracle.matmul_backward(a[None], b[None], gr[None])), masks=masks)
-    own = mlp_train_step(X, T, params_h, lambda a, b: oracle.matmul(a, b),
+    cpu = mlp_train_step(X, T, params_h, lambda a, b: oracle.matmul(a, b),
                          lambda a, b, gr: tuple(v[0] for v in oracle.matmul_backward(a[None], b[None], gr[None])))
-    assert sum(int(np.sum(a != b)) for a, b in zip(masks, own["masks"])) <= 8   # z within rounding of 0
+    assert sum(int(np.sum(a != b)) for a, b in zip(masks, cpu["masks"])) <= 8   # z within rounding of 0
     for key in ("y", "dW1", "db1", "dW2", "db2", "dW3", "db3", "dX"):
         assert got[key].shape == want[key].shape, key
         assert max_rel_error(got[key], want[key]) <= 1e-4, key
@@ -141,8 +188,8 @@ def test_fused_mlp_training_step_matches_the_oracle_and_fits_15_launches(tt, ora
     stream = tt.graph.Stream()
     graph = None
     try:
-        graph = tt.graph.Graph(stream, lambda: list(fused_mlp_step(tt, x, t, params).values()))
-        assert graph.num_nodes() <= 15, graph.num_nodes()
+        graph = tt.graph.Graph(stream, lambda: list(fused_mlp_step(tt, x, t, params, own).values()))
+        assert graph.num_nodes() <= (10 if own else 15), graph.num_nodes()
         graph.launch()
         stream.synchronize()
         for k, v in zip(("y", "loss", "dW1", "db1", "dW2", "db2", "dW3", "db3", "dX"), graph.outputs):

@@ -97,6 +97,18 @@ def test_transposed_views_epilogue_and_integers(tt, oracle):
         assert np.array_equal(outs[0], outs[1]) and np.array_equal(outs[0][0], want)
         assert np.array_equal(sums[0].to_numpy(), sums[1].to_numpy())
         assert np.array_equal(sums[0].to_numpy()[0], want.astype(np.float64).sum(0).astype(np.float32))  # integers: exact
+    # the right operand's column sums, from the two-half kernel's staged vectors (x^T . dy at 1024^3) and from a launch of
+    # their own behind a split reduction (320 x 512 x 416): neither allocates
+    for (N, K, M, transposed) in ((1024, 1024, 1024, True), (320, 512, 416, False)):
+        a, b = _pair(rng, np.float32, 1, N, K, M, integer_valued=True)
+        tA = tt.Tensor.from_numpy(np.ascontiguousarray(a.transpose(0, 2, 1))).permute(0, 2, 1) if transposed else tt.Tensor.from_numpy(a)
+        tB = tt.Tensor.from_numpy(b)
+        sums = [tt.Tensor.empty((1, M), capi.F32) for _ in range(2)]
+        outs = []
+        for entry, cs in zip((lib.ttamd_batched_matmul_noalloc, lib.ttamd_batched_matmul), sums):
+            outs.append(_run(tt, entry, tA, tB, capi.Epilogue(None, 0, 0, 0, 0, None, None, None, cs.storage.ptr)))
+        assert np.array_equal(outs[0], outs[1]) and np.array_equal(outs[0][0], oracle.matmul(a[0], b[0]))
+        assert np.array_equal(sums[0].to_numpy(), sums[1].to_numpy()) and np.array_equal(sums[0].to_numpy()[0], b[0].sum(0))
     # integer dtypes take the vector-ALU kernel, which has no scratch
     ai, bi = rng.integers(-100, 100, (2, 70, 90)).astype(np.int32), rng.integers(-100, 100, (2, 90, 50)).astype(np.int32)
     tA, tB = tt.Tensor.from_numpy(ai), tt.Tensor.from_numpy(bi)

@@ -29,7 +29,8 @@ class View4(C.Structure):
 
 class Epilogue(C.Structure):
     _fields_ = [("bias", C.c_void_p), ("bias_mode", C.c_int32), ("relu", C.c_int32), ("accumulate", C.c_int32),
-                ("reserved", C.c_int32), ("relu_out", C.c_void_p), ("relu_grad_input", C.c_void_p), ("colsum_out", C.c_void_p)]
+                ("reserved", C.c_int32), ("relu_out", C.c_void_p), ("relu_grad_input", C.c_void_p), ("colsum_out", C.c_void_p),
+                ("rhs_colsum_out", C.c_void_p)]
 
 
 def _bind(lib: C.CDLL) -> None:

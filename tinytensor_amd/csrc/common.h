@@ -91,6 +91,10 @@ struct GemmArgs {
     void *colsum_out;      // [batch, N], written by the kernel that adds the partial rows
     void *colsum_partial;  // [batch, colsum_rows, N] partial sums, filled in by the launcher (scratch)
     int colsum_rows;
+    // [batch, N] = B summed over k (B dense row-major), or null.  A launcher whose kernel writes it sets *rhs_colsum_done
+    // (host side only); otherwise the dispatcher adds B's rows in a launch of its own after the product.
+    void *rhs_colsum;
+    bool *rhs_colsum_done;
 };
 
 // Launchers (defined in gemm_mfma.hip / gemm_simt.hip).  `variant_only`: fill *variant with the

@@ -67,8 +67,18 @@ ttamd_status build_args(ttamd_dtype dtype, int B, int N, int K, int M, const tta
             set_error("batched_matmul: colsum_out is implemented for f32 and f64");
             return TTAMD_ERR_UNSUPPORTED_DTYPE;
         }
+        if (ep->rhs_colsum_out) {
+            if (dtype != TTAMD_F32 && dtype != TTAMD_F64) {
+                set_error("batched_matmul: rhs_colsum_out is implemented for f32 and f64");
+                return TTAMD_ERR_UNSUPPORTED_DTYPE;
+            }
+            if (rhs->stride[2] != 1 || rhs->stride[1] != M || (B > 1 && rhs->stride[0] != static_cast<int64_t>(K) * M)) {
+                set_error("batched_matmul: rhs_colsum_out needs a dense row-major right operand");
+                return TTAMD_ERR_INVALID_ARGUMENT;
+            }
+        }
         if (reinterpret_cast<uintptr_t>(ep->relu_out) % esz != 0 || reinterpret_cast<uintptr_t>(ep->relu_grad_input) % esz != 0 ||
-            reinterpret_cast<uintptr_t>(ep->colsum_out) % esz != 0) {
+            reinterpret_cast<uintptr_t>(ep->colsum_out) % esz != 0 || reinterpret_cast<uintptr_t>(ep->rhs_colsum_out) % esz != 0) {
             set_error("batched_matmul: epilogue pointers must be aligned to the element size");
             return TTAMD_ERR_INVALID_ARGUMENT;
         }
@@ -95,19 +105,15 @@ ttamd_status build_args(ttamd_dtype dtype, int B, int N, int K, int M, const tta
     g->colsum_out = ep ? ep->colsum_out : nullptr;
     g->colsum_partial = nullptr;
     g->colsum_rows = 0;
+    g->rhs_colsum = ep ? ep->rhs_colsum_out : nullptr;
+    g->rhs_colsum_done = nullptr;
     return TTAMD_OK;
 }
 
-ttamd_status batched_matmul(int device, ttamd_dtype dtype, int B, int N, int K, int M, const ttamd_view3 *lhs,
-                            const ttamd_view3 *rhs, void *out, const ttamd_epilogue *epilogue, void *stream, bool fixed_scratch) {
-    GemmArgs g;
-    if (ttamd_status s = build_args(dtype, B, N, K, M, lhs, rhs, out, epilogue, &g, true)) return s;
-    if (ttamd_status s = use_device(device)) return s;
-    if (B == 0 || N == 0 || M == 0) return TTAMD_OK;
-    hipStream_t st = static_cast<hipStream_t>(stream);
+ttamd_status run_product(ttamd_dtype dtype, const GemmArgs &g, int device, hipStream_t st, bool fixed_scratch) {
     const char *variant = nullptr;
     bool handled = false;
-    if (K > 0) {
+    if (g.K > 0) {
         if (ttamd_status s = launch_gemm_thin(dtype, g, device, st, &variant, false, &handled, fixed_scratch)) return s;
         if (handled) return TTAMD_OK;
         if (ttamd_status s = launch_gemm_mfma(dtype, g, device, st, &variant, false, &handled, fixed_scratch)) return s;
@@ -119,6 +125,21 @@ ttamd_status batched_matmul(int device, ttamd_dtype dtype, int B, int N, int K, 
         return TTAMD_ERR_INVALID_ARGUMENT;
     }
     return launch_gemm_simt(dtype, g, st, &variant, false);
+}
+
+ttamd_status batched_matmul(int device, ttamd_dtype dtype, int B, int N, int K, int M, const ttamd_view3 *lhs,
+                            const ttamd_view3 *rhs, void *out, const ttamd_epilogue *epilogue, void *stream, bool fixed_scratch) {
+    GemmArgs g;
+    if (ttamd_status s = build_args(dtype, B, N, K, M, lhs, rhs, out, epilogue, &g, true)) return s;
+    if (ttamd_status s = use_device(device)) return s;
+    if (B == 0 || N == 0 || M == 0) return TTAMD_OK;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    bool rhs_sums_done = false;
+    g.rhs_colsum_done = &rhs_sums_done;
+    if (ttamd_status s = run_product(dtype, g, device, st, fixed_scratch)) return s;
+    // The right operand's sums over k, unless the product's kernel has written them: its rows added in order.
+    if (g.rhs_colsum && !rhs_sums_done) return launch_colsum_reduce(dtype, g.B, g.K, g.N, g.batch, g.rhs_colsum, st);
+    return TTAMD_OK;
 }
 
 }  // namespace

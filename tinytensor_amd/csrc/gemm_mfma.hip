@@ -139,13 +139,20 @@ gemm_mfma_kernel(GemmArgs g, int tiles_m, int tiles_n, int ksplit, int k_chunk, 
 // run the same number of k tiles (the host only launches this when ceil(k_half / BK) == ceil((K - k_half) / BK)), so
 // they pass the engine's barriers in step; a half whose length is not a whole number of tiles takes the masked loop,
 // which has the same barriers.  The sum is (first half) + (second half), each accumulated in k order: deterministic.
-template <typename T, int BM, int BN, int BK, int WGM, int WGN, bool A_KC, int A_VEC, bool B_KC, int B_VEC, int PF>
+// BSUM (B with its columns contiguous, 16-byte vectors): the workgroups of the first row of tiles also add up the
+// vectors of B that they stage -- every element of B's column panel passes through their registers once -- and write
+// g.rhs_colsum[batch][n] = sum over k of B[k][n]: the bias gradient of a Linear layer when this product is its weight
+// gradient x^T . dy (nn/linear.cpp:45-48: the bias is an expanded view, its gradient sums the batch dimension).  Order:
+// a lane adds its k rows in k order, the 16 lanes of a column are added in lane order, lower half + upper half.
+template <typename T, int BM, int BN, int BK, int WGM, int WGN, bool A_KC, int A_VEC, bool B_KC, int B_VEC, int PF, bool BSUM = false>
 __global__ void __launch_bounds__(2 * kThreads, 1)
 gemm_mfma_dual_kernel(GemmArgs g, int tiles_m, int tiles_n, int k_half) {
     using StA = Stager<T, BM, BK, A_KC, A_VEC, PF>;
-    using StB = Stager<T, BN, BK, B_KC, B_VEC, PF>;
+    using StB = Stager<T, BN, BK, B_KC, B_VEC, PF, BSUM>;
     using Engine = TileEngine<T, BM, BN, BK, WGM, WGN, StA, StB>;
-    static_assert(Engine::kAccPerLane * kThreads * sizeof(T) <= 2 * Engine::kLdsBytes, "the parked accumulators fit the two halves' buffers");
+    constexpr size_t kExchangeBytes = Engine::kAccPerLane * kThreads * sizeof(T);
+    constexpr size_t kSumBytes = BSUM ? 2 * StB::kSumParts * BN * sizeof(T) : 0;
+    static_assert(kExchangeBytes + kSumBytes <= 2 * Engine::kLdsBytes, "the parked accumulators (and operand sums) fit the two halves' buffers");
     extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
     // The half is the same for every lane of a wave.  Said through readfirstlane so that the compiler keeps it, and the
     // half's length, k tile count and every loop condition and mask decision derived from it, in scalar registers
@@ -166,15 +173,32 @@ gemm_mfma_dual_kernel(GemmArgs g, int tiles_m, int tiles_n, int k_half) {
     StB sb;
     sa.init(a_base, tid, g.M - m0, g.a_sm, g.a_sk, Kc);
     sb.init(b_base, tid, g.N - n0, g.b_sn, g.b_sk, Kc);
+    if constexpr (BSUM) sb.start_sums(tm == 0);
     Engine eng;
     eng.init(tid);
     eng.run(sa, sb, smem, Kc, !sa.row_mask && !sb.row_mask);
     __syncthreads();  // every wave is done with its tiles: the lower half's buffers become the exchange area
     T *const exchange = reinterpret_cast<T *>(smem_raw);
+    T *const sums = reinterpret_cast<T *>(smem_raw + kExchangeBytes);  // [half][part][BN]
     if (half == 1) eng.park_acc(exchange, tid);
+    if constexpr (BSUM) {
+        if (tm == 0)
+            *reinterpret_cast<typename StB::V *>(&sums[(half * StB::kSumParts + sb.sum_part()) * BN + sb.sum_row0()]) = sb.sum;
+    }
     __syncthreads();
     if (half == 1) return;
     eng.add_parked_acc(exchange, tid);
+    if constexpr (BSUM) {
+        if (tm == 0 && tid < BN && n0 + tid < g.N) {
+            T lower = T(0), upper = T(0);
+#pragma unroll
+            for (int r = 0; r < StB::kSumParts; ++r) {
+                lower += sums[r * BN + tid];
+                upper += sums[(StB::kSumParts + r) * BN + tid];
+            }
+            static_cast<T *>(g.rhs_colsum)[static_cast<int64_t>(batch) * g.N + n0 + tid] = lower + upper;
+        }
+    }
     T *C = static_cast<T *>(g.C) + static_cast<int64_t>(batch) * g.M * g.N;
     if (plain_store(g))
         store_tile_dense<T, true>(eng, C, g.M, g.N, m0, n0, static_cast<const T *>(nullptr), 0, 0, 0);
@@ -395,12 +419,12 @@ int dual_k_half(int K) {
     return ((K + 1) / 2 + VK - 1) / VK * VK;
 }
 
-template <typename T, int BM, int BN, int BK, int WGM, int WGN, bool A_KC, int A_VEC, bool B_KC, int B_VEC, int PF>
+template <typename T, int BM, int BN, int BK, int WGM, int WGN, bool A_KC, int A_VEC, bool B_KC, int B_VEC, int PF, bool BSUM = false>
 ttamd_status launch_dual_variant(const GemmArgs &g, int device, hipStream_t stream, bool fixed_scratch) {
     using StA = Stager<T, BM, BK, A_KC, A_VEC, PF>;
-    using StB = Stager<T, BN, BK, B_KC, B_VEC, PF>;
+    using StB = Stager<T, BN, BK, B_KC, B_VEC, PF, BSUM>;
     constexpr size_t lds_bytes = 2 * TileEngine<T, BM, BN, BK, WGM, WGN, StA, StB>::kLdsBytes;
-    auto kernel = gemm_mfma_dual_kernel<T, BM, BN, BK, WGM, WGN, A_KC, A_VEC, B_KC, B_VEC, PF>;
+    auto kernel = gemm_mfma_dual_kernel<T, BM, BN, BK, WGM, WGN, A_KC, A_VEC, B_KC, B_VEC, PF, BSUM>;
     static bool configured[kMaxDevices] = {};  // once per kernel and device
     const int slot = device >= 0 && device < kMaxDevices ? device : 0;
     if (!configured[slot] || slot != device) {
@@ -422,8 +446,14 @@ ttamd_status launch_dual_variant(const GemmArgs &g, int device, hipStream_t stre
     return finish_colsum<T>(ga, stream);
 }
 
-template <typename T, int BM, int BN, int BK, int WGM, int WGN, int VEC, int PF>
+template <typename T, int BM, int BN, int BK, int WGM, int WGN, int VEC, int PF, bool BSUM_OK = false>
 ttamd_status launch_dual_layouts(const GemmArgs &g, bool a_kc, bool b_kc, int device, hipStream_t stream, bool fixed_scratch) {
+    if constexpr (BSUM_OK) {  // the sums of B in the same launch (the caller has checked that b_kc is false)
+        if (g.rhs_colsum && !b_kc) {
+            if (a_kc) return launch_dual_variant<T, BM, BN, BK, WGM, WGN, true, VEC, false, VEC, PF, true>(g, device, stream, fixed_scratch);
+            return launch_dual_variant<T, BM, BN, BK, WGM, WGN, false, VEC, false, VEC, PF, true>(g, device, stream, fixed_scratch);
+        }
+    }
     if (a_kc && b_kc) return launch_dual_variant<T, BM, BN, BK, WGM, WGN, true, VEC, true, VEC, PF>(g, device, stream, fixed_scratch);
     if (a_kc && !b_kc) return launch_dual_variant<T, BM, BN, BK, WGM, WGN, true, VEC, false, VEC, PF>(g, device, stream, fixed_scratch);
     if (!a_kc && b_kc) return launch_dual_variant<T, BM, BN, BK, WGM, WGN, false, VEC, true, VEC, PF>(g, device, stream, fixed_scratch);
@@ -554,7 +584,10 @@ ttamd_status launch_mfma_typed(const GemmArgs &g, int device, hipStream_t stream
     if constexpr (sizeof(T) == 4)
         if (dual_large) return launch_dual_layouts<T, TS::LBM, TS::LBN, TS::LBK, 2, 2, VK, 1>(g, ca.kc, cb.kc, device, stream, fixed_scratch);
     if (large) return launch_layouts<T, TS::LBM, TS::LBN, TS::LBK, 2, 2, VK, VK>(g, ca.kc, cb.kc, sp, device, stream);
-    if (dual) return launch_dual_layouts<T, TS::SBM, TS::SBN, TS::SBK, 2, 2, VK, TS::SPF_DEEP>(g, ca.kc, cb.kc, device, stream, fixed_scratch);
+    if (dual) {
+        if (g.rhs_colsum && !cb.kc && g.rhs_colsum_done) *g.rhs_colsum_done = true;  // (the kernel's first row of tiles adds B up)
+        return launch_dual_layouts<T, TS::SBM, TS::SBN, TS::SBK, 2, 2, VK, TS::SPF_DEEP, true>(g, ca.kc, cb.kc, device, stream, fixed_scratch);
+    }
     if (ca.vec > 1 && cb.vec > 1) {
         // Register prefetch depth of the small tile: 4 k tiles in flight when a CU holds at most two workgroups and the
         // reduction is long (a lone workgroup otherwise waits for memory in every step), else 2, whose smaller register

@@ -178,7 +178,10 @@ struct TileLayout {
 // Stager for a strided matrix view (ROWS along m or n, BK along k).  Vectors of VEC elements run along k
 // for KC (operand's k stride is 1 when VEC > 1) and along the row index for MC (row stride 1 when VEC > 1).
 // PF register slots hold PF tiles in flight (prefetch distance PF).
-template <typename T, int ROWS, int BK, bool KC, int VEC, int PF = 1>
+// SUM (MC with whole vectors only): every vector that is parked in LDS is also added to `sum` when `sum_on` is set -- a
+// lane's vectors all hold the same VEC rows of the operand (columns of B), so after the reduction `sum` is this
+// lane's share of the operand's sums over k, masked elements counting as zero.
+template <typename T, int ROWS, int BK, bool KC, int VEC, int PF = 1, bool SUM = false>
 struct Stager : TileLayout<T, ROWS, BK, KC> {
     using L = TileLayout<T, ROWS, BK, KC>;
     using V = typename Vec<T, VEC>::type;
@@ -188,7 +191,10 @@ struct Stager : TileLayout<T, ROWS, BK, KC> {
     static constexpr int P = NV / kThreads;
     static_assert(NV % kThreads == 0, "tile must split evenly over the workgroup");
 
+    static_assert(!SUM || (!KC && VEC > 1 && kThreads % VPL == 0), "sums: vectors along the rows, the same rows in every pass of a lane");
     V reg[PF][P];
+    mutable V sum;        // SUM only
+    bool sum_on = false;  // SUM only, workgroup-uniform
     uint32_t voff[P];
     int nval[P];  // MC only: valid components of the vector along the row dimension
     __amdgpu_buffer_rsrc_t rsrc;
@@ -289,7 +295,24 @@ struct Stager : TileLayout<T, ROWS, BK, KC> {
             const int line = line_of(p, tid), col = col_of(p, tid);
             *reinterpret_cast<V *>(&lds[line * L::LD + col]) = reg[SLOT][p];
         }
+        if constexpr (SUM) {
+            if (sum_on) {  // (every tile is parked exactly once: tile 0 by the prologue, tile kt + 1 by step kt)
+#pragma unroll
+                for (int p = 0; p < P; ++p) sum += reg[SLOT][p];
+            }
+        }
     }
+    // SUM: start the sums (before the first tile is parked).
+    __device__ __forceinline__ void start_sums(bool on) {
+        sum_on = on;
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) sum[j] = T(0);
+    }
+    // SUM: the rows this lane's sums belong to (tile-local, VEC consecutive ones) and which of the kThreads / VPL
+    // lanes with the same rows this one is.
+    __device__ __forceinline__ int sum_row0() const { return col_of(0, tid); }
+    __device__ __forceinline__ int sum_part() const { return tid / VPL; }
+    static constexpr int kSumParts = SUM ? kThreads / VPL : 1;
 };
 
 // ---------------------------------------------------------------------------------------------

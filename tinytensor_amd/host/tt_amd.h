@@ -799,29 +799,37 @@ public:
 // Backward of y = x . W (+ b) for 2-D operands, as autograd emits it (TensorBatchedMatmul::backward on permute views,
 // autograd/binary_ops.cpp:173-179) with the element-wise steps that follow dx fused into its GEMM's store:
 //   dx = dy . W^T;  when x = relu(*relu_input): dx *= where(relu_input < 0, 0, 1) (autograd/unary_ops.cpp:568-573);
-//   when bias_grad: db_prev = dx.sum(0), the bias gradient of the Linear layer that produced relu_input;
-//   dW = x^T . dy.
+//   BiasGrad::kPrev: db = dx.sum(0), the bias gradient of the Linear layer that produced relu_input, from the store of
+//   dx's GEMM;
+//   dW = x^T . dy;
+//   BiasGrad::kOwn: db = dy.sum(0), this layer's own bias gradient (nn/linear.cpp:45-48), from the vectors of dy that dW's
+//   GEMM stages.
+enum class BiasGrad { kNone, kPrev, kOwn };
 struct LinearGrads {
     Tensor dx, dW;
-    std::optional<Tensor> db_prev;
+    std::optional<Tensor> db;
 };
 inline auto linear_backward(const Tensor &grad_output, const Tensor &input, const Tensor &weight, const Tensor *relu_input = nullptr,
-                            bool bias_grad = false) -> LinearGrads {
+                            BiasGrad bias_grad = BiasGrad::kNone) -> LinearGrads {
     const auto *be = get_backend(grad_output.device());
     LinearGrads g;
-    ttamd_epilogue ep{};
+    ttamd_epilogue ep{}, ep_w{};
     std::optional<Tensor> z;
     if (relu_input) {
         if (!(relu_input->shape() == input.shape()) || relu_input->dtype() != input.dtype()) throw TTException("linear_backward: relu_input must match input");
         z = relu_input->contiguous();
         ep.relu_grad_input = z->data_ptr();
     }
-    if (bias_grad) {
-        g.db_prev = Tensor::empty(Shape({input.size(1)}), input.dtype(), input.device());
-        ep.colsum_out = g.db_prev->data_ptr();
+    const Tensor dy = bias_grad == BiasGrad::kOwn ? grad_output.contiguous() : grad_output;  // (its sums need a dense operand)
+    if (bias_grad == BiasGrad::kPrev) {
+        g.db = Tensor::empty(Shape({input.size(1)}), input.dtype(), input.device());
+        ep.colsum_out = g.db->data_ptr();
+    } else if (bias_grad == BiasGrad::kOwn) {
+        g.db = Tensor::empty(Shape({dy.size(1)}), dy.dtype(), dy.device());
+        ep_w.rhs_colsum_out = g.db->data_ptr();
     }
-    g.dx = be->batched_matmul(grad_output.unsqueeze(0), weight.unsqueeze(0).permute({0, 2, 1}), &ep).squeeze(0);
-    g.dW = be->batched_matmul(input.unsqueeze(0).permute({0, 2, 1}), grad_output.unsqueeze(0)).squeeze(0);
+    g.dx = be->batched_matmul(dy.unsqueeze(0), weight.unsqueeze(0).permute({0, 2, 1}), &ep).squeeze(0);
+    g.dW = be->batched_matmul(input.unsqueeze(0).permute({0, 2, 1}), dy.unsqueeze(0), bias_grad == BiasGrad::kOwn ? &ep_w : nullptr).squeeze(0);
     return g;
 }
 

@@ -452,28 +452,31 @@ class BackendAMD:
     def batched_matmul(self, lhs: Tensor, rhs: Tensor, bias: Tensor | None = None, bias_mode: int = 0,
                        relu: bool = False, out: Tensor | None = None, accumulate: bool = False,
                        relu_out: Tensor | None = None, relu_grad_input: Tensor | None = None,
-                       colsum_out: Tensor | None = None) -> Tensor:
+                       colsum_out: Tensor | None = None, rhs_colsum_out: Tensor | None = None) -> Tensor:
         """BackendBase::batched_matmul (backend_base.h:130).  The keyword arguments select the fused
         epilogue of ttamd_batched_matmul; with the defaults this is the reference call exactly.
         relu_out: dense [B,N,M] tensor that receives max(out, 0) while `out` keeps the value before the ReLU;
         relu_grad_input: dense [B,N,M] saved input z of a ReLU, out = result * (z < 0 ? 0 : 1);
-        colsum_out: dense [B,M] tensor that receives out summed over its rows."""
+        colsum_out: dense [B,M] tensor that receives out summed over its rows;
+        rhs_colsum_out: dense [B,M] tensor that receives rhs (dense row-major) summed over its rows."""
         assert lhs.dim() == 3 and rhs.dim() == 3 and lhs.size(2) == rhs.size(1)
         B, N, K = lhs.shape
         M = rhs.size(2)
         if out is None:
             out = Tensor.empty((B, N, M), lhs.dtype, lhs.device)
         ep = None
-        if bias is not None or relu or accumulate or relu_out is not None or relu_grad_input is not None or colsum_out is not None:
+        if (bias is not None or relu or accumulate or relu_out is not None or relu_grad_input is not None or colsum_out is not None
+                or rhs_colsum_out is not None):
             ep = _capi.Epilogue()
             ep.bias = (bias.storage.ptr + bias.offset * bias.itemsize) if bias is not None else None
             ep.bias_mode = bias_mode if bias is not None else 0
             ep.relu = int(relu)
             ep.accumulate = int(accumulate)
-            for name, t in (("relu_out", relu_out), ("relu_grad_input", relu_grad_input), ("colsum_out", colsum_out)):
+            for name, t in (("relu_out", relu_out), ("relu_grad_input", relu_grad_input), ("colsum_out", colsum_out),
+                            ("rhs_colsum_out", rhs_colsum_out)):
                 if t is None:
                     continue
-                want = (B, M) if name == "colsum_out" else (B, N, M)
+                want = (B, M) if name in ("colsum_out", "rhs_colsum_out") else (B, N, M)
                 dense = all(n == 1 or st == d for n, st, d in zip(t.shape, t.stride, _dense_strides(t.shape)))
                 if not dense or t.numel() != int(np.prod(want)) or t.dtype != lhs.dtype:
                     raise TTException(f"batched_matmul: {name} must be a dense tensor of {want} elements of the operands' dtype")
@@ -813,22 +816,28 @@ def linear_relu(input: Tensor, weight: Tensor, bias: Tensor | None = None):
 
 
 def linear_backward(grad_output: Tensor, input: Tensor, weight: Tensor, relu_input: Tensor | None = None,
-                    bias_grad: bool = True):
+                    bias_grad: bool | str = True):
     """Backward of y = x . W (+ b) for 2-D operands dy = grad_output [n, out], x = input [n, in], W = weight [in, out],
     as autograd emits it (TensorBatchedMatmul::backward on permute views, autograd/binary_ops.cpp:173-179) with the
     element-wise steps that follow dx fused into its GEMM:
         dx = dy . W^T;
         when x = relu(relu_input): dx *= where(relu_input < 0, 0, 1)   (TensorRelu::backward, unary_ops.cpp:568-573);
-        when bias_grad: db_prev = dx.sum(0), the bias gradient of the Linear layer that produced relu_input;
-        dW = x^T . dy.
-    Returns (dx, dW, db_prev | None)."""
+        when bias_grad is True: db_prev = dx.sum(0), the bias gradient of the Linear layer that produced relu_input,
+            from the store of dx's GEMM;
+        dW = x^T . dy;
+        when bias_grad == "own": db = dy.sum(0), this layer's own bias gradient, from the vectors of dy that dW's GEMM
+            stages (dy must be dense).
+    Returns (dx, dW, db_prev | db | None)."""
     be = get_backend(grad_output.device)
     n, fin = input.shape
-    db = Tensor.empty((1, fin), grad_output.dtype, grad_output.device) if bias_grad else None
+    own = bias_grad == "own"
+    fout = grad_output.size(1)
+    db = Tensor.empty((1, fout if own else fin), grad_output.dtype, grad_output.device) if bias_grad else None
     dx = be.batched_matmul(grad_output.unsqueeze(0), weight.unsqueeze(0).permute(0, 2, 1),
-                           relu_grad_input=relu_input.unsqueeze(0) if relu_input is not None else None, colsum_out=db)
-    dW = be.batched_matmul(input.unsqueeze(0).permute(0, 2, 1), grad_output.unsqueeze(0))
-    return dx.squeeze(0), dW.squeeze(0), (db.reshape([fin]) if db is not None else None)
+                           relu_grad_input=relu_input.unsqueeze(0) if relu_input is not None else None,
+                           colsum_out=None if own else db)
+    dW = be.batched_matmul(input.unsqueeze(0).permute(0, 2, 1), grad_output.unsqueeze(0), rhs_colsum_out=db if own else None)
+    return dx.squeeze(0), dW.squeeze(0), (db.reshape([fout if own else fin]) if db is not None else None)
 
 
 def mse_loss(input: Tensor, target: Tensor, grad: bool = True, bias_grad: bool = False):
