@@ -99,7 +99,8 @@ typedef struct ttamd_epilogue {
      * gradient x^T . dy (TensorBatchedMatmul::backward, autograd/binary_ops.cpp:173-179), the right operand is dy and
      * its column sums are the bias gradient (nn/linear.cpp:45-48), taken from the vectors the product stages anyway
      * where its kernel can, else by a launch of its own.  The right operand must be dense row-major; f32/f64.  Added
-     * in a fixed order (deterministic; not the reference's row-by-row order). */
+     * in a fixed order (deterministic; not the reference's row-by-row order).  Written whenever the right operand has
+     * columns (K = 0: zeros; a left operand without rows: no product, the sums all the same). */
     void *rhs_colsum_out;
 } ttamd_epilogue;
 

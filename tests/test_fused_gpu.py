@@ -153,6 +153,20 @@ def test_right_operand_column_sums(tt, dtype, a_transposed, shape):
     assert np.array_equal(sums2.to_numpy(), b.sum(axis=1))
 
 
+def test_right_operand_column_sums_of_degenerate_products(tt):
+    be = tt.get_backend(tt.kAMD)
+    f32 = tt._capi.F32
+    # K = 0: the empty sum
+    sums = tt.Tensor.from_numpy(np.full((2, 7), 5, np.float32))
+    out = be.batched_matmul(tt.Tensor.empty((2, 5, 0), f32), tt.Tensor.empty((2, 0, 7), f32), rhs_colsum_out=sums).to_numpy()
+    assert np.all(out == 0) and np.all(sums.to_numpy() == 0)
+    # no rows on the left: no product, but the right operand still has its sums
+    b = np.arange(2 * 3 * 7, dtype=np.float32).reshape(2, 3, 7)
+    sums = tt.Tensor.from_numpy(np.zeros((2, 7), np.float32))
+    assert be.batched_matmul(tt.Tensor.empty((2, 0, 3), f32), tt.Tensor.from_numpy(b), rhs_colsum_out=sums).shape == (2, 0, 7)
+    assert np.array_equal(sums.to_numpy(), b.sum(axis=1))
+
+
 def test_right_operand_column_sums_need_a_dense_operand(tt):
     be = tt.get_backend(tt.kAMD)
     a = tt.Tensor.from_numpy(np.ones((1, 64, 64), np.float32))

@@ -132,8 +132,11 @@ ttamd_status batched_matmul(int device, ttamd_dtype dtype, int B, int N, int K, 
     GemmArgs g;
     if (ttamd_status s = build_args(dtype, B, N, K, M, lhs, rhs, out, epilogue, &g, true)) return s;
     if (ttamd_status s = use_device(device)) return s;
-    if (B == 0 || N == 0 || M == 0) return TTAMD_OK;
     hipStream_t st = static_cast<hipStream_t>(stream);
+    if (B == 0 || N == 0 || M == 0) {  // no product; the right operand's sums exist all the same when it has columns
+        if (g.rhs_colsum && B > 0 && M > 0) return launch_colsum_reduce(dtype, g.B, g.K, g.N, g.batch, g.rhs_colsum, st);
+        return TTAMD_OK;
+    }
     bool rhs_sums_done = false;
     g.rhs_colsum_done = &rhs_sums_done;
     if (ttamd_status s = run_product(dtype, g, device, st, fixed_scratch)) return s;
