@@ -92,8 +92,8 @@ typedef struct ttamd_epilogue {
     const void *relu_grad_input;
     /* Sum of `out` over its rows, [B,M] (or NULL): the gradient of a Linear layer's bias, which nn/linear.cpp:45-48
      * adds as an expanded view, so its gradient sums the batch dimension.  Per-tile partial sums are added in a fixed
-     * order by a second small kernel (deterministic; not the reference's row-by-row order).  f32/f64 on the
-     * matrix-core kernels only; not together with `accumulate`. */
+     * order by a second small kernel (deterministic; not the reference's row-by-row order).  f32/f64; not together
+     * with `accumulate`.  Written whenever the result has columns (no rows: zeros; K = 0: rows x bias). */
     void *colsum_out;
     /* Sum of the right operand over its rows (k), [B,M] (or NULL): when the product is a Linear layer's weight
      * gradient x^T . dy (TensorBatchedMatmul::backward, autograd/binary_ops.cpp:173-179), the right operand is dy and
@@ -177,8 +177,10 @@ ttamd_status ttamd_batched_matmul(int device, ttamd_dtype dtype, int B, int N, i
  * buffer that ttamd_batched_matmul grows with hipMalloc.  The call makes no hipMalloc / hipFree.  A product whose
  * partial tiles exceed the array (possible for some f64 shapes with fewer than 128 output tiles of 64 x 64) is refused
  * with TTAMD_ERR_INVALID_ARGUMENT and a message naming the sizes.  All calls on one GPU share that GPU's array:
- * calls that may overlap in time on one GPU (different streams, several threads) race and must be serialised by the
- * caller.  The first call on a device looks up the array's device address; make that call outside a capture. */
+ * calls that may overlap in time on one GPU race.  Calls on one stream are ordered by the stream.  A call that needs
+ * the array on a different stream than the last call that used it is refused (TTAMD_ERR_INVALID_ARGUMENT) unless
+ * ttamd_device_synchronize has run in between; several host threads launching on one stream are the caller's to
+ * serialise.  The first call on a device looks up the array's device address; make that call outside a capture. */
 ttamd_status ttamd_batched_matmul_noalloc(int device, ttamd_dtype dtype, int B, int N, int K, int M,
                                           const ttamd_view3 *lhs, const ttamd_view3 *rhs, void *out,
                                           const ttamd_epilogue *epilogue, void *stream);
@@ -303,6 +305,17 @@ ttamd_status ttamd_random_fill_view(int device, ttamd_dtype dtype, int dist, dou
 ttamd_status ttamd_random_fill_states(int device, ttamd_dtype dtype, int dist, double p0, double p1, const uint64_t *states,
                                       int ndim, const int64_t *shape, const int64_t *stride, void *data, int64_t offset,
                                       void *stream);
+
+/* The tensor forms of BackendBase::uniform_real / normal (backend_base.h:83-103; GPU peer cuda/distribution.cu:32-99):
+ * a parameter pair per element.  p0 / p1 (low / high, or mu / std) are device views over the same `shape` as the result
+ * -- storage pointer, element offset, element strides (0 for an expanded value) -- and element i of the result, i its
+ * row-major rank, reads them at rank i, as the CPU backend reads params[i] of the parameters made contiguous
+ * (cpu/distribution.cpp:42-47, cpu/kernel/distribution.hpp:28-32).  low < high per element is the caller's to keep
+ * (the reference asserts it, common/kernel/distribution.hpp:95). */
+ttamd_status ttamd_random_fill_states_params(int device, ttamd_dtype dtype, int dist, const void *p0, int64_t p0_offset,
+                                             const int64_t *p0_stride, const void *p1, int64_t p1_offset,
+                                             const int64_t *p1_stride, const uint64_t *states, int ndim, const int64_t *shape,
+                                             const int64_t *stride, void *data, int64_t offset, void *stream);
 
 /* ---- timing (no reference counterpart: the reference has no timers; used by the benchmark
  * to bracket kernels with HIP events on the stream they run on) ------------------------ */

@@ -141,6 +141,33 @@ void tto_uniform_real_view_f64(uint64_t *state, double low, double high, double 
         data[to_flat_index(i, ndim, shape, stride, offset)] = uniform_sample_f64(low, high, &st);
     }
 }
+/* Draws with a parameter pair per element (the tensor forms, backend_base.h:83-103; cpu/distribution.cpp:42-139):
+ * the parameters are made contiguous first, so element i reads p0[i], p1[i]; the result is written through the view
+ * (dense: stride of a row-major tensor, offset 0).  dist 0 = uniform_real(low, high), 1 = normal(mu, std). */
+#define TTO_DRAW_PARAMS(NAME, T, SAMPLE, SQRT, LOG1P, SIN, PI)                                                                \
+    void NAME(uint64_t *state, int dist, const T *p0, const T *p1, T *data, int ndim, const int *shape, const int *stride, \
+              int offset) {                                                                                                 \
+        int n = 1;                                                                                                          \
+        for (int d = 0; d < ndim; ++d) n *= shape[d];                                                                       \
+        for (int i = 0; i < n; ++i) {                                                                                       \
+            uint64_t st = tto_xorshift64(state);                                                                            \
+            T value;                                                                                                        \
+            if (dist == 0) {                                                                                                \
+                value = SAMPLE(p0[i], p1[i], &st);                                                                          \
+            } else {                                                                                                        \
+                const T u1 = SAMPLE((T)0, (T)1, &st);                                                                       \
+                const T u2 = SAMPLE((T)0, (T)1, &st);                                                                       \
+                const T r = SQRT((T)-2 * LOG1P(-u1));                                                                       \
+                const T theta = (T)2 * PI * u2;                                                                             \
+                value = p1[i] * (r * SIN(theta)) + p0[i];                                                                   \
+            }                                                                                                               \
+            data[to_flat_index(i, ndim, shape, stride, offset)] = value;                                                    \
+        }                                                                                                                   \
+    }
+TTO_DRAW_PARAMS(tto_draw_params_f32, float, uniform_sample_f32, sqrtf, log1pf, sinf, 3.14159265358979323846f)
+TTO_DRAW_PARAMS(tto_draw_params_f64, double, uniform_sample_f64, sqrt, log1p, sin, 3.14159265358979323846)
+#undef TTO_DRAW_PARAMS
+
 /* identity op into a dense result (cpu/unary.cpp:26-58) */
 void tto_contiguous(const void *src, void *dst, int elem_size, int ndim, const int *shape, const int *stride,
                     int offset) {

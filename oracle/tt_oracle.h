@@ -37,6 +37,9 @@
  *   tto_uniform_real_view_*  the dense draw in the view's order scattered by explicit index loops
  *                         (brute force), and numpy's transposition of the dense draw for the
  *                         permuted view that nn::Conv2d's initialisation uses.
+ *   tto_draw_params_*     element by element against the scalar-parameter draws above: element i equals
+ *                         element i of a dense draw from the same seed with (p0[i], p1[i]) as the scalars
+ *                         (brute force over every element), through dense and permuted views.
  *   tto_normal_*          closed form: every element's (u1, u2) rebuilt from the integer
  *                         generator and mu + std*sqrt(-2*log1p(-u1))*sin(2*pi*u2) evaluated
  *                         with 200-bit transcendentals, each step rounded to the type; f32
@@ -86,6 +89,13 @@ void tto_uniform_real_view_f32(uint64_t *state, float low, float high, float *da
                                const int *stride, int offset);
 void tto_uniform_real_view_f64(uint64_t *state, double low, double high, double *data, int ndim, const int *shape,
                                const int *stride, int offset);
+
+/* Draws with a parameter pair per element (backend_base.h:83-103; cpu/distribution.cpp:42-139): dense parameter arrays
+ * p0 / p1 (low / high for dist 0, mu / std for dist 1), element i of the view reads p0[i], p1[i]. */
+void tto_draw_params_f32(uint64_t *state, int dist, const float *p0, const float *p1, float *data, int ndim, const int *shape,
+                         const int *stride, int offset);
+void tto_draw_params_f64(uint64_t *state, int dist, const double *p0, const double *p1, double *data, int ndim, const int *shape,
+                         const int *stride, int offset);
 
 /* ---- strided view -> dense copy (Tensor::contiguous via the identity op:
  * cpu/unary.cpp:26-58 with common/util.h:18-34) ---- */

@@ -55,6 +55,10 @@ def _load(flavour: str) -> C.CDLL:
     lib.tto_normal_f64.argtypes = [u64p, C.c_double, C.c_double, vp, i64]
     lib.tto_uniform_real_view_f32.argtypes = [u64p, C.c_float, C.c_float, vp, i32, ip, ip, i32]
     lib.tto_uniform_real_view_f64.argtypes = [u64p, C.c_double, C.c_double, vp, i32, ip, ip, i32]
+    lib.tto_draw_params_f32.argtypes = [u64p, i32, vp, vp, vp, i32, ip, ip, i32]
+    lib.tto_draw_params_f64.argtypes = [u64p, i32, vp, vp, vp, i32, ip, ip, i32]
+    lib.tto_draw_params_f32.restype = None
+    lib.tto_draw_params_f64.restype = None
     for f in ("tto_uniform_real_f32", "tto_uniform_real_f64", "tto_normal_f32", "tto_normal_f64", "tto_uniform_real_view_f32",
               "tto_uniform_real_view_f64"):
         getattr(lib, f).restype = None
@@ -131,6 +135,16 @@ class Generator:
         base, offset = view_base(view)
         fn = lib().tto_uniform_real_view_f32 if view.dtype == np.float32 else lib().tto_uniform_real_view_f64
         fn(C.byref(self._state), low, high, _ptr(base), view.ndim, _ints(view.shape), _ints(elem_strides(view)), offset)
+
+    def draw_params_(self, view: np.ndarray, dist: int, p0: np.ndarray, p1: np.ndarray) -> None:
+        """uniform_real_ (dist 0) / normal_ (dist 1) with parameter tensors, in place through `view`
+        (cpu/distribution.cpp:96-139): p0 / p1 are broadcast to the view's shape and made contiguous, element i of
+        the view (row-major rank) reads p0[i], p1[i]."""
+        base, offset = view_base(view)
+        a = np.ascontiguousarray(np.broadcast_to(p0, view.shape), dtype=view.dtype)
+        b = np.ascontiguousarray(np.broadcast_to(p1, view.shape), dtype=view.dtype)
+        fn = lib().tto_draw_params_f32 if view.dtype == np.float32 else lib().tto_draw_params_f64
+        fn(C.byref(self._state), dist, _ptr(a), _ptr(b), _ptr(base), view.ndim, _ints(view.shape), _ints(elem_strides(view)), offset)
 
     def normal(self, mu: float, std: float, shape, dtype=np.float32) -> np.ndarray:
         out = np.empty(int(np.prod(shape)), dtype=dtype)

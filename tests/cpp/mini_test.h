@@ -78,6 +78,19 @@ inline int run_all(int argc, char **argv) {
         }                                                                       \
     } while (0)
 
+// allclose with the reference's defaults rtol 1e-5 / atol 1e-8 (include/tt/tensor.h:3396-3398), on host vectors.
+template <typename T>
+bool allclose(const std::vector<T> &a, const std::vector<T> &b, double rtol = 1e-5, double atol = 1e-8) {
+    if (a.size() != b.size()) return false;
+    for (std::size_t i = 0; i < a.size(); ++i) {
+        const double x = static_cast<double>(a[i]), y = static_cast<double>(b[i]);
+        if (!(std::fabs(x - y) <= atol + rtol * std::fabs(y))) return false;
+    }
+    return true;
+}
+
+// (a test that brings its own Tensor defines MINI_TEST_NO_HOST_LAYER and its own fan-out)
+#ifndef MINI_TEST_NO_HOST_LAYER
 // Device / dtype fan-out in the style of the reference's tests/test_util.h:5-45.
 #include "tt_amd.h"
 template <typename T, typename F>
@@ -102,16 +115,6 @@ template <typename F>
 void runner_boolean(F &&f) {
     runner_single_type<bool>(f);
 }
-
-// allclose with the reference's defaults rtol 1e-5 / atol 1e-8 (include/tt/tensor.h:3396-3398), on host vectors.
-template <typename T>
-bool allclose(const std::vector<T> &a, const std::vector<T> &b, double rtol = 1e-5, double atol = 1e-8) {
-    if (a.size() != b.size()) return false;
-    for (std::size_t i = 0; i < a.size(); ++i) {
-        const double x = static_cast<double>(a[i]), y = static_cast<double>(b[i]);
-        if (!(std::fabs(x - y) <= atol + rtol * std::fabs(y))) return false;
-    }
-    return true;
-}
+#endif  // MINI_TEST_NO_HOST_LAYER
 
 #endif  // TT_AMD_MINI_TEST_H_

@@ -83,7 +83,7 @@ TEST_CASE("Batched Matrix Matrix product") {
     };
     runner_boolean(test_bool);
     auto test = []<typename T>(Device device) {
-        constexpr int B = 4, N = 256 + 123, M = 200, K = 512 + 123;
+        constexpr int B = 4, N = 256 + 123, M = 1024 + 123, K = 512 + 123;  // tests/test_matmul.cpp:200-236, at its own size
         std::vector<T> lhs, rhs;
         for (int b = 0; b < B; ++b) {
             for (int i = 0; i < N; ++i)

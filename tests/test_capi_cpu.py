@@ -63,6 +63,15 @@ def test_validation_without_gpu(tt):
     assert b"dense row-major" in lib.ttamd_last_error_string()
     b.stride[1], b.stride[2] = 2, 1
     assert lib.ttamd_batched_matmul(0, capi.I32, 1, 2, 2, 2, C.byref(a), C.byref(b), C.c_void_p(1024), C.byref(ep), None) == capi.ERR_UNSUPPORTED_DTYPE
+    # an empty product (no rows on the left) still reads the right operand for its sums: its pointer is checked on the host
+    a0, b0 = capi.View3(), capi.View3()
+    for i, st in enumerate((6, 2, 1)):
+        a0.stride[i] = b0.stride[i] = st
+    b0.stride[0], b0.stride[1] = 6, 2
+    assert lib.ttamd_batched_matmul(0, capi.F32, 1, 0, 3, 2, C.byref(a0), C.byref(b0), None, C.byref(ep), None) == capi.ERR_INVALID_ARGUMENT
+    assert b"right operand's data" in lib.ttamd_last_error_string()
+    b0.data = 258   # not a multiple of the element size
+    assert lib.ttamd_batched_matmul(0, capi.F32, 1, 0, 3, 2, C.byref(a0), C.byref(b0), None, C.byref(ep), None) == capi.ERR_INVALID_ARGUMENT
     # conv geometry errors
     v4 = capi.View4()
     assert lib.ttamd_conv2d_forward(0, capi.F32, C.byref(v4), C.byref(v4), None, None, 1, 3, 8, 8, 4, 3, 0, 0, None) == capi.ERR_INVALID_ARGUMENT

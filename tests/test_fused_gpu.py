@@ -60,6 +60,37 @@ def test_store_extensions_match_numpy(tt, dtype, shape):
     assert np.array_equal(be.batched_matmul(ta, tb).to_numpy(), prod.astype(dtype))
 
 
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+@pytest.mark.parametrize("shape", [(1, 200, 96, 136), (1, 1024, 1024, 1024), (1, 320, 512, 416), (1, 1024, 10, 1024), (1, 300, 64, 10),
+                                   (1, 4096, 32, 4096)])
+def test_relu_backward_mask_multiplies_like_the_reference(tt, dtype, shape):
+    """TensorRelu::backward is grad_output * where(input < 0, 0, 1) (autograd/unary_ops.cpp:568-573), a product: an
+    infinite or NaN gradient under the mask gives NaN, a negative one -0.  The fused store does the same (every kernel
+    family: tiles, two halves, split k, short reduction, thin output, 256 x 256)."""
+    B, N, K, M = shape
+    rng = np.random.default_rng(N * 3 + K + M)
+    a = rng.integers(-3, 4, (B, N, K)).astype(dtype)
+    b = rng.integers(-3, 4, (B, K, M)).astype(dtype)
+    z = rng.integers(-2, 3, (B, N, M)).astype(dtype)
+    a[0, 3, :] = 1
+    a[0, 3, 0] = np.inf                                    # row 3 of the product: +-inf, or NaN where b[0, 0, m] is 0
+    a[0, N - 1, K - 1] = np.nan                            # last row: NaN everywhere
+    z[0, 3, : M // 2] = -1
+    z[0, N - 1, ::2] = -1
+    be = tt.get_backend(tt.kAMD)
+    ta, tb, tz = (tt.Tensor.from_numpy(v) for v in (a, b, z))
+    with np.errstate(invalid="ignore"):
+        prod = np.matmul(a.astype(np.float64), b.astype(np.float64)) + 0.0   # (a sum of -0 terms: the kernels start from +0)
+        want = (prod * np.where(z < 0, 0.0, 1.0)).astype(dtype)
+    got = be.batched_matmul(ta, tb, relu_grad_input=tz).to_numpy()
+    variant = _variant(tt, ta, tb)
+    assert np.array_equal(np.isnan(got), np.isnan(want)), variant
+    assert np.isnan(want[0, 3, : M // 2]).all() and np.isnan(got[0, N - 1]).all()
+    finite = ~np.isnan(want)
+    assert np.array_equal(got[finite], want[finite]), variant
+    assert np.array_equal(np.signbit(got[finite]), np.signbit(want[finite])), variant    # -0 where a negative value is masked
+
+
 def test_store_extension_argument_checks(tt):
     be = tt.get_backend(tt.kAMD)
     a = tt.Tensor.from_numpy(np.ones((1, 8, 8), np.float32))
@@ -165,6 +196,24 @@ def test_right_operand_column_sums_of_degenerate_products(tt):
     sums = tt.Tensor.from_numpy(np.zeros((2, 7), np.float32))
     assert be.batched_matmul(tt.Tensor.empty((2, 0, 3), f32), tt.Tensor.from_numpy(b), rhs_colsum_out=sums).shape == (2, 0, 7)
     assert np.array_equal(sums.to_numpy(), b.sum(axis=1))
+
+
+def test_result_column_sums_of_degenerate_products(tt):
+    """colsum_out follows the same rule as rhs_colsum_out: it is written whenever the result has columns."""
+    be = tt.get_backend(tt.kAMD)
+    f32 = tt._capi.F32
+    # no rows: the sums over zero rows are zeros (the buffer held something else)
+    cs = tt.Tensor.from_numpy(np.full((2, 7), 5, np.float32))
+    b = np.arange(2 * 3 * 7, dtype=np.float32).reshape(2, 3, 7)
+    assert be.batched_matmul(tt.Tensor.empty((2, 0, 3), f32), tt.Tensor.from_numpy(b), colsum_out=cs).shape == (2, 0, 7)
+    assert np.all(cs.to_numpy() == 0)
+    # K = 0: every element is the empty sum plus the bias, so a column's sum is rows x bias
+    bias = np.arange(7, dtype=np.float32) - 3
+    cs = tt.Tensor.from_numpy(np.full((2, 7), 5, np.float32))
+    out = be.batched_matmul(tt.Tensor.empty((2, 5, 0), f32), tt.Tensor.empty((2, 0, 7), f32), bias=tt.Tensor.from_numpy(bias),
+                            bias_mode=1, colsum_out=cs).to_numpy()
+    assert np.array_equal(out, np.broadcast_to(bias, (2, 5, 7)))
+    assert np.array_equal(cs.to_numpy(), np.broadcast_to(5 * bias, (2, 7)))
 
 
 def test_right_operand_column_sums_need_a_dense_operand(tt):

@@ -92,7 +92,7 @@ def test_matrix_matrix_reference_size_exact(tt, oracle, dtype):
 
 @pytest.mark.parametrize("dtype", ALL_NON_BOOL)
 def test_batched_reference_pattern_exact(tt, dtype):
-    lhs, rhs = ref_batched(dtype, B=4, N=379, M=200, K=635)
+    lhs, rhs = ref_batched(dtype, B=4, N=379, M=1147, K=635)  # tests/test_matmul.cpp:200-236, at its own size
     got = tt.matmul(dev(tt, lhs), dev(tt, rhs)).to_numpy()
     want = np.stack([naive_exact(lhs[b], rhs[b]) for b in range(4)])
     assert np.array_equal(got, want)

@@ -36,6 +36,41 @@ def test_in_place_draws_through_views_match_the_cpu_generator(tt, oracle, dtype)
 
 
 @pytest.mark.parametrize("dtype", [np.float32, np.float64])
+def test_draws_with_parameter_tensors_match_the_cpu_generator(tt, oracle, dtype):
+    """uniform_real_ / normal_ with a parameter pair per element (backend_base.h:96-103, cuda/distribution.cu:32-99):
+    non-constant `high` / `std`, parameters given as a dense tensor, as a permuted view and as a value expanded with
+    stride 0, the result written through a permuted view with an offset."""
+    code = tt._capi.F32 if dtype == np.float32 else tt._capi.F64
+    rng = np.random.default_rng(8)
+    base_h = np.full((4, 6, 5), -7.0, dtype=dtype)
+    base_d = tt.Tensor.from_numpy(base_h)
+    view_h = base_h.transpose(1, 0, 2)[1:, :, 1:4]                               # [5,4,3]
+    view_d = tt.Tensor(base_d.storage, code, (5, 4, 3), (5, 30, 1), 6)
+    low = rng.uniform(-2.0, 1.0, (5, 4, 3)).astype(dtype)
+    high_src = (low.transpose(2, 0, 1) + rng.uniform(0.1, 3.0, (3, 5, 4))).astype(dtype)   # stored as [3,5,4]
+    high = high_src.transpose(1, 2, 0)                                             # the [5,4,3] view of it
+    t_low = tt.Tensor.from_numpy(low)
+    t_high = tt.Tensor.from_numpy(np.ascontiguousarray(high_src)).permute(1, 2, 0)
+    assert not t_high.is_contiguous()
+    g_dev, g_cpu = tt.Generator(13), oracle.Generator(13)
+    view_d.uniform_real_(t_low, t_high, g_dev)
+    g_cpu.draw_params_(view_h, 0, low, high)
+    assert np.array_equal(base_d.to_numpy(), base_h)                              # bit construction + one fma: exact
+    assert g_dev.state.value == g_cpu.state
+    # normal: mu one value expanded over the shape (stride 0), std per element
+    std = rng.uniform(0.05, 2.0, (5, 4, 3)).astype(dtype)
+    t_mu = tt.Tensor.from_numpy(np.array([[[0.25]]], dtype=dtype)).expand((5, 4, 3))
+    view_d.normal_(t_mu, tt.Tensor.from_numpy(std), g_dev)
+    g_cpu.draw_params_(view_h, 1, np.array(0.25, dtype=dtype), std)
+    got = base_d.to_numpy()
+    assert np.array_equal(got[:, 0], base_h[:, 0]) and np.array_equal(got[:, :, 0], base_h[:, :, 0])   # untouched elements
+    assert np.max(np.abs(got - base_h)) <= (2e-5 if dtype == np.float32 else 1e-12)  # |z| <= ~6, std <= 2: libm rounding
+    assert g_dev.state.value == g_cpu.state
+    with pytest.raises(tt.TTException):
+        view_d.uniform_real_(t_low, tt.Tensor.from_numpy(np.zeros((5, 4), dtype=dtype)), g_dev)   # shapes must agree
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
 def test_conv2d_default_init_equals_cpu_init(tt, oracle, dtype):
     code = tt._capi.F32 if dtype == np.float32 else tt._capi.F64
     g_dev, g_cpu = tt.Generator(0), oracle.Generator(0)

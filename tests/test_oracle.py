@@ -405,10 +405,15 @@ def test_linear_default_init(oracle):
     assert W.shape == (784, 16) and b.shape == (16,)
     bw, bb = np.sqrt(3.0) / 28.0, 1.0 / 28.0
     assert np.abs(W).max() < bw and np.abs(W).max() > 0.99 * bw
-    assert np.abs(b).max() < bb
+    assert np.abs(b).max() < bb and np.abs(b).max() > 0.5 * bb
     g2 = oracle.Generator(0)
     W2 = g2.uniform_real(-bw, bw, (784, 16))
     assert np.array_equal(W, W2)
+    # the bias is the SECOND draw of the same generator at bound 1/sqrt(in) (nn/linear.cpp:33-38, nn/init.cpp:106-112),
+    # exactly: a bound from the wrong fan (out = 16 -> 0.25) or a fresh generator gives other values
+    assert np.array_equal(b, g2.uniform_real(-bb, bb, (16,)))
+    assert g.state == g2.state
+    assert not np.array_equal(b, oracle.Generator(0).uniform_real(-bb, bb, (16,)))
     assert abs(W.astype(np.float64).var() - bw * bw / 3) < 2e-5
 
 
@@ -434,6 +439,39 @@ def test_in_place_draw_through_a_view_brute_force(oracle, dtype):
     g2 = oracle.Generator(9)
     g2.uniform_real(-0.5, 0.25, (view.size,), dtype)
     assert g.state == g2.state  # one master output per element, nothing else
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+@pytest.mark.parametrize("dist", [0, 1])
+def test_draws_with_a_parameter_pair_per_element_brute_force(oracle, dtype, dist):
+    # The tensor forms of uniform_real_ / normal_ (cpu/distribution.cpp:96-139): element i of the view takes the i-th
+    # master output as its state and the i-th pair of the (contiguous) parameters.  Independent statement, element by
+    # element: a dense draw from the same seed with that element's pair as the scalars agrees at index i -- every
+    # element depends on its own state and its own pair only.
+    rng = np.random.default_rng(5)
+    base = np.full((4, 6, 5), -7.0, dtype=dtype)
+    view = base.transpose(1, 0, 2)[1:, :, 1:4]              # shape [5,4,3], permuted, offset, non-dense
+    n = view.size
+    p0 = rng.uniform(-2.0, 1.0, view.shape).astype(dtype)
+    p1 = (p0 + rng.uniform(0.1, 3.0, view.shape)).astype(dtype) if dist == 0 else rng.uniform(0.1, 2.0, view.shape).astype(dtype)
+    g = oracle.Generator(21)
+    g.draw_params_(view, dist, p0, p1)
+    want = np.full((4, 6, 5), -7.0, dtype=dtype)
+    i = 0
+    for a in range(5):
+        for b in range(4):
+            for c in range(3):
+                ref = oracle.Generator(21)
+                dense = (ref.uniform_real if dist == 0 else ref.normal)(float(p0[a, b, c]), float(p1[a, b, c]), (n,), dtype)
+                want[b, a + 1, c + 1] = dense[i]
+                i += 1
+    assert np.array_equal(base, want)
+    assert g.state == ref.state                              # n master outputs consumed
+    # exchanging the two parameter tensors, or reading them in the view's storage order, gives other values
+    other = np.full((4, 6, 5), -7.0, dtype=dtype)
+    oview = other.transpose(1, 0, 2)[1:, :, 1:4]
+    oracle.Generator(21).draw_params_(oview, dist, np.ascontiguousarray(p0.transpose(1, 0, 2)).reshape(view.shape), p1)
+    assert not np.array_equal(other, want)
 
 
 def test_conv2d_default_init(oracle):

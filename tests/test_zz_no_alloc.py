@@ -134,3 +134,45 @@ def test_products_beyond_the_fixed_array_are_refused(tt):
     st = lib.ttamd_batched_matmul(0, capi.F64, B, N, K, M, C.byref(lv), C.byref(rv), C.c_void_p(out.storage.ptr), None, None)
     assert st == capi.OK, capi.last_error()
     be.synchronize(0)
+
+
+def test_a_second_stream_is_refused_until_the_device_has_been_synchronised(tt):
+    """Every stream of a GPU shares the fixed array: a call that needs it on another stream than the last one is
+    refused (two products in flight would overwrite each other's partial tiles) until ttamd_device_synchronize has run;
+    products that use no scratch are not affected."""
+    from tinytensor_amd.graph import Stream
+    capi, lib = tt._capi, tt._capi.lib
+    be = tt.get_backend(tt.kAMD)
+    rng = np.random.default_rng(7)
+    a, b = _pair(rng, np.float32, 1, 320, 512, 416, integer_valued=True)
+    tA, tB = tt.Tensor.from_numpy(a), tt.Tensor.from_numpy(b)
+    assert "splitk" in be.batched_matmul_variant(tA, tB)
+    out = tt.Tensor.empty((1, 320, 416), capi.F32)
+    lv, rv = tA.view3(), tB.view3()
+
+    def call(stream_handle, lhs=lv, rhs=rv, dims=(1, 320, 512, 416), dst=out):
+        return lib.ttamd_batched_matmul_noalloc(0, capi.F32, *dims, C.byref(lhs), C.byref(rhs), C.c_void_p(dst.storage.ptr), None,
+                                                C.c_void_p(stream_handle) if stream_handle else None)
+
+    be.synchronize(0)
+    side = Stream(non_blocking=True)
+    try:
+        assert call(None) == capi.OK, capi.last_error()                    # default stream
+        assert call(None) == capi.OK, capi.last_error()                    # the same stream again: ordered by the stream
+        assert call(side.handle) == capi.ERR_INVALID_ARGUMENT              # another stream, nothing synchronised
+        assert "another stream" in capi.last_error()
+        # a product without scratch goes through on any stream
+        small_a, small_b = tt.Tensor.from_numpy(a[:, :130, :70].copy()), tt.Tensor.from_numpy(b[:, :70, :150].copy())
+        small_out = tt.Tensor.empty((1, 130, 150), capi.F32)
+        assert "splitk" not in be.batched_matmul_variant(small_a, small_b)
+        assert call(side.handle, small_a.view3(), small_b.view3(), (1, 130, 70, 150), small_out) == capi.OK, capi.last_error()
+        be.synchronize(0)                                                   # ttamd_device_synchronize
+        assert call(side.handle) == capi.OK, capi.last_error()
+        side.synchronize()
+        assert np.array_equal(out.to_numpy()[0], (a[0].astype(np.float64) @ b[0].astype(np.float64)).astype(np.float32))
+        assert call(None) == capi.ERR_INVALID_ARGUMENT                      # and back: the same rule
+        be.synchronize(0)
+        assert call(None) == capi.OK, capi.last_error()
+        be.synchronize(0)
+    finally:
+        side.close()

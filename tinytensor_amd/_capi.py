@@ -68,6 +68,9 @@ def _bind(lib: C.CDLL) -> None:
                                        C.POINTER(C.c_int64), vp, C.c_int64, vp]),
         "ttamd_random_fill_states": (i, [i, i, i, C.c_double, C.c_double, C.POINTER(C.c_uint64), i, C.POINTER(C.c_int64),
                                          C.POINTER(C.c_int64), vp, C.c_int64, vp]),
+        "ttamd_random_fill_states_params": (i, [i, i, i, vp, C.c_int64, C.POINTER(C.c_int64), vp, C.c_int64, C.POINTER(C.c_int64),
+                                                C.POINTER(C.c_uint64), i, C.POINTER(C.c_int64), C.POINTER(C.c_int64), vp,
+                                                C.c_int64, vp]),
         "ttamd_batched_matmul": (i, [i, i, i, i, i, i, C.POINTER(View3), C.POINTER(View3), vp, C.POINTER(Epilogue), vp]),
         "ttamd_batched_matmul_noalloc": (i, [i, i, i, i, i, i, C.POINTER(View3), C.POINTER(View3), vp, C.POINTER(Epilogue), vp]),
         "ttamd_batched_matmul_variant": (C.c_char_p, [i, i, i, i, i, C.POINTER(View3), C.POINTER(View3)]),

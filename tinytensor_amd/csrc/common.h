@@ -72,6 +72,10 @@ inline FastDiv make_fastdiv(uint32_t d) {
 // buffers.  Growing allocates (hipMalloc, at least double the size); the outgrown buffer is kept until the process
 // ends, because kernels in flight and captured graphs may still refer to it.
 ttamd_status stream_scratch(int device, hipStream_t stream, size_t bytes, void **out);
+// Whole-device synchronisations (ttamd_device_synchronize) of `device`: how many have started, how many have finished.
+// A use of shared memory that notes `started` at its launch is known to be over once `completed` exceeds that note.
+uint64_t device_sync_started(int device);
+uint64_t device_sync_completed(int device);
 
 // One GEMM problem as the kernels see it.  Conventional letters inside the kernels:
 // C[M,N] = A[M,K] . B[K,N]  (the C ABI's N,K,M map to M,K,N here).

@@ -480,6 +480,32 @@ __global__ void __launch_bounds__(256) normal_kernel(const uint64_t *__restrict_
     out[dense ? i : flat_of(i, v)] = stddev * (r * sin(theta)) + mu;
 }
 
+// The same draws with a parameter pair per element (the tensor forms of BackendBase::uniform_real / normal,
+// backend_base.h:83-103): element i reads its parameters at rank i of the parameter views, which is what the CPU
+// backend's params[i] on the parameters made contiguous reads (cpu/distribution.cpp:42-47, cpu/kernel/distribution.hpp:28-32).
+template <typename T, int DIST>
+__global__ void __launch_bounds__(256) random_params_kernel(const uint64_t *__restrict__ states, const T *__restrict__ p0, ViewDesc v0,
+                                                           const T *__restrict__ p1, ViewDesc v1, T *__restrict__ out, ViewDesc v, bool dense,
+                                                           int64_t n) {
+    const int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    uint64_t st = states[i];
+    const T a = p0[flat_of(i, v0)];
+    const T b = p1[flat_of(i, v1)];
+    T value;
+    if (DIST == 0) {
+        const T r = unit_sample(st, T(0));
+        value = fma(r, b - a, a);
+    } else {
+        const T u1 = unit_sample(st, T(0));
+        const T u2 = unit_sample(st, T(0));
+        const T r = sqrt(T(-2) * log1p(-u1));
+        const T theta = T(2) * T(3.14159265358979323846) * u2;
+        value = b * (r * sin(theta)) + a;
+    }
+    out[dense ? i : flat_of(i, v)] = value;
+}
+
 // to(dtype): out[i] = static_cast<R>(view[i]) (tinytensor/tensor/backend/cpu/cast.cpp:27-34; bool keeps C++'s
 // "non-zero is true").
 template <typename T, typename R>
@@ -785,7 +811,8 @@ __global__ void __launch_bounds__(THREADS) mse_loss_kernel(const T *__restrict__
     __shared__ T red[RL][CP + 1];
     __shared__ T red_loss[THREADS];
     const int cl = threadIdx.x % CP, rl = threadIdx.x / CP;
-    const T scale = inv_n * T(2);
+    const T scale = inv_n * T(2);                                  // (1 / numel) * 2, the factor the reference's backward forms
+    const T n = static_cast<T>(rows * static_cast<int64_t>(cols));  // the forward divides each term by numel (reduce_ops.cpp:199)
     T csum = T(0), lsum = T(0);
     if (cl < cols) {
         const int64_t step = static_cast<int64_t>(gridDim.x) * RL;
@@ -802,7 +829,7 @@ __global__ void __launch_bounds__(THREADS) mse_loss_kernel(const T *__restrict__
             for (int u = 0; u < U; ++u) {
                 const int64_t r = r0 + u * step;
                 const T d = r < rows ? yv[u] - tv[u] : T(0);
-                lsum += d * d * inv_n;
+                lsum += d * d / n;
                 const T g = scale * d;
                 if (grad && r < rows) grad[r * cols + cl] = g;
                 csum += g;
@@ -1197,6 +1224,18 @@ ttamd_status ttamd_full(int device, ttamd_dtype dtype, const void *value, int64_
 // dist: 0 = uniform_real(low = p0, high = p1), 1 = normal(mu = p0, std = p1).  `states`: one generator state per element
 // of the view, in the view's row-major order, produced on the host (cpu/distribution.cpp:31-38 draws them from the
 // caller's Generator one by one; the reference's GPU backend uploads them the same way, cuda/distribution.cu:32-99).
+namespace {
+// Parameters of a draw: one pair of values for the whole tensor, or a pair of views read per element
+struct DrawParams {
+    double p0 = 0.0, p1 = 0.0;
+    const void *d0 = nullptr, *d1 = nullptr;  // per-element parameter data (at the views' offsets) when both are set
+    ViewDesc v0{}, v1{};
+};
+
+ttamd_status random_fill_impl(int device, ttamd_dtype dtype, int dist, const DrawParams &par, const uint64_t *states, const ViewDesc &v,
+                              int64_t numel, void *data, int64_t offset, void *stream);
+}  // namespace
+
 ttamd_status ttamd_random_fill_states(int device, ttamd_dtype dtype, int dist, double p0, double p1, const uint64_t *states, int ndim,
                                       const int64_t *shape, const int64_t *stride, void *data, int64_t offset, void *stream) {
     if (dtype != TTAMD_F32 && dtype != TTAMD_F64) {
@@ -1210,6 +1249,47 @@ ttamd_status ttamd_random_fill_states(int device, ttamd_dtype dtype, int dist, d
     ViewDesc v;
     int64_t numel = 0;
     if (ttamd_status s = make_view("random_fill", ndim, shape, stride, &v, &numel)) return s;
+    DrawParams par;
+    par.p0 = p0;
+    par.p1 = p1;
+    return random_fill_impl(device, dtype, dist, par, states, v, numel, data, offset, stream);
+}
+
+// The draws with a parameter pair per element: p0 / p1 are views over the same shape as the result (element offsets and
+// strides, stride 0 for an expanded parameter), read on the device.  uniform_real expects low < high in every element,
+// which the reference only asserts (common/kernel/distribution.hpp:95); it is not checked here.
+ttamd_status ttamd_random_fill_states_params(int device, ttamd_dtype dtype, int dist, const void *p0, int64_t p0_offset,
+                                             const int64_t *p0_stride, const void *p1, int64_t p1_offset, const int64_t *p1_stride,
+                                             const uint64_t *states, int ndim, const int64_t *shape, const int64_t *stride, void *data,
+                                             int64_t offset, void *stream) {
+    if (dtype != TTAMD_F32 && dtype != TTAMD_F64) {
+        set_error("random_fill: floating point dtypes only");
+        return TTAMD_ERR_UNSUPPORTED_DTYPE;
+    }
+    if (offset < 0 || p0_offset < 0 || p1_offset < 0 || (dist != 0 && dist != 1)) {
+        set_error("random_fill: invalid arguments (negative offset or unknown distribution)");
+        return TTAMD_ERR_INVALID_ARGUMENT;
+    }
+    ViewDesc v;
+    DrawParams par;
+    int64_t numel = 0;
+    if (ttamd_status s = make_view("random_fill", ndim, shape, stride, &v, &numel)) return s;
+    if (ttamd_status s = make_view("random_fill", ndim, shape, p0_stride, &par.v0, nullptr)) return s;
+    if (ttamd_status s = make_view("random_fill", ndim, shape, p1_stride, &par.v1, nullptr)) return s;
+    if (numel > 0 && (!p0 || !p1)) {
+        set_error("random_fill: NULL parameter pointer");
+        return TTAMD_ERR_INVALID_ARGUMENT;
+    }
+    const int64_t es = static_cast<int64_t>(dtype_size(dtype));
+    par.d0 = static_cast<const char *>(p0) + p0_offset * es;
+    par.d1 = static_cast<const char *>(p1) + p1_offset * es;
+    return random_fill_impl(device, dtype, dist, par, states, v, numel, data, offset, stream);
+}
+
+namespace {
+ttamd_status random_fill_impl(int device, ttamd_dtype dtype, int dist, const DrawParams &par, const uint64_t *states, const ViewDesc &v,
+                              int64_t numel, void *data, int64_t offset, void *stream) {
+    const double p0 = par.p0, p1 = par.p1;
     if (ttamd_status s = use_device(device)) return s;
     if (numel == 0) return TTAMD_OK;
     if (!data || !states) {
@@ -1242,7 +1322,15 @@ ttamd_status ttamd_random_fill_states(int device, ttamd_dtype dtype, int dist, d
     if (rc == TTAMD_OK) {
         const unsigned blocks = static_cast<unsigned>((numel + 255) / 256);
         const uint64_t *sp = static_cast<const uint64_t *>(dev_states);
-        if (dtype == TTAMD_F32) {
+        if (par.d0 && par.d1) {
+            auto launch = [&]<typename T>(T) {
+                const T *a = static_cast<const T *>(par.d0), *b = static_cast<const T *>(par.d1);
+                if (dist == 0) random_params_kernel<T, 0><<<dim3(blocks), dim3(256), 0, st>>>(sp, a, par.v0, b, par.v1, static_cast<T *>(out), v, dense, numel);
+                else random_params_kernel<T, 1><<<dim3(blocks), dim3(256), 0, st>>>(sp, a, par.v0, b, par.v1, static_cast<T *>(out), v, dense, numel);
+            };
+            if (dtype == TTAMD_F32) launch(float{});
+            else launch(double{});
+        } else if (dtype == TTAMD_F32) {
             if (dist == 0) uniform_real_kernel<float><<<dim3(blocks), dim3(256), 0, st>>>(sp, static_cast<float>(p0), static_cast<float>(p1), static_cast<float *>(out), v, dense, numel);
             else normal_kernel<float><<<dim3(blocks), dim3(256), 0, st>>>(sp, static_cast<float>(p0), static_cast<float>(p1), static_cast<float *>(out), v, dense, numel);
         } else {
@@ -1256,6 +1344,7 @@ ttamd_status ttamd_random_fill_states(int device, ttamd_dtype dtype, int dist, d
     (void)hipHostFree(host_states);
     return rc;
 }
+}  // namespace
 
 // The same with the states drawn here: *master_state is the caller's master generator state (Generator::state, xorshift64
 // with shifts 13, 7, 17: tensor/random.cpp:36-43); it advances by one output per element of the view.

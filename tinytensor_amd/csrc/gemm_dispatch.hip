@@ -119,22 +119,35 @@ ttamd_status run_product(ttamd_dtype dtype, const GemmArgs &g, int device, hipSt
         if (ttamd_status s = launch_gemm_mfma(dtype, g, device, st, &variant, false, &handled, fixed_scratch)) return s;
         if (handled) return TTAMD_OK;
     }
-    // K == 0 also lands here: the vector-ALU kernel then stores the empty sum (0, + bias).  It uses no scratch.
-    if (g.colsum_out) {
-        set_error("batched_matmul: colsum_out needs the matrix-core kernels (K > 0, rows under a tile below 2 GiB)");
-        return TTAMD_ERR_INVALID_ARGUMENT;
-    }
-    return launch_gemm_simt(dtype, g, st, &variant, false);
+    // K == 0 also lands here: the vector-ALU kernel then stores the empty sum (0, + bias).  It uses no scratch.  The
+    // column sums of the result, which that kernel does not form, are taken from the dense result afterwards (its rows
+    // added in order).
+    if (ttamd_status s = launch_gemm_simt(dtype, g, st, &variant, false)) return s;
+    if (g.colsum_out) return launch_colsum_reduce(dtype, g.C, g.M, g.N, g.batch, g.colsum_out, st);
+    return TTAMD_OK;
 }
 
 ttamd_status batched_matmul(int device, ttamd_dtype dtype, int B, int N, int K, int M, const ttamd_view3 *lhs,
                             const ttamd_view3 *rhs, void *out, const ttamd_epilogue *epilogue, void *stream, bool fixed_scratch) {
     GemmArgs g;
     if (ttamd_status s = build_args(dtype, B, N, K, M, lhs, rhs, out, epilogue, &g, true)) return s;
+    // build_args has not looked at the data pointers of an empty product; the one such a call still reads (the right
+    // operand, for its sums over k) is checked here, before any device work
+    if (N == 0 && B > 0 && M > 0 && K > 0 && g.rhs_colsum &&
+        (!rhs->data || reinterpret_cast<uintptr_t>(rhs->data) % dtype_size(dtype) != 0)) {
+        set_error("batched_matmul: rhs_colsum_out needs the right operand's data (NULL or misaligned pointer)");
+        return TTAMD_ERR_INVALID_ARGUMENT;
+    }
     if (ttamd_status s = use_device(device)) return s;
     hipStream_t st = static_cast<hipStream_t>(stream);
-    if (B == 0 || N == 0 || M == 0) {  // no product; the right operand's sums exist all the same when it has columns
-        if (g.rhs_colsum && B > 0 && M > 0) return launch_colsum_reduce(dtype, g.B, g.K, g.N, g.batch, g.rhs_colsum, st);
+    if (B == 0 || N == 0 || M == 0) {
+        // No product.  With batches and columns but no rows (N == 0) the sums over the rows exist all the same: the
+        // result's column sums are zeros, the right operand's are what they always are.
+        if (B > 0 && M > 0) {
+            if (g.colsum_out)
+                if (ttamd_status s = launch_colsum_reduce(dtype, nullptr, 0, g.N, g.batch, g.colsum_out, st)) return s;
+            if (g.rhs_colsum) return launch_colsum_reduce(dtype, g.B, g.K, g.N, g.batch, g.rhs_colsum, st);
+        }
         return TTAMD_OK;
     }
     bool rhs_sums_done = false;

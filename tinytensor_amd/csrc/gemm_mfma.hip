@@ -7,6 +7,7 @@
 // tinytensor/tensor/backend/cpu/matmul.cpp:37-38 and cuda/matmul.cu:40-41.
 // The tile engine (LDS double buffering, MFMA loop, layouts) lives in mfma_core.h; this file adds the
 // kernel entry, the workgroup -> tile mapping and the host-side operand classification.
+#include <atomic>
 #include "mfma_core.h"
 
 #include <algorithm>
@@ -241,7 +242,7 @@ __global__ void __launch_bounds__(256) splitk_reduce_kernel(GemmArgs g, const T 
     const T *bias = static_cast<const T *>(g.bias);
     if (g.bias_mode == 1) v += bias[i % g.N];
     if (g.bias_mode == 2) v += bias[i / g.N];
-    if (g.zmask && static_cast<const T *>(g.zmask)[static_cast<int64_t>(batch) * mn + i] < T(0)) v = T(0);
+    if (g.zmask && static_cast<const T *>(g.zmask)[static_cast<int64_t>(batch) * mn + i] < T(0)) v = v * T(0);  // the reference multiplies by 0 (NaN / -0 propagate)
     if (g.relu) v = v > T(0) ? v : T(0);
     T *C = static_cast<T *>(g.C) + static_cast<int64_t>(batch) * mn;
     if (g.accumulate) v += C[i];
@@ -328,6 +329,33 @@ ttamd_status launch_scratch(int device, hipStream_t stream, size_t bytes, bool f
                   "the column sums' rows); the fixed scratch holds %zu (use ttamd_batched_matmul)", bytes, kFixedScratchBytes);
         return TTAMD_ERR_INVALID_ARGUMENT;
     }
+    // Every stream of a GPU shares the one array.  The last stream that used it is remembered; a call on another stream
+    // is only let through once the whole device has been synchronised since that use (ttamd_device_synchronize), because
+    // two products in flight at once would overwrite each other's partial results without any error.
+    {
+        struct LastUse {
+            bool used = false;
+            hipStream_t stream = nullptr;
+            uint64_t syncs_started = 0;
+        };
+        static std::mutex mu;
+        static LastUse last[kMaxDevices];
+        if (device < 0 || device >= kMaxDevices) {
+            set_error("batched_matmul_noalloc: device id %d beyond the %d devices the fixed scratch serves", device, kMaxDevices);
+            return TTAMD_ERR_INVALID_DEVICE;
+        }
+        std::lock_guard<std::mutex> lock(mu);
+        LastUse &u = last[device];
+        if (u.used && u.stream != stream && device_sync_completed(device) <= u.syncs_started) {
+            set_error("batched_matmul_noalloc: the fixed scratch of device %d was last used on another stream and the device has "
+                      "not been synchronised since (ttamd_device_synchronize); products in flight on two streams would "
+                      "overwrite each other's partial results", device);
+            return TTAMD_ERR_INVALID_ARGUMENT;
+        }
+        u.used = true;
+        u.stream = stream;
+        u.syncs_started = device_sync_started(device);
+    }
     return fixed_scratch_address(device, out);
 }
 
@@ -374,12 +402,12 @@ ttamd_status launch_variant(const GemmArgs &g, const SplitPlan &sp, int device, 
                   : which == 1 ? gemm_mfma_kernel<T, BM, BN, BK, WGM, WGN, A_KC, A_VEC, B_KC, B_VEC, PF, kEpiB>
                   : which == 2 ? gemm_mfma_kernel<T, BM, BN, BK, WGM, WGN, A_KC, A_VEC, B_KC, B_VEC, PF, kEpiC>
                                : gemm_mfma_kernel<T, BM, BN, BK, WGM, WGN, A_KC, A_VEC, B_KC, B_VEC, PF, kEpiD>;
-    static bool configured[kMaxDevices][4] = {};  // raising the dynamic LDS limit: once per kernel and device
+    static std::atomic<bool> configured[kMaxDevices][4] = {};  // raising the dynamic LDS limit: once per kernel and device (host threads may race here: setting the attribute twice is harmless, a torn flag would not be)
     const int slot = device >= 0 && device < kMaxDevices ? device : 0;
-    if ((!configured[slot][which] || slot != device) && lds_bytes > 48 * 1024) {
+    if ((!configured[slot][which].load(std::memory_order_acquire) || slot != device) && lds_bytes > 48 * 1024) {
         TTAMD_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
                                             hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds_bytes)));
-        configured[slot][which] = true;
+        configured[slot][which].store(true, std::memory_order_release);
     }
     const int tiles_m = (g.M + BM - 1) / BM, tiles_n = (g.N + BN - 1) / BN;
     const int64_t blocks = static_cast<int64_t>(tiles_m) * tiles_n * g.batch * sp.ksplit;
@@ -425,12 +453,12 @@ ttamd_status launch_dual_variant(const GemmArgs &g, int device, hipStream_t stre
     using StB = Stager<T, BN, BK, B_KC, B_VEC, PF, BSUM>;
     constexpr size_t lds_bytes = 2 * TileEngine<T, BM, BN, BK, WGM, WGN, StA, StB>::kLdsBytes;
     auto kernel = gemm_mfma_dual_kernel<T, BM, BN, BK, WGM, WGN, A_KC, A_VEC, B_KC, B_VEC, PF, BSUM>;
-    static bool configured[kMaxDevices] = {};  // once per kernel and device
+    static std::atomic<bool> configured[kMaxDevices] = {};  // once per kernel and device
     const int slot = device >= 0 && device < kMaxDevices ? device : 0;
-    if (!configured[slot] || slot != device) {
+    if (!configured[slot].load(std::memory_order_acquire) || slot != device) {
         TTAMD_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
                                             static_cast<int>(lds_bytes)));
-        configured[slot] = true;
+        configured[slot].store(true, std::memory_order_release);
     }
     const int k_half = dual_k_half<T>(g.K);
     if (k_half <= 0 || (k_half + BK - 1) / BK != (g.K - k_half + BK - 1) / BK) {  // the halves share the engine's barriers

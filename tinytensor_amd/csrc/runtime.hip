@@ -186,6 +186,13 @@ ttamd_status stream_scratch(int device, hipStream_t stream, size_t bytes, void *
     return TTAMD_OK;
 }
 
+uint64_t device_sync_started(int device) {
+    return device >= 0 && device < kMaxDevices ? g_cache[device].epoch.load() : 0;
+}
+uint64_t device_sync_completed(int device) {
+    return device >= 0 && device < kMaxDevices ? g_cache[device].synced.load() : 0;
+}
+
 }  // namespace ttamd
 
 using namespace ttamd;

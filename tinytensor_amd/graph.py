@@ -29,7 +29,7 @@ def _runtime():
         vp = C.c_void_p
         for name, args in {
             "hipStreamCreate": [C.POINTER(vp)], "hipStreamCreateWithFlags": [C.POINTER(vp), C.c_uint],
-            "hipStreamSynchronize": [vp], "hipStreamDestroy": [vp],
+            "hipStreamSynchronize": [vp], "hipStreamDestroy": [vp], "hipStreamQuery": [vp],
             "hipStreamBeginCapture": [vp, C.c_int], "hipStreamEndCapture": [vp, C.POINTER(vp)],
             "hipGraphInstantiate": [C.POINTER(vp), vp, C.POINTER(vp), C.c_char_p, C.c_size_t],
             "hipGraphLaunch": [vp, vp], "hipGraphExecDestroy": [vp], "hipGraphDestroy": [vp],
@@ -74,6 +74,13 @@ class Stream:
 
     def synchronize(self) -> None:
         _call("hipStreamSynchronize", self._h)
+
+    def is_idle(self) -> bool:
+        """Whether everything enqueued on the stream so far has finished (hipStreamQuery; not during a capture)."""
+        rc = _runtime().hipStreamQuery(self._h)
+        if rc not in (0, 600):  # hipSuccess, hipErrorNotReady
+            raise TTException(f"hipStreamQuery failed with HIP error {rc}")
+        return rc == 0
 
     def run(self, fn):
         """Calls fn() with every backend launch going to this stream (asynchronously); returns fn's result."""

@@ -6,9 +6,10 @@
 //   the GEMM path  batched_matmul, conv2d, conv2d_backward (operands are read through their strides, no contiguous copy)
 //   around it      identity (= clone / contiguous), to, assign, add/sub/mul/div/pow/maximum/minimum and their in-place
 //                  forms, eq/ne/lt/le/gt/ge, negate/abs/sqrt/exp/log/sigmoid/tanh/relu and their in-place forms, where,
-//                  sum, max/min/avg pooling forward and backward, uniform_real / normal with parameters that are one
-//                  value expanded over the shape (what Tensor::uniform_real_(double, double) and nn::init pass,
-//                  tensor/tensor.cpp:1795-1801)
+//                  sum, all / any of a whole tensor (the frontend's argument checks use them, e.g. CHECK_UNIFORM,
+//                  tensor/tensor.cpp:1753-1759), max/min/avg pooling forward and backward, uniform_real / normal with
+//                  parameter tensors (a pair per element, or one value expanded over the shape as
+//                  Tensor::uniform_real_(double, double) and nn::init pass, tensor/tensor.cpp:1795-1801)
 // Everything else throws TTException("<op> is not implemented on the AMD device").
 //
 // Status codes of the C ABI map to the reference's error model: TTException for what a caller can act on, TT_ERROR
@@ -236,39 +237,24 @@ auto draw_states(Generator &gen, std::size_t n) -> std::vector<uint64_t> {
     return states;
 }
 
-// The value of a parameter tensor that is one element expanded over the shape (every stride 0), which is what the
-// scalar overloads of the frontend build (tensor/tensor.cpp:1795-1801); anything else is not served.
-auto expanded_scalar(const Tensor &param, const char *op) -> double {
-    const auto &shape = param.shape().to_vec();
-    const auto &stride = param.stride().to_vec();
-    for (std::size_t i = 0; i < shape.size(); ++i) {
-        if (shape[i] != 1 && stride[i] != 0) {
-            TT_EXCEPTION(std::string(op) + " with per-element parameters is not implemented on the AMD device");
-        }
-    }
-    double value = 0.0;
-    if (param.dtype() == kF32) {
-        float v = 0.0F;
-        check(ttamd_memcpy_d2h(param.device().id, &v, data_at_offset(param), sizeof(v)));
-        value = static_cast<double>(v);
-    } else {
-        check(ttamd_memcpy_d2h(param.device().id, &value, data_at_offset(param), sizeof(value)));
-    }
-    return value;
-}
-
-// dist: 0 uniform_real(low, high), 1 normal(mu, std); written through `tensor`'s view in its row-major order
+// dist: 0 uniform_real(low, high), 1 normal(mu, std); written through `tensor`'s view in its row-major order.  The
+// parameters are tensors of the same shape (the frontend checks it and casts them to the result's dtype,
+// tensor/tensor.cpp:1783-1794); element i reads its pair at rank i of their views, whether they hold a value per element
+// or one value expanded with stride 0 (what the scalar overloads build, tensor/tensor.cpp:1795-1801).
 void fill_random(Tensor &tensor, int dist, const Tensor &a, const Tensor &b, Generator &gen, const char *op) {
     if (!is_float_dtype(tensor.dtype())) {
         TT_EXCEPTION(std::string(op) + " expects a floating point tensor");
     }
-    const double p0 = expanded_scalar(a, op);
-    const double p1 = expanded_scalar(b, op);
+    if (a.dtype() != tensor.dtype() || b.dtype() != tensor.dtype() || a.numel() != tensor.numel() || b.numel() != tensor.numel()) {
+        TT_EXCEPTION(std::string(op) + " expects parameters of the result's shape and dtype");
+    }
     const std::vector<uint64_t> states = draw_states(gen, static_cast<std::size_t>(tensor.numel()));
     const View v(tensor);
-    check(ttamd_random_fill_states(
-        tensor.device().id, code(tensor.dtype()), dist, p0, p1, states.data(), v.ndim, v.shape.data(), v.stride.data(), v.data,
-        v.offset, nullptr
+    const View pa(a);
+    const View pb(b);
+    check(ttamd_random_fill_states_params(
+        tensor.device().id, code(tensor.dtype()), dist, pa.data, pa.offset, pa.stride.data(), pb.data, pb.offset, pb.stride.data(),
+        states.data(), v.ndim, v.shape.data(), v.stride.data(), v.data, v.offset, nullptr
     ));
 }
 
@@ -563,6 +549,22 @@ auto BackendAMD::sum(const Tensor &tensor, int dim) const -> Tensor {
     return sum_op(tensor, dim);
 }
 
+// all / any of a whole tensor: the number of non-zero elements (a cast to bool writes 0 or 1, its sum is 64-bit)
+namespace {
+auto count_nonzero(const BackendAMD &backend, const Tensor &tensor) -> int64_t {
+    const Tensor flags = tensor.dtype() == kBool ? tensor : backend.to(tensor, kBool);
+    return backend.item(sum_op(flags, -1)).to<int64_t>();
+}
+}    // namespace
+
+auto BackendAMD::all(const Tensor &tensor) const -> bool {
+    return count_nonzero(*this, tensor) == static_cast<int64_t>(tensor.numel());
+}
+
+auto BackendAMD::any(const Tensor &tensor) const -> bool {
+    return count_nonzero(*this, tensor) != 0;
+}
+
 // binary operators on the device, and the in-place forms (result into a temporary, then written through lhs's view)
 #define TT_AMD_DEVICE_BINARY(X)                                                                                        \
     X(add, TTAMD_BIN_ADD) X(sub, TTAMD_BIN_SUB) X(mul, TTAMD_BIN_MUL) X(div, TTAMD_BIN_DIV) X(pow, TTAMD_BIN_POW)      \
@@ -600,7 +602,7 @@ TT_AMD_DEVICE_UNARY(X)
 
 void BackendAMD::identity_(Tensor & /*tensor*/) const {}
 
-// seeded draws: uniform_real and normal with expanded-scalar parameters
+// seeded draws: uniform_real and normal
 auto BackendAMD::uniform_real(const Tensor &low, const Tensor &high, Generator &gen) const -> Tensor {
     return new_random(0, low, high, gen, "uniform_real");
 }
@@ -648,12 +650,6 @@ X(min) X(argmin) X(max) X(argmax) X(isinf) X(isnan) X(isfinite)
     }
 X(min) X(argmin) X(max) X(argmax) X(all) X(any) X(softmax) X(log_softmax)
 #undef X
-auto BackendAMD::all(const Tensor & /*tensor*/) const -> bool {
-    not_implemented("all");
-}
-auto BackendAMD::any(const Tensor & /*tensor*/) const -> bool {
-    not_implemented("any");
-}
 
 // Tensor f(const Tensor &lhs, const Tensor &rhs)
 #define X(NAME)                                                                            \

@@ -251,20 +251,28 @@ class Tensor:
     def item(self):
         return self.to_numpy().reshape(-1)[0]
 
-    def uniform_real_(self, low: float, high: float, gen: "Generator") -> "Tensor":
+    def uniform_real_(self, low, high, gen: "Generator") -> "Tensor":
         """Tensor::uniform_real_(low, high, gen) (tensor/tensor.cpp:1783-1801) -> BackendBase::uniform_real_: in place,
-        through this tensor's view (element i of the view takes the i-th draw, cpu/kernel/distribution.hpp:28-32)."""
+        through this tensor's view (element i of the view takes the i-th draw, cpu/kernel/distribution.hpp:28-32).
+        `low` / `high` are two numbers, or two tensors of this tensor's shape and dtype (a pair per element)."""
         if self.dtype not in (_capi.F32, _capi.F64):
             raise TTException("uniform_real_ expects a floating point tensor")
+        if isinstance(low, Tensor) or isinstance(high, Tensor):
+            get_backend(self.device).random_fill_params_(self, 0, low, high, gen)
+            return self
         if not low < high:
             raise TTException("Expected low < high. At least one element violates this.")
         get_backend(self.device).random_fill_(self, 0, low, high, gen)
         return self
 
-    def normal_(self, mu: float, std: float, gen: "Generator") -> "Tensor":
-        """Tensor::normal_(mu, std, gen) -> BackendBase::normal_, in place through this tensor's view."""
+    def normal_(self, mu, std, gen: "Generator") -> "Tensor":
+        """Tensor::normal_(mu, std, gen) -> BackendBase::normal_, in place through this tensor's view; the parameters
+        are two numbers or two tensors of this tensor's shape and dtype."""
         if self.dtype not in (_capi.F32, _capi.F64):
             raise TTException("normal_ expects a floating point tensor")
+        if isinstance(mu, Tensor) or isinstance(std, Tensor):
+            get_backend(self.device).random_fill_params_(self, 1, mu, std, gen)
+            return self
         get_backend(self.device).random_fill_(self, 1, mu, std, gen)
         return self
 
@@ -408,6 +416,27 @@ class BackendAMD:
         view `t` in place; `gen` advances by t.numel() outputs."""
         _check(lib.ttamd_random_fill_view(t.device.id, t.dtype, dist, p0, p1, C.byref(gen.state), t.dim(), self._i64(t.shape),
                                           self._i64(t.stride), C.c_void_p(t.storage.ptr), t.offset, _stream_arg()))
+
+    def random_fill_params_(self, t: Tensor, dist: int, a: Tensor, b: Tensor, gen: "Generator") -> None:
+        """BackendBase::uniform_real_ / normal_ (backend_base.h:96-103) with parameter tensors: element i of `t` reads
+        its pair at rank i of `a` and `b` (views over t's shape).  The states are drawn here, one per element, as
+        create_gen_states does (cpu/distribution.cpp:31-38)."""
+        if not (isinstance(a, Tensor) and isinstance(b, Tensor)) or a.shape != t.shape or b.shape != t.shape \
+                or a.dtype != t.dtype or b.dtype != t.dtype:
+            raise TTException("distribution parameters must be tensors of the result's shape and dtype")
+        n = t.numel()
+        states = (C.c_uint64 * max(n, 1))()
+        x, m = gen.state.value, (1 << 64) - 1
+        for i in range(n):
+            x ^= (x << 13) & m
+            x ^= x >> 7
+            x ^= (x << 17) & m
+            states[i] = x
+        _check(lib.ttamd_random_fill_states_params(
+            t.device.id, t.dtype, dist, C.c_void_p(a.storage.ptr), a.offset, self._i64(a.stride), C.c_void_p(b.storage.ptr),
+            b.offset, self._i64(b.stride), states, t.dim(), self._i64(t.shape), self._i64(t.stride), C.c_void_p(t.storage.ptr),
+            t.offset, _stream_arg()))
+        gen.state = C.c_uint64(x)
 
     def to(self, t: Tensor, dtype: int) -> Tensor:
         """BackendBase::to(tensor, dtype) (backend_base.h:74): element-wise static_cast into dense storage."""
@@ -711,6 +740,10 @@ def _constant(shape, value, dtype: int, device: Device) -> Tensor:
             if len(_CONSTANTS) >= 256:
                 _CONSTANTS.pop(next(iter(_CONSTANTS)))
             _CONSTANTS[key] = one
+    elif _PINNED is not None:
+        # a cached constant read inside a capture: the graph replays with this address, so the storage must outlive
+        # its eviction from the cache (otherwise the block could go to another tensor between replays)
+        _PINNED.append(one.storage)
     return Tensor(one.storage, dtype, shape, (0,) * len(shape), 0)
 
 
