@@ -74,7 +74,8 @@ typedef struct ttamd_view4 {
  * that follows it in an MLP, conv2d's per-channel bias (cpu/conv.cpp:115-124), and the
  * element-wise steps that autograd places around the backward GEMMs of a Linear layer.
  * Order of application to each element v of A.B:
- *   v += bias;  v = 0 where relu_grad_input < 0;  v = max(v, 0) if relu;  v += out if accumulate;
+ *   v += bias;  v *= 0 where relu_grad_input < 0 (a product: NaN or infinite v stays NaN);  v = max(v, 0) if relu;
+ *   v += out if accumulate;
  *   out = v;  relu_out = max(v, 0);  colsum_out[column] += v.
  * rhs_colsum_out does not depend on the product. */
 typedef struct ttamd_epilogue {
@@ -88,7 +89,8 @@ typedef struct ttamd_epilogue {
      * Not together with `relu`. */
     void *relu_out;
     /* TensorRelu::backward (autograd/unary_ops.cpp:568-573: grad_output * where(input < 0, 0, 1)) applied by the
-     * GEMM that computes grad_output: dense [B,N,M] like out, the ReLU's saved input, or NULL. */
+     * GEMM that computes grad_output: dense [B,N,M] like out, the ReLU's saved input, or NULL.  (A masked zero
+     * comes out as +0 where the reference's product leaves -0 under a negative value; the two compare equal.) */
     const void *relu_grad_input;
     /* Sum of `out` over its rows, [B,M] (or NULL): the gradient of a Linear layer's bias, which nn/linear.cpp:45-48
      * adds as an expanded view, so its gradient sums the batch dimension.  Per-tile partial sums are added in a fixed
@@ -133,8 +135,11 @@ ttamd_status ttamd_memory_allocated(int device, uint64_t *current_bytes, uint64_
  * completed, and to anyone after ttamd_device_synchronize.  A caller that uses a block on a third stream
  * synchronises that stream before the free.  TTAMD_ALLOC_CACHE=0 switches the cache off.  ttamd_empty_cache waits
  * for the device and returns every cached block to the driver; ttamd_memory_cached reports the bytes currently
- * cached.  No counterpart in the reference, whose DeviceMemory<T> calls cudaMalloc / cudaFree directly
- * (cuda/data_types.cuh:28-101). */
+ * cached.  Several host threads: a request that considers a block of another stream records and queries events, and
+ * a request that the driver cannot serve synchronises the device before it tries again; either would invalidate a
+ * graph capture that ANOTHER thread has open in global capture mode, so threads that capture use thread-local or
+ * relaxed capture mode, or keep other threads from allocating meanwhile.  No counterpart in the reference, whose
+ * DeviceMemory<T> calls cudaMalloc / cudaFree directly (cuda/data_types.cuh:28-101). */
 ttamd_status ttamd_malloc_on_stream(int device, size_t bytes, void *stream, void **out);
 ttamd_status ttamd_free_on_stream(int device, void *ptr, size_t bytes, void *stream);
 

@@ -242,7 +242,7 @@ __global__ void __launch_bounds__(256) splitk_reduce_kernel(GemmArgs g, const T 
     const T *bias = static_cast<const T *>(g.bias);
     if (g.bias_mode == 1) v += bias[i % g.N];
     if (g.bias_mode == 2) v += bias[i / g.N];
-    if (g.zmask && static_cast<const T *>(g.zmask)[static_cast<int64_t>(batch) * mn + i] < T(0)) v = v * T(0);  // the reference multiplies by 0 (NaN / -0 propagate)
+    if (g.zmask && static_cast<const T *>(g.zmask)[static_cast<int64_t>(batch) * mn + i] < T(0)) v = v * T(0);  // the reference multiplies by 0: an infinite or NaN value under the mask stays NaN
     if (g.relu) v = v > T(0) ? v : T(0);
     T *C = static_cast<T *>(g.C) + static_cast<int64_t>(batch) * mn;
     if (g.accumulate) v += C[i];

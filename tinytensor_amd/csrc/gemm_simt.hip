@@ -133,7 +133,7 @@ __global__ void __launch_bounds__(256) gemm_simt_kernel(GemmArgs g, int tiles_m,
             if (g.bias_mode == 1) v = static_cast<T>(v + bias[n]);
             if (g.bias_mode == 2) v = static_cast<T>(v + bias[m]);
             const int64_t idx = static_cast<int64_t>(m) * g.N + n;
-            if (g.zmask && static_cast<const T *>(g.zmask)[static_cast<int64_t>(batch) * g.M * g.N + idx] < T(0)) v = static_cast<T>(v * T(0));  // the reference multiplies by 0 (NaN / -0 propagate)
+            if (g.zmask && static_cast<const T *>(g.zmask)[static_cast<int64_t>(batch) * g.M * g.N + idx] < T(0)) v = static_cast<T>(v * T(0));  // the reference multiplies by 0: an infinite or NaN value under the mask stays NaN
             if (g.relu) v = relu_of<T>(v);
             if (g.accumulate) v = static_cast<T>(v + C[idx]);
             C[idx] = v;

@@ -126,7 +126,7 @@ __global__ void __launch_bounds__(64 * kThinWaves) gemm_thin_kernel(GemmArgs g) 
     const T *bias = static_cast<const T *>(g.bias);
     if (g.bias_mode == 1) v += bias[n];
     if (g.bias_mode == 2) v += bias[m];
-    if (g.zmask && static_cast<const T *>(g.zmask)[idx] < T(0)) v = v * T(0);  // the reference multiplies by 0 (NaN / -0 propagate)
+    if (g.zmask && static_cast<const T *>(g.zmask)[idx] < T(0)) v = v * T(0);  // the reference multiplies by 0: an infinite or NaN value under the mask stays NaN
     if (g.relu) v = v > T(0) ? v : T(0);
     T *C = static_cast<T *>(g.C);
     if (g.accumulate) v += C[idx];
@@ -267,7 +267,7 @@ __global__ void __launch_bounds__(64 * kThinWaves) gemm_thin_k_kernel(GemmArgs g
             T v = acc[e];
             if (g.bias_mode == 1 && in[e]) v += bias[n];
             if (g.bias_mode == 2 && in[e]) v += bias[m];
-            if (zv[u][e] < T(0)) v = v * T(0);  // the reference multiplies by 0 (NaN / -0 propagate)
+            if (zv[u][e] < T(0)) v = v * T(0);  // the reference multiplies by 0: an infinite or NaN value under the mask stays NaN
             if (g.relu) v = v > T(0) ? v : T(0);
             if (g.accumulate && in[e]) v += C[static_cast<int64_t>(m) * g.N + n];
             out[e] = v;

@@ -981,7 +981,7 @@ __device__ __forceinline__ void store_tile_dense(Engine &eng, T *__restrict__ C,
                 if constexpr (!LEAN) {
                     v += l_bn[e][j];
                     v += l_bm[e];
-                    if constexpr (EXT) v = l_z[e][j] < T(0) ? v * T(0) : v;  // grad * where(input < 0, 0, 1): a non-finite grad stays NaN, a negative one gives -0
+                    if constexpr (EXT) v = l_z[e][j] < T(0) ? v * T(0) : v;  // grad * where(input < 0, 0, 1): a product, so an infinite or NaN grad under the mask stays NaN
                     v = (v > T(0) || !relu) ? v : T(0);
                     v += l_p[e][j];
                     if constexpr (EXT) csum[slot + j] += off != kOob ? v : T(0);
