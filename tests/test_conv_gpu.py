@@ -91,6 +91,47 @@ def test_backward_exact_on_integer_data_and_adjoints(tt, oracle, dtype):
     assert lhs == np.sum(gx.to_numpy().astype(np.float64) * x) == np.sum(gw.to_numpy().astype(np.float64) * w)
 
 
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+@pytest.mark.parametrize("geom", [
+    # stride 2 on dense rows with output rows of whole 16-byte vectors: forward gathers two vectors per vector of
+    # positions instead of single elements; grad_input's classes store straight into grad_input.  B, C, O, H, W, k, P
+    (2, 8, 16, 16, 16, 3, 1),      # the top-left corner under padding (a vector that would start before the image)
+    (2, 4, 70, 17, 15, 3, 1),      # odd height and width: the last tap's column lies outside the row (W = 15 -> Wo = 8)
+    (1, 12, 8, 20, 24, 5, 2),      # 5 x 5 taps, two columns of padding
+    (2, 8, 8, 19, 24, 7, 3),       # 7 x 7 taps (a stem's geometry on more channels)
+    (1, 16, 40, 10, 16, 2, 0),     # even kernel, no padding
+    (3, 4, 4, 9, 8, 1, 0),         # 1 x 1 taps: every second element of every second row
+    (1, 64, 128, 56, 56, 3, 1),    # a layer's real size: several tiles per image, 18 k tiles
+])
+def test_stride_two_vector_gathers_exact(tt, oracle, dtype, geom):
+    Bn, Cc, O, H, W, k, P = geom
+    S = 2
+    rng = np.random.default_rng(sum(geom))
+    x = rng.integers(-3, 4, (Bn, Cc, H, W)).astype(dtype)
+    w = rng.integers(-3, 4, (O, Cc, k, k)).astype(dtype)
+    b = rng.integers(-3, 4, (O,)).astype(dtype)
+    out = tt.conv2d(dev(tt, x), dev(tt, w), dev(tt, b), S, P)
+    assert _last_kernel(0) == 0x102
+    want = oracle.conv2d_forward(x, w, b, S, P)
+    assert np.array_equal(out.to_numpy(), want)
+    g = rng.integers(-3, 4, want.shape).astype(dtype)
+    gx, gw, gb = tt.conv2d_backward(dev(tt, g), dev(tt, x), dev(tt, w), dev(tt, b), S, P)
+    wx, ww, wb = oracle.conv2d_backward(g, x, w, True, S, P)
+    assert np.array_equal(gw.to_numpy(), ww)
+    assert np.array_equal(gx.to_numpy(), wx) and np.array_equal(gb.to_numpy(), wb)
+    # the input as a window of a larger tensor whose other elements are NaN: nothing outside the window is summed
+    big = np.full((Bn, Cc + 1, H + 3, W + 4), np.nan, dtype)
+    big[:, 1:, 2:2 + H, 4:] = x                 # (a unit column stride and rows that end with the storage's rows)
+    tb = dev(tt, big)
+    es = big.strides
+    view = tt.Tensor(tb.storage, tb.dtype, (Bn, Cc, H, W), tuple(st // big.itemsize for st in es),
+                     (es[1] + 2 * es[2] + 4 * es[3]) // big.itemsize)
+    assert np.array_equal(tt.conv2d(view, dev(tt, w), dev(tt, b), S, P).to_numpy(), want)
+    assert _last_kernel(0) == 0x102
+    gx2, gw2, _ = tt.conv2d_backward(dev(tt, g), view, dev(tt, w), None, S, P)
+    assert np.array_equal(gw2.to_numpy(), ww) and np.array_equal(gx2.to_numpy(), wx)
+
+
 def _last_kernel(which):
     from tinytensor_amd import _capi
     return _capi.lib.ttamd_conv2d_last_kernel(which)

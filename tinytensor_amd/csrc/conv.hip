@@ -44,6 +44,10 @@ struct ConvGeom {
     // crosses a row although the width is no multiple of it; the columns past the row are computed and dropped.
     int row_pad;
     FastDiv d_row_pad;
+    // Not 0: this is one class of a strided grad_input (a unit-stride sub-problem over every sc_S-th row and column):
+    // position (i, j) of its H x W positions is element (sc_y0 + sc_S * i, sc_x0 + sc_S * j) of a plane of
+    // sc_H x sc_W elements, and the kernel writes it there instead of into a dense result of its own.
+    int sc_S, sc_y0, sc_x0, sc_H, sc_W;
 };
 
 // ---------------------------------------------------------------------------------------------
@@ -319,9 +323,29 @@ __device__ __forceinline__ typename Vec<T, VEC>::type clear_outside_row(typename
     return v;
 }
 
+// The VEC positions of a lane at stride STRIDE: source columns x0, x0 + STRIDE, ...  They lie inside STRIDE consecutive
+// vectors that start at x0 (gathered as they are, at any 4-byte alignment); this picks them out and clears the ones
+// outside the row.  STRIDE = 1 is clear_outside_row.
+template <typename T, int VEC, int STRIDE>
+__device__ __forceinline__ typename Vec<T, VEC>::type pick_strided(const typename Vec<T, VEC>::type *v, int x0, int src_w) {
+    if constexpr (STRIDE == 1) {
+        return clear_outside_row<T, VEC>(v[0], x0, src_w);
+    } else {
+        typename Vec<T, VEC>::type out;
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) {
+            const T e = v[(j * STRIDE) / VEC][(j * STRIDE) % VEC];
+            out[j] = static_cast<unsigned>(x0 + j * STRIDE) >= static_cast<unsigned>(src_w) ? T(0) : e;
+        }
+        return out;
+    }
+}
+
 // MC layout (positions contiguous in LDS), vectors along the positions: B operand of forward and of
 // grad_input.  Requires positions-per-row % VEC == 0 so that a vector never crosses a plane row.
-template <typename T, int ROWS, int BK, int VEC, bool FLIP, int PF = 1>
+// STRIDE (forward only): the convolution's stride.  Position (py, px) then reads source element
+// (STRIDE * py + dy, STRIDE * px + dx), and a lane's VEC positions come out of STRIDE gathered vectors (pick_strided).
+template <typename T, int ROWS, int BK, int VEC, bool FLIP, int PF = 1, int STRIDE = 1>
 struct TapStagerMC : TileLayout<T, ROWS, BK, false> {
     using L = TileLayout<T, ROWS, BK, false>;
     using V = typename Vec<T, VEC>::type;
@@ -329,8 +353,9 @@ struct TapStagerMC : TileLayout<T, ROWS, BK, false> {
     static constexpr int LPP = kThreads / VPL;   // k lines per pass
     static constexpr int P = BK / LPP;
     static_assert(VEC > 1 && ROWS % VEC == 0 && kThreads % VPL == 0 && BK % LPP == 0, "tile must split evenly");
+    static_assert(STRIDE == 1 || !FLIP, "the strided gather serves the forward product");
     static constexpr int kPF = PF;
-    V reg[PF][P];
+    V reg[PF][P][STRIDE];
     int col0[PF][P];  // first source column of each gathered vector
     __amdgpu_buffer_rsrc_t rsrc;
     TapView<FLIP> tv;
@@ -362,9 +387,11 @@ struct TapStagerMC : TileLayout<T, ROWS, BK, false> {
             int32_t ch_off;
             int dy, dx;
             tv.tap(static_cast<uint32_t>(k_ok ? kk : 0), ch_off, dy, dx);
-            const int y = py + dy, x0 = px0 + dx;
+            const int y = STRIDE * py + dy, x0 = STRIDE * px0 + dx;
             const bool row_ok = n_ok && k_ok && static_cast<unsigned>(y) < static_cast<unsigned>(tv.src_h);
-            reg[SLOT][p] = gather_row_vector<T, VEC>(rsrc, row_ok, ch_off + y * tv.s_h + x0);
+            const int32_t e0 = ch_off + y * tv.s_h + x0;
+#pragma unroll
+            for (int v = 0; v < STRIDE; ++v) reg[SLOT][p][v] = gather_row_vector<T, VEC>(rsrc, row_ok, e0 + v * VEC);
             col0[SLOT][p] = x0;
         }
         k_next += BK;
@@ -374,7 +401,7 @@ struct TapStagerMC : TileLayout<T, ROWS, BK, false> {
     __device__ __forceinline__ void store(T *lds) const {
 #pragma unroll
         for (int p = 0; p < P; ++p)
-            *reinterpret_cast<V *>(&lds[(p * LPP + line0) * L::LD + n_local]) = clear_outside_row<T, VEC>(reg[SLOT][p], col0[SLOT][p], tv.src_w);
+            *reinterpret_cast<V *>(&lds[(p * LPP + line0) * L::LD + n_local]) = pick_strided<T, VEC, STRIDE>(reg[SLOT][p], col0[SLOT][p], tv.src_w);
     }
 };
 
@@ -597,6 +624,29 @@ __device__ __forceinline__ void store_tile_padded_rows(Engine &eng, T *__restric
         });
 }
 
+// Store of one class of a strided grad_input (ConvGeom::sc_S): tile column n = i * row + j, the class's positions
+// numbered over rows of `row` columns (its own width or the padded one), goes to
+// C[m][(sc_y0 + sc_S * i) * sc_W + sc_x0 + sc_S * j] when i, j lie inside the class, C being [M, sc_H * sc_W].
+template <typename T, class Engine>
+__device__ __forceinline__ void store_tile_class_scatter(Engine &eng, T *__restrict__ C, int M_, const ConvGeom &geo, const FastDiv &d_row,
+                                                         int m0, int n0) {
+    constexpr uint32_t kSz = sizeof(T);
+    const int plane = geo.sc_H * geo.sc_W;
+    const int rows = M_ - m0 < Engine::kBM ? M_ - m0 : Engine::kBM;
+    const __amdgpu_buffer_rsrc_t out = make_rsrc(C + static_cast<int64_t>(m0) * plane, static_cast<int64_t>(rows) * plane * kSz);
+    const int h = geo.H, w = geo.W;
+    auto offset_of = [&](int ml, int nl) {
+        uint32_t i, j;
+        d_row.divmod(static_cast<uint32_t>(n0 + nl), i, j);
+        const bool inside = ml < rows && static_cast<int>(i) < h && static_cast<int>(j) < w;
+        const int e = (geo.sc_y0 + geo.sc_S * static_cast<int>(i)) * geo.sc_W + geo.sc_x0 + geo.sc_S * static_cast<int>(j);
+        return inside ? static_cast<uint32_t>(ml * plane + e) * kSz : kOob;
+    };
+    eng.template for_each<true, false>(
+        false, [&]<int PHASE>(int ml, int nl, T v, int, int) { buffer_store(out, offset_of(ml, nl), v); },
+        [&]<int PHASE>(int, int, T, T, int, int) {});
+}
+
 // forward: M = O, N = Ho*Wo, K = C*k*k, one GEMM per image.  StB gathers the image.
 template <typename T, int BM, int BN, int BK, int A_VEC, class StB>
 __global__ void __launch_bounds__(kThreads, 2)
@@ -650,17 +700,18 @@ struct DgradClasses {
     DgradClass cls[kMaxDgradStride * kMaxDgradStride];
 };
 
-// wtc[c][(o, pi, qi)] = w[o][c][ry + S pi][rx + S qi]
+// Class blockIdx.y of the table: wtc[c][(o, pi, qi)] = w[o][c][ry + S pi][rx + S qi], at the class's own offset in wt.
 template <typename T>
 __global__ void __launch_bounds__(256)
-weight_class_pack_kernel(ConvGeom geo, const T *__restrict__ w, T *__restrict__ wtc, DgradClass cl, int total) {
+weight_class_pack_kernel(ConvGeom geo, const T *__restrict__ w, T *__restrict__ wt, DgradClasses tab) {
+    const DgradClass &cl = tab.cls[blockIdx.y];
+    const int kpq = cl.kp * cl.kq, row = geo.O * kpq, total = geo.C * row;
     const int idx = blockIdx.x * blockDim.x + threadIdx.x;
     if (idx >= total) return;
-    const int kpq = cl.kp * cl.kq, row = geo.O * kpq;
     const int c = idx / row, rem = idx - c * row;
     const int o = rem / kpq, r = rem - o * kpq;
     const int pi = r / cl.kq, qi = r - pi * cl.kq;
-    wtc[idx] = w[static_cast<int64_t>(o) * geo.w_so + (c * geo.k + cl.ry + geo.S * pi) * geo.k + cl.rx + geo.S * qi];
+    wt[cl.wt_off + idx] = w[static_cast<int64_t>(o) * geo.w_so + (c * geo.k + cl.ry + geo.S * pi) * geo.k + cl.rx + geo.S * qi];
 }
 
 // gin[b][c][y][x] = the class result that owns (y, x), or 0 where no window reaches.
@@ -686,7 +737,9 @@ dgrad_interleave_kernel(ConvGeom geo, const T *__restrict__ tmp, T *__restrict__
 
 // grad_input: M = C, N = H*W, K = O*k*k, one GEMM per image.  wt is the transposed weight [C, O*k*k];
 // StB gathers grad_out.
-template <typename T, int BM, int BN, int BK, int A_VEC, class StB>
+// SCATTER: the problem is one class of a strided grad_input and its result goes straight to that class's elements of
+// grad_input (ConvGeom::sc_S, store_tile_class_scatter).
+template <typename T, int BM, int BN, int BK, int A_VEC, class StB, bool SCATTER = false>
 __global__ void __launch_bounds__(kThreads, 2)
 conv_dgrad_kernel(ConvGeom geo, const T *gout, const T *wt, T *gin, int tiles_m, int tiles_n) {
     using StA = Stager<T, BM, BK, true, A_VEC, kConvPF>;
@@ -706,7 +759,9 @@ conv_dgrad_kernel(ConvGeom geo, const T *gout, const T *wt, T *gin, int tiles_m,
     Engine eng;
     eng.init(tid);
     eng.run(sa, sb, smem, K, false);
-    if (geo.row_pad)
+    if constexpr (SCATTER)
+        store_tile_class_scatter<T>(eng, gin + static_cast<int64_t>(b) * M_ * geo.sc_H * geo.sc_W, M_, geo, geo.row_pad ? geo.d_row_pad : geo.d_W, m0, n0);
+    else if (geo.row_pad)
         store_tile_padded_rows<T>(eng, gin + static_cast<int64_t>(b) * M_ * N_, M_, geo.H, geo.W, geo.d_row_pad, m0, n0, static_cast<const T *>(nullptr));
     else
         store_tile_dense<T, true>(eng, gin + static_cast<int64_t>(b) * M_ * N_, M_, N_, m0, n0, static_cast<const T *>(nullptr), 0, 0, 0);
@@ -1124,6 +1179,15 @@ inline bool patch_kernel_enabled() {
     return on;
 }
 
+// TTAMD_CONV_STRIDED_VEC=0 keeps strided layers on the element-wise gathers (for comparisons).
+inline bool strided_vector_gather_enabled() {
+    static const bool on = [] {
+        const char *e = std::getenv("TTAMD_CONV_STRIDED_VEC");
+        return !(e && e[0] == '0');
+    }();
+    return on;
+}
+
 template <typename T>
 struct ConvTiles {
     static constexpr int BK = sizeof(T) == 4 ? 32 : 16;
@@ -1186,6 +1250,12 @@ ttamd_status forward_mfma_tile(const ConvPlan &pl, const void *bias, void *out, 
     using VecB = TapStagerMC<T, BN, BK, VK, false, kConvPF>;
     using OneB = Im2colStager<T, BN, BK, kConvPF>;
     if (a_vec && b_vec) return go(conv_fwd_kernel<T, BM, BN, BK, VK, VecB>, conv_lds_bytes<T, BM, BN, VK, VecB>());
+    // stride 2 on dense rows with output rows of whole vectors: two 16-byte gathers per vector of positions
+    if (a_vec && g.S == 2 && g.xs_w == 1 && g.Wo % VK == 0 && strided_vector_gather_enabled()) {
+        using Vec2B = TapStagerMC<T, BN, BK, VK, false, kConvPF, 2>;
+        t_last_kernel[0] = 0x102;
+        return go(conv_fwd_kernel<T, BM, BN, BK, VK, Vec2B>, conv_lds_bytes<T, BM, BN, VK, Vec2B>());
+    }
     if constexpr (sizeof(T) == 4) {  // rows of 2n elements: 8-byte gathers
         using PairB = TapStagerMC<T, BN, BK, 2, false, kConvPF>;
         if (a_vec && g.S == 1 && g.xs_w == 1 && g.Wo % 2 == 0)
@@ -1476,7 +1546,7 @@ ttamd_status backward_mfma(const ConvPlan &pl, const void *gout, void *gin, void
         // [C, O*kh*kw], dense result dst [B, C, gg.H*gg.W].
         auto dgrad_gemm = [&](const ConvGeom &gg, const T *wts, T *dst) -> ttamd_status {
           const int Kd = gg.O * gg.kh * gg.kw;
-          auto run = [&]<int BM, int BN>() -> ttamd_status {
+          auto run = [&]<int BM, int BN, bool SC>() -> ttamd_status {
             ConvGeom g = gg;
             const T *wt = wts;
             T *gin = dst;
@@ -1495,29 +1565,38 @@ ttamd_status backward_mfma(const ConvPlan &pl, const void *gout, void *gin, void
             };
             using VecB = TapStagerMC<T, BN, BK, VK, true, kConvPF>;
             using OneB = DgradStager<T, BN, BK, kConvPF>;
-            if (a_vec && b_vec) return go(conv_dgrad_kernel<T, BM, BN, BK, VK, VecB>, conv_lds_bytes<T, BM, BN, VK, VecB>());
+            if (a_vec && b_vec) return go(conv_dgrad_kernel<T, BM, BN, BK, VK, VecB, SC>, conv_lds_bytes<T, BM, BN, VK, VecB>());
             if constexpr (sizeof(T) == 4) {
                 using PairB = TapStagerMC<T, BN, BK, 2, true, kConvPF>;
                 if (a_vec && g.S == 1 && g.W % 2 == 0)
-                    return go(conv_dgrad_kernel<T, BM, BN, BK, VK, PairB>, conv_lds_bytes<T, BM, BN, VK, PairB>());
+                    return go(conv_dgrad_kernel<T, BM, BN, BK, VK, PairB, SC>, conv_lds_bytes<T, BM, BN, VK, PairB>());
             }
-            if (a_vec) return go(conv_dgrad_kernel<T, BM, BN, BK, VK, OneB>, conv_lds_bytes<T, BM, BN, VK, OneB>());
-            if (b_vec) return go(conv_dgrad_kernel<T, BM, BN, BK, 1, VecB>, conv_lds_bytes<T, BM, BN, 1, VecB>());
-            return go(conv_dgrad_kernel<T, BM, BN, BK, 1, OneB>, conv_lds_bytes<T, BM, BN, 1, OneB>());
+            if (a_vec) return go(conv_dgrad_kernel<T, BM, BN, BK, VK, OneB, SC>, conv_lds_bytes<T, BM, BN, VK, OneB>());
+            if (b_vec) return go(conv_dgrad_kernel<T, BM, BN, BK, 1, VecB, SC>, conv_lds_bytes<T, BM, BN, 1, VecB>());
+            return go(conv_dgrad_kernel<T, BM, BN, BK, 1, OneB, SC>, conv_lds_bytes<T, BM, BN, 1, OneB>());
           };
-          return gg.C <= 32 ? run.template operator()<32, 128>() : run.template operator()<64, 64>();
+          if (gg.sc_S) return gg.C <= 32 ? run.template operator()<32, 128, true>() : run.template operator()<64, 64, true>();
+          return gg.C <= 32 ? run.template operator()<32, 128, false>() : run.template operator()<64, 64, false>();
         };
         t_last_kernel[1] = 0x100;
         const DgradClassPlan dc = plan_dgrad_classes(sizeof(T), g.B, g.C, g.H, g.W, g.O, g.k, g.S, g.P);
         if (dc.use) {
             T *const tmp = reinterpret_cast<T *>(static_cast<char *>(ws) + plan.class_tmp_offset);
+            // Every class's weights in one launch (an empty class has no elements).  When every class has taps, every
+            // element of grad_input belongs to a class that writes it and the classes store straight into grad_input;
+            // otherwise (k < S) they go to dense buffers and dgrad_interleave_kernel adds the zeros.
+            int most = 0;
+            bool every_class_has_taps = true;
+            for (int ci = 0; ci < g.S * g.S; ++ci) {
+                const DgradClass &cl = dc.tab.cls[ci];
+                most = std::max(most, g.C * g.O * cl.kp * cl.kq);
+                if (cl.kp == 0 || cl.kq == 0) every_class_has_taps = false;
+            }
+            weight_class_pack_kernel<T><<<dim3((most + 255) / 256, g.S * g.S), dim3(256), 0, st>>>(g, static_cast<const T *>(pl.w), wt, dc.tab);
+            TTAMD_HIP_CHECK(hipGetLastError());
             for (int ci = 0; ci < g.S * g.S; ++ci) {
                 const DgradClass &cl = dc.tab.cls[ci];
                 if (cl.kp == 0 || cl.kq == 0 || cl.Hc == 0 || cl.Wc == 0) continue;
-                const int total = g.C * g.O * cl.kp * cl.kq;
-                weight_class_pack_kernel<T><<<dim3((total + 255) / 256), dim3(256), 0, st>>>(g, static_cast<const T *>(pl.w),
-                                                                                             wt + cl.wt_off, cl, total);
-                TTAMD_HIP_CHECK(hipGetLastError());
                 ConvGeom gc = g;  // the class as a unit-stride problem over its own positions
                 gc.H = cl.Hc;
                 gc.W = cl.Wc;
@@ -1530,16 +1609,25 @@ ttamd_status backward_mfma(const ConvPlan &pl, const void *gout, void *gin, void
                 gc.d_k = make_fastdiv(static_cast<uint32_t>(cl.kq));
                 gc.d_W = make_fastdiv(static_cast<uint32_t>(cl.Wc));
                 gc.d_S = make_fastdiv(1u);
-                if (ttamd_status rc = dgrad_gemm(gc, wt + cl.wt_off, tmp + cl.tmp_off)) return rc;
+                if (every_class_has_taps) {
+                    gc.sc_S = g.S;
+                    gc.sc_y0 = cl.y0;
+                    gc.sc_x0 = cl.x0;
+                    gc.sc_H = g.H;
+                    gc.sc_W = g.W;
+                }
+                if (ttamd_status rc = dgrad_gemm(gc, wt + cl.wt_off, every_class_has_taps ? static_cast<T *>(gin) : tmp + cl.tmp_off)) return rc;
             }
-            const int64_t total = static_cast<int64_t>(g.B) * g.C * g.H * g.W;
-            const int64_t blocks = (total + 255) / 256;
-            if (blocks > 0x7fffffff) {
-                set_error("conv2d_backward: too many workgroups");
-                return TTAMD_ERR_INVALID_ARGUMENT;
+            if (!every_class_has_taps) {
+                const int64_t total = static_cast<int64_t>(g.B) * g.C * g.H * g.W;
+                const int64_t blocks = (total + 255) / 256;
+                if (blocks > 0x7fffffff) {
+                    set_error("conv2d_backward: too many workgroups");
+                    return TTAMD_ERR_INVALID_ARGUMENT;
+                }
+                dgrad_interleave_kernel<T><<<dim3(static_cast<unsigned>(blocks)), dim3(256), 0, st>>>(g, tmp, static_cast<T *>(gin), dc.tab, total);
+                TTAMD_HIP_CHECK(hipGetLastError());
             }
-            dgrad_interleave_kernel<T><<<dim3(static_cast<unsigned>(blocks)), dim3(256), 0, st>>>(g, tmp, static_cast<T *>(gin), dc.tab, total);
-            TTAMD_HIP_CHECK(hipGetLastError());
         } else {
             bool handled = false;
             if constexpr (std::is_same_v<T, float>) {
