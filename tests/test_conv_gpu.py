@@ -102,6 +102,8 @@ def test_backward_exact_on_integer_data_and_adjoints(tt, oracle, dtype):
     (1, 16, 40, 10, 16, 2, 0),     # even kernel, no padding
     (3, 4, 4, 9, 8, 1, 0),         # 1 x 1 taps: every second element of every second row
     (1, 64, 128, 56, 56, 3, 1),    # a layer's real size: several tiles per image, 18 k tiles
+    (2, 16, 24, 28, 28, 3, 1),     # output rows of 14: numbered over rows padded to 16 (f32), the padding columns dropped
+    (1, 8, 8, 11, 13, 3, 1),       # output rows of 7, padded to 8
 ])
 def test_stride_two_vector_gathers_exact(tt, oracle, dtype, geom):
     Bn, Cc, O, H, W, k, P = geom

@@ -1235,7 +1235,8 @@ ttamd_status forward_mfma_tile(const ConvPlan &pl, const void *bias, void *out, 
     constexpr int BK = ConvTiles<T>::BK, VK = Mfma<T>::VK;
     ConvGeom g = pl.geo;
     const bool a_vec = rows_vectorizable<T>(pl.w, g.w_so, 0);
-    if (a_vec && g.S == 1 && g.xs_w == 1) {
+    const bool stride_two = g.S == 2 && strided_vector_gather_enabled();
+    if (a_vec && (g.S == 1 || stride_two) && g.xs_w == 1) {
         g.row_pad = padded_row_width(sizeof(T), g.Wo);
         g.d_row_pad = make_fastdiv(static_cast<uint32_t>(g.row_pad ? g.row_pad : 1));
     }
@@ -1251,7 +1252,7 @@ ttamd_status forward_mfma_tile(const ConvPlan &pl, const void *bias, void *out, 
     using OneB = Im2colStager<T, BN, BK, kConvPF>;
     if (a_vec && b_vec) return go(conv_fwd_kernel<T, BM, BN, BK, VK, VecB>, conv_lds_bytes<T, BM, BN, VK, VecB>());
     // stride 2 on dense rows with output rows of whole vectors: two 16-byte gathers per vector of positions
-    if (a_vec && g.S == 2 && g.xs_w == 1 && g.Wo % VK == 0 && strided_vector_gather_enabled()) {
+    if (a_vec && stride_two && g.xs_w == 1 && (g.row_pad || g.Wo % VK == 0)) {
         using Vec2B = TapStagerMC<T, BN, BK, VK, false, kConvPF, 2>;
         t_last_kernel[0] = 0x102;
         return go(conv_fwd_kernel<T, BM, BN, BK, VK, Vec2B>, conv_lds_bytes<T, BM, BN, VK, Vec2B>());
