@@ -559,3 +559,5 @@ def test_config3_4096_properties(tt, oracle, dtype):
     # (3) transposition identity through the strided path: (B^T.A^T)^T == A.B within tolerance
     Ct = tt.matmul(tB.permute(1, 0), tA.permute(1, 0)).to_numpy().T
     assert max_rel_error(Ct, Cg) <= tol_of(dtype)
+    # (4) every element of the product against the oracle's whole 4096^3 product (a few seconds of one host core)
+    check_close(Cg, oracle.matmul(A, B), A, B, dtype)

@@ -767,6 +767,46 @@ conv_dgrad_kernel(ConvGeom geo, const T *gout, const T *wt, T *gin, int tiles_m,
         store_tile_dense<T, true>(eng, gin + static_cast<int64_t>(b) * M_ * N_, M_, N_, m0, n0, static_cast<const T *>(nullptr), 0, 0, 0);
 }
 
+// Every class of a strided grad_input in one launch: the classes are short products (a quarter of the taps each at stride
+// 2, a reduction of O to 4 O), and launched one after the other each fills and drains the chip by itself.  Workgroups
+// [first_block[i], first_block[i + 1]) run class i as conv_dgrad_kernel<..., SCATTER = true> would.
+constexpr int kMaxDgradClasses = kMaxDgradStride * kMaxDgradStride;
+struct DgradClassGeoms {
+    ConvGeom geo[kMaxDgradClasses];
+    int64_t wt_off[kMaxDgradClasses];  // element offset of the class's packed weight
+    int first_block[kMaxDgradClasses + 1];
+    int tiles_m[kMaxDgradClasses], tiles_n[kMaxDgradClasses];
+    int n;
+};
+static_assert(sizeof(DgradClassGeoms) <= 3584, "kernel arguments are limited to 4 KiB");
+
+template <typename T, int BM, int BN, int BK, int A_VEC, class StB>
+__global__ void __launch_bounds__(kThreads, 2)
+conv_dgrad_classes_kernel(DgradClassGeoms tab, const T *gout, const T *wt, T *gin) {
+    using StA = Stager<T, BM, BK, true, A_VEC, kConvPF>;
+    using Engine = ConvEngine<T, BM, BN, BK, StA, StB>;
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
+    T *const smem = reinterpret_cast<T *>(smem_raw);
+    const int tid = threadIdx.x;
+    int ci = 0;
+    while (ci + 1 < tab.n && static_cast<int>(blockIdx.x) >= tab.first_block[ci + 1]) ++ci;  // (uniform, at most 8 steps)
+    const ConvGeom &geo = tab.geo[ci];
+    const int first = tab.first_block[ci], count = tab.first_block[ci + 1] - first;
+    int b, tm, tn;
+    decode_tile(remap_xcd(static_cast<int>(blockIdx.x) - first, count), tab.tiles_m[ci], tab.tiles_n[ci], b, tm, tn);
+    const int m0 = tm * BM, n0 = tn * BN;
+    const int M_ = geo.C, K = geo.O * geo.kh * geo.kw;
+    const int64_t g_image = static_cast<int64_t>(geo.O) * geo.Ho * geo.Wo;
+    StA sa;
+    StB sb(geo);
+    sa.init(wt + tab.wt_off[ci] + static_cast<int64_t>(m0) * K, tid, M_ - m0, K, 1, K);
+    sb.init(gout + static_cast<int64_t>(b) * g_image, g_image * static_cast<int64_t>(sizeof(T)), tid, n0);
+    Engine eng;
+    eng.init(tid);
+    eng.run(sa, sb, smem, K, false);
+    store_tile_class_scatter<T>(eng, gin + static_cast<int64_t>(b) * M_ * geo.sc_H * geo.sc_W, M_, geo, geo.row_pad ? geo.d_row_pad : geo.d_W, m0, n0);
+}
+
 // grad_weight: M = O, N = C*k*k, K = Ho*Wo per image.  Workgroup column `part` = (image group, k slice)
 // accumulates slice [k0, k0 + k_chunk) of images [grp*group, min(B, (grp+1)*group)) in registers and writes one
 // partial tile; k_chunk is a multiple of BK.
@@ -1188,6 +1228,15 @@ inline bool strided_vector_gather_enabled() {
     return on;
 }
 
+// TTAMD_CONV_MERGED_CLASSES=0 launches the classes of a strided grad_input one after the other (for comparisons).
+inline bool merged_dgrad_classes_enabled() {
+    static const bool on = [] {
+        const char *e = std::getenv("TTAMD_CONV_MERGED_CLASSES");
+        return !(e && e[0] == '0');
+    }();
+    return on;
+}
+
 template <typename T>
 struct ConvTiles {
     static constexpr int BK = sizeof(T) == 4 ? 32 : 16;
@@ -1595,9 +1644,7 @@ ttamd_status backward_mfma(const ConvPlan &pl, const void *gout, void *gin, void
             }
             weight_class_pack_kernel<T><<<dim3((most + 255) / 256, g.S * g.S), dim3(256), 0, st>>>(g, static_cast<const T *>(pl.w), wt, dc.tab);
             TTAMD_HIP_CHECK(hipGetLastError());
-            for (int ci = 0; ci < g.S * g.S; ++ci) {
-                const DgradClass &cl = dc.tab.cls[ci];
-                if (cl.kp == 0 || cl.kq == 0 || cl.Hc == 0 || cl.Wc == 0) continue;
+            auto class_geometry = [&](const DgradClass &cl) {
                 ConvGeom gc = g;  // the class as a unit-stride problem over its own positions
                 gc.H = cl.Hc;
                 gc.W = cl.Wc;
@@ -1617,6 +1664,56 @@ ttamd_status backward_mfma(const ConvPlan &pl, const void *gout, void *gin, void
                     gc.sc_H = g.H;
                     gc.sc_W = g.W;
                 }
+                return gc;
+            };
+            // One launch for all classes when each of them takes the 16-byte gathers on both operands (the usual case:
+            // class rows of whole vectors, or padded to them); otherwise a launch per class.
+            bool merged = false;
+            if (every_class_has_taps && merged_dgrad_classes_enabled()) {
+                DgradClassGeoms tab{};
+                const int BM = g.C <= 32 ? 32 : 64, BN = g.C <= 32 ? 128 : 64;
+                int64_t blocks = 0;
+                bool ok = true;
+                for (int ci = 0; ci < g.S * g.S && ok; ++ci) {
+                    const DgradClass &cl = dc.tab.cls[ci];
+                    if (cl.Hc == 0 || cl.Wc == 0) continue;
+                    ConvGeom gc = class_geometry(cl);
+                    const int Kd = gc.O * gc.kh * gc.kw;
+                    gc.row_pad = padded_row_width(sizeof(T), gc.W);
+                    gc.d_row_pad = make_fastdiv(static_cast<uint32_t>(gc.row_pad ? gc.row_pad : 1));
+                    ok = rows_vectorizable<T>(wt + cl.wt_off, Kd, 0) && (gc.row_pad || gc.W % VK == 0);
+                    const int N_ = gc.H * (gc.row_pad ? gc.row_pad : gc.W);
+                    const int i = tab.n++;
+                    tab.geo[i] = gc;
+                    tab.wt_off[i] = cl.wt_off;
+                    tab.tiles_m[i] = (gc.C + BM - 1) / BM;
+                    tab.tiles_n[i] = (N_ + BN - 1) / BN;
+                    tab.first_block[i] = static_cast<int>(blocks);
+                    blocks += static_cast<int64_t>(tab.tiles_m[i]) * tab.tiles_n[i] * g.B;
+                    ok = ok && blocks < 0x7fffffff;
+                    tab.first_block[i + 1] = static_cast<int>(blocks);
+                }
+                if (ok && tab.n > 0) {
+                    auto go = [&](auto kernel, size_t lds) {
+                        return launch_conv(kernel, lds, blocks, st, tab, static_cast<const T *>(gout), static_cast<const T *>(wt), static_cast<T *>(gin));
+                    };
+                    ttamd_status rc;
+                    if (g.C <= 32) {
+                        using VecB = TapStagerMC<T, 128, BK, VK, true, kConvPF>;
+                        rc = go(conv_dgrad_classes_kernel<T, 32, 128, BK, VK, VecB>, conv_lds_bytes<T, 32, 128, VK, VecB>());
+                    } else {
+                        using VecB = TapStagerMC<T, 64, BK, VK, true, kConvPF>;
+                        rc = go(conv_dgrad_classes_kernel<T, 64, 64, BK, VK, VecB>, conv_lds_bytes<T, 64, 64, VK, VecB>());
+                    }
+                    if (rc) return rc;
+                    merged = true;
+                    t_last_kernel[1] = 0x101;
+                }
+            }
+            for (int ci = 0; ci < g.S * g.S && !merged; ++ci) {
+                const DgradClass &cl = dc.tab.cls[ci];
+                if (cl.kp == 0 || cl.kq == 0 || cl.Hc == 0 || cl.Wc == 0) continue;
+                const ConvGeom gc = class_geometry(cl);
                 if (ttamd_status rc = dgrad_gemm(gc, wt + cl.wt_off, every_class_has_taps ? static_cast<T *>(gin) : tmp + cl.tmp_off)) return rc;
             }
             if (!every_class_has_taps) {
