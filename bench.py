@@ -379,8 +379,11 @@ def main():
                     help="only run N training steps of benchmark configuration 5 (batch 1024, 784-1024-1024-10, mse_loss) from the fused "
                          "forms (a short target for profilers), print the wall-clock time per step and exit")
     ap.add_argument("--mlp-ops", action="store_true", help="with --mlp-loop: the step op by op (unfused) instead")
-    ap.add_argument("--conv-shape", metavar="B,C,O,H,W", default="64,32,64,28,28",
-                    help="geometry for --conv-loop (3x3 kernel, stride 1, padding 1); the default is benchmark configuration 4")
+    ap.add_argument("--conv-shape", metavar="B,C,O,H,W[,k,S,P]", default="64,32,64,28,28",
+                    help="geometry for --conv-loop (kernel 3, stride 1, padding 1 unless given); the default is benchmark "
+                         "configuration 4")
+    ap.add_argument("--conv-time", action="store_true",
+                    help="with --conv-loop: also time forward and backward by HIP events (min of three bursts of N passes)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
@@ -399,17 +402,26 @@ def main():
     if args.conv_loop:
         be = tt.get_backend(tt.kAMD)
         rng = np.random.default_rng(0)
-        cb, cc, co, ch, cw = (int(v) for v in args.conv_shape.split(","))
+        dims = [int(v) for v in args.conv_shape.split(",")]
+        cb, cc, co, ch, cw = dims[:5]
+        ck, cs, cp = (dims[5:] + [3, 1, 1][len(dims) - 5:]) if len(dims) > 5 else (3, 1, 1)
         x = tt.Tensor.from_numpy(rng.normal(0, 0.1, (cb, cc, ch, cw)).astype(np.float32))
-        w = tt.Tensor.from_numpy(rng.normal(0, 0.1, (co, cc, 3, 3)).astype(np.float32))
-        out = be.conv2d(x, w, None, 1, 1)
+        w = tt.Tensor.from_numpy(rng.normal(0, 0.1, (co, cc, ck, ck)).astype(np.float32))
+        out = be.conv2d(x, w, None, cs, cp)
         go = tt.Tensor.from_numpy(np.ones(out.shape, np.float32))
-        bufs = be.conv2d_backward(go, x, w, None, 1, 1, return_buffers=True)
+        bufs = be.conv2d_backward(go, x, w, None, cs, cp, return_buffers=True)
         for _ in range(args.conv_loop):
-            be.conv2d(x, w, None, 1, 1, out=out)
-            be.conv2d_backward(go, x, w, None, 1, 1, buffers=bufs)
+            be.conv2d(x, w, None, cs, cp, out=out)
+            be.conv2d_backward(go, x, w, None, cs, cp, buffers=bufs)
         be.synchronize(0)
-        print(json.dumps({"conv_loop": args.conv_loop, "config": f"input [{cb},{cc},{ch},{cw}], weight [{co},{cc},3,3], s1 p1, f32"}))
+        line = {"conv_loop": args.conv_loop, "config": f"input [{cb},{cc},{ch},{cw}], weight [{co},{cc},{ck},{ck}], s{cs} p{cp}, f32"}
+        if args.conv_time:
+            fwd_ms = min(time_launches(tt, lambda: be.conv2d(x, w, None, cs, cp, out=out), args.conv_loop, 3) for _ in range(3))
+            bwd_ms = min(time_launches(tt, lambda: be.conv2d_backward(go, x, w, None, cs, cp, buffers=bufs), args.conv_loop, 3) for _ in range(3))
+            flop = 2.0 * cb * co * out.shape[2] * out.shape[3] * cc * ck * ck
+            line.update({"forward_us": round(fwd_ms * 1e3, 2), "forward_tflops": round(flop / fwd_ms / 1e9, 1),
+                         "backward_us": round(bwd_ms * 1e3, 2), "backward_tflops": round(2 * flop / bwd_ms / 1e9, 1)})
+        print(json.dumps(line))
         return
 
     if args.mlp_loop:
