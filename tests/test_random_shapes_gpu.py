@@ -117,3 +117,39 @@ def test_random_convs(tt, oracle, seed):
         assert np.array_equal(gx.to_numpy(), wx), tag
         assert np.array_equal(gw.to_numpy(), ww), tag
         assert np.array_equal(gb.to_numpy(), wb), tag
+
+
+@pytest.mark.parametrize("seed", range(4))
+def test_random_stride_two_convs(tt, oracle, seed):
+    """Stride-2 layers around the conditions of the vector gathers and of grad_input's one-launch classes: channel
+    counts that are (mostly) multiples of 4, output rows of every length (whole vectors, padded rows, neither), kernels 1
+    to 7 with every padding below them, odd and even extents, the input as a window of a NaN-filled tensor."""
+    rng = np.random.default_rng(4000 + seed)
+    for case in range(16):
+        dtype = [np.float32, np.float64][int(rng.integers(0, 2))]
+        Bn, O = int(rng.integers(1, 4)), int(rng.integers(1, 80))
+        Cc = 4 * int(rng.integers(1, 12)) if rng.integers(0, 5) else int(rng.integers(1, 40))
+        k = int(rng.integers(1, 8))
+        P = int(rng.integers(0, k))
+        H, W = int(rng.integers(max(1, k - 2 * P), 40)), int(rng.integers(max(1, k - 2 * P), 40))
+        x = rng.integers(-3, 4, (Bn, Cc, H, W)).astype(dtype)
+        w = rng.integers(-3, 4, (O, Cc, k, k)).astype(dtype)
+        tag = f"seed {seed} case {case}: B{Bn} C{Cc} O{O} {H}x{W} k{k} s2 p{P} {np.dtype(dtype).name}"
+        if rng.integers(0, 2):      # a window of a larger tensor (unit column stride), NaN around it
+            big = np.full((Bn, Cc + 1, H + 2, W + 3), np.nan, dtype)
+            big[:, 1:, 1:1 + H, 3:] = x
+            tb = tt.Tensor.from_numpy(big)
+            es = [s // big.itemsize for s in big.strides]
+            tx = tt.Tensor(tb.storage, tb.dtype, (Bn, Cc, H, W), tuple(es), es[1] + es[2] + 3 * es[3])
+        else:
+            tx = tt.Tensor.from_numpy(x)
+        tw = tt.Tensor.from_numpy(w)
+        out = tt.conv2d(tx, tw, None, 2, P).to_numpy()
+        want = oracle.conv2d_forward(x, w, None, 2, P)
+        assert np.array_equal(out, want), tag
+        g = rng.integers(-3, 4, want.shape).astype(dtype)
+        gx, gw, gb = tt.conv2d_backward(tt.Tensor.from_numpy(g), tx, tw, None, 2, P)
+        wx, ww, _ = oracle.conv2d_backward(g, x, w, False, 2, P)
+        assert gb is None
+        assert np.array_equal(gx.to_numpy(), wx), tag
+        assert np.array_equal(gw.to_numpy(), ww), tag
