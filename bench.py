@@ -379,6 +379,8 @@ def main():
                     help="only run N training steps of benchmark configuration 5 (batch 1024, 784-1024-1024-10, mse_loss) from the fused "
                          "forms (a short target for profilers), print the wall-clock time per step and exit")
     ap.add_argument("--mlp-ops", action="store_true", help="with --mlp-loop: the step op by op (unfused) instead")
+    ap.add_argument("--mlp-separate-head", action="store_true",
+                    help="with --mlp-loop: the last layer, the loss and their backward as four launches instead of the two of linear_mse_head")
     ap.add_argument("--conv-shape", metavar="B,C,O,H,W[,k,S,P]", default="64,32,64,28,28",
                     help="geometry for --conv-loop (kernel 3, stride 1, padding 1 unless given); the default is benchmark "
                          "configuration 4")
@@ -435,10 +437,14 @@ def main():
                                         for a, b in ((784, 1024), (1024, 1024), (1024, 10))]
 
         def fused_step():
-            z1, a1 = tt.linear_relu(xs, P1, c1); z2, a2 = tt.linear_relu(a1, P2, c2); y = tt.linear(a2, P3, c3)
-            loss, gy, db3 = tt.mse_loss(y, ts, grad=True, bias_grad=True)
+            z1, a1 = tt.linear_relu(xs, P1, c1); z2, a2 = tt.linear_relu(a1, P2, c2)
+            if args.mlp_separate_head:
+                y = tt.linear(a2, P3, c3)
+                loss, gy, db3 = tt.mse_loss(y, ts, grad=True, bias_grad=True)
+                dz2, dW3, _ = tt.linear_backward(gy, a2, P3, relu_input=z2, bias_grad=False)
+            else:  # the 10-class layer, the loss and their backward: two launches
+                y, loss, dz2, dW3, db3 = tt.linear_mse_head(a2, P3, c3, ts, relu_input=z2)
             # (bias gradients of layers 1 and 2 from the vectors of dz that the weight-gradient products stage)
-            dz2, dW3, _ = tt.linear_backward(gy, a2, P3, relu_input=z2, bias_grad=False)
             dz1, dW2, db2 = tt.linear_backward(dz2, a1, P2, relu_input=z1, bias_grad="own")
             dX, dW1, db1 = tt.linear_backward(dz1, xs, P1, bias_grad="own")
             return [loss, dW1, db1, dW2, db2, dW3, db3, dX]

@@ -289,6 +289,25 @@ ttamd_status ttamd_mse_loss(int device, ttamd_dtype dtype, int64_t rows, int64_t
                             const void *target, void *loss_out, void *grad_input_out, void *grad_colsum_out,
                             void *stream);
 
+/* The last Linear layer of a network together with the loss it feeds, forward and backward, for layers of at most 64
+ * outputs (the 10 classes of the reference's MLP): what nn::Linear::forward (nn/linear.cpp:42-50), nn::mse_loss with
+ * mean reduction (nn/loss.cpp:69-72) and their autograd nodes (autograd/reduce_ops.cpp:195-205,
+ * binary_ops.cpp:153-159,173-179, unary_ops.cpp:568-573) compute op by op:
+ *   output [rows, out]          = input [rows, in] . weight [in, out] + bias [out] (bias may be NULL)
+ *   loss_out [1]                = mean((output - target)^2)
+ *   grad_output_out [rows, out] = (1 / numel) * 2 * (output - target)
+ *   grad_input_out [rows, in]   = (grad_output . weight^T) * where(relu_input < 0, 0, 1)  (relu_input [rows, in], the
+ *                                 saved input of the ReLU that produced `input`, or NULL: no mask)
+ *   grad_weight_out [in, out]   = input^T . grad_output;   grad_bias_out [out] (or NULL) = grad_output summed over rows.
+ * All operands dense row-major, f32 / f64.  With f32, at most 16 outputs, in_features a multiple of 4 and 16-byte
+ * aligned input / relu_input / grad_input_out these are two launches (every step but the sums over the rows is local
+ * to a block of 16 rows); otherwise the call runs ttamd_batched_matmul and ttamd_mse_loss one after the other, with
+ * the same results up to the order of the sums (all orders fixed: deterministic either way). */
+ttamd_status ttamd_linear_mse_head(int device, ttamd_dtype dtype, int64_t rows, int64_t in_features, int64_t out_features,
+                                   const void *input, const void *weight, const void *bias, const void *target,
+                                   const void *relu_input, void *output, void *loss_out, void *grad_output_out,
+                                   void *grad_input_out, void *grad_weight_out, void *grad_bias_out, void *stream);
+
 /* BackendBase::uniform_real_ / normal_ (backend_base.h:96-103) for a dense float tensor with scalar parameters, as
  * nn::Linear's default initialisation calls them (nn/init.cpp:30-52,106-112).  dist 0 = uniform_real(low = p0,
  * high = p1), 1 = normal(mu = p0, std = p1).  *master_state is the caller's Generator state (tensor/random.cpp:46-63);

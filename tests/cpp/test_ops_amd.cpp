@@ -350,9 +350,16 @@ MlpGrads mlp_step(const Tensor &x, const Tensor &t, const nn::Linear &l1, const 
 }
 // The same step from the fused forms: Linear + ReLU in one launch, the loss with its gradient and the head's bias
 // gradient in one, and per layer one GEMM for dx (ReLU mask and bias gradient in its store) and one for dW.
-MlpGrads mlp_step_fused(const Tensor &x, const Tensor &t, const nn::Linear &l1, const nn::Linear &l2, const nn::Linear &l3, bool own_bias = false) {
+MlpGrads mlp_step_fused(const Tensor &x, const Tensor &t, const nn::Linear &l1, const nn::Linear &l2, const nn::Linear &l3, bool own_bias = false,
+                        bool head = false) {
     const auto [z1, a1] = l1.forward_relu(x);
     const auto [z2, a2] = l2.forward_relu(a1);
+    if (head) {  // the last layer, the loss and their backward in one call; the other two layers as with own_bias
+        const nn::HeadResult h = nn::linear_mse_head(a2, l3.weight, &*l3.bias, t, &z2);
+        const nn::LinearGrads g2 = nn::linear_backward(h.dx, a1, l2.weight, &z1, nn::BiasGrad::kOwn);
+        const nn::LinearGrads g1 = nn::linear_backward(g2.dx, x, l1.weight, nullptr, nn::BiasGrad::kOwn);
+        return MlpGrads{h.loss, g1.dW, *g1.db, g2.dW, *g2.db, h.dW, *h.db, g1.dx};
+    }
     const Tensor y = l3.forward(a2);
     const nn::MseLoss loss = nn::mse_loss(y, t, true);
     MlpGrads g;
@@ -462,6 +469,24 @@ TEST_CASE("MLP training step") {
     const double ms_own = std::chrono::duration<double, std::milli>(std::chrono::steady_clock::now() - t2).count() / iters;
     std::printf("  the same with the bias gradients from the weight-gradient products (10 launches): %.3f ms per step\n", ms_own);
     CHECK(ms_own < 50.0);
+    // ... and with the last layer, the loss and their backward in one call (8 launches)
+    const MlpGrads hd = mlp_step_fused(X, T, b1, b2, b3, true, true);
+    CHECK(close(hd.loss, ref.loss));
+    CHECK(close(hd.db1, ref.db1));
+    CHECK(close(hd.db2, ref.db2));
+    CHECK(close(hd.db3, ref.db3));
+    CHECK(close(hd.dW1, ref.dW1));
+    CHECK(close(hd.dW2, ref.dW2));
+    CHECK(close(hd.dW3, ref.dW3));
+    CHECK(close(hd.dX, ref.dX));
+    for (int i = 0; i < 5; ++i) (void)mlp_step_fused(X, T, b1, b2, b3, true, true);
+    check(ttamd_device_synchronize(0));
+    const auto t3 = std::chrono::steady_clock::now();
+    for (int i = 0; i < iters; ++i) (void)mlp_step_fused(X, T, b1, b2, b3, true, true);
+    check(ttamd_device_synchronize(0));
+    const double ms_head = std::chrono::duration<double, std::milli>(std::chrono::steady_clock::now() - t3).count() / iters;
+    std::printf("  the same with the last layer and the loss in one call (8 launches): %.3f ms per step\n", ms_head);
+    CHECK(ms_head < 50.0);
 }
 
 int main(int argc, char **argv) { return mini::run_all(argc, argv); }

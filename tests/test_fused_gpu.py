@@ -139,10 +139,16 @@ def fused_mlp_step(tt, x, t, params, own=False):
     """The training step of benchmark configuration 5 from the fused forms: 3 forward launches, the loss with its
     gradient and the head's bias gradient in one, and per layer one GEMM for dx (the ReLU-backward mask in its store) and
     one for dW.  The bias gradients of layers 1 and 2 are column sums of dz: taken in the store of the GEMM that writes
-    dz (+ the sum of the partial rows), or (`own`) from the vectors of dz that the layer's dW GEMM stages."""
+    dz (+ the sum of the partial rows), or (`own`) from the vectors of dz that the layer's dW GEMM stages.  own == "head":
+    as `own`, and the last layer, the loss and their backward in one call of two launches."""
     (W1, b1), (W2, b2), (W3, b3) = params
     z1, a1 = tt.linear_relu(x, W1, b1)
     z2, a2 = tt.linear_relu(a1, W2, b2)
+    if own == "head":
+        y, loss, dz2, dW3, db3 = tt.linear_mse_head(a2, W3, b3, t, relu_input=z2)
+        dz1, dW2, db2 = tt.linear_backward(dz2, a1, W2, relu_input=z1, bias_grad="own")
+        dX, dW1, db1 = tt.linear_backward(dz1, x, W1, bias_grad="own")
+        return dict(y=y, loss=loss, dW1=dW1, db1=db1, dW2=dW2, db2=db2, dW3=dW3, db3=db3, dX=dX, z1=z1, z2=z2)
     y = tt.linear(a2, W3, b3)
     loss, gy, db3 = tt.mse_loss(y, t, grad=True, bias_grad=True)
     if own:
@@ -228,7 +234,104 @@ def test_right_operand_column_sums_need_a_dense_operand(tt):
         be.batched_matmul(ai, ai, rhs_colsum_out=tt.Tensor.from_numpy(np.zeros((1, 64), np.int32)))
 
 
-@pytest.mark.parametrize("own", [False, True])
+def _head_reference(x, w, b, t, z):
+    """The head's results from numpy, in float64 where a sum is involved."""
+    dtype = x.dtype.type
+    y = (x.astype(np.float64) @ w.astype(np.float64) + (0 if b is None else b)).astype(dtype)
+    d = y - t
+    dy = (dtype(1) / dtype(y.size) * dtype(2)) * d
+    dx = dy.astype(np.float64) @ w.astype(np.float64).T
+    if z is not None:
+        dx = dx * np.where(z < 0, 0.0, 1.0)
+    return dict(y=y, loss=np.mean(d.astype(np.float64) ** 2), dy=dy, dx=dx, dW=x.astype(np.float64).T @ dy.astype(np.float64),
+                db=dy.astype(np.float64).sum(0))
+
+
+# (rows, in_features, out_features): configuration 5's head; ragged rows, columns and k tiles; more row blocks than groups
+# (several blocks to a workgroup); k parts of more than one tile per wave; the widest k one part takes and one beyond;
+# out_features 16 and 1; shapes the two-launch form leaves to the separate calls (17 outputs, k not a multiple of 4, k < 16)
+HEAD_SHAPES = [(1024, 1024, 10), (4096, 1024, 16), (2048, 512, 8), (64, 256, 32), (1000, 260, 7), (5000, 64, 16), (33, 2048, 3), (2100, 516, 10), (16, 16, 1), (1, 20, 5),
+               (700, 4096, 10), (300, 8196, 2), (1500, 1028, 13), (64, 256, 17), (130, 70, 10), (50, 12, 4), (257, 1000, 64)]
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+@pytest.mark.parametrize("with_bias,with_mask", [(True, True), (False, False)])
+@pytest.mark.parametrize("shape", HEAD_SHAPES)
+def test_linear_mse_head_exact_on_integers(tt, dtype, with_bias, with_mask, shape):
+    """Integer-valued operands and a power-of-two element count: every product and sum is exact in any order, so each
+    output must equal numpy's bit for bit, whichever kernels the call runs."""
+    R, K, N = shape
+    rng = np.random.default_rng(R * 31 + K + N)
+    x = rng.integers(-2, 3, (R, K)).astype(dtype)
+    w = rng.integers(-2, 3, (K, N)).astype(dtype)
+    b = rng.integers(-3, 4, (N,)).astype(dtype) if with_bias else None
+    t = rng.integers(-4, 5, (R, N)).astype(dtype)
+    z = rng.integers(-2, 3, (R, K)).astype(dtype) if with_mask else None
+    d = lambda v: tt.Tensor.from_numpy(v) if v is not None else None
+    y, loss, dx, dW, db = tt.linear_mse_head(d(x), d(w), d(b), d(t), d(z))
+    want = _head_reference(x, w, b, t, z)
+    assert np.array_equal(y.to_numpy(), want["y"])
+    numel = R * N
+    tol = 2e-5 if dtype == np.float32 else 1e-12
+    assert abs(float(loss.to_numpy()[0]) - want["loss"]) <= tol * want["loss"]
+    if numel & (numel - 1) == 0:   # 1 / numel is a power of two: the gradients are exact as well
+        assert np.array_equal(dx.to_numpy(), want["dx"].astype(dtype))
+        assert np.array_equal(dW.to_numpy(), want["dW"].astype(dtype))
+        if with_bias:
+            assert np.array_equal(db.to_numpy(), want["db"].astype(dtype))
+    else:
+        for got, key in ((dx, "dx"), (dW, "dW")) + (((db, "db"),) if with_bias else ()):
+            scale = np.abs(want[key]).max() + 1e-30
+            assert np.max(np.abs(got.to_numpy() - want[key])) <= tol * scale, key
+    assert (db is None) == (not with_bias)
+
+
+@pytest.mark.parametrize("shape", [(1024, 1024, 10), (1000, 260, 7), (2100, 516, 10), (700, 4096, 10)])
+def test_linear_mse_head_matches_the_separate_calls(tt, shape):
+    """Real-valued data: the one call against Linear, mse_loss and linear_backward one after the other.  y, and with it dy, come
+    from the same order of sums in both (bit-equal); dx, dW, db and the loss add in other orders."""
+    R, K, N = shape
+    rng = np.random.default_rng(R + K + N)
+    x = np.maximum(rng.normal(0, 1, (R, K)), 0).astype(np.float32)
+    z = rng.normal(0, 1, (R, K)).astype(np.float32)
+    w = rng.uniform(-0.05, 0.05, (K, N)).astype(np.float32)
+    b = rng.uniform(-0.05, 0.05, (N,)).astype(np.float32)
+    t = rng.uniform(0, 1, (R, N)).astype(np.float32)
+    d = tt.Tensor.from_numpy
+    tx, tw, tb_, tt_, tz = d(x), d(w), d(b), d(t), d(z)
+    y, loss, dx, dW, db = tt.linear_mse_head(tx, tw, tb_, tt_, tz)
+    y2 = tt.linear(tx, tw, tb_)
+    loss2, gy2, db2 = tt.mse_loss(y2, tt_, grad=True, bias_grad=True)
+    dx2, dW2, _ = tt.linear_backward(gy2, tx, tw, relu_input=tz, bias_grad=False)
+    assert np.array_equal(y.to_numpy(), y2.to_numpy())
+    assert abs(float(loss.to_numpy()[0]) - float(loss2.to_numpy()[0])) <= 1e-5 * float(loss2.to_numpy()[0])
+    want = _head_reference(x, w, b, t, z)
+    for got, sep, key in ((dx, dx2, "dx"), (dW, dW2, "dW"), (db, db2, "db")):
+        scale = np.abs(want[key]).max()
+        err, err_sep = (np.max(np.abs(v.to_numpy().reshape(want[key].shape) - want[key])) / scale for v in (got, sep))
+        assert err <= 2e-6, (key, err, err_sep)
+    # the masked elements are zeros, the others are not touched by the mask
+    assert np.all(dx.to_numpy()[z < 0] == 0)
+
+
+def test_linear_mse_head_keeps_nan_under_the_mask_and_checks_arguments(tt):
+    x = np.ones((32, 64), np.float32)
+    w = np.ones((64, 4), np.float32)
+    t = np.zeros((32, 4), np.float32)
+    t[:, 2] = np.inf                       # column 2 of dy = scale * (y - inf) is -inf, and with it every element of dy . W^T
+    z = -np.ones((32, 64), np.float32)
+    d = tt.Tensor.from_numpy
+    _, _, dx, _, _ = tt.linear_mse_head(d(x), d(w), None, d(t), d(z))
+    assert np.all(np.isnan(dx.to_numpy()))  # -inf times the mask's 0 is NaN, as in the reference's product
+    with pytest.raises(tt.TTException):
+        tt.linear_mse_head(d(x), d(w), None, d(np.zeros((32, 5), np.float32)), None)
+    with pytest.raises(tt.TTException):
+        tt.linear_mse_head(d(x), d(np.ones((64, 65), np.float32)), None, d(np.zeros((32, 65), np.float32)), None)
+    with pytest.raises(tt.TTException):
+        tt.linear_mse_head(d(x), d(w.astype(np.float64)), None, d(t), None)
+
+
+@pytest.mark.parametrize("own", [False, True, "head"])
 def test_fused_mlp_training_step_matches_the_oracle_and_fits_15_launches(tt, oracle, own):
     X = oracle.Generator(0).uniform_real(0.0, 1.0, (1024, 784))
     T = oracle.Generator(1).uniform_real(0.0, 1.0, (1024, 10))
@@ -253,7 +356,7 @@ def test_fused_mlp_training_step_matches_the_oracle_and_fits_15_launches(tt, ora
     graph = None
     try:
         graph = tt.graph.Graph(stream, lambda: list(fused_mlp_step(tt, x, t, params, own).values()))
-        assert graph.num_nodes() <= (10 if own else 15), graph.num_nodes()
+        assert graph.num_nodes() <= {False: 15, True: 10, "head": 8}[own], graph.num_nodes()
         graph.launch()
         stream.synchronize()
         for k, v in zip(("y", "loss", "dW1", "db1", "dW2", "db2", "dW3", "db3", "dX"), graph.outputs):

@@ -6,7 +6,7 @@ tests and the benchmark: same names, argument meaning and error behaviour as the
 """
 from .tensor import (  # noqa: F401
     BackendAMD, Conv2d, Device, Generator, Linear, Tensor, TTException, calc_fan_in_out, default_generator, kaiming_uniform_,
-    set_default_generator_seed, broadcast_tensors, linear_backward, linear_init, linear_relu, mse_loss, normal, uniform_real, conv2d, conv2d_backward, full, get_backend, kAMD, linear,
+    set_default_generator_seed, broadcast_tensors, linear_backward, linear_init, linear_relu, linear_mse_head, mse_loss, normal, uniform_real, conv2d, conv2d_backward, full, get_backend, kAMD, linear,
     matmul, matmul_backward, where, max_pool2d, min_pool2d, avg_pool2d, pool2d_backward,
 )
 from . import _capi  # noqa: F401

@@ -64,6 +64,7 @@ def _bind(lib: C.CDLL) -> None:
         "ttamd_full": (i, [i, i, vp, C.c_int64, vp, vp]),
         "ttamd_random_fill": (i, [i, i, i, C.c_double, C.c_double, C.POINTER(C.c_uint64), C.c_int64, vp, vp]),
         "ttamd_mse_loss": (i, [i, i, C.c_int64, C.c_int64, vp, vp, vp, vp, vp, vp]),
+        "ttamd_linear_mse_head": (i, [i, i, C.c_int64, C.c_int64, C.c_int64, vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, vp]),
         "ttamd_random_fill_view": (i, [i, i, i, C.c_double, C.c_double, C.POINTER(C.c_uint64), i, C.POINTER(C.c_int64),
                                        C.POINTER(C.c_int64), vp, C.c_int64, vp]),
         "ttamd_random_fill_states": (i, [i, i, i, C.c_double, C.c_double, C.POINTER(C.c_uint64), i, C.POINTER(C.c_int64),

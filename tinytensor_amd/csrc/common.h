@@ -114,6 +114,11 @@ ttamd_status launch_gemm_simt(ttamd_dtype dt, const GemmArgs &g, hipStream_t str
 // *handled says whether the product is one of them (nothing is launched otherwise).
 ttamd_status launch_gemm_thin(ttamd_dtype dt, const GemmArgs &g, int device, hipStream_t stream, const char **variant,
                               bool variant_only, bool *handled, bool fixed_scratch = false);
+// A Linear layer of at most 16 outputs with mse_loss, forward and backward, in two launches (gemm_thin.hip); f32.
+ttamd_status launch_linear_mse_head(int device, int64_t rows, int64_t in_features, int64_t out_features, const void *input,
+                                    const void *weight, const void *bias, const void *target, const void *relu_input, void *output,
+                                    void *loss_out, void *grad_output_out, void *grad_input_out, void *grad_weight_out,
+                                    void *grad_bias_out, hipStream_t stream, bool *handled);
 // The GEMM launchers' scratch (the stream's growing buffer, or the library's fixed array when `fixed`) and the kernel
 // that adds `rows` partial rows of column sums: out[b][n] = sum over r of partial[b][r][n], r ascending.
 ttamd_status gemm_scratch(int device, hipStream_t stream, size_t bytes, bool fixed, void **out);

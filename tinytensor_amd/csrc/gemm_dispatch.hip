@@ -172,6 +172,52 @@ ttamd_status ttamd_batched_matmul_noalloc(int device, ttamd_dtype dtype, int B, 
     return batched_matmul(device, dtype, B, N, K, M, lhs, rhs, out, epilogue, stream, true);
 }
 
+ttamd_status ttamd_linear_mse_head(int device, ttamd_dtype dtype, int64_t rows, int64_t in_features, int64_t out_features,
+                                   const void *input, const void *weight, const void *bias, const void *target,
+                                   const void *relu_input, void *output, void *loss_out, void *grad_output_out,
+                                   void *grad_input_out, void *grad_weight_out, void *grad_bias_out, void *stream) {
+    if (dtype != TTAMD_F32 && dtype != TTAMD_F64) {
+        set_error("linear_mse_head: floating point dtypes only");
+        return TTAMD_ERR_UNSUPPORTED_DTYPE;
+    }
+    if (rows < 1 || in_features < 1 || out_features < 1 || rows > 0x7fffffffLL || in_features > 0x7fffffffLL ||
+        out_features > 64 || rows * in_features > 0x7fffffffLL) {
+        set_error("linear_mse_head: rows %lld, in_features %lld, out_features %lld: each at least 1, at most 64 outputs, "
+                  "fewer than 2^31 input elements", static_cast<long long>(rows), static_cast<long long>(in_features),
+                  static_cast<long long>(out_features));
+        return TTAMD_ERR_INVALID_ARGUMENT;
+    }
+    if (!input || !weight || !target || !output || !loss_out || !grad_output_out || !grad_input_out || !grad_weight_out) {
+        set_error("linear_mse_head: NULL data pointer");
+        return TTAMD_ERR_INVALID_ARGUMENT;
+    }
+    if (ttamd_status s = use_device(device)) return s;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    if (dtype == TTAMD_F32) {
+        bool handled = false;
+        if (ttamd_status s = launch_linear_mse_head(device, rows, in_features, out_features, input, weight, bias, target, relu_input,
+                                                    output, loss_out, grad_output_out, grad_input_out, grad_weight_out,
+                                                    grad_bias_out, st, &handled))
+            return s;
+        if (handled) return TTAMD_OK;
+    }
+    // The same results from the separate calls: y = x . W + b, the loss with dy and db, dx = (dy . W^T) * mask, dW = x^T . dy.
+    const int R = static_cast<int>(rows), K = static_cast<int>(in_features), N = static_cast<int>(out_features);
+    const ttamd_view3 x{input, 0, {rows * in_features, in_features, 1}}, xt{input, 0, {rows * in_features, 1, in_features}};
+    const ttamd_view3 w{weight, 0, {in_features * out_features, out_features, 1}}, wt{weight, 0, {in_features * out_features, 1, out_features}};
+    const ttamd_view3 dy{grad_output_out, 0, {rows * out_features, out_features, 1}};
+    ttamd_epilogue fwd{};
+    fwd.bias = bias;
+    fwd.bias_mode = bias ? 1 : 0;
+    if (ttamd_status s = batched_matmul(device, dtype, 1, R, K, N, &x, &w, output, &fwd, stream, false)) return s;
+    if (ttamd_status s = ttamd_mse_loss(device, dtype, rows, out_features, output, target, loss_out, grad_output_out, grad_bias_out, stream))
+        return s;
+    ttamd_epilogue back{};
+    back.relu_grad_input = relu_input;
+    if (ttamd_status s = batched_matmul(device, dtype, 1, R, N, K, &dy, &wt, grad_input_out, &back, stream, false)) return s;
+    return batched_matmul(device, dtype, 1, K, R, N, &xt, &dy, grad_weight_out, nullptr, stream, false);
+}
+
 const char *ttamd_batched_matmul_variant(ttamd_dtype dtype, int B, int N, int K, int M, const ttamd_view3 *lhs,
                                          const ttamd_view3 *rhs) {
     GemmArgs g;

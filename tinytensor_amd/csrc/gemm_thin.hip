@@ -369,7 +369,347 @@ ttamd_status launch_thin_typed(const GemmArgs &g, hipStream_t stream, const char
     return TTAMD_OK;
 }
 
+// ---------------------------------------------------------------------------------------------------------------
+// The head of an MLP in two launches: y = x . W + b of a Linear layer with at most 16 outputs (nn/linear.cpp:42-50),
+// nn::mse_loss(y, t) with mean reduction (nn/loss.cpp:69-72) and the backward of both -- dy = (1 / numel) * 2 * (y - t)
+// (autograd/reduce_ops.cpp:201-205, binary_ops.cpp:153-159), dx = (dy . W^T) * where(relu_input < 0, 0, 1)
+// (binary_ops.cpp:173-179, unary_ops.cpp:568-573), dW = x^T . dy, db = dy summed over the rows.  As four separate
+// launches (the two kernels above, the short-reduction product of the general kernels and mse_loss) each step is a
+// launch and a memory round trip long, 5 - 6 us, for a few MFLOP.  Here the first kernel is gemm_thin_kernel with the
+// loss's element-wise steps in its store (y, dy, and per block of 16 rows the parts of the loss and of db), and the
+// second runs gemm_thin_k_kernel's strips of 16 columns of dx and, in workgroups of their own beside them, the same
+// strips of dW (each a sum over all the rows; beyond 1024 rows in stretches that a third small kernel adds up), and
+// one workgroup that adds up the first kernel's parts of db and of the loss.  All sums in fixed orders.
+struct HeadArgs {
+    const float *x, *w, *bias, *t, *z;  // x [R,K], w [K,N], bias [N] or null, t [R,N], z [R,K] or null; all dense
+    float *y, *dy, *dx, *dw, *db, *loss;  // y, dy [R,N], dx [R,K], dw [K,N], db [N] or null, loss [1]
+    float *part_b, *part_l;             // [row blocks][16], [row blocks]
+    // dy once more for the second kernel's 16-byte loads, per block of 16 rows and zero beyond R and N:
+    // dy_rows[block][r][j] and dy_cols[block][j][r]
+    float *dy_rows, *dy_cols;
+    float *part_w;  // [stretches of 1024 rows][strips of 16 k][16 x 16]: the stretches' tiles of dW (more than one stretch)
+    int R, K, N;
+    float inv_n;  // 1 / (R * N)
+};
+
+// y = x . W + b for a block of 16 rows (gemm_thin_kernel<float, true>), then d = y - t, dy = ((1 / numel) * 2) * d, and the
+// block's sums of d * d / numel and of dy's columns.
+__global__ void __launch_bounds__(64 * kThinWaves) linear_mse_head_forward_kernel(HeadArgs a) {
+    using MI = ThinMma<float>;
+    using acc_t = MI::acc_t;
+    __shared__ float red[kThinWaves][256];
+    __shared__ float dyt[16][17];
+    __shared__ float lterm[256];
+    const int tid = threadIdx.x, wave = tid / 64, lane = tid % 64;
+    const int li = lane % 16, q = lane / 16;
+    const int m0 = blockIdx.x * 16;
+    const int row = m0 + li < a.R ? m0 + li : a.R - 1;
+    const int col = li < a.N ? li : a.N - 1;
+    const bool col_ok = li < a.N;
+    const float *__restrict__ A = a.x + static_cast<int64_t>(row) * a.K;
+    const float *__restrict__ B = a.w + col;
+    acc_t acc0 = {}, acc1 = {};
+    for (int kb = wave * 64; kb < a.K; kb += kThinWaves * 64) {
+        float av[4][4], bv[4][4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {  // every load of the chunk goes out before the first is used
+            const int k = kb + (j * 4 + q) * 4;
+            const bool ok = k < a.K;
+            const int kc = ok ? k : 0;
+            const thin_f32x4 v = *reinterpret_cast<const thin_f32x4 *>(A + kc);
+#pragma unroll
+            for (int s = 0; s < 4; ++s) av[j][s] = ok ? v[s] : 0.f;
+#pragma unroll
+            for (int s = 0; s < 4; ++s) {
+                const float b = B[static_cast<int64_t>(kc + s) * a.N];
+                bv[j][s] = ok && col_ok ? b : 0.f;
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+#pragma unroll
+            for (int s = 0; s < 4; ++s) {
+                if ((j * 4 + s) & 1) acc1 = MI::mma(av[j][s], bv[j][s], acc1);
+                else acc0 = MI::mma(av[j][s], bv[j][s], acc0);
+            }
+        }
+    }
+#pragma unroll
+    for (int e = 0; e < 4; ++e) red[wave][e * 64 + lane] = acc0[e] + acc1[e];
+    __syncthreads();
+    if (tid < 256) {
+        float v = 0.f;
+#pragma unroll
+        for (int w = 0; w < kThinWaves; ++w) v += red[w][tid];  // wave order: deterministic (and gemm_thin_kernel's order)
+        const int e = tid / 64, l = tid % 64;
+        const int ml = MI::acc_row(e, l), n = l % 16, m = m0 + ml;
+        float g = 0.f, term = 0.f;
+        if (m < a.R && n < a.N) {
+            const int64_t idx = static_cast<int64_t>(m) * a.N + n;
+            if (a.bias) v += a.bias[n];
+            const float d = v - a.t[idx];
+            g = (a.inv_n * 2.0f) * d;
+            term = d * d * a.inv_n;
+            a.y[idx] = v;
+            a.dy[idx] = g;
+        }
+        dyt[ml][n] = g;
+        lterm[tid] = term;
+    }
+    __syncthreads();
+    if (tid < 256) {
+        const int64_t o = static_cast<int64_t>(blockIdx.x) * 256 + tid;
+        a.dy_rows[o] = dyt[tid / 16][tid % 16];
+        a.dy_cols[o] = dyt[tid % 16][tid / 16];
+    }
+    if (wave == 0) {
+        float s = (lterm[lane] + lterm[lane + 64]) + (lterm[lane + 128] + lterm[lane + 192]);
+#pragma unroll
+        for (int d = 32; d > 0; d >>= 1) s += __shfl_down(s, d, 64);
+        if (lane == 0) a.part_l[blockIdx.x] = s;
+    } else if (wave == 1 && lane < 16) {
+        float s = 0.f;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) s += dyt[r][lane];
+        a.part_b[blockIdx.x * 16 + lane] = s;
+    }
+}
+
+constexpr int kHeadTiles = 4;  // 16-row tiles per wave of the second kernel
+
+// db's columns and the loss from the first kernel's parts, by one workgroup of 256: column c (16 = the loss) is summed by
+// 15 lanes, lane p over the blocks p, p + 15, ... in ascending order, and their sums are added in the order of p: a fixed
+// order.  The parts pass through LDS, 240 blocks at a time, so that their loads are in flight together.
+__device__ __forceinline__ void head_sums(const HeadArgs &a, int row_blocks) {
+    constexpr int kChunk = 240, kLanes = 15;  // 17 * 15 = 255 threads at work
+    __shared__ float buf[kChunk * 17];
+    __shared__ float part[17 * kLanes];
+    const int tid = threadIdx.x, c = tid / kLanes, p = tid % kLanes;
+    float acc = 0.f;
+    for (int b0 = 0; b0 < row_blocks; b0 += kChunk) {
+        const int nb = row_blocks - b0 < kChunk ? row_blocks - b0 : kChunk;
+        for (int e = tid; e < nb * 17; e += 64 * 4) {
+            const int b = b0 + e / 17, col = e % 17;
+            buf[e] = col < 16 ? a.part_b[b * 16 + col] : a.part_l[b];
+        }
+        __syncthreads();
+        if (c < 17)
+            for (int b = p; b < nb; b += kLanes) acc += buf[b * 17 + c];
+        __syncthreads();
+    }
+    if (c < 17) part[c * kLanes + p] = acc;
+    __syncthreads();
+    if (tid < 17) {
+        float s = 0.f;
+#pragma unroll
+        for (int i = 0; i < kLanes; ++i) s += part[tid * kLanes + i];
+        if (tid == 16) a.loss[0] = s;
+        else if (a.db && tid < a.N) a.db[tid] = s;
+    }
+}
+
+// The second kernel: workgroups of four waves in two roles, told apart by blockIdx.y.  Both products as transposed
+// tiles, and with the reduced index of a step's slice q numbered 4 q + s (s the step), so that a lane's four values of
+// dy are one 16-byte load.
+//   blockIdx.y >= stretches: columns k0 .. k0 + 15 of dx = (dy . W^T) * mask for a chunk of 256 rows, four 16-row tiles per
+//     wave.  dx^T = W . dy^T: first operand W[k0 + li][j], second dy[r = li][j], j = 4 q + s: the lane holds
+//     dx[m0 + li][k0 + 4 q + e], four consecutive columns -- the mask's 16-byte load, the result's 16-byte store.
+//   blockIdx.y < stretches: rows k0 .. k0 + 15 of dW = x^T . dy over a stretch of 1024 rows, sixteen tiles per wave.
+//     dW^T = dy^T . x: first operand dy[r][j = li], second x[r][k0 + li], r = 4 q + s: the lane holds
+//     dW[k0 + li][4 q + e]; the four waves' tiles are added through LDS in wave order.  With one stretch that is dW's
+//     tile; with more, part_w[stretch][strip] receives it and the finishing kernel adds the stretches in order.
+// One workgroup beside the strips' adds up the first kernel's parts of db and of the loss.
+constexpr int kHeadWaves = 4;
+constexpr int kHeadChunkRows = kHeadWaves * kHeadTiles * 16;  // 256
+constexpr int kHeadStretchRows = 4 * kHeadChunkRows;           // 1024
+__global__ void __launch_bounds__(64 * kHeadWaves) linear_mse_head_backward_kernel(HeadArgs a, int row_blocks, int chunks, int stretches) {
+    using MI = ThinMma<float>;
+    using acc_t = MI::acc_t;
+    const int tid = threadIdx.x, wave = tid / 64, lane = tid % 64;
+    const int li = lane % 16, q = lane / 16;
+    const int strips = gridDim.x - 1;
+    if (static_cast<int>(blockIdx.x) == strips) {  // (uniform: no barrier is left waiting)
+        if (blockIdx.y == 0) head_sums(a, row_blocks);
+        return;
+    }
+    const int k0 = blockIdx.x * 16;
+    const bool k_ok = k0 + li < a.K;  // this lane's row of W / column of x
+    const int kr = k_ok ? k0 + li : 0;
+    // Neighbouring strips start at different row tiles (tile u of this wave: u * 4 + wave, rotated by the strip's number):
+    // rows are a multiple of the memory channels' interleave apart when K is a power of two, and strips that walked the
+    // rows in step would all queue at the same channels.
+    const int rot = blockIdx.x % (kHeadWaves * kHeadTiles);
+    if (static_cast<int>(blockIdx.y) >= stretches) {  // (the longer-running role is launched first)
+        const bool kv_ok = k0 + 4 * q < a.K;  // this lane's four columns of dx (K is a multiple of 4: in range together)
+        const int kz = kv_ok ? k0 + 4 * q : 0;
+        const int base = (blockIdx.y - stretches) * kHeadChunkRows;
+        float wf[4];
+        thin_f32x4 dyb[kHeadTiles], zv[kHeadTiles];
+#pragma unroll
+        for (int s = 0; s < 4; ++s) {  // every load of the wave goes out before the first is used
+            const int j = 4 * q + s;
+            wf[s] = a.w[static_cast<int64_t>(kr) * a.N + (j < a.N ? j : 0)];
+        }
+#pragma unroll
+        for (int u = 0; u < kHeadTiles; ++u) {
+            const int m0 = base + ((u * kHeadWaves + wave + rot) % (kHeadWaves * kHeadTiles)) * 16;
+            const int blk = m0 / 16 < row_blocks ? m0 / 16 : row_blocks - 1;
+            const int rl = m0 + li < a.R ? m0 + li : a.R - 1;
+            dyb[u] = *reinterpret_cast<const thin_f32x4 *>(a.dy_rows + static_cast<int64_t>(blk) * 256 + li * 16 + 4 * q);
+            zv[u] = a.z ? *reinterpret_cast<const thin_f32x4 *>(a.z + static_cast<int64_t>(rl) * a.K + kz) : thin_f32x4{0.f, 0.f, 0.f, 0.f};
+        }
+#pragma unroll
+        for (int s = 0; s < 4; ++s) {
+            keep(wf[s]);
+            wf[s] = k_ok && 4 * q + s < a.N ? wf[s] : 0.f;  // (dy's copies are zero beyond R and N: no stand-in value meets a zero)
+        }
+#pragma unroll
+        for (int u = 0; u < kHeadTiles; ++u) {
+            keep(dyb[u]);
+            keep(zv[u]);
+        }
+#pragma unroll
+        for (int u = 0; u < kHeadTiles; ++u) {
+            const int m0 = base + ((u * kHeadWaves + wave + rot) % (kHeadWaves * kHeadTiles)) * 16;
+            if (m0 >= a.R) continue;  // wave-uniform (every lane of the wave takes part in an MFMA)
+            acc_t dxa = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int s = 0; s < 4; ++s) dxa = MI::mma(wf[s], dyb[u][s], dxa);
+            thin_f32x4 o;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) o[e] = zv[u][e] < 0.f ? dxa[e] * 0.f : dxa[e];  // a product, as the reference's mask is
+            if (m0 + li < a.R && kv_ok) *reinterpret_cast<thin_f32x4 *>(a.dx + static_cast<int64_t>(m0 + li) * a.K + k0 + 4 * q) = o;
+        }
+        return;
+    }
+    __shared__ float red[kHeadWaves][256];
+    const int stretch = blockIdx.y;
+    const int first = stretch * kHeadStretchRows;
+    const int end = first + kHeadStretchRows < a.R ? first + kHeadStretchRows : a.R;
+    constexpr int kTiles = kHeadTiles;  // per wave and pass (256 rows): their loads are in flight together
+    const int rot_w = blockIdx.x % (kHeadWaves * kTiles);
+    acc_t wacc0 = {0.f, 0.f, 0.f, 0.f}, wacc1 = {0.f, 0.f, 0.f, 0.f};
+    for (int base = first; base < end; base += kHeadWaves * kTiles * 16) {
+        thin_f32x4 dya[kTiles];
+        float xf[kTiles][4];
+#pragma unroll
+        for (int u = 0; u < kTiles; ++u) {
+            const int m0 = base + ((u * kHeadWaves + wave + rot_w) % (kHeadWaves * kTiles)) * 16;
+            const int blk = m0 / 16 < row_blocks ? m0 / 16 : row_blocks - 1;
+            dya[u] = *reinterpret_cast<const thin_f32x4 *>(a.dy_cols + static_cast<int64_t>(blk) * 256 + li * 16 + 4 * q);
+#pragma unroll
+            for (int s = 0; s < 4; ++s) {
+                const int r = m0 + 4 * q + s;
+                xf[u][s] = a.x[static_cast<int64_t>(r < a.R ? r : a.R - 1) * a.K + kr];
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < kTiles; ++u) {
+#pragma unroll
+            for (int s = 0; s < 4; ++s) keep(xf[u][s]);
+            keep(dya[u]);
+        }
+#pragma unroll
+        for (int u = 0; u < kTiles; ++u) {
+            const int m0 = base + ((u * kHeadWaves + wave + rot_w) % (kHeadWaves * kTiles)) * 16;
+#pragma unroll
+            for (int s = 0; s < 4; ++s) {
+                // beyond R the stand-in row of x is zeroed, and beyond K its stand-in column: dy's zeros there meet zeros
+                const float xv = m0 + 4 * q + s < a.R && k_ok ? xf[u][s] : 0.f;
+                const float dv = m0 < a.R ? dya[u][s] : 0.f;  // (a tile beyond R: the stand-in block's dy is not this tile's)
+                if (s & 1) wacc1 = MI::mma(dv, xv, wacc1);
+                else wacc0 = MI::mma(dv, xv, wacc0);
+            }
+        }
+    }
+#pragma unroll
+    for (int e = 0; e < 4; ++e) red[wave][e * 64 + lane] = wacc0[e] + wacc1[e];
+    __syncthreads();
+    // element tid of the tile: e = tid / 64, lane l = tid % 64: dW[k0 + l % 16][4 (l / 16) + e]
+    float v = 0.f;
+#pragma unroll
+    for (int w = 0; w < kHeadWaves; ++w) v += red[w][tid];  // wave order: deterministic
+    const int k = k0 + tid % 16, j = 4 * ((tid % 64) / 16) + tid / 64;
+    if (stretches > 1) a.part_w[(static_cast<int64_t>(stretch) * strips + blockIdx.x) * 256 + tid] = v;
+    else if (k < a.K && j < a.N) a.dw[static_cast<int64_t>(k) * a.N + j] = v;
+}
+
+// dW's 16 x 16 tiles from the stretches' tiles, added in the order of the stretches.
+__global__ void __launch_bounds__(256) linear_mse_head_finish_kernel(HeadArgs a, int strips, int stretches) {
+    const int tid = threadIdx.x;
+    const float *tiles = a.part_w + static_cast<int64_t>(blockIdx.x) * 256 + tid;
+    float sum = 0.f;
+    int c = 0;
+    for (; c + 8 <= stretches; c += 8) {  // eight loads in flight, added in order
+        float t[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) t[i] = tiles[static_cast<int64_t>(c + i) * strips * 256];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) sum += t[i];
+    }
+    for (; c < stretches; ++c) sum += tiles[static_cast<int64_t>(c) * strips * 256];
+    const int k = blockIdx.x * 16 + tid % 16, j = 4 * ((tid % 64) / 16) + tid / 64;
+    if (k < a.K && j < a.N) a.dw[static_cast<int64_t>(k) * a.N + j] = sum;
+}
+
+constexpr int64_t kHeadMaxRows = 16384;  // (16 stretches of 1024 rows)
+constexpr int64_t kHeadMaxElements = int64_t(1) << 26;  // of the input (the stretches' tiles of dW take a 64th of that); larger
+                                                        // layers fill the chip with the separate products
+
 }  // namespace
+
+// The launcher of the two kernels above; *handled = false (and nothing launched) when the operands rule them out.
+ttamd_status launch_linear_mse_head(int device, int64_t rows, int64_t in_features, int64_t out_features, const void *input,
+                                    const void *weight, const void *bias, const void *target, const void *relu_input, void *output,
+                                    void *loss_out, void *grad_output_out, void *grad_input_out, void *grad_weight_out,
+                                    void *grad_bias_out, hipStream_t stream, bool *handled) {
+    *handled = false;
+    auto aligned = [](const void *p) { return reinterpret_cast<uintptr_t>(p) % 16 == 0; };
+    if (rows < 1 || rows > kHeadMaxRows || in_features < 16 || in_features % 4 != 0 || in_features > (1 << 20) || out_features < 1 ||
+        out_features > 16 || rows * in_features > kHeadMaxElements)
+        return TTAMD_OK;
+    if (!aligned(input) || !aligned(relu_input) || !aligned(grad_input_out)) return TTAMD_OK;
+    HeadArgs a{};
+    a.x = static_cast<const float *>(input);
+    a.w = static_cast<const float *>(weight);
+    a.bias = static_cast<const float *>(bias);
+    a.t = static_cast<const float *>(target);
+    a.z = static_cast<const float *>(relu_input);
+    a.y = static_cast<float *>(output);
+    a.dy = static_cast<float *>(grad_output_out);
+    a.dx = static_cast<float *>(grad_input_out);
+    a.dw = static_cast<float *>(grad_weight_out);
+    a.db = static_cast<float *>(grad_bias_out);
+    a.loss = static_cast<float *>(loss_out);
+    a.R = static_cast<int>(rows);
+    a.K = static_cast<int>(in_features);
+    a.N = static_cast<int>(out_features);
+    a.inv_n = 1.0f / static_cast<float>(rows * out_features);
+    const int row_blocks = static_cast<int>((rows + 15) / 16);
+    const int strips = (a.K + 15) / 16, chunks = (a.R + kHeadChunkRows - 1) / kHeadChunkRows;
+    const int stretches = (a.R + kHeadStretchRows - 1) / kHeadStretchRows;
+    const size_t tile_floats = stretches > 1 ? static_cast<size_t>(stretches) * strips * 256 : 0;
+    void *ws = nullptr;
+    if (ttamd_status st = stream_scratch(device, stream, (static_cast<size_t>(row_blocks) * (512 + 17) + tile_floats) * sizeof(float), &ws))
+        return st;
+    a.dy_rows = static_cast<float *>(ws);
+    a.dy_cols = a.dy_rows + static_cast<size_t>(row_blocks) * 256;
+    a.part_w = a.dy_cols + static_cast<size_t>(row_blocks) * 256;
+    a.part_b = a.part_w + tile_floats;
+    a.part_l = a.part_b + static_cast<size_t>(row_blocks) * 16;
+    *handled = true;
+    linear_mse_head_forward_kernel<<<dim3(static_cast<unsigned>(row_blocks)), dim3(64 * kThinWaves), 0, stream>>>(a);
+    TTAMD_HIP_CHECK(hipGetLastError());
+    // (one column of workgroups more than strips: its first adds up db and the loss while the strips run)
+    linear_mse_head_backward_kernel<<<dim3(static_cast<unsigned>(strips + 1), static_cast<unsigned>(chunks + stretches)), dim3(64 * kHeadWaves), 0,
+                                      stream>>>(a, row_blocks, chunks, stretches);
+    TTAMD_HIP_CHECK(hipGetLastError());
+    if (stretches > 1) {
+        linear_mse_head_finish_kernel<<<dim3(static_cast<unsigned>(strips)), dim3(256), 0, stream>>>(a, strips, stretches);
+        TTAMD_HIP_CHECK(hipGetLastError());
+    }
+    return TTAMD_OK;
+}
 
 ttamd_status launch_gemm_thin(ttamd_dtype dt, const GemmArgs &g, int device, hipStream_t stream, const char **variant,
                               bool variant_only, bool *handled, bool fixed_scratch) {

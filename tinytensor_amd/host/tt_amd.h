@@ -851,6 +851,44 @@ inline auto mse_loss(const Tensor &input, const Tensor &target, bool bias_grad =
                          r.grad_input.data_ptr(), r.grad_colsum ? r.grad_colsum->data_ptr() : nullptr, nullptr));
     return r;
 }
+
+// A network's last Linear layer with the loss behind it, forward and backward in one call (ttamd_linear_mse_head):
+// y = nn::Linear::forward(input) (nn/linear.cpp:42-50), loss = nn::mse_loss(y, target) (nn/loss.cpp:69-72) and what
+// autograd makes of them: dx = (dy . W^T) * where(relu_input < 0, 0, 1) with dy = (1 / numel) * 2 * (y - target),
+// dW = x^T . dy, db = dy.sum(0) (autograd/reduce_ops.cpp:195-205, binary_ops.cpp:153-159,173-179, unary_ops.cpp:568-573).
+// 2-D operands of one float dtype, at most 64 outputs; two launches for f32 layers of at most 16 outputs.
+struct HeadResult {
+    Tensor output, loss, grad_output, dx, dW;
+    std::optional<Tensor> db;
+};
+inline auto linear_mse_head(const Tensor &input, const Tensor &weight, const Tensor *bias, const Tensor &target, const Tensor *relu_input = nullptr)
+    -> HeadResult {
+    if (input.dim() != 2 || weight.dim() != 2 || target.dim() != 2) throw TTException("linear_mse_head: input, weight and target must be 2-D");
+    const int64_t rows = input.size(0), fin = input.size(1), fout = weight.size(1);
+    if (weight.size(0) != fin) throw TTException("Invalid shape for matrix multiplication");
+    if (target.size(0) != rows || target.size(1) != fout || (relu_input && !(relu_input->shape() == input.shape())))
+        throw TTException("linear_mse_head: target must be [rows, out_features] and relu_input [rows, in_features]");
+    if (bias && bias->numel() != fout) throw TTException("linear_mse_head: bias must hold out_features elements");
+    const ScalarType dt = input.dtype();
+    if (weight.dtype() != dt || target.dtype() != dt || (bias && bias->dtype() != dt) || (relu_input && relu_input->dtype() != dt))
+        throw TTException("linear_mse_head: operands of one dtype");
+    const Tensor x = input.contiguous(), w = weight.contiguous(), t = target.contiguous();
+    std::optional<Tensor> b, z;
+    if (bias) b = bias->contiguous();
+    if (relu_input) z = relu_input->contiguous();
+    HeadResult r;
+    const Device dev = x.device();
+    r.output = Tensor::empty(Shape({rows, fout}), dt, dev);
+    r.loss = Tensor::empty(Shape({1}), dt, dev);
+    r.grad_output = Tensor::empty(Shape({rows, fout}), dt, dev);
+    r.dx = Tensor::empty(Shape({rows, fin}), dt, dev);
+    r.dW = Tensor::empty(Shape({fin, fout}), dt, dev);
+    if (bias) r.db = Tensor::empty(Shape({fout}), dt, dev);
+    check(ttamd_linear_mse_head(dev.id, static_cast<ttamd_dtype>(dt), rows, fin, fout, x.data_ptr(), w.data_ptr(), b ? b->data_ptr() : nullptr,
+                                t.data_ptr(), z ? z->data_ptr() : nullptr, r.output.data_ptr(), r.loss.data_ptr(), r.grad_output.data_ptr(),
+                                r.dx.data_ptr(), r.dW.data_ptr(), r.db ? r.db->data_ptr() : nullptr, nullptr));
+    return r;
+}
 }  // namespace nn
 
 }  // namespace tt_amd

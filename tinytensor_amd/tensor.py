@@ -889,6 +889,40 @@ def mse_loss(input: Tensor, target: Tensor, grad: bool = True, bias_grad: bool =
     return loss, g, cs
 
 
+def linear_mse_head(input: Tensor, weight: Tensor, bias: Tensor | None, target: Tensor, relu_input: Tensor | None = None):
+    """A network's last Linear layer with the loss behind it, forward and backward in one call:
+    y = nn::Linear::forward(input) (nn/linear.cpp:42-50), loss = nn::mse_loss(y, target) (nn/loss.cpp:69-72) and what
+    autograd makes of them -- dy = (1 / numel) * 2 * (y - target) (reduce_ops.cpp:195-205, binary_ops.cpp:153-159),
+    dx = (dy . W^T) * where(relu_input < 0, 0, 1), dW = x^T . dy (binary_ops.cpp:173-179, unary_ops.cpp:568-573),
+    db = dy.sum(0).  2-D operands of one float dtype, at most 64 outputs.
+    Returns (y, loss [1], dx, dW, db | None)."""
+    if input.dim() != 2 or weight.dim() != 2 or target.dim() != 2:
+        raise TTException("linear_mse_head: input, weight and target must be 2-D")
+    rows, fin = input.shape
+    fout = weight.size(1)
+    if weight.size(0) != fin:
+        raise TTException(f"Invalid shape for matrix multiplication. LHS={input.shape} and RHS={weight.shape}")
+    if tuple(target.shape) != (rows, fout) or (relu_input is not None and tuple(relu_input.shape) != (rows, fin)):
+        raise TTException("linear_mse_head: target must be [rows, out_features] and relu_input [rows, in_features]")
+    if bias is not None and bias.numel() != fout:
+        raise TTException("linear_mse_head: bias must hold out_features elements")
+    others = [t for t in (weight, bias, target, relu_input) if t is not None]
+    if any(t.dtype != input.dtype for t in others) or input.dtype not in (_capi.F32, _capi.F64):
+        raise TTException("linear_mse_head: operands of one floating point dtype")
+    if rows < 1 or fin < 1 or fout < 1 or fout > 64:
+        raise TTException("linear_mse_head: at least one row, input and output; at most 64 outputs")
+    input, weight, target = input.contiguous(), weight.contiguous(), target.contiguous()
+    bias = bias.contiguous() if bias is not None else None
+    relu_input = relu_input.contiguous() if relu_input is not None else None
+    new = lambda *shape: Tensor.empty(shape, input.dtype, input.device)
+    y, loss, dy, dx, dW = new(rows, fout), new(1), new(rows, fout), new(rows, fin), new(fin, fout)
+    db = new(fout) if bias is not None else None
+    ptr = lambda t: C.c_void_p(t.storage.ptr + t.offset * t.itemsize) if t is not None else None
+    _check(lib.ttamd_linear_mse_head(input.device.id, input.dtype, rows, fin, fout, ptr(input), ptr(weight), ptr(bias), ptr(target),
+                                     ptr(relu_input), ptr(y), ptr(loss), ptr(dy), ptr(dx), ptr(dW), ptr(db), _stream_arg()))
+    return y, loss, dx, dW, db
+
+
 def conv2d(input: Tensor, weight: Tensor, bias: Tensor | None = None, stride: int = 1, padding: int = 0) -> Tensor:
     """tinytensor::conv2d argument checks (tensor/tensor.cpp:3089-3167) then BackendBase::conv2d."""
     if input.dim() != 4 or weight.dim() != 4:
