@@ -154,6 +154,9 @@ struct ConvWgradPatchPlan {
     int n_units;          // B * SPI
     int workgroups;       // = partial tiles written
     int blocks_per_wave;
+    int sets;             // 0: four waves with every block of output channels; 2 or 4: sets of four waves that share out the
+                          // positions, one block of 32 output channels per workgroup (workgroups = partial tiles x O / 32)
+    int a_instr, x_instr; // sets: load instructions per grad_out row / per input channel of a stage
     size_t lds_bytes;
 };
 ConvWgradPatchPlan plan_conv_wgrad_patch(int B, int C, int H, int W, int O, int k, int S, int P);
@@ -166,8 +169,8 @@ struct ConvWgradPatchArgs {
     int32_t xs_c, xs_h;
     int64_t image_bytes;   // bytes reachable from an image's first element
     // derived
-    int RS, SPI, RSS, n_sub, n_units, R, pitch, plane, pitch_a, waves_per_ob, col_blocks, blocks_per_wave;
-    FastDiv d_cblocks, d_k, d_2P, d_P, d_R, d_C, d_spi, d_vw;
+    int RS, SPI, RSS, n_sub, n_units, R, pitch, plane, pitch_a, waves_per_ob, col_blocks, blocks_per_wave, a_instr, x_instr;
+    FastDiv d_cblocks, d_k, d_2P, d_P, d_R, d_C, d_spi, d_vw, d_Wo, d_kvecs;
 };
 ttamd_status launch_conv_wgrad_patch_f32(ConvWgradPatchArgs a, const ConvWgradPatchPlan &plan, hipStream_t stream, bool *handled);
 
