@@ -379,25 +379,37 @@ __global__ void __launch_bounds__(256 * KS, 1) conv_wgrad_patch_sets_kernel(Conv
             const int chunks = (np + 7) / 8;
             const int c_lo = set * chunks / KS, n = (set + 1) * chunks / KS - c_lo;
             const int last_off = (rows - 1) * pitch + Wo - 4;  // patch offset of the stage's last four positions
-            int pos = 8 * c_lo + 4 * kg;
-            const int row0 = static_cast<int>(a.d_Wo.div(static_cast<uint32_t>(pos)));
-            int x = pos - row0 * Wo, off = row0 * pitch + x;
+            // Position, column and patch offset of the chunk's two groups of four positions (kg = 0, 1): the same for
+            // all lanes of a group, so they are kept as wave-uniform values (scalar arithmetic) and a lane selects its
+            // group's offset.  Wo and the positions are multiples of 4: a group never straddles a row.
+            int pos_g[2], x_g[2], off_g[2];
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+                pos_g[h] = 8 * c_lo + 4 * h;
+                const int row0 = static_cast<int>(a.d_Wo.div(static_cast<uint32_t>(pos_g[h])));
+                x_g[h] = pos_g[h] - row0 * Wo;
+                off_g[h] = row0 * pitch + x_g[h];
+            }
             auto fetch = [&](int ch, f32x4 &fa, float(&fb)[NBW][4]) {
                 fa = *reinterpret_cast<const f32x4 *>(ap + 8 * (c_lo + ch));
                 // behind the stage's last position grad_out holds zeros; the input is then read at a cell that belongs
                 // to the sum anyway, so that a non-finite input value cannot reach a column it is not part of
-                const int o = pos < np ? off : last_off;
+                const int o0 = pos_g[0] < np ? off_g[0] : last_off, o1 = pos_g[1] < np ? off_g[1] : last_off;
+                const int o = kg ? o1 : o0;
 #pragma unroll
                 for (int i = 0; i < NBW; ++i) {
                     const float *bp = xs + block_base[i] + o;
 #pragma unroll
                     for (int t4 = 0; t4 < 4; ++t4) fb[i][t4] = bp[t4];
                 }
-                pos += 8;
-                x += 8;
-                const bool wrap = x >= Wo;  // (Wo >= 8: at most one wrap)
-                x = wrap ? x - Wo : x;
-                off += wrap ? 8 + pitch - Wo : 8;
+#pragma unroll
+                for (int h = 0; h < 2; ++h) {  // the next chunk: 8 positions on, at most one wrap (Wo >= 8)
+                    pos_g[h] += 8;
+                    x_g[h] += 8;
+                    const bool wrap = x_g[h] >= Wo;
+                    x_g[h] = wrap ? x_g[h] - Wo : x_g[h];
+                    off_g[h] += wrap ? 8 + pitch - Wo : 8;
+                }
             };
             auto multiply = [&](const f32x4 &fa, const float(&fb)[NBW][4]) {
 #pragma unroll
