@@ -181,8 +181,8 @@ def test_lds_resident_kernel_exact(tt, oracle, geom):
 @pytest.mark.parametrize("geom", [
     # fp32, unit stride, 32 output channels, input channels 32 n, rows of whole vectors with at least 8 outputs:
     # grad_weight by the kernel that stages grad_out's and the input's rows in LDS.  B, C, H, W, k, P
-    (3, 32, 28, 28, 3, 1),     # 9 blocks of 32 x 32 over the four waves (3, 3, 3, 0)
-    (2, 64, 12, 16, 3, 1),     # 18 blocks (5, 5, 5, 3)
+    (3, 32, 28, 28, 3, 1),     # 9 blocks of 32 x 32: sets of four waves (3, 2, 2, 2 per set)
+    (2, 64, 12, 16, 3, 1),     # 18 blocks: the four-wave form (5, 5, 5, 3)
     (5, 32, 9, 12, 1, 0),      # 1 x 1: one block, three idle waves
     (2, 32, 20, 20, 5, 2),     # 5 x 5 taps: 25 blocks is more than a wave's five -> the implicit-GEMM kernel
     (2, 32, 10, 12, 3, 0),     # no padding (Wo = 10: not whole vectors -> the implicit-GEMM kernel)
@@ -200,6 +200,59 @@ def test_lds_staged_grad_weight_exact(tt, oracle, geom):
     g = rng.integers(-3, 4, (Bn, O, Ho, Wo)).astype(np.float32)
     gx, gw, gb = tt.conv2d_backward(dev(tt, g), dev(tt, x), dev(tt, w), dev(tt, np.zeros(O, np.float32)), 1, P)
     staged = Wo % 4 == 0 and Wo >= 8 and k * k * (Cc // 32) <= 20
+    assert (_last_kernel(2) == 0x200) == staged, hex(_last_kernel(2))
+    wx, ww, wb = oracle.conv2d_backward(g, x, w, True, 1, P)
+    assert np.array_equal(gw.to_numpy(), ww)
+    assert np.array_equal(gx.to_numpy(), wx) and np.array_equal(gb.to_numpy(), wb)
+
+
+@pytest.mark.parametrize("geom", [
+    # The twelve-wave form of the LDS-resident forward kernel: tiles of 192 positions plus a tail of 0, 4 or 8, taken where
+    # it shares the tiles out over the chip in fewer rounds than tiles of 128.  B, C, O, H, W, k, P, tail
+    (64, 32, 64, 28, 28, 3, 1, 4),     # benchmark configuration 4: four tiles of seven whole rows per image
+    (96, 32, 64, 20, 20, 3, 1, 8),     # tail of eight positions (two groups of four)
+    (80, 32, 64, 24, 24, 3, 1, 0),     # no tail: the exchange-free path with its extra barrier only
+    (96, 32, 64, 33, 12, 3, 1, 8),     # tiles of 200 positions that start and end inside rows of 12
+    (256, 32, 64, 7, 28, 3, 1, 4),     # one tile per image
+    (256, 32, 64, 12, 16, 3, 1, 0),    # one tile per image, no tail
+    (32, 32, 96, 28, 28, 3, 1, 4),     # a second block of output channels that is half empty (rows beyond the last channel)
+    (160, 64, 64, 12, 16, 1, 0, 0),    # 1 x 1 taps, 64 channels in, no padding
+])
+def test_twelve_wave_patch_kernel_exact(tt, oracle, geom):
+    Bn, Cc, O, H, W, k, P, tail = geom
+    rng = np.random.default_rng(sum(geom))
+    x = rng.integers(-3, 4, (Bn, Cc, H, W)).astype(np.float32)
+    w = rng.integers(-3, 4, (O, Cc, k, k)).astype(np.float32)
+    b = rng.integers(-3, 4, (O,)).astype(np.float32)
+    out = tt.conv2d(dev(tt, x), dev(tt, w), dev(tt, b), 1, P).to_numpy()
+    assert _last_kernel(0) == 0x200 + 12 * 16 + 1, hex(_last_kernel(0))
+    assert np.array_equal(out, oracle.conv2d_forward(x, w, b, 1, P))
+    no_bias = tt.conv2d(dev(tt, x), dev(tt, w), None, 1, P).to_numpy()
+    assert np.array_equal(no_bias, out - b[None, :, None, None])
+
+
+@pytest.mark.parametrize("geom", [
+    # grad_weight by the kernel whose sets of waves share out a stage's positions (up to three 32 x 32 blocks per wave:
+    # 32 input channels with 3 x 3 taps, 64 with 1 x 1 or 2 x 2).  B, C, O, H, W, k, P
+    (64, 32, 64, 28, 28, 3, 1),     # benchmark configuration 4: stages of 14 rows, two load instructions per row and channel
+    (3, 32, 64, 28, 28, 3, 1),      # fewer units than workgroups
+    (5, 32, 96, 12, 16, 3, 1),      # three blocks of output channels
+    (300, 32, 64, 8, 8, 3, 1),      # several stages per workgroup, added up in registers
+    (7, 32, 64, 11, 16, 3, 1),      # units of unequal height, a ragged last chunk
+    (4, 64, 64, 16, 16, 1, 0),      # 1 x 1 taps, 64 input channels: two blocks (1, 1, 0, 0 per set)
+    (4, 64, 32, 12, 12, 2, 1),      # 2 x 2 taps (Wo = 13: not whole vectors -> another kernel)
+    (2, 32, 64, 6, 44, 3, 1),       # wide rows
+    (2, 32, 160, 9, 12, 3, 0),      # five blocks of output channels, no padding (Wo = 10 -> another kernel)
+])
+def test_grad_weight_with_sets_of_waves_exact(tt, oracle, geom):
+    Bn, Cc, O, H, W, k, P = geom
+    rng = np.random.default_rng(sum(geom))
+    x = rng.integers(-3, 4, (Bn, Cc, H, W)).astype(np.float32)
+    w = rng.integers(-3, 4, (O, Cc, k, k)).astype(np.float32)
+    Ho, Wo = H + 2 * P - k + 1, W + 2 * P - k + 1
+    g = rng.integers(-3, 4, (Bn, O, Ho, Wo)).astype(np.float32)
+    gx, gw, gb = tt.conv2d_backward(dev(tt, g), dev(tt, x), dev(tt, w), dev(tt, np.zeros(O, np.float32)), 1, P)
+    staged = Wo % 4 == 0 and Wo >= 8
     assert (_last_kernel(2) == 0x200) == staged, hex(_last_kernel(2))
     wx, ww, wb = oracle.conv2d_backward(g, x, w, True, 1, P)
     assert np.array_equal(gw.to_numpy(), ww)

@@ -142,7 +142,8 @@ struct ConvPatchArgs {
     // derived
     int K, lda, cpad, R, pitch, vecs_per_row, xh, last_vecs, n_items, stage_slots, cl_shift, tiles_m, tiles_n;
     int n_seg, seg_len, segs_per_pass, n_fast, n_wvec, w_dense, w_pass_vecs, n_buf;
-    FastDiv d_wfast, d_segv, d_k, d_ngrp, d_xh, d_R, d_cpad4, d_2P, d_P, d_Wo, d_tiles_n;
+    int bne, tail;  // positions per tile; those of them behind the tile's whole 32-position blocks (twelve waves: 4 or 8)
+    FastDiv d_wfast, d_segv, d_k, d_ngrp, d_xh, d_R, d_cpad4, d_2P, d_P, d_Wo, d_tiles_n, d_tail;
 };
 ttamd_status launch_conv_patch_f32(ConvPatchArgs a, hipStream_t stream, int *variant);
 

@@ -50,6 +50,13 @@ __device__ __forceinline__ void interleave_reads() {
     }
 }
 
+// Tail accumulators per lane of the twelve-wave form: a 4x4x1 MFMA covers 16 / (BM / 4) groups of four positions, and a
+// tail is at most two groups (8 positions).
+template <int WGM>
+constexpr int BMx_tail_accs() {
+    return WGM >= 2 ? 2 : 1;
+}
+
 // WGM x WGN waves of one 32 x 32 MFMA block each: output tile (32 WGM) channels x (32 WGN) positions.
 // CC: chunks of 8 reduction indices (8 channels of one tap) that are read and multiplied as one straight-line group;
 // C / 8 is a multiple of it.
@@ -58,11 +65,16 @@ __device__ __forceinline__ void interleave_reads() {
 // SIMD where a wider tile's patch would not fit in LDS); the upper set hands its accumulators over through LDS.
 template <int WGM, int WGN, int CC, int MAXS, int KS = 1>
 __global__ void __launch_bounds__(64 * WGM * WGN * KS, 1) conv_patch_kernel(ConvPatchArgs a) {
-    constexpr int NW = WGM * WGN * KS, NT = 64 * NW;  // 4 waves (one per SIMD) or 8
-    static_assert(NW == 4 || NW == 8, "4 or 8 waves");
+    constexpr int NW = WGM * WGN * KS, NT = 64 * NW;  // 4 waves (one per SIMD), 8 or 12
+    static_assert(NW == 4 || NW == 8 || NW == 12, "4, 8 or 12 waves");
+    // Twelve waves: the tile is a.bne = 32 WGN + a.tail positions, the tail (4 or 8 positions that would leave a whole
+    // 32-position block all but empty) computed with 4x4x1 MFMAs after the blocks -- see `tail` below.
+    constexpr bool kTail = NW == 12;
+    constexpr int NTA = BMx_tail_accs<WGM>();  // tail accumulators per lane: 8 positions at most
     static_assert(KS == 1 || KS == 2, "one or two halves of the reduction");
     constexpr int WVECS = kWeightLoads / NW;
     constexpr int BM = 32 * WGM, BN = 32 * WGN;
+    const int bne = kTail ? a.bne : BN;  // positions per tile
     extern __shared__ __attribute__((aligned(16))) float smem_patch[];
     float *const A = smem_patch;                   // [BM][lda], k' = tap * C + c
     float *const patch = smem_patch + BM * a.lda;  // [1 or 2][R][pitch][cpad]
@@ -136,7 +148,7 @@ __global__ void __launch_bounds__(64 * WGM * WGN * KS, 1) conv_patch_kernel(Conv
     uint32_t t_b, t_n;
     a.d_tiles_n.divmod(static_cast<uint32_t>(j), t_b, t_n);
     int tile_b = static_cast<int>(t_b), tile_n = static_cast<int>(t_n);
-    int tile_h = static_cast<int>(a.d_Wo.div(static_cast<uint32_t>(tile_n * BN)));  // first output row of the tile
+    int tile_h = static_cast<int>(a.d_Wo.div(static_cast<uint32_t>(tile_n * bne)));  // first output row of the tile
     uint32_t step_b, step_n;
     a.d_tiles_n.divmod(static_cast<uint32_t>(groups), step_b, step_n);
     if (j < n_tiles) request(tile_b, tile_h);  // on its way while the weights are brought in
@@ -281,12 +293,12 @@ __global__ void __launch_bounds__(64 * WGM * WGN * KS, 1) conv_patch_kernel(Conv
     // nothing else would hide it.
     for (int cur = 0; j < n_tiles; j += groups, cur ^= a.n_buf - 1) {
         const int jn = j + groups;
-        const int b = tile_b, n0 = tile_n * BN, h_first = tile_h;
+        const int b = tile_b, n0 = tile_n * bne, h_first = tile_h;
         if (jn < n_tiles) {  // the next tile's rows are in flight during this tile's MFMA work
             tile_n += static_cast<int>(step_n);
             tile_b += static_cast<int>(step_b);
             if (tile_n >= a.tiles_n) tile_n -= a.tiles_n, ++tile_b;
-            tile_h = static_cast<int>(a.d_Wo.div(static_cast<uint32_t>(tile_n * BN)));
+            tile_h = static_cast<int>(a.d_Wo.div(static_cast<uint32_t>(tile_n * bne)));
             request(tile_b, tile_h);
         }
         const int n = n0 + wn * 32 + li;
@@ -331,7 +343,90 @@ __global__ void __launch_bounds__(64 * WGM * WGN * KS, 1) conv_patch_kernel(Conv
         }
         if (g < g_end) multiply(fa0, fb0);
 
-        if constexpr (KS == 2) {
+        if constexpr (kTail) {
+            // ---- the tile's last a.tail positions, n0 + BN ...: D[channel][position] in 4 x 4 blocks, sixteen to a
+            // v_mfma_f32_4x4x1 -- lane l supplies A[block l / 4][row l % 4] and B[block l / 4][column l % 4] and receives
+            // column l % 4 of its block, rows 0 .. 3.  A block is four channels by four positions: BM / 4 channel groups
+            // times 16 / (BM / 4) position groups per instruction.  The waves share out the reduction groups; their
+            // partial tails are added in wave order below.
+            constexpr int NCG = BM / 4, PPM = 16 / NCG;
+            f32x4 tacc[NTA];
+#pragma unroll
+            for (int u = 0; u < NTA; ++u) tacc[u] = f32x4{0.f, 0.f, 0.f, 0.f};
+            if (a.tail > 0) {
+                const int blk = lane / 4, ti = lane % 4;
+                const int t_ch = 4 * (blk % NCG) + ti;
+                const float *tb[NTA];
+#pragma unroll
+                for (int u = 0; u < NTA; ++u) {
+                    const int pt = 4 * (u * PPM + blk / NCG) + ti;
+                    int nt = n0 + BN + (pt < a.tail ? pt : 0);  // (beyond the tail: a column nobody reads)
+                    nt = nt < HoWo ? nt : HoWo - 1;
+                    uint32_t th, tw;
+                    a.d_Wo.divmod(static_cast<uint32_t>(nt), th, tw);
+                    tb[u] = patch + cur * patch_elems + ((static_cast<int>(th) - h_first) * pitch + static_cast<int>(tw)) * cpad;
+                }
+                const float *const ta = A + t_ch * a.lda;
+                const int tg_lo = wave * n_groups / NW, tg_hi = (wave + 1) * n_groups / NW;
+                const int n_tacc = (a.tail / 4 + PPM - 1) / PPM;
+#pragma unroll 1
+                for (int tg = tg_lo; tg < tg_hi; ++tg) {
+                    uint32_t tap, cg, p, q;
+                    a.d_ngrp.divmod(static_cast<uint32_t>(tg), tap, cg);
+                    a.d_k.divmod(tap, p, q);
+                    const int boff = (static_cast<int>(p) * pitch + static_cast<int>(q)) * cpad + static_cast<int>(cg) * (8 * CC);
+#pragma unroll
+                    for (int i = 0; i < 2 * CC; ++i) {
+                        const f32x4 fa = lds_load4(ta + 8 * CC * tg + 4 * i);
+#pragma unroll
+                        for (int u = 0; u < NTA; ++u) {
+                            if (u < n_tacc) {  // uniform
+                                const f32x4 fb = lds_load4(tb[u] + boff + 4 * i);
+#pragma unroll
+                                for (int t = 0; t < 4; ++t) tacc[u] = __builtin_amdgcn_mfma_f32_4x4x1f32(fa[t], fb[t], tacc[u], 0, 0, 0);
+                            }
+                        }
+                    }
+                }
+            }
+            // The patch has been read: its memory takes the upper set's accumulators and the waves' tails.
+            __syncthreads();
+            float *const exch = patch + cur * patch_elems + (wtile * 64 + lane) * 16;
+            float *const tails = patch + cur * patch_elems + (KS == 2 ? WGM * WGN * 64 * 16 : 0);  // [NW][NTA][64 lanes][4]
+            if (KS == 2 && ks == 1) {
+#pragma unroll
+                for (int e = 0; e < 16; e += 4) *reinterpret_cast<f32x4 *>(exch + e) = f32x4{acc[e], acc[e + 1], acc[e + 2], acc[e + 3]};
+            }
+            if (a.tail > 0) {
+#pragma unroll
+                for (int u = 0; u < NTA; ++u) *reinterpret_cast<f32x4 *>(tails + ((wave * NTA + u) * 64 + lane) * 4) = tacc[u];
+            }
+            __syncthreads();
+            if (KS == 2 && ks == 0) {  // (lower half of the groups) + (upper half): a fixed order
+#pragma unroll
+                for (int e = 0; e < 16; e += 4) {
+                    const f32x4 v = *reinterpret_cast<const f32x4 *>(exch + e);
+#pragma unroll
+                    for (int t = 0; t < 4; ++t) acc[e + t] += v[t];
+                }
+            }
+            if (tid < BM * a.tail) {  // one lane per element of the tail: the waves' parts in wave order, bias, store
+                uint32_t ch, pt;
+                a.d_tail.divmod(static_cast<uint32_t>(tid), ch, pt);
+                const int pg = static_cast<int>(pt) / 4, j = static_cast<int>(pt) % 4;
+                const int u = pg / PPM, src_lane = 4 * ((pg % PPM) * NCG + static_cast<int>(ch) / 4) + j;
+                const float *src = tails + (u * 64 + src_lane) * 4 + static_cast<int>(ch) % 4;
+                float v = 0.f;
+#pragma unroll
+                for (int w = 0; w < NW; ++w) v += src[w * NTA * 256];
+                const int o = m0 + static_cast<int>(ch), nt = n0 + BN + static_cast<int>(pt);
+                if (o < a.O && nt < HoWo) {
+                    if (a.bias) v += a.bias[o];
+                    a.out[(static_cast<int64_t>(b) * a.O + o) * HoWo + nt] = v;
+                }
+            }
+            if (jn < n_tiles) __syncthreads();  // the next tile's rows overwrite what was just read
+        } else if constexpr (KS == 2) {
             // the upper set's sums go to the lower set through LDS (behind the patch buffers), added as
             // (lower half of the groups) + (upper half): a fixed order
             float *const exch = patch + a.n_buf * patch_elems + (wtile * 64 + lane) * 16;
@@ -381,13 +476,21 @@ __global__ void __launch_bounds__(64 * WGM * WGN * KS, 1) conv_patch_kernel(Conv
 }
 
 // Derived geometry for tiles of BM x BN computed by `waves` waves; false when this kernel does not apply.
-bool plan_patch(ConvPatchArgs &a, int BM, int BN, int waves, int n_buf, size_t *lds_bytes, int halves = 1) {
+// bne > 0 (twelve waves): the tile is bne = BN + tail positions, the tail of 4 or 8 computed apart; the exchange of the
+// halves and the waves' tails pass through the patch buffer.
+bool plan_patch(ConvPatchArgs &a, int BM, int BN, int waves, int n_buf, size_t *lds_bytes, int halves = 1, int bne = 0) {
     const int k = a.k, threads = 64 * waves;
     const int HoWo = a.Ho * a.Wo;
+    a.bne = bne > 0 ? bne : BN;
+    a.tail = a.bne - BN;
+    a.d_tail = make_fastdiv(static_cast<uint32_t>(a.tail > 0 ? a.tail : 1));
+    if (a.tail < 0 || a.tail > 8 || a.tail % 4 != 0) return false;
+    BN = a.bne;  // the patch and the tile count follow the whole tile
     a.K = a.C * k * k;
     a.lda = a.K + 4;   // 4 (2 n + 1) floats: the 16-byte reads of 16 consecutive rows cover every bank once
     a.cpad = a.C + 4;  // likewise for 16 consecutive patch columns
-    a.R = (a.Wo - 1 + BN - 1) / a.Wo + 1 + (k - 1);
+    // rows of output positions under a tile (tiles of whole rows all start in column 0), plus the taps' halo rows
+    a.R = (BN % a.Wo == 0 ? BN / a.Wo : (a.Wo - 1 + BN - 1) / a.Wo + 1) + (k - 1);
     a.pitch = a.W + 2 * a.P;  // columns -P .. W - 1 + P at index x + P
     a.vecs_per_row = a.W / 4;
     a.cl_shift = a.C % 16 == 0 ? 4 : 3;
@@ -400,9 +503,10 @@ bool plan_patch(ConvPatchArgs &a, int BM, int BN, int waves, int n_buf, size_t *
     a.tiles_n = (HoWo + BN - 1) / BN;
     const int64_t patch_elems = static_cast<int64_t>(a.R) * a.pitch * a.cpad;
     a.n_buf = n_buf;
-    int64_t lds_floats = static_cast<int64_t>(BM) * a.lda + n_buf * patch_elems + (halves == 2 ? waves / 2 * 64 * 16 : 0);
+    int64_t lds_floats = static_cast<int64_t>(BM) * a.lda + n_buf * patch_elems + (halves == 2 && bne == 0 ? waves / 2 * 64 * 16 : 0);
+    if (bne > 0 && (halves == 2 ? waves / 2 * 64 * 16 : 0) + static_cast<int64_t>(waves) * 2 * 256 > patch_elems) return false;
     if (halves == 2 && (a.C % 32 != 0 || (static_cast<int64_t>(a.C) / 32 * k * k) % 2 != 0)) return false;  // an even number of 32-channel groups
-    if (a.stage_slots > kStageLoads / waves || lds_floats * 4 > kLdsBytes) return false;
+    if (a.stage_slots > (waves == 12 ? 6 : kStageLoads / waves) || lds_floats * 4 > kLdsBytes) return false;
     if (static_cast<int64_t>(a.B) * a.tiles_n > 0x7fffffff || static_cast<int64_t>(a.O) * HoWo * 4 >= 0x7fffffff) return false;
     if (static_cast<int64_t>(a.C) * a.xs_c * 4 + static_cast<int64_t>(a.R) * a.xs_h * 4 >= 0x7fffffff) return false;
     if (static_cast<int64_t>(a.O + BM) * a.w_row * 4 + static_cast<int64_t>(a.C) * a.w_red * 4 >= 0x7fffffff) return false;
@@ -452,7 +556,7 @@ ttamd_status launch_patch(ConvPatchArgs a, hipStream_t st, size_t lds) {
 
 template <int WGM, int WGN, int KS = 1>
 ttamd_status launch_patch_cc(const ConvPatchArgs &a, hipStream_t st, size_t lds) {
-    constexpr int S1 = kStageLoads / (WGM * WGN * KS), S0 = S1 / 2;  // slot counts compiled for
+    constexpr int S1 = WGM * WGN * KS == 12 ? 6 : kStageLoads / (WGM * WGN * KS), S0 = S1 / 2;  // slot counts compiled for
     const bool few = a.stage_slots <= S0;
     if constexpr (KS == 2) {  // (only with 32-channel groups, of which each set takes half)
         return few ? launch_patch<WGM, WGN, 4, S0, 2>(a, st, lds) : launch_patch<WGM, WGN, 4, S1, 2>(a, st, lds);
@@ -478,6 +582,33 @@ ttamd_status launch_conv_patch_f32(ConvPatchArgs a, hipStream_t st, int *variant
     if (a.Ho != a.H + 2 * a.P - k + 1 || a.Wo != a.W + 2 * a.P - k + 1 || a.Ho < 1 || a.Wo < 1) return TTAMD_OK;  // unit stride only
     const bool narrow = a.O <= 32;
     size_t lds = 0;
+    // Twelve waves on a tile of 192 positions and a tail of 4 or 8 where that shares the tiles out better: cost = rounds of
+    // the 256 workgroups times the MFMA blocks (whole reductions) a SIMD runs per tile.  [64,32,28,28] -> 64 channels: 448
+    // tiles of 128 positions (the seventh of an image all but empty) are two rounds of 2 blocks per SIMD, 256 tiles of
+    // 196 one round of 3.
+    static const bool twelve_ok = std::getenv("TTAMD_CONV_PATCH_WAVES") == nullptr || std::atoi(std::getenv("TTAMD_CONV_PATCH_WAVES")) == 12;
+    // (32 output channels -- two sets of six waves on the halves of the reduction -- measured slower than the eight-wave
+    // form on [64,64,28,28] -> 32 channels, 34.3 against 28.9 us: its six staging slots spill; left to that form.)
+    if (twelve_ok && a.C % 32 == 0 && !narrow) {
+        const int64_t HoWo = static_cast<int64_t>(a.Ho) * a.Wo;
+        const int BM = narrow ? 32 : 64;
+        const int64_t tiles_m = (a.O + BM - 1) / BM;
+        const int64_t old_tiles = a.B * ((HoWo + 127) / 128) * tiles_m;
+        const int64_t old_cost2 = ((old_tiles + 255) / 256) * (narrow ? 2 : 4);  // in half blocks per SIMD
+        int best_bne = 0;
+        int64_t best_cost2 = old_cost2;
+        for (int64_t q = (HoWo + 199) / 200; q <= (HoWo + 191) / 192; ++q) {
+            if (q < 1) continue;
+            const int64_t pt = ((HoWo + q - 1) / q + 3) / 4 * 4;
+            if (pt < 192 || pt > 200) continue;
+            const int64_t cost2 = ((a.B * q * tiles_m + 255) / 256) * (narrow ? 3 : 6);
+            if (cost2 < best_cost2) best_cost2 = cost2, best_bne = static_cast<int>(pt);
+        }
+        if (best_bne && plan_patch(a, BM, 192, 12, 1, &lds, narrow ? 2 : 1, best_bne)) {
+            *variant = 12 * 16 + 1;
+            return narrow ? launch_patch_cc<1, 6, 2>(a, st, lds) : launch_patch_cc<2, 6>(a, st, lds);
+        }
+    }
     static const bool wide_ok = std::getenv("TTAMD_CONV_PATCH_WAVES") == nullptr || std::atoi(std::getenv("TTAMD_CONV_PATCH_WAVES")) != 4;
     for (int n_buf = 2; n_buf >= 1; --n_buf) {  // one patch buffer (a second barrier per tile) when two do not fit
         if (wide_ok && plan_patch(a, narrow ? 32 : 64, narrow ? 256 : 128, 8, n_buf, &lds)) {
