@@ -229,6 +229,14 @@ def test_twelve_wave_patch_kernel_exact(tt, oracle, geom):
     assert np.array_equal(out, oracle.conv2d_forward(x, w, b, 1, P))
     no_bias = tt.conv2d(dev(tt, x), dev(tt, w), None, 1, P).to_numpy()
     assert np.array_equal(no_bias, out - b[None, :, None, None])
+    # grad_input is the same kernel on grad_out with 32 result channels: twelve waves as two sets of six on the halves of the
+    # reduction, where the number of 32-channel groups is even and the tile count favours it
+    g = rng.integers(-3, 4, out.shape).astype(np.float32)
+    gx, gw, gb = tt.conv2d_backward(dev(tt, g), dev(tt, x), dev(tt, w), dev(tt, b), 1, P)
+    if (H, W, O) in ((28, 28, 64), (7, 28, 64), (12, 16, 64)):   # (elsewhere its patch of 64 channels takes too many loads per lane)
+        assert _last_kernel(1) == 0x200 + 12 * 16 + 1, hex(_last_kernel(1))
+    wx, ww, wb = oracle.conv2d_backward(g, x, w, True, 1, P)
+    assert np.array_equal(gx.to_numpy(), wx) and np.array_equal(gw.to_numpy(), ww) and np.array_equal(gb.to_numpy(), wb)
 
 
 @pytest.mark.parametrize("geom", [

@@ -559,6 +559,9 @@ ttamd_status launch_patch_cc(const ConvPatchArgs &a, hipStream_t st, size_t lds)
     constexpr int S1 = WGM * WGN * KS == 12 ? 6 : kStageLoads / (WGM * WGN * KS), S0 = S1 / 2;  // slot counts compiled for
     const bool few = a.stage_slots <= S0;
     if constexpr (KS == 2) {  // (only with 32-channel groups, of which each set takes half)
+        // twelve waves have 168 registers each: groups of 16 channels (with groups of 32 the six staging slots of a
+        // 64-channel patch spilled, and grad_input of [64,32,28,28] -> 64 channels took 34.3 us instead of 26.6)
+        if constexpr (WGM * WGN * KS == 12) return few ? launch_patch<WGM, WGN, 2, S0, 2>(a, st, lds) : launch_patch<WGM, WGN, 2, S1, 2>(a, st, lds);
         return few ? launch_patch<WGM, WGN, 4, S0, 2>(a, st, lds) : launch_patch<WGM, WGN, 4, S1, 2>(a, st, lds);
     } else {
         if (a.C % 32 == 0) return few ? launch_patch<WGM, WGN, 4, S0>(a, st, lds) : launch_patch<WGM, WGN, 4, S1>(a, st, lds);
@@ -587,9 +590,8 @@ ttamd_status launch_conv_patch_f32(ConvPatchArgs a, hipStream_t st, int *variant
     // tiles of 128 positions (the seventh of an image all but empty) are two rounds of 2 blocks per SIMD, 256 tiles of
     // 196 one round of 3.
     static const bool twelve_ok = std::getenv("TTAMD_CONV_PATCH_WAVES") == nullptr || std::atoi(std::getenv("TTAMD_CONV_PATCH_WAVES")) == 12;
-    // (32 output channels -- two sets of six waves on the halves of the reduction -- measured slower than the eight-wave
-    // form on [64,64,28,28] -> 32 channels, 34.3 against 28.9 us: its six staging slots spill; left to that form.)
-    if (twelve_ok && a.C % 32 == 0 && !narrow) {
+    // 32 output channels: two sets of six waves on the halves of the reduction.
+    if (twelve_ok && a.C % 32 == 0) {
         const int64_t HoWo = static_cast<int64_t>(a.Ho) * a.Wo;
         const int BM = narrow ? 32 : 64;
         const int64_t tiles_m = (a.O + BM - 1) / BM;
