@@ -564,8 +564,12 @@ ttamd_status launch_patch_cc(const ConvPatchArgs &a, hipStream_t st, size_t lds)
         if constexpr (WGM * WGN * KS == 12) return few ? launch_patch<WGM, WGN, 2, S0, 2>(a, st, lds) : launch_patch<WGM, WGN, 2, S1, 2>(a, st, lds);
         return few ? launch_patch<WGM, WGN, 4, S0, 2>(a, st, lds) : launch_patch<WGM, WGN, 4, S1, 2>(a, st, lds);
     } else {
-        if (a.C % 32 == 0) return few ? launch_patch<WGM, WGN, 4, S0>(a, st, lds) : launch_patch<WGM, WGN, 4, S1>(a, st, lds);
-        return few ? launch_patch<WGM, WGN, 1, S0>(a, st, lds) : launch_patch<WGM, WGN, 1, S1>(a, st, lds);
+        if constexpr (WGM * WGN * KS == 12) {  // (C is a multiple of 32 here; more than three slots: groups of 16 channels, as above)
+            return few ? launch_patch<WGM, WGN, 4, S0>(a, st, lds) : launch_patch<WGM, WGN, 2, S1>(a, st, lds);
+        } else {
+            if (a.C % 32 == 0) return few ? launch_patch<WGM, WGN, 4, S0>(a, st, lds) : launch_patch<WGM, WGN, 4, S1>(a, st, lds);
+            return few ? launch_patch<WGM, WGN, 1, S0>(a, st, lds) : launch_patch<WGM, WGN, 1, S1>(a, st, lds);
+        }
     }
 }
 
