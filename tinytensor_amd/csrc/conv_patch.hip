@@ -53,7 +53,7 @@ __device__ __forceinline__ void interleave_reads() {
 // Tail accumulators per lane of the twelve-wave form: a 4x4x1 MFMA covers 16 / (BM / 4) groups of four positions, and a
 // tail is at most two groups (8 positions).
 template <int WGM>
-constexpr int BMx_tail_accs() {
+constexpr int tail_accumulators() {
     return WGM >= 2 ? 2 : 1;
 }
 
@@ -70,7 +70,7 @@ __global__ void __launch_bounds__(64 * WGM * WGN * KS, 1) conv_patch_kernel(Conv
     // Twelve waves: the tile is a.bne = 32 WGN + a.tail positions, the tail (4 or 8 positions that would leave a whole
     // 32-position block all but empty) computed with 4x4x1 MFMAs after the blocks -- see `tail` below.
     constexpr bool kTail = NW == 12;
-    constexpr int NTA = BMx_tail_accs<WGM>();  // tail accumulators per lane: 8 positions at most
+    constexpr int NTA = tail_accumulators<WGM>();  // tail accumulators per lane: 8 positions at most
     static_assert(KS == 1 || KS == 2, "one or two halves of the reduction");
     constexpr int WVECS = kWeightLoads / NW;
     constexpr int BM = 32 * WGM, BN = 32 * WGN;
