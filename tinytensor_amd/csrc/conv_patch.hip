@@ -166,6 +166,16 @@ __global__ void __launch_bounds__(64 * WGM * WGN * KS, 1) conv_patch_kernel(Conv
         }
     }
 
+    // twelve waves: the bias of the tail element that this lane will add up and store (requested here, with the loads
+    // above, so that its latency is not in front of the tail's store)
+    float tail_bias = 0.f;
+    if constexpr (kTail) {
+        if (a.bias && tid < BM * a.tail) {
+            const int o = m0 + static_cast<int>(a.d_tail.div(static_cast<uint32_t>(tid)));
+            if (o < a.O) tail_bias = a.bias[o];
+        }
+    }
+
     // ---- once per workgroup: the weight block, into A in the order k' = tap * C + c.
     // 3 x 3 kernels: a lane takes (row, reduction channel) pairs, reads the pair's nine taps (consecutive floats in
     // memory in both weight layouts) straight from memory, every load of its pairs in flight together, and writes them
@@ -420,10 +430,7 @@ __global__ void __launch_bounds__(64 * WGM * WGN * KS, 1) conv_patch_kernel(Conv
 #pragma unroll
                 for (int w = 0; w < NW; ++w) v += src[w * NTA * 256];
                 const int o = m0 + static_cast<int>(ch), nt = n0 + BN + static_cast<int>(pt);
-                if (o < a.O && nt < HoWo) {
-                    if (a.bias) v += a.bias[o];
-                    a.out[(static_cast<int64_t>(b) * a.O + o) * HoWo + nt] = v;
-                }
+                if (o < a.O && nt < HoWo) a.out[(static_cast<int64_t>(b) * a.O + o) * HoWo + nt] = v + tail_bias;
             }
             if (jn < n_tiles) __syncthreads();  // the next tile's rows overwrite what was just read
         } else if constexpr (KS == 2) {
