@@ -80,12 +80,14 @@ def test_validation_without_gpu(tt):
     sz = C.c_size_t(1)
     assert lib.ttamd_conv2d_backward_workspace(capi.I32, 4, 3, 8, 8, 4, 3, 1, 0, C.byref(sz)) == capi.ERR_UNSUPPORTED_DTYPE
     assert lib.ttamd_conv2d_backward_workspace(capi.F32, 64, 32, 28, 28, 64, 3, 1, 1, C.byref(sz)) == capi.OK
-    # the transposed weight, one partial grad_weight tile per (image, half of the positions), 256 rows of grad_bias sums
+    # the transposed weight, one partial grad_weight tile per (image, half of the positions) -- the stages of the kernel
+    # whose sets of waves share out the positions; each tile written by two workgroups, one per block of 32 output
+    # channels -- and 256 rows of grad_bias sums
     tile = 64 * 32 * 9 * 4
     assert sz.value == tile + 128 * tile + 256 * 64 * 4
-    assert lib.ttamd_conv2d_backward_workspace(capi.F32, 1, 32, 28, 28, 64, 3, 1, 1, C.byref(sz)) == capi.OK and sz.value == tile + 5 * tile + 256 * 64 * 4
-    # 32 output channels: grad_weight by the kernel that stages both operands in LDS, one partial tile per workgroup
-    # (256 workgroups of a quarter image each)
+    # a single image: one stage per output row (28 partial tiles)
+    assert lib.ttamd_conv2d_backward_workspace(capi.F32, 1, 32, 28, 28, 64, 3, 1, 1, C.byref(sz)) == capi.OK and sz.value == tile + 28 * tile + 256 * 64 * 4
+    # 32 output channels: the same kernel, 256 workgroups of a quarter image each
     half = 32 * 32 * 9 * 4
     assert lib.ttamd_conv2d_backward_workspace(capi.F32, 64, 32, 28, 28, 32, 3, 1, 1, C.byref(sz)) == capi.OK and sz.value == half + 256 * half + 256 * 32 * 4
     assert lib.ttamd_conv2d_backward_workspace(capi.F64, 1, 3, 8, 8, 5, 3, 1, 1, C.byref(sz)) == capi.OK
