@@ -250,6 +250,8 @@ def detail_report(tt, np, path, cpu=True):
     go = tt.Tensor.from_numpy(np.ones((64, 64, 28, 28), f32))
     out = be.conv2d(x, w, None, 1, 1)
     ms = time_launches(tt, lambda: be.conv2d(x, w, None, 1, 1, out=out), 100, 10)
+    lib_last = tt._capi.lib.ttamd_conv2d_last_kernel
+
     def conv_kernel(which, implicit):  # which family the last launch took (include/ttamd.h: ttamd_conv2d_last_kernel)
         code = tt._capi.lib.ttamd_conv2d_last_kernel(which)
         if code & 0xF00 == 0x200:
@@ -261,7 +263,8 @@ def detail_report(tt, np, path, cpu=True):
     bufs = be.conv2d_backward(go, x, w, None, 1, 1, return_buffers=True)
     ms = time_launches(tt, lambda: be.conv2d_backward(go, x, w, None, 1, 1, buffers=bufs), 50, 5)
     rows.append({"case": "cfg4 conv2d backward (grad_input + grad_weight)",
-                 "kernel": conv_kernel(1, "conv_dgrad_kernel (implicit GEMM)") + " + conv_wgrad_kernel + reduce",
+                 "kernel": conv_kernel(1, "conv_dgrad_kernel (implicit GEMM)") + " + "
+                           + ("conv_wgrad_patch kernel (operands staged in LDS)" if lib_last(2) == 0x200 else "conv_wgrad_kernel (implicit GEMM)") + " + reduce",
                  "ms": round(ms, 5), "GFLOP/s": round(3.700e9 / ms / 1e6, 1)})
     # Streaming kernels around the GEMMs (HBM-bound; GB/s counts each operand and the result once), called through
     # the C ABI with preallocated results so that no allocation is timed.
