@@ -153,3 +153,35 @@ def test_random_stride_two_convs(tt, oracle, seed):
         assert gb is None
         assert np.array_equal(gx.to_numpy(), wx), tag
         assert np.array_equal(gw.to_numpy(), ww), tag
+
+
+@pytest.mark.parametrize("seed", range(8))
+def test_random_lds_staged_convs(tt, oracle, seed):
+    """Unit-stride fp32 layers inside and around the conditions of the kernels that keep an operand in LDS: 32 or 64
+    input channels, 32 to 160 output channels, rows of whole 16-byte vectors, 1 x 1 to 3 x 3 taps with every padding below
+    them, and batches from a few images to several hundred -- the plans of those kernels (tiles of 128 or of 192 + 4 / 8
+    positions and how many waves, stages of how many rows, sets of waves) depend on all of these.  Forward with a bias and
+    the whole backward pass, exact against the oracle on integer-valued data."""
+    rng = np.random.default_rng(5000 + seed)
+    for case in range(10):
+        Cc, O = 32 * int(rng.integers(1, 3)), 32 * int(rng.integers(1, 6))
+        k = int(rng.integers(1, 4))
+        P = int(rng.integers(0, k))
+        H, W = int(rng.integers(max(3, k), 34)), 4 * int(rng.integers(2, 9))
+        Bn = int(rng.choice([2, 5, 40, 96, 130, 300]))
+        if Bn * Cc * H * W > 6_000_000:   # (keeps the oracle's share of the run to seconds)
+            Bn = max(2, 6_000_000 // (Cc * H * W))
+        x = rng.integers(-3, 4, (Bn, Cc, H, W)).astype(np.float32)
+        w = rng.integers(-3, 4, (O, Cc, k, k)).astype(np.float32)
+        bias = rng.integers(-3, 4, (O,)).astype(np.float32)
+        tag = f"seed {seed} case {case}: B{Bn} C{Cc} O{O} {H}x{W} k{k} s1 p{P}"
+        tx, tw = tt.Tensor.from_numpy(x), tt.Tensor.from_numpy(w)
+        out = tt.conv2d(tx, tw, tt.Tensor.from_numpy(bias), 1, P).to_numpy()
+        want = oracle.conv2d_forward(x, w, bias, 1, P)
+        assert np.array_equal(out, want), tag
+        g = rng.integers(-3, 4, want.shape).astype(np.float32)
+        gx, gw, gb = tt.conv2d_backward(tt.Tensor.from_numpy(g), tx, tw, tt.Tensor.from_numpy(bias), 1, P)
+        wx, ww, wb = oracle.conv2d_backward(g, x, w, True, 1, P)
+        assert np.array_equal(gx.to_numpy(), wx), tag
+        assert np.array_equal(gw.to_numpy(), ww), tag
+        assert np.array_equal(gb.to_numpy(), wb), tag
