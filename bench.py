@@ -510,8 +510,9 @@ def main():
         oracle.matmul_kernel(A, B, "fast")
         dt = time.perf_counter() - t0
         cpu = {"value": round(flop / dt / 1e9, 3), "unit": "GFLOP/s", "cores": 1, "kind": "port",
-               "sample": f"one full f32 {n}x{n}x{n} product, {dt:.1f} s, gcc -O3 x86-64 128-bit fma, host has "
-                         f"{os.cpu_count()} logical cores"}
+               "sample": f"one full f32 {n}x{n}x{n} product, {dt:.1f} s, oracle built with gcc -O3 -ffp-contract=fast "
+                         + ("-march=x86-64-v4 -mprefer-vector-width=128" if oracle._cpu_has("avx512vl") else "-march=x86-64-v3")
+                         + f" (same arithmetic either way), host has {os.cpu_count()} logical cores"}
 
     line = {
         "metric": f"fp32 GEMM GFLOP/s at {n}^3 on 1 MI355X",
