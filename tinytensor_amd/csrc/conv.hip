@@ -61,6 +61,7 @@ struct Im2colStager : TileLayout<T, ROWS, BK, false> {
     static constexpr int P = BK / LPP;
     static_assert(ROWS % 64 == 0 && BK % LPP == 0, "a wave must share its k line");
     static constexpr int kPF = PF;
+    static constexpr bool kTapTable = false;
     T reg[PF][P];
     __amdgpu_buffer_rsrc_t rsrc;
     const ConvGeom *g;
@@ -123,6 +124,7 @@ struct Im2colTStager : TileLayout<T, ROWS, BK, true> {
     static constexpr int P = ROWS / RPP;
     static_assert(ROWS % RPP == 0, "tile must split evenly");
     static constexpr int kPF = PF;
+    static constexpr bool kTapTable = false;
     T reg[PF][P];
     __amdgpu_buffer_rsrc_t rsrc;
     const ConvGeom *g;
@@ -194,6 +196,7 @@ struct DgradStager : TileLayout<T, ROWS, BK, false> {
     static constexpr int P = BK / LPP;
     static_assert(ROWS % 64 == 0 && BK % LPP == 0, "a wave must share its k line");
     static constexpr int kPF = PF;
+    static constexpr bool kTapTable = false;
     T reg[PF][P];
     __amdgpu_buffer_rsrc_t rsrc;
     const ConvGeom *g;
@@ -341,6 +344,9 @@ __device__ __forceinline__ typename Vec<T, VEC>::type pick_strided(const typenam
     }
 }
 
+constexpr int kTapTableEntries = 128;  // window taps (k * k) served by a stager's (dy, dx) table; behind the tile buffers in LDS
+constexpr size_t kTapTableBytes = kTapTableEntries * sizeof(int2);
+
 // MC layout (positions contiguous in LDS), vectors along the positions: B operand of forward and of
 // grad_input.  Requires positions-per-row % VEC == 0 so that a vector never crosses a plane row.
 // STRIDE (forward only): the convolution's stride.  Position (py, px) then reads source element
@@ -355,6 +361,7 @@ struct TapStagerMC : TileLayout<T, ROWS, BK, false> {
     static_assert(VEC > 1 && ROWS % VEC == 0 && kThreads % VPL == 0 && BK % LPP == 0, "tile must split evenly");
     static_assert(STRIDE == 1 || !FLIP, "the strided gather serves the forward product");
     static constexpr int kPF = PF;
+    static constexpr bool kTapTable = true;
     V reg[PF][P][STRIDE];
     int col0[PF][P];  // first source column of each gathered vector
     __amdgpu_buffer_rsrc_t rsrc;
@@ -362,8 +369,27 @@ struct TapStagerMC : TileLayout<T, ROWS, BK, false> {
     int n_local, line0, k_next;
     int py, px0;
     bool n_ok;
+    // The reduction index of pass p, kept as (index, channel offset, tap within the window) and advanced by BK per
+    // load -- a k tile on is BK / (window taps) channels and BK % (window taps) taps on, with at most one carry --
+    // instead of two divisions per load; the tap's (dy, dx) comes from a table in LDS with one entry per window tap.
+    int kk_p[P], r_p[P];
+    int32_t ch_p[P];
+    const int2 *tab;
 
-    __device__ __forceinline__ explicit TapStagerMC(const ConvGeom &geo) : tv(geo) {}
+    __device__ __forceinline__ explicit TapStagerMC(const ConvGeom &geo) : tv(geo), tab(nullptr) {}
+
+    // The window's taps as (dy, dx), written by the first lanes of the workgroup (a barrier must follow before the first
+    // load).  The host sends windows of more than kTapTableEntries taps to the element-wise stagers.
+    __device__ __forceinline__ void fill_tap_table(int2 *table, int tid) {
+        const int window = static_cast<int>(tv.d_kk.d);
+        tab = table;
+        if (tid < window && tid < kTapTableEntries) {
+            int32_t ch_off;
+            int dy, dx;
+            tv.tap(static_cast<uint32_t>(tid), ch_off, dy, dx);
+            table[tid] = int2{dy, dx};
+        }
+    }
 
     __device__ __forceinline__ void init(const T *image, int64_t image_bytes, int tid, int n0) {
         rsrc = make_rsrc(image, image_bytes);
@@ -376,17 +402,33 @@ struct TapStagerMC : TileLayout<T, ROWS, BK, false> {
         tv.d_pw.divmod(static_cast<uint32_t>(n_ok ? n : 0), y, x);
         py = static_cast<int>(y);
         px0 = static_cast<int>(x);
+#pragma unroll
+        for (int p = 0; p < P; ++p) {
+            kk_p[p] = p * LPP + line0;
+            uint32_t ch, r;
+            tv.d_kk.divmod(static_cast<uint32_t>(kk_p[p]), ch, r);
+            ch_p[p] = static_cast<int32_t>(ch) * tv.s_ch;
+            r_p[p] = static_cast<int>(r);
+        }
     }
 
     template <bool MASK, int SLOT = 0>
     __device__ __forceinline__ void load(int /*k_left*/) {
+        const int window = static_cast<int>(tv.d_kk.d);
+        const int step_r = BK % window;                                    // (wave-uniform: scalar arithmetic)
+        const int32_t step_ch = static_cast<int32_t>(BK / window) * tv.s_ch;
 #pragma unroll
         for (int p = 0; p < P; ++p) {
-            const int kk = k_next + p * LPP + line0;
+            const int kk = kk_p[p];
             const bool k_ok = kk < tv.taps;
-            int32_t ch_off;
-            int dy, dx;
-            tv.tap(static_cast<uint32_t>(k_ok ? kk : 0), ch_off, dy, dx);
+            const int2 t = tab[r_p[p]];
+            const int32_t ch_off = ch_p[p];
+            const int dy = t.x, dx = t.y;
+            kk_p[p] = kk + BK;
+            const int r = r_p[p] + step_r;
+            const bool carry = r >= window;
+            r_p[p] = carry ? r - window : r;
+            ch_p[p] += carry ? step_ch + tv.s_ch : step_ch;
             const int y = STRIDE * py + dy, x0 = STRIDE * px0 + dx;
             const bool row_ok = n_ok && k_ok && static_cast<unsigned>(y) < static_cast<unsigned>(tv.src_h);
             const int32_t e0 = ch_off + y * tv.s_h + x0;
@@ -418,6 +460,7 @@ struct TapStagerKC : TileLayout<T, ROWS, BK, true> {
     static constexpr int P = ROWS / RPP;
     static_assert(VEC > 1 && BK % VEC == 0 && kThreads % VPL == 0 && ROWS % RPP == 0, "tile must split evenly");
     static constexpr int kPF = PF;
+    static constexpr bool kTapTable = false;
     V reg[PF][P];
     int col0[PF];  // source column of the lane's first position, before the tap's dx
     __amdgpu_buffer_rsrc_t rsrc;
@@ -511,6 +554,7 @@ struct PaddedRowsStager : TileLayout<T, ROWS, BK, true> {
     static constexpr int VEC = Mfma<T>::VK;
     using V = typename Vec<T, VEC>::type;
     static constexpr int kPF = PF;
+    static constexpr bool kTapTable = false;
     static constexpr int VPL = BK / VEC;
     static constexpr int RPP = kThreads / VPL;  // rows per pass
     static constexpr int P = ROWS / RPP;
@@ -662,6 +706,10 @@ conv_fwd_kernel(ConvGeom geo, const T *x, const T *w, const T *bias, T *out, int
     const int M_ = geo.O, N_ = geo.Ho * geo.Wo, K = geo.C * geo.k * geo.k;
     StA sa;
     StB sb(geo);
+    if constexpr (StB::kTapTable) {  // the window's (dy, dx) table, behind the tile buffers
+        sb.fill_tap_table(reinterpret_cast<int2 *>(smem_raw + Engine::kLdsBytes), tid);
+        __syncthreads();
+    }
     sa.init(w + static_cast<int64_t>(m0) * geo.w_so, tid, M_ - m0, geo.w_so, 1, K);
     sb.init(x + static_cast<int64_t>(b) * geo.xs_b, image_bytes, tid, n0);
     Engine eng;
@@ -754,6 +802,10 @@ conv_dgrad_kernel(ConvGeom geo, const T *gout, const T *wt, T *gin, int tiles_m,
     const int64_t g_image = static_cast<int64_t>(geo.O) * geo.Ho * geo.Wo;
     StA sa;
     StB sb(geo);
+    if constexpr (StB::kTapTable) {
+        sb.fill_tap_table(reinterpret_cast<int2 *>(smem_raw + Engine::kLdsBytes), tid);
+        __syncthreads();
+    }
     sa.init(wt + static_cast<int64_t>(m0) * K, tid, M_ - m0, K, 1, K);
     sb.init(gout + static_cast<int64_t>(b) * g_image, g_image * static_cast<int64_t>(sizeof(T)), tid, n0);
     Engine eng;
@@ -799,6 +851,10 @@ conv_dgrad_classes_kernel(DgradClassGeoms tab, const T *gout, const T *wt, T *gi
     const int64_t g_image = static_cast<int64_t>(geo.O) * geo.Ho * geo.Wo;
     StA sa;
     StB sb(geo);
+    if constexpr (StB::kTapTable) {
+        sb.fill_tap_table(reinterpret_cast<int2 *>(smem_raw + Engine::kLdsBytes), tid);
+        __syncthreads();
+    }
     sa.init(wt + tab.wt_off[ci] + static_cast<int64_t>(m0) * K, tid, M_ - m0, K, 1, K);
     sb.init(gout + static_cast<int64_t>(b) * g_image, g_image * static_cast<int64_t>(sizeof(T)), tid, n0);
     Engine eng;
@@ -1265,7 +1321,7 @@ ttamd_status launch_conv(Kernel kernel, size_t lds, int64_t blocks, hipStream_t 
 template <typename T, int BM, int BN, int A_VEC, class StB>
 constexpr size_t conv_lds_bytes() {
     constexpr int BK = ConvTiles<T>::BK;
-    return ConvEngine<T, BM, BN, BK, Stager<T, BM, BK, true, A_VEC, kConvPF>, StB>::kLdsBytes;
+    return ConvEngine<T, BM, BN, BK, Stager<T, BM, BK, true, A_VEC, kConvPF>, StB>::kLdsBytes + (StB::kTapTable ? kTapTableBytes : 0);
 }
 
 // Rows of `width` positions that are no whole number of 16-byte vectors: the padded row width with which the
@@ -1285,14 +1341,15 @@ ttamd_status forward_mfma_tile(const ConvPlan &pl, const void *bias, void *out, 
     ConvGeom g = pl.geo;
     const bool a_vec = rows_vectorizable<T>(pl.w, g.w_so, 0);
     const bool stride_two = g.S == 2 && strided_vector_gather_enabled();
-    if (a_vec && (g.S == 1 || stride_two) && g.xs_w == 1) {
+    const bool table_ok = g.k * g.k <= kTapTableEntries;  // (the vector gathers read a window's taps from a table in LDS)
+    if (a_vec && table_ok && (g.S == 1 || stride_two) && g.xs_w == 1) {
         g.row_pad = padded_row_width(sizeof(T), g.Wo);
         g.d_row_pad = make_fastdiv(static_cast<uint32_t>(g.row_pad ? g.row_pad : 1));
     }
     const int M_ = g.O, N_ = g.Ho * (g.row_pad ? g.row_pad : g.Wo);
     const int tiles_m = (M_ + BM - 1) / BM, tiles_n = (N_ + BN - 1) / BN;
     const int64_t blocks = static_cast<int64_t>(tiles_m) * tiles_n * g.B;
-    const bool b_vec = g.S == 1 && g.xs_w == 1 && (g.row_pad || g.Wo % VK == 0);
+    const bool b_vec = table_ok && g.S == 1 && g.xs_w == 1 && (g.row_pad || g.Wo % VK == 0);
     auto go = [&](auto kernel, size_t lds) {
         return launch_conv(kernel, lds, blocks, st, g, static_cast<const T *>(pl.x), static_cast<const T *>(pl.w),
                            static_cast<const T *>(bias), static_cast<T *>(out), pl.image_bytes, tiles_m, tiles_n);
@@ -1301,14 +1358,14 @@ ttamd_status forward_mfma_tile(const ConvPlan &pl, const void *bias, void *out, 
     using OneB = Im2colStager<T, BN, BK, kConvPF>;
     if (a_vec && b_vec) return go(conv_fwd_kernel<T, BM, BN, BK, VK, VecB>, conv_lds_bytes<T, BM, BN, VK, VecB>());
     // stride 2 on dense rows with output rows of whole vectors: two 16-byte gathers per vector of positions
-    if (a_vec && stride_two && g.xs_w == 1 && (g.row_pad || g.Wo % VK == 0)) {
+    if (a_vec && table_ok && stride_two && g.xs_w == 1 && (g.row_pad || g.Wo % VK == 0)) {
         using Vec2B = TapStagerMC<T, BN, BK, VK, false, kConvPF, 2>;
         t_last_kernel[0] = 0x102;
         return go(conv_fwd_kernel<T, BM, BN, BK, VK, Vec2B>, conv_lds_bytes<T, BM, BN, VK, Vec2B>());
     }
     if constexpr (sizeof(T) == 4) {  // rows of 2n elements: 8-byte gathers
         using PairB = TapStagerMC<T, BN, BK, 2, false, kConvPF>;
-        if (a_vec && g.S == 1 && g.xs_w == 1 && g.Wo % 2 == 0)
+        if (a_vec && table_ok && g.S == 1 && g.xs_w == 1 && g.Wo % 2 == 0)
             return go(conv_fwd_kernel<T, BM, BN, BK, VK, PairB>, conv_lds_bytes<T, BM, BN, VK, PairB>());
     }
     if (a_vec) return go(conv_fwd_kernel<T, BM, BN, BK, VK, OneB>, conv_lds_bytes<T, BM, BN, VK, OneB>());
@@ -1601,14 +1658,15 @@ ttamd_status backward_mfma(const ConvPlan &pl, const void *gout, void *gin, void
             const T *wt = wts;
             T *gin = dst;
             const bool a_vec = rows_vectorizable<T>(wt, Kd, 0);
-            if (a_vec && g.S == 1) {
+            const bool table_ok = g.kh * g.kw <= kTapTableEntries;
+            if (a_vec && table_ok && g.S == 1) {
                 g.row_pad = padded_row_width(sizeof(T), g.W);
                 g.d_row_pad = make_fastdiv(static_cast<uint32_t>(g.row_pad ? g.row_pad : 1));
             }
             const int M_ = g.C, N_ = g.H * (g.row_pad ? g.row_pad : g.W);
             const int tiles_m = (M_ + BM - 1) / BM, tiles_n = (N_ + BN - 1) / BN;
             const int64_t blocks = static_cast<int64_t>(tiles_m) * tiles_n * g.B;
-            const bool b_vec = g.S == 1 && (g.row_pad || g.W % VK == 0);
+            const bool b_vec = table_ok && g.S == 1 && (g.row_pad || g.W % VK == 0);
             auto go = [&](auto kernel, size_t lds) {
                 return launch_conv(kernel, lds, blocks, st, g, static_cast<const T *>(gout), static_cast<const T *>(wt),
                                    static_cast<T *>(gin), tiles_m, tiles_n);
@@ -1618,7 +1676,7 @@ ttamd_status backward_mfma(const ConvPlan &pl, const void *gout, void *gin, void
             if (a_vec && b_vec) return go(conv_dgrad_kernel<T, BM, BN, BK, VK, VecB, SC>, conv_lds_bytes<T, BM, BN, VK, VecB>());
             if constexpr (sizeof(T) == 4) {
                 using PairB = TapStagerMC<T, BN, BK, 2, true, kConvPF>;
-                if (a_vec && g.S == 1 && g.W % 2 == 0)
+                if (a_vec && table_ok && g.S == 1 && g.W % 2 == 0)
                     return go(conv_dgrad_kernel<T, BM, BN, BK, VK, PairB, SC>, conv_lds_bytes<T, BM, BN, VK, PairB>());
             }
             if (a_vec) return go(conv_dgrad_kernel<T, BM, BN, BK, VK, OneB, SC>, conv_lds_bytes<T, BM, BN, VK, OneB>());
@@ -1681,7 +1739,7 @@ ttamd_status backward_mfma(const ConvPlan &pl, const void *gout, void *gin, void
                     const int Kd = gc.O * gc.kh * gc.kw;
                     gc.row_pad = padded_row_width(sizeof(T), gc.W);
                     gc.d_row_pad = make_fastdiv(static_cast<uint32_t>(gc.row_pad ? gc.row_pad : 1));
-                    ok = rows_vectorizable<T>(wt + cl.wt_off, Kd, 0) && (gc.row_pad || gc.W % VK == 0);
+                    ok = rows_vectorizable<T>(wt + cl.wt_off, Kd, 0) && (gc.row_pad || gc.W % VK == 0) && gc.kh * gc.kw <= kTapTableEntries;
                     const int N_ = gc.H * (gc.row_pad ? gc.row_pad : gc.W);
                     const int i = tab.n++;
                     tab.geo[i] = gc;
