@@ -267,6 +267,32 @@ def test_grad_weight_with_sets_of_waves_exact(tt, oracle, geom):
     assert np.array_equal(gx.to_numpy(), wx) and np.array_equal(gb.to_numpy(), wb)
 
 
+def test_twelve_wave_and_sets_kernels_on_an_input_window(tt, oracle):
+    """Benchmark configuration 4 with the input as a window of a larger, NaN-filled tensor (row stride 32, a channel more,
+    two rows more, 16-byte aligned start): the twelve-wave forward and grad_input kernels and grad_weight's sets of waves
+    read it through its strides."""
+    rng = np.random.default_rng(404)
+    Bn, Cc, O, H, W = 64, 32, 64, 28, 28
+    big = np.full((Bn, Cc + 1, H + 2, W + 4), np.nan, np.float32)
+    x = rng.integers(-3, 4, (Bn, Cc, H, W)).astype(np.float32)
+    big[:, 1:, 1:1 + H, 4:] = x
+    w = rng.integers(-3, 4, (O, Cc, 3, 3)).astype(np.float32)
+    b = rng.integers(-3, 4, (O,)).astype(np.float32)
+    tb = dev(tt, big)
+    es = [v // 4 for v in big.strides]
+    tx = tt.Tensor(tb.storage, tb.dtype, (Bn, Cc, H, W), tuple(es), es[1] + es[2] + 4)
+    assert not tx.is_contiguous()
+    out = tt.conv2d(tx, dev(tt, w), dev(tt, b), 1, 1).to_numpy()
+    assert _last_kernel(0) == 0x200 + 12 * 16 + 1, hex(_last_kernel(0))
+    want = oracle.conv2d_forward(x, w, b, 1, 1)
+    assert np.array_equal(out, want)
+    g = rng.integers(-3, 4, want.shape).astype(np.float32)
+    gx, gw, gb = tt.conv2d_backward(dev(tt, g), tx, dev(tt, w), dev(tt, b), 1, 1)
+    assert _last_kernel(1) == 0x200 + 12 * 16 + 1 and _last_kernel(2) == 0x200, (hex(_last_kernel(1)), hex(_last_kernel(2)))
+    wx, ww, wb = oracle.conv2d_backward(g, x, w, True, 1, 1)
+    assert np.array_equal(gx.to_numpy(), wx) and np.array_equal(gw.to_numpy(), ww) and np.array_equal(gb.to_numpy(), wb)
+
+
 def test_lds_resident_kernel_on_views(tt, oracle):
     # an input window of a larger tensor (row stride 16, 16-byte aligned start) and, through the C ABI, a weight whose
     # output-channel stride is larger than C k k (the row-wise weight loads)
