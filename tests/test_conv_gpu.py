@@ -401,6 +401,35 @@ def test_padding_columns_of_padded_rows_carry_nothing(tt, oracle, dtype, W):
     assert np.array_equal(gw.to_numpy(), ww) and np.array_equal(gx.to_numpy(), wx)
 
 
+def test_infinite_values_reach_exactly_their_windows_in_the_lds_staged_kernels(tt, oracle):
+    """Benchmark configuration 4's geometry, whose forward and grad_input tiles end in a tail of four positions computed
+    apart and whose grad_weight stages end in a chunk that is half empty: positions beyond a tile, a tail or a stage are
+    read at stand-in cells.  Infinite input / gradient values at the last positions of tiles, stages and images must
+    come out as the reference's infinities (and its NaNs, where it has them) and nowhere else."""
+    rng = np.random.default_rng(11)
+    Bn, Cc, O, H, W = 64, 32, 64, 28, 28
+    x = rng.integers(0, 3, (Bn, Cc, H, W)).astype(np.float32)
+    w = rng.integers(1, 3, (O, Cc, 3, 3)).astype(np.float32)
+    for (b, c, y, xx) in ((0, 0, 6, 27), (1, 5, 7, 0), (2, 31, 27, 27), (3, 7, 13, 27), (63, 16, 27, 24)):
+        x[b, c, y, xx] = np.inf
+    out = tt.conv2d(dev(tt, x), dev(tt, w), None, 1, 1).to_numpy()
+    assert _last_kernel(0) == 0x200 + 12 * 16 + 1
+    want = oracle.conv2d_forward(x, w, None, 1, 1)
+    assert np.isinf(want).any() and not np.isnan(want).any()
+    assert np.array_equal(out, want)
+    g = rng.integers(1, 3, want.shape).astype(np.float32)
+    for (b, o, y, xx) in ((0, 0, 6, 27), (5, 63, 27, 27), (9, 31, 13, 24), (63, 32, 14, 0)):
+        g[b, o, y, xx] = np.inf
+    x2 = rng.integers(1, 3, x.shape).astype(np.float32)   # (finite and positive: no inf - inf)
+    gx, gw, _ = tt.conv2d_backward(dev(tt, g), dev(tt, x2), dev(tt, w), None, 1, 1)
+    assert _last_kernel(1) == 0x200 + 12 * 16 + 1 and _last_kernel(2) == 0x200
+    wx, ww, _ = oracle.conv2d_backward(g, x2, w, False, 1, 1)
+    # (the reference's im2col holds real zeros where a window reaches into the padding: an infinite gradient at the image's
+    # edge times such a zero is a NaN in its grad_weight -- in those taps and no others)
+    assert np.isinf(wx).any() and not np.isnan(wx).any() and np.isnan(ww).any() and np.isinf(ww).any()
+    assert np.array_equal(gx.to_numpy(), wx) and np.array_equal(gw.to_numpy(), ww, equal_nan=True)
+
+
 @pytest.mark.parametrize("dtype", [np.float32, np.float64])
 def test_unaligned_window_of_a_larger_image(tt, oracle, dtype):
     # the input is a window [1:9, 3:15] of a stored [2,3,10,20] tensor: rows start at odd element offsets,
