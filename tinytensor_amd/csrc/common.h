@@ -139,7 +139,15 @@ struct ConvPatchArgs {
     int w_flip;            // taps used in reverse order (gradient with respect to the input)
     int w_rows_fast;       // lanes of the weight loader run along the rows (the axis whose stride is k*k) instead of the channels
     int64_t image_bytes, weight_bytes;  // bytes reachable from an image's / the weight's first element
+    // Optional second job of the launch: red_out[i] = sum over s < red_splits of red_partial[s * red_n + i], carried out by
+    // workgroups appended to the grid (a sum that some earlier launch on the stream left in parts, e.g. grad_weight's partial
+    // tiles, spared a launch of its own).  red_n a multiple of 4, both pointers 16-byte aligned, red_splits * red_n * 4 < 2^31;
+    // red_splits == 0: none.
+    const float *red_partial;
+    float *red_out;
+    int red_n, red_splits;
     // derived
+    int red_blocks;
     int K, lda, cpad, R, pitch, vecs_per_row, xh, last_vecs, n_items, stage_slots, cl_shift, tiles_m, tiles_n;
     int n_seg, seg_len, segs_per_pass, n_fast, n_wvec, w_dense, w_pass_vecs, n_buf;
     int bne, tail;  // positions per tile; those of them behind the tile's whole 32-position blocks (twelve waves: 4 or 8)

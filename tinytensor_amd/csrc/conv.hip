@@ -1264,7 +1264,7 @@ ttamd_status set_lds(Kernel kernel, size_t lds_bytes) {
 // Which kernel family the calling thread's last forward ([0]), grad_input ([1]) and grad_weight ([2]) launches took: 0x100 the
 // implicit-GEMM kernels of this file, 0x200 + 16 * waves + patch buffers the persistent kernel of conv_patch.hip,
 // 0 anything else.  Read through ttamd_conv2d_last_kernel by the tests that mean to cover a particular kernel.
-thread_local int t_last_kernel[3] = {0, 0, 0};
+thread_local int t_last_kernel[4] = {0, 0, 0, 0};
 
 // TTAMD_CONV_PATCH=0 keeps every convolution on the implicit-GEMM kernels of this file (for comparisons).
 inline bool patch_kernel_enabled() {
@@ -1614,6 +1614,29 @@ ttamd_status backward_mfma(const ConvPlan &pl, const void *gout, void *gin, void
     }
     T *const wt = static_cast<T *>(ws);
     T *const partials = reinterpret_cast<T *>(static_cast<char *>(ws) + plan.wt_bytes);
+    // grad_weight by the LDS-staged kernel goes first where it applies: the sum over its partial tiles can then ride in
+    // grad_input's launch (ConvPatchArgs::red_*) instead of one of its own.
+    bool wgrad_staged = false;
+    int parts_to_add = 0;  // partial tiles of grad_weight that still wait to be added up
+    t_last_kernel[3] = 0;
+    const int64_t gw_elems = static_cast<int64_t>(g.O) * g.C * g.k * g.k;
+    if constexpr (std::is_same_v<T, float>) {
+        // unit stride, channel counts that are multiples of 32, rows of whole vectors: both operands staged in LDS
+        if (g.xs_w == 1 && patch_kernel_enabled()) {
+            const ConvWgradPatchPlan pp = plan_conv_wgrad_patch(g.B, g.C, g.H, g.W, g.O, g.k, g.S, g.P);
+            if (pp.use) {
+                ConvWgradPatchArgs a{};
+                a.gout = static_cast<const float *>(gout);
+                a.x = static_cast<const float *>(pl.x);
+                a.partial = pp.workgroups > 1 ? partials : static_cast<float *>(gw);
+                a.B = g.B; a.C = g.C; a.H = g.H; a.W = g.W; a.O = g.O; a.k = g.k; a.P = g.P; a.Ho = g.Ho; a.Wo = g.Wo;
+                a.xs_b = g.xs_b; a.xs_c = g.xs_c; a.xs_h = g.xs_h;
+                a.image_bytes = pl.image_bytes;
+                if (ttamd_status rc = launch_conv_wgrad_patch_f32(a, pp, st, &wgrad_staged)) return rc;
+                if (wgrad_staged && pp.workgroups > 1) parts_to_add = pp.workgroups;
+            }
+        }
+    }
     // grad_input
     t_last_kernel[1] = 0;
     const int np = (g.k + g.S - 1) / g.S;
@@ -1801,10 +1824,19 @@ ttamd_status backward_mfma(const ConvPlan &pl, const void *gout, void *gin, void
                     a.w_row = static_cast<int64_t>(g.k) * g.k; a.w_red = g.w_so; a.w_flip = 1; a.w_rows_fast = 1;
                     a.image_bytes = static_cast<int64_t>(g.O) * HoWo * 4;
                     a.weight_bytes = pl.weight_bytes;
+                    const bool rides = parts_to_add > 0 && gw_elems % 4 == 0 && reinterpret_cast<uintptr_t>(gw) % 16 == 0 &&
+                                       reinterpret_cast<uintptr_t>(partials) % 16 == 0 && parts_to_add * gw_elems * 4 < 0x7fffffffLL;
+                    if (rides) {
+                        a.red_partial = partials;
+                        a.red_out = static_cast<float *>(gw);
+                        a.red_n = static_cast<int>(gw_elems);
+                        a.red_splits = parts_to_add;
+                    }
                     int variant = 0;
                     if (ttamd_status rc = launch_conv_patch_f32(a, st, &variant)) return rc;
                     handled = variant != 0;
                     if (handled) t_last_kernel[1] = 0x200 + variant;
+                    if (handled && rides) parts_to_add = 0, t_last_kernel[3] = 2;
                 }
             }
             if (!handled) {
@@ -1815,29 +1847,15 @@ ttamd_status backward_mfma(const ConvPlan &pl, const void *gout, void *gin, void
             }
         }
     }
+    if (parts_to_add > 0) {
+        if (ttamd_status rc = launch_reduce_splits<T>(partials, static_cast<T *>(gw), gw_elems, parts_to_add, st)) return rc;
+        t_last_kernel[3] = 1;
+    }
     // grad_weight
     {
         const int M_ = g.O, N_ = g.C * g.k * g.k;
         const int64_t tile_elems = static_cast<int64_t>(M_) * N_;
-        bool staged = false;
-        if constexpr (std::is_same_v<T, float>) {
-            // unit stride, channel counts that are multiples of 32, rows of whole vectors: both operands staged in LDS
-            if (g.xs_w == 1 && patch_kernel_enabled()) {
-                const ConvWgradPatchPlan pp = plan_conv_wgrad_patch(g.B, g.C, g.H, g.W, g.O, g.k, g.S, g.P);
-                if (pp.use) {
-                    ConvWgradPatchArgs a{};
-                    a.gout = static_cast<const float *>(gout);
-                    a.x = static_cast<const float *>(pl.x);
-                    a.partial = pp.workgroups > 1 ? partials : static_cast<float *>(gw);
-                    a.B = g.B; a.C = g.C; a.H = g.H; a.W = g.W; a.O = g.O; a.k = g.k; a.P = g.P; a.Ho = g.Ho; a.Wo = g.Wo;
-                    a.xs_b = g.xs_b; a.xs_c = g.xs_c; a.xs_h = g.xs_h;
-                    a.image_bytes = pl.image_bytes;
-                    if (ttamd_status rc = launch_conv_wgrad_patch_f32(a, pp, st, &staged)) return rc;
-                    if (staged && pp.workgroups > 1)
-                        if (ttamd_status rc = launch_reduce_splits<T>(partials, static_cast<T *>(gw), tile_elems, pp.workgroups, st)) return rc;
-                }
-            }
-        }
+        const bool staged = wgrad_staged;
         t_last_kernel[2] = staged ? 0x200 : 0x100;
         if (!staged) {
         const int parts = plan.parts();
@@ -1911,7 +1929,7 @@ using namespace ttamd;
 
 extern "C" {
 
-int ttamd_conv2d_last_kernel(int which) { return which >= 0 && which <= 2 ? ttamd::t_last_kernel[which] : 0; }
+int ttamd_conv2d_last_kernel(int which) { return which >= 0 && which <= 3 ? ttamd::t_last_kernel[which] : 0; }
 
 ttamd_status ttamd_conv2d_forward(int device, ttamd_dtype dtype, const ttamd_view4 *input, const ttamd_view4 *weight,
                                   const void *bias, void *out, int B, int C, int H, int W, int O, int k, int stride,

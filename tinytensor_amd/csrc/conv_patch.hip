@@ -57,6 +57,40 @@ constexpr int tail_accumulators() {
     return WGM >= 2 ? 2 : 1;
 }
 
+// The launch's second job (ConvPatchArgs::red_*): workgroup r of the appended ones owns the 16-byte vectors 64 r .. 64 r + 63
+// of the result; each of its NW waves adds a contiguous share of the parts in increasing order, every load in flight
+// together (parts beyond the share arrive as +0 from the buffer load, which changes no sum that started at +0), and the
+// waves' sums are added in wave order.
+template <int NW>
+__device__ __forceinline__ void add_up_parts(const ConvPatchArgs &a, int r, float *lds) {
+    const int lane = threadIdx.x % 64;
+    const int w = __builtin_amdgcn_readfirstlane(threadIdx.x / 64);
+    const int v = r * 64 + lane;
+    const bool ok = 4 * v < a.red_n;
+    const int per = (a.red_splits + NW - 1) / NW;
+    const int s0 = w * per, s1 = s0 + per < a.red_splits ? s0 + per : a.red_splits;
+    const __amdgpu_buffer_rsrc_t src = make_rsrc(a.red_partial, static_cast<int64_t>(a.red_splits) * a.red_n * 4);
+    const uint32_t voff = ok ? static_cast<uint32_t>(v) * 16u : kOob;
+    f32x4 acc = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll 1
+    for (int s = s0; s < s1; s += 16) {
+        f32x4 part[16];
+#pragma unroll
+        for (int u = 0; u < 16; ++u)
+            part[u] = Vec<float, 4>::load_at(src, s + u < s1 ? voff : kOob, static_cast<uint32_t>(s + u) * static_cast<uint32_t>(a.red_n) * 4u);
+#pragma unroll
+        for (int u = 0; u < 16; ++u) acc += part[u];
+    }
+    *reinterpret_cast<f32x4 *>(lds + (w * 64 + lane) * 4) = acc;
+    __syncthreads();
+    if (w == 0 && ok) {
+        f32x4 sum = acc;
+#pragma unroll
+        for (int k = 1; k < NW; ++k) sum += *reinterpret_cast<const f32x4 *>(lds + (k * 64 + lane) * 4);
+        *reinterpret_cast<f32x4 *>(a.red_out + 4 * static_cast<int64_t>(v)) = sum;
+    }
+}
+
 // WGM x WGN waves of one 32 x 32 MFMA block each: output tile (32 WGM) channels x (32 WGN) positions.
 // CC: chunks of 8 reduction indices (8 channels of one tap) that are read and multiplied as one straight-line group;
 // C / 8 is a multiple of it.
@@ -76,6 +110,11 @@ __global__ void __launch_bounds__(64 * WGM * WGN * KS, 1) conv_patch_kernel(Conv
     constexpr int BM = 32 * WGM, BN = 32 * WGN;
     const int bne = kTail ? a.bne : BN;  // positions per tile
     extern __shared__ __attribute__((aligned(16))) float smem_patch[];
+    const int conv_blocks = static_cast<int>(gridDim.x) - a.red_blocks;
+    if (static_cast<int>(blockIdx.x) >= conv_blocks) {  // an appended workgroup: the launch's second job
+        add_up_parts<NW>(a, static_cast<int>(blockIdx.x) - conv_blocks, smem_patch);
+        return;
+    }
     float *const A = smem_patch;                   // [BM][lda], k' = tap * C + c
     float *const patch = smem_patch + BM * a.lda;  // [1 or 2][R][pitch][cpad]
     const int tid = threadIdx.x, lane = tid % 64;
@@ -87,7 +126,7 @@ __global__ void __launch_bounds__(64 * WGM * WGN * KS, 1) conv_patch_kernel(Conv
     const int patch_elems = a.R * pitch * cpad;
 
     // which tiles: workgroup (m, gi) of `groups` per output-channel block walks j = gi, gi + groups, ...
-    const int groups = gridDim.x / a.tiles_m;
+    const int groups = conv_blocks / a.tiles_m;
     const int mblk = blockIdx.x % a.tiles_m, gi = blockIdx.x / a.tiles_m;
     const int m0 = mblk * BM;
     const int n_tiles = a.B * a.tiles_n;
@@ -401,11 +440,11 @@ __global__ void __launch_bounds__(64 * WGM * WGN * KS, 1) conv_patch_kernel(Conv
             }
             // The patch has been read: its memory takes the upper set's accumulators and the waves' tails.
             __syncthreads();
-            float *const exch = patch + cur * patch_elems + (wtile * 64 + lane) * 16;
+            float *const exch = patch + cur * patch_elems + wtile * 1024 + lane * 4;  // [wave][e / 4][lane][4]: consecutive lanes, consecutive vectors
             float *const tails = patch + cur * patch_elems + (KS == 2 ? WGM * WGN * 64 * 16 : 0);  // [NW][NTA][64 lanes][4]
             if (KS == 2 && ks == 1) {
 #pragma unroll
-                for (int e = 0; e < 16; e += 4) *reinterpret_cast<f32x4 *>(exch + e) = f32x4{acc[e], acc[e + 1], acc[e + 2], acc[e + 3]};
+                for (int e = 0; e < 16; e += 4) *reinterpret_cast<f32x4 *>(exch + e * 64) = f32x4{acc[e], acc[e + 1], acc[e + 2], acc[e + 3]};
             }
             if (a.tail > 0) {
 #pragma unroll
@@ -415,7 +454,7 @@ __global__ void __launch_bounds__(64 * WGM * WGN * KS, 1) conv_patch_kernel(Conv
             if (KS == 2 && ks == 0) {  // (lower half of the groups) + (upper half): a fixed order
 #pragma unroll
                 for (int e = 0; e < 16; e += 4) {
-                    const f32x4 v = *reinterpret_cast<const f32x4 *>(exch + e);
+                    const f32x4 v = *reinterpret_cast<const f32x4 *>(exch + e * 64);
 #pragma unroll
                     for (int t = 0; t < 4; ++t) acc[e + t] += v[t];
                 }
@@ -436,16 +475,16 @@ __global__ void __launch_bounds__(64 * WGM * WGN * KS, 1) conv_patch_kernel(Conv
         } else if constexpr (KS == 2) {
             // the upper set's sums go to the lower set through LDS (behind the patch buffers), added as
             // (lower half of the groups) + (upper half): a fixed order
-            float *const exch = patch + a.n_buf * patch_elems + (wtile * 64 + lane) * 16;
+            float *const exch = patch + a.n_buf * patch_elems + wtile * 1024 + lane * 4;  // [wave][e / 4][lane][4]
             if (ks == 1) {
 #pragma unroll
-                for (int e = 0; e < 16; e += 4) *reinterpret_cast<f32x4 *>(exch + e) = f32x4{acc[e], acc[e + 1], acc[e + 2], acc[e + 3]};
+                for (int e = 0; e < 16; e += 4) *reinterpret_cast<f32x4 *>(exch + e * 64) = f32x4{acc[e], acc[e + 1], acc[e + 2], acc[e + 3]};
             }
             __syncthreads();  // (also: every wave has left the patch buffer)
             if (ks == 0) {
 #pragma unroll
                 for (int e = 0; e < 16; e += 4) {
-                    const f32x4 v = *reinterpret_cast<const f32x4 *>(exch + e);
+                    const f32x4 v = *reinterpret_cast<const f32x4 *>(exch + e * 64);
 #pragma unroll
                     for (int t = 0; t < 4; ++t) acc[e + t] += v[t];
                 }
@@ -556,7 +595,9 @@ ttamd_status launch_patch(ConvPatchArgs a, hipStream_t st, size_t lds) {
     a.d_ngrp = make_fastdiv(static_cast<uint32_t>(a.C / (8 * CC)));
     auto kernel = conv_patch_kernel<WGM, WGN, CC, MAXS, KS>;
     TTAMD_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds)));
-    kernel<<<dim3(static_cast<unsigned>(groups * a.tiles_m)), dim3(64 * WGM * WGN * KS), lds, st>>>(a);
+    a.red_blocks = a.red_splits > 0 ? (a.red_n / 4 + 63) / 64 : 0;
+    if (lds < static_cast<size_t>(64 * WGM * WGN * KS) * 16) lds = static_cast<size_t>(64 * WGM * WGN * KS) * 16;  // (the second job's sums)
+    kernel<<<dim3(static_cast<unsigned>(groups * a.tiles_m + a.red_blocks)), dim3(64 * WGM * WGN * KS), lds, st>>>(a);
     TTAMD_HIP_CHECK(hipGetLastError());
     return TTAMD_OK;
 }
