@@ -231,23 +231,35 @@ __global__ void __launch_bounds__(64 * WGM * WGN * KS, 1) conv_patch_kernel(Conv
         for (int v = tid; v < n_pairs; v += kPairs * NT) {
             float *dst[kPairs];
             float taps[kPairs][9];
+            bool have[kPairs];
 #pragma unroll
             for (int i = 0; i < kPairs; ++i) {
-                const int vv = v + i * NT < n_pairs ? v + i * NT : v;  // (beyond the end: the first one again)
-                uint32_t slow, fast;
-                a.d_wfast.divmod(static_cast<uint32_t>(vv), slow, fast);
-                const int row = a.w_rows_fast ? static_cast<int>(fast) : static_cast<int>(slow);
-                const int red = a.w_rows_fast ? static_cast<int>(slow) : static_cast<int>(fast);
+                have[i] = v + i * NT < n_pairs;
+                const uint32_t vv = static_cast<uint32_t>(v + i * NT);
+                int row, red;
+                if (a.w_rows_fast) {
+                    // 16 rows x 4 reduction channels per wave: the loads cover four stretches of 16 x 9 floats, and the
+                    // stores -- rows 4 (2 n + 1) floats apart, channels one float apart -- every bank once
+                    const uint32_t t = vv >> 6;
+                    row = static_cast<int>((t % (BM / 16)) * 16 + (vv & 15));
+                    red = static_cast<int>((t / (BM / 16)) * 4 + ((vv >> 4) & 3));
+                } else {
+                    uint32_t slow, fast;
+                    a.d_wfast.divmod(vv, slow, fast);
+                    row = static_cast<int>(slow), red = static_cast<int>(fast);
+                }
                 // rows beyond the last output channel are requested out of range and arrive as zeros
-                const uint32_t off = m0 + row < a.O ? static_cast<uint32_t>((m0 + row) * a.w_row + red * a.w_red) * 4u : kOob;
+                const uint32_t off = have[i] && m0 + row < a.O ? static_cast<uint32_t>((m0 + row) * a.w_row + red * a.w_red) * 4u : kOob;
                 dst[i] = A + row * a.lda + red + (a.w_flip ? 8 * C : 0);
 #pragma unroll
                 for (int u = 0; u < 9; ++u) taps[i][u] = Vec<float, 1>::load(wsrc, off + 4u * u);
             }
 #pragma unroll
             for (int i = 0; i < kPairs; ++i)
+                if (have[i]) {
 #pragma unroll
-                for (int u = 0; u < 9; ++u) dst[i][u * step] = taps[i][u];
+                    for (int u = 0; u < 9; ++u) dst[i][u * step] = taps[i][u];
+                }
         }
     } else {
         const int k2 = a.k * a.k;

@@ -61,7 +61,8 @@ ttamd_status fixed_scratch_address(int device, void **out) {
 // walks in one kernel the register allocator spills accumulators ahead of the branch for the sake of the heaviest
 // walk, and the plain store pays for it.
 constexpr int kEpiAny = 0, kEpiLean = 1, kEpiFull = 2, kEpiExt = 3;
-// kEpiLean for a problem made of whole tiles (M, N, K multiples of BM, BN, BK): no masked loop in the kernel, whose
+// kEpiLean for a problem of whole k tiles and whole vectors along m and n (K a multiple of BK; M, N multiples of the
+// vector length of an operand that is contiguous along them): no masked loop in the kernel, whose
 // registers otherwise cost the plain kernel of the biggest tiles 228 bytes of scratch per lane.
 constexpr int kEpiLeanWhole = 4;
 
@@ -396,7 +397,9 @@ ttamd_status launch_variant(const GemmArgs &g, const SplitPlan &sp, int device, 
     // (fp32 256 x 256 only: the fp64 256 x 128 kernel has no scratch with its masked loop and 460 bytes without)
     constexpr bool kHasWhole = sizeof(T) == 4 && BM * BN >= 256 * 256 && A_VEC > 1 && B_VEC > 1;
     constexpr int kEpiD = kHasWhole ? kEpiLeanWhole : kEpiA;
-    const bool whole = kHasWhole && lean && sp.ksplit == 1 && g.M % BM == 0 && g.N % BN == 0 && g.K % BK == 0 && g.K > 0;
+    // (rows and columns outside the matrix need no masked loop: their loads carry out-of-range offsets either way; what
+    // needs it is a k tile that reaches past K, or a 16-byte vector along m or n that straddles the matrix's edge)
+    const bool whole = kHasWhole && lean && sp.ksplit == 1 && g.K % BK == 0 && g.K > 0 && (A_KC || g.M % A_VEC == 0) && (B_KC || g.N % B_VEC == 0);
     const int which = whole ? 3 : (lean ? 0 : (ext_store(g) ? 2 : 1));
     auto kernel = which == 0   ? gemm_mfma_kernel<T, BM, BN, BK, WGM, WGN, A_KC, A_VEC, B_KC, B_VEC, PF, kEpiA>
                   : which == 1 ? gemm_mfma_kernel<T, BM, BN, BK, WGM, WGN, A_KC, A_VEC, B_KC, B_VEC, PF, kEpiB>
