@@ -175,6 +175,24 @@ ttamd_status ttamd_batched_matmul(int device, ttamd_dtype dtype, int B, int N, i
                                   const ttamd_view3 *lhs, const ttamd_view3 *rhs, void *out,
                                   const ttamd_epilogue *epilogue, void *stream);
 
+/* Two independent products in one call: what TensorBatchedMatmul::backward (autograd/binary_ops.cpp:173-179) asks of
+ * the backend -- dA = dC . B^T and dB = A^T . dC, two batched_matmul calls on permuted views -- and nn::Linear's backward
+ * with it (nn/linear.cpp:42-50).  Each product has ttamd_batched_matmul's contract and gives the bits that call gives
+ * ... or, where the pair is launched as one grid, the bits of the same kernel family's plain 64 x 64 tile (every sum
+ * in k order, so equal to the separate calls' wherever those do not split the reduction).  Neither product may read
+ * the other's result.  One grid is launched when both are dense fp32 products of 128 to 256 tiles of 64 x 64 with a
+ * reduction of 512 or more, `first` in the layouts of dA (both operands contiguous along k), `second` in those of dB
+ * (left operand contiguous along its rows' index m, right operand along n); otherwise the two products run one after
+ * the other exactly as two ttamd_batched_matmul calls would. */
+typedef struct ttamd_product {
+    int B, N, K, M;
+    const ttamd_view3 *lhs, *rhs;
+    void *out;
+    const ttamd_epilogue *epilogue; /* may be NULL */
+} ttamd_product;
+ttamd_status ttamd_batched_matmul_pair(int device, ttamd_dtype dtype, const ttamd_product *first,
+                                       const ttamd_product *second, void *stream);
+
 /* ttamd_batched_matmul for callers that cannot allocate device memory (code under HIP graph capture, tight serving
  * loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  Same arguments, same kernels and
  * bit-identical results; the difference is where the partial tiles of a split reduction live: in a fixed 8 MiB

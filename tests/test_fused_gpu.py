@@ -331,6 +331,109 @@ def test_linear_mse_head_keeps_nan_under_the_mask_and_checks_arguments(tt):
         tt.linear_mse_head(d(x), d(w.astype(np.float64)), None, d(t), None)
 
 
+# (rows, in_features, out_features, one grid): the two gradients of a Linear layer as one call.  One grid when both products
+# are dense fp32 with 128 to 256 tiles of 64 x 64 and reductions of 512 or more; everything else runs as two calls.
+PAIR_SHAPES = [(1024, 1024, 1024, True), (1024, 784, 1024, True), (520, 1000, 640, True), (576, 900, 700, True),
+               (512, 1024, 1024, True), (1024, 2048, 520, True),
+               (256, 512, 384, False), (1024, 1024, 10, False), (300, 2000, 2000, False), (2048, 1024, 1024, False)]
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+@pytest.mark.parametrize("bias_grad", ["own", False, True])
+@pytest.mark.parametrize("shape", PAIR_SHAPES, ids=lambda s: "x".join(map(str, s[:3])))
+def test_linear_backward_pair_exact_on_integers(tt, dtype, bias_grad, shape):
+    """nn::Linear's backward (TensorBatchedMatmul::backward, autograd/binary_ops.cpp:173-179, with the ReLU mask of
+    unary_ops.cpp:568-573 and the bias gradient) through ttamd_batched_matmul_pair: integer-valued data, exact in any
+    order of summation, in the one-grid form and in the two-call form alike; grad_output's NaN under the mask stays."""
+    n, fin, fout, _ = shape
+    rng = np.random.default_rng(n + fin + fout)
+    dy = rng.integers(-3, 4, (n, fout)).astype(dtype)
+    x = rng.integers(-3, 4, (n, fin)).astype(dtype)
+    w = rng.integers(-3, 4, (fin, fout)).astype(dtype)
+    z = rng.integers(-2, 3, (n, fin)).astype(dtype)
+    tdy, tx, tw, tz = (tt.Tensor.from_numpy(v) for v in (dy, x, w, z))
+    dx, dW, db = tt.linear_backward(tdy, tx, tw, relu_input=tz, bias_grad=bias_grad)
+    want_dx = (dy.astype(np.float64) @ w.T.astype(np.float64)) * np.where(z < 0, 0.0, 1.0)
+    assert np.array_equal(dx.to_numpy(), want_dx.astype(dtype))
+    assert np.array_equal(dW.to_numpy(), (x.T.astype(np.float64) @ dy.astype(np.float64)).astype(dtype))
+    if bias_grad == "own":
+        assert np.array_equal(db.to_numpy(), dy.sum(0))
+    elif bias_grad:
+        assert np.array_equal(db.to_numpy(), want_dx.sum(0).astype(dtype))
+    else:
+        assert db is None
+    # without the mask, and a second call: the same bits
+    dx2, dW2, _ = tt.linear_backward(tdy, tx, tw, bias_grad=False)
+    assert np.array_equal(dx2.to_numpy(), (dy.astype(np.float64) @ w.T.astype(np.float64)).astype(dtype))
+    assert np.array_equal(dW2.to_numpy(), dW.to_numpy())
+
+
+@pytest.mark.parametrize("shape", [s for s in PAIR_SHAPES if s[3]][:4], ids=lambda s: "x".join(map(str, s[:3])))
+def test_batched_matmul_pair_on_real_data(tt, oracle, shape):
+    """Real-valued data in the one-grid form: each product within the bound of a k-ordered fp32 sum of the oracle's
+    product, the same bits on a second call, NaN and infinity kept where the reference's multiplication by the mask keeps
+    them, and the right operand's column sums equal to numpy's sum in float64 to rounding."""
+    n, fin, fout, _ = shape
+    rng = np.random.default_rng(n * 3 + fin + fout)
+    dy = rng.standard_normal((n, fout)).astype(np.float32)
+    x = rng.standard_normal((n, fin)).astype(np.float32)
+    w = rng.standard_normal((fin, fout)).astype(np.float32)
+    z = rng.standard_normal((n, fin)).astype(np.float32)
+    dy[3, 5] = np.inf
+    tdy, tx, tw, tz = (tt.Tensor.from_numpy(v) for v in (dy, x, w, z))
+    be = tt.get_backend(tt.kAMD)
+    db = tt.Tensor.empty((1, fout), tdy.dtype)
+    first = (tdy.unsqueeze(0), tw.unsqueeze(0).permute(0, 2, 1), dict(relu_grad_input=tz.unsqueeze(0)))
+    second = (tx.unsqueeze(0).permute(0, 2, 1), tdy.unsqueeze(0), dict(rhs_colsum_out=db))
+    dx, dW = (t.to_numpy()[0] for t in be.batched_matmul_pair(first, second))
+    dx_b, dW_b = (t.to_numpy()[0] for t in be.batched_matmul_pair(first, second))
+    assert np.array_equal(dx, dx_b, equal_nan=True) and np.array_equal(dW, dW_b, equal_nan=True)
+    fin_dy = np.where(np.isfinite(dy), dy, 0).astype(np.float32)
+    want_dx = oracle.matmul(fin_dy, np.ascontiguousarray(w.T), "fast") * np.where(z < 0, 0, 1).astype(np.float32)
+    want_dW = oracle.matmul(np.ascontiguousarray(x.T), fin_dy, "fast")
+    rows, cols = np.ones(n, bool), np.ones(fout, bool)
+    rows[3] = False
+    cols[5] = False
+    scale_dx = np.abs(fin_dy).astype(np.float64) @ np.abs(w.T).astype(np.float64)
+    scale_dW = np.abs(x.T).astype(np.float64) @ np.abs(fin_dy).astype(np.float64)
+    assert np.max(np.abs(dx[rows] - want_dx[rows]) / scale_dx[rows]) < 2e-6   # ~ 2^-19: fp32 sums of 520 to 1024 terms in another order
+    assert np.max(np.abs(dW[:, cols] - want_dW[:, cols]) / scale_dW[:, cols]) < 2e-6
+    # row 3 of dx holds inf . w = +-inf, times the mask: NaN under a 0, +-inf under a 1, as `grad * where(z < 0, 0, 1)` gives
+    with np.errstate(invalid="ignore"):
+        want_row = (np.float32(np.inf) * w[:, 5]) * np.where(z[3] < 0, np.float32(0), np.float32(1))
+    assert np.array_equal(np.isnan(dx[3]), np.isnan(want_row)) and np.array_equal(dx[3][~np.isnan(want_row)], want_row[~np.isnan(want_row)])
+    assert np.all(np.isinf(dW[:, 5]) | np.isnan(dW[:, 5]))
+    got_db = db.to_numpy()[0]
+    assert np.isinf(got_db[5]) and np.allclose(got_db[cols], dy[:, cols].astype(np.float64).sum(0), rtol=0, atol=2e-4)
+
+
+def test_batched_matmul_pair_general_operands_and_argument_checks(tt):
+    """Operands outside the one-grid form -- integer dtypes, offset and strided views, empty products, batches -- give the
+    bits of two ttamd_batched_matmul calls (they are two such calls); a NULL product is refused."""
+    from tinytensor_amd import _capi
+    be = tt.get_backend(tt.kAMD)
+    rng = np.random.default_rng(77)
+    for dtype in (np.int32, np.uint8, np.float64, np.float32):
+        a = rng.integers(0, 5, (2, 70, 33)).astype(dtype)
+        b = rng.integers(0, 5, (2, 33, 41)).astype(dtype)
+        big = tt.Tensor.from_numpy(np.concatenate([np.zeros((1, 70, 33), dtype), a]))
+        ta = tt.Tensor(big.storage, big.dtype, (2, 70, 33), big.stride, 70 * 33)      # an offset view
+        tb = tt.Tensor.from_numpy(np.ascontiguousarray(b.transpose(0, 2, 1))).permute(0, 2, 1)  # a permuted view
+        g = rng.integers(0, 5, (2, 70, 41)).astype(dtype)
+        tg = tt.Tensor.from_numpy(g)
+        da, db = be.batched_matmul_pair((tg, tb.permute(0, 2, 1)), (ta.permute(0, 2, 1), tg))
+        assert np.array_equal(da.to_numpy(), be.batched_matmul(tg, tb.permute(0, 2, 1)).to_numpy())
+        assert np.array_equal(db.to_numpy(), be.batched_matmul(ta.permute(0, 2, 1), tg).to_numpy())
+        assert np.array_equal(da.to_numpy(), np.matmul(g, b.transpose(0, 2, 1)))
+        assert np.array_equal(db.to_numpy(), np.matmul(a.transpose(0, 2, 1), g))
+    # empty products: no rows in one, no reduction in the other
+    e0, e1 = be.batched_matmul_pair((tt.Tensor.empty((1, 0, 8), _capi.F32), tt.Tensor.empty((1, 8, 4), _capi.F32)),
+                                    (tt.Tensor.empty((1, 5, 0), _capi.F32), tt.Tensor.empty((1, 0, 3), _capi.F32)))
+    assert e0.shape == (1, 0, 4) and np.array_equal(e1.to_numpy(), np.zeros((1, 5, 3), np.float32))
+    assert _capi.lib.ttamd_batched_matmul_pair(0, _capi.F32, None, None, None) != 0
+    assert "NULL product" in _capi.last_error()
+
+
 @pytest.mark.parametrize("own", [False, True, "head"])
 def test_fused_mlp_training_step_matches_the_oracle_and_fits_15_launches(tt, oracle, own):
     X = oracle.Generator(0).uniform_real(0.0, 1.0, (1024, 784))

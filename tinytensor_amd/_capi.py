@@ -33,6 +33,11 @@ class Epilogue(C.Structure):
                 ("rhs_colsum_out", C.c_void_p)]
 
 
+class Product(C.Structure):
+    _fields_ = [("B", C.c_int), ("N", C.c_int), ("K", C.c_int), ("M", C.c_int), ("lhs", C.POINTER(View3)),
+                ("rhs", C.POINTER(View3)), ("out", C.c_void_p), ("epilogue", C.POINTER(Epilogue))]
+
+
 def _bind(lib: C.CDLL) -> None:
     i, vp, sz = C.c_int, C.c_void_p, C.c_size_t
     sig = {
@@ -73,6 +78,7 @@ def _bind(lib: C.CDLL) -> None:
                                                 C.POINTER(C.c_uint64), i, C.POINTER(C.c_int64), C.POINTER(C.c_int64), vp,
                                                 C.c_int64, vp]),
         "ttamd_batched_matmul": (i, [i, i, i, i, i, i, C.POINTER(View3), C.POINTER(View3), vp, C.POINTER(Epilogue), vp]),
+        "ttamd_batched_matmul_pair": (i, [i, i, C.POINTER(Product), C.POINTER(Product), vp]),
         "ttamd_batched_matmul_noalloc": (i, [i, i, i, i, i, i, C.POINTER(View3), C.POINTER(View3), vp, C.POINTER(Epilogue), vp]),
         "ttamd_batched_matmul_variant": (C.c_char_p, [i, i, i, i, i, C.POINTER(View3), C.POINTER(View3)]),
         "ttamd_conv2d_forward": (i, [i, i, C.POINTER(View4), C.POINTER(View4), vp, vp] + [i] * 8 + [vp]),

@@ -109,6 +109,9 @@ ttamd_status launch_gemm_mfma(ttamd_dtype dt, const GemmArgs &g, int device, hip
                               bool variant_only, bool *handled, bool fixed_scratch = false);
 ttamd_status launch_gemm_simt(ttamd_dtype dt, const GemmArgs &g, hipStream_t stream, const char **variant,
                               bool variant_only);
+// Two independent products as one grid (gemm_mfma.hip) when both are dense fp32 products of 128 to 256 small tiles in the
+// layouts of a product's two gradients; *handled = false: nothing was launched, run them one after the other.
+ttamd_status launch_gemm_pair(ttamd_dtype dt, const GemmArgs &g0, const GemmArgs &g1, int device, hipStream_t stream, bool *handled);
 // Products of at most 16 columns and a reduction long enough to share out, and products with a reduction of at most
 // 16 (gemm_thin.hip): one launch; only the column sums of the second kind may take scratch.
 // *handled says whether the product is one of them (nothing is launched otherwise).

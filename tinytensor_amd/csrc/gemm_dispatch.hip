@@ -167,6 +167,42 @@ ttamd_status ttamd_batched_matmul(int device, ttamd_dtype dtype, int B, int N, i
     return batched_matmul(device, dtype, B, N, K, M, lhs, rhs, out, epilogue, stream, false);
 }
 
+ttamd_status ttamd_batched_matmul_pair(int device, ttamd_dtype dtype, const ttamd_product *first, const ttamd_product *second,
+                                       void *stream) {
+    if (!first || !second) {
+        set_error("batched_matmul_pair: NULL product");
+        return TTAMD_ERR_INVALID_ARGUMENT;
+    }
+    const ttamd_product *const p[2] = {first, second};
+    GemmArgs g[2];
+    bool plain = true;  // both products have work on the device and nothing special about them
+    for (int i = 0; i < 2; ++i) {
+        if (ttamd_status s = build_args(dtype, p[i]->B, p[i]->N, p[i]->K, p[i]->M, p[i]->lhs, p[i]->rhs, p[i]->out, p[i]->epilogue,
+                                        &g[i], true))
+            return s;
+        plain = plain && p[i]->B > 0 && p[i]->N > 0 && p[i]->M > 0 && p[i]->K > 0;
+    }
+    if (plain) {
+        if (ttamd_status s = use_device(device)) return s;
+        hipStream_t st = static_cast<hipStream_t>(stream);
+        bool handled = false, sums_done = false;
+        g[1].rhs_colsum_done = &sums_done;
+        if (ttamd_status s = launch_gemm_pair(dtype, g[0], g[1], device, st, &handled)) return s;
+        if (handled) {
+            // the first product's right-operand sums (the pair's kernel does not form them) and the second's, unless written
+            if (g[0].rhs_colsum)
+                if (ttamd_status s = launch_colsum_reduce(dtype, g[0].B, g[0].K, g[0].N, g[0].batch, g[0].rhs_colsum, st)) return s;
+            if (g[1].rhs_colsum && !sums_done) return launch_colsum_reduce(dtype, g[1].B, g[1].K, g[1].N, g[1].batch, g[1].rhs_colsum, st);
+            return TTAMD_OK;
+        }
+    }
+    for (int i = 0; i < 2; ++i)
+        if (ttamd_status s = batched_matmul(device, dtype, p[i]->B, p[i]->N, p[i]->K, p[i]->M, p[i]->lhs, p[i]->rhs, p[i]->out,
+                                            p[i]->epilogue, stream, false))
+            return s;
+    return TTAMD_OK;
+}
+
 ttamd_status ttamd_batched_matmul_noalloc(int device, ttamd_dtype dtype, int B, int N, int K, int M, const ttamd_view3 *lhs,
                                           const ttamd_view3 *rhs, void *out, const ttamd_epilogue *epilogue, void *stream) {
     return batched_matmul(device, dtype, B, N, K, M, lhs, rhs, out, epilogue, stream, true);

@@ -499,6 +499,114 @@ ttamd_status launch_layouts(const GemmArgs &g, bool a_kc, bool b_kc, const Split
     return launch_variant<T, BM, BN, BK, WGM, WGN, false, A_VEC, false, B_VEC, PF>(g, sp, device, stream);
 }
 
+// Two independent products in one launch (fp32, the 64 x 64 tile, whole reductions): workgroups [0, blocks0) compute
+// tiles of the first, the rest tiles of the second.  Each product alone would leave the chip a single workgroup per CU
+// (a Linear layer's two gradients at batch 1024: 256 tiles each) and pay its launch, its first loads and its stores with
+// nothing else running; together two workgroups share every CU and each covers the other's waits.  BSUM: the second
+// product's first row of tiles also adds up the vectors of B that it stages (see gemm_mfma_dual_kernel).
+template <typename T, bool A_KC, bool B_KC, int PF, bool BSUM>
+__device__ __forceinline__ void small_tile_product(const GemmArgs &g, int tiles_m, int tiles_n, unsigned block, unsigned blocks, unsigned char *smem_raw) {
+    using TS = TileShapes<T>;
+    constexpr int BM = TS::SBM, BN = TS::SBN, BK = TS::SBK, VK = Mfma<T>::VK;
+    using StA = Stager<T, BM, BK, A_KC, VK, PF>;
+    using StB = Stager<T, BN, BK, B_KC, VK, PF, BSUM>;
+    using Engine = TileEngine<T, BM, BN, BK, 2, 2, StA, StB>;
+    static_assert(!BSUM || static_cast<size_t>(StB::kSumParts) * BN * sizeof(T) <= Engine::kLdsBytes, "the operand sums fit the tile buffers");
+    T *const smem = reinterpret_cast<T *>(smem_raw);
+    const int tid = threadIdx.x;
+    int batch, tm, tn;
+    decode_tile(remap_xcd(block, blocks), tiles_m, tiles_n, batch, tm, tn);
+    const int m0 = tm * BM, n0 = tn * BN;
+    const T *a_base = static_cast<const T *>(g.A) + static_cast<int64_t>(batch) * g.a_sb + static_cast<int64_t>(m0) * g.a_sm;
+    const T *b_base = static_cast<const T *>(g.B) + static_cast<int64_t>(batch) * g.b_sb + static_cast<int64_t>(n0) * g.b_sn;
+    StA sa;
+    StB sb;
+    sa.init(a_base, tid, g.M - m0, g.a_sm, g.a_sk, g.K);
+    sb.init(b_base, tid, g.N - n0, g.b_sn, g.b_sk, g.K);
+    if constexpr (BSUM) sb.start_sums(tm == 0);
+    Engine eng;
+    eng.init(tid);
+    eng.run(sa, sb, smem, g.K, !sa.row_mask && !sb.row_mask);
+    if constexpr (BSUM) {
+        if (tm == 0) {  // (workgroup-uniform) a lane's k rows were added in k order; the lanes of a column follow in lane order
+            __syncthreads();  // every wave is done with the tile buffers
+            *reinterpret_cast<typename StB::V *>(&smem[sb.sum_part() * BN + sb.sum_row0()]) = sb.sum;
+            __syncthreads();
+            if (tid < BN && n0 + tid < g.N) {
+                T v = T(0);
+#pragma unroll
+                for (int r = 0; r < StB::kSumParts; ++r) v += smem[r * BN + tid];
+                static_cast<T *>(g.rhs_colsum)[static_cast<int64_t>(batch) * g.N + n0 + tid] = v;
+            }
+        }
+    }
+    T *C = static_cast<T *>(g.C) + static_cast<int64_t>(batch) * g.M * g.N;
+    if (plain_store(g))
+        store_tile_dense<T, true>(eng, C, g.M, g.N, m0, n0, static_cast<const T *>(nullptr), 0, 0, 0);
+    else if (!ext_store(g))
+        store_tile_dense<T, false>(eng, C, g.M, g.N, m0, n0, static_cast<const T *>(g.bias), g.bias_mode, g.relu, g.accumulate);
+    else
+        store_tile_dense<T, false, true>(eng, C, g.M, g.N, m0, n0, static_cast<const T *>(g.bias), g.bias_mode, g.relu, g.accumulate,
+                                         make_ext<T>(g, batch, tm, 2));
+}
+
+template <typename T, bool A0_KC, bool B0_KC, bool A1_KC, bool B1_KC, int PF, bool BSUM1>
+__global__ void __launch_bounds__(kThreads, 2)  // (two workgroups per CU: at most 256 registers per lane)
+gemm_mfma_pair_kernel(GemmArgs g0, int tiles_m0, int tiles_n0, GemmArgs g1, int tiles_m1, int tiles_n1, unsigned blocks0) {
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
+    if (blockIdx.x < blocks0)
+        small_tile_product<T, A0_KC, B0_KC, PF, false>(g0, tiles_m0, tiles_n0, blockIdx.x, blocks0, smem_raw);
+    else
+        small_tile_product<T, A1_KC, B1_KC, PF, BSUM1>(g1, tiles_m1, tiles_n1, blockIdx.x - blocks0, gridDim.x - blocks0, smem_raw);
+}
+
+// Launches the two products as one grid when each is a dense fp32 product that would take the small tile with one
+// workgroup per CU at most: first operand pair (k contiguous, k contiguous), second (m contiguous, n contiguous) -- the
+// layouts of TensorBatchedMatmul::backward's two products on dense operands (autograd/binary_ops.cpp:173-179:
+// dA = dC . B^T, dB = A^T . dC).  *handled = false: nothing was launched.
+ttamd_status launch_pair_f32(const GemmArgs &g0, const GemmArgs &g1, int device, hipStream_t stream, bool *handled) {
+    using T = float;
+    using TS = TileShapes<T>;
+    constexpr int VK = Mfma<T>::VK, PF = TS::SPF_DEEP;
+    auto tiles_of = [](const GemmArgs &g) {
+        return static_cast<int64_t>((g.M + TS::SBM - 1) / TS::SBM) * ((g.N + TS::SBN - 1) / TS::SBN) * g.batch;
+    };
+    auto fits = [&](const GemmArgs &g, bool kc) {
+        if (g.M < 256 || g.N < 256 || g.K < 16 * TS::SBK || g.batch < 1 || g.colsum_out) return false;
+        const OperandClass ca = classify<T>(g.A, g.a_sm, g.a_sk, g.a_sb, g.batch);
+        const OperandClass cb = classify<T>(g.B, g.b_sn, g.b_sk, g.b_sb, g.batch);
+        if (ca.vec != VK || cb.vec != VK || ca.kc != kc || cb.kc != kc) return false;
+        // 32-bit byte offsets inside a tile's operand panels and output rows
+        const int64_t a_reach = (static_cast<int64_t>(TS::SBM - 1) * g.a_sm + static_cast<int64_t>(g.K - 1) * g.a_sk + VK) * sizeof(T);
+        const int64_t b_reach = (static_cast<int64_t>(TS::SBN - 1) * g.b_sn + static_cast<int64_t>(g.K - 1) * g.b_sk + VK) * sizeof(T);
+        const int64_t c_reach = static_cast<int64_t>(TS::SBM) * g.N * static_cast<int64_t>(sizeof(T));
+        if (a_reach >= 0x7fffffffLL || b_reach >= 0x7fffffffLL || c_reach >= 0x7fffffffLL) return false;
+        const int64_t tiles = tiles_of(g);
+        return tiles >= 128 && tiles <= 256;
+    };
+    *handled = false;
+    static const bool enabled = std::getenv("TTAMD_MATMUL_PAIR") == nullptr || std::atoi(std::getenv("TTAMD_MATMUL_PAIR")) != 0;
+    if (!enabled || !fits(g0, true) || !fits(g1, false)) return TTAMD_OK;
+    const bool bsum = g1.rhs_colsum != nullptr;
+    using StK = Stager<T, TS::SBM, TS::SBK, true, VK, PF>;
+    using StM = Stager<T, TS::SBM, TS::SBK, false, VK, PF>;
+    constexpr size_t lds0 = TileEngine<T, TS::SBM, TS::SBN, TS::SBK, 2, 2, StK, StK>::kLdsBytes;
+    constexpr size_t lds1 = TileEngine<T, TS::SBM, TS::SBN, TS::SBK, 2, 2, StM, StM>::kLdsBytes;
+    constexpr size_t lds_bytes = lds0 > lds1 ? lds0 : lds1;
+    static_assert(lds_bytes <= 48 * 1024, "within the default dynamic LDS limit");
+    const unsigned blocks0 = static_cast<unsigned>(tiles_of(g0)), blocks1 = static_cast<unsigned>(tiles_of(g1));
+    const int tm0 = (g0.M + TS::SBM - 1) / TS::SBM, tn0 = (g0.N + TS::SBN - 1) / TS::SBN;
+    const int tm1 = (g1.M + TS::SBM - 1) / TS::SBM, tn1 = (g1.N + TS::SBN - 1) / TS::SBN;
+    if (bsum)
+        gemm_mfma_pair_kernel<T, true, true, false, false, PF, true><<<dim3(blocks0 + blocks1), dim3(kThreads), lds_bytes, stream>>>(g0, tm0, tn0, g1, tm1, tn1, blocks0);
+    else
+        gemm_mfma_pair_kernel<T, true, true, false, false, PF, false><<<dim3(blocks0 + blocks1), dim3(kThreads), lds_bytes, stream>>>(g0, tm0, tn0, g1, tm1, tn1, blocks0);
+    TTAMD_HIP_CHECK(hipGetLastError());
+    if (bsum && g1.rhs_colsum_done) *g1.rhs_colsum_done = true;
+    *handled = true;
+    return TTAMD_OK;
+}
+
 // Split the reduction when the output has too few tiles to fill 256 CUs and K is long enough to share out.
 // Every split gets a whole number of BK tiles; at most 64 splits and 32 MiB of partial tiles.
 template <typename T>
@@ -647,6 +755,12 @@ ttamd_status launch_colsum_reduce(ttamd_dtype dt, const void *partial, int rows,
     else
         colsum_reduce_kernel<double><<<grid, dim3(64), 0, stream>>>(static_cast<const double *>(partial), rows, N, static_cast<double *>(out));
     TTAMD_HIP_CHECK(hipGetLastError());
+    return TTAMD_OK;
+}
+
+ttamd_status launch_gemm_pair(ttamd_dtype dt, const GemmArgs &g0, const GemmArgs &g1, int device, hipStream_t stream, bool *handled) {
+    *handled = false;
+    if (dt == TTAMD_F32) return launch_pair_f32(g0, g1, device, stream, handled);
     return TTAMD_OK;
 }
 

@@ -290,6 +290,21 @@ public:
         check(ttamd_batched_matmul(lhs.device().id, static_cast<ttamd_dtype>(lhs.dtype()), B, N, K, M, &l, &r, out->ptr_, epilogue, nullptr));
         return {out, lhs.dtype(), Shape({B, N, M}), lhs.device()};
     }
+    // Two independent products in one call (ttamd_batched_matmul_pair): what TensorBatchedMatmul::backward
+    // (autograd/binary_ops.cpp:173-179) asks of the backend for its two gradients.
+    [[nodiscard]] auto batched_matmul_pair(const Tensor &lhs0, const Tensor &rhs0, const ttamd_epilogue *ep0, const Tensor &lhs1,
+                                           const Tensor &rhs1, const ttamd_epilogue *ep1) const -> std::pair<Tensor, Tensor> {
+        if (lhs0.dtype() != lhs1.dtype() || lhs0.device().id != lhs1.device().id) throw TTException("batched_matmul_pair: one dtype and device");
+        const ttamd_view3 l0 = view3(lhs0), r0 = view3(rhs0), l1 = view3(lhs1), r1 = view3(rhs1);
+        ttamd_product p0{lhs0.size(0), lhs0.size(1), lhs0.size(2), rhs0.size(2), &l0, &r0, nullptr, ep0};
+        ttamd_product p1{lhs1.size(0), lhs1.size(1), lhs1.size(2), rhs1.size(2), &l1, &r1, nullptr, ep1};
+        auto out0 = std::make_shared<StorageAMD>(checked_numel({p0.B, p0.N, p0.M}) * dtype_size(lhs0.dtype()), lhs0.device().id);
+        auto out1 = std::make_shared<StorageAMD>(checked_numel({p1.B, p1.N, p1.M}) * dtype_size(lhs1.dtype()), lhs1.device().id);
+        p0.out = out0->ptr_;
+        p1.out = out1->ptr_;
+        check(ttamd_batched_matmul_pair(lhs0.device().id, static_cast<ttamd_dtype>(lhs0.dtype()), &p0, &p1, nullptr));
+        return {Tensor{out0, lhs0.dtype(), Shape({p0.B, p0.N, p0.M}), lhs0.device()}, Tensor{out1, lhs1.dtype(), Shape({p1.B, p1.N, p1.M}), lhs1.device()}};
+    }
     [[nodiscard]] auto conv2d(const Tensor &input, const Tensor &weight, const std::optional<Tensor> &bias, int stride, int padding) const
         -> Tensor {
         const int B = input.size(0), C = input.size(1), H = input.size(2), W = input.size(3), O = weight.size(0), k = weight.size(2);
@@ -828,8 +843,10 @@ inline auto linear_backward(const Tensor &grad_output, const Tensor &input, cons
         g.db = Tensor::empty(Shape({dy.size(1)}), dy.dtype(), dy.device());
         ep_w.rhs_colsum_out = g.db->data_ptr();
     }
-    g.dx = be->batched_matmul(dy.unsqueeze(0), weight.unsqueeze(0).permute({0, 2, 1}), &ep).squeeze(0);
-    g.dW = be->batched_matmul(input.unsqueeze(0).permute({0, 2, 1}), dy.unsqueeze(0), bias_grad == BiasGrad::kOwn ? &ep_w : nullptr).squeeze(0);
+    auto [dx, dW] = be->batched_matmul_pair(dy.unsqueeze(0), weight.unsqueeze(0).permute({0, 2, 1}), &ep, input.unsqueeze(0).permute({0, 2, 1}),
+                                            dy.unsqueeze(0), bias_grad == BiasGrad::kOwn ? &ep_w : nullptr);
+    g.dx = dx.squeeze(0);
+    g.dW = dW.squeeze(0);
     return g;
 }
 

@@ -488,6 +488,18 @@ class BackendAMD:
         relu_grad_input: dense [B,N,M] saved input z of a ReLU, out = result * (z < 0 ? 0 : 1);
         colsum_out: dense [B,M] tensor that receives out summed over its rows;
         rhs_colsum_out: dense [B,M] tensor that receives rhs (dense row-major) summed over its rows."""
+        out, ep = self._product(lhs, rhs, out, bias=bias, bias_mode=bias_mode, relu=relu, accumulate=accumulate, relu_out=relu_out,
+                                relu_grad_input=relu_grad_input, colsum_out=colsum_out, rhs_colsum_out=rhs_colsum_out)
+        B, N, K = lhs.shape
+        lv, rv = lhs.view3(), rhs.view3()
+        _check(lib.ttamd_batched_matmul(lhs.device.id, lhs.dtype, B, N, K, rhs.size(2), C.byref(lv), C.byref(rv),
+                                        C.c_void_p(out.storage.ptr), C.byref(ep) if ep is not None else None, _stream_arg()))
+        return out
+
+    @staticmethod
+    def _product(lhs: Tensor, rhs: Tensor, out: Tensor | None, bias=None, bias_mode=0, relu=False, accumulate=False,
+                 relu_out=None, relu_grad_input=None, colsum_out=None, rhs_colsum_out=None):
+        """The result tensor and the ttamd_epilogue (or None) of one product; checks the epilogue's tensors."""
         assert lhs.dim() == 3 and rhs.dim() == 3 and lhs.size(2) == rhs.size(1)
         B, N, K = lhs.shape
         M = rhs.size(2)
@@ -510,10 +522,27 @@ class BackendAMD:
                 if not dense or t.numel() != int(np.prod(want)) or t.dtype != lhs.dtype:
                     raise TTException(f"batched_matmul: {name} must be a dense tensor of {want} elements of the operands' dtype")
                 setattr(ep, name, t.storage.ptr + t.offset * t.itemsize)
-        lv, rv = lhs.view3(), rhs.view3()
-        _check(lib.ttamd_batched_matmul(lhs.device.id, lhs.dtype, B, N, K, M, C.byref(lv), C.byref(rv),
-                                        C.c_void_p(out.storage.ptr), C.byref(ep) if ep is not None else None, _stream_arg()))
-        return out
+        return out, ep
+
+    def batched_matmul_pair(self, first: tuple, second: tuple) -> tuple:
+        """Two independent products in one call (ttamd_batched_matmul_pair): what TensorBatchedMatmul::backward
+        (autograd/binary_ops.cpp:173-179) asks of the backend.  Each argument is (lhs, rhs) or (lhs, rhs, kwargs) with
+        batched_matmul's keyword arguments; returns the two results."""
+        prods, keep = [], []
+        for spec in (first, second):
+            lhs, rhs = spec[0], spec[1]
+            kw = dict(spec[2]) if len(spec) > 2 else {}
+            out, ep = self._product(lhs, rhs, kw.pop("out", None), **kw)
+            lv, rv = lhs.view3(), rhs.view3()
+            B, N, K = lhs.shape
+            pr = _capi.Product(B, N, K, rhs.size(2), C.pointer(lv), C.pointer(rv), C.c_void_p(out.storage.ptr),
+                               C.pointer(ep) if ep is not None else None)
+            prods.append(pr)
+            keep.append((lv, rv, ep, out))
+        if keep[0][3].dtype != keep[1][3].dtype or first[0].device != second[0].device:
+            raise TTException("batched_matmul_pair: both products must have one dtype and device")
+        _check(lib.ttamd_batched_matmul_pair(first[0].device.id, first[0].dtype, C.byref(prods[0]), C.byref(prods[1]), _stream_arg()))
+        return keep[0][3], keep[1][3]
 
     def batched_matmul_variant(self, lhs: Tensor, rhs: Tensor) -> str:
         B, N, K = lhs.shape
@@ -866,10 +895,10 @@ def linear_backward(grad_output: Tensor, input: Tensor, weight: Tensor, relu_inp
     own = bias_grad == "own"
     fout = grad_output.size(1)
     db = Tensor.empty((1, fout if own else fin), grad_output.dtype, grad_output.device) if bias_grad else None
-    dx = be.batched_matmul(grad_output.unsqueeze(0), weight.unsqueeze(0).permute(0, 2, 1),
-                           relu_grad_input=relu_input.unsqueeze(0) if relu_input is not None else None,
-                           colsum_out=None if own else db)
-    dW = be.batched_matmul(input.unsqueeze(0).permute(0, 2, 1), grad_output.unsqueeze(0), rhs_colsum_out=db if own else None)
+    dx, dW = be.batched_matmul_pair(
+        (grad_output.unsqueeze(0), weight.unsqueeze(0).permute(0, 2, 1),
+         dict(relu_grad_input=relu_input.unsqueeze(0) if relu_input is not None else None, colsum_out=None if own else db)),
+        (input.unsqueeze(0).permute(0, 2, 1), grad_output.unsqueeze(0), dict(rhs_colsum_out=db if own else None)))
     return dx.squeeze(0), dW.squeeze(0), (db.reshape([fout if own else fin]) if db is not None else None)
 
 
