@@ -176,14 +176,15 @@ ttamd_status ttamd_batched_matmul(int device, ttamd_dtype dtype, int B, int N, i
                                   const ttamd_epilogue *epilogue, void *stream);
 
 /* Two independent products in one call: what TensorBatchedMatmul::backward (autograd/binary_ops.cpp:173-179) asks of
- * the backend -- dA = dC . B^T and dB = A^T . dC, two batched_matmul calls on permuted views -- and nn::Linear's backward
- * with it (nn/linear.cpp:42-50).  Each product has ttamd_batched_matmul's contract and gives the bits that call gives
- * ... or, where the pair is launched as one grid, the bits of the same kernel family's plain 64 x 64 tile (every sum
- * in k order, so equal to the separate calls' wherever those do not split the reduction).  Neither product may read
- * the other's result.  One grid is launched when both are dense fp32 products of 128 to 256 tiles of 64 x 64 with a
- * reduction of 512 or more, `first` in the layouts of dA (both operands contiguous along k), `second` in those of dB
- * (left operand contiguous along its rows' index m, right operand along n); otherwise the two products run one after
- * the other exactly as two ttamd_batched_matmul calls would. */
+ * the backend -- dA = dC . B^T and dB = A^T . dC, two batched_matmul calls on permuted views -- and with it the backward
+ * of nn::Linear (nn/linear.cpp:42-50).  Each product has ttamd_batched_matmul's contract (operands, epilogue, errors);
+ * neither may read the other's result.  Both run as ONE grid when each is a dense fp32 product of 128 to 256 tiles of
+ * 64 x 64 with a reduction of 512 or more, `first` with both operands contiguous along k (dC and B^T of dense dC, B),
+ * `second` with the left operand contiguous along m and the right along n (A^T and dC of dense A, dC), no colsum_out:
+ * a Linear layer of 784 to 1024 features at batch 1024, whose two products alone would each leave the chip one
+ * workgroup per CU.  Every element is then summed in k order from 0 (the separate calls add two halves of the
+ * reduction): equal on integer-valued data, equal to rounding otherwise, and the same bits on every call.  Anything
+ * else runs as two ttamd_batched_matmul calls, first then second. */
 typedef struct ttamd_product {
     int B, N, K, M;
     const ttamd_view3 *lhs, *rhs;
