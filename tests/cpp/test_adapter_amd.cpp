@@ -18,6 +18,7 @@
 #include <tt/shape.h>
 #include <tt/tensor.h>
 
+#include "tensor/backend/amd/backend_amd.h"
 #include "tensor/backend_base.h"
 
 #include <algorithm>
@@ -250,6 +251,41 @@ TEST_CASE("batched_matmul on a permuted operand with an offset, read in place") 
                     }
         CHECK(be.batched_matmul(lhs, shared).to_vec<T>() == expected_shared);
     });
+}
+
+TEST_CASE("batched_matmul_pair: the two products of TensorBatchedMatmul::backward in one call") {
+    // autograd/binary_ops.cpp:173-179: {grad . rhs^T, lhs^T . grad} on permuted views.  Not a virtual of BackendBase: called
+    // on the adapter's class.  float at a Linear layer's size (both products in one grid) and every dtype at a small one (two
+    // calls inside); data i % 7 - 3, every sum an integer below 2^24.
+    const auto &be = dynamic_cast<const tinytensor::amd::BackendAMD &>(backend());
+    auto run = [&]<typename T>(int B, int N, int K, int M) {
+        const std::vector<T> lhs = pattern<T>(B * N * K, 7, 3), rhs = pattern<T>(B * K * M, 5, 2), grad = pattern<T>(B * N * M, 3, 1);
+        const Tensor tl(lhs, {B, N, K}, kAMD), tr(rhs, {B, K, M}, kAMD), tg(grad, {B, N, M}, kAMD);
+        const auto [dl, dr] = be.batched_matmul_pair(tg, tr.permute({0, 2, 1}), tl.permute({0, 2, 1}), tg);
+        std::vector<T> want_l(lhs.size(), T(0)), want_r(rhs.size(), T(0));
+        for (int b = 0; b < B; ++b)
+            for (int n = 0; n < N; ++n)
+                for (int m = 0; m < M; ++m) {
+                    const T g = grad[(static_cast<std::size_t>(b) * N + n) * M + m];
+                    for (int k = 0; k < K; ++k) {
+                        T &a = want_l[(static_cast<std::size_t>(b) * N + n) * K + k];
+                        a = static_cast<T>(a + static_cast<T>(g * rhs[(static_cast<std::size_t>(b) * K + k) * M + m]));
+                        T &c = want_r[(static_cast<std::size_t>(b) * K + k) * M + m];
+                        c = static_cast<T>(c + static_cast<T>(lhs[(static_cast<std::size_t>(b) * N + n) * K + k] * g));
+                    }
+                }
+        CHECK(dl.shape() == Shape({B, N, K}));
+        CHECK(dr.shape() == Shape({B, K, M}));
+        CHECK(dl.to_vec<T>() == want_l);
+        CHECK(dr.to_vec<T>() == want_r);
+        // the same bits as the two calls of the interface where those run the same kernels (the small size)
+        if (N < 256) {
+            CHECK(be.batched_matmul(tg, tr.permute({0, 2, 1})).template to_vec<T>() == dl.template to_vec<T>());
+            CHECK(be.batched_matmul(tl.permute({0, 2, 1}), tg).template to_vec<T>() == dr.template to_vec<T>());
+        }
+    };
+    for_all_except_bool([&]<typename T>() { run.template operator()<T>(2, 37, 29, 45); });
+    run.template operator()<float>(1, 576, 1000, 704);  // 144 and 176 tiles of 64 x 64, reductions of 704 and 576
 }
 
 TEST_CASE("conv2d: the reference's two geometries, all dtypes") {

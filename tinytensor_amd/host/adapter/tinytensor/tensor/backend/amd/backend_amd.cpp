@@ -414,6 +414,23 @@ auto BackendAMD::batched_matmul(const Tensor &lhs, const Tensor &rhs) const -> T
     return make_result(std::move(out), lhs.dtype(), std::move(result_shape), lhs.device());
 }
 
+auto BackendAMD::batched_matmul_pair(const Tensor &lhs0, const Tensor &rhs0, const Tensor &lhs1, const Tensor &rhs1) const
+    -> std::pair<Tensor, Tensor> {
+    if (lhs0.dtype() != lhs1.dtype() || lhs0.device() != lhs1.device()) {
+        TT_EXCEPTION("batched_matmul_pair: both products must have one dtype and device");
+    }
+    const ttamd_view3 l0 = view3(lhs0), r0 = view3(rhs0), l1 = view3(lhs1), r1 = view3(rhs1);
+    Shape shape0({lhs0.size(0), lhs0.size(1), rhs0.size(2)});
+    Shape shape1({lhs1.size(0), lhs1.size(1), rhs1.size(2)});
+    auto out0 = make_storage(lhs0.device().id, static_cast<std::size_t>(shape0.numel()), lhs0.dtype());
+    auto out1 = make_storage(lhs1.device().id, static_cast<std::size_t>(shape1.numel()), lhs1.dtype());
+    const ttamd_product p0{lhs0.size(0), lhs0.size(1), lhs0.size(2), rhs0.size(2), &l0, &r0, out0->ptr, nullptr};
+    const ttamd_product p1{lhs1.size(0), lhs1.size(1), lhs1.size(2), rhs1.size(2), &l1, &r1, out1->ptr, nullptr};
+    check(ttamd_batched_matmul_pair(lhs0.device().id, code(lhs0.dtype()), &p0, &p1, nullptr));
+    return {make_result(std::move(out0), lhs0.dtype(), std::move(shape0), lhs0.device()),
+            make_result(std::move(out1), lhs1.dtype(), std::move(shape1), lhs1.device())};
+}
+
 auto BackendAMD::conv2d(
     const Tensor &input,
     const Tensor &weight,

@@ -19,6 +19,7 @@
 #include <cstddef>
 #include <cstdint>
 #include <optional>
+#include <utility>
 #include <ostream>
 #include <tuple>
 #include <vector>
@@ -117,6 +118,11 @@ public:
 #define X(NAME) void NAME(Tensor &lhs, const Tensor &rhs) const override;
     TT_AMD_BINARY_INPLACE(X)
 #undef X
+
+    // Not a virtual of BackendBase: the two products of TensorBatchedMatmul::backward (autograd/binary_ops.cpp:173-179)
+    // in one call, {lhs0 . rhs0, lhs1 . rhs1}, as one grid where ttamd_batched_matmul_pair can run them so.
+    [[nodiscard]] auto batched_matmul_pair(const Tensor &lhs0, const Tensor &rhs0, const Tensor &lhs1, const Tensor &rhs1) const
+        -> std::pair<Tensor, Tensor>;
 
     // Reductions, unary operators and activations
 #define X(NAME) [[nodiscard]] auto NAME(const Tensor &tensor) const -> Tensor override;
