@@ -135,6 +135,10 @@ def test_every_override_has_exactly_one_definition():
         found.append((m.group(1), _types_only(_squash(m.group(2))), _squash(m.group(3) or "void")))
     found.sort()
     assert len(found) == len(set(found)), "a member is defined twice"
+    # one const member beside the overrides: the two products of a matmul's backward in one call, no virtual of BackendBase
+    extra = [f for f in found if f not in declared]
+    assert extra == [("batched_matmul_pair", "const Tensor&, const Tensor&, const Tensor&, const Tensor&", "std::pair<Tensor, Tensor>")], extra
+    found = [f for f in found if f not in extra]
     assert found == declared, (sorted(set(declared) - set(found))[:6], sorted(set(found) - set(declared))[:6])
 
 

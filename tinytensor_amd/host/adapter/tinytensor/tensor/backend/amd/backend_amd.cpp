@@ -416,7 +416,7 @@ auto BackendAMD::batched_matmul(const Tensor &lhs, const Tensor &rhs) const -> T
 
 auto BackendAMD::batched_matmul_pair(const Tensor &lhs0, const Tensor &rhs0, const Tensor &lhs1, const Tensor &rhs1) const
     -> std::pair<Tensor, Tensor> {
-    if (lhs0.dtype() != lhs1.dtype() || lhs0.device() != lhs1.device()) {
+    if (lhs0.dtype() != lhs1.dtype() || lhs0.device().id != lhs1.device().id) {
         TT_EXCEPTION("batched_matmul_pair: both products must have one dtype and device");
     }
     const ttamd_view3 l0 = view3(lhs0), r0 = view3(rhs0), l1 = view3(lhs1), r1 = view3(rhs1);
