@@ -189,6 +189,29 @@ def detail_report(tt, np, path, cpu=True):
                  "ms": round(graph_ms, 4), "GFLOP/s": round(step_flop / graph_ms / 1e6, 1)})
     graph.close()
     gstream.close()
+    # the same step from the fused forms (Linear + ReLU, the last layer with the loss, each layer's two gradients as one call)
+
+    def fused_step():
+        z1, a1 = tt.linear_relu(xs, P1, c1); z2, a2 = tt.linear_relu(a1, P2, c2)
+        y, loss, dz2, dW3, db3 = tt.linear_mse_head(a2, P3, c3, ts, relu_input=z2)
+        dz1, dW2, db2 = tt.linear_backward(dz2, a1, P2, relu_input=z1, bias_grad="own")
+        dX, dW1, db1 = tt.linear_backward(dz1, xs, P1, bias_grad="own")
+        return [loss, dW1, db1, dW2, db2, dW3, db3, dX]
+
+    gstream = tt.graph.Stream()
+    graph = tt.graph.Graph(gstream, fused_step)
+    for _ in range(20):
+        graph.launch()
+    gstream.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(100):
+        graph.launch()
+    gstream.synchronize()
+    fused_ms = (time.perf_counter() - t0) / 100 * 1e3
+    rows.append({"case": "cfg5 whole MLP training step from the fused forms, replayed from a HIP graph", "kernel": f"{graph.num_nodes()} graph nodes",
+                 "ms": round(fused_ms, 4), "GFLOP/s": round(step_flop / fused_ms / 1e6, 1)})
+    graph.close()
+    gstream.close()
     # one training step of the network of the reference's examples/mnist_cnn_example.cpp:31-63 at its batch size of 256
     # (conv 1->32, ReLU, conv 32->64, ReLU, max-pool, Linear 9216->128, ReLU, Linear 128->10; no dropout; squared error)
     crng = np.random.default_rng(3)
