@@ -156,7 +156,7 @@ struct ConvPatchArgs {
     int bne, tail;  // positions per tile; those of them behind the tile's whole 32-position blocks (twelve waves: 4 or 8)
     FastDiv d_wfast, d_segv, d_k, d_ngrp, d_xh, d_R, d_cpad4, d_2P, d_P, d_Wo, d_tiles_n, d_tail;
 };
-ttamd_status launch_conv_patch_f32(ConvPatchArgs a, hipStream_t stream, int *variant);
+ttamd_status launch_conv_patch_f32(ConvPatchArgs a, hipStream_t stream, int *variant, bool launch = true);
 
 // grad_weight with both operands staged in LDS (conv_wgrad_patch.hip).  The plan depends on the shape alone.
 struct ConvWgradPatchPlan {

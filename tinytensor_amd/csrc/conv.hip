@@ -783,20 +783,50 @@ dgrad_interleave_kernel(ConvGeom geo, const T *__restrict__ tmp, T *__restrict__
     gin[idx] = v;
 }
 
+// A small job that rides in a convolution launch as `blocks` workgroups appended to its grid (spared a launch of its
+// own, which for these sizes is all launch floor): kind 1, dst[i] = sum over s < splits of src[s * n + i] (grad_weight's
+// partial tiles, mfma::add_up_parts); kind 2, the transposed weight of grad_input (weight_transpose_kernel's work).
+struct ConvRide {
+    int kind = 0, blocks = 0;
+    const void *src = nullptr;
+    void *dst = nullptr;
+    int n = 0, splits = 0;
+};
+template <typename T>
+__device__ __forceinline__ void conv_ride(const ConvRide &r, const ConvGeom &geo, int block, T *smem) {
+    if (r.kind == 1) {
+        add_up_parts<T, kThreads / 64>(static_cast<const T *>(r.src), static_cast<T *>(r.dst), r.n, r.splits, block, smem);
+    } else {
+        const int idx = block * kThreads + static_cast<int>(threadIdx.x);
+        if (idx >= r.n) return;
+        const uint32_t k2 = static_cast<uint32_t>(geo.k * geo.k);
+        const uint32_t row = k2 * static_cast<uint32_t>(geo.O);
+        const uint32_t c = static_cast<uint32_t>(idx) / row, rem = static_cast<uint32_t>(idx) - c * row;
+        uint32_t o, t;
+        geo.d_kk.divmod(rem, o, t);
+        static_cast<T *>(r.dst)[idx] = static_cast<const T *>(r.src)[static_cast<int64_t>(o) * geo.w_so + c * k2 + t];
+    }
+}
+
 // grad_input: M = C, N = H*W, K = O*k*k, one GEMM per image.  wt is the transposed weight [C, O*k*k];
 // StB gathers grad_out.
 // SCATTER: the problem is one class of a strided grad_input and its result goes straight to that class's elements of
 // grad_input (ConvGeom::sc_S, store_tile_class_scatter).
 template <typename T, int BM, int BN, int BK, int A_VEC, class StB, bool SCATTER = false>
 __global__ void __launch_bounds__(kThreads, 2)
-conv_dgrad_kernel(ConvGeom geo, const T *gout, const T *wt, T *gin, int tiles_m, int tiles_n) {
+conv_dgrad_kernel(ConvGeom geo, const T *gout, const T *wt, T *gin, int tiles_m, int tiles_n, ConvRide ride) {
     using StA = Stager<T, BM, BK, true, A_VEC, kConvPF>;
     using Engine = ConvEngine<T, BM, BN, BK, StA, StB>;
     extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
     T *const smem = reinterpret_cast<T *>(smem_raw);
     const int tid = threadIdx.x;
+    const unsigned conv_blocks = gridDim.x - static_cast<unsigned>(ride.blocks);
+    if (blockIdx.x >= conv_blocks) {  // an appended workgroup
+        conv_ride<T>(ride, geo, static_cast<int>(blockIdx.x - conv_blocks), smem);
+        return;
+    }
     int b, tm, tn;
-    decode_tile(remap_xcd(blockIdx.x, gridDim.x), tiles_m, tiles_n, b, tm, tn);
+    decode_tile(remap_xcd(blockIdx.x, conv_blocks), tiles_m, tiles_n, b, tm, tn);
     const int m0 = tm * BM, n0 = tn * BN;
     const int M_ = geo.C, N_ = geo.H * geo.W, K = geo.O * geo.kh * geo.kw;
     const int64_t g_image = static_cast<int64_t>(geo.O) * geo.Ho * geo.Wo;
@@ -872,15 +902,20 @@ conv_dgrad_classes_kernel(DgradClassGeoms tab, const T *gout, const T *wt, T *gi
 template <typename T, int BK, int A_VEC, class StB, bool PADDED = false>
 __global__ void __launch_bounds__(kThreads, 2)
 conv_wgrad_kernel(ConvGeom geo, const T *gout, const T *x, T *partial, int64_t image_bytes, int group, int kslices, int k_chunk,
-                  int tiles_m, int tiles_n, int joint_k) {
+                  int tiles_m, int tiles_n, int joint_k, ConvRide ride) {
     constexpr int BM = 64, BN = 64;
     using StA = std::conditional_t<PADDED, PaddedRowsStager<T, BM, BK, kConvPF>, Stager<T, BM, BK, true, A_VEC, kConvPF>>;
     using Engine = ConvEngine<T, BM, BN, BK, StA, StB>;
     extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
     T *const smem = reinterpret_cast<T *>(smem_raw);
     const int tid = threadIdx.x;
+    const unsigned conv_blocks = gridDim.x - static_cast<unsigned>(ride.blocks);
+    if (blockIdx.x >= conv_blocks) {  // an appended workgroup
+        conv_ride<T>(ride, geo, static_cast<int>(blockIdx.x - conv_blocks), smem);
+        return;
+    }
     int part, tm, tn;
-    decode_tile(remap_xcd(blockIdx.x, gridDim.x), tiles_m, tiles_n, part, tm, tn);
+    decode_tile(remap_xcd(blockIdx.x, conv_blocks), tiles_m, tiles_n, part, tm, tn);
     const int m0 = tm * BM, n0 = tn * BN;
     const int plane = geo.Ho * geo.Wo;
     const int M_ = geo.O, N_ = geo.C * geo.k * geo.k, K = PADDED ? geo.Ho * geo.row_pad : plane;
@@ -1637,6 +1672,65 @@ ttamd_status backward_mfma(const ConvPlan &pl, const void *gout, void *gin, void
             }
         }
     }
+    // grad_weight on the implicit-GEMM kernel, with `ride` appended to its grid; leaves its partial tiles (if any) in
+    // parts_to_add for whoever adds them up.
+    t_last_kernel[2] = wgrad_staged ? 0x200 : 0x100;
+    bool wgrad_done = wgrad_staged;
+    auto wgrad_implicit = [&](const ConvRide &ride) -> ttamd_status {
+        const int M_ = g.O, N_ = g.C * g.k * g.k;
+        const int parts = plan.parts();
+        T *const partial = parts > 1 ? partials : static_cast<T *>(gw);
+        const int tiles_m = (M_ + 63) / 64, tiles_n = (N_ + 63) / 64;
+        const int64_t blocks = static_cast<int64_t>(tiles_m) * tiles_n * parts;
+        const bool a_vec = rows_vectorizable<T>(gout, HoWo, static_cast<int64_t>(g.O) * HoWo);
+        const bool b_vec = g.S == 1 && g.xs_w == 1 && g.Wo % VK == 0;
+        ConvGeom gw_geo = g;
+        if (wgrad_padded) {
+            gw_geo.row_pad = g.Wo % VK == 0 ? g.Wo : padded_row_width(sizeof(T), g.Wo);  // whole vectors already: joint mode only
+            gw_geo.d_row_pad = make_fastdiv(static_cast<uint32_t>(gw_geo.row_pad));
+        }
+        auto go = [&](auto kernel, size_t lds) {
+            return launch_conv(kernel, lds, blocks + ride.blocks, st, gw_geo, static_cast<const T *>(gout), static_cast<const T *>(pl.x), partial,
+                               pl.image_bytes, plan.group, plan.kslices, plan.k_chunk, tiles_m, tiles_n, wgrad_mode == 2 ? joint_k : 0, ride);
+        };
+        using VecB = TapStagerKC<T, 64, BK, VK, kConvPF>;
+        using OneB = Im2colTStager<T, 64, BK, kConvPF>;
+        ttamd_status s;
+        bool pair = false;
+        if constexpr (sizeof(T) == 4) pair = a_vec && !b_vec && g.S == 1 && g.xs_w == 1 && g.Wo % 2 == 0;
+        using PaddedB = TapStagerKC<T, 64, BK, VK, kConvPF, true>;
+        if (wgrad_padded) s = go(conv_wgrad_kernel<T, BK, VK, PaddedB, true>, conv_lds_bytes<T, 64, 64, VK, PaddedB>());
+        else if (a_vec && b_vec) s = go(conv_wgrad_kernel<T, BK, VK, VecB>, conv_lds_bytes<T, 64, 64, VK, VecB>());
+        else if (pair) {
+            if constexpr (sizeof(T) == 4) {
+                using PairB = TapStagerKC<T, 64, BK, 2, kConvPF>;
+                s = go(conv_wgrad_kernel<T, BK, VK, PairB>, conv_lds_bytes<T, 64, 64, VK, PairB>());
+            } else {
+                s = TTAMD_OK;
+            }
+        } else if (a_vec) s = go(conv_wgrad_kernel<T, BK, VK, OneB>, conv_lds_bytes<T, 64, 64, VK, OneB>());
+        else if (b_vec) s = go(conv_wgrad_kernel<T, BK, 1, VecB>, conv_lds_bytes<T, 64, 64, 1, VecB>());
+        else s = go(conv_wgrad_kernel<T, BK, 1, OneB>, conv_lds_bytes<T, 64, 64, 1, OneB>());
+        if (s) return s;
+        wgrad_done = true;
+        if (parts > 1) parts_to_add = parts;
+        return TTAMD_OK;
+    };
+    // the sum over grad_weight's partial tiles as a job appended to another launch, where vectors of 16 bytes can carry it
+    auto sum_ride = [&]() {
+        ConvRide r;
+        constexpr int VEC = 16 / static_cast<int>(sizeof(T));
+        if (parts_to_add > 0 && gw_elems % VEC == 0 && reinterpret_cast<uintptr_t>(gw) % 16 == 0 && reinterpret_cast<uintptr_t>(partials) % 16 == 0 &&
+            parts_to_add * gw_elems * static_cast<int64_t>(sizeof(T)) < 0x7fffffffLL) {
+            r.kind = 1;
+            r.blocks = static_cast<int>((gw_elems / VEC + 63) / 64);
+            r.src = partials;
+            r.dst = gw;
+            r.n = static_cast<int>(gw_elems);
+            r.splits = parts_to_add;
+        }
+        return r;
+    };
     // grad_input
     t_last_kernel[1] = 0;
     const int np = (g.k + g.S - 1) / g.S;
@@ -1674,7 +1768,7 @@ ttamd_status backward_mfma(const ConvPlan &pl, const void *gout, void *gin, void
     } else {
         // One unit-stride (or, without the class split, strided) grad_input GEMM: geometry gg, transposed weight wts
         // [C, O*kh*kw], dense result dst [B, C, gg.H*gg.W].
-        auto dgrad_gemm = [&](const ConvGeom &gg, const T *wts, T *dst) -> ttamd_status {
+        auto dgrad_gemm = [&](const ConvGeom &gg, const T *wts, T *dst, const ConvRide &ride = ConvRide{}) -> ttamd_status {
           const int Kd = gg.O * gg.kh * gg.kw;
           auto run = [&]<int BM, int BN, bool SC>() -> ttamd_status {
             ConvGeom g = gg;
@@ -1691,8 +1785,8 @@ ttamd_status backward_mfma(const ConvPlan &pl, const void *gout, void *gin, void
             const int64_t blocks = static_cast<int64_t>(tiles_m) * tiles_n * g.B;
             const bool b_vec = table_ok && g.S == 1 && (g.row_pad || g.W % VK == 0);
             auto go = [&](auto kernel, size_t lds) {
-                return launch_conv(kernel, lds, blocks, st, g, static_cast<const T *>(gout), static_cast<const T *>(wt),
-                                   static_cast<T *>(gin), tiles_m, tiles_n);
+                return launch_conv(kernel, lds, blocks + ride.blocks, st, g, static_cast<const T *>(gout), static_cast<const T *>(wt),
+                                   static_cast<T *>(gin), tiles_m, tiles_n, ride);
             };
             using VecB = TapStagerMC<T, BN, BK, VK, true, kConvPF>;
             using OneB = DgradStager<T, BN, BK, kConvPF>;
@@ -1808,13 +1902,15 @@ ttamd_status backward_mfma(const ConvPlan &pl, const void *gout, void *gin, void
                 TTAMD_HIP_CHECK(hipGetLastError());
             }
         } else {
-            bool handled = false;
+            // Unit stride.  grad_input is the convolution of grad_out with the reversed taps, padding k - 1 - P and the
+            // weight's two channel axes exchanged: the persistent kernel of conv_patch.hip reads the weight in that order
+            // itself (no transposed copy) where its geometry fits; the implicit-GEMM kernel reads a transposed copy.
+            // grad_weight goes first: the transposition then rides in its launch, and the sum over its partial tiles in
+            // grad_input's.
+            ConvPatchArgs a{};
+            bool resident = false;
             if constexpr (std::is_same_v<T, float>) {
-                // unit stride: grad_input is the convolution of grad_out with the reversed taps, padding k - 1 - P and
-                // the weight's two channel axes exchanged -- the persistent kernel of conv_patch.hip reads the weight
-                // in that order itself (no transposed copy)
                 if (g.S == 1 && g.kh == g.k && g.kw == g.k && g.P < g.k && patch_kernel_enabled()) {
-                    ConvPatchArgs a{};
                     a.x = static_cast<const float *>(gout);
                     a.w = static_cast<const float *>(pl.w);
                     a.bias = nullptr;
@@ -1824,77 +1920,53 @@ ttamd_status backward_mfma(const ConvPlan &pl, const void *gout, void *gin, void
                     a.w_row = static_cast<int64_t>(g.k) * g.k; a.w_red = g.w_so; a.w_flip = 1; a.w_rows_fast = 1;
                     a.image_bytes = static_cast<int64_t>(g.O) * HoWo * 4;
                     a.weight_bytes = pl.weight_bytes;
-                    const bool rides = parts_to_add > 0 && gw_elems % 4 == 0 && reinterpret_cast<uintptr_t>(gw) % 16 == 0 &&
-                                       reinterpret_cast<uintptr_t>(partials) % 16 == 0 && parts_to_add * gw_elems * 4 < 0x7fffffffLL;
-                    if (rides) {
+                    int variant = 0;
+                    if (ttamd_status rc = launch_conv_patch_f32(a, st, &variant, false)) return rc;  // (only asks)
+                    resident = variant != 0;
+                }
+            }
+            const int total = g.C * g.O * g.k * g.k;
+            bool transposed = false;
+            if (!wgrad_done) {
+                ConvRide ride;
+                if (!resident) {
+                    ride.kind = 2;
+                    ride.blocks = (total + kThreads - 1) / kThreads;
+                    ride.src = pl.w;
+                    ride.dst = wt;
+                    ride.n = total;
+                    transposed = true;
+                }
+                if (ttamd_status rc = wgrad_implicit(ride)) return rc;
+            }
+            const ConvRide sum = sum_ride();
+            if (resident) {
+                if constexpr (std::is_same_v<T, float>) {
+                    if (sum.kind) {
                         a.red_partial = partials;
                         a.red_out = static_cast<float *>(gw);
-                        a.red_n = static_cast<int>(gw_elems);
-                        a.red_splits = parts_to_add;
+                        a.red_n = sum.n;
+                        a.red_splits = sum.splits;
                     }
                     int variant = 0;
                     if (ttamd_status rc = launch_conv_patch_f32(a, st, &variant)) return rc;
-                    handled = variant != 0;
-                    if (handled) t_last_kernel[1] = 0x200 + variant;
-                    if (handled && rides) parts_to_add = 0, t_last_kernel[3] = 2;
+                    t_last_kernel[1] = 0x200 + variant;
                 }
+            } else {
+                if (!transposed) {
+                    weight_transpose_kernel<T><<<dim3((total + 255) / 256), dim3(256), 0, st>>>(g, static_cast<const T *>(pl.w), wt, total);
+                    TTAMD_HIP_CHECK(hipGetLastError());
+                }
+                if (ttamd_status rc = dgrad_gemm(g, wt, static_cast<T *>(gin), sum)) return rc;
             }
-            if (!handled) {
-                const int total = g.C * g.O * g.k * g.k;
-                weight_transpose_kernel<T><<<dim3((total + 255) / 256), dim3(256), 0, st>>>(g, static_cast<const T *>(pl.w), wt, total);
-                TTAMD_HIP_CHECK(hipGetLastError());
-                if (ttamd_status rc = dgrad_gemm(g, wt, static_cast<T *>(gin))) return rc;
-            }
+            if (sum.kind) parts_to_add = 0, t_last_kernel[3] = 2;
         }
     }
+    if (!wgrad_done)
+        if (ttamd_status rc = wgrad_implicit(ConvRide{})) return rc;
     if (parts_to_add > 0) {
         if (ttamd_status rc = launch_reduce_splits<T>(partials, static_cast<T *>(gw), gw_elems, parts_to_add, st)) return rc;
         t_last_kernel[3] = 1;
-    }
-    // grad_weight
-    {
-        const int M_ = g.O, N_ = g.C * g.k * g.k;
-        const int64_t tile_elems = static_cast<int64_t>(M_) * N_;
-        const bool staged = wgrad_staged;
-        t_last_kernel[2] = staged ? 0x200 : 0x100;
-        if (!staged) {
-        const int parts = plan.parts();
-        T *const partial = parts > 1 ? partials : static_cast<T *>(gw);
-        const int tiles_m = (M_ + 63) / 64, tiles_n = (N_ + 63) / 64;
-        const int64_t blocks = static_cast<int64_t>(tiles_m) * tiles_n * parts;
-        const bool a_vec = rows_vectorizable<T>(gout, HoWo, static_cast<int64_t>(g.O) * HoWo);
-        const bool b_vec = g.S == 1 && g.xs_w == 1 && g.Wo % VK == 0;
-        ConvGeom gw_geo = g;
-        if (wgrad_padded) {
-            gw_geo.row_pad = g.Wo % VK == 0 ? g.Wo : padded_row_width(sizeof(T), g.Wo);  // whole vectors already: joint mode only
-            gw_geo.d_row_pad = make_fastdiv(static_cast<uint32_t>(gw_geo.row_pad));
-        }
-        auto go = [&](auto kernel, size_t lds) {
-            return launch_conv(kernel, lds, blocks, st, gw_geo, static_cast<const T *>(gout), static_cast<const T *>(pl.x), partial,
-                               pl.image_bytes, plan.group, plan.kslices, plan.k_chunk, tiles_m, tiles_n, wgrad_mode == 2 ? joint_k : 0);
-        };
-        using VecB = TapStagerKC<T, 64, BK, VK, kConvPF>;
-        using OneB = Im2colTStager<T, 64, BK, kConvPF>;
-        ttamd_status s;
-        bool pair = false;
-        if constexpr (sizeof(T) == 4) pair = a_vec && !b_vec && g.S == 1 && g.xs_w == 1 && g.Wo % 2 == 0;
-        using PaddedB = TapStagerKC<T, 64, BK, VK, kConvPF, true>;
-        if (wgrad_padded) s = go(conv_wgrad_kernel<T, BK, VK, PaddedB, true>, conv_lds_bytes<T, 64, 64, VK, PaddedB>());
-        else if (a_vec && b_vec) s = go(conv_wgrad_kernel<T, BK, VK, VecB>, conv_lds_bytes<T, 64, 64, VK, VecB>());
-        else if (pair) {
-            if constexpr (sizeof(T) == 4) {
-                using PairB = TapStagerKC<T, 64, BK, 2, kConvPF>;
-                s = go(conv_wgrad_kernel<T, BK, VK, PairB>, conv_lds_bytes<T, 64, 64, VK, PairB>());
-            } else {
-                s = TTAMD_OK;
-            }
-        } else if (a_vec) s = go(conv_wgrad_kernel<T, BK, VK, OneB>, conv_lds_bytes<T, 64, 64, VK, OneB>());
-        else if (b_vec) s = go(conv_wgrad_kernel<T, BK, 1, VecB>, conv_lds_bytes<T, 64, 64, 1, VecB>());
-        else s = go(conv_wgrad_kernel<T, BK, 1, OneB>, conv_lds_bytes<T, 64, 64, 1, OneB>());
-        if (s) return s;
-        if (parts > 1)
-            if (ttamd_status rc = launch_reduce_splits<T>(partial, static_cast<T *>(gw), tile_elems, parts, st)) return rc;
-        }
     }
     if (gb) {
         using V = std::conditional_t<sizeof(T) == 4, float4, double2>;

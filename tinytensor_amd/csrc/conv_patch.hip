@@ -57,40 +57,6 @@ constexpr int tail_accumulators() {
     return WGM >= 2 ? 2 : 1;
 }
 
-// The launch's second job (ConvPatchArgs::red_*): workgroup r of the appended ones owns the 16-byte vectors 64 r .. 64 r + 63
-// of the result; each of its NW waves adds a contiguous share of the parts in increasing order, every load in flight
-// together (parts beyond the share arrive as +0 from the buffer load, which changes no sum that started at +0), and the
-// waves' sums are added in wave order.
-template <int NW>
-__device__ __forceinline__ void add_up_parts(const ConvPatchArgs &a, int r, float *lds) {
-    const int lane = threadIdx.x % 64;
-    const int w = __builtin_amdgcn_readfirstlane(threadIdx.x / 64);
-    const int v = r * 64 + lane;
-    const bool ok = 4 * v < a.red_n;
-    const int per = (a.red_splits + NW - 1) / NW;
-    const int s0 = w * per, s1 = s0 + per < a.red_splits ? s0 + per : a.red_splits;
-    const __amdgpu_buffer_rsrc_t src = make_rsrc(a.red_partial, static_cast<int64_t>(a.red_splits) * a.red_n * 4);
-    const uint32_t voff = ok ? static_cast<uint32_t>(v) * 16u : kOob;
-    f32x4 acc = f32x4{0.f, 0.f, 0.f, 0.f};
-#pragma unroll 1
-    for (int s = s0; s < s1; s += 16) {
-        f32x4 part[16];
-#pragma unroll
-        for (int u = 0; u < 16; ++u)
-            part[u] = Vec<float, 4>::load_at(src, s + u < s1 ? voff : kOob, static_cast<uint32_t>(s + u) * static_cast<uint32_t>(a.red_n) * 4u);
-#pragma unroll
-        for (int u = 0; u < 16; ++u) acc += part[u];
-    }
-    *reinterpret_cast<f32x4 *>(lds + (w * 64 + lane) * 4) = acc;
-    __syncthreads();
-    if (w == 0 && ok) {
-        f32x4 sum = acc;
-#pragma unroll
-        for (int k = 1; k < NW; ++k) sum += *reinterpret_cast<const f32x4 *>(lds + (k * 64 + lane) * 4);
-        *reinterpret_cast<f32x4 *>(a.red_out + 4 * static_cast<int64_t>(v)) = sum;
-    }
-}
-
 // WGM x WGN waves of one 32 x 32 MFMA block each: output tile (32 WGM) channels x (32 WGN) positions.
 // CC: chunks of 8 reduction indices (8 channels of one tap) that are read and multiplied as one straight-line group;
 // C / 8 is a multiple of it.
@@ -113,7 +79,7 @@ __global__ void __launch_bounds__(64 * WGM * WGN * KS, 1) conv_patch_kernel(Conv
     extern __shared__ __attribute__((aligned(16))) float smem_patch[];
     const int conv_blocks = static_cast<int>(gridDim.x) - a.red_blocks;
     if (static_cast<int>(blockIdx.x) >= conv_blocks) {  // an appended workgroup: the launch's second job
-        add_up_parts<NW>(a, static_cast<int>(blockIdx.x) - conv_blocks, smem_patch);
+        add_up_parts<float, NW>(a.red_partial, a.red_out, a.red_n, a.red_splits, static_cast<int>(blockIdx.x) - conv_blocks, smem_patch);
         return;
     }
     float *const A = smem_patch;                   // [BM][lda], k' = tap * C + c
@@ -644,12 +610,12 @@ ttamd_status launch_patch_cc(const ConvPatchArgs &a, hipStream_t st, size_t lds)
 
 }  // namespace
 
-// Launches when the geometry fits this kernel: *variant is 0 when it does not, else 16 * waves + patch buffers.  Expects in `a`: the tensors and their
+// Launches (unless `launch` is false: then only *variant is set) when the geometry fits this kernel: *variant is 0 when it does not, else 16 * waves + patch buffers.  Expects in `a`: the tensors and their
 // strides, B C H W O k P Ho Wo, and the weight access (w_row, w_red, w_flip, w_rows_fast): tap t of (row, reduction
 // channel) is at element  row * w_row + red * w_red + t  of the weight and is used as tap k*k - 1 - t when w_flip is
 // set.  Eight waves (two per SIMD, which hide each other's staging and store latencies) where their larger patch
 // fits in LDS, four otherwise; two patch buffers where they fit, one otherwise.
-ttamd_status launch_conv_patch_f32(ConvPatchArgs a, hipStream_t st, int *variant) {
+ttamd_status launch_conv_patch_f32(ConvPatchArgs a, hipStream_t st, int *variant, bool launch) {
     *variant = 0;
     const int k = a.k;
     if (a.B <= 0 || k < 1 || a.P >= k || a.C % 8 != 0 || a.W % 4 != 0) return TTAMD_OK;
@@ -681,6 +647,7 @@ ttamd_status launch_conv_patch_f32(ConvPatchArgs a, hipStream_t st, int *variant
         }
         if (best_bne && plan_patch(a, BM, 192, 12, 1, &lds, narrow ? 2 : 1, best_bne)) {
             *variant = 12 * 16 + 1;
+            if (!launch) return TTAMD_OK;
             return narrow ? launch_patch_cc<1, 6, 2>(a, st, lds) : launch_patch_cc<2, 6>(a, st, lds);
         }
     }
@@ -688,15 +655,18 @@ ttamd_status launch_conv_patch_f32(ConvPatchArgs a, hipStream_t st, int *variant
     for (int n_buf = 2; n_buf >= 1; --n_buf) {  // one patch buffer (a second barrier per tile) when two do not fit
         if (wide_ok && plan_patch(a, narrow ? 32 : 64, narrow ? 256 : 128, 8, n_buf, &lds)) {
             *variant = 8 * 16 + n_buf;
+            if (!launch) return TTAMD_OK;
             return narrow ? launch_patch_cc<1, 8>(a, st, lds) : launch_patch_cc<2, 4>(a, st, lds);
         }
         // the four-wave tile with a second set of waves on the other half of the reduction
         if (wide_ok && plan_patch(a, narrow ? 32 : 64, narrow ? 128 : 64, 8, n_buf, &lds, 2)) {
             *variant = 8 * 16 + n_buf;
+            if (!launch) return TTAMD_OK;
             return narrow ? launch_patch_cc<1, 4, 2>(a, st, lds) : launch_patch_cc<2, 2, 2>(a, st, lds);
         }
         if (plan_patch(a, narrow ? 32 : 64, narrow ? 128 : 64, 4, n_buf, &lds)) {
             *variant = 4 * 16 + n_buf;
+            if (!launch) return TTAMD_OK;
             return narrow ? launch_patch_cc<1, 4>(a, st, lds) : launch_patch_cc<2, 2>(a, st, lds);
         }
     }

@@ -1035,6 +1035,46 @@ __device__ __forceinline__ void store_tile_dense(Engine &eng, T *__restrict__ C,
     }
 }
 
+// A small second job that rides in a launch as workgroups appended to its grid: out[i] = sum over s < splits of
+// partial[s * n + i] (a sum that an earlier launch on the stream left in parts, spared a launch of its own).  Workgroup r
+// of the appended ones owns the 16-byte vectors 64 r .. 64 r + 63 of the result; each of its NW waves adds a contiguous
+// share of the parts in increasing order, every load in flight together (parts beyond the share arrive as +0 from the
+// buffer load, which changes no sum that started at +0), and the waves' sums are added through `lds` (NW * 64 vectors) in
+// wave order: a fixed order.  n a multiple of the vector length, both pointers 16-byte aligned, splits * n * sizeof(T) < 2^31.
+template <typename T, int NW>
+__device__ __forceinline__ void add_up_parts(const T *partial, T *out, int n, int splits, int r, T *lds) {
+    constexpr int VEC = 16 / sizeof(T);
+    using V = typename Vec<T, VEC>::type;
+    const int lane = threadIdx.x % 64;
+    const int w = __builtin_amdgcn_readfirstlane(threadIdx.x / 64);
+    const int v = r * 64 + lane;
+    const bool ok = VEC * v < n;
+    const int per = (splits + NW - 1) / NW;
+    const int s0 = w * per, s1 = s0 + per < splits ? s0 + per : splits;
+    const __amdgpu_buffer_rsrc_t src = make_rsrc(partial, static_cast<int64_t>(splits) * n * static_cast<int64_t>(sizeof(T)));
+    const uint32_t voff = ok ? static_cast<uint32_t>(v) * 16u : kOob;
+    V acc;
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) acc[j] = T(0);
+#pragma unroll 1
+    for (int s = s0; s < s1; s += 16) {
+        V part[16];
+#pragma unroll
+        for (int u = 0; u < 16; ++u)
+            part[u] = Vec<T, VEC>::load_at(src, s + u < s1 ? voff : kOob, static_cast<uint32_t>(s + u) * static_cast<uint32_t>(n) * static_cast<uint32_t>(sizeof(T)));
+#pragma unroll
+        for (int u = 0; u < 16; ++u) acc += part[u];
+    }
+    *reinterpret_cast<V *>(lds + (w * 64 + lane) * VEC) = acc;
+    __syncthreads();
+    if (w == 0 && ok) {
+        V sum = acc;
+#pragma unroll
+        for (int k = 1; k < NW; ++k) sum += *reinterpret_cast<const V *>(lds + (k * 64 + lane) * VEC);
+        *reinterpret_cast<V *>(out + static_cast<int64_t>(VEC) * v) = sum;
+    }
+}
+
 }  // namespace mfma
 }  // namespace ttamd
 
