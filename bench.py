@@ -287,7 +287,8 @@ def detail_report(tt, np, path, cpu=True):
     ms = time_launches(tt, lambda: be.conv2d_backward(go, x, w, None, 1, 1, buffers=bufs), 50, 5)
     rows.append({"case": "cfg4 conv2d backward (grad_input + grad_weight)",
                  "kernel": conv_kernel(1, "conv_dgrad_kernel (implicit GEMM)") + " + "
-                           + ("conv_wgrad_patch kernel (operands staged in LDS)" if lib_last(2) == 0x200 else "conv_wgrad_kernel (implicit GEMM)") + " + reduce",
+                           + ("conv_wgrad_patch kernel (operands staged in LDS)" if lib_last(2) == 0x200 else "conv_wgrad_kernel (implicit GEMM)")
+                           + {0: "", 1: " + a launch that adds up its partial tiles", 2: "; its partial tiles added up by workgroups appended to grad_input's launch"}[lib_last(3)],
                  "ms": round(ms, 5), "GFLOP/s": round(3.700e9 / ms / 1e6, 1)})
     # Streaming kernels around the GEMMs (HBM-bound; GB/s counts each operand and the result once), called through
     # the C ABI with preallocated results so that no allocation is timed.

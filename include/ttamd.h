@@ -237,9 +237,9 @@ ttamd_status ttamd_conv2d_backward(int device, ttamd_dtype dtype, const void *gr
  * implicit-GEMM MFMA kernels; 0x200 + 16 * waves + patch buffers: the persistent kernel that keeps the weight block in
  * LDS (fp32, unit stride, channel counts that are multiples of 8, rows of whole 16-byte vectors), 0x200 for
  * grad_weight: the kernel that stages both operands in LDS; 0: neither (another dtype, a direct kernel) or no call
- * yet.  which = 3: how the partial tiles of that LDS-staged grad_weight were added up -- 0: there were none, 1: by a
- * launch of their own, 2: by workgroups appended to grad_input's launch.  For tests and profiles that mean to cover a
- * particular kernel. */
+ * yet.  which = 3: how the partial tiles of that grad_weight were added up -- 0: there were none, 1: by a launch of
+ * their own, 2: by workgroups appended to grad_input's launch.  For tests and profiles that mean to cover a particular
+ * kernel. */
 int ttamd_conv2d_last_kernel(int which);
 
 /* BackendBase::max_pool2d / min_pool2d / avg_pool2d (backend_base.h:286-311; CPU: cpu/conv.cpp:296-349 over

@@ -327,6 +327,40 @@ def test_grad_weight_parts_added_in_grad_inputs_launch_exact(tt, oracle, shape):
     assert np.allclose(a, want, rtol=2e-4, atol=2e-3 * np.sqrt(Bn * H * W))
 
 
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+@pytest.mark.parametrize("geom", [
+    # B, C, H, W, O, k, S, P: layers on the implicit-GEMM kernels (weight blocks beyond LDS, odd widths, 5 x 5 taps, strides)
+    (4, 64, 28, 28, 128, 3, 1, 1), (3, 128, 14, 14, 128, 3, 1, 1), (6, 48, 9, 13, 40, 3, 1, 1), (2, 32, 20, 20, 32, 5, 1, 2),
+    (5, 64, 7, 7, 64, 3, 1, 1), (4, 64, 16, 16, 64, 1, 1, 0), (4, 64, 28, 28, 128, 3, 2, 1), (3, 8, 12, 12, 16, 3, 1, 0),
+], ids=lambda g: "x".join(map(str, g)))
+def test_backward_small_jobs_ride_in_the_big_launches_exact(tt, oracle, geom, dtype):
+    """conv2d_backward launches grad_weight first; the transposed weight that the implicit-GEMM grad_input reads is written
+    by workgroups appended to grad_weight's grid, and the sums over grad_weight's partial tiles and over grad_bias's parts
+    by workgroups appended to grad_input's.  Integer data: grad_input, grad_weight and grad_bias exact for both dtypes,
+    with and without a bias, and the same bits on a second call into the same workspace."""
+    Bn, Cc, H, W, O, k, S, P = geom
+    rng = np.random.default_rng(sum(geom))
+    x = rng.integers(-3, 4, (Bn, Cc, H, W)).astype(dtype)
+    w = rng.integers(-3, 4, (O, Cc, k, k)).astype(dtype)
+    b = rng.integers(-3, 4, (O,)).astype(dtype)
+    Ho, Wo = (H + 2 * P - k) // S + 1, (W + 2 * P - k) // S + 1
+    g = rng.integers(-3, 4, (Bn, O, Ho, Wo)).astype(dtype)
+    wx, ww, wb = oracle.conv2d_backward(g, x, w, True, S, P)
+    tg, tx, tw, tb = dev(tt, g), dev(tt, x), dev(tt, w), dev(tt, b)
+    be = tt.get_backend(tt.kAMD)
+    bufs = be.conv2d_backward(tg, tx, tw, tb, S, P, return_buffers=True)
+    route = _last_kernel(3)
+    for _ in range(2):
+        gx, gw, gb, _ws = bufs
+        assert np.array_equal(gx.to_numpy(), wx) and np.array_equal(gw.to_numpy(), ww) and np.array_equal(gb.to_numpy(), wb)
+        bufs = be.conv2d_backward(tg, tx, tw, tb, S, P, buffers=bufs, return_buffers=True)
+        assert _last_kernel(3) == route
+    if S == 1 and (O * Cc * k * k) % 4 == 0:
+        assert route in (0, 2), route              # unit stride: no launch of its own for the sum
+    gx, gw, none = tt.conv2d_backward(tg, tx, tw, None, S, P)
+    assert none is None and np.array_equal(gx.to_numpy(), wx) and np.array_equal(gw.to_numpy(), ww)
+
+
 def test_lds_resident_kernel_on_views(tt, oracle):
     # an input window of a larger tensor (row stride 16, 16-byte aligned start) and, through the C ABI, a weight whose
     # output-channel stride is larger than C k k (the row-wise weight loads)

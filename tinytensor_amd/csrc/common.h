@@ -149,8 +149,12 @@ struct ConvPatchArgs {
     const float *red_partial;
     float *red_out;
     int red_n, red_splits;
-    // derived
-    int red_blocks;
+    // a second such sum (grad_bias's parts), same conditions
+    const float *red2_partial;
+    float *red2_out;
+    int red2_n, red2_splits;
+    // derived: appended workgroups in all, those of them for the second sum
+    int red_blocks, red2_blocks;
     int K, lda, cpad, R, pitch, vecs_per_row, xh, last_vecs, n_items, stage_slots, cl_shift, tiles_m, tiles_n;
     int n_seg, seg_len, segs_per_pass, n_fast, n_wvec, w_dense, w_pass_vecs, n_buf;
     int bne, tail;  // positions per tile; those of them behind the tile's whole 32-position blocks (twelve waves: 4 or 8)

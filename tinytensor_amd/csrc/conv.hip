@@ -785,17 +785,24 @@ dgrad_interleave_kernel(ConvGeom geo, const T *__restrict__ tmp, T *__restrict__
 
 // A small job that rides in a convolution launch as `blocks` workgroups appended to its grid (spared a launch of its
 // own, which for these sizes is all launch floor): kind 1, dst[i] = sum over s < splits of src[s * n + i] (grad_weight's
-// partial tiles, mfma::add_up_parts); kind 2, the transposed weight of grad_input (weight_transpose_kernel's work).
+// partial tiles, mfma::add_up_parts) and a second such sum (grad_bias's parts); kind 2, the transposed weight of grad_input (weight_transpose_kernel's work).
 struct ConvRide {
     int kind = 0, blocks = 0;
     const void *src = nullptr;
     void *dst = nullptr;
     int n = 0, splits = 0;
+    // kind 1: a second sum (grad_bias's parts) by the last blocks2 of the appended workgroups
+    int blocks2 = 0;
+    const void *src2 = nullptr;
+    void *dst2 = nullptr;
+    int n2 = 0, splits2 = 0;
 };
 template <typename T>
 __device__ __forceinline__ void conv_ride(const ConvRide &r, const ConvGeom &geo, int block, T *smem) {
     if (r.kind == 1) {
-        add_up_parts<T, kThreads / 64>(static_cast<const T *>(r.src), static_cast<T *>(r.dst), r.n, r.splits, block, smem);
+        const int first = r.blocks - r.blocks2;
+        if (block < first) add_up_parts<T, kThreads / 64>(static_cast<const T *>(r.src), static_cast<T *>(r.dst), r.n, r.splits, block, smem);
+        else add_up_parts<T, kThreads / 64>(static_cast<const T *>(r.src2), static_cast<T *>(r.dst2), r.n2, r.splits2, block - first, smem);
     } else {
         const int idx = block * kThreads + static_cast<int>(threadIdx.x);
         if (idx >= r.n) return;
@@ -1649,6 +1656,31 @@ ttamd_status backward_mfma(const ConvPlan &pl, const void *gout, void *gin, void
     }
     T *const wt = static_cast<T *>(ws);
     T *const partials = reinterpret_cast<T *>(static_cast<char *>(ws) + plan.wt_bytes);
+    // grad_bias's parts first (they need grad_out alone): their sum can then ride in grad_input's launch
+    int bias_parts_to_add = 0;
+    T *bias_sums = nullptr;
+    if (gb) {
+        using V = std::conditional_t<sizeof(T) == 4, float4, double2>;
+        const bool vec = rows_vectorizable<T>(gout, HoWo, static_cast<int64_t>(g.O) * HoWo);
+        const int per_image = vec ? HoWo / VK : HoWo;
+        const int64_t total = static_cast<int64_t>(g.B) * per_image;
+        if (total > 0x7fffffff || g.O > 65535) {
+            set_error("conv2d_backward: grad_bias over %lld loads per channel and %d channels exceeds the launch limits",
+                      static_cast<long long>(total), g.O);
+            return TTAMD_ERR_INVALID_ARGUMENT;
+        }
+        const int bparts = bias_grad_parts(g.O, total);
+        const uint32_t chunk = static_cast<uint32_t>((total + bparts - 1) / bparts);
+        bias_sums = bparts > 1 ? reinterpret_cast<T *>(static_cast<char *>(ws) + plan.wt_bytes + plan.partial_bytes) : static_cast<T *>(gb);
+        const dim3 grid(static_cast<unsigned>(g.O), static_cast<unsigned>(bparts));
+        const FastDiv d = make_fastdiv(static_cast<uint32_t>(per_image));
+        if (vec)
+            bias_grad_kernel<T, V><<<grid, dim3(256), 0, st>>>(static_cast<const T *>(gout), bias_sums, g.O, HoWo, static_cast<uint32_t>(total), chunk, d);
+        else
+            bias_grad_kernel<T, T><<<grid, dim3(256), 0, st>>>(static_cast<const T *>(gout), bias_sums, g.O, HoWo, static_cast<uint32_t>(total), chunk, d);
+        TTAMD_HIP_CHECK(hipGetLastError());
+        if (bparts > 1) bias_parts_to_add = bparts;
+    }
     // grad_weight by the LDS-staged kernel goes first where it applies: the sum over its partial tiles can then ride in
     // grad_input's launch (ConvPatchArgs::red_*) instead of one of its own.
     bool wgrad_staged = false;
@@ -1729,7 +1761,22 @@ ttamd_status backward_mfma(const ConvPlan &pl, const void *gout, void *gin, void
             r.n = static_cast<int>(gw_elems);
             r.splits = parts_to_add;
         }
+        if (bias_parts_to_add > 0 && g.O % VEC == 0 && reinterpret_cast<uintptr_t>(gb) % 16 == 0 && reinterpret_cast<uintptr_t>(bias_sums) % 16 == 0) {
+            r.kind = 1;
+            r.blocks2 = (g.O / VEC + 63) / 64;
+            r.blocks += r.blocks2;
+            r.src2 = bias_sums;
+            r.dst2 = gb;
+            r.n2 = g.O;
+            r.splits2 = bias_parts_to_add;
+        }
         return r;
+    };
+    // (what a launch has taken along is no longer pending)
+    auto rode = [&](const ConvRide &r) {
+        if (r.kind != 1) return;
+        if (r.blocks > r.blocks2) parts_to_add = 0, t_last_kernel[3] = 2;
+        if (r.blocks2 > 0) bias_parts_to_add = 0;
     };
     // grad_input
     t_last_kernel[1] = 0;
@@ -1942,11 +1989,17 @@ ttamd_status backward_mfma(const ConvPlan &pl, const void *gout, void *gin, void
             const ConvRide sum = sum_ride();
             if (resident) {
                 if constexpr (std::is_same_v<T, float>) {
-                    if (sum.kind) {
-                        a.red_partial = partials;
-                        a.red_out = static_cast<float *>(gw);
+                    if (sum.blocks > sum.blocks2) {
+                        a.red_partial = static_cast<const float *>(sum.src);
+                        a.red_out = static_cast<float *>(sum.dst);
                         a.red_n = sum.n;
                         a.red_splits = sum.splits;
+                    }
+                    if (sum.blocks2 > 0) {
+                        a.red2_partial = static_cast<const float *>(sum.src2);
+                        a.red2_out = static_cast<float *>(sum.dst2);
+                        a.red2_n = sum.n2;
+                        a.red2_splits = sum.splits2;
                     }
                     int variant = 0;
                     if (ttamd_status rc = launch_conv_patch_f32(a, st, &variant)) return rc;
@@ -1959,7 +2012,7 @@ ttamd_status backward_mfma(const ConvPlan &pl, const void *gout, void *gin, void
                 }
                 if (ttamd_status rc = dgrad_gemm(g, wt, static_cast<T *>(gin), sum)) return rc;
             }
-            if (sum.kind) parts_to_add = 0, t_last_kernel[3] = 2;
+            rode(sum);
         }
     }
     if (!wgrad_done)
@@ -1968,29 +2021,8 @@ ttamd_status backward_mfma(const ConvPlan &pl, const void *gout, void *gin, void
         if (ttamd_status rc = launch_reduce_splits<T>(partials, static_cast<T *>(gw), gw_elems, parts_to_add, st)) return rc;
         t_last_kernel[3] = 1;
     }
-    if (gb) {
-        using V = std::conditional_t<sizeof(T) == 4, float4, double2>;
-        const bool vec = rows_vectorizable<T>(gout, HoWo, static_cast<int64_t>(g.O) * HoWo);
-        const int per_image = vec ? HoWo / VK : HoWo;
-        const int64_t total = static_cast<int64_t>(g.B) * per_image;
-        if (total > 0x7fffffff || g.O > 65535) {
-            set_error("conv2d_backward: grad_bias over %lld loads per channel and %d channels exceeds the launch limits",
-                      static_cast<long long>(total), g.O);
-            return TTAMD_ERR_INVALID_ARGUMENT;
-        }
-        const int bparts = bias_grad_parts(g.O, total);
-        const uint32_t chunk = static_cast<uint32_t>((total + bparts - 1) / bparts);
-        T *const sums = bparts > 1 ? reinterpret_cast<T *>(static_cast<char *>(ws) + plan.wt_bytes + plan.partial_bytes) : static_cast<T *>(gb);
-        const dim3 grid(static_cast<unsigned>(g.O), static_cast<unsigned>(bparts));
-        const FastDiv d = make_fastdiv(static_cast<uint32_t>(per_image));
-        if (vec)
-            bias_grad_kernel<T, V><<<grid, dim3(256), 0, st>>>(static_cast<const T *>(gout), sums, g.O, HoWo, static_cast<uint32_t>(total), chunk, d);
-        else
-            bias_grad_kernel<T, T><<<grid, dim3(256), 0, st>>>(static_cast<const T *>(gout), sums, g.O, HoWo, static_cast<uint32_t>(total), chunk, d);
-        TTAMD_HIP_CHECK(hipGetLastError());
-        if (bparts > 1)
-            if (ttamd_status rc = launch_reduce_splits<T>(sums, static_cast<T *>(gb), g.O, bparts, st)) return rc;
-    }
+    if (bias_parts_to_add > 0)
+        if (ttamd_status rc = launch_reduce_splits<T>(bias_sums, static_cast<T *>(gb), g.O, bias_parts_to_add, st)) return rc;
     return TTAMD_OK;
 }
 

@@ -79,7 +79,9 @@ __global__ void __launch_bounds__(64 * WGM * WGN * KS, 1) conv_patch_kernel(Conv
     extern __shared__ __attribute__((aligned(16))) float smem_patch[];
     const int conv_blocks = static_cast<int>(gridDim.x) - a.red_blocks;
     if (static_cast<int>(blockIdx.x) >= conv_blocks) {  // an appended workgroup: the launch's second job
-        add_up_parts<float, NW>(a.red_partial, a.red_out, a.red_n, a.red_splits, static_cast<int>(blockIdx.x) - conv_blocks, smem_patch);
+        const int r = static_cast<int>(blockIdx.x) - conv_blocks, first = a.red_blocks - a.red2_blocks;
+        if (r < first) add_up_parts<float, NW>(a.red_partial, a.red_out, a.red_n, a.red_splits, r, smem_patch);
+        else add_up_parts<float, NW>(a.red2_partial, a.red2_out, a.red2_n, a.red2_splits, r - first, smem_patch);
         return;
     }
     float *const A = smem_patch;                   // [BM][lda], k' = tap * C + c
@@ -582,7 +584,8 @@ ttamd_status launch_patch(ConvPatchArgs a, hipStream_t st, size_t lds) {
     a.d_ngrp = make_fastdiv(static_cast<uint32_t>(a.C / (8 * CC)));
     auto kernel = conv_patch_kernel<WGM, WGN, CC, MAXS, KS>;
     TTAMD_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds)));
-    a.red_blocks = a.red_splits > 0 ? (a.red_n / 4 + 63) / 64 : 0;
+    a.red2_blocks = a.red2_splits > 0 ? (a.red2_n / 4 + 63) / 64 : 0;
+    a.red_blocks = (a.red_splits > 0 ? (a.red_n / 4 + 63) / 64 : 0) + a.red2_blocks;
     if (lds < static_cast<size_t>(64 * WGM * WGN * KS) * 16) lds = static_cast<size_t>(64 * WGM * WGN * KS) * 16;  // (the second job's sums)
     kernel<<<dim3(static_cast<unsigned>(groups * a.tiles_m + a.red_blocks)), dim3(64 * WGM * WGN * KS), lds, st>>>(a);
     TTAMD_HIP_CHECK(hipGetLastError());
