@@ -785,7 +785,7 @@ dgrad_interleave_kernel(ConvGeom geo, const T *__restrict__ tmp, T *__restrict__
 
 // A small job that rides in a convolution launch as `blocks` workgroups appended to its grid (spared a launch of its
 // own, which for these sizes is all launch floor): kind 1, dst[i] = sum over s < splits of src[s * n + i] (grad_weight's
-// partial tiles, mfma::add_up_parts) and a second such sum (grad_bias's parts); kind 2, the transposed weight of grad_input (weight_transpose_kernel's work).
+// partial tiles, mfma::add_up_parts) and a second such sum (grad_bias's parts); kind 3, the packed class weights of a strided grad_input (weight_class_pack_kernel's work); kind 2, the transposed weight of grad_input (weight_transpose_kernel's work).
 struct ConvRide {
     int kind = 0, blocks = 0;
     const void *src = nullptr;
@@ -798,8 +798,18 @@ struct ConvRide {
     int n2 = 0, splits2 = 0;
 };
 template <typename T>
-__device__ __forceinline__ void conv_ride(const ConvRide &r, const ConvGeom &geo, int block, T *smem) {
-    if (r.kind == 1) {
+__device__ __forceinline__ void conv_ride(const ConvRide &r, const ConvGeom &geo, int block, T *smem, const DgradClasses *classes = nullptr) {
+    if (r.kind == 3) {  // weight_class_pack_kernel's work: r.splits blocks per class of a strided grad_input
+        const int ci = block / r.splits, idx = (block - ci * r.splits) * kThreads + static_cast<int>(threadIdx.x);
+        const DgradClass &cl = classes->cls[ci];
+        const int kpq = cl.kp * cl.kq, row = geo.O * kpq, total = geo.C * row;
+        if (idx >= total) return;
+        const int c = idx / row, rem = idx - c * row;
+        const int o = rem / kpq, t = rem - o * kpq;
+        const int pi = t / cl.kq, qi = t - pi * cl.kq;
+        static_cast<T *>(r.dst)[cl.wt_off + idx] =
+            static_cast<const T *>(r.src)[static_cast<int64_t>(o) * geo.w_so + (c * geo.k + cl.ry + geo.S * pi) * geo.k + cl.rx + geo.S * qi];
+    } else if (r.kind == 1) {
         const int first = r.blocks - r.blocks2;
         if (block < first) add_up_parts<T, kThreads / 64>(static_cast<const T *>(r.src), static_cast<T *>(r.dst), r.n, r.splits, block, smem);
         else add_up_parts<T, kThreads / 64>(static_cast<const T *>(r.src2), static_cast<T *>(r.dst2), r.n2, r.splits2, block - first, smem);
@@ -871,12 +881,16 @@ static_assert(sizeof(DgradClassGeoms) <= 3584, "kernel arguments are limited to 
 
 template <typename T, int BM, int BN, int BK, int A_VEC, class StB>
 __global__ void __launch_bounds__(kThreads, 2)
-conv_dgrad_classes_kernel(DgradClassGeoms tab, const T *gout, const T *wt, T *gin) {
+conv_dgrad_classes_kernel(DgradClassGeoms tab, const T *gout, const T *wt, T *gin, ConvRide ride) {
     using StA = Stager<T, BM, BK, true, A_VEC, kConvPF>;
     using Engine = ConvEngine<T, BM, BN, BK, StA, StB>;
     extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
     T *const smem = reinterpret_cast<T *>(smem_raw);
     const int tid = threadIdx.x;
+    if (static_cast<int>(blockIdx.x) >= tab.first_block[tab.n]) {  // an appended workgroup (sums only: no geometry needed)
+        conv_ride<T>(ride, tab.geo[0], static_cast<int>(blockIdx.x) - tab.first_block[tab.n], smem);
+        return;
+    }
     int ci = 0;
     while (ci + 1 < tab.n && static_cast<int>(blockIdx.x) >= tab.first_block[ci + 1]) ++ci;  // (uniform, at most 8 steps)
     const ConvGeom &geo = tab.geo[ci];
@@ -909,7 +923,7 @@ conv_dgrad_classes_kernel(DgradClassGeoms tab, const T *gout, const T *wt, T *gi
 template <typename T, int BK, int A_VEC, class StB, bool PADDED = false>
 __global__ void __launch_bounds__(kThreads, 2)
 conv_wgrad_kernel(ConvGeom geo, const T *gout, const T *x, T *partial, int64_t image_bytes, int group, int kslices, int k_chunk,
-                  int tiles_m, int tiles_n, int joint_k, ConvRide ride) {
+                  int tiles_m, int tiles_n, int joint_k, ConvRide ride, DgradClasses classes) {
     constexpr int BM = 64, BN = 64;
     using StA = std::conditional_t<PADDED, PaddedRowsStager<T, BM, BK, kConvPF>, Stager<T, BM, BK, true, A_VEC, kConvPF>>;
     using Engine = ConvEngine<T, BM, BN, BK, StA, StB>;
@@ -918,7 +932,7 @@ conv_wgrad_kernel(ConvGeom geo, const T *gout, const T *x, T *partial, int64_t i
     const int tid = threadIdx.x;
     const unsigned conv_blocks = gridDim.x - static_cast<unsigned>(ride.blocks);
     if (blockIdx.x >= conv_blocks) {  // an appended workgroup
-        conv_ride<T>(ride, geo, static_cast<int>(blockIdx.x - conv_blocks), smem);
+        conv_ride<T>(ride, geo, static_cast<int>(blockIdx.x - conv_blocks), smem, &classes);
         return;
     }
     int part, tm, tn;
@@ -1708,7 +1722,7 @@ ttamd_status backward_mfma(const ConvPlan &pl, const void *gout, void *gin, void
     // parts_to_add for whoever adds them up.
     t_last_kernel[2] = wgrad_staged ? 0x200 : 0x100;
     bool wgrad_done = wgrad_staged;
-    auto wgrad_implicit = [&](const ConvRide &ride) -> ttamd_status {
+    auto wgrad_implicit = [&](const ConvRide &ride, const DgradClasses &classes = DgradClasses{}) -> ttamd_status {
         const int M_ = g.O, N_ = g.C * g.k * g.k;
         const int parts = plan.parts();
         T *const partial = parts > 1 ? partials : static_cast<T *>(gw);
@@ -1723,7 +1737,7 @@ ttamd_status backward_mfma(const ConvPlan &pl, const void *gout, void *gin, void
         }
         auto go = [&](auto kernel, size_t lds) {
             return launch_conv(kernel, lds, blocks + ride.blocks, st, gw_geo, static_cast<const T *>(gout), static_cast<const T *>(pl.x), partial,
-                               pl.image_bytes, plan.group, plan.kslices, plan.k_chunk, tiles_m, tiles_n, wgrad_mode == 2 ? joint_k : 0, ride);
+                               pl.image_bytes, plan.group, plan.kslices, plan.k_chunk, tiles_m, tiles_n, wgrad_mode == 2 ? joint_k : 0, ride, classes);
         };
         using VecB = TapStagerKC<T, 64, BK, VK, kConvPF>;
         using OneB = Im2colTStager<T, 64, BK, kConvPF>;
@@ -1864,8 +1878,21 @@ ttamd_status backward_mfma(const ConvPlan &pl, const void *gout, void *gin, void
                 most = std::max(most, g.C * g.O * cl.kp * cl.kq);
                 if (cl.kp == 0 || cl.kq == 0) every_class_has_taps = false;
             }
-            weight_class_pack_kernel<T><<<dim3((most + 255) / 256, g.S * g.S), dim3(256), 0, st>>>(g, static_cast<const T *>(pl.w), wt, dc.tab);
-            TTAMD_HIP_CHECK(hipGetLastError());
+            // grad_weight first, the packing of the class weights appended to its grid; the sums over its partial tiles and
+            // grad_bias's parts then ride in the classes' launch
+            if (!wgrad_done) {
+                ConvRide pack;
+                pack.kind = 3;
+                pack.splits = (most + kThreads - 1) / kThreads;  // workgroups per class
+                pack.blocks = pack.splits * g.S * g.S;
+                pack.src = pl.w;
+                pack.dst = wt;
+                if (ttamd_status rc = wgrad_implicit(pack, dc.tab)) return rc;
+            } else {
+                weight_class_pack_kernel<T><<<dim3((most + 255) / 256, g.S * g.S), dim3(256), 0, st>>>(g, static_cast<const T *>(pl.w), wt, dc.tab);
+                TTAMD_HIP_CHECK(hipGetLastError());
+            }
+            ConvRide sum = sum_ride();
             auto class_geometry = [&](const DgradClass &cl) {
                 ConvGeom gc = g;  // the class as a unit-stride problem over its own positions
                 gc.H = cl.Hc;
@@ -1917,7 +1944,7 @@ ttamd_status backward_mfma(const ConvPlan &pl, const void *gout, void *gin, void
                 }
                 if (ok && tab.n > 0) {
                     auto go = [&](auto kernel, size_t lds) {
-                        return launch_conv(kernel, lds, blocks, st, tab, static_cast<const T *>(gout), static_cast<const T *>(wt), static_cast<T *>(gin));
+                        return launch_conv(kernel, lds, blocks + sum.blocks, st, tab, static_cast<const T *>(gout), static_cast<const T *>(wt), static_cast<T *>(gin), sum);
                     };
                     ttamd_status rc;
                     if (g.C <= 32) {
@@ -1930,13 +1957,17 @@ ttamd_status backward_mfma(const ConvPlan &pl, const void *gout, void *gin, void
                     if (rc) return rc;
                     merged = true;
                     t_last_kernel[1] = 0x101;
+                    rode(sum);
+                    sum = ConvRide{};
                 }
             }
             for (int ci = 0; ci < g.S * g.S && !merged; ++ci) {
                 const DgradClass &cl = dc.tab.cls[ci];
                 if (cl.kp == 0 || cl.kq == 0 || cl.Hc == 0 || cl.Wc == 0) continue;
                 const ConvGeom gc = class_geometry(cl);
-                if (ttamd_status rc = dgrad_gemm(gc, wt + cl.wt_off, every_class_has_taps ? static_cast<T *>(gin) : tmp + cl.tmp_off)) return rc;
+                if (ttamd_status rc = dgrad_gemm(gc, wt + cl.wt_off, every_class_has_taps ? static_cast<T *>(gin) : tmp + cl.tmp_off, sum)) return rc;
+                rode(sum);  // (the first class's launch takes the sums along)
+                sum = ConvRide{};
             }
             if (!every_class_has_taps) {
                 const int64_t total = static_cast<int64_t>(g.B) * g.C * g.H * g.W;
