@@ -1140,9 +1140,15 @@ conv_fwd_direct_kernel(ConvGeom geo, const T *__restrict__ x, const T *__restric
 // no per-lane LDS read per product.
 template <typename T, int CMAX, int NP, bool UNIT = false>
 __global__ void __launch_bounds__(256)
-conv_dgrad_slots_kernel(ConvGeom geo, const T *__restrict__ gout, const T *__restrict__ w, T *__restrict__ gin, int blocks_per_image) {
+conv_dgrad_slots_kernel(ConvGeom geo, const T *__restrict__ gout, const T *__restrict__ w, T *__restrict__ gin, int blocks_per_image,
+                        ConvRide ride) {
     extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
     T *const wl = reinterpret_cast<T *>(smem_raw);
+    const unsigned conv_blocks = gridDim.x - static_cast<unsigned>(ride.blocks);
+    if (blockIdx.x >= conv_blocks) {  // an appended workgroup (sums only; the launch reserves their 4 KB of LDS)
+        conv_ride<T>(ride, geo, static_cast<int>(blockIdx.x - conv_blocks), wl);
+        return;
+    }
     const int kk = geo.k * geo.k, HW = geo.H * geo.W, HoWo = geo.Ho * geo.Wo;
     if constexpr (!UNIT) {
         for (int i = threadIdx.x; i < geo.O * kk * CMAX; i += 256) {
@@ -1797,17 +1803,22 @@ ttamd_status backward_mfma(const ConvPlan &pl, const void *gout, void *gin, void
     const int np = (g.k + g.S - 1) / g.S;
     const size_t slots_lds = static_cast<size_t>(g.O) * g.k * g.k * g.C * sizeof(T);
     if (g.C <= kDirectDgradChannels && np <= 4 && slots_lds <= 64 * 1024) {
+        // grad_weight first: the sums over its partial tiles and grad_bias's parts ride in grad_input's launch
+        if (!wgrad_done)
+            if (ttamd_status rc = wgrad_implicit(ConvRide{})) return rc;
+        const ConvRide sum = sum_ride();
+        const size_t ride_lds = sum.kind ? kThreads / 64 * 64 * 16 : 0;  // add_up_parts: a 16-byte vector per lane
         const int bpi = (g.H * g.W + 255) / 256;
         const int64_t blocks = static_cast<int64_t>(g.B) * bpi;
         auto go = [&](auto kernel) -> ttamd_status {
-            return launch_conv(kernel, slots_lds, blocks, st, g, static_cast<const T *>(gout), static_cast<const T *>(pl.w),
-                               static_cast<T *>(gin), bpi);
+            return launch_conv(kernel, slots_lds > ride_lds ? slots_lds : ride_lds, blocks + sum.blocks, st, g, static_cast<const T *>(gout),
+                               static_cast<const T *>(pl.w), static_cast<T *>(gin), bpi, sum);
         };
         auto by_windows = [&]<int CMAX>() -> ttamd_status {  // CMAX = C: no padded channel is multiplied
             if (g.S == 1) {  // np == k: the weights are wave-uniform scalars, no LDS copy
                 auto unit = [&](auto kernel) -> ttamd_status {
-                    return launch_conv(kernel, 0, blocks, st, g, static_cast<const T *>(gout), static_cast<const T *>(pl.w),
-                                       static_cast<T *>(gin), bpi);
+                    return launch_conv(kernel, ride_lds, blocks + sum.blocks, st, g, static_cast<const T *>(gout), static_cast<const T *>(pl.w),
+                                       static_cast<T *>(gin), bpi, sum);
                 };
                 if (np == 1) return unit(conv_dgrad_slots_kernel<T, CMAX, 1, true>);
                 if (np == 2) return unit(conv_dgrad_slots_kernel<T, CMAX, 2, true>);
@@ -1826,6 +1837,7 @@ ttamd_status backward_mfma(const ConvPlan &pl, const void *gout, void *gin, void
         else if (g.C == 3) rc = by_windows.template operator()<3>();
         else rc = by_windows.template operator()<4>();
         if (rc) return rc;
+        rode(sum);
     } else {
         // One unit-stride (or, without the class split, strided) grad_input GEMM: geometry gg, transposed weight wts
         // [C, O*kh*kw], dense result dst [B, C, gg.H*gg.W].
