@@ -571,6 +571,11 @@ inline auto matmul(const Tensor &lhs_, const Tensor &rhs_) -> Tensor {
 
 // TensorBatchedMatmul::backward (autograd/binary_ops.cpp:173-179): both gradients, on permuted VIEWS.
 inline auto matmul_backward(const Tensor &lhs, const Tensor &rhs, const Tensor &grad_output) -> std::pair<Tensor, Tensor> {
+    if (lhs.dim() == 3 && rhs.dim() == 3 && grad_output.dim() == 3 && lhs.dtype() == rhs.dtype() && lhs.dtype() == grad_output.dtype() &&
+        lhs.dtype() != kBool && lhs.size(0) == rhs.size(0) && lhs.size(2) == rhs.size(1) && grad_output.size(0) == lhs.size(0) &&
+        grad_output.size(1) == lhs.size(1) && grad_output.size(2) == rhs.size(2))
+        // what forward stored: 3-D operands of one dtype -- both products in one backend call (one grid where that pays)
+        return get_backend(lhs.device())->batched_matmul_pair(grad_output, rhs.permute({0, 2, 1}), nullptr, lhs.permute({0, 2, 1}), grad_output, nullptr);
     return {matmul(grad_output, rhs.permute({0, 2, 1})), matmul(lhs.permute({0, 2, 1}), grad_output)};
 }
 

@@ -845,6 +845,11 @@ def matmul(lhs: Tensor, rhs: Tensor) -> Tensor:
 def matmul_backward(lhs: Tensor, rhs: Tensor, grad_output: Tensor):
     """TensorBatchedMatmul::backward (autograd/binary_ops.cpp:173-179): dA = dC.B^T, dB = A^T.dC, both
     on permute({0,2,1}) VIEWS.  Both gradients are always computed, as in the reference."""
+    if (lhs.dim() == 3 and rhs.dim() == 3 and grad_output.dim() == 3 and lhs.dtype == rhs.dtype == grad_output.dtype
+            and lhs.dtype != _capi.BOOL and lhs.device == rhs.device == grad_output.device
+            and grad_output.shape == (lhs.size(0), lhs.size(1), rhs.size(2)) and lhs.size(2) == rhs.size(1) and lhs.size(0) == rhs.size(0)):
+        # what forward stored: 3-D operands of one dtype -- both products in one backend call (one grid where that pays)
+        return get_backend(lhs.device).batched_matmul_pair((grad_output, rhs.permute(0, 2, 1)), (lhs.permute(0, 2, 1), grad_output))
     return matmul(grad_output, rhs.permute(0, 2, 1)), matmul(lhs.permute(0, 2, 1), grad_output)
 
 
