@@ -1655,6 +1655,12 @@ BackwardWorkspace backward_workspace(size_t esz, int B, int C, int H, int W, int
 // against 7.3 ms on the padded MFMA tile; 3x3 stride-1 first layers of 28 x 28 and 32 x 32 images: 10 - 25 % faster).
 constexpr int kDirectDgradChannels = 4;
 
+// TTAMD_CONV_RIDE=0: every small job of a backward pass as a launch of its own (for comparisons).
+bool conv_rides_enabled() {
+    static const bool on = std::getenv("TTAMD_CONV_RIDE") == nullptr || std::atoi(std::getenv("TTAMD_CONV_RIDE")) != 0;
+    return on;
+}
+
 template <typename T>
 ttamd_status backward_mfma(const ConvPlan &pl, const void *gout, void *gin, void *gw, void *gb, void *ws, size_t ws_bytes,
                            hipStream_t st) {
@@ -1771,6 +1777,7 @@ ttamd_status backward_mfma(const ConvPlan &pl, const void *gout, void *gin, void
     // the sum over grad_weight's partial tiles as a job appended to another launch, where vectors of 16 bytes can carry it
     auto sum_ride = [&]() {
         ConvRide r;
+        if (!conv_rides_enabled()) return r;
         constexpr int VEC = 16 / static_cast<int>(sizeof(T));
         if (parts_to_add > 0 && gw_elems % VEC == 0 && reinterpret_cast<uintptr_t>(gw) % 16 == 0 && reinterpret_cast<uintptr_t>(partials) % 16 == 0 &&
             parts_to_add * gw_elems * static_cast<int64_t>(sizeof(T)) < 0x7fffffffLL) {
@@ -1892,7 +1899,7 @@ ttamd_status backward_mfma(const ConvPlan &pl, const void *gout, void *gin, void
             }
             // grad_weight first, the packing of the class weights appended to its grid; the sums over its partial tiles and
             // grad_bias's parts then ride in the classes' launch
-            if (!wgrad_done) {
+            if (!wgrad_done && conv_rides_enabled()) {
                 ConvRide pack;
                 pack.kind = 3;
                 pack.splits = (most + kThreads - 1) / kThreads;  // workgroups per class
@@ -2019,7 +2026,7 @@ ttamd_status backward_mfma(const ConvPlan &pl, const void *gout, void *gin, void
             bool transposed = false;
             if (!wgrad_done) {
                 ConvRide ride;
-                if (!resident) {
+                if (!resident && conv_rides_enabled()) {
                     ride.kind = 2;
                     ride.blocks = (total + kThreads - 1) / kThreads;
                     ride.src = pl.w;
