@@ -185,3 +185,36 @@ def test_random_lds_staged_convs(tt, oracle, seed):
         assert np.array_equal(gx.to_numpy(), wx), tag
         assert np.array_equal(gw.to_numpy(), ww), tag
         assert np.array_equal(gb.to_numpy(), wb), tag
+
+
+@pytest.mark.parametrize("seed", range(10))
+def test_random_pairs_of_gradient_products(tt, seed):
+    """ttamd_batched_matmul_pair on random Linear-layer sizes on both sides of the one-grid conditions (128 to 256 tiles of
+    64 x 64 per product, reductions of 512 or more, dense fp32), with random batches, a ReLU mask, the right operand's column
+    sums and, now and then, operands that are views: integer-valued data, every element exact, whichever way it ran."""
+    rng = np.random.default_rng(9000 + seed)
+    dtype = [np.float32, np.float32, np.float32, np.float64][int(rng.integers(0, 4))]
+    batch = int(rng.choice([1, 1, 1, 2]))
+    # rows n, in_features fin, out_features fout: dx = dy . W^T is [n, fin] with reduction fout, dW = x^T . dy is [fin, fout] with reduction n
+    n = int(rng.choice([448, 512, 520, 640, 1000, 1024]))
+    fin = int(rng.choice([500, 784, 1000, 1024, 1600]))
+    fout = int(rng.choice([448, 512, 576, 1024, 1030]))
+    if batch == 2:
+        n, fin, fout = n // 2 + 8, fin // 2 + 4, max(fout // 2, 512)
+    dy = rng.integers(-3, 4, (batch, n, fout)).astype(dtype)
+    x = rng.integers(-3, 4, (batch, n, fin)).astype(dtype)
+    w = rng.integers(-3, 4, (batch, fin, fout)).astype(dtype)
+    z = rng.integers(-2, 3, (batch, n, fin)).astype(dtype)
+    tdy, tx, tz = (tt.Tensor.from_numpy(v) for v in (dy, x, z))
+    if seed % 3 == 2:   # the weight as a transposed store: dy . W^T then reads a plain matrix, a layout outside the pair's
+        tw = tt.Tensor.from_numpy(np.ascontiguousarray(w.transpose(0, 2, 1))).permute(0, 2, 1)
+    else:
+        tw = tt.Tensor.from_numpy(w)
+    be = tt.get_backend(tt.kAMD)
+    db = tt.Tensor.empty((batch, fout), tdy.dtype)
+    dx, dW = be.batched_matmul_pair((tdy, tw.permute(0, 2, 1), dict(relu_grad_input=tz)), (tx.permute(0, 2, 1), tdy, dict(rhs_colsum_out=db)))
+    want_dx = np.matmul(dy.astype(np.float64), w.transpose(0, 2, 1).astype(np.float64)) * np.where(z < 0, 0.0, 1.0)
+    want_dW = np.matmul(x.transpose(0, 2, 1).astype(np.float64), dy.astype(np.float64))
+    assert np.array_equal(dx.to_numpy(), want_dx.astype(dtype)), (seed, batch, n, fin, fout, dtype)
+    assert np.array_equal(dW.to_numpy(), want_dW.astype(dtype)), (seed, batch, n, fin, fout, dtype)
+    assert np.array_equal(db.to_numpy(), dy.sum(1)), (seed, batch, n, fin, fout, dtype)
